@@ -1,0 +1,221 @@
+/* Kernel-level C ABI of the MI355X (gfx950) action-expert attention path.
+ *
+ * Conventions (those of the reference's in-tree kernel layer,
+ * src/kernels/bitvla/bitvla_lm_cuda.h:28-30): extern "C", device pointers,
+ * plain ints, the stream passed explicitly as the last argument, no device
+ * synchronisation inside.  Unlike the reference's void launchers every entry
+ * point returns a vla_kstatus, so a bad shape is reported instead of aborting
+ * the process (the reference aborts, src/kernels/bitvla/bitnet_kernels.cu:22-29).
+ *
+ * bf16 values are raw 16-bit patterns (uint16_t); `dtype` arguments take
+ * VLA_DT_F32 or VLA_DT_BF16.  "token-major" is [token][head][head_dim], i.e.
+ * ggml's [head_dim, n_heads, n_tokens] with ne0 innermost, the layout the
+ * reference's projections produce (src/models/smolvla.cpp:825-827).
+ *
+ * Resident KV cache layout (one K and one V buffer per layer):
+ *     K  : [batch][n_kv_heads][t_max][head_dim]
+ *     V^T: [batch][n_kv_heads][head_dim][t_max]        (t_max % 8 == 0)
+ * The prefix occupies tokens [0, P) and is written once per observation; the
+ * action suffix of every denoise step overwrites tokens [P, P+S) in place.
+ */
+#ifndef VLA_KERNELS_H
+#define VLA_KERNELS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VLA_KAPI __attribute__((visibility("default")))
+
+typedef void* vla_stream_t; /* a hipStream_t */
+
+typedef enum { VLA_DT_F32 = 0, VLA_DT_BF16 = 1 } vla_dtype;
+
+typedef enum {
+    VLA_K_OK = 0,
+    VLA_K_ERR_ARG = -1,    /* null pointer or negative size */
+    VLA_K_ERR_SHAPE = -2,  /* a size the kernels do not support (alignment, head_dim, ...) */
+    VLA_K_ERR_LAUNCH = -3, /* hipGetLastError() after the launch */
+} vla_kstatus;
+
+/* Suffix-block mask generated inside the attention kernel (the reference builds
+ * these on the host as additive 0/-inf matrices and uploads them):
+ *   NONE          pi0.5 / GR00T DiT / BitVLA: every key visible.
+ *   CAUSAL_SUFFIX SmolVLA mask_full (src/models/smolvla.cpp:1651-1664):
+ *                 suffix key j (>= n_prefix) is hidden from query i when
+ *                 j - n_prefix > i.
+ *   PI0_STATE     pi0 full mask (src/models/pi0.cpp:638-653): query 0 (the
+ *                 state token) sees only suffix key 0; other queries see all.
+ * In every kind, prefix keys in [pad_start, pad_end) are hidden (SmolVLA's
+ * padded language tokens); pass pad_start == pad_end for none. */
+typedef enum { VLA_MASK_NONE = 0, VLA_MASK_CAUSAL_SUFFIX = 1, VLA_MASK_PI0_STATE = 2 } vla_mask_kind;
+
+/* ---------------------------------------------------------------- KV cache */
+
+/* In-place append, replacing ggml_concat(cached_K, k_rope, 2) /
+ * ggml_concat(cached_V, v_h, 2) (src/models/smolvla.cpp:832-833,
+ * src/models/pi0.cpp:198-201, src/models/pi05.cpp:255-256).  k_src / v_src are
+ * token-major [batch][n_tok][n_kv_heads][head_dim]; they land at tokens
+ * [tok_offset, tok_offset + n_tok) of the cache.  Either pair may be NULL. */
+VLA_KAPI int vla_kv_append(void* k_cache, void* vt_cache, const void* k_src, const void* v_src, int dtype,
+                           int batch, int n_kv_heads, int head_dim, int t_max, int tok_offset, int n_tok,
+                           vla_stream_t stream);
+
+/* Inverse of vla_kv_append: reads tokens [tok_offset, tok_offset + n_tok) back
+ * into token-major buffers (the [D, Hkv, T] tensor the reference's concat
+ * would have produced). */
+VLA_KAPI int vla_kv_gather(const void* k_cache, const void* vt_cache, void* k_dst, void* v_dst, int dtype,
+                           int batch, int n_kv_heads, int head_dim, int t_max, int tok_offset, int n_tok,
+                           vla_stream_t stream);
+
+/* --------------------------------------------------------------- RoPE, norms */
+
+/* Host helper: cos/sin tables [n][head_dim/2] for NeoX RoPE,
+ * theta = pos * base^(-2i/D) evaluated in double and rounded once
+ * (ggml_rope_ext(..., NEOX, base, freq_scale 1, ext_factor 0, attn_factor 1),
+ * src/models/smolvla.cpp:759-766; table form of
+ * src/kernels/bitvla/bitvla_lm_cuda.cu:333-342). */
+VLA_KAPI int vla_rope_tables_host(const int32_t* pos, int n, int head_dim, double base, float* cos_tab,
+                                  float* sin_tab);
+
+/* NeoX rotation in place on a token-major tensor x [n_rows][n_heads][head_dim];
+ * row r uses table row r % table_rows (tables [table_rows][head_dim/2]). */
+VLA_KAPI int vla_rope_neox(void* x, const float* cos_tab, const float* sin_tab, int dtype, int n_rows,
+                           int table_rows, int n_heads, int head_dim, vla_stream_t stream);
+
+/* y = rms_norm(x) * w (src/models/smolvla.cpp:820, src/models/pi0.cpp:170).
+ * x, y [M][K] in `dtype`; w [K] in `dtype` or NULL. */
+VLA_KAPI int vla_rms_norm(const void* x, const void* w, void* y, int dtype, int M, int K, float eps,
+                          vla_stream_t stream);
+
+/* adaLN: y = xn + xn*sc + sh with xn = layer_norm(x) without affine
+ * (src/layers/norm.h:37-46, used by src/modules/dit_head.cpp:111).  sc, sh are
+ * fp32 [K], shared by all rows. */
+VLA_KAPI int vla_adaln(const void* x, const float* sc, const float* sh, void* y, int dtype, int M, int K,
+                       float eps, vla_stream_t stream);
+
+/* ---------------------------------------------------------------- projections */
+
+/* y[M][N] = x[M][K] . W[N][K]^T (+ bias[N], fp32) (+ residual[M][N]), the
+ * ggml_mul_mat shape rule (src/act_dtype.h:62-76; src/layers/linear.h:24-27;
+ * the Wo + residual of src/models/smolvla.cpp:843, src/models/pi0.cpp:224-225).
+ * x, W in `dtype`; residual and y in `out_dtype`; fp32 accumulation. */
+VLA_KAPI int vla_linear(const void* x, const void* W, const float* bias, const void* residual, void* y,
+                        int dtype, int out_dtype, int M, int N, int K, vla_stream_t stream);
+
+/* Fused QKV projection + RoPE + KV append for M = batch*S suffix (or prefix)
+ * rows: replaces mm_w(Wq/Wk/Wv) -> reshape -> rope_q_or_k -> ggml_concat
+ * (src/models/smolvla.cpp:821-833, src/models/pi0.cpp:174-201,
+ * src/modules/dit_head.cpp:113-119).
+ *   W    [n_q_heads*D + nk*D + nv*D][K] rows ordered Q, K, V, where
+ *        nk = has_k ? n_kv_heads : 0 and nv = has_v ? n_kv_heads : 0
+ *   bias fp32 over the same rows, or NULL
+ *   cos/sin [S][D/2] (row m uses m % S) or NULL for no rotation (V is never
+ *        rotated)
+ *   q_out [M][n_q_heads*D] token-major in `dtype` (ignored if n_q_heads == 0)
+ *   K rows go to k_cache, V rows to vt_cache at token tok_offset + (m % S) of
+ *   batch m / S. */
+VLA_KAPI int vla_attn_qkv_rope(const void* x, const void* W, const float* bias, int dtype, int M, int K, int S,
+                               int n_q_heads, int n_kv_heads, int has_k, int has_v, int head_dim,
+                               const float* cos_tab, const float* sin_tab, void* q_out, void* k_cache,
+                               void* vt_cache, int t_max, int tok_offset, vla_stream_t stream);
+
+/* ------------------------------------------------------------------ attention */
+
+/* out = softmax(scale * Q K^T + mask) V over keys [0, n_keys) of the resident
+ * cache, GQA by head-group sharing (q head h reads kv head h / (Hq/Hkv)):
+ * replaces ggml_flash_attn_ext / mul_mat + soft_max_ext + mul_mat
+ * (src/models/smolvla.cpp:835-842, src/models/pi0.cpp:215-223,
+ * src/layers/attn.h:38-58) and the repeat_kv + cuBLAS + softmax sequence of
+ * src/kernels/bitvla/bitvla_lm_cuda.cu:446-486.
+ *   q   [batch][S][n_q_heads][D] token-major, out [batch][S][n_q_heads*D]
+ *   mask: additive fp32 [S][n_keys] shared by heads and batch, or NULL to use
+ *   the generated mask (mask_kind, n_prefix, pad_start, pad_end). */
+VLA_KAPI int vla_attn_prefix_suffix(const void* q, const void* k_cache, const void* vt_cache, void* out,
+                                    int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
+                                    int t_max, int n_keys, float scale, int mask_kind, int n_prefix,
+                                    int pad_start, int pad_end, const float* mask, vla_stream_t stream);
+
+/* --------------------------------------------------------- flow-matching glue */
+
+/* Suffix embedding h[b][s][:] for one denoise step (stand-in for
+ * build_embed_suffix, src/models/pi0.cpp:232-247, and the action_emb of
+ * src/models/smolvla.cpp:1398): rows s < n_lead copy lead[b][s][:] (pi0 / DiT
+ * state token); other rows are W_in . x_t[b][s - n_lead] + bias_step.
+ *   x_t fp32 [batch][S - n_lead][A]; W_in fp32 [W][A]; bias_step fp32 [W];
+ *   lead fp32 [batch][n_lead][W] or NULL; h in `out_dtype`. */
+VLA_KAPI int vla_embed_suffix(const float* x_t, const float* W_in, const float* bias_step, const float* lead,
+                              void* h, int out_dtype, int batch, int S, int n_lead, int A, int W,
+                              vla_stream_t stream);
+
+/* Output projection + Euler update (src/models/smolvla.cpp:1416-1418,
+ * src/models/pi0.cpp:577-587): x_t[b][s] += dt * (W_out . hn[b][n_lead + s] + b_out).
+ *   hn [batch][S][W] in `dtype` (already normalised); W_out fp32 [A][W]. */
+VLA_KAPI int vla_euler_step(float* x_t, const void* hn, const float* W_out, const float* b_out, int dtype,
+                            int batch, int S, int n_lead, int A, int W, float dt, vla_stream_t stream);
+
+/* ------------------------------------------------------------ BitVLA ternary */
+
+/* Per-row int8 quantisation (act_quant_kernel,
+ * src/kernels/bitvla/bitnet_kernels.h:465-521): scales[m] = 127 / max(amax, 1e-5).
+ * rowsum[m] = sum_k q[m][k] (int32) feeds the ternary GEMM's code-offset
+ * correction; may be NULL. */
+VLA_KAPI int vla_act_quant_bf16(const uint16_t* in, int8_t* out, float* scales, int32_t* rowsum, int M, int K,
+                                vla_stream_t stream);
+
+/* Ternary weight quantisation on the host (recover_ternary_and_scale,
+ * src/models/bitvla.cpp:430-451). */
+VLA_KAPI int vla_ternary_quant_host(const float* W, int64_t n, int8_t* ternary, float* absmean);
+
+/* Host packers.  The gfx950 layout is [N][K/16] 32-bit words; word (n, w)
+ * holds codes t+2 of k = 16w .. 16w+15 with value b+4j at bits 8b+2j, i.e. the
+ * reference's 16-value slot format (src/models/bitvla.cpp:470-480) in plain
+ * row-major word order instead of the wmma "ladder" order. */
+VLA_KAPI int vla_ternary_pack_host(const int8_t* ternary, int N, int K, uint32_t* packed);
+VLA_KAPI int vla_ternary_repack_ladder_host(const uint8_t* ladder, int N, int K, uint32_t* packed);
+
+/* out[m][n] = bf16(float(acc) / s[m] * ws[n / (N/ws_num)]),
+ * acc = sum_k A[m][k] * t[n][k] exact in int32
+ * (ladder_int8xint2_kernel_m_wide, bitnet_kernels.h:285-409).  acc_out
+ * (int32 [M][N]) receives the raw accumulators when not NULL; out may then be
+ * NULL. */
+VLA_KAPI int vla_ternary_gemm(const int8_t* A, const uint32_t* W_packed, uint16_t* out, int32_t* acc_out,
+                              const float* s, const int32_t* rowsum, const float* ws, int ws_num, int M, int N,
+                              int K, vla_stream_t stream);
+
+/* -------------------------------------- BitVLA layer helpers (same signatures
+ * as src/kernels/bitvla/bitvla_lm_cuda.h:54-155 with hipStream_t / uint16_t) */
+VLA_KAPI int bitvla_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* out, float eps, int M, int K,
+                                 vla_stream_t stream);
+VLA_KAPI int bitvla_rope_neox_bf16(uint16_t* inout, const float* cos_tab, const float* sin_tab, int H, int S,
+                                   int D, vla_stream_t stream);
+VLA_KAPI int bitvla_softmax_scaled_bf16(uint16_t* inout, float scale, int n_rows, int S, vla_stream_t stream);
+VLA_KAPI int bitvla_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out, int N, vla_stream_t stream);
+VLA_KAPI int bitvla_repeat_kv_bf16(const uint16_t* in, uint16_t* out, int n_q, int n_kv, int seq, int hd,
+                                   vla_stream_t stream);
+VLA_KAPI int bitvla_transpose_sNhd_to_NshHd_bf16(const uint16_t* in, uint16_t* out, int S, int N, int hd,
+                                                 vla_stream_t stream);
+VLA_KAPI int bitvla_transpose_NshHd_to_sNhd_bf16(const uint16_t* in, uint16_t* out, int N, int S, int hd,
+                                                 vla_stream_t stream);
+VLA_KAPI int bitvla_gather_rows_bf16(const uint16_t* in, uint16_t* out, const int32_t* row_ids, int n_rows,
+                                     int K, vla_stream_t stream);
+/* bitvla_act_quant_cuda / bitlinear_int8xint2_m / bitlinear_int8xint2
+ * (src/kernels/bitvla/bitnet_kernels.cu:31,76,118) with the reference's exact
+ * argument lists.  B is the gfx950 packed layout (see vla_ternary_pack_host);
+ * the row sums the GEMM needs are computed on the same stream into a buffer
+ * the library owns, so one call at a time per process. */
+VLA_KAPI int bitvla_act_quant(const uint16_t* in, int8_t* out, float* scales, int M, int K, vla_stream_t stream);
+VLA_KAPI int bitlinear_int8xint2_m(int8_t* A, int8_t* B, uint16_t* out, float* s, float* ws, int M, int N, int K,
+                                   vla_stream_t stream);
+VLA_KAPI int bitlinear_int8xint2(int8_t* A, int8_t* B, uint16_t* out, float* s, float* ws, int M, int N, int K,
+                                 vla_stream_t stream);
+
+/* Library identification, for a loader that wants to check what it bound. */
+VLA_KAPI const char* vla_kernels_arch(void); /* "gfx950" */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VLA_KERNELS_H */

@@ -1,0 +1,69 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every declared
+symbol, and its host-only helpers (no GPU needed) agree with the oracle."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from util import declared_symbols, pkg
+
+
+def test_library_exports_every_declared_kernel_symbol():
+    lib = pkg.lib()
+    names = declared_symbols("vla_kernels.h")
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), "libvla.so does not export %s" % n
+    assert set(names) == set(pkg.KERNEL_API), "ctypes table and header disagree"
+    assert lib.vla_kernels_arch() == b"gfx950"
+
+
+def test_rope_tables_host_equals_oracle_tables():
+    lib = pkg.lib()
+    pos = np.int32([0, 1, 49, 241, 290, 866])
+    for D, base in ((64, 10000.0), (256, 10000.0), (128, 500000.0)):
+        c = np.empty((pos.size, D // 2), np.float32)
+        s = np.empty_like(c)
+        assert lib.vla_rope_tables_host(pos.ctypes.data, pos.size, D, base, c.ctypes.data, s.ctypes.data) == 0
+        oc, os_ = orc.rope_tables(pos, D, base)
+        assert np.array_equal(c, oc) and np.array_equal(s, os_)
+    assert lib.vla_rope_tables_host(pos.ctypes.data, pos.size, 63, 1e4, c.ctypes.data, s.ctypes.data) == pkg.VLA_K_ERR_ARG
+
+
+def test_ternary_quant_and_packers_against_oracle():
+    lib = pkg.lib()
+    r = np.random.default_rng(21)
+    N, K = 64, 256
+    W = (r.standard_normal((N, K)) * 0.02).astype(np.float32)
+    t = np.empty((N, K), np.int8)
+    am = ctypes.c_float()
+    assert lib.vla_ternary_quant_host(W.ctypes.data, W.size, t.ctypes.data, ctypes.addressof(am)) == 0
+    ot, oam = orc.weight_quant_ternary(W)
+    assert np.array_equal(t, ot) and np.float32(am.value) == oam
+    # plain packing: word (n, w) decodes (reference decode) to the 16 values k = 16w..16w+15
+    packed = np.empty((N, K // 16), np.uint32)
+    assert lib.vla_ternary_pack_host(t.ctypes.data, N, K, packed.ctypes.data) == 0
+    for n, w in ((0, 0), (5, 3), (63, 15)):
+        assert np.array_equal(orc.decode_i2s_to_i8s(packed[n, w]), t[n, 16 * w:16 * w + 16])
+    # ladder -> plain repack is a word permutation that inverts the reference's swizzle
+    ladder = orc.pack_ladder_int2(t)
+    rep = np.empty_like(packed)
+    assert lib.vla_ternary_repack_ladder_host(ladder.ctypes.data, N, K, rep.ctypes.data) == 0
+    assert np.array_equal(rep, packed)
+    # raw ladder bytes (code 0 -> -2 allowed) survive the repack too
+    raw = r.integers(0, 256, N * K // 4).astype(np.uint8)
+    assert lib.vla_ternary_repack_ladder_host(raw.ctypes.data, N, K, rep.ctypes.data) == 0
+    U = orc.unpack_ladder_int2(raw, N, K)
+    dec = np.stack([[orc.decode_i2s_to_i8s(rep[n, w]) for w in range(K // 16)] for n in range(N)]).reshape(N, K)
+    assert np.array_equal(dec, U)
+    assert lib.vla_ternary_repack_ladder_host(raw.ctypes.data, 24, K, rep.ctypes.data) == pkg.VLA_K_ERR_SHAPE
+
+
+def test_null_and_shape_errors_are_reported_not_fatal():
+    lib = pkg.lib()
+    assert lib.vla_kv_append(None, None, None, None, 0, 1, 0, 64, 64, 0, 1, None) == pkg.VLA_K_ERR_ARG
+    assert lib.vla_rope_neox(None, None, None, 0, 1, 1, 1, 64, None) == pkg.VLA_K_ERR_ARG
+    assert lib.vla_linear(None, None, None, None, None, 0, 0, 1, 1, 4, None) == pkg.VLA_K_ERR_ARG
+    assert lib.vla_attn_prefix_suffix(None, None, None, None, 0, 1, 1, 1, 1, 64, 64, 1, 1.0, 0, 0, 0, 0, None, None) == pkg.VLA_K_ERR_ARG
+    assert lib.vla_ternary_gemm(None, None, None, None, None, None, None, 1, 1, 16, 128, None) == pkg.VLA_K_ERR_ARG

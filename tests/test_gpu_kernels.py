@@ -1,0 +1,437 @@
+"""Kernel-level parity on a real MI355X: every C-ABI entry point against the CPU
+oracle on the same seeded inputs.
+
+Bars: bit-exact for copies / integer work (KV append+gather, layout helpers,
+act-quant, ternary int32 accumulators and their bf16 epilogue); fp32 kernels
+within 1e-5 relative (max-abs error over max-abs value); bf16 kernels within
+2e-2 relative / 1e-2 absolute.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as orc
+from conftest import mt19937_raw
+from util import dev, host, pkg, rel_err
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = pkg.VLA_DT_F32, pkg.VLA_DT_BF16
+FP32_TOL = 1e-5
+
+
+def sync():
+    torch.cuda.synchronize()
+
+
+def bf16_close(got, want):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    return bool(np.all(np.abs(got - want) <= 1e-2 + 2e-2 * np.abs(want)))
+
+
+def as_f32(t, dtype):
+    a = host(t)
+    return orc.from_bf16(a.view(np.uint16)) if dtype == BF16 else a
+
+
+def to_dev(a, dtype):
+    return dev(orc.to_bf16(a)) if dtype == BF16 else dev(np.asarray(a, np.float32))
+
+
+def empty(shape, dtype):
+    return torch.zeros(shape, dtype=torch.int16 if dtype == BF16 else torch.float32, device="cuda")
+
+
+# ------------------------------------------------------------------ KV cache
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("B,Hkv,D,P,S", [(1, 5, 64, 241, 50), (3, 1, 256, 816, 51), (2, 32, 48, 296, 0), (2, 5, 128, 512, 7)])
+def test_kv_append_then_gather_is_the_reference_concat(dtype, B, Hkv, D, P, S):
+    r = np.random.default_rng(100 + B + D)
+    npdt = np.uint16 if dtype == BF16 else np.float32
+    mk = lambda n: (r.integers(0, 65536, (B, n, Hkv, D)).astype(np.uint16) if dtype == BF16
+                    else r.standard_normal((B, n, Hkv, D)).astype(np.float32))
+    kp, vp, ks, vs = mk(P), mk(P), mk(S), mk(S)
+    t_max = (P + S + 63) // 64 * 64
+    kc, vc = empty((B, Hkv, t_max, D), dtype), empty((B, Hkv, D, t_max), dtype)
+    pkg.call("vla_kv_append", kc, vc, dev(kp), dev(vp), dtype, B, Hkv, D, t_max, 0, P)
+    # two denoise steps overwrite the same suffix slots; the prefix is untouched
+    junk = mk(S)
+    pkg.call("vla_kv_append", kc, vc, dev(junk), dev(junk), dtype, B, Hkv, D, t_max, P, S)
+    pkg.call("vla_kv_append", kc, vc, dev(ks), dev(vs), dtype, B, Hkv, D, t_max, P, S)
+    kd, vd = empty((B, P + S, Hkv, D), dtype), empty((B, P + S, Hkv, D), dtype)
+    pkg.call("vla_kv_gather", kc, vc, kd, vd, dtype, B, Hkv, D, t_max, 0, P + S)
+    sync()
+    for b in range(B):
+        assert np.array_equal(host(kd, npdt)[b], orc.kv_concat(kp[b], ks[b]))
+        assert np.array_equal(host(vd, npdt)[b], orc.kv_concat(vp[b], vs[b]))
+    # layouts: K [B][Hkv][t][D], V^T [B][Hkv][D][t]
+    assert np.array_equal(host(kc, npdt)[:, :, :P], kp.transpose(0, 2, 1, 3))
+    assert np.array_equal(host(vc, npdt)[:, :, :, :P], vp.transpose(0, 2, 3, 1))
+    lib = pkg.lib()
+    assert lib.vla_kv_append(kc.data_ptr(), vc.data_ptr(), kd.data_ptr(), vd.data_ptr(), dtype, B, Hkv, D, t_max,
+                             t_max - 1, 2, None) == pkg.VLA_K_ERR_SHAPE
+
+
+# --------------------------------------------------------------- RoPE / norms
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_rope_neox(dtype):
+    r = np.random.default_rng(101)
+    B, S, H, D = 2, 50, 15, 64
+    x = r.standard_normal((B * S, H, D)).astype(np.float32)
+    if dtype == BF16:
+        x = orc.round_bf16(x)
+    pos = np.arange(S, dtype=np.int32) + 242
+    c, s = orc.rope_tables(pos, D, 10000.0)
+    xd = to_dev(x, dtype)
+    pkg.call("vla_rope_neox", xd, dev(c), dev(s), dtype, B * S, S, H, D)
+    sync()
+    want = np.concatenate([orc.rope_neox(x[b * S:(b + 1) * S], c, s) for b in range(B)])
+    got = as_f32(xd, dtype)
+    if dtype == F32:
+        assert rel_err(got, want) < 1e-6
+    else:
+        assert np.array_equal(got, orc.round_bf16(want)) or bf16_close(got, want)
+
+
+def test_bitvla_rope_head_major_bf16():
+    r = np.random.default_rng(102)
+    H, S, D = 20, 37, 128
+    x = orc.round_bf16(r.standard_normal((H, S, D)).astype(np.float32))
+    c, s = orc.rope_tables(np.arange(S, dtype=np.int32), D, 500000.0)
+    xd = dev(orc.to_bf16(x))
+    pkg.call("bitvla_rope_neox_bf16", xd, dev(c), dev(s), H, S, D)
+    sync()
+    want = orc.rope_neox(x.transpose(1, 0, 2).copy(), c, s).transpose(1, 0, 2)
+    got = orc.from_bf16(host(xd, np.uint16))
+    assert bf16_close(got, want) and rel_err(got, want) < 8e-3
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("M,K", [(50, 720), (51, 1024), (17, 1536), (3, 2560)])
+def test_rms_norm_and_adaln(dtype, M, K):
+    r = np.random.default_rng(103)
+    x = (r.standard_normal((M, K)) * 2 + 0.5).astype(np.float32)
+    w = (1 + 0.1 * r.standard_normal(K)).astype(np.float32)
+    sc, sh = (0.1 * r.standard_normal(K)).astype(np.float32), (0.1 * r.standard_normal(K)).astype(np.float32)
+    if dtype == BF16:
+        x, w = orc.round_bf16(x), orc.round_bf16(w)
+    y = empty((M, K), dtype)
+    pkg.call("vla_rms_norm", to_dev(x, dtype), to_dev(w, dtype), y, dtype, M, K, 1e-5)
+    y2 = empty((M, K), dtype)
+    pkg.call("vla_adaln", to_dev(x, dtype), dev(sc), dev(sh), y2, dtype, M, K, 1e-5)
+    sync()
+    want, want2 = orc.rms_norm(x, w, 1e-5), orc.adaln(x, sc, sh, 1e-5)
+    if dtype == F32:
+        assert rel_err(host(y), want) < FP32_TOL and rel_err(host(y2), want2) < FP32_TOL
+    else:
+        assert bf16_close(as_f32(y, dtype), want) and bf16_close(as_f32(y2, dtype), want2)
+    if dtype == BF16:  # the BitVLA-named entry point is the same kernel
+        y3 = empty((M, K), dtype)
+        pkg.call("bitvla_rmsnorm_bf16", to_dev(x, dtype), to_dev(w, dtype), y3, 1e-5, M, K)
+        sync()
+        assert np.array_equal(host(y3), host(y))
+
+
+# ---------------------------------------------------------------- projections
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("M,N,K", [(50, 720, 960), (1, 64, 128), (130, 200, 72), (17, 1536, 1536), (64, 32, 720)])
+def test_linear_bias_residual(dtype, M, N, K):
+    r = np.random.default_rng(104 + M)
+    x = r.standard_normal((M, K)).astype(np.float32)
+    W = (0.02 * r.standard_normal((N, K))).astype(np.float32)
+    b = (0.1 * r.standard_normal(N)).astype(np.float32)
+    res = r.standard_normal((M, N)).astype(np.float32)
+    if dtype == BF16:
+        x, W, res = orc.round_bf16(x), orc.round_bf16(W), orc.round_bf16(res)
+    y = empty((M, N), dtype)
+    pkg.call("vla_linear", to_dev(x, dtype), to_dev(W, dtype), dev(b), to_dev(res, dtype), y, dtype, dtype, M, N, K)
+    y0 = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+    pkg.call("vla_linear", to_dev(x, dtype), to_dev(W, dtype), None, None, y0, dtype, F32, M, N, K)
+    sync()
+    want0 = orc.linear(x, W)
+    want = want0 + b + res
+    if dtype == F32:
+        assert rel_err(host(y), want) < FP32_TOL and rel_err(host(y0), want0) < FP32_TOL
+    else:
+        assert rel_err(host(y0), want0) < 1e-5  # fp32 accumulate of exact bf16 products
+        assert bf16_close(as_f32(y, dtype), want)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("name,B,S,Hq,Hkv,D,K,rope,bias,P", [
+    ("smolvla-self", 2, 50, 15, 5, 64, 720, True, False, 241),
+    ("pi0", 1, 51, 8, 1, 256, 1024, True, False, 816),
+    ("dit-self", 2, 17, 32, 32, 48, 1536, False, True, 0),
+    ("bitvla-shape", 1, 7, 20, 5, 128, 256, True, False, 512),
+])
+def test_fused_qkv_rope_append(dtype, name, B, S, Hq, Hkv, D, K, rope, bias, P):
+    r = np.random.default_rng(105)
+    M, N = B * S, (Hq + 2 * Hkv) * D
+    x = r.standard_normal((M, K)).astype(np.float32)
+    W = (0.02 * r.standard_normal((N, K))).astype(np.float32)
+    bvec = (0.1 * r.standard_normal(N)).astype(np.float32) if bias else None
+    if dtype == BF16:
+        x, W = orc.round_bf16(x), orc.round_bf16(W)
+    c, s = orc.rope_tables(np.arange(S, dtype=np.int32) + P + 1, D, 10000.0)
+    t_max = (P + S + 63) // 64 * 64
+    kc, vc = empty((B, Hkv, t_max, D), dtype), empty((B, Hkv, D, t_max), dtype)
+    q = empty((M, Hq * D), dtype)
+    pkg.call("vla_attn_qkv_rope", to_dev(x, dtype), to_dev(W, dtype), None if bvec is None else dev(bvec), dtype, M, K, S,
+             Hq, Hkv, 1, 1, D, dev(c) if rope else None, dev(s) if rope else None, q, kc, vc, t_max, P)
+    kd, vd = empty((B, S, Hkv, D), dtype), empty((B, S, Hkv, D), dtype)
+    pkg.call("vla_kv_gather", kc, vc, kd, vd, dtype, B, Hkv, D, t_max, P, S)
+    sync()
+    y = orc.linear(x, W, bvec)
+    qw = y[:, :Hq * D].reshape(M, Hq, D)
+    kw = y[:, Hq * D:(Hq + Hkv) * D].reshape(M, Hkv, D)
+    vw = y[:, (Hq + Hkv) * D:].reshape(M, Hkv, D)
+    if rope:
+        qw = np.concatenate([orc.rope_neox(qw[b * S:(b + 1) * S], c, s) for b in range(B)])
+        kw = np.concatenate([orc.rope_neox(kw[b * S:(b + 1) * S], c, s) for b in range(B)])
+    gq = as_f32(q, dtype).reshape(M, Hq, D)
+    gk = as_f32(kd, dtype).reshape(M, Hkv, D)
+    gv = as_f32(vd, dtype).reshape(M, Hkv, D)
+    if dtype == F32:
+        assert rel_err(gq, qw) < FP32_TOL and rel_err(gk, kw) < FP32_TOL and rel_err(gv, vw) < FP32_TOL
+    else:
+        assert bf16_close(gq, qw) and bf16_close(gk, kw) and bf16_close(gv, vw)
+        assert rel_err(gq, qw) < 8e-3
+    # the prefix region of the cache was not touched
+    assert not host(kc)[:, :, :P].any() and not host(vc)[:, :, :, :P].any()
+
+
+# ------------------------------------------------------------------ attention
+CASES = [
+    # name, B, S, Hq, Hkv, D, P, mask kind, pad
+    ("smolvla-causal", 2, 50, 15, 5, 64, 241, "causal", (230, 240)),
+    ("smolvla-bidir", 1, 50, 15, 5, 64, 241, "none", (0, 0)),
+    ("smolvla-cross", 2, 50, 15, 5, 64, 241, "cross", (200, 240)),
+    ("pi0", 2, 51, 8, 1, 256, 816, "pi0", (0, 0)),
+    ("gr00t-cross", 3, 17, 32, 32, 48, 296, "cross", (0, 0)),
+    ("gr00t-self", 3, 17, 32, 32, 48, 0, "none", (0, 0)),
+    ("bitvla-decode", 2, 1, 20, 5, 128, 515, "cross", (0, 0)),
+    ("bitvla-prefill", 1, 130, 20, 5, 128, 0, "none", (0, 0)),
+]
+
+
+def _mask(kind, P, S, pad):
+    if kind == "causal":
+        return orc.mask_smolvla_full(P, S, pad[0], pad[1]), pkg.VLA_MASK_CAUSAL_SUFFIX, P + S
+    if kind == "pi0":
+        return orc.mask_pi0_full(P, S), pkg.VLA_MASK_PI0_STATE, P + S
+    if kind == "cross":
+        return orc.mask_smolvla_prefix_only(P, S, pad[0], pad[1]), pkg.VLA_MASK_NONE, P
+    m = np.zeros((S, P + S), np.float32)
+    m[:, pad[0]:pad[1]] = -np.inf
+    return m, pkg.VLA_MASK_NONE, P + S
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_attention_against_oracle(dtype, case):
+    name, B, S, Hq, Hkv, D, P, kind, pad = case
+    if dtype == F32 and D == 256:
+        pytest.skip("fp32 tiles for 256-wide heads are not built (LDS budget); pi0 runs in bf16")
+    r = np.random.default_rng(106)
+    mask, mkind, T = _mask(kind, P, S, pad)
+    t_max = (T + 63) // 64 * 64
+    Q = r.standard_normal((B, S, Hq, D)).astype(np.float32)
+    K = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    V = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    if dtype == BF16:
+        Q, K, V = orc.round_bf16(Q), orc.round_bf16(K), orc.round_bf16(V)
+    # stale cache contents past n_keys must not matter: poison them
+    kc = torch.full((B, Hkv, t_max, D), float("nan"), device="cuda")
+    vc = torch.full((B, Hkv, D, t_max), float("nan"), device="cuda")
+    if dtype == BF16:
+        kc, vc = kc.to(torch.bfloat16).view(torch.int16), vc.to(torch.bfloat16).view(torch.int16)
+    pkg.call("vla_kv_append", kc, vc, to_dev(K, dtype), to_dev(V, dtype), dtype, B, Hkv, D, t_max, 0, T)
+    scale = 1.0 / math.sqrt(D)
+    out = empty((B, S, Hq * D), dtype)
+    pkg.call("vla_attn_prefix_suffix", to_dev(Q, dtype), kc, vc, out, dtype, B, S, Hq, Hkv, D, t_max, T, scale, mkind, P,
+             pad[0], pad[1], None)
+    out_m = empty((B, S, Hq * D), dtype)
+    pkg.call("vla_attn_prefix_suffix", to_dev(Q, dtype), kc, vc, out_m, dtype, B, S, Hq, Hkv, D, t_max, T, scale,
+             pkg.VLA_MASK_NONE, 0, 0, 0, dev(mask))
+    sync()
+    want = np.stack([orc.attention(Q[b], K[b], V[b], mask, scale) for b in range(B)])
+    got, got_m = as_f32(out, dtype), as_f32(out_m, dtype)
+    assert np.isfinite(got).all()
+    if dtype == F32:
+        assert rel_err(got, want) < FP32_TOL, rel_err(got, want)
+        assert rel_err(got_m, want) < FP32_TOL
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+    else:
+        assert bf16_close(got, want) and bf16_close(got_m, want)
+        assert rel_err(got, want) < 1e-2
+    # generated mask and mask-as-data run the same arithmetic
+    assert np.array_equal(host(out), host(out_m))
+
+
+def test_attention_special_cases_fp32():
+    # all-zero Q -> mean of the visible V rows; permuting keys changes nothing
+    r = np.random.default_rng(107)
+    B, S, Hq, Hkv, D, T = 1, 5, 6, 2, 64, 100
+    t_max = 128
+    K = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    V = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    kc, vc = empty((B, Hkv, t_max, D), F32), empty((B, Hkv, D, t_max), F32)
+    pkg.call("vla_kv_append", kc, vc, dev(K), dev(V), F32, B, Hkv, D, t_max, 0, T)
+    out = empty((B, S, Hq * D), F32)
+    pkg.call("vla_attn_prefix_suffix", dev(np.zeros((B, S, Hq, D), np.float32)), kc, vc, out, F32, B, S, Hq, Hkv, D,
+             t_max, T, 0.125, pkg.VLA_MASK_NONE, T, 10, 30, None)
+    sync()
+    keep = [t for t in range(T) if not 10 <= t < 30]
+    got = host(out).reshape(S, Hq, D)
+    for h in range(Hq):
+        assert np.allclose(got[2, h], V[0, keep, h // 3].mean(0), atol=1e-6)
+    Q = r.standard_normal((B, S, Hq, D)).astype(np.float32)
+    perm = r.permutation(T)
+    outs = []
+    for Kx, Vx in ((K, V), (K[:, perm], V[:, perm])):
+        pkg.call("vla_kv_append", kc, vc, dev(Kx), dev(Vx), F32, B, Hkv, D, t_max, 0, T)
+        o = empty((B, S, Hq * D), F32)
+        pkg.call("vla_attn_prefix_suffix", dev(Q), kc, vc, o, F32, B, S, Hq, Hkv, D, t_max, T, 0.125,
+                 pkg.VLA_MASK_NONE, T, 0, 0, None)
+        sync()
+        outs.append(host(o))
+    assert rel_err(outs[1], outs[0]) < FP32_TOL
+
+
+# -------------------------------------------------------------------- ternary
+def test_act_quant_bit_exact():
+    r = np.random.default_rng(108)
+    M, K = 67, 2560
+    x = orc.round_bf16((r.standard_normal((M, K)) * 3).astype(np.float32))
+    x[3] = 0.0  # amax floor
+    x[4, :8] = [127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -127.0, 3.5]
+    x[4, 8:] = 0.0  # scale exactly 1: ties go to even
+    x = orc.round_bf16(x)
+    q = torch.zeros((M, K), dtype=torch.int8, device="cuda")
+    s = torch.zeros(M, dtype=torch.float32, device="cuda")
+    rs = torch.zeros(M, dtype=torch.int32, device="cuda")
+    pkg.call("vla_act_quant_bf16", dev(orc.to_bf16(x)), q, s, rs, M, K)
+    q2 = torch.zeros_like(q)
+    s2 = torch.zeros_like(s)
+    pkg.call("bitvla_act_quant", dev(orc.to_bf16(x)), q2, s2, M, K)
+    sync()
+    wq, ws = orc.act_quant(x)
+    assert np.array_equal(host(q), wq) and np.array_equal(host(s), ws)
+    assert np.array_equal(host(rs), wq.astype(np.int32).sum(1))
+    assert np.array_equal(host(q2), wq) and np.array_equal(host(s2), ws)
+    assert list(wq[4, :8]) == [127, 0, 2, 2, 0, -2, -127, 4]
+
+
+def _pack_plain(t):
+    N, K = t.shape
+    out = np.empty((N, K // 16), np.uint32)
+    assert pkg.lib().vla_ternary_pack_host(t.ctypes.data, N, K, out.ctypes.data) == 0
+    return out
+
+
+@pytest.mark.parametrize("M,N,K,ws_num", [(600, 3840, 2560, 3), (517, 640, 2560, 1), (1, 2560, 2560, 1), (8, 3840, 2560, 6),
+                                          (256, 1152, 1152 + 128, 1)])
+def test_ternary_gemm_accumulators_and_epilogue_bit_exact(M, N, K, ws_num):
+    # Inputs drawn the way the reference's GEMM check draws them
+    # (tests/bitvla_gemm_check.cu:81-88): mt19937(1234 + N + M), A in [-127,127],
+    # raw weight bytes (code 0 -> -2 included), s = 40 + rng%100, ws = 0.01 + 0.001*(rng%50).
+    raw = mt19937_raw(1234 + N + M, M * K + N * K // 4 + M + ws_num)
+    A = ((raw[:M * K] % 255).astype(np.int32) - 127).astype(np.int8).reshape(M, K)
+    ladder = (raw[M * K:M * K + N * K // 4] % 256).astype(np.uint8)
+    s = (40.0 + (raw[M * K + N * K // 4:M * K + N * K // 4 + M] % 100)).astype(np.float32)
+    ws = (0.01 + 0.001 * (raw[-ws_num:] % 50).astype(np.float32)).astype(np.float32)
+    Wt = orc.unpack_ladder_int2(ladder, N, K)
+    packed = np.empty((N, K // 16), np.uint32)
+    assert pkg.lib().vla_ternary_repack_ladder_host(ladder.ctypes.data, N, K, packed.ctypes.data) == 0
+    acc = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+    rowsum = dev(A.astype(np.int32).sum(1).astype(np.int32))
+    pkg.call("vla_ternary_gemm", dev(A), dev(packed), out, acc, dev(s), rowsum, dev(ws), ws_num, M, N, K)
+    sync()
+    want_acc = orc.ternary_gemm_i32(A, Wt)
+    assert np.array_equal(host(acc), want_acc)
+    assert np.array_equal(host(out, np.uint16), orc.ternary_epilogue(want_acc, s, ws))
+    if (N, K, ws_num) in ((3840, 2560, 3), (640, 2560, 1), (2560, 2560, 1)):
+        out2 = torch.zeros_like(out)
+        pkg.call("bitlinear_int8xint2_m", dev(A), dev(packed), out2, dev(s), dev(ws), M, N, K)
+        sync()
+        assert np.array_equal(host(out2), host(out))
+
+
+def test_ternary_pipeline_matches_cpu_twin():
+    # act-quant + ternary GEMM + epilogue against the reference's CPU formulation
+    # (fp32 fake-quant GEMM, src/models/bitvla.cpp:173-176): same number up to bf16 rounding.
+    r = np.random.default_rng(109)
+    M, N, K = 40, 640, 2560
+    x = orc.round_bf16(r.standard_normal((M, K)).astype(np.float32))
+    W = (0.02 * r.standard_normal((N, K))).astype(np.float32)
+    t, am = orc.weight_quant_ternary(W)
+    q = torch.zeros((M, K), dtype=torch.int8, device="cuda")
+    s = torch.zeros(M, dtype=torch.float32, device="cuda")
+    rs = torch.zeros(M, dtype=torch.int32, device="cuda")
+    pkg.call("vla_act_quant_bf16", dev(orc.to_bf16(x)), q, s, rs, M, K)
+    out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+    pkg.call("vla_ternary_gemm", q, dev(_pack_plain(t)), out, None, s, rs, dev(np.float32([am])), 1, M, N, K)
+    sync()
+    want = orc.bit_linear_f32(x, t, am)
+    got = orc.from_bf16(host(out, np.uint16))
+    assert bf16_close(got, want) and rel_err(got, want) < 5e-3
+
+
+# ------------------------------------------------------- BitVLA layer helpers
+def test_bitvla_layout_helpers_and_softmax():
+    r = np.random.default_rng(110)
+    S, H, hd, n_kv = 37, 20, 128, 5
+    x = r.integers(0, 65536, (S, H * hd)).astype(np.uint16)
+    t = torch.zeros((H, S, hd), dtype=torch.int16, device="cuda")
+    pkg.call("bitvla_transpose_sNhd_to_NshHd_bf16", dev(x), t, S, H, hd)
+    back = torch.zeros((S, H * hd), dtype=torch.int16, device="cuda")
+    pkg.call("bitvla_transpose_NshHd_to_sNhd_bf16", t, back, H, S, hd)
+    rep = torch.zeros((H, S, hd), dtype=torch.int16, device="cuda")
+    pkg.call("bitvla_repeat_kv_bf16", t[:n_kv].contiguous(), rep, H, n_kv, S, hd)
+    ids = np.int32([5, 5, 0, 36])
+    gat = torch.zeros((4, H * hd), dtype=torch.int16, device="cuda")
+    pkg.call("bitvla_gather_rows_bf16", dev(x), gat, dev(ids), 4, H * hd)
+    sync()
+    want_t = orc.transpose_sHd_to_Hsd(x, H)
+    assert np.array_equal(host(t, np.uint16), want_t)
+    assert np.array_equal(host(back, np.uint16), x)
+    assert np.array_equal(host(rep, np.uint16), orc.repeat_kv(want_t[:n_kv], H))
+    assert np.array_equal(host(gat, np.uint16), orc.gather_rows(x, ids))
+    sc = orc.to_bf16((r.standard_normal((40, 519)) * 8).astype(np.float32))
+    sd = dev(sc)
+    pkg.call("bitvla_softmax_scaled_bf16", sd, 0.0883883, 40, 519)
+    a, b = dev(orc.to_bf16(r.standard_normal(1000).astype(np.float32))), dev(orc.to_bf16(r.standard_normal(1000).astype(np.float32)))
+    c = torch.zeros(1000, dtype=torch.int16, device="cuda")
+    pkg.call("bitvla_add_bf16", a, b, c, 1000)
+    sync()
+    want = orc.from_bf16(orc.softmax_scaled_bf16(sc, 0.0883883))
+    got = orc.from_bf16(host(sd, np.uint16))
+    assert np.abs(got - want).max() <= 2 ** -8 * max(want.max(), 1e-3)
+    assert np.array_equal(host(c, np.uint16), orc.to_bf16(orc.from_bf16(host(a, np.uint16)) + orc.from_bf16(host(b, np.uint16))))
+
+
+# ---------------------------------------------------------- flow-matching glue
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_embed_suffix_and_euler_step(out_dtype):
+    r = np.random.default_rng(111)
+    B, S, n_lead, A, W = 3, 51, 1, 32, 1024
+    x_t = r.standard_normal((B, S - n_lead, A)).astype(np.float32)
+    W_in = (0.1 * r.standard_normal((W, A))).astype(np.float32)
+    bias = r.standard_normal(W).astype(np.float32)
+    lead = r.standard_normal((B, n_lead, W)).astype(np.float32)
+    h = empty((B, S, W), out_dtype)
+    pkg.call("vla_embed_suffix", dev(x_t), dev(W_in), dev(bias), dev(lead), h, out_dtype, B, S, n_lead, A, W)
+    sync()
+    want = np.concatenate([lead, (orc.linear(x_t.reshape(-1, A), W_in, bias)).reshape(B, S - n_lead, W)], axis=1)
+    got = as_f32(h, out_dtype)
+    assert rel_err(got, want) < (FP32_TOL if out_dtype == F32 else 8e-3)
+    W_out = (0.05 * r.standard_normal((A, W))).astype(np.float32)
+    b_out = r.standard_normal(A).astype(np.float32)
+    xd = dev(x_t)
+    pkg.call("vla_euler_step", xd, h, dev(W_out), dev(b_out), out_dtype, B, S, n_lead, A, W, -0.1)
+    sync()
+    v = orc.linear(got[:, n_lead:].reshape(-1, W), W_out, b_out).reshape(B, S - n_lead, A)
+    assert rel_err(host(xd), x_t - 0.1 * v) < FP32_TOL

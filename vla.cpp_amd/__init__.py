@@ -1,0 +1,102 @@
+"""MI355X-native action-expert attention path: loader for ``libvla.so``.
+
+The product is the C-ABI shared library built from ``csrc/`` (HIP kernels) and
+``host/`` (C++ host layer); this module only locates it, declares the ctypes
+signatures of ``include/vla_kernels.h`` / ``include/vla.h`` and offers thin
+helpers that pass torch device pointers through.  There is no fallback: if the
+library is missing, loading raises.
+
+The directory name is not a Python identifier, so import it through
+``load_package()`` in ``__graft_entry__`` (module name ``vla_cpp_amd``).
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libvla.so")
+
+VLA_DT_F32, VLA_DT_BF16 = 0, 1
+VLA_MASK_NONE, VLA_MASK_CAUSAL_SUFFIX, VLA_MASK_PI0_STATE = 0, 1, 2
+VLA_K_OK, VLA_K_ERR_ARG, VLA_K_ERR_SHAPE, VLA_K_ERR_LAUNCH = 0, -1, -2, -3
+
+_lib = None
+
+_vp, _i, _f, _d, _i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_double, ctypes.c_int64
+
+# name -> argtypes (restype int unless listed in _RESTYPES)
+KERNEL_API = {
+    "vla_kv_append": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "vla_kv_gather": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "vla_rope_tables_host": [_vp, _i, _i, _d, _vp, _vp],
+    "vla_rope_neox": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "vla_rms_norm": [_vp, _vp, _vp, _i, _i, _i, _f, _vp],
+    "vla_adaln": [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _vp],
+    "vla_linear": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "vla_attn_qkv_rope": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    "vla_attn_prefix_suffix": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp],
+    "vla_embed_suffix": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "vla_euler_step": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
+    "vla_act_quant_bf16": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+    "vla_ternary_quant_host": [_vp, _i64, _vp, _vp],
+    "vla_ternary_pack_host": [_vp, _i, _i, _vp],
+    "vla_ternary_repack_ladder_host": [_vp, _i, _i, _vp],
+    "vla_ternary_gemm": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "bitvla_rmsnorm_bf16": [_vp, _vp, _vp, _f, _i, _i, _vp],
+    "bitvla_rope_neox_bf16": [_vp, _vp, _vp, _i, _i, _i, _vp],
+    "bitvla_softmax_scaled_bf16": [_vp, _f, _i, _i, _vp],
+    "bitvla_add_bf16": [_vp, _vp, _vp, _i, _vp],
+    "bitvla_repeat_kv_bf16": [_vp, _vp, _i, _i, _i, _i, _vp],
+    "bitvla_transpose_sNhd_to_NshHd_bf16": [_vp, _vp, _i, _i, _i, _vp],
+    "bitvla_transpose_NshHd_to_sNhd_bf16": [_vp, _vp, _i, _i, _i, _vp],
+    "bitvla_gather_rows_bf16": [_vp, _vp, _vp, _i, _i, _vp],
+    "bitvla_act_quant": [_vp, _vp, _vp, _i, _i, _vp],
+    "bitlinear_int8xint2_m": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "bitlinear_int8xint2": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "vla_kernels_arch": [],
+}
+_RESTYPES = {"vla_kernels_arch": ctypes.c_char_p}
+
+
+def lib():
+    """The loaded C-ABI library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                "libvla.so is missing (%s): build it with __graft_entry__.build(); there is no CPU fallback" % LIB_PATH)
+        _lib = ctypes.CDLL(LIB_PATH)
+        for name, argtypes in KERNEL_API.items():
+            fn = getattr(_lib, name)
+            fn.argtypes = argtypes
+            fn.restype = _RESTYPES.get(name, ctypes.c_int)
+    return _lib
+
+
+def ptr(t):
+    """Device (or host) address of a torch tensor / numpy array, or None."""
+    if t is None:
+        return None
+    if hasattr(t, "data_ptr"):
+        assert t.is_contiguous(), "kernels take contiguous buffers"
+        return t.data_ptr()
+    return t.ctypes.data
+
+
+def stream():
+    """The current torch HIP stream as a hipStream_t value."""
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def check(rc, what=""):
+    if rc != VLA_K_OK:
+        raise RuntimeError("%s failed with vla_kstatus %d" % (what or "kernel call", rc))
+
+
+def call(name, *args):
+    """Call a kernel entry point, translating tensors to pointers and appending the current stream."""
+    fn = getattr(lib(), name)
+    conv = [ptr(a) if (a is None or hasattr(a, "data_ptr") or hasattr(a, "ctypes")) else a for a in args]
+    rc = fn(*conv, stream())
+    check(rc, name)
+    return rc

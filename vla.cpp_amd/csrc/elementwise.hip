@@ -1,0 +1,390 @@
+// Row-wise and element-wise kernels around the attention path: NeoX RoPE,
+// RMSNorm / adaLN pre-norms, the flow-matching embed / Euler glue, and the
+// BitVLA layer helpers whose signatures follow
+// src/kernels/bitvla/bitvla_lm_cuda.h:54-155.  All are HBM / latency bound;
+// each row is handled by one workgroup with 64-lane shuffle reductions.
+
+#include <math.h>
+
+#include "common.h"
+#include "vla_kernels.h"
+
+namespace {
+
+using namespace vk;
+
+#define VLA_CHECK_LAUNCH() (hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH)
+
+// ------------------------------------------------------------------ RoPE ---
+// x [n_rows][H][D]; one thread per rotation pair.  (a, b) = (x[i], x[i + D/2])
+// -> (a c - b s, b c + a s), computed in fp32.
+template <typename T>
+__global__ void rope_neox_kernel(T* __restrict__ x, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+                                 int table_rows, int H, int D, long total_pairs) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total_pairs) return;
+    const int half = D >> 1;
+    const int p = (int)(i % half);
+    const long rh = i / half;  // row * H + head
+    const int row = (int)(rh / H);
+    const int tr = row % table_rows;
+    const float c = cos_t[(long)tr * half + p], s = sin_t[(long)tr * half + p];
+    T* base = x + rh * D;
+    const float a = Elem<T>::load(base + p), b = Elem<T>::load(base + p + half);
+    Elem<T>::store(base + p, a * c - b * s);
+    Elem<T>::store(base + p + half, b * c + a * s);
+}
+
+// Head-major variant of the BitVLA layer: inout [H][S][D], tables [S][D/2].
+__global__ void rope_neox_hsd_bf16_kernel(bf16_t* __restrict__ x, const float* __restrict__ cos_t,
+                                          const float* __restrict__ sin_t, int S, int D, long total_pairs) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total_pairs) return;
+    const int half = D >> 1;
+    const int p = (int)(i % half);
+    const long hs = i / half;  // head * S + s
+    const int s_idx = (int)(hs % S);
+    const float c = cos_t[(long)s_idx * half + p], s = sin_t[(long)s_idx * half + p];
+    bf16_t* base = x + hs * D;
+    const float a = bf2f(base[p]), b = bf2f(base[p + half]);
+    base[p] = f2bf(a * c - b * s);
+    base[p + half] = f2bf(b * c + a * s);
+}
+
+// ----------------------------------------------------------------- norms ---
+template <typename T>
+__global__ void rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y, int K, float eps) {
+    __shared__ float red[16];
+    const T* xr = x + (long)blockIdx.x * K;
+    T* yr = y + (long)blockIdx.x * K;
+    float ss = 0.f;
+    for (int k = threadIdx.x; k < K; k += blockDim.x) {
+        const float v = Elem<T>::load(xr + k);
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)K + eps);
+    for (int k = threadIdx.x; k < K; k += blockDim.x) {
+        float v = Elem<T>::load(xr + k) * scale;
+        if (w) v *= Elem<T>::load(w + k);
+        Elem<T>::store(yr + k, v);
+    }
+}
+
+template <typename T>
+__global__ void adaln_kernel(const T* __restrict__ x, const float* __restrict__ sc, const float* __restrict__ sh,
+                             T* __restrict__ y, int K, float eps) {
+    __shared__ float red[16];
+    const T* xr = x + (long)blockIdx.x * K;
+    T* yr = y + (long)blockIdx.x * K;
+    float s1 = 0.f;
+    for (int k = threadIdx.x; k < K; k += blockDim.x) s1 += Elem<T>::load(xr + k);
+    const float mean = block_sum(s1, red) / (float)K;
+    float s2 = 0.f;
+    for (int k = threadIdx.x; k < K; k += blockDim.x) {
+        const float d = Elem<T>::load(xr + k) - mean;
+        s2 += d * d;
+    }
+    const float inv = 1.0f / sqrtf(block_sum(s2, red) / (float)K + eps);
+    for (int k = threadIdx.x; k < K; k += blockDim.x) {
+        const float xn = (Elem<T>::load(xr + k) - mean) * inv;
+        Elem<T>::store(yr + k, xn + xn * sc[k] + sh[k]);
+    }
+}
+
+// ------------------------------------------------- flow-matching glue ---
+// grid (batch*S), block covers W columns; A (the action width) is small, so
+// each thread does its own dot product.
+template <typename T>
+__global__ void embed_suffix_kernel(const float* __restrict__ x_t, const float* __restrict__ W_in,
+                                    const float* __restrict__ bias_step, const float* __restrict__ lead,
+                                    T* __restrict__ h, int S, int n_lead, int A, int W) {
+    const int row = blockIdx.x, b = row / S, s = row % S;
+    T* hr = h + (long)row * W;
+    if (s < n_lead) {
+        const float* lr = lead + ((long)b * n_lead + s) * W;
+        for (int c = threadIdx.x; c < W; c += blockDim.x) Elem<T>::store(hr + c, lr[c]);
+        return;
+    }
+    const float* xr = x_t + ((long)b * (S - n_lead) + (s - n_lead)) * A;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+        const float* wr = W_in + (long)c * A;
+        float acc = 0.f;
+        for (int a = 0; a < A; ++a) acc += wr[a] * xr[a];
+        Elem<T>::store(hr + c, acc + bias_step[c]);
+    }
+}
+
+// grid (batch*(S - n_lead)), one wavefront per output column group.
+template <typename T>
+__global__ void euler_step_kernel(float* __restrict__ x_t, const T* __restrict__ hn, const float* __restrict__ W_out,
+                                  const float* __restrict__ b_out, int S, int n_lead, int A, int W, float dt) {
+    const int Sa = S - n_lead;
+    const int b = blockIdx.x / Sa, s = blockIdx.x % Sa;
+    const T* hr = hn + ((long)b * S + n_lead + s) * W;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    for (int a = wave; a < A; a += nw) {
+        const float* wr = W_out + (long)a * W;
+        float acc = 0.f;
+        for (int k = lane; k < W; k += 64) acc += wr[k] * Elem<T>::load(hr + k);
+        acc = wave_sum(acc);
+        if (lane == 0) {
+            float* xp = x_t + ((long)b * Sa + s) * A + a;
+            *xp = *xp + dt * (acc + (b_out ? b_out[a] : 0.f));
+        }
+    }
+}
+
+// ------------------------------------------------ BitVLA layer helpers ---
+// bitvla_softmax_scaled_bf16 (bitvla_lm_cuda.cu:100-159): in-place, no mask.
+__global__ void softmax_scaled_bf16_kernel(bf16_t* __restrict__ inout, float scale, int S) {
+    __shared__ float red[16];
+    bf16_t* r = inout + (long)blockIdx.x * S;
+    float mx = -INFINITY;
+    for (int i = threadIdx.x; i < S; i += blockDim.x) mx = fmaxf(mx, bf2f(r[i]) * scale);
+    mx = block_max(mx, red);
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < S; i += blockDim.x) sum += expf(bf2f(r[i]) * scale - mx);
+    sum = block_sum(sum, red);
+    const float inv = 1.0f / sum;
+    for (int i = threadIdx.x; i < S; i += blockDim.x) r[i] = f2bf(expf(bf2f(r[i]) * scale - mx) * inv);
+}
+
+__global__ void add_bf16_kernel(const bf16_t* a, const bf16_t* b, bf16_t* out, int N) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < N) out[i] = f2bf(bf2f(a[i]) + bf2f(b[i]));
+}
+
+// Generic 3-level permuting copy of rows of `hd` elements:
+// out[(o0*n1 + o1)*hd + k] = in[(i0*s0 + i1)*hd + k] with per-kernel index maps.
+enum { MAP_REPEAT_KV = 0, MAP_SHD_TO_HSD = 1, MAP_HSD_TO_SHD = 2 };
+template <int kMap>
+__global__ void row_permute_bf16_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, int a, int b, int c,
+                                        int hd) {
+    // grid (x, y); meaning depends on kMap (mirrors the reference's launches)
+    const int x = blockIdx.x, y = blockIdx.y;
+    long src, dst;
+    if (kMap == MAP_REPEAT_KV) {  // a=n_q, b=n_kv, c=seq; x=q_h, y=s
+        const int kv_h = x * b / a;
+        dst = ((long)x * c + y) * hd;
+        src = ((long)kv_h * c + y) * hd;
+    } else if (kMap == MAP_SHD_TO_HSD) {  // a=S, b=H; x=h, y=s
+        dst = ((long)x * a + y) * hd;
+        src = ((long)y * b + x) * hd;
+    } else {  // MAP_HSD_TO_SHD: a=H, b=S; x=h, y=s
+        dst = ((long)y * a + x) * hd;
+        src = ((long)x * b + y) * hd;
+    }
+    for (int k = threadIdx.x; k < hd; k += blockDim.x) out[dst + k] = in[src + k];
+}
+
+__global__ void gather_rows_bf16_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out,
+                                        const int32_t* __restrict__ ids, int K) {
+    const long r = ids[blockIdx.x];
+    for (int k = threadIdx.x; k < K; k += blockDim.x) out[(long)blockIdx.x * K + k] = in[r * K + k];
+}
+
+// --------------------------------------------------------- act quant ---
+// act_quant_kernel (bitnet_kernels.h:465-521) plus the per-row sum of the
+// quantised values.  One workgroup per row.
+__global__ void act_quant_bf16_kernel(const bf16_t* __restrict__ in, int8_t* __restrict__ out,
+                                      float* __restrict__ scales, int32_t* __restrict__ rowsum, int K) {
+    __shared__ float red[16];
+    __shared__ int redi[16];
+    const bf16_t* xr = in + (long)blockIdx.x * K;
+    int8_t* qr = out + (long)blockIdx.x * K;
+    float amax = 0.f;
+    for (int k = threadIdx.x; k < K; k += blockDim.x) amax = fmaxf(amax, fabsf(bf2f(xr[k])));
+    amax = block_max(amax, red);
+    if (amax < 1e-5f) amax = 1e-5f;
+    const float scale = 127.0f / amax;
+    int sum = 0;
+    for (int k = threadIdx.x; k < K; k += blockDim.x) {
+        float q = rintf(bf2f(xr[k]) * scale);
+        q = fminf(fmaxf(q, -128.0f), 127.0f);
+        const int qi = (int)q;
+        qr[k] = (int8_t)qi;
+        sum += qi;
+    }
+    sum = wave_sum_i(sum);
+    const int w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    if ((threadIdx.x & 63) == 0) redi[w] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int t = 0;
+        for (int i = 0; i < nw; ++i) t += redi[i];
+        scales[blockIdx.x] = scale;
+        if (rowsum) rowsum[blockIdx.x] = t;
+    }
+}
+
+inline int row_threads(int K) { return K >= 2048 ? 256 : (K >= 512 ? 128 : 64); }
+
+}  // namespace
+
+extern "C" {
+
+int vla_rope_tables_host(const int32_t* pos, int n, int head_dim, double base, float* cos_tab, float* sin_tab) {
+    if (!pos || !cos_tab || !sin_tab || n < 0 || head_dim <= 0 || (head_dim & 1)) return VLA_K_ERR_ARG;
+    const int half = head_dim / 2;
+    for (int s = 0; s < n; ++s)
+        for (int i = 0; i < half; ++i) {
+            const double ang = (double)pos[s] * pow(base, -2.0 * (double)i / (double)head_dim);
+            cos_tab[(size_t)s * half + i] = (float)cos(ang);
+            sin_tab[(size_t)s * half + i] = (float)sin(ang);
+        }
+    return VLA_K_OK;
+}
+
+int vla_rope_neox(void* x, const float* cos_tab, const float* sin_tab, int dtype, int n_rows, int table_rows,
+                  int n_heads, int head_dim, vla_stream_t stream) {
+    if (!x || !cos_tab || !sin_tab || n_rows < 0 || table_rows <= 0 || n_heads <= 0) return VLA_K_ERR_ARG;
+    if (head_dim <= 0 || (head_dim & 1)) return VLA_K_ERR_SHAPE;
+    const long total = (long)n_rows * n_heads * (head_dim / 2);
+    if (total == 0) return VLA_K_OK;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == VLA_DT_F32)
+        rope_neox_kernel<float><<<blocks, 256, 0, st>>>((float*)x, cos_tab, sin_tab, table_rows, n_heads, head_dim, total);
+    else if (dtype == VLA_DT_BF16)
+        rope_neox_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)x, cos_tab, sin_tab, table_rows, n_heads, head_dim, total);
+    else
+        return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_rms_norm(const void* x, const void* w, void* y, int dtype, int M, int K, float eps, vla_stream_t stream) {
+    if (!x || !y || M < 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (M == 0) return VLA_K_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int th = row_threads(K);
+    if (dtype == VLA_DT_F32)
+        rms_norm_kernel<float><<<M, th, 0, st>>>((const float*)x, (const float*)w, (float*)y, K, eps);
+    else if (dtype == VLA_DT_BF16)
+        rms_norm_kernel<bf16_t><<<M, th, 0, st>>>((const bf16_t*)x, (const bf16_t*)w, (bf16_t*)y, K, eps);
+    else
+        return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_adaln(const void* x, const float* sc, const float* sh, void* y, int dtype, int M, int K, float eps,
+              vla_stream_t stream) {
+    if (!x || !y || !sc || !sh || M < 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (M == 0) return VLA_K_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int th = row_threads(K);
+    if (dtype == VLA_DT_F32)
+        adaln_kernel<float><<<M, th, 0, st>>>((const float*)x, sc, sh, (float*)y, K, eps);
+    else if (dtype == VLA_DT_BF16)
+        adaln_kernel<bf16_t><<<M, th, 0, st>>>((const bf16_t*)x, sc, sh, (bf16_t*)y, K, eps);
+    else
+        return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_embed_suffix(const float* x_t, const float* W_in, const float* bias_step, const float* lead, void* h,
+                     int out_dtype, int batch, int S, int n_lead, int A, int W, vla_stream_t stream) {
+    if (!x_t || !W_in || !bias_step || !h || batch < 0 || S <= 0 || n_lead < 0 || n_lead > S || A <= 0 || W <= 0)
+        return VLA_K_ERR_ARG;
+    if (n_lead > 0 && !lead) return VLA_K_ERR_ARG;
+    if (batch == 0) return VLA_K_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (out_dtype == VLA_DT_F32)
+        embed_suffix_kernel<float><<<batch * S, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, S, n_lead, A, W);
+    else if (out_dtype == VLA_DT_BF16)
+        embed_suffix_kernel<bf16_t><<<batch * S, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, S, n_lead, A, W);
+    else
+        return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_euler_step(float* x_t, const void* hn, const float* W_out, const float* b_out, int dtype, int batch, int S,
+                   int n_lead, int A, int W, float dt, vla_stream_t stream) {
+    if (!x_t || !hn || !W_out || batch < 0 || S <= 0 || n_lead < 0 || n_lead >= S || A <= 0 || W <= 0)
+        return VLA_K_ERR_ARG;
+    if (batch == 0) return VLA_K_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int blocks = batch * (S - n_lead);
+    if (dtype == VLA_DT_F32)
+        euler_step_kernel<float><<<blocks, 256, 0, st>>>(x_t, (const float*)hn, W_out, b_out, S, n_lead, A, W, dt);
+    else if (dtype == VLA_DT_BF16)
+        euler_step_kernel<bf16_t><<<blocks, 256, 0, st>>>(x_t, (const bf16_t*)hn, W_out, b_out, S, n_lead, A, W, dt);
+    else
+        return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_act_quant_bf16(const uint16_t* in, int8_t* out, float* scales, int32_t* rowsum, int M, int K,
+                       vla_stream_t stream) {
+    if (!in || !out || !scales || M < 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (M == 0) return VLA_K_OK;
+    act_quant_bf16_kernel<<<M, 256, 0, (hipStream_t)stream>>>(in, out, scales, rowsum, K);
+    return VLA_CHECK_LAUNCH();
+}
+
+int bitvla_act_quant(const uint16_t* in, int8_t* out, float* scales, int M, int K, vla_stream_t stream) {
+    return vla_act_quant_bf16(in, out, scales, nullptr, M, K, stream);
+}
+
+int bitvla_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* out, float eps, int M, int K,
+                        vla_stream_t stream) {
+    return vla_rms_norm(x, w, out, VLA_DT_BF16, M, K, eps, stream);
+}
+
+int bitvla_rope_neox_bf16(uint16_t* inout, const float* cos_tab, const float* sin_tab, int H, int S, int D,
+                          vla_stream_t stream) {
+    if (!inout || !cos_tab || !sin_tab || H < 0 || S < 0 || D <= 0 || (D & 1)) return VLA_K_ERR_ARG;
+    const long total = (long)H * S * (D / 2);
+    if (total == 0) return VLA_K_OK;
+    rope_neox_hsd_bf16_kernel<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(inout, cos_tab,
+                                                                                               sin_tab, S, D, total);
+    return VLA_CHECK_LAUNCH();
+}
+
+int bitvla_softmax_scaled_bf16(uint16_t* inout, float scale, int n_rows, int S, vla_stream_t stream) {
+    if (!inout || n_rows < 0 || S <= 0) return VLA_K_ERR_ARG;
+    if (n_rows == 0) return VLA_K_OK;
+    softmax_scaled_bf16_kernel<<<n_rows, 256, 0, (hipStream_t)stream>>>(inout, scale, S);
+    return VLA_CHECK_LAUNCH();
+}
+
+int bitvla_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out, int N, vla_stream_t stream) {
+    if (!a || !b || !out || N < 0) return VLA_K_ERR_ARG;
+    if (N == 0) return VLA_K_OK;
+    add_bf16_kernel<<<(N + 255) / 256, 256, 0, (hipStream_t)stream>>>(a, b, out, N);
+    return VLA_CHECK_LAUNCH();
+}
+
+int bitvla_repeat_kv_bf16(const uint16_t* in, uint16_t* out, int n_q, int n_kv, int seq, int hd, vla_stream_t stream) {
+    if (!in || !out || n_q <= 0 || n_kv <= 0 || seq < 0 || hd <= 0) return VLA_K_ERR_ARG;
+    if (n_q % n_kv != 0) return VLA_K_ERR_SHAPE;
+    if (seq == 0) return VLA_K_OK;
+    row_permute_bf16_kernel<MAP_REPEAT_KV><<<dim3(n_q, seq), 64, 0, (hipStream_t)stream>>>(in, out, n_q, n_kv, seq, hd);
+    return VLA_CHECK_LAUNCH();
+}
+
+int bitvla_transpose_sNhd_to_NshHd_bf16(const uint16_t* in, uint16_t* out, int S, int N, int hd, vla_stream_t stream) {
+    if (!in || !out || S < 0 || N <= 0 || hd <= 0) return VLA_K_ERR_ARG;
+    if (S == 0) return VLA_K_OK;
+    row_permute_bf16_kernel<MAP_SHD_TO_HSD><<<dim3(N, S), 64, 0, (hipStream_t)stream>>>(in, out, S, N, 0, hd);
+    return VLA_CHECK_LAUNCH();
+}
+
+int bitvla_transpose_NshHd_to_sNhd_bf16(const uint16_t* in, uint16_t* out, int N, int S, int hd, vla_stream_t stream) {
+    if (!in || !out || S < 0 || N <= 0 || hd <= 0) return VLA_K_ERR_ARG;
+    if (S == 0) return VLA_K_OK;
+    row_permute_bf16_kernel<MAP_HSD_TO_SHD><<<dim3(N, S), 64, 0, (hipStream_t)stream>>>(in, out, N, S, 0, hd);
+    return VLA_CHECK_LAUNCH();
+}
+
+int bitvla_gather_rows_bf16(const uint16_t* in, uint16_t* out, const int32_t* row_ids, int n_rows, int K,
+                            vla_stream_t stream) {
+    if (!in || !out || !row_ids || n_rows < 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (n_rows == 0) return VLA_K_OK;
+    gather_rows_bf16_kernel<<<n_rows, 128, 0, (hipStream_t)stream>>>(in, out, row_ids, K);
+    return VLA_CHECK_LAUNCH();
+}
+
+const char* vla_kernels_arch(void) { return "gfx950"; }
+
+}  // extern "C"
