@@ -92,6 +92,11 @@ template <> struct Traits<int8_t> {
     }
 };
 
+// Accumulator element -> raw 32-bit LDS cell (by value: a bit_cast applied
+// directly to a vector element expression reads element 0).
+__device__ __forceinline__ uint32_t acc_bits(float v) { return __float_as_uint(v); }
+__device__ __forceinline__ uint32_t acc_bits(int v) { return (uint32_t)v; }
+
 // W-row bases of the two 32-column halves of output tile `nt`.
 struct TileCols {
     int base0, base1;  // rows of W feeding tile columns [0,32) and [32,64)
@@ -246,7 +251,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
         for (int i = 0; i < 4; ++i) {
             const int row = wm * 32 + 8 * j + 4 * g + i;
             const int col = wn * 32 + r;
-            C[row * C_STRIDE + col] = __builtin_bit_cast(uint32_t, acc[4 * j + i]);
+            C[row * C_STRIDE + col] = acc_bits(acc[4 * j + i]);
         }
     __syncthreads();
 
