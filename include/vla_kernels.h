@@ -122,6 +122,14 @@ VLA_KAPI int vla_attn_qkv_rope(const void* x, const void* W, const float* bias, 
                                const float* cos_tab, const float* sin_tab, void* q_out, void* k_cache,
                                void* vt_cache, int t_max, int tok_offset, vla_stream_t stream);
 
+/* Unfused tail of the same step for a projection that already exists as a
+ * [M][(n_q_heads + 2 n_kv_heads) * D] matrix (the BitVLA ternary GEMM output,
+ * src/kernels/bitvla/bitvla_lm_cuda.cu:428-446: transposes, RoPE on Q and K,
+ * then K/V into the cache instead of repeat_kv). */
+VLA_KAPI int vla_qkv_split_rope_append(const void* qkv, const float* cos_tab, const float* sin_tab, void* q_out,
+                                       void* k_cache, void* vt_cache, int dtype, int M, int S, int n_q_heads,
+                                       int n_kv_heads, int head_dim, int t_max, int tok_offset, vla_stream_t stream);
+
 /* ------------------------------------------------------------------ attention */
 
 /* out = softmax(scale * Q K^T + mask) V over keys [0, n_keys) of the resident

@@ -1,0 +1,273 @@
+"""Whole-chunk CPU oracle (TEST INFRASTRUCTURE ONLY): the reference's op sequence
+for one observation, composed from the primitives of oracle.cpp.
+
+It keeps what the reference does today, including the per-layer, per-step
+ggml_concat(cached_K, k_rope) / ggml_concat(cached_V, v) copies
+(src/models/smolvla.cpp:832-833, src/models/pi0.cpp:198-201), so timing it gives
+the "restated CPU reference" baseline.
+
+Scope of a layer (the FFN, the VLM backbone between prefix layers and the vision
+towers are outside the hot path): pre-norm -> Q/K/V -> RoPE -> concat ->
+attention -> Wo + residual.
+
+`emulate_bf16` rounds to bf16 at the points where the GPU path stores bf16
+(hidden stream, normalised activations, Q, K, V, attention output); everything
+else (scores, softmax, accumulation, RoPE, the Euler state) is fp32/fp64 in both
+modes, the reference's precision split (src/act_dtype.h:29-35).
+"""
+import math
+
+import numpy as np
+
+import oracle as orc
+
+
+def _rnd(emulate):
+    return orc.round_bf16 if emulate else (lambda x: np.asarray(x, np.float32))
+
+
+def _is_self(cfg, l):
+    if cfg["arch"] == "pi0":
+        return True
+    if cfg["arch"] == "smolvla":
+        return l % cfg["self_attn_every_n"] == 0
+    return l % 2 == 1
+
+
+def _split_heads(y, Hq, Hkv, D):
+    M = y.shape[0]
+    q = y[:, :Hq * D].reshape(M, Hq, D)
+    k = y[:, Hq * D:(Hq + Hkv) * D].reshape(M, Hkv, D)
+    v = y[:, (Hq + Hkv) * D:].reshape(M, Hkv, D)
+    return q, k, v
+
+
+def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
+    """SmolVLA / pi0 / GR00T N1.5 action chunk for one observation.
+
+    obs: img_emb [views*n_img, hidden], n_views, lang (int32 or None), state, noise
+    [n_actions, max_action_dim].  Returns [n_actions, max_action_dim] fp32.
+    Follows build_compute_graph (src/models/smolvla.cpp:1376-1419), the pi0 main
+    graph (src/models/pi0.cpp:559-588) and the GR00T solver loop
+    (src/models/gr00tn1d5.cpp:359-381).
+    """
+    arch = cfg["arch"]
+    rnd = _rnd(emulate_bf16)
+    L, Hq, Hkv, D = cfg["n_layers"], cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    W, Wv, A, S, steps = cfg["expert_h"], cfg["hidden"], cfg["max_action_dim"], cfg["n_suffix"], cfg["num_steps"]
+    kvd = Hkv * D
+    eps = cfg["rms_eps"]
+    scale = 1.0 / math.sqrt(D)
+    views = obs["n_views"]
+    n_img_tot = views * cfg["n_img"]
+    img = np.asarray(obs["img_emb"], np.float32).reshape(n_img_tot, Wv)
+    state = np.zeros(cfg["max_state_dim"], np.float32) if obs.get("state") is None else np.asarray(obs["state"], np.float32)
+    gr00t = arch == "gr00t_n1d5"
+    n_lead = 0 if arch == "smolvla" else 1
+    Sa = S - n_lead
+
+    # ---- prefix embeddings, positions, masks
+    pad = (0, 0)
+    if gr00t:
+        pe = img
+        P = n_img_tot
+    else:
+        lang = np.asarray(obs["lang"], np.int32)
+        n_lang = lang.size
+        lscale = np.float32(math.sqrt(Wv))
+        if arch == "smolvla":
+            Lmax = cfg["n_lang"]
+            ids = np.zeros(Lmax, np.int32)
+            ids[:n_lang] = lang
+            st = orc.linear(state[None, :], w["prefix.Wstate"], w["prefix.bstate"])
+            pe = np.concatenate([img * lscale, w["prefix.E_lang"][ids] * lscale, st], 0)
+            P = n_img_tot + Lmax + 1
+            state_pos = n_img_tot + n_lang
+            pad = (n_img_tot + n_lang, n_img_tot + Lmax)
+            _, pos_prefill = orc.mask_smolvla_prefill(P, pad[0], pad[1], state_pos)
+            pos_self = state_pos + 1 + np.arange(S, dtype=np.int32)
+        else:
+            pe = np.concatenate([img, w["prefix.E_lang"][lang] * lscale], 0)
+            P = n_img_tot + n_lang
+            pos_prefill = np.arange(P, dtype=np.int32)
+            pos_self = P + np.arange(S, dtype=np.int32)
+        pos_cross = np.arange(S, dtype=np.int32)
+        base = cfg["rope_freq_base"]
+        cp, sp = orc.rope_tables(pos_prefill, D, base)
+        cs, ss = orc.rope_tables(pos_self, D, base)
+        cc, sc_ = orc.rope_tables(pos_cross, D, base)
+    pe = rnd(pe)
+
+    if cfg["suffix_mask"] == 1:
+        mask_self = orc.mask_smolvla_full(P, S, pad[0], pad[1])
+    elif cfg["suffix_mask"] == 2:
+        mask_self = orc.mask_pi0_full(P, S)
+    else:
+        mask_self = np.zeros((S, P + S), np.float32)
+        mask_self[:, pad[0]:pad[1]] = -np.inf
+    mask_cross = orc.mask_smolvla_prefix_only(P, S, pad[0], pad[1])
+
+    # ---- prefix K/V per layer, once per observation
+    cacheK, cacheV = [None] * L, [None] * L
+    for l in range(L):
+        self_l = _is_self(cfg, l)
+        if gr00t:
+            if self_l:
+                continue
+            kv = orc.linear(pe, w["vlm.%d.Wkv" % l], w["vlm.%d.bkv" % l])
+            cacheK[l] = rnd(kv[:, :kvd]).reshape(P, Hkv, D)
+            cacheV[l] = rnd(kv[:, kvd:]).reshape(P, Hkv, D)
+            continue
+        xn = rnd(orc.rms_norm(pe, w["vlm.%d.ln" % l], eps))
+        kv = orc.linear(xn, w["vlm.%d.Wkv" % l])
+        k = rnd(orc.rope_neox(kv[:, :kvd].reshape(P, Hkv, D), cp, sp))
+        v = rnd(kv[:, kvd:]).reshape(P, Hkv, D)
+        if arch == "smolvla" and not self_l:
+            # expert_cross_kv (smolvla.cpp:853-860): re-project the cached, already rotated K and V
+            k = rnd(orc.linear(k.reshape(P, kvd), w["ex.%d.Wk_x" % l])).reshape(P, Hkv, D)
+            v = rnd(orc.linear(v.reshape(P, kvd), w["ex.%d.Wv_x" % l])).reshape(P, Hkv, D)
+        cacheK[l], cacheV[l] = k, v
+
+    # ---- per-step constants
+    dt = (1.0 if gr00t else -1.0) / steps
+    dt32 = np.float32(dt)
+    if gr00t:
+        ada = []
+        for s in range(steps):
+            tp = orc.timesteps_proj(int(s / steps * 1000.0))
+            t1 = orc.silu(orc.linear(tp[None, :], w["te.l1W"], w["te.l1b"]))
+            temb = orc.linear(t1, w["te.l2W"], w["te.l2b"])
+            st = orc.silu(temb)
+            ada.append([orc.linear(st, w["ex.%d.adaln_w" % l], w["ex.%d.adaln_b" % l])[0] for l in range(L)])
+    lead = None
+    if n_lead:
+        lead = orc.linear(state[None, :], w["act.W_sp"], w["act.b_sp"])
+
+    x = np.asarray(obs["noise"], np.float32).reshape(Sa, A).copy()
+    debug = {}
+    for s in range(steps):
+        bias = w["act.b_in"].copy()
+        if not gr00t:
+            t = np.float32(1.0) + np.float32(s) * dt32
+            bias = bias + orc.sinusoidal_time_emb(float(t), W, cfg["min_period"], cfg["max_period"])
+        h = orc.linear(x, w["act.W_in"], bias)
+        if n_lead:
+            h = np.concatenate([lead, h], 0)
+        h = rnd(h)
+        for l in range(L):
+            p = "ex.%d." % l
+            self_l = _is_self(cfg, l)
+            if gr00t:
+                c = ada[s][l]
+                hn = rnd(orc.adaln(h, c[:W], c[W:], eps))
+            else:
+                hn = rnd(orc.rms_norm(h, w[p + "ln"], eps))
+            if self_l:
+                y = orc.linear(hn, w[p + "Wqkv"], w.get(p + "bqkv"))
+                q, k, v = _split_heads(y, Hq, Hkv, D)
+                if not gr00t:
+                    q, k = orc.rope_neox(q, cs, ss), orc.rope_neox(k, cs, ss)
+                q, k, v = rnd(q), rnd(k), rnd(v)
+                if cacheK[l] is not None:
+                    K_full, V_full = orc.kv_concat(cacheK[l], k), orc.kv_concat(cacheV[l], v)
+                    m = mask_self
+                else:  # GR00T self-attention over the suffix tokens only
+                    K_full, V_full, m = k, v, None
+            else:
+                q = orc.linear(hn, w[p + "Wq"], w.get(p + "bq")).reshape(S, Hq, D)
+                if not gr00t:
+                    q = orc.rope_neox(q, cc, sc_)
+                q = rnd(q)
+                K_full, V_full = cacheK[l], cacheV[l]
+                m = mask_cross if (pad[1] > pad[0]) else None
+            att = rnd(orc.attention(q, K_full, V_full, m, scale))
+            h = rnd(orc.linear(att, w[p + "Wo"], w.get(p + "bo")) + h)
+            if return_debug and s == 0 and l == 0:
+                debug["q0"], debug["att0"], debug["h0"] = q, att, h
+        if gr00t:
+            hn = rnd(orc.layer_norm(h, None, None, cfg.get("norm_out_eps", 1e-6)))
+        else:
+            hn = rnd(orc.rms_norm(h, w["act.norm"], eps))
+        v_t = orc.linear(hn[n_lead:], w["act.W_out"], w["act.b_out"])
+        x = (x + dt32 * v_t).astype(np.float32)
+    x[:, cfg["real_action_dim"]:] = 0
+    return (x, debug) if return_debug else x
+
+
+def bitvla_ternary(cfg, w, name, from_fp32):
+    """(ternary int8 [N,K], per-row-group scales expanded to ws groups) as the loader derives them."""
+    kvd = cfg["n_kv_heads"] * cfg["head_dim"]
+    t = w[name + ".t"]
+    parts = [cfg["hidden"], kvd, kvd] if name.endswith("Wqkv") else [t.shape[0]]
+    group = kvd if name.endswith("Wqkv") else t.shape[0]
+    if from_fp32:
+        scales, row, tt = [], 0, np.empty_like(t)
+        for n, s in zip(parts, w[name + ".ws"]):
+            deq = t[row:row + n].astype(np.float32) * np.float32(s)
+            q, am = orc.weight_quant_ternary(deq)
+            tt[row:row + n] = q
+            scales.append(am)
+            row += n
+        t = tt
+    else:
+        scales = list(w[name + ".ws"])
+    ws = np.float32([s for n, s in zip(parts, scales) for _ in range(n // group)])
+    return t, ws
+
+
+def bitvla_chunk(cfg, w, obs, from_fp32=False):
+    """BitVLA-shape prefix prefill + autoregressive-style append of the action tokens.
+
+    One layer = run_layer's attention half (src/kernels/bitvla/bitvla_lm_cuda.cu:422-486):
+    bf16 rmsnorm -> act-quant -> ternary GEMM (int32, bf16 out) -> RoPE(Q,K) ->
+    attention -> bf16 sub-norm -> act-quant -> ternary O GEMM -> bf16 add.
+    Returns (actions [n_act, A], int32 accumulators of layer 0's QKV GEMM over the prefix).
+    """
+    L, Hq, Hkv, D, H = cfg["n_layers"], cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["hidden"]
+    kvd, n_act, A = Hkv * D, cfg["n_suffix"], cfg["max_action_dim"]
+    eps, scale = cfg["rms_eps"], 1.0 / math.sqrt(D)
+    P = cfg["n_img"] + cfg["n_lang"]
+    rb = orc.round_bf16
+    tern = [(bitvla_ternary(cfg, w, "lm.%d.Wqkv" % l, from_fp32), bitvla_ternary(cfg, w, "lm.%d.Wo" % l, from_fp32))
+            for l in range(L)]
+    cos_t, sin_t = orc.rope_tables(np.arange(P + n_act, dtype=np.int32), D, cfg["rope_freq_base"])
+    cacheK, cacheV = [None] * L, [None] * L
+    acc0 = [None]
+
+    def bitlinear(x_bf, t, ws, keep=False):
+        q, s = orc.act_quant(x_bf)
+        acc = orc.ternary_gemm_i32(q, t)
+        if keep and acc0[0] is None:
+            acc0[0] = acc
+        return orc.from_bf16(orc.ternary_epilogue(acc, s, ws))
+
+    def layers(h, tok0):
+        n = h.shape[0]
+        for l in range(L):
+            (tq, wsq), (to, wso) = tern[l]
+            hn = rb(orc.rms_norm(h, w["lm.%d.attn_norm" % l], eps))
+            y = bitlinear(hn, tq, wsq, keep=(l == 0))
+            q, k, v = _split_heads(y, Hq, Hkv, D)
+            q = rb(orc.rope_neox(q, cos_t[tok0:tok0 + n], sin_t[tok0:tok0 + n]))
+            k = rb(orc.rope_neox(k, cos_t[tok0:tok0 + n], sin_t[tok0:tok0 + n]))
+            if tok0 == 0:
+                cacheK[l], cacheV[l] = k, v.copy()
+            else:
+                cacheK[l], cacheV[l] = orc.kv_concat(cacheK[l][:tok0], k), orc.kv_concat(cacheV[l][:tok0], v)
+            att = rb(orc.attention(q, cacheK[l], cacheV[l], None, scale))
+            sub = rb(orc.rms_norm(att, w["lm.%d.sub_norm" % l], eps))
+            o = bitlinear(sub, to, wso)
+            h = rb(h + o)
+        return h
+
+    emb = np.concatenate([np.asarray(obs["img_emb"], np.float32).reshape(cfg["n_img"], H),
+                          w["prefix.E_lang"][np.asarray(obs["lang"], np.int32)]], 0)
+    layers(rb(emb), 0)
+    hfin = []
+    for t in range(n_act):
+        h = layers(rb(w["act.emb"][t][None, :]), P + t)
+        hfin.append(rb(orc.rms_norm(h, w["act.norm"], eps)))
+    hf = np.concatenate(hfin, 0)
+    x = orc.linear(hf, w["act.W_out"], w["act.b_out"])
+    x[:, cfg["real_action_dim"]:] = 0
+    return x, acc0[0]

@@ -1,0 +1,157 @@
+"""Whole action-chunk parity through the model-level C ABI (vla_model_load /
+vla_predict / vla_predict_batch) against the chunk oracle, one test per BASELINE
+configuration family.
+
+Tolerances: fp32 (config 0) 1e-5 relative on the chunk output; bf16 configs
+2e-2 relative / 1e-2 absolute on the chunk output.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from oracle import chunk as orc_chunk
+from util import pkg, rel_err
+
+pytestmark = pytest.mark.gpu
+
+from vla_cpp_amd import checkpoint as ckpt  # noqa: E402
+from vla_cpp_amd import ffi  # noqa: E402
+
+
+def bf16_close(got, want):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    return bool(np.all(np.abs(got - want) <= 1e-2 + 2e-2 * np.abs(want)))
+
+
+def make_obs(cfg, r, n_views, n_lang=None, bf16_inputs=False):
+    A = cfg["max_action_dim"]
+    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "bitvla") else 1)
+    img = r.standard_normal((n_views * cfg["n_img"], cfg["hidden"])).astype(np.float32)
+    if cfg["arch"] == "smolvla":
+        img /= np.sqrt(cfg["hidden"])  # the prefix builder scales image rows by sqrt(hidden)
+    obs = dict(img_emb=img, n_views=n_views, noise=r.standard_normal((n_act, A)).astype(np.float32))
+    if cfg.get("vocab", 0) > 0:
+        n_lang = cfg["n_lang"] if n_lang is None else n_lang
+        obs["lang"] = r.integers(0, cfg["vocab"], n_lang).astype(np.int32)
+    if cfg.get("max_state_dim", 0) > 0:
+        obs["state"] = r.standard_normal(cfg["max_state_dim"]).astype(np.float32)
+    return obs
+
+
+def load(tmp_path, cfg, w, name, **kw):
+    path = os.path.join(str(tmp_path), name + ".vlaw")
+    ckpt.write_synthetic(path, cfg, w, **kw)
+    return ffi.Model(path)
+
+
+@pytest.mark.parametrize("suffix_mask,n_lang", [(0, 48), (1, 48), (1, 37)])
+def test_config0_smolvla_single_layer_fp32(tmp_path, suffix_mask, n_lang):
+    cfg = ckpt.smolvla_config(n_layers=1, dtype="f32", suffix_mask=suffix_mask)
+    w = ckpt.synth_weights(cfg, seed=0x5EED)
+    r = np.random.default_rng(200 + suffix_mask + n_lang)
+    obs = make_obs(cfg, r, n_views=3, n_lang=n_lang)
+    m = load(tmp_path, cfg, w, "cfg0")
+    got = m.predict(obs).reshape(50, 32)
+    c = m.config()
+    assert (c.n_q_heads, c.n_kv_heads, c.head_dim, c.n_suffix, c.num_steps) == (15, 5, 64, 50, 10)
+    want = orc_chunk.flow_expert_chunk(cfg, w, obs)
+    assert rel_err(got, want) < 1e-5, rel_err(got, want)
+    st = m.stats()
+    assert st.ms_total > 0
+    # the same handle, a second observation: the resident cache is rebuilt, not reused
+    obs2 = make_obs(cfg, r, n_views=3, n_lang=n_lang)
+    got2 = m.predict(obs2).reshape(50, 32)
+    assert rel_err(got2, orc_chunk.flow_expert_chunk(cfg, w, obs2)) < 1e-5
+    m.close()
+
+
+@pytest.mark.parametrize("n_layers,batch", [(4, 1), (16, 3)])
+def test_config1_smolvla_stack_bf16(tmp_path, n_layers, batch):
+    cfg = ckpt.smolvla_config(n_layers=n_layers, dtype="bf16", suffix_mask=0)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 1)
+    r = np.random.default_rng(210 + n_layers)
+    obs = [make_obs(cfg, r, n_views=3) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "cfg1")
+    got = m.predict_batch(obs).reshape(batch, 50, 32)
+    for b in range(batch):
+        want_e = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+        assert bf16_close(got[b], want_e), np.abs(got[b] - want_e).max()
+        if b == 0:
+            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=False)
+            assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    # batch elements are independent: element 0 alone gives the same chunk
+    solo = m.predict(obs[0]).reshape(50, 32)
+    assert np.array_equal(solo, got[0])
+    m.close()
+
+
+def test_config1_reference_causal_mask_and_language_padding(tmp_path):
+    cfg = ckpt.smolvla_config(n_layers=4, dtype="bf16", suffix_mask=1)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 2)
+    r = np.random.default_rng(220)
+    obs = make_obs(cfg, r, n_views=2, n_lang=30)
+    m = load(tmp_path, cfg, w, "cfg1c")
+    got = m.predict(obs).reshape(50, 32)
+    assert bf16_close(got, orc_chunk.flow_expert_chunk(cfg, w, obs, emulate_bf16=True))
+    m.close()
+
+
+@pytest.mark.parametrize("n_layers,batch", [(3, 2), (18, 1)])
+def test_config2_pi0_mqa_bf16(tmp_path, n_layers, batch):
+    cfg = ckpt.pi0_config(n_layers=n_layers)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 3)
+    r = np.random.default_rng(230)
+    obs = [make_obs(cfg, r, n_views=3) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "cfg2")
+    got = m.predict_batch(obs).reshape(batch, 50, 32)
+    for b in range(batch):
+        want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+        assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    m.close()
+
+
+@pytest.mark.parametrize("n_layers,batch", [(4, 2), (16, 1)])
+def test_config3_gr00t_dit_bf16(tmp_path, n_layers, batch):
+    cfg = ckpt.gr00t_config(n_layers=n_layers)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 4)
+    r = np.random.default_rng(240)
+    obs = [make_obs(cfg, r, n_views=2) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "cfg3")
+    got = m.predict_batch(obs).reshape(batch, 16, 32)
+    for b in range(batch):
+        want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+        assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    m.close()
+
+
+@pytest.mark.parametrize("from_fp32", [False, True])
+def test_config4_bitvla_ternary_append(tmp_path, from_fp32):
+    cfg = ckpt.bitvla_config(n_layers=2)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 5)
+    r = np.random.default_rng(250)
+    obs = [make_obs(cfg, r, n_views=1) for _ in range(2)]
+    m = load(tmp_path, cfg, w, "cfg4", ladder_pack=None if from_fp32 else orc.pack_ladder_int2)
+    got = m.predict_batch(obs).reshape(2, 7, 32)
+    for b in range(2):
+        want, _ = orc_chunk.bitvla_chunk(cfg, w, obs[b], from_fp32=from_fp32)
+        assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    m.close()
+
+
+def test_bad_inputs_are_argument_errors_not_crashes(tmp_path):
+    cfg = ckpt.smolvla_config(n_layers=1, dtype="f32")
+    w = ckpt.synth_weights(cfg)
+    m = load(tmp_path, cfg, w, "bad")
+    r = np.random.default_rng(260)
+    obs = make_obs(cfg, r, n_views=1)
+    obs["lang"] = np.int32([cfg["vocab"] + 5] * 4)  # out-of-vocabulary ids (smolvla.cpp:1582-1589)
+    with pytest.raises(RuntimeError, match="-1"):
+        m.predict(obs)
+    obs = make_obs(cfg, r, n_views=9)
+    with pytest.raises(RuntimeError, match="-1"):
+        m.predict(obs)
+    m.close()
+    with pytest.raises(RuntimeError):
+        ffi.Model(os.path.join(str(tmp_path), "missing.vlaw"))

@@ -218,9 +218,21 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
             if (EB == 2) {
 #pragma unroll
                 for (int hh = 0; hh < 2; ++hh) {
+                    // The probabilities enter the bf16 MFMA as hi + lo (two bf16 terms,
+                    // ~16 mantissa bits): the P.V product then matches an fp32-probability
+                    // reference instead of carrying an extra 2^-9 rounding per weight.
                     const float* pp = &p[kb][hh * 8];
-                    const u32x4_t pf = {pack_bf2(pp[0], pp[1]), pack_bf2(pp[2], pp[3]), pack_bf2(pp[4], pp[5]),
-                                        pack_bf2(pp[6], pp[7])};
+                    float lo[8];
+                    uint32_t hi16[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        hi16[e] = f2bf(pp[e]);
+                        lo[e] = pp[e] - bf2f((bf16_t)hi16[e]);
+                    }
+                    const u32x4_t pf = {hi16[0] | (hi16[1] << 16), hi16[2] | (hi16[3] << 16), hi16[4] | (hi16[5] << 16),
+                                        hi16[6] | (hi16[7] << 16)};
+                    const u32x4_t pl = {pack_bf2(lo[0], lo[1]), pack_bf2(lo[2], lo[3]), pack_bf2(lo[4], lo[5]),
+                                        pack_bf2(lo[6], lo[7])};
                     const int key_off = (kb * 32 + hh * 16 + 4 * g) * EB;
 #pragma unroll
                     for (int db = 0; db < NDB; ++db) {
@@ -229,6 +241,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
                         const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(vr + 8 * EB);
                         const u32x4_t vf = {v0[0], v0[1], v1[0], v1[1]};
                         A::mma(o[db], vf, pf);
+                        A::mma(o[db], vf, pl);
                     }
                 }
             } else {

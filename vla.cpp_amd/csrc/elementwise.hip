@@ -51,6 +51,46 @@ __global__ void rope_neox_hsd_bf16_kernel(bf16_t* __restrict__ x, const float* _
     base[p + half] = f2bf(b * c + a * s);
 }
 
+// Split a fused [M][(Hq+2Hkv)*D] projection (Q | K | V columns), rotate Q and K
+// and scatter: Q token-major, K / V into the resident cache.  One thread per
+// rotation pair (Q, K) or per element pair (V).
+template <typename T>
+__global__ void qkv_split_rope_append_kernel(const T* __restrict__ qkv, const float* __restrict__ cos_t,
+                                             const float* __restrict__ sin_t, T* __restrict__ q_out,
+                                             T* __restrict__ k_cache, T* __restrict__ vt_cache, int S, int Hq, int Hkv,
+                                             int D, int t_max, int tok_offset, long total) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int half = D >> 1;
+    const int heads = Hq + 2 * Hkv;
+    const int p = (int)(i % half);
+    long rh = i / half;
+    const int hh = (int)(rh % heads);
+    const int m = (int)(rh / heads);
+    const int b = m / S, s = m % S;
+    const T* src = qkv + ((long)m * heads + hh) * D;
+    float a = Elem<T>::load(src + p), c2 = Elem<T>::load(src + p + half);
+    if (hh < Hq + Hkv && cos_t) {
+        const float c = cos_t[(long)s * half + p], sn = sin_t[(long)s * half + p];
+        const float x0 = a, x1 = c2;
+        a = x0 * c - x1 * sn;
+        c2 = x1 * c + x0 * sn;
+    }
+    if (hh < Hq) {
+        T* dst = q_out + ((long)m * Hq + hh) * D;
+        Elem<T>::store(dst + p, a);
+        Elem<T>::store(dst + p + half, c2);
+    } else if (hh < Hq + Hkv) {
+        T* dst = k_cache + (((long)b * Hkv + (hh - Hq)) * t_max + tok_offset + s) * D;
+        Elem<T>::store(dst + p, a);
+        Elem<T>::store(dst + p + half, c2);
+    } else {
+        T* dst = vt_cache + ((long)b * Hkv + (hh - Hq - Hkv)) * D * (long)t_max + tok_offset + s;
+        Elem<T>::store(dst + (long)p * t_max, a);
+        Elem<T>::store(dst + (long)(p + half) * t_max, c2);
+    }
+}
+
 // ----------------------------------------------------------------- norms ---
 template <typename T>
 __global__ void rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y, int K, float eps) {
@@ -248,6 +288,30 @@ int vla_rope_neox(void* x, const float* cos_tab, const float* sin_tab, int dtype
         rope_neox_kernel<float><<<blocks, 256, 0, st>>>((float*)x, cos_tab, sin_tab, table_rows, n_heads, head_dim, total);
     else if (dtype == VLA_DT_BF16)
         rope_neox_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)x, cos_tab, sin_tab, table_rows, n_heads, head_dim, total);
+    else
+        return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_qkv_split_rope_append(const void* qkv, const float* cos_tab, const float* sin_tab, void* q_out, void* k_cache,
+                              void* vt_cache, int dtype, int M, int S, int n_q_heads, int n_kv_heads, int head_dim,
+                              int t_max, int tok_offset, vla_stream_t stream) {
+    if (!qkv || !q_out || !k_cache || !vt_cache || M < 0 || S <= 0 || n_q_heads <= 0 || n_kv_heads <= 0)
+        return VLA_K_ERR_ARG;
+    if ((cos_tab == nullptr) != (sin_tab == nullptr)) return VLA_K_ERR_ARG;
+    if (head_dim <= 0 || (head_dim & 1) || M % S || tok_offset < 0 || tok_offset + S > t_max) return VLA_K_ERR_SHAPE;
+    const long total = (long)M * (n_q_heads + 2 * n_kv_heads) * (head_dim / 2);
+    if (total == 0) return VLA_K_OK;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == VLA_DT_F32)
+        qkv_split_rope_append_kernel<float><<<blocks, 256, 0, st>>>((const float*)qkv, cos_tab, sin_tab, (float*)q_out,
+                                                                   (float*)k_cache, (float*)vt_cache, S, n_q_heads,
+                                                                   n_kv_heads, head_dim, t_max, tok_offset, total);
+    else if (dtype == VLA_DT_BF16)
+        qkv_split_rope_append_kernel<bf16_t><<<blocks, 256, 0, st>>>((const bf16_t*)qkv, cos_tab, sin_tab, (bf16_t*)q_out,
+                                                                    (bf16_t*)k_cache, (bf16_t*)vt_cache, S, n_q_heads,
+                                                                    n_kv_heads, head_dim, t_max, tok_offset, total);
     else
         return VLA_K_ERR_ARG;
     return VLA_CHECK_LAUNCH();

@@ -1,0 +1,252 @@
+// BitVLA-shape ternary (b1.58) attention path with a resident KV cache.
+//
+// Arithmetic of one layer follows the reference's CUDA forward, run_layer
+// (src/kernels/bitvla/bitvla_lm_cuda.cu:422-486): bf16 RMSNorm -> per-token
+// int8 act-quant -> ternary QKV GEMM (int32 accumulate, bf16 out) -> NeoX RoPE
+// on Q and K -> attention -> bf16 sub-norm -> act-quant -> ternary O GEMM ->
+// bf16 residual add.  Differences, all by design: Q|K|V is one fused GEMM
+// (N = 3840, the shape bitnet_kernels.cu:112 registers as "head.qkv"); K/V are
+// written into the resident cache instead of being expanded by repeat_kv; the
+// attention is one fused kernel with fp32 scores instead of two cuBLAS GEMMs
+// around a bf16 score buffer; the FFN half of the layer is not on this path.
+//
+// The reference runs one bidirectional pass with no cache
+// (src/models/bitvla.cpp:205-238).  Here the prefix (image + text tokens) is
+// prefilled once, then action tokens are appended one at a time, each
+// attending to the prefix and to the tokens appended before it.
+//
+// Weight preparation at load restates recover_ternary_and_scale and the
+// per-source scales of pack_and_upload_fused (src/models/bitvla.cpp:430-451,
+// 523-543); ladder-packed tensors ("*.i2") are re-ordered word by word into the
+// gfx950 layout.
+
+#include <algorithm>
+#include <cmath>
+#include <random>
+
+#include "checkpoint.h"
+#include "layers.h"
+#include "model.h"
+
+namespace vla {
+namespace {
+
+int round_up(int x, int m) { return (x + m - 1) / m * m; }
+
+struct TernaryW {
+    DevBuf packed;  // [N][K/16] words
+    DevBuf ws;      // fp32 [ws_num]
+    int N = 0, K = 0, ws_num = 1;
+};
+
+// `parts` = row counts of the tensors fused into `name` (one absmean each).
+TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::vector<int>& parts, int K, int ws_group) {
+    TernaryW w;
+    w.K = K;
+    for (int n : parts) w.N += n;
+    std::vector<uint32_t> packed((size_t)w.N * (K / 16));
+    std::vector<float> scales;
+    if (ck.has(name + ".i2")) {
+        VLA_K(vla_ternary_repack_ladder_host((const uint8_t*)ck.data(name + ".i2"), w.N, K, packed.data()));
+        scales = ck.f32(name + ".ws");
+        if (scales.size() != parts.size()) throw std::runtime_error("vla: " + name + ".ws has the wrong length");
+    } else {
+        const std::vector<float> W = ck.f32(name);
+        std::vector<int8_t> tern((size_t)w.N * K);
+        size_t row = 0;
+        for (int n : parts) {
+            float am = 0.f;
+            VLA_K(vla_ternary_quant_host(W.data() + row * K, (int64_t)n * K, tern.data() + row * K, &am));
+            scales.push_back(am);
+            row += n;
+        }
+        VLA_K(vla_ternary_pack_host(tern.data(), w.N, K, packed.data()));
+    }
+    // The epilogue indexes scales by n / (N / ws_num): expand to equal groups.
+    std::vector<float> ws;
+    for (size_t p = 0; p < parts.size(); ++p)
+        for (int g = 0; g < parts[p] / ws_group; ++g) ws.push_back(scales[p]);
+    w.ws_num = (int)ws.size();
+    w.packed.upload(packed.data(), packed.size() * 4);
+    w.ws.upload(ws.data(), ws.size() * 4);
+    return w;
+}
+
+struct LmLayer {
+    DevBuf attn_norm, sub_norm;
+    TernaryW Wqkv, Wo;
+    KVLayer kv;
+};
+
+class BitvlaLm : public ModelArch {
+  public:
+    explicit BitvlaLm(const Checkpoint& ck);
+    void prefill(const Inputs* in, int batch) override;
+    void denoise(int chunks, void* stream) override;
+    std::vector<float> fetch() override;
+    int64_t n_actions() const override { return n_act_; }
+
+  private:
+    void run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys);
+    int L_, Hq_, Hkv_, D_, H_, A_, n_act_, n_img_, n_lang_, vocab_, P_ = 0, B_ = 0;
+    float eps_;
+    std::vector<LmLayer> layers_;
+    std::vector<float> E_lang_, act_emb_;
+    DevBuf out_norm_, W_out_, b_out_;
+    RopeTable rope_;
+    DevBuf h_, hn_, q8_, s_, rowsum_, qkv_, q_, att_, o_, emb_bcast_, hfin_, x_;
+    hipStream_t last_stream_ = nullptr;
+};
+
+BitvlaLm::BitvlaLm(const Checkpoint& ck) {
+    L_ = (int)ck.i64("n_layers");
+    Hq_ = (int)ck.i64("n_q_heads");
+    Hkv_ = (int)ck.i64("n_kv_heads");
+    D_ = (int)ck.i64("head_dim");
+    H_ = (int)ck.i64("hidden");
+    A_ = (int)ck.i64("max_action_dim");
+    n_act_ = (int)ck.i64("n_suffix");
+    n_img_ = (int)ck.i64("n_img");
+    n_lang_ = (int)ck.i64("n_lang");
+    vocab_ = (int)ck.i64("vocab");
+    eps_ = (float)ck.f64("rms_eps", 1e-5);
+    if (Hq_ * D_ != H_) throw std::runtime_error("vla(bitvla): n_q_heads * head_dim must equal hidden");
+    cfg.n_img = n_img_; cfg.n_lang = n_lang_; cfg.n_prefix = n_img_ + n_lang_; cfg.n_suffix = n_act_;
+    cfg.n_full = cfg.n_prefix + n_act_;
+    cfg.hidden = H_; cfg.expert_h = H_; cfg.n_q_heads = Hq_; cfg.n_kv_heads = Hkv_; cfg.head_dim = D_;
+    cfg.q_full_dim = H_; cfg.kv_full_dim = (int64_t)Hkv_ * D_; cfg.n_layers = L_;
+    cfg.max_action_dim = A_; cfg.real_action_dim = ck.i64("real_action_dim", A_);
+    cfg.max_state_dim = 0; cfg.real_state_dim = 0;
+    cfg.num_steps = n_act_; cfg.rms_eps = eps_; cfg.rope_n_dims = D_;
+    cfg.rope_freq_base = (float)ck.f64("rope_freq_base", 500000.0);
+
+    E_lang_ = ck.f32("prefix.E_lang");
+    act_emb_ = ck.f32("act.emb");
+    std::vector<float> nf = ck.f32("act.norm");
+    upload_as(out_norm_, nf.data(), nf.size(), VLA_DT_BF16);
+    { std::vector<float> t = ck.f32("act.W_out"); W_out_.upload(t.data(), t.size() * 4); }
+    { std::vector<float> t = ck.f32("act.b_out"); b_out_.upload(t.data(), t.size() * 4); }
+    const int kvd = Hkv_ * D_;
+    layers_.resize(L_);
+    for (int l = 0; l < L_; ++l) {
+        const std::string p = "lm." + std::to_string(l) + ".";
+        LmLayer& w = layers_[l];
+        std::vector<float> a = ck.f32(p + "attn_norm"), s = ck.f32(p + "sub_norm");
+        upload_as(w.attn_norm, a.data(), a.size(), VLA_DT_BF16);
+        upload_as(w.sub_norm, s.data(), s.size(), VLA_DT_BF16);
+        w.Wqkv = load_ternary(ck, p + "Wqkv", {H_, kvd, kvd}, H_, kvd);
+        w.Wo = load_ternary(ck, p + "Wo", {H_}, H_, H_);
+    }
+}
+
+void BitvlaLm::prefill(const Inputs* in, int batch) {
+    if (!in || batch <= 0) throw std::invalid_argument("vla: prefill needs at least one observation");
+    const int P = n_img_ + n_lang_, B = batch;
+    for (int b = 0; b < B; ++b) {
+        if (!in[b].precomputed_img_emb || in[b].n_img_views != 1) throw std::invalid_argument("vla(bitvla): one view of precomputed_img_emb is required");
+        if (in[b].n_lang != n_lang_ || !in[b].lang_tokens) throw std::invalid_argument("vla(bitvla): n_lang must equal the configured text length");
+        for (int i = 0; i < n_lang_; ++i)
+            if (in[b].lang_tokens[i] < 0 || in[b].lang_tokens[i] >= vocab_) throw std::invalid_argument("vla: language token outside the vocabulary");
+    }
+    const int t_max = round_up(P + n_act_, 64);
+    if (B != B_ || P != P_) {
+        B_ = B;
+        P_ = P;
+        const size_t M = (size_t)B * P;
+        for (LmLayer& w : layers_) {
+            w.kv.create(VLA_DT_BF16, B, Hkv_, D_, t_max);
+            w.kv.n_prefix = P;
+        }
+        h_.alloc(M * H_ * 2); hn_.alloc(M * H_ * 2); q8_.alloc(M * H_); s_.alloc(M * 4); rowsum_.alloc(M * 4);
+        qkv_.alloc(M * (H_ + 2 * Hkv_ * D_) * 2); q_.alloc(M * H_ * 2); att_.alloc(M * H_ * 2); o_.alloc(M * H_ * 2);
+        hfin_.alloc((size_t)n_act_ * B * H_ * 2);
+        x_.alloc((size_t)n_act_ * B * A_ * 4);
+        std::vector<int32_t> pos(P + n_act_);
+        for (int i = 0; i < P + n_act_; ++i) pos[i] = i;  // src/models/bitvla.cpp positions 0..seq-1
+        rope_.build(RopeSpec{D_, cfg.rope_freq_base}, pos);
+        std::vector<uint16_t> eb((size_t)n_act_ * B * H_);
+        for (int t = 0; t < n_act_; ++t)
+            for (int b = 0; b < B; ++b)
+                for (int c = 0; c < H_; ++c) eb[((size_t)t * B + b) * H_ + c] = f32_to_bf16(act_emb_[(size_t)t * H_ + c]);
+        emb_bcast_.upload(eb.data(), eb.size() * 2);
+    }
+    std::vector<uint16_t> emb((size_t)B * P * H_);
+    for (int b = 0; b < B; ++b) {
+        uint16_t* dst = emb.data() + (size_t)b * P * H_;
+        for (size_t i = 0; i < (size_t)n_img_ * H_; ++i) dst[i] = f32_to_bf16(in[b].precomputed_img_emb[i]);
+        for (int i = 0; i < n_lang_; ++i) {
+            const float* e = E_lang_.data() + (size_t)in[b].lang_tokens[i] * H_;
+            for (int c = 0; c < H_; ++c) dst[(size_t)(n_img_ + i) * H_ + c] = f32_to_bf16(e[c]);
+        }
+    }
+    h_.upload(emb.data(), emb.size() * 2);
+    Ctx C;
+    run_layers(C, B * P, P, 0, P);
+    VLA_HIP(hipDeviceSynchronize());
+}
+
+// One pass of all layers over M = B*S rows sitting in h_ (S consecutive tokens
+// per observation starting at cache slot tok_offset, attending to n_keys keys).
+void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
+    const int kvd = Hkv_ * D_, Nqkv = H_ + 2 * kvd;
+    const int half = D_ / 2;
+    const float scale = 1.0f / std::sqrt((float)D_);
+    const float* cos_t = rope_.cos.as<float>() + (size_t)tok_offset * half;
+    const float* sin_t = rope_.sin.as<float>() + (size_t)tok_offset * half;
+    for (LmLayer& w : layers_) {
+        VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), hn_.as<uint16_t>(), eps_, M, H_, C.stream));
+        VLA_K(vla_act_quant_bf16(hn_.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(), rowsum_.as<int32_t>(), M, H_, C.stream));
+        VLA_K(vla_ternary_gemm(q8_.as<int8_t>(), w.Wqkv.packed.as<uint32_t>(), qkv_.as<uint16_t>(), nullptr, s_.as<float>(),
+                               rowsum_.as<int32_t>(), w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_, C.stream));
+        VLA_K(vla_qkv_split_rope_append(qkv_.get(), cos_t, sin_t, q_.get(), w.kv.k.get(), w.kv.vt.get(), VLA_DT_BF16, M, S,
+                                        Hq_, Hkv_, D_, w.kv.t_max, tok_offset, C.stream));
+        VLA_K(vla_attn_prefix_suffix(q_.get(), w.kv.k.get(), w.kv.vt.get(), att_.get(), VLA_DT_BF16, M / S, S, Hq_, Hkv_,
+                                     D_, w.kv.t_max, n_keys, scale, VLA_MASK_NONE, n_keys, 0, 0, nullptr, C.stream));
+        VLA_K(bitvla_rmsnorm_bf16(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), hn_.as<uint16_t>(), eps_, M, H_, C.stream));
+        VLA_K(vla_act_quant_bf16(hn_.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(), rowsum_.as<int32_t>(), M, H_, C.stream));
+        VLA_K(vla_ternary_gemm(q8_.as<int8_t>(), w.Wo.packed.as<uint32_t>(), o_.as<uint16_t>(), nullptr, s_.as<float>(),
+                               rowsum_.as<int32_t>(), w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_, C.stream));
+        VLA_K(bitvla_add_bf16(h_.as<uint16_t>(), o_.as<uint16_t>(), h_.as<uint16_t>(), M * H_, C.stream));
+    }
+}
+
+void BitvlaLm::denoise(int chunks, void* stream) {
+    if (B_ == 0) throw std::logic_error("vla: denoise before prefill");
+    Ctx C;
+    C.stream = (hipStream_t)stream;
+    last_stream_ = C.stream;
+    const int B = B_;
+    const size_t row = (size_t)B * H_;
+    for (int c = 0; c < chunks; ++c) {
+        for (int t = 0; t < n_act_; ++t) {
+            // token t enters as its learned embedding; it depends on the tokens before it
+            // through the K/V they left in the cache
+            VLA_HIP(hipMemcpyAsync(h_.get(), emb_bcast_.as<uint16_t>() + (size_t)t * row, row * 2, hipMemcpyDeviceToDevice,
+                                   C.stream));
+            run_layers(C, B, 1, P_ + t, P_ + t + 1);
+            VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), out_norm_.as<uint16_t>(), hfin_.as<uint16_t>() + (size_t)t * row, eps_, B,
+                                      H_, C.stream));
+        }
+        VLA_HIP(hipMemsetAsync(x_.get(), 0, (size_t)n_act_ * B * A_ * 4, C.stream));
+        // x[t][b] = W_out . hfin[t][b] + b_out (batch' = n_act, rows = B, unit step)
+        VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B, 0, A_,
+                             H_, 1.0f, C.stream));
+    }
+}
+
+std::vector<float> BitvlaLm::fetch() {
+    VLA_HIP(hipStreamSynchronize(last_stream_));
+    std::vector<float> tb((size_t)n_act_ * B_ * A_), out(tb.size());
+    x_.download(tb.data(), tb.size() * 4);
+    for (int t = 0; t < n_act_; ++t)
+        for (int b = 0; b < B_; ++b)
+            for (int j = 0; j < A_; ++j)
+                out[((size_t)b * n_act_ + t) * A_ + j] = j < cfg.real_action_dim ? tb[((size_t)t * B_ + b) * A_ + j] : 0.f;
+    return out;
+}
+
+}  // namespace
+
+ModelArch* bitvla_create(const Checkpoint& ck) { return new BitvlaLm(ck); }
+
+}  // namespace vla

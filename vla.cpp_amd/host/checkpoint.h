@@ -1,0 +1,124 @@
+// Reader for "VLAW" checkpoints: the flat container this library loads in place
+// of the reference's GGUF files (src/gguf_reader.h, src/loader.cpp; reading
+// GGUF is outside this library's scope).  Layout:
+//
+//   bytes 0..7   "VLAW0001"
+//   bytes 8..15  header length H (little-endian uint64)
+//   H bytes      text header, one record per line:
+//                  K <key> <value>
+//                  T <name> <dtype> <ndim> <d0> [<d1> ...] <offset> <nbytes>
+//   data         starts at the next multiple of 64 after the header; tensor
+//                offsets are relative to it.  dtype in {f32, bf16, i8, u8, i32}.
+//
+// Written by vla.cpp_amd/checkpoint.py.
+#pragma once
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+namespace vla {
+
+struct CkptTensor {
+    std::string dtype;
+    std::vector<int64_t> shape;
+    size_t offset = 0, nbytes = 0;
+    int64_t numel() const {
+        int64_t n = 1;
+        for (int64_t d : shape) n *= d;
+        return n;
+    }
+};
+
+class Checkpoint {
+  public:
+    explicit Checkpoint(const std::string& path) {
+        FILE* f = std::fopen(path.c_str(), "rb");
+        if (!f) throw std::runtime_error("vla: cannot open checkpoint " + path);
+        std::fseek(f, 0, SEEK_END);
+        const long sz = std::ftell(f);
+        std::fseek(f, 0, SEEK_SET);
+        blob_.resize((size_t)sz);
+        const size_t got = std::fread(blob_.data(), 1, (size_t)sz, f);
+        std::fclose(f);
+        if (got != (size_t)sz || sz < 16 || std::string(blob_.data(), 8) != "VLAW0001")
+            throw std::runtime_error("vla: " + path + " is not a VLAW0001 checkpoint");
+        uint64_t hlen = 0;
+        std::memcpy(&hlen, blob_.data() + 8, 8);
+        if (16 + hlen > (uint64_t)sz) throw std::runtime_error("vla: truncated checkpoint header");
+        data_ = (16 + (size_t)hlen + 63) / 64 * 64;
+        std::istringstream hs(std::string(blob_.data() + 16, (size_t)hlen));
+        std::string line;
+        while (std::getline(hs, line)) {
+            std::istringstream ls(line);
+            std::string tag;
+            ls >> tag;
+            if (tag == "K") {
+                std::string k, v;
+                ls >> k >> v;
+                kv_[k] = v;
+            } else if (tag == "T") {
+                std::string name;
+                CkptTensor t;
+                int ndim = 0;
+                ls >> name >> t.dtype >> ndim;
+                t.shape.resize(ndim);
+                for (int i = 0; i < ndim; ++i) ls >> t.shape[i];
+                ls >> t.offset >> t.nbytes;
+                if (!ls || data_ + t.offset + t.nbytes > blob_.size())
+                    throw std::runtime_error("vla: tensor " + name + " lies outside the checkpoint");
+                tensors_[name] = t;
+            }
+        }
+    }
+
+    bool has(const std::string& name) const { return tensors_.count(name) != 0; }
+    const CkptTensor& info(const std::string& name) const {
+        auto it = tensors_.find(name);
+        if (it == tensors_.end()) throw std::runtime_error("vla: checkpoint has no tensor " + name);
+        return it->second;
+    }
+    const void* data(const std::string& name) const { return blob_.data() + data_ + info(name).offset; }
+
+    // Tensor as fp32 on the host (bf16 widened exactly).
+    std::vector<float> f32(const std::string& name) const {
+        const CkptTensor& t = info(name);
+        std::vector<float> out((size_t)t.numel());
+        if (t.dtype == "f32") {
+            std::memcpy(out.data(), data(name), out.size() * 4);
+        } else if (t.dtype == "bf16") {
+            const uint16_t* p = (const uint16_t*)data(name);
+            for (size_t i = 0; i < out.size(); ++i) {
+                uint32_t u = ((uint32_t)p[i]) << 16;
+                std::memcpy(&out[i], &u, 4);
+            }
+        } else {
+            throw std::runtime_error("vla: tensor " + name + " is not floating point");
+        }
+        return out;
+    }
+
+    std::string str(const std::string& key) const {
+        auto it = kv_.find(key);
+        if (it == kv_.end()) throw std::runtime_error("vla: checkpoint has no key " + key);
+        return it->second;
+    }
+    bool has_key(const std::string& key) const { return kv_.count(key) != 0; }
+    int64_t i64(const std::string& key) const { return std::stoll(str(key)); }
+    int64_t i64(const std::string& key, int64_t dflt) const { return has_key(key) ? i64(key) : dflt; }
+    double f64(const std::string& key) const { return std::stod(str(key)); }
+    double f64(const std::string& key, double dflt) const { return has_key(key) ? f64(key) : dflt; }
+
+  private:
+    std::vector<char> blob_;
+    size_t data_ = 0;
+    std::map<std::string, std::string> kv_;
+    std::map<std::string, CkptTensor> tensors_;
+};
+
+}  // namespace vla

@@ -1,0 +1,471 @@
+// Flow-matching / DiT action experts on the resident-KV attention path:
+// SmolVLA, pi0 and GR00T N1.5 schedules over the same kernels.
+//
+// What is restated from the reference (graph builders that record ggml nodes
+// there, eager launches here):
+//   SmolVLA  build_vlm_layer's K/V outputs, expert_cross_kv,
+//            build_expert_self_attn_layer, build_expert_cross_attn_layer and
+//            the denoise loop of build_compute_graph
+//            (src/models/smolvla.cpp:778-888, 1376-1419), masks and positions
+//            of predict (1608-1672)
+//   pi0      build_gemma_layer prefix / suffix passes, build_embed_suffix, the
+//            step loop and the full mask (src/models/pi0.cpp:159-248, 536-661)
+//   GR00T    DitHead::kv hoisted out of the solver loop, DitHead::block's
+//            adaLN -> Q(KV) -> attention -> Wo, the Euler loop
+//            (src/modules/dit_head.cpp:87-133, src/models/gr00tn1d5.cpp:359-381)
+// The FFN half of each layer, the VLM backbone between prefix layers and the
+// vision towers are not part of this path: every prefix layer projects the same
+// prefix embeddings, and a layer is pre-norm -> QKV(+RoPE, +append) ->
+// attention -> Wo + residual.
+//
+// The prefix K/V of every layer is written once per observation and stays in
+// HBM; each denoise step overwrites only the S suffix slots behind it.
+
+#include <algorithm>
+#include <chrono>
+#include <cmath>
+#include <random>
+#include <thread>
+
+#include "checkpoint.h"
+#include "layers.h"
+#include "model.h"
+
+namespace vla {
+namespace {
+
+enum class Arch { SMOLVLA, PI0, GR00T };
+
+int round_up(int x, int m) { return (x + m - 1) / m * m; }
+
+DevBuf load_w(const Checkpoint& ck, const std::string& name, int dtype) {
+    const CkptTensor& t = ck.info(name);
+    DevBuf b;
+    if ((dtype == VLA_DT_F32 && t.dtype == "f32") || (dtype == VLA_DT_BF16 && t.dtype == "bf16")) {
+        b.upload(ck.data(name), t.nbytes);
+    } else {
+        std::vector<float> f = ck.f32(name);
+        upload_as(b, f.data(), f.size(), dtype);
+    }
+    return b;
+}
+DevBuf load_f32(const Checkpoint& ck, const std::string& name) { return load_w(ck, name, VLA_DT_F32); }
+
+// y = W x + b on the host, W [N][K] row-major, double accumulation.
+void host_linear(const float* W, const float* b, const float* x, float* y, int N, int K) {
+    for (int n = 0; n < N; ++n) {
+        double a = 0.0;
+        const float* wr = W + (size_t)n * K;
+        for (int k = 0; k < K; ++k) a += (double)wr[k] * (double)x[k];
+        y[n] = (float)(a + (b ? (double)b[n] : 0.0));
+    }
+}
+float host_silu(float x) { return x / (1.0f + std::exp(-x)); }
+
+struct LayerW {
+    bool is_self = true;
+    DevBuf ln;                  // expert pre-norm weight (RMS archs)
+    DevBuf Wqkv, bqkv;          // self: Q|K|V rows, cross: Q rows
+    DevBuf Wo, bo;
+    DevBuf vlm_ln, Wkv_pre, bkv_pre;  // prefix K|V producer
+    DevBuf Wk_x, Wv_x;          // SmolVLA cross layers: re-projection of the cached prefix K / V
+    KVLayer kv;
+    bool needs_prefix = true;
+};
+
+class FlowExpert : public ModelArch {
+  public:
+    explicit FlowExpert(const Checkpoint& ck);
+    void prefill(const Inputs* in, int batch) override;
+    void denoise(int chunks, void* stream) override;
+    std::vector<float> fetch() override;
+    int64_t n_actions() const override { return S_ - n_lead_; }
+
+  private:
+    void allocate(int B, int P);
+
+    Arch arch_;
+    int dt_ = VLA_DT_F32;
+    int L_ = 0, Hq_ = 0, Hkv_ = 0, D_ = 0, W_ = 0, Wv_ = 0, A_ = 0, S_ = 0, n_lead_ = 0, steps_ = 0;
+    int n_img_ = 0, n_lang_max_ = 0, max_views_ = 1, vocab_ = 0, max_state_ = 0;
+    int suffix_mask_ = VLA_MASK_NONE;
+    float eps_ = 1e-5f, final_eps_ = 1e-6f, dt_step_ = -0.1f;
+    bool rope_ = true;
+
+    std::vector<LayerW> layers_;
+    // small fp32 tensors kept on the host for per-observation work
+    std::vector<float> E_lang_, Wstate_, bstate_, W_sp_, b_sp_;
+    DevBuf W_in_, W_out_, b_out_, final_norm_;
+    DevBuf bias_step_;   // [steps][W] fp32: b_in (+ time embedding of the step)
+    DevBuf ada_;         // GR00T: [steps][L+1][2][W] fp32 (scale, shift); slot L is the final norm (zeros)
+
+    // per-call state
+    int B_ = 0, P_ = 0, pad_start_ = 0, pad_end_ = 0;
+    RopeTable rope_prefill_, rope_self_, rope_cross_;
+    DevBuf prefix_, prefix_n_, tmpk_, tmpv_, lead_, x0_, xt_, h_, hn_, q_, att_;
+    KVLayer tmp_kv_;
+    std::mt19937 rng_{std::random_device{}()};
+    hipStream_t last_stream_ = nullptr;
+};
+
+FlowExpert::FlowExpert(const Checkpoint& ck) {
+    const std::string arch = ck.str("arch");
+    arch_ = arch == "smolvla" ? Arch::SMOLVLA : arch == "pi0" ? Arch::PI0 : Arch::GR00T;
+    dt_ = ck.str("dtype") == "bf16" ? VLA_DT_BF16 : VLA_DT_F32;
+    L_ = (int)ck.i64("n_layers");
+    Hq_ = (int)ck.i64("n_q_heads");
+    Hkv_ = (int)ck.i64("n_kv_heads");
+    D_ = (int)ck.i64("head_dim");
+    W_ = (int)ck.i64("expert_h");
+    Wv_ = (int)ck.i64("hidden");
+    A_ = (int)ck.i64("max_action_dim");
+    S_ = (int)ck.i64("n_suffix");
+    steps_ = (int)ck.i64("num_steps");
+    n_img_ = (int)ck.i64("n_img");
+    n_lang_max_ = (int)ck.i64("n_lang", 0);
+    max_views_ = (int)ck.i64("max_views", 4);
+    vocab_ = (int)ck.i64("vocab", 0);
+    max_state_ = (int)ck.i64("max_state_dim", 32);
+    eps_ = (float)ck.f64("rms_eps", arch_ == Arch::PI0 ? 1e-6 : 1e-5);
+    final_eps_ = (float)ck.f64("norm_out_eps", 1e-6);
+    suffix_mask_ = (int)ck.i64("suffix_mask", arch_ == Arch::SMOLVLA ? VLA_MASK_CAUSAL_SUFFIX
+                                              : arch_ == Arch::PI0   ? VLA_MASK_PI0_STATE
+                                                                     : VLA_MASK_NONE);
+    n_lead_ = arch_ == Arch::SMOLVLA ? 0 : 1;
+    rope_ = arch_ != Arch::GR00T;
+    dt_step_ = (arch_ == Arch::GR00T ? 1.0f : -1.0f) / (float)steps_;
+    const int every = (int)ck.i64("self_attn_every_n", arch_ == Arch::PI0 ? 1 : 2);
+
+    cfg.n_img = n_img_;
+    cfg.n_lang = n_lang_max_;
+    cfg.n_state = arch_ == Arch::SMOLVLA ? 1 : 0;
+    cfg.n_suffix = S_;
+    cfg.hidden = Wv_;
+    cfg.expert_h = W_;
+    cfg.n_q_heads = Hq_;
+    cfg.n_kv_heads = Hkv_;
+    cfg.head_dim = D_;
+    cfg.q_full_dim = (int64_t)Hq_ * D_;
+    cfg.kv_full_dim = (int64_t)Hkv_ * D_;
+    cfg.n_layers = L_;
+    cfg.self_attn_every_n = every;
+    cfg.max_state_dim = max_state_;
+    cfg.max_action_dim = A_;
+    cfg.real_state_dim = ck.i64("real_state_dim", max_state_);
+    cfg.real_action_dim = ck.i64("real_action_dim", A_);
+    cfg.min_period = ck.f64("min_period", 4e-3);
+    cfg.max_period = ck.f64("max_period", 4.0);
+    cfg.num_steps = steps_;
+    cfg.rms_eps = eps_;
+    cfg.rope_n_dims = D_;
+    cfg.rope_freq_base = (float)ck.f64("rope_freq_base", 10000.0);
+    cfg.denormalized = arch_ != Arch::GR00T;
+    cfg.n_prefix = (int64_t)n_img_ + n_lang_max_ + cfg.n_state;
+    cfg.n_full = cfg.n_prefix + S_;
+    if (!config_is_sane(cfg)) throw std::runtime_error("vla: real_* dims exceed max_* dims");
+
+    if (vocab_ > 0) E_lang_ = ck.f32("prefix.E_lang");
+    if (arch_ == Arch::SMOLVLA) {
+        Wstate_ = ck.f32("prefix.Wstate");
+        bstate_ = ck.f32("prefix.bstate");
+    } else {
+        W_sp_ = ck.f32("act.W_sp");
+        b_sp_ = ck.f32("act.b_sp");
+    }
+    W_in_ = load_f32(ck, "act.W_in");
+    W_out_ = load_f32(ck, "act.W_out");
+    b_out_ = load_f32(ck, "act.b_out");
+    if (arch_ != Arch::GR00T) final_norm_ = load_w(ck, "act.norm", dt_);
+
+    layers_.resize(L_);
+    for (int l = 0; l < L_; ++l) {
+        LayerW& w = layers_[l];
+        const std::string p = "ex." + std::to_string(l) + ".";
+        // SmolVLA: self iff l % every == 0 (src/models/smolvla.cpp:1182); GR00T N1.5:
+        // cross on even, self on odd layers (src/models/gr00tn1d5.cpp:361-375).
+        w.is_self = arch_ == Arch::PI0 ? true : arch_ == Arch::SMOLVLA ? (l % every == 0) : (l % 2 == 1);
+        w.needs_prefix = !(arch_ == Arch::GR00T && w.is_self);
+        if (arch_ != Arch::GR00T) w.ln = load_w(ck, p + "ln", dt_);
+        w.Wqkv = load_w(ck, p + (w.is_self ? "Wqkv" : "Wq"), dt_);
+        if (ck.has(p + (w.is_self ? "bqkv" : "bq"))) w.bqkv = load_f32(ck, p + (w.is_self ? "bqkv" : "bq"));
+        w.Wo = load_w(ck, p + "Wo", dt_);
+        if (ck.has(p + "bo")) w.bo = load_f32(ck, p + "bo");
+        if (w.needs_prefix) {
+            const std::string v = "vlm." + std::to_string(l) + ".";
+            if (arch_ != Arch::GR00T) w.vlm_ln = load_w(ck, v + "ln", dt_);
+            w.Wkv_pre = load_w(ck, v + "Wkv", dt_);
+            if (ck.has(v + "bkv")) w.bkv_pre = load_f32(ck, v + "bkv");
+        }
+        if (arch_ == Arch::SMOLVLA && !w.is_self) {
+            w.Wk_x = load_w(ck, p + "Wk_x", dt_);
+            w.Wv_x = load_w(ck, p + "Wv_x", dt_);
+        }
+    }
+
+    // Per-step constants.  The time conditioning depends on the step index only,
+    // so it is evaluated once here instead of inside every denoise step.
+    const std::vector<float> b_in = ck.f32("act.b_in");
+    std::vector<float> bias((size_t)steps_ * W_);
+    for (int s = 0; s < steps_; ++s) {
+        for (int c = 0; c < W_; ++c) bias[(size_t)s * W_ + c] = b_in[c];
+        if (arch_ != Arch::GR00T) {
+            // t = 1 + step*dt (src/models/pi0.cpp:654-656), embedding of src/layers/embed.h:61-73
+            const float t = 1.0f + (float)s * dt_step_;
+            const std::vector<float> te = sinusoidal_time_emb(t, W_, cfg.min_period, cfg.max_period);
+            for (int c = 0; c < W_; ++c) bias[(size_t)s * W_ + c] += te[c];
+        }
+    }
+    bias_step_.upload(bias.data(), bias.size() * sizeof(float));
+
+    if (arch_ == Arch::GR00T) {
+        // temb = l2(silu(l1(timesteps_proj(bucket)))) (DitHead::time_emb,
+        // src/modules/dit_head.cpp:135-137); per layer (scale, shift) =
+        // adaln_w . silu(temb) + adaln_b (src/layers/norm.h:39-41).
+        const std::vector<float> l1W = ck.f32("te.l1W"), l1b = ck.f32("te.l1b"), l2W = ck.f32("te.l2W"),
+                                 l2b = ck.f32("te.l2b");
+        std::vector<float> ada((size_t)steps_ * (L_ + 1) * 2 * W_, 0.f);
+        std::vector<std::vector<float>> aw(L_), ab(L_);
+        for (int l = 0; l < L_; ++l) {
+            aw[l] = ck.f32("ex." + std::to_string(l) + ".adaln_w");
+            ab[l] = ck.f32("ex." + std::to_string(l) + ".adaln_b");
+        }
+        for (int s = 0; s < steps_; ++s) {
+            std::vector<float> tp, t1(W_), temb(W_), st(W_);
+            timesteps_proj((int64_t)((double)s / (double)steps_ * 1000.0), tp);
+            host_linear(l1W.data(), l1b.data(), tp.data(), t1.data(), W_, 256);
+            for (auto& v : t1) v = host_silu(v);
+            host_linear(l2W.data(), l2b.data(), t1.data(), temb.data(), W_, W_);
+            for (int c = 0; c < W_; ++c) st[c] = host_silu(temb[c]);
+            const int nthr = std::min(default_cpu_threads(), L_);
+            std::vector<std::thread> pool;
+            for (int t = 0; t < nthr; ++t)
+                pool.emplace_back([&, t]() {
+                    for (int l = t; l < L_; l += nthr)
+                        host_linear(aw[l].data(), ab[l].data(), st.data(),
+                                    ada.data() + ((size_t)s * (L_ + 1) + l) * 2 * W_, 2 * W_, W_);
+                });
+            for (auto& th : pool) th.join();
+        }
+        ada_.upload(ada.data(), ada.size() * sizeof(float));
+    }
+}
+
+void FlowExpert::allocate(int B, int P) {
+    if (B == B_ && P == P_) return;
+    B_ = B;
+    P_ = P;
+    const size_t es = dtype_size(dt_);
+    for (LayerW& w : layers_) {
+        const int prefix = w.needs_prefix ? P : 0;
+        const int tmax = round_up(prefix + (w.is_self ? S_ : 0), 64);
+        w.kv.create(dt_, B, Hkv_, D_, tmax);
+        w.kv.n_prefix = prefix;
+    }
+    if (arch_ == Arch::SMOLVLA) {
+        tmp_kv_.create(dt_, B, Hkv_, D_, round_up(P, 64));
+        tmpk_.alloc((size_t)B * P * Hkv_ * D_ * es);
+        tmpv_.alloc((size_t)B * P * Hkv_ * D_ * es);
+    }
+    prefix_.alloc((size_t)B * P * Wv_ * es);
+    prefix_n_.alloc((size_t)B * P * Wv_ * es);
+    lead_.alloc((size_t)B * std::max(n_lead_, 1) * W_ * sizeof(float));
+    x0_.alloc((size_t)B * (S_ - n_lead_) * A_ * sizeof(float));
+    xt_.alloc((size_t)B * (S_ - n_lead_) * A_ * sizeof(float));
+    h_.alloc((size_t)B * S_ * W_ * es);
+    hn_.alloc((size_t)B * S_ * W_ * es);
+    q_.alloc((size_t)B * S_ * Hq_ * D_ * es);
+    att_.alloc((size_t)B * S_ * Hq_ * D_ * es);
+}
+
+void FlowExpert::prefill(const Inputs* in, int batch) {
+    if (!in || batch <= 0) throw std::invalid_argument("vla: prefill needs at least one observation");
+    const int views = in[0].n_img_views, n_lang = arch_ == Arch::GR00T ? 0 : in[0].n_lang;
+    if (views < 1 || views > max_views_) throw std::invalid_argument("vla: n_img_views out of range");
+    if (n_lang < 0 || n_lang > n_lang_max_) throw std::invalid_argument("vla: n_lang out of range");
+    for (int b = 0; b < batch; ++b) {
+        if (!in[b].precomputed_img_emb) throw std::invalid_argument("vla: precomputed_img_emb is required");
+        if (in[b].n_img_views != views || (arch_ != Arch::GR00T && in[b].n_lang != n_lang))
+            throw std::invalid_argument("vla: a batch shares one n_img_views and one n_lang");
+        if (n_lang > 0 && !in[b].lang_tokens) throw std::invalid_argument("vla: lang_tokens missing");
+        for (int i = 0; i < n_lang; ++i)
+            if (in[b].lang_tokens[i] < 0 || in[b].lang_tokens[i] >= vocab_)
+                throw std::invalid_argument("vla: language token outside the vocabulary");
+    }
+    const int n_img_tot = views * n_img_;
+    // SmolVLA pads the language block to its capacity and appends a state token
+    // (src/models/smolvla.cpp:1608-1612); pi0 uses the real length (pi0.cpp:526-528).
+    const int P = arch_ == Arch::SMOLVLA ? n_img_tot + n_lang_max_ + 1
+                  : arch_ == Arch::PI0   ? n_img_tot + n_lang
+                                         : n_img_tot;
+    allocate(batch, P);
+    const int B = batch;
+    Ctx C;  // prefill runs on the default stream and is synchronous
+
+    // ---- prefix embeddings, assembled in fp32 on the host
+    std::vector<float> pe((size_t)B * P * Wv_, 0.f);
+    const float lang_scale = std::sqrt((float)Wv_);
+    for (int b = 0; b < B; ++b) {
+        float* dst = pe.data() + (size_t)b * P * Wv_;
+        const float img_scale = arch_ == Arch::SMOLVLA ? lang_scale : 1.0f;  // smolvla.cpp:1363 vs pi0.cpp:554-555
+        for (size_t i = 0; i < (size_t)n_img_tot * Wv_; ++i) dst[i] = in[b].precomputed_img_emb[i] * img_scale;
+        if (arch_ != Arch::GR00T) {
+            const int rows = arch_ == Arch::SMOLVLA ? n_lang_max_ : n_lang;
+            for (int i = 0; i < rows; ++i) {
+                const int tok = i < n_lang ? in[b].lang_tokens[i] : 0;  // zero-padded ids, smolvla.cpp:1628-1629
+                const float* e = E_lang_.data() + (size_t)tok * Wv_;
+                float* row = dst + (size_t)(n_img_tot + i) * Wv_;
+                for (int c = 0; c < Wv_; ++c) row[c] = e[c] * lang_scale;
+            }
+        }
+        std::vector<float> st(max_state_, 0.f);
+        if (in[b].state) std::copy(in[b].state, in[b].state + max_state_, st.begin());
+        if (arch_ == Arch::SMOLVLA) {
+            host_linear(Wstate_.data(), bstate_.data(), st.data(), dst + (size_t)(P - 1) * Wv_, Wv_, max_state_);
+        } else {
+            std::vector<float> ld(W_);
+            host_linear(W_sp_.data(), b_sp_.data(), st.data(), ld.data(), W_, max_state_);
+            VLA_HIP(hipMemcpy(lead_.as<float>() + (size_t)b * W_, ld.data(), W_ * sizeof(float), hipMemcpyHostToDevice));
+        }
+    }
+    upload_as(prefix_, pe.data(), pe.size(), dt_);
+
+    // ---- positions and masks (smolvla.cpp:1633-1672, pi0.cpp:612-616)
+    pad_start_ = pad_end_ = 0;
+    if (rope_) {
+        const RopeSpec rs{D_, cfg.rope_freq_base};
+        std::vector<int32_t> pp(P), ps(S_), pc(S_);
+        for (int i = 0; i < P; ++i) pp[i] = i;
+        int suffix_base = P;
+        if (arch_ == Arch::SMOLVLA) {
+            const int state_pos = n_img_tot + n_lang;
+            pp[P - 1] = state_pos;
+            suffix_base = state_pos + 1;
+            pad_start_ = n_img_tot + n_lang;
+            pad_end_ = n_img_tot + n_lang_max_;
+        }
+        for (int i = 0; i < S_; ++i) {
+            ps[i] = suffix_base + i;
+            pc[i] = i;
+        }
+        rope_prefill_.build(rs, pp);
+        rope_self_.build(rs, ps);
+        rope_cross_.build(rs, pc);
+    }
+
+    // ---- prefix K/V of every layer, once per observation
+    Tensor xp = tensor_2d(prefix_.get(), dt_, Wv_, (int64_t)B * P);
+    Tensor xn = tensor_2d(prefix_n_.get(), dt_, Wv_, (int64_t)B * P);
+    const int kvd = Hkv_ * D_;
+    for (LayerW& w : layers_) {
+        if (!w.needs_prefix) continue;
+        Tensor Wkv = tensor_2d(w.Wkv_pre.get(), dt_, Wv_, 2 * kvd);
+        const float* bkv = w.bkv_pre ? w.bkv_pre.as<float>() : nullptr;
+        if (arch_ == Arch::GR00T) {
+            qkv_rope_append(C, xp, Wkv, bkv, P, 0, true, true, nullptr, nullptr, w.kv, 0);
+            continue;
+        }
+        rms_norm(C, xp, w.vlm_ln.get(), eps_, xn);
+        if (arch_ == Arch::SMOLVLA && !w.is_self) {
+            // expert_cross_kv: K = Wk_x . cachedK_flat, V = Wv_x . cachedV_flat, no second rotation
+            qkv_rope_append(C, xn, Wkv, bkv, P, 0, true, true, &rope_prefill_, nullptr, tmp_kv_, 0);
+            VLA_K(vla_kv_gather(tmp_kv_.k.get(), tmp_kv_.vt.get(), tmpk_.get(), tmpv_.get(), dt_, B, Hkv_, D_,
+                                tmp_kv_.t_max, 0, P, C.stream));
+            Tensor tk = tensor_2d(tmpk_.get(), dt_, kvd, (int64_t)B * P), tv = tensor_2d(tmpv_.get(), dt_, kvd, (int64_t)B * P);
+            Tensor Wkx = tensor_2d(w.Wk_x.get(), dt_, kvd, kvd), Wvx = tensor_2d(w.Wv_x.get(), dt_, kvd, kvd);
+            qkv_rope_append(C, tk, Wkx, nullptr, P, 0, true, false, nullptr, nullptr, w.kv, 0);
+            qkv_rope_append(C, tv, Wvx, nullptr, P, 0, false, true, nullptr, nullptr, w.kv, 0);
+        } else {
+            qkv_rope_append(C, xn, Wkv, bkv, P, 0, true, true, &rope_prefill_, nullptr, w.kv, 0);
+        }
+    }
+
+    // ---- initial noise
+    const size_t nx = (size_t)(S_ - n_lead_) * A_;
+    std::vector<float> x0((size_t)B * nx);
+    for (int b = 0; b < B; ++b) {
+        if (in[b].noise) {
+            std::copy(in[b].noise, in[b].noise + nx, x0.begin() + (size_t)b * nx);
+        } else {
+            std::normal_distribution<float> nd(0.f, 1.f);
+            for (size_t i = 0; i < nx; ++i) x0[(size_t)b * nx + i] = nd(rng_);
+        }
+    }
+    x0_.upload(x0.data(), x0.size() * sizeof(float));
+    VLA_HIP(hipDeviceSynchronize());
+}
+
+void FlowExpert::denoise(int chunks, void* stream) {
+    if (B_ == 0) throw std::logic_error("vla: denoise before prefill");
+    Ctx C;
+    C.stream = (hipStream_t)stream;
+    last_stream_ = C.stream;
+    const int B = B_, M = B * S_;
+    const float scale = 1.0f / std::sqrt((float)D_);
+    Tensor h = tensor_2d(h_.get(), dt_, W_, M), hn = tensor_2d(hn_.get(), dt_, W_, M);
+    Tensor att = tensor_2d(att_.get(), dt_, (int64_t)Hq_ * D_, M);
+    Tensor Q;
+    Q.data = q_.get();
+    Q.dtype = dt_;
+    Q.ne[0] = D_; Q.ne[1] = Hq_; Q.ne[2] = S_; Q.ne[3] = B;
+    const size_t xbytes = (size_t)B * (S_ - n_lead_) * A_ * sizeof(float);
+    for (int c = 0; c < chunks; ++c) {
+        VLA_HIP(hipMemcpyAsync(xt_.get(), x0_.get(), xbytes, hipMemcpyDeviceToDevice, C.stream));
+        for (int s = 0; s < steps_; ++s) {
+            VLA_K(vla_embed_suffix(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
+                                   n_lead_ ? lead_.as<float>() : nullptr, h.data, dt_, B, S_, n_lead_, A_, W_, C.stream));
+            for (int l = 0; l < L_; ++l) {
+                LayerW& w = layers_[l];
+                if (arch_ == Arch::GR00T) {
+                    const float* sc = ada_.as<float>() + ((size_t)s * (L_ + 1) + l) * 2 * W_;
+                    adaln(C, h, sc, sc + W_, eps_, hn);
+                } else {
+                    rms_norm(C, h, w.ln.get(), eps_, hn);
+                }
+                const float* bq = w.bqkv ? w.bqkv.as<float>() : nullptr;
+                MaskSpec mask;
+                mask.pad_start = pad_start_;
+                mask.pad_end = pad_end_;
+                int n_keys;
+                if (w.is_self) {
+                    Tensor Wqkv = tensor_2d(w.Wqkv.get(), dt_, W_, (int64_t)(Hq_ + 2 * Hkv_) * D_);
+                    qkv_rope_append(C, hn, Wqkv, bq, S_, Hq_, true, true, rope_ ? &rope_self_ : nullptr, Q.data, w.kv,
+                                    w.kv.n_prefix);
+                    mask.kind = suffix_mask_;
+                    n_keys = w.kv.n_prefix + S_;
+                } else {
+                    Tensor Wq = tensor_2d(w.Wqkv.get(), dt_, W_, (int64_t)Hq_ * D_);
+                    qkv_rope_append(C, hn, Wq, bq, S_, Hq_, false, false, rope_ ? &rope_cross_ : nullptr, Q.data, w.kv, 0);
+                    mask.kind = VLA_MASK_NONE;
+                    n_keys = w.kv.n_prefix;
+                }
+                flash_attention(C, Q, w.kv, n_keys, mask, scale, att);
+                Tensor Wo = tensor_2d(w.Wo.get(), dt_, (int64_t)Hq_ * D_, W_);
+                linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
+            }
+            if (arch_ == Arch::GR00T) {
+                const float* z = ada_.as<float>() + ((size_t)s * (L_ + 1) + L_) * 2 * W_;  // zeros: plain LayerNorm
+                adaln(C, h, z, z + W_, final_eps_, hn);
+            } else {
+                rms_norm(C, h, final_norm_.get(), eps_, hn);
+            }
+            VLA_K(vla_euler_step(xt_.as<float>(), hn.data, W_out_.as<float>(), b_out_.as<float>(), dt_, B, S_, n_lead_,
+                                 A_, W_, dt_step_, C.stream));
+        }
+    }
+}
+
+std::vector<float> FlowExpert::fetch() {
+    VLA_HIP(hipStreamSynchronize(last_stream_));
+    const int Sa = S_ - n_lead_;
+    std::vector<float> out((size_t)B_ * Sa * A_);
+    xt_.download(out.data(), out.size() * sizeof(float));
+    for (size_t r = 0; r < (size_t)B_ * Sa; ++r)
+        for (int j = (int)cfg.real_action_dim; j < A_; ++j) out[r * A_ + j] = 0.0f;
+    return out;
+}
+
+}  // namespace
+
+ModelArch* flow_expert_create(const Checkpoint& ck) { return new FlowExpert(ck); }
+
+}  // namespace vla

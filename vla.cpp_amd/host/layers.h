@@ -1,0 +1,152 @@
+// Host-side op fragments with the names and argument order of the reference's
+// src/layers (attn.h:27-58, rope.h:28-48, linear.h:24-27, norm.h:27-46,
+// embed.h:61-73).  The reference's versions record ggml graph nodes on
+// ggml_tensor*; these run eagerly on a HIP stream over a light tensor view and
+// the resident KV cache, by calling the kernel C ABI (include/vla_kernels.h)
+// and nothing else.
+#pragma once
+
+#include <cmath>
+#include <cstdint>
+#include <vector>
+
+#include "device.h"
+#include "vla_kernels.h"
+
+namespace vla {
+
+// ne[0] is the innermost dimension, as in ggml.
+struct Tensor {
+    void* data = nullptr;
+    int dtype = VLA_DT_F32;
+    int64_t ne[4] = {1, 1, 1, 1};
+    int64_t rows() const { return ne[1] * ne[2] * ne[3]; }
+};
+
+inline Tensor tensor_2d(void* data, int dtype, int64_t ne0, int64_t ne1) {
+    Tensor t;
+    t.data = data;
+    t.dtype = dtype;
+    t.ne[0] = ne0;
+    t.ne[1] = ne1;
+    return t;
+}
+
+// Execution context in place of ggml_context: the stream every op is queued on.
+struct Ctx {
+    hipStream_t stream = nullptr;
+};
+
+// rope.h:28-38 without the fields this path never varies (NeoX only, freq_scale
+// 1, no YaRN).  The angle tables are built once per observation on the host.
+struct RopeSpec {
+    int n_dims = 0;
+    float freq_base = 10000.0f;
+};
+
+struct RopeTable {
+    DevBuf cos, sin;
+    int rows = 0;
+    void build(const RopeSpec& r, const std::vector<int32_t>& pos) {
+        rows = (int)pos.size();
+        const size_t n = pos.size() * (size_t)(r.n_dims / 2);
+        std::vector<float> c(n), s(n);
+        VLA_K(vla_rope_tables_host(pos.data(), rows, r.n_dims, (double)r.freq_base, c.data(), s.data()));
+        cos.upload(c.data(), n * sizeof(float));
+        sin.upload(s.data(), n * sizeof(float));
+    }
+};
+
+// One layer's resident cache: K [B][Hkv][t_max][D], V^T [B][Hkv][D][t_max].
+struct KVLayer {
+    DevBuf k, vt;
+    int dtype = VLA_DT_F32, batch = 0, n_kv_heads = 0, head_dim = 0, t_max = 0;
+    int n_prefix = 0;  // tokens [0, n_prefix) are the observation's prefix
+    void create(int dt, int B, int Hkv, int D, int tmax) {
+        dtype = dt; batch = B; n_kv_heads = Hkv; head_dim = D; t_max = tmax;
+        const size_t bytes = (size_t)B * Hkv * D * tmax * dtype_size(dt);
+        k.alloc(bytes);
+        vt.alloc(bytes);
+        k.zero();
+        vt.zero();
+    }
+};
+
+// Mask as the attention kernel generates it (masks are data in the reference:
+// src/models/smolvla.cpp:1651-1669, src/models/pi0.cpp:638-653).
+struct MaskSpec {
+    int kind = VLA_MASK_NONE;
+    int pad_start = 0, pad_end = 0;
+};
+
+// linear.h:24-27: y = W x + b, optionally fused with the residual add that
+// follows it in every layer (h1 = x_in + Wo att).
+inline void linear(Ctx& C, const Tensor& W, const float* b, const Tensor& x, const void* residual, Tensor& y) {
+    VLA_K(vla_linear(x.data, W.data, b, residual, y.data, x.dtype, y.dtype, (int)x.rows(), (int)W.ne[1], (int)W.ne[0],
+                     C.stream));
+}
+
+// norm.h:31-34.
+inline void rms_norm(Ctx& C, const Tensor& x, const void* w, float eps, Tensor& y) {
+    VLA_K(vla_rms_norm(x.data, w, y.data, x.dtype, (int)x.rows(), (int)x.ne[0], eps, C.stream));
+}
+
+// norm.h:37-46 with the (scale, shift) pair already evaluated for this step.
+inline void adaln(Ctx& C, const Tensor& x, const float* sc, const float* sh, float eps, Tensor& y) {
+    VLA_K(vla_adaln(x.data, sc, sh, y.data, x.dtype, (int)x.rows(), (int)x.ne[0], eps, C.stream));
+}
+
+// rope.h:40-48 on a token-major tensor [D, H, rows].
+inline void rope(Ctx& C, const RopeTable& tab, Tensor& x) {
+    VLA_K(vla_rope_neox(x.data, tab.cos.as<float>(), tab.sin.as<float>(), x.dtype, (int)(x.ne[2] * x.ne[3]), tab.rows,
+                        (int)x.ne[1], (int)x.ne[0], C.stream));
+}
+
+// The QKV projections, head split, rotation and ggml_concat of a layer
+// (src/models/smolvla.cpp:821-833) as one launch.  `S` rows per observation land
+// at tokens [kv.n_prefix, kv.n_prefix + S) of the cache unless tok_offset >= 0.
+inline void qkv_rope_append(Ctx& C, const Tensor& x, const Tensor& W, const float* bias, int S, int n_q_heads,
+                            bool has_k, bool has_v, const RopeTable* tab, void* q_out, KVLayer& kv, int tok_offset) {
+    VLA_K(vla_attn_qkv_rope(x.data, W.data, bias, x.dtype, (int)x.rows(), (int)x.ne[0], S, n_q_heads, kv.n_kv_heads,
+                            has_k ? 1 : 0, has_v ? 1 : 0, kv.head_dim, tab ? tab->cos.as<float>() : nullptr,
+                            tab ? tab->sin.as<float>() : nullptr, q_out, kv.k.get(), kv.vt.get(), kv.t_max, tok_offset,
+                            C.stream));
+}
+
+// attn.h:48-58 (flash_attention) over the resident cache: Q [D, Hq, S, B]
+// token-major, keys [0, n_keys).
+inline void flash_attention(Ctx& C, const Tensor& Q, const KVLayer& kv, int n_keys, const MaskSpec& mask, float scale,
+                            Tensor& out) {
+    VLA_K(vla_attn_prefix_suffix(Q.data, kv.k.get(), kv.vt.get(), out.data, Q.dtype, (int)Q.ne[3], (int)Q.ne[2],
+                                 (int)Q.ne[1], kv.n_kv_heads, (int)Q.ne[0], kv.t_max, n_keys, scale, mask.kind,
+                                 kv.n_prefix, mask.pad_start, mask.pad_end, nullptr, C.stream));
+}
+
+// embed.h:61-73, log-spaced periods, sin first.
+inline std::vector<float> sinusoidal_time_emb(double t, int64_t dim, double min_p, double max_p) {
+    const int64_t half = dim / 2;
+    std::vector<float> out((size_t)dim);
+    for (int64_t i = 0; i < half; ++i) {
+        const double frac = (half == 1) ? 0.0 : double(i) / double(half - 1);
+        const double period = min_p * std::pow(max_p / min_p, frac);
+        const double s = (2.0 * 3.14159265358979323846 / period) * t;
+        out[i] = (float)std::sin(s);
+        out[half + i] = (float)std::cos(s);
+    }
+    return out;
+}
+
+// embed.h:32-44, cos first.
+inline void timesteps_proj(int64_t bucket, std::vector<float>& out) {
+    const int64_t half = 128;
+    const float lm = std::log(10000.0f);
+    const float t = (float)bucket;
+    out.assign(256, 0.0f);
+    for (int64_t i = 0; i < half; ++i) {
+        const float emb = t * std::exp(-lm * (float)i / (float)(half - 1));
+        out[i] = std::cos(emb);
+        out[half + i] = std::sin(emb);
+    }
+}
+
+}  // namespace vla

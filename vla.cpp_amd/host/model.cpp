@@ -1,0 +1,73 @@
+// Engine API: checkpoint loading, architecture dispatch and the one-shot
+// predict() of src/model.cpp:200-296 over this library's architectures.
+
+#include "model.h"
+
+#include <algorithm>
+#include <chrono>
+#include <cstdlib>
+#include <thread>
+
+#include "checkpoint.h"
+#include "device.h"
+
+namespace vla {
+
+int default_cpu_threads() {
+    if (const char* e = std::getenv("VLA_N_THREADS")) {
+        char* end = nullptr;
+        const long n = std::strtol(e, &end, 10);
+        if (end && *end == '\0' && n > 0 && n <= 1024) return (int)n;
+        std::fprintf(stderr, "vla: ignoring VLA_N_THREADS='%s'\n", e);
+    }
+    const unsigned hw = std::thread::hardware_concurrency();
+    return hw == 0 ? 4 : (int)std::min(hw, 16u);
+}
+
+bool config_is_sane(const Config& c) {
+    return c.real_action_dim <= c.max_action_dim && c.real_state_dim <= c.max_state_dim && c.real_action_dim >= 0 &&
+           c.real_state_dim >= 0;
+}
+
+Model* model_load(const std::string&, const std::string& ckpt_path, const std::string&) {
+    Checkpoint ck(ckpt_path);
+    const std::string arch = ck.str("arch");
+    ModelArch* a = nullptr;
+    if (arch == "smolvla" || arch == "pi0" || arch == "gr00t_n1d5") a = flow_expert_create(ck);
+    else if (arch == "bitvla") a = bitvla_create(ck);
+    else throw std::runtime_error("vla: unknown architecture '" + arch + "'");
+    Model* m = new Model();
+    m->arch = a;
+    return m;
+}
+
+void model_free(Model* m) {
+    if (!m) return;
+    delete m->arch;
+    delete m;
+}
+
+const Config& model_config(const Model* m) { return m->arch->cfg; }
+const Stats& last_stats(const Model* m) { return m->arch->stats; }
+
+std::vector<float> predict(Model* m, const Inputs& in) {
+    using clk = std::chrono::steady_clock;
+    const auto t0 = clk::now();
+    ModelArch& a = *m->arch;
+    a.stats = Stats{};
+    a.prefill(&in, 1);
+    const auto t1 = clk::now();
+    a.denoise(1, nullptr);
+    std::vector<float> out = a.fetch();
+    const auto t2 = clk::now();
+    const auto ms = [](clk::time_point x, clk::time_point y) { return std::chrono::duration<float, std::milli>(y - x).count(); };
+    a.stats.ms_total = ms(t0, t2);
+    a.stats.ms_inference = ms(t0, t2);
+    if (in.timing_detail == TimingDetail::PHASE) {
+        a.stats.ms_prefill = ms(t0, t1);
+        a.stats.ms_denoise = ms(t1, t2);
+    }
+    return out;
+}
+
+}  // namespace vla
