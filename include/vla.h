@@ -151,6 +151,9 @@ VLA_API int32_t vla_prefill_batch(vla_model * m, const vla_inputs * in, int32_t 
  * re-staged before every chunk) on `stream` (a hipStream_t or NULL), without
  * synchronising. */
 VLA_API int32_t vla_denoise_async(vla_model * m, int32_t chunks, void * stream);
+/* Same, counted in denoise steps (the step index cycles through the chunk), for
+ * timing a given number of steps. */
+VLA_API int32_t vla_denoise_steps_async(vla_model * m, int32_t n_steps, void * stream);
 /* Synchronises and copies the last chunk's actions:
  * [batch, n_actions, max_action_dim] floats, malloc'd. */
 VLA_API int32_t vla_fetch_actions(vla_model * m, float ** out_actions, int64_t * out_n);

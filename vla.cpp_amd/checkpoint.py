@@ -189,11 +189,11 @@ def synth_weights(cfg, seed=0x5EED):
 _F32_NAMES = ("prefix.", "act.", "te.")
 
 
-def write_synthetic(path, cfg, weights, ladder_pack=None):
+def write_synthetic(path, cfg, weights, ladder_pack=None, plain_pack=None):
     """Write `weights` (from synth_weights) as a VLAW file.  BitVLA ternary tensors are
     stored ladder-packed ("*.i2" + "*.ws") when ladder_pack (a function
-    int8 [N,K] -> uint8 bytes) is given, else as dequantised fp32 the loader
-    re-quantises."""
+    int8 [N,K] -> uint8 bytes) is given, in the gfx950 word order ("*.p2" + "*.ws") when
+    plain_pack is given, else as dequantised fp32 the loader re-quantises."""
     bf = cfg["dtype"] == "bf16"
     out = {}
     for name, t in weights.items():
@@ -201,6 +201,9 @@ def write_synthetic(path, cfg, weights, ladder_pack=None):
             base = name[:-2]
             if ladder_pack is not None:
                 out[base + ".i2"] = np.ascontiguousarray(ladder_pack(t), np.uint8)
+                out[base + ".ws"] = weights[base + ".ws"]
+            elif plain_pack is not None:
+                out[base + ".p2"] = np.ascontiguousarray(plain_pack(t), np.uint8)
                 out[base + ".ws"] = weights[base + ".ws"]
             else:
                 # fp32 weights whose absmean quantisation gives back (t, scale): t * scale

@@ -4,16 +4,20 @@
 // softmax, fp32 scores / statistics / accumulation in every mode (the
 // reference's precision split, src/act_dtype.h:29-35).
 //
-// Work decomposition.  A workgroup owns one (batch, kv head) and a group of
-// 32-row tiles of that head's query rows; the rows of all g = Hq/Hkv query
-// heads sharing the kv head are flattened (row = head_in_group * S + s), so a
-// K/V tile staged in LDS is read once per query-head group (GQA / MQA sharing)
-// instead of being copied per query head as bitvla_repeat_kv_bf16 does
-// (src/kernels/bitvla/bitvla_lm_cuda.cu:181-190).  Each 64-lane wavefront owns
-// one row tile.
+// Work decomposition.  A workgroup owns one (batch, kv head) pair, a group of
+// 32-row tiles of that head's query rows and (optionally) a slice of the keys.
+// The rows of all g = Hq/Hkv query heads sharing the kv head are flattened
+// (row = head_in_group * S + s), so a K/V tile staged in LDS is read once per
+// query-head group (GQA / MQA sharing) instead of being copied per query head
+// as bitvla_repeat_kv_bf16 does (src/kernels/bitvla/bitvla_lm_cuda.cu:181-190).
+// Each 64-lane wavefront owns one row tile.
 //
-// The cache layout makes both tiles plain block copies: K [t][D] of one head is
-// contiguous, V^T [D][t] has the keys innermost.
+// Memory.  The cache layout makes both tiles plain block copies: K [t][D] of one
+// head is contiguous, V^T [D][t] has the keys innermost.  A tile's 16-byte
+// global loads are all issued before any is consumed, and the next tile's loads
+// are in flight while the current tile is multiplied.  Workgroups that share a
+// (batch, kv head) get linear ids equal modulo 8, so they land on the same XCD
+// and share its L2.
 //
 // MFMA formulation (transposed, so softmax statistics are per lane):
 //   S^T[key][row] = K . Q^T     A = K tile rows (lane r <-> key), B = Q rows
@@ -24,8 +28,13 @@
 // k-slot (g, e) of that product is bound to key 8(e/4)+4g+(e%4), and V^T is
 // fetched from LDS in the same order.  No score matrix is ever written
 // (the reference's explicit path writes and re-reads Hq*S*T scores).
+//
+// Few query rows (single-token decode, batch 1): the keys are split across
+// workgroups, each writes an unnormalised partial (max, sum, O) and a second
+// kernel merges them.
 
 #include <math.h>
+#include <stdlib.h>
 
 #include "common.h"
 #include "vla_kernels.h"
@@ -45,6 +54,9 @@ struct AttnArgs {
     float scale;
     int mask_kind, n_prefix, pad_start, pad_end;
     const float* mask;
+    int n_groups, n_split, tiles_per_split, r_pad;
+    float* part_o;   // [pair][split][r_pad][D]
+    float* part_ml;  // [pair][split][r_pad][2]
 };
 
 template <typename T> struct AT;
@@ -55,7 +67,7 @@ template <> struct AT<bf16_t> {
         acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b),
                                                       acc, 0, 0, 0);
     }
-    __device__ static __forceinline__ float fexp(float x) { return __expf(x); }
+    __device__ static __forceinline__ float fexp2(float x) { return __builtin_amdgcn_exp2f(x); }
 };
 template <> struct AT<float> {
     static constexpr int EB = 4;
@@ -65,7 +77,7 @@ template <> struct AT<float> {
 #pragma unroll
         for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[t], fb[t], acc, 0, 0, 0);
     }
-    __device__ static __forceinline__ float fexp(float x) { return expf(x); }
+    __device__ static __forceinline__ float fexp2(float x) { return exp2f(x); }
 };
 
 template <typename T, int D, int NW>
@@ -78,22 +90,40 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     constexpr int KS = D * EB + 16;         // LDS stride of a K row (bytes)
     constexpr int VS = TK * EB + 16;        // LDS stride of a V^T row (bytes)
     constexpr int NT = NW * 64;
+    constexpr int KV_PER_ROW = D * EB / 16;   // 16-byte vectors per K row
+    constexpr int VV_PER_ROW = TK * EB / 16;  // 16-byte vectors per V^T row
+    constexpr int EPV = 16 / EB;              // elements per vector
+    constexpr int NVEC = TK * KV_PER_ROW;     // vectors in a K tile == vectors in a V^T tile
+    constexpr int IT = (NVEC + NT - 1) / NT;  // vectors per thread per tile and operand
+    constexpr bool PREFETCH = (2 * IT <= 16); // keep the next tile in registers across the multiply
     static_assert(D % CE == 0 && (D * EB) % 16 == 0, "head_dim must be whole MFMA groups and 16-byte rows");
+    static_assert(NVEC == D * VV_PER_ROW, "K and V^T tiles hold the same number of vectors");
 
     __shared__ __attribute__((aligned(16))) unsigned char ldsK[TK * KS];
     __shared__ __attribute__((aligned(16))) unsigned char ldsV[DP * VS];
 
+    // ---- XCD-aware decode of the linear workgroup id
+    const int GS = a.n_groups * a.n_split;
+    const int id = blockIdx.x;
+    const int pair = (id / (8 * GS)) * 8 + (id & 7);
+    if (pair >= a.batch * a.Hkv) return;
+    const int t_idx = (id >> 3) % GS;
+    const int group = t_idx / a.n_split, split = t_idx % a.n_split;
+    const int b = pair / a.Hkv, hk = pair % a.Hkv;
+
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, r = lane & 31;
-    const int hk = blockIdx.y, b = blockIdx.z;
     const int grp = a.Hq / a.Hkv;
     const int R = grp * a.S;
-    const int row = (blockIdx.x * NW + wave) * 32 + r;
-    const bool wave_active = (blockIdx.x * NW + wave) * 32 < R;
+    const int row = (group * NW + wave) * 32 + r;
+    const bool wave_active = (group * NW + wave) * 32 < R;
     const bool row_valid = row < R;
     const int hg = row_valid ? row / a.S : 0;
     const int s = row_valid ? row % a.S : 0;
     const int h = hk * grp + hg;
+
+    const int k_begin = split * a.tiles_per_split * TK;
+    const int k_end = min(a.n_keys, k_begin + a.tiles_per_split * TK);
 
     // Q fragments: B operand, lane (g, r) holds 16 bytes of query row r per group.
     u32x4_t qf[NQ];
@@ -111,50 +141,97 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     for (int db = 0; db < NDB; ++db)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+    // Scores are kept in the base-2 exponent domain: s2 = score * scale * log2(e).
     float m_run = -INFINITY, l_run = 0.f;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float c2 = a.scale * LOG2E;
 
     const unsigned char* kbase = (const unsigned char*)a.k_cache + ((long)b * a.Hkv + hk) * a.t_max * D * EB;
     const unsigned char* vbase = (const unsigned char*)a.vt_cache + ((long)b * a.Hkv + hk) * D * (long)a.t_max * EB;
 
-    for (int k0 = 0; k0 < a.n_keys; k0 += TK) {
-        __syncthreads();  // previous tile fully consumed
-        // K tile: TK rows of D*EB contiguous bytes.
-        constexpr int KV_PER_ROW = D * EB / 16;
-        for (int v = tid; v < TK * KV_PER_ROW; v += NT) {
+    u32x4_t kreg[IT], vreg[IT];
+    auto load_k = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int v = tid + i * NT;
             const int key = v / KV_PER_ROW, c = v % KV_PER_ROW;
             u32x4_t val = {0u, 0u, 0u, 0u};
-            if (k0 + key < a.n_keys) val = *reinterpret_cast<const u32x4_t*>(kbase + ((long)(k0 + key) * D * EB) + c * 16);
-            *reinterpret_cast<u32x4_t*>(ldsK + key * KS + c * 16) = val;
+            if (v < NVEC && k0 + key < a.n_keys)
+                val = *reinterpret_cast<const u32x4_t*>(kbase + ((long)(k0 + key) * D * EB) + c * 16);
+            kreg[i] = val;
         }
-        // V^T tile: D rows of TK keys; keys past n_keys are zeroed element-wise so
-        // that stale cache contents cannot reach the accumulators.
-        constexpr int VV_PER_ROW = TK * EB / 16;
-        constexpr int EPV = 16 / EB;  // elements per vector
-        for (int v = tid; v < D * VV_PER_ROW; v += NT) {
+    };
+    auto load_v = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int v = tid + i * NT;
             const int d = v / VV_PER_ROW, c = v % VV_PER_ROW;
             const int key = k0 + c * EPV;
             u32x4_t val = {0u, 0u, 0u, 0u};
-            if (key < a.n_keys) {
-                val = *reinterpret_cast<const u32x4_t*>(vbase + ((long)d * a.t_max + key) * EB);
-                if (key + EPV > a.n_keys) {
-                    const int nvalid = a.n_keys - key;
-                    if (EB == 2) {
+            if (v < NVEC && key < a.n_keys) val = *reinterpret_cast<const u32x4_t*>(vbase + ((long)d * a.t_max + key) * EB);
+            vreg[i] = val;
+        }
+    };
+    auto store_k = [&]() {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint32_t lo = (2 * e < nvalid) ? 0xffffu : 0u, hi = (2 * e + 1 < nvalid) ? 0xffff0000u : 0u;
-                            val[e] &= (lo | hi);
-                        }
-                    } else {
+        for (int i = 0; i < IT; ++i) {
+            const int v = tid + i * NT;
+            if (v < NVEC) *reinterpret_cast<u32x4_t*>(ldsK + (v / KV_PER_ROW) * KS + (v % KV_PER_ROW) * 16) = kreg[i];
+        }
+    };
+    // Keys past n_keys are zeroed element-wise so that stale cache contents cannot
+    // reach the accumulators (0 * NaN).
+    auto store_v = [&](int k0) {
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (e >= nvalid) val[e] = 0u;
+        for (int i = 0; i < IT; ++i) {
+            const int v = tid + i * NT;
+            const int d = v / VV_PER_ROW, c = v % VV_PER_ROW;
+            const int key = k0 + c * EPV;
+            u32x4_t val = vreg[i];
+            if (key < a.n_keys && key + EPV > a.n_keys) {
+                const int nvalid = a.n_keys - key;
+                if (EB == 2) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t lo = (2 * e < nvalid) ? 0xffffu : 0u, hi = (2 * e + 1 < nvalid) ? 0xffff0000u : 0u;
+                        val[e] &= (lo | hi);
                     }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (e >= nvalid) val[e] = 0u;
                 }
             }
-            *reinterpret_cast<u32x4_t*>(ldsV + d * VS + c * 16) = val;
+            if (v < NVEC) *reinterpret_cast<u32x4_t*>(ldsV + d * VS + c * 16) = val;
+        }
+    };
+
+    if (PREFETCH && k_begin < k_end) {
+        load_k(k_begin);
+        load_v(k_begin);
+    }
+    for (int k0 = k_begin; k0 < k_end; k0 += TK) {
+        __syncthreads();  // previous tile fully consumed
+        if (PREFETCH) {
+            store_k();
+            store_v(k0);
+        } else {
+            load_k(k0);
+            load_v(k0);
+            store_k();
+            store_v(k0);
         }
         __syncthreads();
+        if (PREFETCH && k0 + TK < k_end) {
+            load_k(k0 + TK);
+            load_v(k0 + TK);
+        }
         if (!wave_active) continue;
+
+        // Whether any key of this tile can be hidden from any row (uniform per tile).
+        const bool tile_masked = a.mask != nullptr || k0 + TK > a.n_keys ||
+                                 (k0 < a.pad_end && k0 + TK > a.pad_start && a.pad_start < a.pad_end) ||
+                                 (a.mask_kind != VLA_MASK_NONE && k0 + TK > a.n_prefix);
 
         // ---- scores S^T for the two 32-key blocks of the tile
         float p[2][16];
@@ -169,38 +246,47 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
                 const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(ldsK + (kb * 32 + r) * KS + (c * CE + g * (CE / 2)) * EB);
                 A::mma(sc, kf, qf[c]);
             }
+            if (!tile_masked) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int key = k0 + kb * 32 + 8 * j + 4 * g + i;
-                    float v = sc[4 * j + i] * a.scale;
-                    bool blocked = key >= a.n_keys;
-                    if (a.mask) {
-                        if (!blocked) v += a.mask[(long)s * a.n_keys + key];
-                    } else if (key < a.n_prefix) {
-                        blocked |= (key >= a.pad_start && key < a.pad_end);
-                    } else {
-                        const int si = key - a.n_prefix;
-                        if (a.mask_kind == VLA_MASK_CAUSAL_SUFFIX) blocked |= si > s;
-                        else if (a.mask_kind == VLA_MASK_PI0_STATE) blocked |= (s == 0 && si != 0);
-                    }
-                    v = blocked ? -INFINITY : v;
-                    p[kb][4 * j + i] = v;
+                for (int i = 0; i < 16; ++i) {
+                    const float v = sc[i] * c2;
+                    p[kb][i] = v;
                     m_tile = fmaxf(m_tile, v);
                 }
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int key = k0 + kb * 32 + 8 * j + 4 * g + i;
+                        float v = sc[4 * j + i] * c2;
+                        bool blocked = key >= a.n_keys;
+                        if (a.mask) {
+                            if (!blocked) v += a.mask[(long)s * a.n_keys + key] * LOG2E;
+                        } else if (key < a.n_prefix) {
+                            blocked |= (key >= a.pad_start && key < a.pad_end);
+                        } else {
+                            const int si = key - a.n_prefix;
+                            if (a.mask_kind == VLA_MASK_CAUSAL_SUFFIX) blocked |= si > s;
+                            else if (a.mask_kind == VLA_MASK_PI0_STATE) blocked |= (s == 0 && si != 0);
+                        }
+                        v = blocked ? -INFINITY : v;
+                        p[kb][4 * j + i] = v;
+                        m_tile = fmaxf(m_tile, v);
+                    }
+            }
         }
         m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
         const float m_new = fmaxf(m_run, m_tile);
         // m_new == -inf: nothing visible yet, keep everything at zero.
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = A::fexp(m_run - m_use);  // exp(-inf) = 0 on the first visible tile
+        const float alpha = A::fexp2(m_run - m_use);  // 2^-inf = 0 on the first visible tile
         float psum = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const float e = A::fexp(p[kb][i] - m_use);
+                const float e = A::fexp2(p[kb][i] - m_use);
                 p[kb][i] = e;
                 psum += e;
             }
@@ -222,17 +308,13 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
                     // ~16 mantissa bits): the P.V product then matches an fp32-probability
                     // reference instead of carrying an extra 2^-9 rounding per weight.
                     const float* pp = &p[kb][hh * 8];
-                    float lo[8];
-                    uint32_t hi16[8];
+                    u32x4_t pf, pl;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        hi16[e] = f2bf(pp[e]);
-                        lo[e] = pp[e] - bf2f((bf16_t)hi16[e]);
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t hi = pack_bf2(pp[2 * e], pp[2 * e + 1]);
+                        pf[e] = hi;
+                        pl[e] = pack_bf2(pp[2 * e] - __uint_as_float(hi << 16), pp[2 * e + 1] - __uint_as_float(hi & 0xffff0000u));
                     }
-                    const u32x4_t pf = {hi16[0] | (hi16[1] << 16), hi16[2] | (hi16[3] << 16), hi16[4] | (hi16[5] << 16),
-                                        hi16[6] | (hi16[7] << 16)};
-                    const u32x4_t pl = {pack_bf2(lo[0], lo[1]), pack_bf2(lo[2], lo[3]), pack_bf2(lo[4], lo[5]),
-                                        pack_bf2(lo[6], lo[7])};
                     const int key_off = (kb * 32 + hh * 16 + 4 * g) * EB;
 #pragma unroll
                     for (int db = 0; db < NDB; ++db) {
@@ -262,6 +344,25 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     }
 
     if (!row_valid) return;
+    if (a.n_split > 1) {
+        // unnormalised partial for the merge kernel
+        const long prow = ((long)pair * a.n_split + split) * a.r_pad + row;
+        if (g == 0) {
+            a.part_ml[prow * 2] = m_run;
+            a.part_ml[prow * 2 + 1] = l_run;
+        }
+        float* po = a.part_o + prow * D;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int d = db * 32 + 8 * j + 4 * g;
+                if (d >= D) continue;
+                const f32x4_t pk = {o[db][4 * j], o[db][4 * j + 1], o[db][4 * j + 2], o[db][4 * j + 3]};
+                *reinterpret_cast<f32x4_t*>(po + d) = pk;
+            }
+        return;
+    }
     const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
     unsigned char* orow = (unsigned char*)a.out + (((long)b * a.S + s) * a.Hq + h) * D * EB;
 #pragma unroll
@@ -282,26 +383,110 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
         }
 }
 
+// Merge of key-split partials: one thread per (pair, row, d).
+template <typename T>
+__global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, T* __restrict__ out,
+                                  int n_pairs, int n_split, int r_pad, int R, int S, int Hq, int Hkv, int D) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)n_pairs * R * D;
+    if (i >= total) return;
+    const int d = (int)(i % D);
+    const int row = (int)((i / D) % R);
+    const int pair = (int)(i / ((long)D * R));
+    float m = -INFINITY;
+    for (int sp = 0; sp < n_split; ++sp) m = fmaxf(m, part_ml[(((long)pair * n_split + sp) * r_pad + row) * 2]);
+    float l = 0.f, acc = 0.f;
+    if (m > -INFINITY) {
+        for (int sp = 0; sp < n_split; ++sp) {
+            const long prow = ((long)pair * n_split + sp) * r_pad + row;
+            const float w = exp2f(part_ml[prow * 2] - m);
+            l += part_ml[prow * 2 + 1] * w;
+            acc += part_o[prow * D + d] * w;
+        }
+    }
+    const int grp = Hq / Hkv, b = pair / Hkv, hk = pair % Hkv;
+    const int h = hk * grp + row / S, s = row % S;
+    Elem<T>::store(out + (((long)b * S + s) * Hq + h) * D + d, l > 0.f ? acc / l : 0.f);
+}
+
+// Workspace for key-split partials, grown on demand (never under stream capture:
+// run the shape once before capturing it).
+float* g_ws = nullptr;
+size_t g_ws_floats = 0;
+
+float* workspace(size_t floats) {
+    if (floats > g_ws_floats) {
+        if (g_ws) (void)hipFree(g_ws);
+        g_ws = nullptr;
+        g_ws_floats = 0;
+        const size_t want = floats < (1u << 20) ? (1u << 20) : floats;
+        if (hipMalloc((void**)&g_ws, want * sizeof(float)) != hipSuccess) return nullptr;
+        g_ws_floats = want;
+    }
+    return g_ws;
+}
+
+template <typename T, int D, int NW>
+int launch_nw(AttnArgs& a, hipStream_t st) {
+    const int n_pairs = a.batch * a.Hkv;
+    const int grid = (n_pairs + 7) / 8 * 8 * a.n_groups * a.n_split;
+    attn_kernel<T, D, NW><<<grid, NW * 64, 0, st>>>(a);
+    if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
+    if (a.n_split > 1) {
+        const int R = (a.Hq / a.Hkv) * a.S;
+        const long total = (long)n_pairs * R * D;
+        attn_merge_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs,
+                                                                              a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
+        if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
+    }
+    return VLA_K_OK;
+}
+
 template <typename T, int D>
-int launch_d(const AttnArgs& a, vla_stream_t stream) {
+int launch_d(AttnArgs& a, vla_stream_t stream) {
+    constexpr int NW_MAX = 4;  // at most one wavefront of a workgroup per SIMD
     const int R = (a.Hq / a.Hkv) * a.S;
     const int n_tiles = (R + 31) / 32;
-    // Fewer wavefronts per workgroup -> more workgroups; go down until the grid
-    // covers the 256 compute units, but keep at least two wavefronts loading.
-    const long pairs = (long)a.batch * a.Hkv;
-    int nw = 4;
-    if (n_tiles < 4 || pairs * ((n_tiles + 3) / 4) < 512) nw = 2;
-    if (n_tiles < 2) nw = 1;
+    // One wavefront per row tile; more than NW_MAX tiles are spread evenly over groups.
+    a.n_groups = (n_tiles + NW_MAX - 1) / NW_MAX;
+    const int nw = (n_tiles + a.n_groups - 1) / a.n_groups;
+    a.r_pad = a.n_groups * nw * 32;
+    // Too few workgroups to cover the 256 compute units: split the keys as well.
+    const long wgs = (long)a.batch * a.Hkv * a.n_groups;
+    const int key_tiles = (a.n_keys + TK - 1) / TK;
+    a.n_split = 1;
+    // Only worthwhile while a partial (r_pad rows of D+2 floats) stays small next to the
+    // K/V slice it summarises; with many query rows the partials would outweigh the cache.
+    const size_t partial_bytes = (size_t)a.r_pad * (D + 2) * 4, tile_bytes = (size_t)2 * TK * D * sizeof(T);
+    if (wgs < 256 && key_tiles > 1 && partial_bytes <= tile_bytes) {
+        int want = (int)((512 + wgs - 1) / wgs);
+        if (want > key_tiles) want = key_tiles;
+        if (want > 32) want = 32;
+        a.n_split = want;
+    }
+    if (const char* e = getenv("VLA_ATTN_SPLIT")) a.n_split = atoi(e) > 0 ? (atoi(e) < key_tiles ? atoi(e) : key_tiles) : 1;
+    a.tiles_per_split = (key_tiles + a.n_split - 1) / a.n_split;
+    a.n_split = (key_tiles + a.tiles_per_split - 1) / a.tiles_per_split;  // no empty slices
+    if (a.n_split > 1) {
+        const size_t rows = (size_t)a.batch * a.Hkv * a.n_split * a.r_pad;
+        float* ws = workspace(rows * (D + 2));
+        if (!ws) return VLA_K_ERR_LAUNCH;
+        a.part_o = ws;
+        a.part_ml = ws + rows * D;
+    }
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid((n_tiles + nw - 1) / nw, a.Hkv, a.batch);
-    if (nw == 4) attn_kernel<T, D, 4><<<grid, 256, 0, st>>>(a);
-    else if (nw == 2) attn_kernel<T, D, 2><<<grid, 128, 0, st>>>(a);
-    else attn_kernel<T, D, 1><<<grid, 64, 0, st>>>(a);
-    return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+    switch (nw) {
+        case 1: return launch_nw<T, D, 1>(a, st);
+        case 2: return launch_nw<T, D, 2>(a, st);
+        case 3: return launch_nw<T, D, 3>(a, st);
+        case 4: return launch_nw<T, D, 4>(a, st);
+        default: break;
+    }
+    return VLA_K_ERR_SHAPE;
 }
 
 template <typename T>
-int launch_t(const AttnArgs& a, int D, vla_stream_t stream) {
+int launch_t(AttnArgs& a, int D, vla_stream_t stream) {
     switch (D) {
         case 48: return launch_d<T, 48>(a, stream);
         case 64: return launch_d<T, 64>(a, stream);
@@ -325,7 +510,7 @@ extern "C" int vla_attn_prefix_suffix(const void* q, const void* k_cache, const 
     if (n_q_heads % n_kv_heads || t_max % 8 || n_keys <= 0 || n_keys > t_max) return VLA_K_ERR_SHAPE;
     if (mask_kind < VLA_MASK_NONE || mask_kind > VLA_MASK_PI0_STATE) return VLA_K_ERR_ARG;
     if (batch == 0) return VLA_K_OK;
-    AttnArgs a;
+    AttnArgs a = {};
     a.q = q; a.k_cache = k_cache; a.vt_cache = vt_cache; a.out = out;
     a.batch = batch; a.S = S; a.Hq = n_q_heads; a.Hkv = n_kv_heads; a.t_max = t_max; a.n_keys = n_keys;
     a.scale = scale; a.mask_kind = mask_kind;

@@ -133,25 +133,54 @@ __global__ void adaln_kernel(const T* __restrict__ x, const float* __restrict__ 
 }
 
 // ------------------------------------------------- flow-matching glue ---
-// grid (batch*S), block covers W columns; A (the action width) is small, so
-// each thread does its own dot product.
+// One workgroup per EMB_ROWS consecutive (batch, token) rows.  The action rows and a
+// 64-column slab of W_in at a time sit in LDS (both read from HBM with contiguous,
+// coalesced loads); thread (rr, c) then forms the dot products of rows rr, rr+4 with
+// column c, and stores are coalesced along the width.
+constexpr int EMB_ROWS = 8;
+constexpr int EMB_MAX_A = 64;
+constexpr int EMB_COLS = 64;
 template <typename T>
-__global__ void embed_suffix_kernel(const float* __restrict__ x_t, const float* __restrict__ W_in,
-                                    const float* __restrict__ bias_step, const float* __restrict__ lead,
-                                    T* __restrict__ h, int S, int n_lead, int A, int W) {
-    const int row = blockIdx.x, b = row / S, s = row % S;
-    T* hr = h + (long)row * W;
-    if (s < n_lead) {
-        const float* lr = lead + ((long)b * n_lead + s) * W;
-        for (int c = threadIdx.x; c < W; c += blockDim.x) Elem<T>::store(hr + c, lr[c]);
-        return;
+__global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restrict__ x_t, const float* __restrict__ W_in,
+                                                            const float* __restrict__ bias_step,
+                                                            const float* __restrict__ lead, T* __restrict__ h, int n_rows,
+                                                            int S, int n_lead, int A, int W) {
+    __shared__ float xs[EMB_ROWS][EMB_MAX_A];
+    __shared__ float ws[EMB_COLS][EMB_MAX_A + 1];
+    const int row0 = blockIdx.x * EMB_ROWS;
+    for (int i = threadIdx.x; i < EMB_ROWS * A; i += blockDim.x) {
+        const int rr = i / A, a = i % A, row = row0 + rr;
+        float v = 0.f;
+        if (row < n_rows) {
+            const int b = row / S, s = row % S;
+            if (s >= n_lead) v = x_t[((long)b * (S - n_lead) + (s - n_lead)) * A + a];
+        }
+        xs[rr][a] = v;
     }
-    const float* xr = x_t + ((long)b * (S - n_lead) + (s - n_lead)) * A;
-    for (int c = threadIdx.x; c < W; c += blockDim.x) {
-        const float* wr = W_in + (long)c * A;
-        float acc = 0.f;
-        for (int a = 0; a < A; ++a) acc += wr[a] * xr[a];
-        Elem<T>::store(hr + c, acc + bias_step[c]);
+    const int cl = threadIdx.x & 63, rq = threadIdx.x >> 6;  // column in slab, row quarter
+    for (int c0 = 0; c0 < W; c0 += EMB_COLS) {
+        __syncthreads();
+        const int ncol = min(EMB_COLS, W - c0);
+        for (int i = threadIdx.x; i < ncol * A; i += blockDim.x) ws[i / A][i % A] = W_in[(long)c0 * A + i];
+        __syncthreads();
+        const int c = c0 + cl;
+        if (c >= W) continue;
+        const float bias = bias_step[c];
+#pragma unroll
+        for (int k = 0; k < EMB_ROWS / 4; ++k) {
+            const int rr = rq + 4 * k, row = row0 + rr;
+            if (row >= n_rows) continue;
+            const int b = row / S, s = row % S;
+            float v;
+            if (s < n_lead) {
+                v = lead[((long)b * n_lead + s) * W + c];
+            } else {
+                float acc = 0.f;
+                for (int a = 0; a < A; ++a) acc += ws[cl][a] * xs[rr][a];
+                v = acc + bias;
+            }
+            Elem<T>::store(h + (long)row * W + c, v);
+        }
     }
 }
 
@@ -351,12 +380,14 @@ int vla_embed_suffix(const float* x_t, const float* W_in, const float* bias_step
     if (!x_t || !W_in || !bias_step || !h || batch < 0 || S <= 0 || n_lead < 0 || n_lead > S || A <= 0 || W <= 0)
         return VLA_K_ERR_ARG;
     if (n_lead > 0 && !lead) return VLA_K_ERR_ARG;
+    if (A > EMB_MAX_A) return VLA_K_ERR_SHAPE;
     if (batch == 0) return VLA_K_OK;
     hipStream_t st = (hipStream_t)stream;
+    const int n_rows = batch * S, blocks = (n_rows + EMB_ROWS - 1) / EMB_ROWS;
     if (out_dtype == VLA_DT_F32)
-        embed_suffix_kernel<float><<<batch * S, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, S, n_lead, A, W);
+        embed_suffix_kernel<float><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W);
     else if (out_dtype == VLA_DT_BF16)
-        embed_suffix_kernel<bf16_t><<<batch * S, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, S, n_lead, A, W);
+        embed_suffix_kernel<bf16_t><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W);
     else
         return VLA_K_ERR_ARG;
     return VLA_CHECK_LAUNCH();

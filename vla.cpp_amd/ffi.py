@@ -69,6 +69,7 @@ def _bind():
     L.vla_last_stats.argtypes = [ctypes.c_void_p, ctypes.POINTER(Stats)]
     L.vla_prefill_batch.argtypes = [ctypes.c_void_p, ctypes.POINTER(Inputs), _i32]
     L.vla_denoise_async.argtypes = [ctypes.c_void_p, _i32, ctypes.c_void_p]
+    L.vla_denoise_steps_async.argtypes = [ctypes.c_void_p, _i32, ctypes.c_void_p]
     L.vla_fetch_actions.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.POINTER(_f32)), ctypes.POINTER(_i64)]
     L.vla_predict_batch.argtypes = [ctypes.c_void_p, ctypes.POINTER(Inputs), _i32,
                                     ctypes.POINTER(ctypes.POINTER(_f32)), ctypes.POINTER(_i64)]
@@ -151,6 +152,11 @@ class Model:
         rc = self._L.vla_denoise_async(self._h, chunks, stream)
         if rc != VLA_OK:
             raise RuntimeError("vla_denoise_async returned %d" % rc)
+
+    def denoise_steps_async(self, n_steps, stream=None):
+        rc = self._L.vla_denoise_steps_async(self._h, n_steps, stream)
+        if rc != VLA_OK:
+            raise RuntimeError("vla_denoise_steps_async returned %d" % rc)
 
     def fetch(self):
         p, n = ctypes.POINTER(_f32)(), _i64()

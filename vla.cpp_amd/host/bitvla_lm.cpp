@@ -50,6 +50,11 @@ TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::
         VLA_K(vla_ternary_repack_ladder_host((const uint8_t*)ck.data(name + ".i2"), w.N, K, packed.data()));
         scales = ck.f32(name + ".ws");
         if (scales.size() != parts.size()) throw std::runtime_error("vla: " + name + ".ws has the wrong length");
+    } else if (ck.has(name + ".p2")) {  // already in the gfx950 word order
+        if (ck.info(name + ".p2").nbytes != packed.size() * 4) throw std::runtime_error("vla: " + name + ".p2 has the wrong size");
+        std::memcpy(packed.data(), ck.data(name + ".p2"), packed.size() * 4);
+        scales = ck.f32(name + ".ws");
+        if (scales.size() != parts.size()) throw std::runtime_error("vla: " + name + ".ws has the wrong length");
     } else {
         const std::vector<float> W = ck.f32(name);
         std::vector<int8_t> tern((size_t)w.N * K);
@@ -82,7 +87,8 @@ class BitvlaLm : public ModelArch {
   public:
     explicit BitvlaLm(const Checkpoint& ck);
     void prefill(const Inputs* in, int batch) override;
-    void denoise(int chunks, void* stream) override;
+    void denoise_steps(int n_steps, void* stream) override;
+    int steps_per_chunk() const override { return n_act_; }
     std::vector<float> fetch() override;
     int64_t n_actions() const override { return n_act_; }
 
@@ -210,27 +216,28 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
     }
 }
 
-void BitvlaLm::denoise(int chunks, void* stream) {
+void BitvlaLm::denoise_steps(int n_steps, void* stream) {
     if (B_ == 0) throw std::logic_error("vla: denoise before prefill");
     Ctx C;
     C.stream = (hipStream_t)stream;
     last_stream_ = C.stream;
     const int B = B_;
     const size_t row = (size_t)B * H_;
-    for (int c = 0; c < chunks; ++c) {
-        for (int t = 0; t < n_act_; ++t) {
-            // token t enters as its learned embedding; it depends on the tokens before it
-            // through the K/V they left in the cache
-            VLA_HIP(hipMemcpyAsync(h_.get(), emb_bcast_.as<uint16_t>() + (size_t)t * row, row * 2, hipMemcpyDeviceToDevice,
-                                   C.stream));
-            run_layers(C, B, 1, P_ + t, P_ + t + 1);
-            VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), out_norm_.as<uint16_t>(), hfin_.as<uint16_t>() + (size_t)t * row, eps_, B,
-                                      H_, C.stream));
+    // one step = one appended action token through every layer; the action head runs
+    // when the last token of a chunk is done
+    for (int it = 0; it < n_steps; ++it) {
+        const int t = it % n_act_;
+        VLA_HIP(hipMemcpyAsync(h_.get(), emb_bcast_.as<uint16_t>() + (size_t)t * row, row * 2, hipMemcpyDeviceToDevice,
+                               C.stream));
+        run_layers(C, B, 1, P_ + t, P_ + t + 1);
+        VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), out_norm_.as<uint16_t>(), hfin_.as<uint16_t>() + (size_t)t * row, eps_, B,
+                                  H_, C.stream));
+        if (t == n_act_ - 1) {
+            VLA_HIP(hipMemsetAsync(x_.get(), 0, (size_t)n_act_ * B * A_ * 4, C.stream));
+            // x[t][b] = W_out . hfin[t][b] + b_out (batch' = n_act, rows = B, unit step)
+            VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B,
+                                 0, A_, H_, 1.0f, C.stream));
         }
-        VLA_HIP(hipMemsetAsync(x_.get(), 0, (size_t)n_act_ * B * A_ * 4, C.stream));
-        // x[t][b] = W_out . hfin[t][b] + b_out (batch' = n_act, rows = B, unit step)
-        VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B, 0, A_,
-                             H_, 1.0f, C.stream));
     }
 }
 

@@ -77,7 +77,8 @@ class FlowExpert : public ModelArch {
   public:
     explicit FlowExpert(const Checkpoint& ck);
     void prefill(const Inputs* in, int batch) override;
-    void denoise(int chunks, void* stream) override;
+    void denoise_steps(int n_steps, void* stream) override;
+    int steps_per_chunk() const override { return steps_; }
     std::vector<float> fetch() override;
     int64_t n_actions() const override { return S_ - n_lead_; }
 
@@ -394,7 +395,7 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
     VLA_HIP(hipDeviceSynchronize());
 }
 
-void FlowExpert::denoise(int chunks, void* stream) {
+void FlowExpert::denoise_steps(int n_steps, void* stream) {
     if (B_ == 0) throw std::logic_error("vla: denoise before prefill");
     Ctx C;
     C.stream = (hipStream_t)stream;
@@ -408,9 +409,10 @@ void FlowExpert::denoise(int chunks, void* stream) {
     Q.dtype = dt_;
     Q.ne[0] = D_; Q.ne[1] = Hq_; Q.ne[2] = S_; Q.ne[3] = B;
     const size_t xbytes = (size_t)B * (S_ - n_lead_) * A_ * sizeof(float);
-    for (int c = 0; c < chunks; ++c) {
-        VLA_HIP(hipMemcpyAsync(xt_.get(), x0_.get(), xbytes, hipMemcpyDeviceToDevice, C.stream));
-        for (int s = 0; s < steps_; ++s) {
+    for (int it = 0; it < n_steps; ++it) {
+        const int s = it % steps_;
+        if (s == 0) VLA_HIP(hipMemcpyAsync(xt_.get(), x0_.get(), xbytes, hipMemcpyDeviceToDevice, C.stream));
+        {
             VLA_K(vla_embed_suffix(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
                                    n_lead_ ? lead_.as<float>() : nullptr, h.data, dt_, B, S_, n_lead_, A_, W_, C.stream));
             for (int l = 0; l < L_; ++l) {

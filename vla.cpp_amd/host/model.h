@@ -52,7 +52,11 @@ class ModelArch {
     // Builds the prefix KV for `batch` observations and stages state / noise.
     virtual void prefill(const Inputs* in, int batch) = 0;
     // Runs `chunks` action chunks on `stream` without synchronising.
-    virtual void denoise(int chunks, void* stream) = 0;
+    void denoise(int chunks, void* stream) { denoise_steps(chunks * steps_per_chunk(), stream); }
+    // Runs `n_steps` denoise steps (step index cycling through the chunk, the
+    // noise re-staged at every chunk boundary) on `stream` without synchronising.
+    virtual void denoise_steps(int n_steps, void* stream) = 0;
+    virtual int steps_per_chunk() const = 0;
     // Synchronises and returns [batch, n_actions, max_action_dim].
     virtual std::vector<float> fetch() = 0;
     virtual int64_t n_actions() const = 0;

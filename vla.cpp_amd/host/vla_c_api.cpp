@@ -6,8 +6,10 @@
 
 #include "vla.h"
 
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <new>
 #include <vector>
 
 #include "model.h"
@@ -159,6 +161,19 @@ int32_t vla_denoise_async(vla_model* h, int32_t chunks, void* stream) {
     if (!h || !h->m || chunks <= 0) return VLA_ERR_ARG;
     try {
         h->m->arch->denoise(chunks, stream);
+        return VLA_OK;
+    } catch (const std::exception& e) {
+        std::fprintf(stderr, "vla: denoise failed: %s\n", e.what());
+        return VLA_ERR_EXCEPTION;
+    } catch (...) {
+        return VLA_ERR_EXCEPTION;
+    }
+}
+
+int32_t vla_denoise_steps_async(vla_model* h, int32_t n_steps, void* stream) {
+    if (!h || !h->m || n_steps <= 0) return VLA_ERR_ARG;
+    try {
+        h->m->arch->denoise_steps(n_steps, stream);
         return VLA_OK;
     } catch (const std::exception& e) {
         std::fprintf(stderr, "vla: denoise failed: %s\n", e.what());
