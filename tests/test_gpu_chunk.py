@@ -140,6 +140,38 @@ def test_config4_bitvla_ternary_append(tmp_path, from_fp32):
     m.close()
 
 
+def test_graph_replays_match_the_eager_chunk(tmp_path):
+    # The first chunk of a shape runs eagerly, the second is captured into a HIP graph,
+    # later ones replay it.  Every replay, with other eager work and synchronisations in
+    # between, must reproduce the eager result bit for bit.
+    import torch
+    cfg = ckpt.smolvla_config(n_layers=4, dtype="bf16", suffix_mask=1)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 6)
+    r = np.random.default_rng(270)
+    obs_a, obs_b = make_obs(cfg, r, n_views=2, n_lang=30), make_obs(cfg, r, n_views=2, n_lang=48)
+    m = load(tmp_path, cfg, w, "graph")
+    eager_a = m.predict(obs_a)
+    eager_b = m.predict(obs_b)  # other padding range: launches change, the graph must follow
+    for i in range(3):
+        assert np.array_equal(m.predict(obs_a), eager_a), "replay %d of observation A" % i
+        torch.zeros(1 << 20, device="cuda").sum().item()  # unrelated eager work + sync
+        assert np.array_equal(m.predict(obs_b), eager_b), "replay %d of observation B" % i
+    assert bf16_close(eager_a.reshape(50, 32), orc_chunk.flow_expert_chunk(cfg, w, obs_a, emulate_bf16=True))
+    # several chunks in one call: the last one is what fetch returns
+    m.prefill_batch([obs_a])
+    m.denoise_async(3, None)
+    assert np.array_equal(m.fetch(), eager_a)
+    m.close()
+    cfg4 = ckpt.bitvla_config(n_layers=2)
+    w4 = ckpt.synth_weights(cfg4, seed=0x5EED + 7)
+    obs4 = make_obs(cfg4, r, n_views=1)
+    m4 = load(tmp_path, cfg4, w4, "graph4", ladder_pack=orc.pack_ladder_int2)
+    first = m4.predict(obs4)
+    for i in range(3):
+        assert np.array_equal(m4.predict(obs4), first)
+    m4.close()
+
+
 def test_bad_inputs_are_argument_errors_not_crashes(tmp_path):
     cfg = ckpt.smolvla_config(n_layers=1, dtype="f32")
     w = ckpt.synth_weights(cfg)

@@ -87,12 +87,17 @@ class BitvlaLm : public ModelArch {
   public:
     explicit BitvlaLm(const Checkpoint& ck);
     void prefill(const Inputs* in, int batch) override;
-    void denoise_steps(int n_steps, void* stream) override;
     int steps_per_chunk() const override { return n_act_; }
     std::vector<float> fetch() override;
     int64_t n_actions() const override { return n_act_; }
 
+  protected:
+    void run_steps(int n_steps, void* stream) override;
+    uint64_t launch_key() const override { return ((uint64_t)alloc_gen_ << 32) ^ (uint64_t)B_; }
+
   private:
+    uint32_t alloc_gen_ = 0;
+    DevBuf zeros_;
     void run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys);
     int L_, Hq_, Hkv_, D_, H_, A_, n_act_, n_img_, n_lang_, vocab_, P_ = 0, B_ = 0;
     float eps_;
@@ -167,6 +172,9 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
         qkv_.alloc(M * (H_ + 2 * Hkv_ * D_) * 2); q_.alloc(M * H_ * 2); att_.alloc(M * H_ * 2); o_.alloc(M * H_ * 2);
         hfin_.alloc((size_t)n_act_ * B * H_ * 2);
         x_.alloc((size_t)n_act_ * B * A_ * 4);
+        zeros_.alloc((size_t)n_act_ * B * A_ * 4);
+        zeros_.zero();
+        ++alloc_gen_;
         std::vector<int32_t> pos(P + n_act_);
         for (int i = 0; i < P + n_act_; ++i) pos[i] = i;  // src/models/bitvla.cpp positions 0..seq-1
         rope_.build(RopeSpec{D_, cfg.rope_freq_base}, pos);
@@ -216,7 +224,7 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
     }
 }
 
-void BitvlaLm::denoise_steps(int n_steps, void* stream) {
+void BitvlaLm::run_steps(int n_steps, void* stream) {
     if (B_ == 0) throw std::logic_error("vla: denoise before prefill");
     Ctx C;
     C.stream = (hipStream_t)stream;
@@ -233,7 +241,8 @@ void BitvlaLm::denoise_steps(int n_steps, void* stream) {
         VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), out_norm_.as<uint16_t>(), hfin_.as<uint16_t>() + (size_t)t * row, eps_, B,
                                   H_, C.stream));
         if (t == n_act_ - 1) {
-            VLA_HIP(hipMemsetAsync(x_.get(), 0, (size_t)n_act_ * B * A_ * 4, C.stream));
+            // cleared by a copy node: memset nodes are kept out of captured graphs
+            VLA_HIP(hipMemcpyAsync(x_.get(), zeros_.get(), (size_t)n_act_ * B * A_ * 4, hipMemcpyDeviceToDevice, C.stream));
             // x[t][b] = W_out . hfin[t][b] + b_out (batch' = n_act, rows = B, unit step)
             VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B,
                                  0, A_, H_, 1.0f, C.stream));
@@ -242,7 +251,7 @@ void BitvlaLm::denoise_steps(int n_steps, void* stream) {
 }
 
 std::vector<float> BitvlaLm::fetch() {
-    VLA_HIP(hipStreamSynchronize(last_stream_));
+    VLA_HIP(hipDeviceSynchronize());
     std::vector<float> tb((size_t)n_act_ * B_ * A_), out(tb.size());
     x_.download(tb.data(), tb.size() * 4);
     for (int t = 0; t < n_act_; ++t)

@@ -77,13 +77,19 @@ class FlowExpert : public ModelArch {
   public:
     explicit FlowExpert(const Checkpoint& ck);
     void prefill(const Inputs* in, int batch) override;
-    void denoise_steps(int n_steps, void* stream) override;
     int steps_per_chunk() const override { return steps_; }
     std::vector<float> fetch() override;
     int64_t n_actions() const override { return S_ - n_lead_; }
 
+  protected:
+    void run_steps(int n_steps, void* stream) override;
+    uint64_t launch_key() const override {
+        return ((uint64_t)alloc_gen_ << 40) ^ ((uint64_t)pad_start_ << 20) ^ (uint64_t)pad_end_ ^ ((uint64_t)P_ << 52);
+    }
+
   private:
     void allocate(int B, int P);
+    uint32_t alloc_gen_ = 0;
 
     Arch arch_;
     int dt_ = VLA_DT_F32;
@@ -255,6 +261,7 @@ void FlowExpert::allocate(int B, int P) {
     if (B == B_ && P == P_) return;
     B_ = B;
     P_ = P;
+    ++alloc_gen_;
     const size_t es = dtype_size(dt_);
     for (LayerW& w : layers_) {
         const int prefix = w.needs_prefix ? P : 0;
@@ -395,7 +402,7 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
     VLA_HIP(hipDeviceSynchronize());
 }
 
-void FlowExpert::denoise_steps(int n_steps, void* stream) {
+void FlowExpert::run_steps(int n_steps, void* stream) {
     if (B_ == 0) throw std::logic_error("vla: denoise before prefill");
     Ctx C;
     C.stream = (hipStream_t)stream;
@@ -457,7 +464,7 @@ void FlowExpert::denoise_steps(int n_steps, void* stream) {
 }
 
 std::vector<float> FlowExpert::fetch() {
-    VLA_HIP(hipStreamSynchronize(last_stream_));
+    VLA_HIP(hipDeviceSynchronize());
     const int Sa = S_ - n_lead_;
     std::vector<float> out((size_t)B_ * Sa * A_);
     xt_.download(out.data(), out.size() * sizeof(float));

@@ -24,6 +24,71 @@ int default_cpu_threads() {
     return hw == 0 ? 4 : (int)std::min(hw, 16u);
 }
 
+// ---- whole-chunk HIP graph -------------------------------------------------
+// A chunk is a fixed sequence of a few hundred short launches; replaying it as
+// one graph removes the per-launch host cost that dominates at batch 1.  The
+// graph holds kernel and device-to-device copy nodes only.
+struct ModelArch::GraphState {
+    hipStream_t cap_stream = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    uint64_t key = 0;
+    bool warmed = false;  // the shape has run eagerly once (lazy workspaces exist)
+};
+
+void ModelArch::drop_graph() {
+    if (!graph_) return;
+    if (graph_->exec) (void)hipGraphExecDestroy(graph_->exec);
+    if (graph_->graph) (void)hipGraphDestroy(graph_->graph);
+    if (graph_->cap_stream) (void)hipStreamDestroy(graph_->cap_stream);
+    delete graph_;
+    graph_ = nullptr;
+}
+
+void ModelArch::denoise_steps(int n_steps, void* stream) {
+    static const bool no_graph = std::getenv("VLA_NO_GRAPH") != nullptr;
+    const int spc = steps_per_chunk();
+    int chunks = n_steps / spc;
+    const int rem = n_steps % spc;
+    hipStream_t st = (hipStream_t)stream;
+    if (!graph_) graph_ = new GraphState();
+    GraphState& g = *graph_;
+    const uint64_t key = launch_key();
+    if (g.key != key) {
+        if (g.exec) (void)hipGraphExecDestroy(g.exec);
+        if (g.graph) (void)hipGraphDestroy(g.graph);
+        g.exec = nullptr;
+        g.graph = nullptr;
+        g.key = key;
+        g.warmed = false;
+    }
+    while (chunks > 0) {
+        if (no_graph || !g.warmed) {
+            run_steps(spc, stream);
+            g.warmed = true;
+            --chunks;
+            continue;
+        }
+        if (!g.exec) {
+            if (!g.cap_stream) VLA_HIP(hipStreamCreateWithFlags(&g.cap_stream, hipStreamNonBlocking));
+            VLA_HIP(hipStreamBeginCapture(g.cap_stream, hipStreamCaptureModeThreadLocal));
+            try {
+                run_steps(spc, g.cap_stream);
+            } catch (...) {
+                hipGraph_t junk = nullptr;
+                (void)hipStreamEndCapture(g.cap_stream, &junk);
+                if (junk) (void)hipGraphDestroy(junk);
+                throw;
+            }
+            VLA_HIP(hipStreamEndCapture(g.cap_stream, &g.graph));
+            VLA_HIP(hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0));
+        }
+        VLA_HIP(hipGraphLaunch(g.exec, st));
+        --chunks;
+    }
+    if (rem > 0) run_steps(rem, stream);
+}
+
 bool config_is_sane(const Config& c) {
     return c.real_action_dim <= c.max_action_dim && c.real_state_dim <= c.max_state_dim && c.real_action_dim >= 0 &&
            c.real_state_dim >= 0;

@@ -46,7 +46,7 @@ struct Stats {
 // per handle (the reference's rule, src/arch.h:85-87).
 class ModelArch {
   public:
-    virtual ~ModelArch() = default;
+    virtual ~ModelArch() { drop_graph(); }
     Config cfg;
     Stats stats;
     // Builds the prefix KV for `batch` observations and stages state / noise.
@@ -55,8 +55,23 @@ class ModelArch {
     void denoise(int chunks, void* stream) { denoise_steps(chunks * steps_per_chunk(), stream); }
     // Runs `n_steps` denoise steps (step index cycling through the chunk, the
     // noise re-staged at every chunk boundary) on `stream` without synchronising.
-    virtual void denoise_steps(int n_steps, void* stream) = 0;
+    // Whole chunks are replayed from a captured HIP graph once the shape has run
+    // eagerly (set VLA_NO_GRAPH=1 to always launch eagerly).
+    void denoise_steps(int n_steps, void* stream);
     virtual int steps_per_chunk() const = 0;
+
+  protected:
+    // Eager launches of steps [0, n_steps) of a chunk on `stream`.
+    virtual void run_steps(int n_steps, void* stream) = 0;
+    // Changes whenever anything baked into the launches changes (buffers, shapes, masks).
+    virtual uint64_t launch_key() const = 0;
+
+  private:
+    struct GraphState;
+    GraphState* graph_ = nullptr;
+
+  public:
+    void drop_graph();
     // Synchronises and returns [batch, n_actions, max_action_dim].
     virtual std::vector<float> fetch() = 0;
     virtual int64_t n_actions() const = 0;
