@@ -67,7 +67,7 @@ def plain_pack(t):
     import __graft_entry__ as entry
     lib = entry.load_package().lib()
     t = np.ascontiguousarray(t, np.int8)
-    out = np.empty((t.shape[0], t.shape[1] // 16), np.uint32)
+    out = np.empty(lib.vla_ternary_packed_words(t.shape[0], t.shape[1]), np.uint32)
     rc = lib.vla_ternary_pack_host(t.ctypes.data, t.shape[0], t.shape[1], out.ctypes.data)
     assert rc == 0
     return out.view(np.uint8).reshape(-1)

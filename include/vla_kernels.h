@@ -177,10 +177,14 @@ VLA_KAPI int vla_act_quant_bf16(const uint16_t* in, int8_t* out, float* scales, 
  * src/models/bitvla.cpp:430-451). */
 VLA_KAPI int vla_ternary_quant_host(const float* W, int64_t n, int8_t* ternary, float* absmean);
 
-/* Host packers.  The gfx950 layout is [N][K/16] 32-bit words; word (n, w)
- * holds codes t+2 of k = 16w .. 16w+15 with value b+4j at bits 8b+2j, i.e. the
- * reference's 16-value slot format (src/models/bitvla.cpp:470-480) in plain
- * row-major word order instead of the wmma "ladder" order. */
+/* Host packers.  A packed word holds the codes t+2 of 16 consecutive k of one
+ * output column, value b+4j at bits 8b+2j: the reference's 16-value slot
+ * (src/models/bitvla.cpp:470-480).  The gfx950 layout orders the words
+ * "MFMA-fragment-major" instead of the wmma "ladder" order: word (n, w), w = k/16,
+ * sits at index (((n/32) * (K/32) + w/2) * 2 + w%2) * 32 + n%32, so the 64 words a
+ * wavefront feeds to one v_mfma_i32_32x32x32_i8 are contiguous.  Buffers hold
+ * vla_ternary_packed_words(N, K) words (N rounded up to 32; pad columns are weight 0). */
+VLA_KAPI long vla_ternary_packed_words(int N, int K);
 VLA_KAPI int vla_ternary_pack_host(const int8_t* ternary, int N, int K, uint32_t* packed);
 VLA_KAPI int vla_ternary_repack_ladder_host(const uint8_t* ladder, int N, int K, uint32_t* packed);
 

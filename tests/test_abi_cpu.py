@@ -41,12 +41,18 @@ def test_ternary_quant_and_packers_against_oracle():
     assert lib.vla_ternary_quant_host(W.ctypes.data, W.size, t.ctypes.data, ctypes.addressof(am)) == 0
     ot, oam = orc.weight_quant_ternary(W)
     assert np.array_equal(t, ot) and np.float32(am.value) == oam
-    # plain packing: word (n, w) decodes (reference decode) to the 16 values k = 16w..16w+15
-    packed = np.empty((N, K // 16), np.uint32)
+    # packing: word (n, w) decodes (reference decode) to the 16 values k = 16w..16w+15
+    nwords = lib.vla_ternary_packed_words(N, K)
+    assert nwords == N * K // 16 and lib.vla_ternary_packed_words(48, K) == 64 * K // 16
+    packed = np.empty(nwords, np.uint32)
     assert lib.vla_ternary_pack_host(t.ctypes.data, N, K, packed.ctypes.data) == 0
-    for n, w in ((0, 0), (5, 3), (63, 15)):
-        assert np.array_equal(orc.decode_i2s_to_i8s(packed[n, w]), t[n, 16 * w:16 * w + 16])
-    # ladder -> plain repack is a word permutation that inverts the reference's swizzle
+    word = lambda buf, n, w: buf[pkg.tern_word_index(n, w, K)]
+    for n, w in ((0, 0), (5, 3), (63, 15), (33, 1), (31, 14)):
+        assert np.array_equal(orc.decode_i2s_to_i8s(word(packed, n, w)), t[n, 16 * w:16 * w + 16])
+    # the 64 words of one (32-column block, 32-k group) are contiguous, [k half][column]
+    assert pkg.tern_word_index(32, 2, K) == (1 * (K // 32) + 1) * 64
+    assert pkg.tern_word_index(32 + 7, 3, K) == (1 * (K // 32) + 1) * 64 + 32 + 7
+    # ladder -> gfx950 repack is a word permutation that inverts the reference's swizzle
     ladder = orc.pack_ladder_int2(t)
     rep = np.empty_like(packed)
     assert lib.vla_ternary_repack_ladder_host(ladder.ctypes.data, N, K, rep.ctypes.data) == 0
@@ -55,8 +61,13 @@ def test_ternary_quant_and_packers_against_oracle():
     raw = r.integers(0, 256, N * K // 4).astype(np.uint8)
     assert lib.vla_ternary_repack_ladder_host(raw.ctypes.data, N, K, rep.ctypes.data) == 0
     U = orc.unpack_ladder_int2(raw, N, K)
-    dec = np.stack([[orc.decode_i2s_to_i8s(rep[n, w]) for w in range(K // 16)] for n in range(N)]).reshape(N, K)
+    dec = np.stack([[orc.decode_i2s_to_i8s(word(rep, n, w)) for w in range(K // 16)] for n in range(N)]).reshape(N, K)
     assert np.array_equal(dec, U)
+    # columns past N (rounded up to 32) are packed as weight 0
+    t48 = t[:48]
+    p48 = np.empty(lib.vla_ternary_packed_words(48, K), np.uint32)
+    assert lib.vla_ternary_pack_host(t48.ctypes.data, 48, K, p48.ctypes.data) == 0
+    assert list(orc.decode_i2s_to_i8s(word(p48, 50, 3))) == [0] * 16
     assert lib.vla_ternary_repack_ladder_host(raw.ctypes.data, 24, K, rep.ctypes.data) == pkg.VLA_K_ERR_SHAPE
 
 

@@ -326,7 +326,7 @@ def test_act_quant_bit_exact():
 
 def _pack_plain(t):
     N, K = t.shape
-    out = np.empty((N, K // 16), np.uint32)
+    out = np.empty(pkg.lib().vla_ternary_packed_words(N, K), np.uint32)
     assert pkg.lib().vla_ternary_pack_host(t.ctypes.data, N, K, out.ctypes.data) == 0
     return out
 
@@ -343,7 +343,7 @@ def test_ternary_gemm_accumulators_and_epilogue_bit_exact(M, N, K, ws_num):
     s = (40.0 + (raw[M * K + N * K // 4:M * K + N * K // 4 + M] % 100)).astype(np.float32)
     ws = (0.01 + 0.001 * (raw[-ws_num:] % 50).astype(np.float32)).astype(np.float32)
     Wt = orc.unpack_ladder_int2(ladder, N, K)
-    packed = np.empty((N, K // 16), np.uint32)
+    packed = np.empty(pkg.lib().vla_ternary_packed_words(N, K), np.uint32)
     assert pkg.lib().vla_ternary_repack_ladder_host(ladder.ctypes.data, N, K, packed.ctypes.data) == 0
     acc = torch.zeros((M, N), dtype=torch.int32, device="cuda")
     out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
@@ -358,6 +358,65 @@ def test_ternary_gemm_accumulators_and_epilogue_bit_exact(M, N, K, ws_num):
         pkg.call("bitlinear_int8xint2_m", dev(A), dev(packed), out2, dev(s), dev(ws), M, N, K)
         sync()
         assert np.array_equal(host(out2), host(out))
+
+
+@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("M,N,K", [(300, 288, 256), (515, 640, 384), (64, 48, 128)])
+def test_ternary_gemm_large_tile_kernels_bit_exact(monkeypatch, tile, M, N, K):
+    # The large-M kernels (weights read straight from the fragment-major layout), pinned
+    # by VLA_TERNARY_TILE, on ragged M and N: same int32 accumulators and bf16 epilogue.
+    r = np.random.default_rng(tile + M)
+    A = r.integers(-127, 128, (M, K)).astype(np.int8)
+    ladder = r.integers(0, 256, N * K // 4).astype(np.uint8)
+    s = (40.0 + r.integers(0, 100, M)).astype(np.float32)
+    s[::7] = (127.0 / np.abs(r.standard_normal(s[::7].size) * 3 + 1e-3)).astype(np.float32)  # arbitrary mantissas
+    if M > 400:  # scales near the exponent limits take the full-range division path
+        s[5], s[100], s[300] = 1e-25, 3e22, 7.5e-21
+    ws_num = 3 if N % 3 == 0 else 1
+    ws = (0.01 + 0.001 * r.integers(0, 50, ws_num)).astype(np.float32)
+    Wt = orc.unpack_ladder_int2(ladder, N, K)
+    packed = np.empty(pkg.lib().vla_ternary_packed_words(N, K), np.uint32)
+    assert pkg.lib().vla_ternary_repack_ladder_host(ladder.ctypes.data, N, K, packed.ctypes.data) == 0
+    acc = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+    rowsum = dev(A.astype(np.int32).sum(1).astype(np.int32))
+    monkeypatch.setenv("VLA_TERNARY_TILE", str(tile))
+    pkg.call("vla_ternary_gemm", dev(A), dev(packed), out, acc, dev(s), rowsum, dev(ws), ws_num, M, N, K)
+    sync()
+    want_acc = orc.ternary_gemm_i32(A, Wt)
+    assert np.array_equal(host(acc), want_acc)
+    assert np.array_equal(host(out, np.uint16), orc.ternary_epilogue(want_acc, s, ws))
+
+
+def test_ternary_gemm_prefill_shape_all_tilings_agree(monkeypatch):
+    # BitVLA prefill QKV at full size (M = 8 x 512 tokens): the shape-selected kernel and
+    # both pinned tilings give identical accumulators and outputs; a sample of rows is
+    # checked against the oracle.
+    M, N, K, ws_num = 4096, 3840, 2560, 6
+    r = np.random.default_rng(4096)
+    A = r.integers(-127, 128, (M, K)).astype(np.int8)
+    t = r.integers(-1, 2, (N, K)).astype(np.int8)
+    s = (40.0 + r.integers(0, 100, M)).astype(np.float32)
+    ws = (0.01 + 0.001 * r.integers(0, 50, ws_num)).astype(np.float32)
+    dA, dW, ds, dws = dev(A), dev(_pack_plain(t)), dev(s), dev(ws)
+    rowsum = dev(A.astype(np.int32).sum(1).astype(np.int32))
+    res = []
+    for tile in (None, 64, 128, 256):
+        if tile is None:
+            monkeypatch.delenv("VLA_TERNARY_TILE", raising=False)
+        else:
+            monkeypatch.setenv("VLA_TERNARY_TILE", str(tile))
+        acc = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+        out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+        pkg.call("vla_ternary_gemm", dA, dW, out, acc, ds, rowsum, dws, ws_num, M, N, K)
+        sync()
+        res.append((acc, out))
+    for acc, out in res[1:]:
+        assert torch.equal(acc, res[0][0]) and torch.equal(out, res[0][1])
+    rows = np.r_[0:8, 255:258, 2047:2050, 4088:4096]
+    want_acc = orc.ternary_gemm_i32(A[rows], t)
+    assert np.array_equal(host(res[0][0])[rows], want_acc)
+    assert np.array_equal(host(res[0][1], np.uint16)[rows], orc.ternary_epilogue(want_acc, s[rows], ws))
 
 
 def test_ternary_pipeline_matches_cpu_twin():

@@ -39,6 +39,7 @@ KERNEL_API = {
     "vla_euler_step": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
     "vla_act_quant_bf16": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "vla_ternary_quant_host": [_vp, _i64, _vp, _vp],
+    "vla_ternary_packed_words": [_i, _i],
     "vla_ternary_pack_host": [_vp, _i, _i, _vp],
     "vla_ternary_repack_ladder_host": [_vp, _i, _i, _vp],
     "vla_ternary_gemm": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
@@ -55,7 +56,12 @@ KERNEL_API = {
     "bitlinear_int8xint2": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "vla_kernels_arch": [],
 }
-_RESTYPES = {"vla_kernels_arch": ctypes.c_char_p}
+_RESTYPES = {"vla_kernels_arch": ctypes.c_char_p, "vla_ternary_packed_words": ctypes.c_long}
+
+
+def tern_word_index(n, w, K):
+    """Index of packed word (column n, 16-k group w) in the gfx950 ternary layout."""
+    return (((n >> 5) * (K // 32) + (w >> 1)) * 2 + (w & 1)) * 32 + (n & 31)
 
 
 def lib():

@@ -23,6 +23,8 @@
 // chunk*kChunk + g*(kChunk/2); the 32x32 result holds, in element 4j+i of lane
 // (g, r), C[8j + 4g + i][r].
 
+#include <stdlib.h>
+
 #include "common.h"
 #include "vla_kernels.h"
 
@@ -30,9 +32,7 @@ namespace {
 
 using namespace vk;
 
-constexpr int BM = 64, BN = 64;
-constexpr int ROW_BYTES = 128;             // bytes of K per tile row
-constexpr int LDS_STRIDE = ROW_BYTES + 16; // padded row, keeps 16-byte reads conflict-free
+constexpr int BN = 64;                     // epilogue sub-tile; column-tile unit of the N mapping
 constexpr int C_STRIDE = BN + 4;           // floats
 
 enum { EPI_PLAIN = 0, EPI_QKV = 1, EPI_TERNARY = 2 };
@@ -41,7 +41,7 @@ struct GemmArgs {
     const void* A;
     const void* W;
     const float* bias;
-    int M, N, K;
+    int M, N, K, n_tiles;
     // PLAIN
     const void* residual;
     void* Y;
@@ -91,6 +91,14 @@ template <> struct Traits<int8_t> {
                                                    0, 0, 0);
     }
 };
+
+// Packed ternary weights are stored "MFMA-fragment-major": for each block of 32 output
+// columns and each group of 32 k, 64 consecutive words [g][r] hold the 16 codes
+// k = 32*kk + 16*g .. +15 of column 32*nb + r -- exactly what lane (g, r) of a wavefront
+// feeds to v_mfma_i32_32x32x32_i8, so a fragment is one coalesced 256-byte load.
+__host__ __device__ __forceinline__ long tern_word_index(long n, int w, int K) {
+    return (((n >> 5) * (K / 32) + (w >> 1)) * 2 + (w & 1)) * 32 + (n & 31);
+}
 
 // Accumulator element -> raw 32-bit LDS cell (by value: a bit_cast applied
 // directly to a vector element expression reads element 0).
@@ -144,118 +152,11 @@ __device__ __forceinline__ TileCols tile_cols(const GemmArgs& a, int nt) {
     return t;
 }
 
+// Epilogue of one 64x64 sub-tile held in the LDS C tile: thread t owns row t/4 and
+// columns jg..jg+7 and 32+jg..32+jg+7 of the sub-tile.
 template <typename T, int kEpi>
-__global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
-    typedef Traits<T> TR;
-    constexpr int EB = TR::kElemBytes;
-    constexpr int BK = ROW_BYTES / EB;  // k elements per tile
-
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * BM * LDS_STRIDE];
-    unsigned char* ldsA = lds;
-    unsigned char* ldsW = lds + BM * LDS_STRIDE;
-    static_assert(sizeof(float) * BM * C_STRIDE <= sizeof(lds), "C tile must fit in the operand buffers");
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int g = lane >> 5, r = lane & 31;
-    const int m0 = blockIdx.y * BM;
-    const int nt = blockIdx.x;
-    const TileCols tc = tile_cols<kEpi>(a, nt);
-
-    typename TR::Acc acc;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0;
-
-    const int nkt = (a.K + BK - 1) / BK;
-
-    // Global -> register staging: two 16-byte vectors of A and of W per thread.
-    u32x4_t ra[2], rw[2];
-    auto load_tile = [&](int kt) {
-        const int k0 = kt * BK;
-#pragma unroll
-        for (int v = 0; v < 2; ++v) {
-            const int idx = tid + v * 256;
-            const int row = idx >> 3, c = idx & 7;
-            const int k = k0 + c * (16 / EB);
-            const int m = m0 + row;
-            u32x4_t z = {0u, 0u, 0u, 0u};
-            ra[v] = z;
-            if (m < a.M && k < a.K)
-                ra[v] = *reinterpret_cast<const u32x4_t*>((const unsigned char*)a.A + ((long)m * a.K + k) * EB);
-            if (kEpi == EPI_TERNARY) continue;
-            const int n = (row < 32) ? tc.base0 + row : tc.base1 + row - 32;
-            rw[v] = z;
-            if (n < a.N && k < a.K)
-                rw[v] = *reinterpret_cast<const u32x4_t*>((const unsigned char*)a.W + ((long)n * a.K + k) * EB);
-        }
-        if (kEpi == EPI_TERNARY) {
-            // 64 rows x 128 k of 2-bit codes = 64 x 8 words; two words per thread.
-            const int row = tid >> 2, q = tid & 3;
-            const int n = nt * BN + row;
-            const int kw = k0 / 16 + q * 2;
-            u32x4_t z = {0u, 0u, 0u, 0u};
-            rw[0] = z;
-            if (n < a.N && kw * 16 < a.K) {
-                const u32x2_t w2 = *reinterpret_cast<const u32x2_t*>((const uint32_t*)a.W + (long)n * (a.K / 16) + kw);
-                rw[0][0] = w2[0];
-                rw[0][1] = w2[1];
-            }
-        }
-    };
-    auto store_tile = [&]() {
-#pragma unroll
-        for (int v = 0; v < 2; ++v) {
-            const int idx = tid + v * 256;
-            const int row = idx >> 3, c = idx & 7;
-            *reinterpret_cast<u32x4_t*>(ldsA + row * LDS_STRIDE + c * 16) = ra[v];
-            if (kEpi != EPI_TERNARY) *reinterpret_cast<u32x4_t*>(ldsW + row * LDS_STRIDE + c * 16) = rw[v];
-        }
-        if (kEpi == EPI_TERNARY) {
-            // Decode 2 words -> 32 codes (unsigned 0..3; the -2 offset is folded
-            // into the epilogue as -2*rowsum).  Word layout: value b+4j sits at
-            // bits 8b+2j, so (w >> 2j) & 0x03030303 is values 4j..4j+3.
-            const int row = tid >> 2, q = tid & 3;
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint32_t w = rw[0][h];
-                u32x4_t d;
-                d[0] = w & 0x03030303u;
-                d[1] = (w >> 2) & 0x03030303u;
-                d[2] = (w >> 4) & 0x03030303u;
-                d[3] = (w >> 6) & 0x03030303u;
-                *reinterpret_cast<u32x4_t*>(ldsW + row * LDS_STRIDE + q * 32 + h * 16) = d;
-            }
-        }
-    };
-
-    load_tile(0);
-    for (int kt = 0; kt < nkt; ++kt) {
-        store_tile();
-        __syncthreads();
-        if (kt + 1 < nkt) load_tile(kt + 1);
-#pragma unroll
-        for (int ch = 0; ch < ROW_BYTES / TR::kChunkBytes; ++ch) {
-            const int off = ch * TR::kChunkBytes + g * 16;
-            const u32x4_t fa = *reinterpret_cast<const u32x4_t*>(ldsA + (wm * 32 + r) * LDS_STRIDE + off);
-            const u32x4_t fw = *reinterpret_cast<const u32x4_t*>(ldsW + (wn * 32 + r) * LDS_STRIDE + off);
-            TR::mma(acc, fa, fw);
-        }
-        __syncthreads();
-    }
-
-    // Accumulators -> LDS C tile (4-byte cells).
-    uint32_t* C = reinterpret_cast<uint32_t*>(lds);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = wm * 32 + 8 * j + 4 * g + i;
-            const int col = wn * 32 + r;
-            C[row * C_STRIDE + col] = acc_bits(acc[4 * j + i]);
-        }
-    __syncthreads();
-
-    // Epilogue: thread t owns row t/4 and tile columns jg..jg+7 and 32+jg..32+jg+7.
+__device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t* C, int m0, int nt, const TileCols& tc,
+                                               int tid) {
     const int erow = tid >> 2, jg = (tid & 3) * 8;
     const int m = m0 + erow;
     if (m >= a.M) return;
@@ -287,22 +188,57 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
 
     if (kEpi == EPI_PLAIN) {
 #pragma unroll
-        for (int hlf = 0; hlf < 2; ++hlf)
+        for (int hlf = 0; hlf < 2; ++hlf) {
+            const int n0 = nt * BN + hlf * 32 + jg;
+            if (n0 >= a.N) continue;
+            float* v = hlf ? hi : lo;
+            const long o = (long)m * a.N + n0;
+            const bool full = (n0 + 8 <= a.N) && (a.N % 8 == 0);
+            if (a.bias) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int n = nt * BN + hlf * 32 + jg + e;
-                if (n >= a.N) continue;
-                float v = hlf ? hi[e] : lo[e];
-                if (a.bias) v += a.bias[n];
-                const long o = (long)m * a.N + n;
-                if (a.out_bf16) {
-                    if (a.residual) v += bf2f(((const bf16_t*)a.residual)[o]);
-                    ((bf16_t*)a.Y)[o] = f2bf(v);
-                } else {
-                    if (a.residual) v += ((const float*)a.residual)[o];
-                    ((float*)a.Y)[o] = v;
+                for (int e = 0; e < 8; ++e)
+                    if (n0 + e < a.N) v[e] += a.bias[n0 + e];
+            }
+            if (full && a.out_bf16) {  // 8 consecutive bf16 = one 16-byte access each way
+                if (a.residual) {
+                    const u32x4_t rr = *reinterpret_cast<const u32x4_t*>((const bf16_t*)a.residual + o);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        v[2 * e] += __uint_as_float(rr[e] << 16);
+                        v[2 * e + 1] += __uint_as_float(rr[e] & 0xffff0000u);
+                    }
+                }
+                const u32x4_t pk = {pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3]), pack_bf2(v[4], v[5]), pack_bf2(v[6], v[7])};
+                *reinterpret_cast<u32x4_t*>((bf16_t*)a.Y + o) = pk;
+            } else if (full) {
+                if (a.residual) {
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const f32x4_t rr = *reinterpret_cast<const f32x4_t*>((const float*)a.residual + o + 4 * q);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) v[4 * q + e] += rr[e];
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const f32x4_t pk = {v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+                    *reinterpret_cast<f32x4_t*>((float*)a.Y + o + 4 * q) = pk;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (n0 + e >= a.N) continue;
+                    float x = v[e];
+                    if (a.out_bf16) {
+                        if (a.residual) x += bf2f(((const bf16_t*)a.residual)[o + e]);
+                        ((bf16_t*)a.Y)[o + e] = f2bf(x);
+                    } else {
+                        if (a.residual) x += ((const float*)a.residual)[o + e];
+                        ((float*)a.Y)[o + e] = x;
+                    }
                 }
             }
+        }
         return;
     }
 
@@ -364,11 +300,409 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     }
 }
 
+// Workgroup tile (64*TM) x (64*TN), 2 x 2 wavefronts; wavefront (wm, wn) owns the 32x32
+// MFMA blocks in block rows wm + 2i (i < TM) and block columns wn + 2j (j < TN), so every
+// 64x64 sub-tile is made of one block from each wavefront.  KB = bytes of K per staged row.
+template <typename T, int kEpi, int TM, int TN, int KB>
+__global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
+    typedef Traits<T> TR;
+    constexpr int EB = TR::kElemBytes;
+    constexpr int BK = KB / EB;        // k elements per tile
+    constexpr int STRIDE = KB + 16;    // padded LDS row
+    constexpr int ROWS_A = 64 * TM, ROWS_W = 64 * TN;
+    constexpr int VPR = KB / 16;       // 16-byte vectors per staged row
+    constexpr int VA = ROWS_A * VPR / 256, VW = ROWS_W * VPR / 256;  // vectors per thread
+    static_assert(kEpi != EPI_TERNARY || (TM == 1 && TN == 1 && KB == 128), "ternary staging assumes 64x64x128 tiles");
+
+    __shared__ __attribute__((aligned(16))) unsigned char lds[(ROWS_A + ROWS_W) * STRIDE];
+    unsigned char* ldsA = lds;
+    unsigned char* ldsW = lds + ROWS_A * STRIDE;
+    static_assert(sizeof(float) * 64 * C_STRIDE <= sizeof(lds), "C sub-tile must fit in the operand buffers");
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int g = lane >> 5, r = lane & 31;
+    // Linear workgroup id -> (M tile, N tile) with the N tiles padded to a multiple of
+    // 8: id % 8 (the XCD a workgroup is dispatched to) then equals nt % 8, so each XCD's
+    // L2 holds one eighth of W plus the A rows instead of the whole of both.
+    const int n_wg_tiles = (a.n_tiles + TN - 1) / TN;
+    const int nt_pad = (n_wg_tiles + 7) & ~7;
+    const int ntw = blockIdx.x % nt_pad;
+    if (ntw >= n_wg_tiles) return;
+    const int m0 = (blockIdx.x / nt_pad) * ROWS_A;
+    TileCols tc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) tc[j] = tile_cols<kEpi>(a, ntw * TN + j);
+
+    typename TR::Acc acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+    const int nkt = (a.K + BK - 1) / BK;
+
+    // Global -> register staging of the next k-tile while the current one is multiplied.
+    u32x4_t ra[VA], rw[VW];
+    auto load_tile = [&](int kt) {
+        const int k0 = kt * BK;
+#pragma unroll
+        for (int v = 0; v < VA; ++v) {
+            const int idx = tid + v * 256;
+            const int row = idx / VPR, c = idx % VPR;
+            const int k = k0 + c * (16 / EB);
+            const int m = m0 + row;
+            u32x4_t z = {0u, 0u, 0u, 0u};
+            ra[v] = z;
+            if (m < a.M && k < a.K)
+                ra[v] = *reinterpret_cast<const u32x4_t*>((const unsigned char*)a.A + ((long)m * a.K + k) * EB);
+        }
+        if (kEpi != EPI_TERNARY) {
+#pragma unroll
+            for (int v = 0; v < VW; ++v) {
+                const int idx = tid + v * 256;
+                const int row = idx / VPR, c = idx % VPR;
+                const int k = k0 + c * (16 / EB);
+                constexpr int RPV = 256 / VPR;          // rows covered by one vector index step
+                const int sub = (v * RPV) / 64, wr = row & 63;  // compile-time per unrolled v
+                const int n = (wr < 32) ? tc[sub].base0 + wr : tc[sub].base1 + wr - 32;
+                const bool tile_ok = (ntw * TN + sub) < a.n_tiles;
+                u32x4_t z = {0u, 0u, 0u, 0u};
+                rw[v] = z;
+                if (tile_ok && n < a.N && k < a.K)
+                    rw[v] = *reinterpret_cast<const u32x4_t*>((const unsigned char*)a.W + ((long)n * a.K + k) * EB);
+            }
+        } else {
+            // 64 rows x 128 k of 2-bit codes = 64 x 8 words; two words per thread.
+            const int row = tid >> 2, q = tid & 3;
+            const int n = ntw * BN + row;
+            const int kw = k0 / 16 + q * 2;
+            u32x4_t z = {0u, 0u, 0u, 0u};
+            rw[0] = z;
+            if (n < a.N && kw * 16 < a.K) {
+                // words kw, kw+1 = the two 16-k halves (g = 0, 1) of 32-k group kw/2
+                const uint32_t* wp = (const uint32_t*)a.W + tern_word_index(n, kw, a.K);
+                rw[0][0] = wp[0];
+                rw[0][1] = wp[32];
+            }
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int v = 0; v < VA; ++v) {
+            const int idx = tid + v * 256;
+            *reinterpret_cast<u32x4_t*>(ldsA + (idx / VPR) * STRIDE + (idx % VPR) * 16) = ra[v];
+        }
+        if (kEpi != EPI_TERNARY) {
+#pragma unroll
+            for (int v = 0; v < VW; ++v) {
+                const int idx = tid + v * 256;
+                *reinterpret_cast<u32x4_t*>(ldsW + (idx / VPR) * STRIDE + (idx % VPR) * 16) = rw[v];
+            }
+        } else {
+            // Decode 2 words -> 32 codes (unsigned 0..3; the -2 offset is folded
+            // into the epilogue as -2*rowsum).  Word layout: value b+4j sits at
+            // bits 8b+2j, so (w >> 2j) & 0x03030303 is values 4j..4j+3.
+            const int row = tid >> 2, q = tid & 3;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t w = rw[0][h];
+                u32x4_t d;
+                d[0] = w & 0x03030303u;
+                d[1] = (w >> 2) & 0x03030303u;
+                d[2] = (w >> 4) & 0x03030303u;
+                d[3] = (w >> 6) & 0x03030303u;
+                *reinterpret_cast<u32x4_t*>(ldsW + row * STRIDE + q * 32 + h * 16) = d;
+            }
+        }
+    };
+
+    load_tile(0);
+    for (int kt = 0; kt < nkt; ++kt) {
+        store_tile();
+        __syncthreads();
+        if (kt + 1 < nkt) load_tile(kt + 1);
+#pragma unroll
+        for (int ch = 0; ch < KB / TR::kChunkBytes; ++ch) {
+            const int off = ch * TR::kChunkBytes + g * 16;
+            u32x4_t fa[TM], fw[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const u32x4_t*>(ldsA + ((wm + 2 * i) * 32 + r) * STRIDE + off);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fw[j] = *reinterpret_cast<const u32x4_t*>(ldsW + ((wn + 2 * j) * 32 + r) * STRIDE + off);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[i], fw[j]);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue, one 64x64 sub-tile at a time through an LDS copy of the accumulators.
+    uint32_t* C = reinterpret_cast<uint32_t*>(lds);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if (i + j > 0) __syncthreads();
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii)
+                    C[(wm * 32 + 8 * jj + 4 * g + ii) * C_STRIDE + wn * 32 + r] = acc_bits(acc[i][j][4 * jj + ii]);
+            __syncthreads();
+            const int nt_sub = ntw * TN + j;
+            if (nt_sub < a.n_tiles) epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid);
+        }
+}
+
+// Large-M ternary GEMM (BitVLA prefill: M = batch x prefix tokens).  Workgroup tile
+// (64*WM) x 256 with WM x 2 wavefronts, each owning 64 x 128 = 2 x 4 MFMA blocks (128
+// accumulator registers), so one 16-byte A fragment feeds four MFMAs and one weight
+// fragment two.  int8 activations go global -> registers -> double-buffered LDS (one
+// barrier per 128-k tile).  The 2-bit weights never touch LDS: the fragment-major layout
+// makes each (32 columns x 32 k) fragment one coalesced 256-byte load per wavefront; a
+// word is expanded to bytes with shift/mask right before use and its register is
+// refilled at once with the word of the next k-tile, a full tile of MFMAs ahead of need.
+template <int WM>
+__global__ void __launch_bounds__(WM * 128, 2) ternary_gemm_big_kernel(GemmArgs a) {
+    constexpr int NT = WM * 128, ROWS = WM * 64, STRIDE = 144, VA = ROWS * 8 / NT;
+    constexpr int T_STRIDE = 272;  // bf16 transpose staging: 128 columns + 16 bytes of padding
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2][ROWS * STRIDE];
+    static_assert(sizeof(lds) >= (size_t)(WM * 2) * 32 * T_STRIDE, "epilogue staging must fit in the A buffers");
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int g = lane >> 5, r = lane & 31;
+    // id % 8 (the XCD) = M tile % 8: workgroups sharing an L2 share their activation rows,
+    // the larger operand, and stream the whole (4x smaller) packed weight matrix.
+    const int m_tiles = (a.M + ROWS - 1) / ROWS, mt_pad = (m_tiles + 7) & ~7;
+    const int mt = blockIdx.x % mt_pad;
+    if (mt >= m_tiles) return;
+    const int m0 = mt * ROWS, n0 = (blockIdx.x / mt_pad) * 256 + wn * 128;
+
+    const int kgroups = a.K / 32, nblocks = (a.N + 31) / 32;
+    const uint32_t* wp[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int nb = n0 / 32 + j;
+        nb = nb < nblocks ? nb : nblocks - 1;  // columns past N: any valid block, result dropped
+        wp[j] = (const uint32_t*)a.W + (long)nb * kgroups * 64 + lane;
+    }
+    const unsigned char* ap[VA];
+#pragma unroll
+    for (int v = 0; v < VA; ++v) {
+        const int idx = tid + v * NT;
+        const int m = min(m0 + idx / 8, a.M - 1);  // rows past M: a valid row, result dropped
+        ap[v] = (const unsigned char*)a.A + (long)m * a.K + (idx % 8) * 16;
+    }
+
+    i32x16_t acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+    u32x4_t ra[VA];
+    uint32_t bw[4][4];  // [k group of the tile][column block]
+    const int nkt = a.K / 128;
+
+#pragma unroll
+    for (int ch = 0; ch < 4; ++ch)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bw[ch][j] = wp[j][ch * 64];
+#pragma unroll
+    for (int v = 0; v < VA; ++v) ra[v] = *reinterpret_cast<const u32x4_t*>(ap[v]);
+#pragma unroll
+    for (int v = 0; v < VA; ++v) {
+        const int idx = tid + v * NT;
+        *reinterpret_cast<u32x4_t*>(&lds[0][(idx / 8) * STRIDE + (idx % 8) * 16]) = ra[v];
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < nkt; ++kt) {
+        const unsigned char* cur = lds[kt & 1];
+        const int kn = kt + 1 < nkt ? kt + 1 : kt;  // the last tile re-reads itself; copy unused
+#pragma unroll
+        for (int v = 0; v < VA; ++v) ra[v] = *reinterpret_cast<const u32x4_t*>(ap[v] + (long)kn * 128);
+        u32x4_t fa[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            fa[0][i] = *reinterpret_cast<const u32x4_t*>(cur + (wm * 64 + i * 32 + r) * STRIDE + g * 16);
+#pragma unroll
+        for (int ch = 0; ch < 4; ++ch) {
+            u32x4_t fw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t w = bw[ch][j];
+                fw[j][0] = w & 0x03030303u;
+                fw[j][1] = (w >> 2) & 0x03030303u;
+                fw[j][2] = (w >> 4) & 0x03030303u;
+                fw[j][3] = (w >> 6) & 0x03030303u;
+                bw[ch][j] = wp[j][(kn * 4 + ch) * 64];
+            }
+            if (ch < 3) {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    fa[(ch + 1) & 1][i] =
+                        *reinterpret_cast<const u32x4_t*>(cur + (wm * 64 + i * 32 + r) * STRIDE + (ch + 1) * 32 + g * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) Traits<int8_t>::mma(acc[i][j], fa[ch & 1][i], fw[j]);
+        }
+        unsigned char* nxt = lds[(kt + 1) & 1];
+#pragma unroll
+        for (int v = 0; v < VA; ++v) {
+            const int idx = tid + v * NT;
+            *reinterpret_cast<u32x4_t*>(nxt + (idx / 8) * STRIDE + (idx % 8) * 16) = ra[v];
+        }
+        __syncthreads();
+    }
+
+    // Accumulator element 4jj+ii of block (i, j) is row 8jj + 4g + ii, column r.
+    if (a.acc_out) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int m = m0 + wm * 64 + i * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
+                if (m >= a.M) continue;
+                const int rs2 = 2 * a.rowsum[m];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int n = n0 + j * 32 + r;
+                    if (n < a.N) a.acc_out[(long)m * a.N + n] = acc[i][j][e] - rs2;
+                }
+            }
+    }
+    if (!a.Y) return;
+
+    // bf16 output: out = float(acc - 2*rowsum) / s[m] * ws[group], staged per wavefront as
+    // 32 rows x 128 columns in LDS and written with 16-byte stores (16 lanes per row).
+    const int group = a.N / a.ws_num;
+    float wsc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = n0 + j * 32 + r;
+        wsc[j] = n < a.N ? a.ws[n / group] : 0.f;
+    }
+    // The division is the correctly rounded IEEE quotient.  When every scale of the
+    // wavefront's 64 rows is far from the exponent limits it is computed as the refinement
+    // sequence of the full-range expansion without its operand scaling (identical bits):
+    // y ~ 1/s by one Newton step on v_rcp_f32, then q0 = a*y, two residual corrections.
+    const float sabs = fabsf(a.s[min(m0 + wm * 64 + lane, a.M - 1)]);
+    const bool fast = __builtin_amdgcn_ballot_w64(sabs > 0x1p-60f && sabs < 0x1p60f) == ~0ull;
+    unsigned char* tp = &lds[0][0] + wave * (32 * T_STRIDE);
+    const bool vec_ok = (a.N % 8) == 0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        if (fast) {
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+                for (int ip = 0; ip < 4; ip += 2) {
+                    const int row = 8 * jj + 4 * g + ip;
+                    float sm[2], y[2];
+                    int rs2[2];
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const int mm = min(m0 + wm * 64 + i * 32 + row + t, a.M - 1);
+                        rs2[t] = 2 * a.rowsum[mm];
+                        sm[t] = a.s[mm];
+                        const float y0 = __builtin_amdgcn_rcpf(sm[t]);
+                        y[t] = __builtin_fmaf(__builtin_fmaf(-sm[t], y0, 1.0f), y0, y0);
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        float o[2];
+#pragma unroll
+                        for (int t = 0; t < 2; ++t) {
+                            const float av = (float)(acc[i][j][4 * jj + ip + t] - rs2[t]);
+                            const float q0 = av * y[t];
+                            const float q1 = __builtin_fmaf(__builtin_fmaf(-sm[t], q0, av), y[t], q0);
+                            o[t] = __builtin_fmaf(__builtin_fmaf(-sm[t], q1, av), y[t], q1) * wsc[j];
+                        }
+                        const uint32_t pk = pack_bf2(o[0], o[1]);
+                        *reinterpret_cast<bf16_t*>(tp + row * T_STRIDE + (j * 32 + r) * 2) = (bf16_t)(pk & 0xffff);
+                        *reinterpret_cast<bf16_t*>(tp + (row + 1) * T_STRIDE + (j * 32 + r) * 2) = (bf16_t)(pk >> 16);
+                    }
+                }
+        } else {
+#pragma unroll 1
+            for (int e = 0; e < 16; ++e) {
+                const int row = 8 * (e >> 2) + 4 * g + (e & 3);
+                const int mm = min(m0 + wm * 64 + i * 32 + row, a.M - 1);
+                const int rs2 = 2 * a.rowsum[mm];
+                const float sm = a.s[mm];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    int v = 0;
+#pragma unroll
+                    for (int e2 = 0; e2 < 16; ++e2) v = (e2 == e) ? acc[i][j][e2] : v;
+                    *reinterpret_cast<bf16_t*>(tp + row * T_STRIDE + (j * 32 + r) * 2) =
+                        f2bf((float)(v - rs2) / sm * wsc[j]);
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const int row = p * 4 + (lane >> 4), c16 = lane & 15;
+            const u32x4_t v = *reinterpret_cast<const u32x4_t*>(tp + row * T_STRIDE + c16 * 16);
+            const int m = m0 + wm * 64 + i * 32 + row, n = n0 + c16 * 8;
+            if (m >= a.M) continue;
+            bf16_t* dst = (bf16_t*)a.Y + (long)m * a.N + n;
+            if (vec_ok && n + 8 <= a.N) {
+                *reinterpret_cast<u32x4_t*>(dst) = v;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (n + e < a.N) dst[e] = (bf16_t)(v[e >> 1] >> (16 * (e & 1)));
+            }
+        }
+    }
+}
+
 template <typename T, int kEpi>
-int launch(const GemmArgs& a, int n_tiles, vla_stream_t stream) {
+int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
     if (a.M == 0 || n_tiles == 0) return VLA_K_OK;
-    dim3 grid(n_tiles, (a.M + BM - 1) / BM);
-    gemm_kernel<T, kEpi><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    a.n_tiles = n_tiles;
+    hipStream_t st = (hipStream_t)stream;
+    // Enough 128x128 tiles to occupy the chip: use them (half the LDS and L2 traffic per
+    // multiply); otherwise 64x64 tiles with 256-byte K rows (half the barriers per K).
+    const long big_tiles = (long)((a.M + 127) / 128) * ((n_tiles + 1) / 2);
+    if constexpr (kEpi != EPI_TERNARY) {
+        if (big_tiles >= 128) {
+            const unsigned grid = (unsigned)(((((n_tiles + 1) / 2) + 7) & ~7) * ((a.M + 127) / 128));
+            gemm_kernel<T, kEpi, 2, 2, 128><<<grid, 256, 0, st>>>(a);
+        } else {
+            const unsigned grid = (unsigned)(((n_tiles + 7) & ~7) * ((a.M + 63) / 64));
+            gemm_kernel<T, kEpi, 1, 1, 256><<<grid, 256, 0, st>>>(a);
+        }
+    } else {
+        // VLA_TERNARY_TILE = 64 | 128 | 256 pins the tile (tests and tuning); unset = by shape.
+        const char* env = getenv("VLA_TERNARY_TILE");
+        const int force = env ? atoi(env) : 0;
+        // Enough 128 x 256 tiles for half the chip: the large-M kernel, two workgroups per
+        // CU (measured faster than one 256 x 256 workgroup: fewer wavefronts per barrier).
+        const int n256 = (a.N + 255) / 256;
+        const long wg128 = (long)((a.M + 127) / 128) * n256;
+        if (force == 256) {
+            const unsigned grid = (unsigned)(((((a.M + 255) / 256) + 7) & ~7) * n256);
+            ternary_gemm_big_kernel<4><<<grid, 512, 0, st>>>(a);
+        } else if (force == 128 || (force == 0 && wg128 >= 128)) {
+            const unsigned grid = (unsigned)(((((a.M + 127) / 128) + 7) & ~7) * n256);
+            ternary_gemm_big_kernel<2><<<grid, 256, 0, st>>>(a);
+        } else {
+            const unsigned grid = (unsigned)(((n_tiles + 7) & ~7) * ((a.M + 63) / 64));
+            gemm_kernel<T, EPI_TERNARY, 1, 1, 128><<<grid, 256, 0, st>>>(a);
+        }
+    }
     return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
 }
 
@@ -495,9 +829,16 @@ int vla_ternary_quant_host(const float* W, int64_t n, int8_t* ternary, float* ab
     return VLA_K_OK;
 }
 
+long vla_ternary_packed_words(int N, int K) { return (long)((N + 31) / 32 * 32) * (K / 16); }
+
+static void tern_fill_pad_rows(int N, int K, uint32_t* packed) {
+    for (long n = N; n < (N + 31) / 32 * 32; ++n)
+        for (int w = 0; w < K / 16; ++w) packed[tern_word_index(n, w, K)] = 0xAAAAAAAAu;  // code 2 = weight 0
+}
+
 int vla_ternary_pack_host(const int8_t* ternary, int N, int K, uint32_t* packed) {
     if (!ternary || !packed || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
-    if (K % 16) return VLA_K_ERR_SHAPE;
+    if (K % 32) return VLA_K_ERR_SHAPE;
     const int kw = K / 16;
     for (long n = 0; n < N; ++n)
         for (int w = 0; w < kw; ++w) {
@@ -507,8 +848,9 @@ int vla_ternary_pack_host(const int8_t* ternary, int N, int K, uint32_t* packed)
                 if (t < -2 || t > 1) return VLA_K_ERR_ARG;
                 word |= (uint32_t)((t + 2) & 3) << (8 * (v & 3) + 2 * (v >> 2));
             }
-            packed[n * kw + w] = word;
+            packed[tern_word_index(n, w, K)] = word;
         }
+    tern_fill_pad_rows(N, K, packed);
     return VLA_K_OK;
 }
 
@@ -526,8 +868,9 @@ int vla_ternary_repack_ladder_host(const uint8_t* ladder, int N, int K, uint32_t
             const int y = (int)(n % 16), y_half = y / 8, y_in_h = y % 8;
             const int k_0 = w / 8, tx = w % 8, major_k = tx / 2, sub_k = tx % 2;
             const long slot = n_block * K + (long)k_0 * 128 + major_k * 32 + y_half * 16 + sub_k * 8 + y_in_h;
-            packed[n * kw + w] = src[slot];
+            packed[tern_word_index(n, w, K)] = src[slot];
         }
+    tern_fill_pad_rows(N, K, packed);
     return VLA_K_OK;
 }
 

@@ -44,7 +44,7 @@ TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::
     TernaryW w;
     w.K = K;
     for (int n : parts) w.N += n;
-    std::vector<uint32_t> packed((size_t)w.N * (K / 16));
+    std::vector<uint32_t> packed((size_t)vla_ternary_packed_words(w.N, K));
     std::vector<float> scales;
     if (ck.has(name + ".i2")) {
         VLA_K(vla_ternary_repack_ladder_host((const uint8_t*)ck.data(name + ".i2"), w.N, K, packed.data()));
