@@ -31,7 +31,10 @@ extern "C" {
 
 typedef void* vla_stream_t; /* a hipStream_t */
 
-typedef enum { VLA_DT_F32 = 0, VLA_DT_BF16 = 1 } vla_dtype;
+/* VLA_DT_BF16_P2 is accepted by vla_attn_prefix_suffix only: bf16 storage as VLA_DT_BF16,
+ * with the softmax probabilities carried as two bf16 terms (about 16 mantissa bits) through
+ * the P.V product, at twice the MFMA work of that product. */
+typedef enum { VLA_DT_F32 = 0, VLA_DT_BF16 = 1, VLA_DT_BF16_P2 = 2 } vla_dtype;
 
 typedef enum {
     VLA_K_OK = 0,

@@ -213,6 +213,10 @@ CASES = [
     ("gr00t-self", 3, 17, 32, 32, 48, 0, "none", (0, 0)),
     ("bitvla-decode", 2, 1, 20, 5, 128, 515, "cross", (0, 0)),
     ("bitvla-prefill", 1, 130, 20, 5, 128, 0, "none", (0, 0)),
+    # at most 32 query rows per kv head: the register-direct kernel, with every mask kind
+    ("short-causal", 2, 10, 6, 2, 64, 100, "causal", (90, 97)),
+    ("short-pi0", 1, 4, 8, 1, 128, 75, "pi0", (0, 0)),
+    ("short-ragged", 5, 3, 4, 4, 48, 37, "cross", (30, 33)),
 ]
 
 
@@ -266,8 +270,40 @@ def test_attention_against_oracle(dtype, case):
     else:
         assert bf16_close(got, want) and bf16_close(got_m, want)
         assert rel_err(got, want) < 1e-2
+        # split-precision probabilities: same storage, P.V product within output rounding
+        out_p2 = empty((B, S, Hq * D), dtype)
+        pkg.call("vla_attn_prefix_suffix", to_dev(Q, dtype), kc, vc, out_p2, pkg.VLA_DT_BF16_P2, B, S, Hq, Hkv, D, t_max, T,
+                 scale, mkind, P, pad[0], pad[1], None)
+        sync()
+        got_p2 = as_f32(out_p2, dtype)
+        assert bf16_close(got_p2, want) and rel_err(got_p2, want) < 4e-3
+        assert rel_err(got_p2, want) <= rel_err(got, want) * 1.05
     # generated mask and mask-as-data run the same arithmetic
     assert np.array_equal(host(out), host(out_m))
+
+
+@pytest.mark.parametrize("split", [1, 2, 5, 64])
+def test_attention_direct_kernel_key_slices_merge(monkeypatch, split):
+    # Few query rows: any slicing of the keys across wavefronts (merged by the second
+    # kernel) gives the same result as the oracle.
+    r = np.random.default_rng(120 + split)
+    B, S, Hq, Hkv, D, T = 2, 5, 6, 2, 64, 333
+    t_max = 336
+    Q = orc.round_bf16(r.standard_normal((B, S, Hq, D)).astype(np.float32))
+    K = orc.round_bf16(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    V = orc.round_bf16(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    kc = torch.full((B, Hkv, t_max, D), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
+    vc = torch.full((B, Hkv, D, t_max), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
+    pkg.call("vla_kv_append", kc, vc, to_dev(K, BF16), to_dev(V, BF16), BF16, B, Hkv, D, t_max, 0, T)
+    monkeypatch.setenv("VLA_ATTN_SPLIT", str(split))
+    out = empty((B, S, Hq * D), BF16)
+    pkg.call("vla_attn_prefix_suffix", to_dev(Q, BF16), kc, vc, out, BF16, B, S, Hq, Hkv, D, t_max, T, 0.125,
+             pkg.VLA_MASK_CAUSAL_SUFFIX, T - S, 100, 120, None)
+    sync()
+    mask = orc.mask_smolvla_full(T - S, S, 100, 120)
+    want = np.stack([orc.attention(Q[b], K[b], V[b], mask, 0.125) for b in range(B)])
+    got = as_f32(out, BF16)
+    assert np.isfinite(got).all() and bf16_close(got, want) and rel_err(got, want) < 1e-2
 
 
 def test_attention_special_cases_fp32():

@@ -15,7 +15,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libvla.so")
 
-VLA_DT_F32, VLA_DT_BF16 = 0, 1
+VLA_DT_F32, VLA_DT_BF16, VLA_DT_BF16_P2 = 0, 1, 2
 VLA_MASK_NONE, VLA_MASK_CAUSAL_SUFFIX, VLA_MASK_PI0_STATE = 0, 1, 2
 VLA_K_OK, VLA_K_ERR_ARG, VLA_K_ERR_SHAPE, VLA_K_ERR_LAUNCH = 0, -1, -2, -3
 

@@ -36,6 +36,8 @@
 #include <math.h>
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "vla_kernels.h"
 
@@ -43,7 +45,8 @@ namespace {
 
 using namespace vk;
 
-constexpr int TK = 64;  // keys per LDS tile
+constexpr float RESCALE_LOG2 = 8.0f;  // see the online softmax
+constexpr int SPLIT_KEYS = 64;  // granularity of key slices; keys per LDS tile of narrow heads
 
 struct AttnArgs {
     const void* q;
@@ -54,7 +57,7 @@ struct AttnArgs {
     float scale;
     int mask_kind, n_prefix, pad_start, pad_end;
     const float* mask;
-    int n_groups, n_split, tiles_per_split, r_pad;
+    int n_groups, n_split, tiles_per_split, r_pad, p2;
     float* part_o;   // [pair][split][r_pad][D]
     float* part_ml;  // [pair][split][r_pad][2]
 };
@@ -80,10 +83,14 @@ template <> struct AT<float> {
     __device__ static __forceinline__ float fexp2(float x) { return exp2f(x); }
 };
 
-template <typename T, int D, int NW>
-__global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
+template <typename T, int D, int NW, bool P2>
+__global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_kernel(AttnArgs a) {
     typedef AT<T> A;
     constexpr int EB = A::EB, CE = A::CE;
+    // Keys per staged tile: 64, or 32 for wide heads (rows of 512 bytes and more), whose
+    // accumulators and query fragments leave too few registers to stage 64 keys.
+    constexpr int TK = (D * EB >= 512) ? 32 : SPLIT_KEYS;
+    constexpr int NKB = TK / 32;
     constexpr int DP = (D + 31) / 32 * 32;  // head_dim padded to whole 32-row output blocks
     constexpr int NQ = D / CE;              // MFMA groups along head_dim
     constexpr int NDB = DP / 32;            // 32-row blocks of O^T
@@ -122,8 +129,8 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     const int s = row_valid ? row % a.S : 0;
     const int h = hk * grp + hg;
 
-    const int k_begin = split * a.tiles_per_split * TK;
-    const int k_end = min(a.n_keys, k_begin + a.tiles_per_split * TK);
+    const int k_begin = split * a.tiles_per_split * SPLIT_KEYS;
+    const int k_end = min(a.n_keys, k_begin + a.tiles_per_split * SPLIT_KEYS);
 
     // Q fragments: B operand, lane (g, r) holds 16 bytes of query row r per group.
     u32x4_t qf[NQ];
@@ -149,95 +156,90 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
     const unsigned char* kbase = (const unsigned char*)a.k_cache + ((long)b * a.Hkv + hk) * a.t_max * D * EB;
     const unsigned char* vbase = (const unsigned char*)a.vt_cache + ((long)b * a.Hkv + hk) * D * (long)a.t_max * EB;
 
+    // Per-row visibility of the generated masks, branch-free: a key is visible iff
+    // key < hi and it is not inside the padded-language range of the prefix.
+    int hi = a.n_keys;
+    if (a.mask_kind == VLA_MASK_CAUSAL_SUFFIX) hi = min(a.n_keys, a.n_prefix + s + 1);
+    else if (a.mask_kind == VLA_MASK_PI0_STATE && s == 0) hi = min(a.n_keys, a.n_prefix + 1);
+    const int pad_lo = a.pad_start, pad_hi = min(a.pad_end, a.n_prefix);
+
+    // Staging.  Full tiles are plain block copies with no bounds checks; only the last,
+    // partial tile clamps K rows to a valid key and zeroes V^T elements past n_keys, so
+    // that stale cache contents (possibly NaN) cannot reach the accumulators.
+    constexpr bool EXACT = (NVEC % NT) == 0;
     u32x4_t kreg[IT], vreg[IT];
-    auto load_k = [&](int k0) {
+    auto load_k = [&](int k0) __attribute__((always_inline)) {
+        if (k0 + TK <= a.n_keys) {  // uniform
 #pragma unroll
-        for (int i = 0; i < IT; ++i) {
-            const int v = tid + i * NT;
-            const int key = v / KV_PER_ROW, c = v % KV_PER_ROW;
-            u32x4_t val = {0u, 0u, 0u, 0u};
-            if (v < NVEC && k0 + key < a.n_keys)
-                val = *reinterpret_cast<const u32x4_t*>(kbase + ((long)(k0 + key) * D * EB) + c * 16);
-            kreg[i] = val;
+            for (int i = 0; i < IT; ++i) {
+                const int v = tid + i * NT;
+                if (EXACT || i < IT - 1 || v < NVEC) kreg[i] = *reinterpret_cast<const u32x4_t*>(kbase + (long)k0 * D * EB + v * 16);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < IT; ++i) {
+                const int v = tid + i * NT;
+                if (!(EXACT || i < IT - 1 || v < NVEC)) continue;
+                const int key = min(k0 + v / KV_PER_ROW, a.n_keys - 1);
+                kreg[i] = *reinterpret_cast<const u32x4_t*>(kbase + (long)key * D * EB + (v % KV_PER_ROW) * 16);
+            }
         }
     };
-    auto load_v = [&](int k0) {
+    auto load_v = [&](int k0) __attribute__((always_inline)) {
+        if (k0 + TK <= a.n_keys) {  // uniform
 #pragma unroll
-        for (int i = 0; i < IT; ++i) {
-            const int v = tid + i * NT;
-            const int d = v / VV_PER_ROW, c = v % VV_PER_ROW;
-            const int key = k0 + c * EPV;
-            u32x4_t val = {0u, 0u, 0u, 0u};
-            if (v < NVEC && key < a.n_keys) val = *reinterpret_cast<const u32x4_t*>(vbase + ((long)d * a.t_max + key) * EB);
-            vreg[i] = val;
-        }
-    };
-    auto store_k = [&]() {
+            for (int i = 0; i < IT; ++i) {
+                const int v = tid + i * NT;
+                if (EXACT || i < IT - 1 || v < NVEC)
+                    vreg[i] = *reinterpret_cast<const u32x4_t*>(vbase + ((long)(v / VV_PER_ROW) * a.t_max + k0 + (v % VV_PER_ROW) * EPV) * EB);
+            }
+        } else {
 #pragma unroll
-        for (int i = 0; i < IT; ++i) {
-            const int v = tid + i * NT;
-            if (v < NVEC) *reinterpret_cast<u32x4_t*>(ldsK + (v / KV_PER_ROW) * KS + (v % KV_PER_ROW) * 16) = kreg[i];
-        }
-    };
-    // Keys past n_keys are zeroed element-wise so that stale cache contents cannot
-    // reach the accumulators (0 * NaN).
-    auto store_v = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < IT; ++i) {
-            const int v = tid + i * NT;
-            const int d = v / VV_PER_ROW, c = v % VV_PER_ROW;
-            const int key = k0 + c * EPV;
-            u32x4_t val = vreg[i];
-            if (key < a.n_keys && key + EPV > a.n_keys) {
-                const int nvalid = a.n_keys - key;
+            for (int i = 0; i < IT; ++i) {
+                const int v = tid + i * NT;
+                if (!(EXACT || i < IT - 1 || v < NVEC)) continue;
+                const int d = v / VV_PER_ROW, key0 = k0 + (v % VV_PER_ROW) * EPV;
+                u32x4_t val = {0u, 0u, 0u, 0u};
+                if (key0 < a.n_keys) val = *reinterpret_cast<const u32x4_t*>(vbase + ((long)d * a.t_max + key0) * EB);
+                const int nvalid = a.n_keys - key0;  // elements of this vector that are real keys
                 if (EB == 2) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t lo = (2 * e < nvalid) ? 0xffffu : 0u, hi = (2 * e + 1 < nvalid) ? 0xffff0000u : 0u;
-                        val[e] &= (lo | hi);
-                    }
+                    for (int e = 0; e < 4; ++e)
+                        val[e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (e >= nvalid) val[e] = 0u;
+                    for (int e = 0; e < 4; ++e) val[e] = e < nvalid ? val[e] : 0u;
                 }
+                vreg[i] = val;
             }
-            if (v < NVEC) *reinterpret_cast<u32x4_t*>(ldsV + d * VS + c * 16) = val;
+        }
+    };
+    auto store_k = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int v = tid + i * NT;
+            if (!(EXACT || i < IT - 1 || v < NVEC)) continue;
+            *reinterpret_cast<u32x4_t*>(ldsK + (v / KV_PER_ROW) * KS + (v % KV_PER_ROW) * 16) = kreg[i];
+        }
+    };
+    auto store_v = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int v = tid + i * NT;
+            if (!(EXACT || i < IT - 1 || v < NVEC)) continue;
+            *reinterpret_cast<u32x4_t*>(ldsV + (v / VV_PER_ROW) * VS + (v % VV_PER_ROW) * 16) = vreg[i];
         }
     };
 
-    if (PREFETCH && k_begin < k_end) {
-        load_k(k_begin);
-        load_v(k_begin);
-    }
-    for (int k0 = k_begin; k0 < k_end; k0 += TK) {
-        __syncthreads();  // previous tile fully consumed
-        if (PREFETCH) {
-            store_k();
-            store_v(k0);
-        } else {
-            load_k(k0);
-            load_v(k0);
-            store_k();
-            store_v(k0);
-        }
-        __syncthreads();
-        if (PREFETCH && k0 + TK < k_end) {
-            load_k(k0 + TK);
-            load_v(k0 + TK);
-        }
-        if (!wave_active) continue;
-
+    // Scores and online softmax of the staged K tile; leaves the probabilities in p.
+    float p[NKB][16];
+    auto scores_softmax = [&](int k0) __attribute__((always_inline)) {
         // Whether any key of this tile can be hidden from any row (uniform per tile).
-        const bool tile_masked = a.mask != nullptr || k0 + TK > a.n_keys ||
-                                 (k0 < a.pad_end && k0 + TK > a.pad_start && a.pad_start < a.pad_end) ||
+        const bool tile_masked = a.mask != nullptr || k0 + TK > a.n_keys || (k0 < pad_hi && k0 + TK > pad_lo) ||
                                  (a.mask_kind != VLA_MASK_NONE && k0 + TK > a.n_prefix);
-
-        // ---- scores S^T for the two 32-key blocks of the tile
-        float p[2][16];
         float m_tile = -INFINITY;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < NKB; ++kb) {
             f32x16_t sc;
 #pragma unroll
             for (int i = 0; i < 16; ++i) sc[i] = 0.f;
@@ -246,44 +248,54 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
                 const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(ldsK + (kb * 32 + r) * KS + (c * CE + g * (CE / 2)) * EB);
                 A::mma(sc, kf, qf[c]);
             }
-            if (!tile_masked) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float v = sc[i] * c2;
-                    p[kb][i] = v;
-                    m_tile = fmaxf(m_tile, v);
-                }
+            for (int i = 0; i < 16; ++i) p[kb][i] = sc[i] * c2;
+        }
+        if (tile_masked) {
+            if (a.mask) {  // mask given as data: additive, one fp32 per (query, key)
+#pragma unroll
+                for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int key = k0 + kb * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
+                        p[kb][e] = key < a.n_keys ? p[kb][e] + a.mask[(long)s * a.n_keys + key] * LOG2E : -INFINITY;
+                    }
             } else {
+                const int kl = k0 + 4 * g;
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int key = k0 + kb * 32 + 8 * j + 4 * g + i;
-                        float v = sc[4 * j + i] * c2;
-                        bool blocked = key >= a.n_keys;
-                        if (a.mask) {
-                            if (!blocked) v += a.mask[(long)s * a.n_keys + key] * LOG2E;
-                        } else if (key < a.n_prefix) {
-                            blocked |= (key >= a.pad_start && key < a.pad_end);
-                        } else {
-                            const int si = key - a.n_prefix;
-                            if (a.mask_kind == VLA_MASK_CAUSAL_SUFFIX) blocked |= si > s;
-                            else if (a.mask_kind == VLA_MASK_PI0_STATE) blocked |= (s == 0 && si != 0);
-                        }
-                        v = blocked ? -INFINITY : v;
-                        p[kb][4 * j + i] = v;
-                        m_tile = fmaxf(m_tile, v);
+                    for (int e = 0; e < 16; ++e) {
+                        const int key = kl + kb * 32 + 8 * (e >> 2) + (e & 3);
+                        const bool visible = (key < hi) & !((key >= pad_lo) & (key < pad_hi));
+                        p[kb][e] = visible ? p[kb][e] : -INFINITY;
                     }
             }
         }
+#pragma unroll
+        for (int kb = 0; kb < NKB; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) m_tile = fmaxf(m_tile, p[kb][i]);
         m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
-        const float m_new = fmaxf(m_run, m_tile);
-        // m_new == -inf: nothing visible yet, keep everything at zero.
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = A::fexp2(m_run - m_use);  // 2^-inf = 0 on the first visible tile
+        // Online softmax with a lazily updated reference: m_run moves (and the accumulators
+        // are rescaled) only when some row's maximum exceeds it by more than 2^RESCALE_LOG2;
+        // until then the probabilities are taken against the older reference, at most
+        // 2^RESCALE_LOG2 large, and the common factor cancels in o / l at the end.
+        if (__builtin_amdgcn_ballot_w64(m_tile > m_run + RESCALE_LOG2) != 0) {
+            const float m_new = fmaxf(m_run, m_tile);
+            // m_new == -inf: nothing visible yet, keep everything at zero.
+            const float alpha = A::fexp2(m_run - ((m_new == -INFINITY) ? 0.f : m_new));  // 2^-inf = 0 at the first visible tile
+            l_run *= alpha;
+            m_run = m_new;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
         float psum = 0.f;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const float e = A::fexp2(p[kb][i] - m_use);
@@ -291,29 +303,27 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
                 psum += e;
             }
         psum += __shfl_xor(psum, 32, 64);
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
+        l_run += psum;
+    };
+    // O^T += V^T . P^T from the staged V^T tile.
+    auto output_product = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
-
-        // ---- O^T += V^T . P^T
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int kb = 0; kb < NKB; ++kb) {
             if (EB == 2) {
 #pragma unroll
                 for (int hh = 0; hh < 2; ++hh) {
-                    // The probabilities enter the bf16 MFMA as hi + lo (two bf16 terms,
-                    // ~16 mantissa bits): the P.V product then matches an fp32-probability
-                    // reference instead of carrying an extra 2^-9 rounding per weight.
+                    // P2: the probabilities enter the bf16 MFMA as hi + lo (two bf16 terms,
+                    // ~16 mantissa bits), so the P.V product matches an fp32-probability
+                    // reference instead of carrying a 2^-9 rounding per weight; otherwise
+                    // one bf16 term (the rounding is of the size of the output's own).
                     const float* pp = &p[kb][hh * 8];
                     u32x4_t pf, pl;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const uint32_t hi = pack_bf2(pp[2 * e], pp[2 * e + 1]);
-                        pf[e] = hi;
-                        pl[e] = pack_bf2(pp[2 * e] - __uint_as_float(hi << 16), pp[2 * e + 1] - __uint_as_float(hi & 0xffff0000u));
+                        const uint32_t hi16 = pack_bf2(pp[2 * e], pp[2 * e + 1]);
+                        pf[e] = hi16;
+                        if (P2)
+                            pl[e] = pack_bf2(pp[2 * e] - __uint_as_float(hi16 << 16), pp[2 * e + 1] - __uint_as_float(hi16 & 0xffff0000u));
                     }
                     const int key_off = (kb * 32 + hh * 16 + 4 * g) * EB;
 #pragma unroll
@@ -323,7 +333,7 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
                         const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(vr + 8 * EB);
                         const u32x4_t vf = {v0[0], v0[1], v1[0], v1[1]};
                         A::mma(o[db], vf, pf);
-                        A::mma(o[db], vf, pl);
+                        if (P2) A::mma(o[db], vf, pl);
                     }
                 }
             } else {
@@ -340,6 +350,50 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
                     }
                 }
             }
+        }
+    };
+
+    if (PREFETCH) {
+        // Small tiles: the whole next tile waits in registers while the current one is used.
+        if (k_begin < k_end) {
+            load_k(k_begin);
+            load_v(k_begin);
+        }
+        for (int k0 = k_begin; k0 < k_end; k0 += TK) {
+            __syncthreads();  // previous tile fully consumed
+            store_k();
+            store_v();
+            __syncthreads();
+            if (k0 + TK < k_end) {
+                load_k(k0 + TK);
+                load_v(k0 + TK);
+            }
+            // keep the loads above the math: left alone, the scheduler sinks them next to
+            // their first use (the next iteration's LDS stores) and the prefetch is lost
+            __builtin_amdgcn_sched_barrier(0);
+            if (wave_active) {
+                scores_softmax(k0);
+                output_product();
+            }
+        }
+    } else {
+        // Wide heads: one operand in registers at a time.  V^T of this tile is fetched
+        // under the score product, K of the next tile under the output product.  Nobody
+        // reads the K buffer between the second barrier of a tile and the first of the
+        // next, nor the V^T buffer between a tile's output product and the next first
+        // barrier, so two barriers per tile suffice.
+        if (k_begin < k_end) load_k(k_begin);
+        for (int k0 = k_begin; k0 < k_end; k0 += TK) {
+            store_k();
+            __syncthreads();
+            load_v(k0);
+            __builtin_amdgcn_sched_barrier(0);  // loads stay above the math they hide behind
+            if (wave_active) scores_softmax(k0);
+            store_v();
+            __syncthreads();
+            if (k0 + TK < k_end) load_k(k0 + TK);
+            __builtin_amdgcn_sched_barrier(0);
+            if (wave_active) output_product();
         }
     }
 
@@ -380,6 +434,233 @@ __global__ void __launch_bounds__(NW * 64) attn_kernel(AttnArgs a) {
                 const f32x4_t pk = {v0, v1, v2, v3};
                 *reinterpret_cast<f32x4_t*>(orow + d * EB) = pk;
             }
+        }
+}
+
+// Few query rows per (batch, kv head) -- at most one 32-row tile: GR00T's 17 DiT tokens,
+// single-token decode.  Nothing is shared between wavefronts then, so K and V^T go straight
+// from the cache into MFMA operand registers (no LDS, no barriers): lane (g, r) of a
+// wavefront reads 16 bytes of key row r for the score product and two 8-byte runs of V^T
+// row r for the output product, exactly the fragments the LDS kernel would fetch.  A
+// wavefront owns one (pair, key slice) and keeps ST 32-key blocks of loads in flight.
+template <int D, bool P2, int ST>
+__global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attn_direct_kernel(AttnArgs a) {
+    constexpr int EB = 2, CE = 16;
+    constexpr int NQ = D / CE, NDB = (D + 31) / 32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int g = lane >> 5, r = lane & 31;
+    const int unit = blockIdx.x * 4 + wave;
+    const int pair = unit / a.n_split, split = unit % a.n_split;
+    if (pair >= a.batch * a.Hkv) return;  // whole wavefront; the kernel has no barriers
+    const int b = pair / a.Hkv, hk = pair % a.Hkv;
+    const int grp = a.Hq / a.Hkv, R = grp * a.S;
+    const bool row_valid = r < R;
+    const int hg = row_valid ? r / a.S : 0, s = row_valid ? r % a.S : 0;
+    const int h = hk * grp + hg;
+
+    const int nb_total = (a.n_keys + 31) / 32;
+    const int kb0 = split * a.tiles_per_split, kb1 = min(nb_total, kb0 + a.tiles_per_split);
+
+    u32x4_t qf[NQ];
+    {
+        const unsigned char* qrow = (const unsigned char*)a.q + (((long)b * a.S + s) * a.Hq + h) * D * EB;
+#pragma unroll
+        for (int c = 0; c < NQ; ++c) {
+            u32x4_t z = {0u, 0u, 0u, 0u};
+            qf[c] = row_valid ? *reinterpret_cast<const u32x4_t*>(qrow + (c * CE + g * 8) * EB) : z;
+        }
+    }
+    f32x16_t o[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float c2 = a.scale * LOG2E;
+
+    const unsigned char* kbase = (const unsigned char*)a.k_cache + ((long)b * a.Hkv + hk) * a.t_max * D * EB;
+    const unsigned char* vbase = (const unsigned char*)a.vt_cache + ((long)b * a.Hkv + hk) * D * (long)a.t_max * EB;
+
+    u32x4_t kr[ST][NQ];
+    u32x2_t vr[ST][NDB][2][2];  // [stage][32-row block of d][16-key half][8-byte run]
+    // Rows of V^T past head_dim (D = 48: the upper half of the second 32-row block) are
+    // read from row D-1 instead, so every lane loads valid memory; their outputs are dropped.
+    const unsigned char* vrow[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) vrow[db] = vbase + ((long)min(db * 32 + r, D - 1) * a.t_max + 4 * g) * EB;
+    auto load_full = [&](int st, int kb) __attribute__((always_inline)) {  // no checks at all
+        const unsigned char* kp = kbase + (long)(kb * 32 + r) * D * EB + g * 16;
+#pragma unroll
+        for (int c = 0; c < NQ; ++c) kr[st][c] = *reinterpret_cast<const u32x4_t*>(kp + c * CE * EB);
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+                for (int q = 0; q < 2; ++q)
+                    vr[st][db][hh][q] = *reinterpret_cast<const u32x2_t*>(vrow[db] + (kb * 32 + hh * 16 + q * 8) * EB);
+    };
+    // A partial block: K rows past n_keys repeat the last key (their scores are masked);
+    // V^T elements past n_keys are zeroed so that stale cache contents (possibly NaN)
+    // cannot reach the accumulators.
+    auto load_partial = [&](int st, int kb) __attribute__((always_inline)) {
+        const int key = min(kb * 32 + r, a.n_keys - 1);
+        const unsigned char* kp = kbase + (long)key * D * EB + g * 16;
+#pragma unroll
+        for (int c = 0; c < NQ; ++c) kr[st][c] = *reinterpret_cast<const u32x4_t*>(kp + c * CE * EB);
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int k4 = kb * 32 + hh * 16 + q * 8 + 4 * g;  // first of 4 consecutive keys
+                    u32x2_t val = {0u, 0u};
+                    // n_keys <= t_max and t_max is a multiple of 8: a group starting below n_keys is inside the row
+                    if (k4 < a.n_keys) val = *reinterpret_cast<const u32x2_t*>(vrow[db] + (kb * 32 + hh * 16 + q * 8) * EB);
+                    const int nvalid = a.n_keys - k4;
+                    val[0] &= (nvalid > 0 ? 0xffffu : 0u) | (nvalid > 1 ? 0xffff0000u : 0u);
+                    val[1] &= (nvalid > 2 ? 0xffffu : 0u) | (nvalid > 3 ? 0xffff0000u : 0u);
+                    vr[st][db][hh][q] = val;
+                }
+    };
+    // Per-row visibility of the generated masks, branch-free (see the LDS kernel).
+    int hi = a.n_keys;
+    if (a.mask_kind == VLA_MASK_CAUSAL_SUFFIX) hi = min(a.n_keys, a.n_prefix + s + 1);
+    else if (a.mask_kind == VLA_MASK_PI0_STATE && s == 0) hi = min(a.n_keys, a.n_prefix + 1);
+    const int pad_lo = a.pad_start, pad_hi = min(a.pad_end, a.n_prefix);
+    // `live` = false: a phantom block past the slice (the pipeline is padded to whole groups
+    // of ST blocks); every key is hidden, so it leaves the state untouched.
+    auto compute = [&](int st, int kb, bool live) __attribute__((always_inline)) {
+        const int k0 = kb * 32;
+        f32x16_t sc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NQ; ++c) AT<bf16_t>::mma(sc, kr[st][c], qf[c]);
+        const bool blk_masked = !live || a.mask != nullptr || k0 + 32 > a.n_keys || (k0 < pad_hi && k0 + 32 > pad_lo) ||
+                                (a.mask_kind != VLA_MASK_NONE && k0 + 32 > a.n_prefix);
+        float p[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) p[i] = sc[i] * c2;
+        if (blk_masked) {
+            if (a.mask && live) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = k0 + 8 * (e >> 2) + 4 * g + (e & 3);
+                    p[e] = key < a.n_keys ? p[e] + a.mask[(long)s * a.n_keys + key] * LOG2E : -INFINITY;
+                }
+            } else {
+                const int kl = k0 + 4 * g, hi_blk = live ? hi : 0;
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int key = kl + 8 * (e >> 2) + (e & 3);
+                    const bool visible = (key < hi_blk) & !((key >= pad_lo) & (key < pad_hi));
+                    p[e] = visible ? p[e] : -INFINITY;
+                }
+            }
+        }
+        float m_blk = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) m_blk = fmaxf(m_blk, p[i]);
+        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
+        if (__builtin_amdgcn_ballot_w64(m_blk > m_run + RESCALE_LOG2) != 0) {  // lazy reference update
+            const float m_new = fmaxf(m_run, m_blk);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - ((m_new == -INFINITY) ? 0.f : m_new));
+            l_run *= alpha;
+            m_run = m_new;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            p[i] = __builtin_amdgcn_exp2f(p[i] - m_use);
+            psum += p[i];
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        l_run += psum;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            const float* pp = &p[hh * 8];
+            u32x4_t pf, pl;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t hi = pack_bf2(pp[2 * e], pp[2 * e + 1]);
+                pf[e] = hi;
+                if (P2) pl[e] = pack_bf2(pp[2 * e] - __uint_as_float(hi << 16), pp[2 * e + 1] - __uint_as_float(hi & 0xffff0000u));
+            }
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) {
+                const u32x4_t vf = {vr[st][db][hh][0][0], vr[st][db][hh][0][1], vr[st][db][hh][1][0], vr[st][db][hh][1][1]};
+                AT<bf16_t>::mma(o[db], vf, pf);
+                if (P2) AT<bf16_t>::mma(o[db], vf, pl);
+            }
+        }
+    };
+
+    // Software pipeline over the slice's full blocks [kb0, kbf): ST - 1 blocks of loads
+    // stay in flight ahead of the block being multiplied.  The loop body is branch-free:
+    // the block count is padded to whole groups of ST, loads past the last full block
+    // re-read it, and the padded blocks are multiplied as phantoms.  A trailing partial
+    // block (only the slice that reaches n_keys has one) is loaded first, into the stage
+    // the pipeline needs last, and consumed while the first pipeline loads are in flight.
+    const bool has_partial = kb1 * 32 > a.n_keys;  // uniform
+    const int kbf = has_partial ? kb1 - 1 : kb1;
+    const int n_full = kbf - kb0;
+    if (has_partial) load_partial(ST - 1, kb1 - 1);
+    if (n_full > 0) {
+#pragma unroll
+        for (int i = 0; i < ST - 1; ++i) load_full(i, min(kb0 + i, kbf - 1));
+    }
+    if (has_partial) compute(ST - 1, kb1 - 1, true);
+    if (n_full > 0) {
+        const int groups = (n_full + ST - 1) / ST;
+        for (int gi = 0; gi < groups; ++gi) {
+#pragma unroll
+            for (int st = 0; st < ST; ++st) {
+                const int cur = kb0 + gi * ST + st;
+                load_full((st + ST - 1) % ST, min(cur + ST - 1, kbf - 1));
+                __builtin_amdgcn_sched_barrier(0);  // loads stay above the math they hide behind
+                compute(st, cur, cur < kbf);
+            }
+        }
+    }
+
+    if (!row_valid) return;
+    if (a.n_split > 1) {
+        const long prow = ((long)pair * a.n_split + split) * a.r_pad + r;
+        if (g == 0) {
+            a.part_ml[prow * 2] = m_run;
+            a.part_ml[prow * 2 + 1] = l_run;
+        }
+        float* po = a.part_o + prow * D;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int d = db * 32 + 8 * j + 4 * g;
+                if (d >= D) continue;
+                const f32x4_t pk = {o[db][4 * j], o[db][4 * j + 1], o[db][4 * j + 2], o[db][4 * j + 3]};
+                *reinterpret_cast<f32x4_t*>(po + d) = pk;
+            }
+        return;
+    }
+    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+    unsigned char* orow = (unsigned char*)a.out + (((long)b * a.S + s) * a.Hq + h) * D * EB;
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int d = db * 32 + 8 * j + 4 * g;
+            if (d >= D) continue;
+            const u32x2_t pk = {pack_bf2(o[db][4 * j] * inv, o[db][4 * j + 1] * inv),
+                                pack_bf2(o[db][4 * j + 2] * inv, o[db][4 * j + 3] * inv)};
+            *reinterpret_cast<u32x2_t*>(orow + d * EB) = pk;
         }
 }
 
@@ -430,7 +711,12 @@ template <typename T, int D, int NW>
 int launch_nw(AttnArgs& a, hipStream_t st) {
     const int n_pairs = a.batch * a.Hkv;
     const int grid = (n_pairs + 7) / 8 * 8 * a.n_groups * a.n_split;
-    attn_kernel<T, D, NW><<<grid, NW * 64, 0, st>>>(a);
+    if constexpr (sizeof(T) == 2) {
+        if (a.p2) attn_kernel<T, D, NW, true><<<grid, NW * 64, 0, st>>>(a);
+        else attn_kernel<T, D, NW, false><<<grid, NW * 64, 0, st>>>(a);
+    } else {
+        attn_kernel<T, D, NW, false><<<grid, NW * 64, 0, st>>>(a);
+    }
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     if (a.n_split > 1) {
         const int R = (a.Hq / a.Hkv) * a.S;
@@ -442,10 +728,51 @@ int launch_nw(AttnArgs& a, hipStream_t st) {
     return VLA_K_OK;
 }
 
+template <int D>
+int launch_direct(AttnArgs& a, hipStream_t st) {
+    constexpr int ST = D <= 64 ? 3 : 2;
+    const int n_pairs = a.batch * a.Hkv;
+    const int nb_total = (a.n_keys + 31) / 32;
+    // Enough wavefronts to keep every CU's memory pipeline busy (8 per CU); a slice is
+    // at least two 32-key blocks unless the whole sequence is shorter.
+    int n_split = 1;
+    if (n_pairs < 2048) n_split = (2048 + n_pairs - 1) / n_pairs;
+    if (n_split > (nb_total + 1) / 2) n_split = (nb_total + 1) / 2;
+    if (n_split < 1) n_split = 1;
+    if (const char* e = getenv("VLA_ATTN_SPLIT")) n_split = atoi(e) > 0 ? (atoi(e) < nb_total ? atoi(e) : nb_total) : 1;
+    a.tiles_per_split = (nb_total + n_split - 1) / n_split;
+    a.n_split = (nb_total + a.tiles_per_split - 1) / a.tiles_per_split;
+    a.r_pad = 32;
+    a.n_groups = 1;
+    if (a.n_split > 1) {
+        const size_t rows = (size_t)n_pairs * a.n_split * a.r_pad;
+        float* ws = workspace(rows * (D + 2));
+        if (!ws) return VLA_K_ERR_LAUNCH;
+        a.part_o = ws;
+        a.part_ml = ws + rows * D;
+    }
+    const unsigned grid = (unsigned)(((long)n_pairs * a.n_split + 3) / 4);
+    if (a.p2) attn_direct_kernel<D, true, ST><<<grid, 256, 0, st>>>(a);
+    else attn_direct_kernel<D, false, ST><<<grid, 256, 0, st>>>(a);
+    if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
+    if (a.n_split > 1) {
+        const int R = (a.Hq / a.Hkv) * a.S;
+        const long total = (long)n_pairs * R * D;
+        attn_merge_kernel<bf16_t><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a.part_o, a.part_ml, (bf16_t*)a.out, n_pairs,
+                                                                                   a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
+        if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
+    }
+    return VLA_K_OK;
+}
+
 template <typename T, int D>
 int launch_d(AttnArgs& a, vla_stream_t stream) {
     constexpr int NW_MAX = 4;  // at most one wavefront of a workgroup per SIMD
     const int R = (a.Hq / a.Hkv) * a.S;
+    if constexpr (sizeof(T) == 2 && D <= 128) {
+        static const bool no_direct = getenv("VLA_ATTN_NO_DIRECT") != nullptr;
+        if (R <= 32 && !no_direct) return launch_direct<D>(a, (hipStream_t)stream);
+    }
     const int n_tiles = (R + 31) / 32;
     // One wavefront per row tile; more than NW_MAX tiles are spread evenly over groups.
     a.n_groups = (n_tiles + NW_MAX - 1) / NW_MAX;
@@ -453,11 +780,11 @@ int launch_d(AttnArgs& a, vla_stream_t stream) {
     a.r_pad = a.n_groups * nw * 32;
     // Too few workgroups to cover the 256 compute units: split the keys as well.
     const long wgs = (long)a.batch * a.Hkv * a.n_groups;
-    const int key_tiles = (a.n_keys + TK - 1) / TK;
+    const int key_tiles = (a.n_keys + SPLIT_KEYS - 1) / SPLIT_KEYS;
     a.n_split = 1;
     // Only worthwhile while a partial (r_pad rows of D+2 floats) stays small next to the
     // K/V slice it summarises; with many query rows the partials would outweigh the cache.
-    const size_t partial_bytes = (size_t)a.r_pad * (D + 2) * 4, tile_bytes = (size_t)2 * TK * D * sizeof(T);
+    const size_t partial_bytes = (size_t)a.r_pad * (D + 2) * 4, tile_bytes = (size_t)2 * SPLIT_KEYS * D * sizeof(T);
     if (wgs < 256 && key_tiles > 1 && partial_bytes <= tile_bytes) {
         int want = (int)((512 + wgs - 1) / wgs);
         if (want > key_tiles) want = key_tiles;
@@ -516,7 +843,8 @@ extern "C" int vla_attn_prefix_suffix(const void* q, const void* k_cache, const 
     a.scale = scale; a.mask_kind = mask_kind;
     a.n_prefix = n_prefix < 0 ? 0 : (n_prefix > n_keys ? n_keys : n_prefix);
     a.pad_start = pad_start; a.pad_end = pad_end; a.mask = mask;
-    if (dtype == VLA_DT_BF16) return launch_t<bf16_t>(a, head_dim, stream);
+    a.p2 = dtype == VLA_DT_BF16_P2;
+    if (dtype == VLA_DT_BF16 || dtype == VLA_DT_BF16_P2) return launch_t<bf16_t>(a, head_dim, stream);
     if (dtype == VLA_DT_F32) return launch_t<float>(a, head_dim, stream);
     return VLA_K_ERR_ARG;
 }

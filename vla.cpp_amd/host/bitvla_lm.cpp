@@ -214,7 +214,7 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
                                rowsum_.as<int32_t>(), w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_, C.stream));
         VLA_K(vla_qkv_split_rope_append(qkv_.get(), cos_t, sin_t, q_.get(), w.kv.k.get(), w.kv.vt.get(), VLA_DT_BF16, M, S,
                                         Hq_, Hkv_, D_, w.kv.t_max, tok_offset, C.stream));
-        VLA_K(vla_attn_prefix_suffix(q_.get(), w.kv.k.get(), w.kv.vt.get(), att_.get(), VLA_DT_BF16, M / S, S, Hq_, Hkv_,
+        VLA_K(vla_attn_prefix_suffix(q_.get(), w.kv.k.get(), w.kv.vt.get(), att_.get(), VLA_DT_BF16_P2, M / S, S, Hq_, Hkv_,
                                      D_, w.kv.t_max, n_keys, scale, VLA_MASK_NONE, n_keys, 0, 0, nullptr, C.stream));
         VLA_K(bitvla_rmsnorm_bf16(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), hn_.as<uint16_t>(), eps_, M, H_, C.stream));
         VLA_K(vla_act_quant_bf16(hn_.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(), rowsum_.as<int32_t>(), M, H_, C.stream));
