@@ -303,11 +303,12 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
 // Workgroup tile (64*TM) x (64*TN), 2 x 2 wavefronts; wavefront (wm, wn) owns the 32x32
 // MFMA blocks in block rows wm + 2i (i < TM) and block columns wn + 2j (j < TN), so every
 // 64x64 sub-tile is made of one block from each wavefront.  KB = bytes of K per staged row.
-template <typename T, int kEpi, int TM, int TN, int KB>
+template <typename T, int kEpi, int TM, int TN, int KB, int DEPTH>
 __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     typedef Traits<T> TR;
     constexpr int EB = TR::kElemBytes;
     constexpr int BK = KB / EB;        // k elements per tile
+    constexpr int EPV = 16 / EB;       // elements per 16-byte vector
     constexpr int STRIDE = KB + 16;    // padded LDS row
     constexpr int ROWS_A = 64 * TM, ROWS_W = 64 * TN;
     constexpr int VPR = KB / 16;       // 16-byte vectors per staged row
@@ -344,62 +345,85 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
 
     const int nkt = (a.K + BK - 1) / BK;
 
-    // Global -> register staging of the next k-tile while the current one is multiplied.
-    u32x4_t ra[VA], rw[VW];
-    auto load_tile = [&](int kt) {
+    // Operand staging: global -> registers -> LDS, with DEPTH k-tiles of loads in flight
+    // (a ring of register stages with compile-time indices).  The loads are unconditional:
+    // rows past M or N and k past K are redirected to valid addresses (their products land
+    // in outputs that are dropped, or are zeroed when the one partial k-tile is stored), and
+    // the ring keeps re-reading the last tile once the real ones are exhausted, so the loop
+    // body has no load under a branch and the wait counts stay exact.
+    const unsigned char* ap[VA];
+    int a_koff[VA];
+#pragma unroll
+    for (int v = 0; v < VA; ++v) {
+        const int idx = tid + v * 256;
+        const int m = min(m0 + idx / VPR, a.M - 1);
+        a_koff[v] = (idx % VPR) * EPV;
+        ap[v] = (const unsigned char*)a.A + (long)m * a.K * EB;
+    }
+    const unsigned char* wp[VW];
+    if (kEpi != EPI_TERNARY) {
+#pragma unroll
+        for (int v = 0; v < VW; ++v) {
+            const int idx = tid + v * 256;
+            constexpr int RPV = 256 / VPR;                     // rows covered by one vector index step
+            const int sub = (v * RPV) / 64, wr = (idx / VPR) & 63;  // sub is compile-time per unrolled v
+            int n = (wr < 32) ? tc[sub].base0 + wr : tc[sub].base1 + wr - 32;
+            n = min(max(n, 0), a.N - 1);
+            wp[v] = (const unsigned char*)a.W + (long)n * a.K * EB;
+        }
+    } else {
+        // 64 rows x 128 k of 2-bit codes = 64 x 8 words; two words per thread: the two
+        // 16-k halves (g = 0, 1) of 32-k group q of the tile.
+        const int n = min(ntw * BN + (tid >> 2), a.N - 1);
+        wp[0] = (const unsigned char*)((const uint32_t*)a.W + tern_word_index(n, (tid & 3) * 2, a.K));
+    }
+    u32x4_t ra[DEPTH][VA], rw[DEPTH][VW];
+    auto load_tile = [&](int st, int kt) __attribute__((always_inline)) {
         const int k0 = kt * BK;
 #pragma unroll
         for (int v = 0; v < VA; ++v) {
-            const int idx = tid + v * 256;
-            const int row = idx / VPR, c = idx % VPR;
-            const int k = k0 + c * (16 / EB);
-            const int m = m0 + row;
-            u32x4_t z = {0u, 0u, 0u, 0u};
-            ra[v] = z;
-            if (m < a.M && k < a.K)
-                ra[v] = *reinterpret_cast<const u32x4_t*>((const unsigned char*)a.A + ((long)m * a.K + k) * EB);
+            const int k = min(k0 + a_koff[v], a.K - EPV);
+            ra[st][v] = *reinterpret_cast<const u32x4_t*>(ap[v] + (long)k * EB);
         }
         if (kEpi != EPI_TERNARY) {
 #pragma unroll
             for (int v = 0; v < VW; ++v) {
-                const int idx = tid + v * 256;
-                const int row = idx / VPR, c = idx % VPR;
-                const int k = k0 + c * (16 / EB);
-                constexpr int RPV = 256 / VPR;          // rows covered by one vector index step
-                const int sub = (v * RPV) / 64, wr = row & 63;  // compile-time per unrolled v
-                const int n = (wr < 32) ? tc[sub].base0 + wr : tc[sub].base1 + wr - 32;
-                const bool tile_ok = (ntw * TN + sub) < a.n_tiles;
-                u32x4_t z = {0u, 0u, 0u, 0u};
-                rw[v] = z;
-                if (tile_ok && n < a.N && k < a.K)
-                    rw[v] = *reinterpret_cast<const u32x4_t*>((const unsigned char*)a.W + ((long)n * a.K + k) * EB);
+                const int k = min(k0 + a_koff[v % VA], a.K - EPV);  // same column pattern as A (VPR | 256)
+                rw[st][v] = *reinterpret_cast<const u32x4_t*>(wp[v] + (long)k * EB);
             }
         } else {
-            // 64 rows x 128 k of 2-bit codes = 64 x 8 words; two words per thread.
-            const int row = tid >> 2, q = tid & 3;
-            const int n = ntw * BN + row;
-            const int kw = k0 / 16 + q * 2;
-            u32x4_t z = {0u, 0u, 0u, 0u};
-            rw[0] = z;
-            if (n < a.N && kw * 16 < a.K) {
-                // words kw, kw+1 = the two 16-k halves (g = 0, 1) of 32-k group kw/2
-                const uint32_t* wp = (const uint32_t*)a.W + tern_word_index(n, kw, a.K);
-                rw[0][0] = wp[0];
-                rw[0][1] = wp[32];
-            }
+            const uint32_t* w = (const uint32_t*)wp[0] + (long)(k0 / 32) * 64;
+            rw[st][0][0] = w[0];
+            rw[st][0][1] = w[32];
         }
     };
-    auto store_tile = [&]() {
+    auto mask_partial = [&](int st, int kt) __attribute__((always_inline)) {  // zero what lies past K
+#pragma unroll
+        for (int v = 0; v < VA; ++v)
+            if (kt * BK + a_koff[v] >= a.K) {
+                const u32x4_t z = {0u, 0u, 0u, 0u};
+                ra[st][v] = z;
+            }
+        if (kEpi != EPI_TERNARY) {
+#pragma unroll
+            for (int v = 0; v < VW; ++v)
+                if (kt * BK + a_koff[v % VA] >= a.K) {
+                    const u32x4_t z = {0u, 0u, 0u, 0u};
+                    rw[st][v] = z;
+                }
+        }
+    };
+    auto store_tile = [&](int st) __attribute__((always_inline)) {
 #pragma unroll
         for (int v = 0; v < VA; ++v) {
             const int idx = tid + v * 256;
-            *reinterpret_cast<u32x4_t*>(ldsA + (idx / VPR) * STRIDE + (idx % VPR) * 16) = ra[v];
+            *reinterpret_cast<u32x4_t*>(ldsA + (idx / VPR) * STRIDE + (idx % VPR) * 16) = ra[st][v];
         }
         if (kEpi != EPI_TERNARY) {
 #pragma unroll
             for (int v = 0; v < VW; ++v) {
                 const int idx = tid + v * 256;
-                *reinterpret_cast<u32x4_t*>(ldsW + (idx / VPR) * STRIDE + (idx % VPR) * 16) = rw[v];
+                *reinterpret_cast<u32x4_t*>(ldsW + (idx / VPR) * STRIDE + (idx % VPR) * 16) = rw[st][v];
             }
         } else {
             // Decode 2 words -> 32 codes (unsigned 0..3; the -2 offset is folded
@@ -408,7 +432,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
             const int row = tid >> 2, q = tid & 3;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const uint32_t w = rw[0][h];
+                const uint32_t w = rw[st][0][h];
                 u32x4_t d;
                 d[0] = w & 0x03030303u;
                 d[1] = (w >> 2) & 0x03030303u;
@@ -418,12 +442,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
             }
         }
     };
-
-    load_tile(0);
-    for (int kt = 0; kt < nkt; ++kt) {
-        store_tile();
-        __syncthreads();
-        if (kt + 1 < nkt) load_tile(kt + 1);
+    auto multiply = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int ch = 0; ch < KB / TR::kChunkBytes; ++ch) {
             const int off = ch * TR::kChunkBytes + g * 16;
@@ -437,7 +456,36 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[i], fw[j]);
         }
-        __syncthreads();
+    };
+
+    // Stage st of the ring holds tile kt with kt % DEPTH == st.  Main loop: whole groups
+    // of DEPTH full tiles, no branch in the body.  The remaining tiles (fewer than DEPTH
+    // full ones and at most one partial) are already in flight when the main loop ends
+    // and are drained without further loads.
+#pragma unroll
+    for (int st = 0; st < DEPTH; ++st) load_tile(st, min(st, nkt - 1));
+    const int n_main = (a.K / BK) / DEPTH;
+    for (int gi = 0; gi < n_main; ++gi) {
+#pragma unroll
+        for (int st = 0; st < DEPTH; ++st) {
+            store_tile(st);
+            __syncthreads();
+            load_tile(st, min(gi * DEPTH + st + DEPTH, nkt - 1));
+            __builtin_amdgcn_sched_barrier(0);  // the loads stay above the multiply they hide behind
+            multiply();
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int st = 0; st < DEPTH; ++st) {
+        const int kt = n_main * DEPTH + st;
+        if (kt < nkt) {  // uniform
+            if (kt * BK + BK > a.K) mask_partial(st, kt);
+            store_tile(st);
+            __syncthreads();
+            multiply();
+            __syncthreads();
+        }
     }
 
     // Epilogue, one 64x64 sub-tile at a time through an LDS copy of the accumulators.
@@ -668,21 +716,34 @@ __global__ void __launch_bounds__(WM * 128, 2) ternary_gemm_big_kernel(GemmArgs 
     }
 }
 
+template <typename T, int kEpi, int TM, int TN, int KB, int DEPTH>
+void launch_cfg(const GemmArgs& a, hipStream_t st) {
+    const unsigned grid = (unsigned)(((((a.n_tiles + TN - 1) / TN) + 7) & ~7) * ((a.M + 64 * TM - 1) / (64 * TM)));
+    gemm_kernel<T, kEpi, TM, TN, KB, DEPTH><<<grid, 256, 0, st>>>(a);
+}
+
 template <typename T, int kEpi>
 int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
     if (a.M == 0 || n_tiles == 0) return VLA_K_OK;
     a.n_tiles = n_tiles;
     hipStream_t st = (hipStream_t)stream;
-    // Enough 128x128 tiles to occupy the chip: use them (half the LDS and L2 traffic per
-    // multiply); otherwise 64x64 tiles with 256-byte K rows (half the barriers per K).
-    const long big_tiles = (long)((a.M + 127) / 128) * ((n_tiles + 1) / 2);
     if constexpr (kEpi != EPI_TERNARY) {
-        if (big_tiles >= 128) {
-            const unsigned grid = (unsigned)(((((n_tiles + 1) / 2) + 7) & ~7) * ((a.M + 127) / 128));
-            gemm_kernel<T, kEpi, 2, 2, 128><<<grid, 256, 0, st>>>(a);
-        } else {
-            const unsigned grid = (unsigned)(((n_tiles + 7) & ~7) * ((a.M + 63) / 64));
-            gemm_kernel<T, kEpi, 1, 1, 256><<<grid, 256, 0, st>>>(a);
+        // VLA_GEMM_TILE = 0..4 pins the tile configuration (tuning); unset = by shape.
+        const char* env = getenv("VLA_GEMM_TILE");
+        int cfg = env ? atoi(env) : -1;
+        if (cfg < 0) {
+            // Enough 128x128 tiles to occupy the chip: use them (half the LDS and L2 traffic
+            // per multiply); else 128x64 tiles if those fill it; else 64x64 tiles with
+            // 256-byte K rows (half the barriers per K).
+            const long m128 = (a.M + 127) / 128;
+            cfg = m128 * ((n_tiles + 1) / 2) >= 128 ? 0 : (m128 * n_tiles >= 150 ? 2 : 1);
+        }
+        switch (cfg) {
+            case 0: launch_cfg<T, kEpi, 2, 2, 128, 3>(a, st); break;
+            case 1: launch_cfg<T, kEpi, 1, 1, 256, 4>(a, st); break;
+            case 2: launch_cfg<T, kEpi, 2, 1, 128, 4>(a, st); break;
+            case 3: launch_cfg<T, kEpi, 1, 2, 128, 4>(a, st); break;
+            default: launch_cfg<T, kEpi, 1, 1, 128, 6>(a, st); break;
         }
     } else {
         // VLA_TERNARY_TILE = 64 | 128 | 256 pins the tile (tests and tuning); unset = by shape.
@@ -699,8 +760,7 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             const unsigned grid = (unsigned)(((((a.M + 127) / 128) + 7) & ~7) * n256);
             ternary_gemm_big_kernel<2><<<grid, 256, 0, st>>>(a);
         } else {
-            const unsigned grid = (unsigned)(((n_tiles + 7) & ~7) * ((a.M + 63) / 64));
-            gemm_kernel<T, EPI_TERNARY, 1, 1, 128><<<grid, 256, 0, st>>>(a);
+            launch_cfg<T, EPI_TERNARY, 1, 1, 128, 4>(a, st);
         }
     }
     return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
