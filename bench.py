@@ -218,7 +218,20 @@ def kernel_breakdown(pkg, cfg, B, P):
     return out
 
 
-def roofline_of(name, k):
+# HBM-side bytes per launch (L2 misses) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# on this command, KiB per dispatch, each scaled by what the same counter reads for a plain
+# 256 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the per-kernel tables and
+# the commands are in profiles/*_pmc.txt.  Kernels without a measurement report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("cfg1_smolvla_16layer_bf16_b32", "wo_residual"): int((7769.0 * 2 + 2250.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "attention_self"): int((7690.8 * 2 + 3000.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "attention_cross"): int((6547.5 * 2 + 3000.0) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "attention_cross"): int((69292.2 * 2 + 3282.5) * 1024),
+    ("cfg4_bitvla_30layer_b8", "ternary_qkv_gemm_prefill"): int((14920.0 * 2 + 30720.0) * 1024),
+}
+
+
+def roofline_of(name, k, workload=None):
     if k["bound"] == "hbm":
         achieved = k["work"] / (k["us"] * 1e-6) / 1e9
         peak, unit = HBM_PEAK_GBS, "GB/s"
@@ -226,7 +239,8 @@ def roofline_of(name, k):
         achieved = k["work"] / (k["us"] * 1e-6) / 1e12
         peak, unit = PEAK_TFLOPS[k["peak_key"]], "TFLOP/s"
     return dict(kernel=name, bound=k["bound"], achieved=round(achieved, 3), peak=peak, unit=unit,
-                frac=round(achieved / peak, 5), traffic=None, avg_us=round(k["us"], 3),
+                frac=round(achieved / peak, 5), traffic=MEASURED_TRAFFIC_BYTES.get((workload, name)),
+                avg_us=round(k["us"], 3),
                 algorithmic_work_per_launch=k["work"])
 
 
@@ -308,11 +322,11 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir):
         us_per_action_chunk=round(ms_per_step * 1e3 * steps_per_chunk, 1), steps_per_chunk=steps_per_chunk,
         device_us_per_step=round(dev_ms * 1e3 / steps, 2), prefix_kv_build_ms=round(prefill_ms, 2),
         sum_kernel_us_per_step=round(sum(v["us"] * v["per_step"] for v in step_kern.values()), 2),
-        roofline=roofline_of(dominant, kern[dominant]), roofline_kv=roofline_of(kv_name, kern[kv_name]),
+        roofline=roofline_of(dominant, kern[dominant], name), roofline_kv=roofline_of(kv_name, kern[kv_name], name),
         kernels={k: dict(us=round(v["us"], 2), per_step=v["per_step"]) for k, v in kern.items()},
     )
     if "ternary_qkv_gemm_prefill" in kern:
-        res["roofline_ternary_prefill"] = roofline_of("ternary_qkv_gemm_prefill", kern["ternary_qkv_gemm_prefill"])
+        res["roofline_ternary_prefill"] = roofline_of("ternary_qkv_gemm_prefill", kern["ternary_qkv_gemm_prefill"], name)
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(cfg, w, obs[0], B)
     m.close()
@@ -330,6 +344,8 @@ def main():
     ap.add_argument("--others", default="cfg3_gr00t_16dit_bf16_b64,cfg4_bitvla_30layer_b8",
                     help="comma-separated extra workloads reported under other_configs")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="only run plain device copies of a known size (reference for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (the path shards over observations with no collectives); "
@@ -339,6 +355,15 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
+    if args.traffic_calibration:
+        n = 64 << 20  # fp32 elements: each copy reads 256 MiB and writes 256 MiB
+        src = torch.ones(n, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "device copy", "copies": 5, "bytes_read_per_copy": 4 * n, "bytes_written_per_copy": 4 * n}))
+        return
     import __graft_entry__ as entry
     entry.load_package().lib()
     wl = workloads()

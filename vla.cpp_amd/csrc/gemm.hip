@@ -41,7 +41,7 @@ struct GemmArgs {
     const void* A;
     const void* W;
     const float* bias;
-    int M, N, K, n_tiles;
+    int M, N, K, n_tiles, xm, xn;
     // PLAIN
     const void* residual;
     void* Y;
@@ -323,14 +323,17 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     const int g = lane >> 5, r = lane & 31;
-    // Linear workgroup id -> (M tile, N tile) with the N tiles padded to a multiple of
-    // 8: id % 8 (the XCD a workgroup is dispatched to) then equals nt % 8, so each XCD's
-    // L2 holds one eighth of W plus the A rows instead of the whole of both.
-    const int n_wg_tiles = (a.n_tiles + TN - 1) / TN;
-    const int nt_pad = (n_wg_tiles + 7) & ~7;
-    const int ntw = blockIdx.x % nt_pad;
-    if (ntw >= n_wg_tiles) return;
-    const int m0 = (blockIdx.x / nt_pad) * ROWS_A;
+    // Linear workgroup id -> (M tile, N tile).  id % 8 is the XCD a workgroup is dispatched
+    // to; the 8 XCDs form an xm x xn grid and XCD (i, j) owns the M tiles = i (mod xm) and
+    // the N tiles = j (mod xn), so each L2 fetches 1/xm of A and 1/xn of W instead of the
+    // whole of either (the host picks the split that minimises the total).
+    const int n_wg_tiles = (a.n_tiles + TN - 1) / TN, m_wg_tiles = (a.M + ROWS_A - 1) / ROWS_A;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int cn = (n_wg_tiles + a.xn - 1) / a.xn;  // N tiles per XCD column (padded)
+    const int ntw = (local % cn) * a.xn + xcd % a.xn;
+    const int mtw = (local / cn) * a.xm + xcd / a.xn;
+    if (ntw >= n_wg_tiles || mtw >= m_wg_tiles) return;
+    const int m0 = mtw * ROWS_A;
     TileCols tc[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) tc[j] = tile_cols<kEpi>(a, ntw * TN + j);
@@ -717,8 +720,23 @@ __global__ void __launch_bounds__(WM * 128, 2) ternary_gemm_big_kernel(GemmArgs 
 }
 
 template <typename T, int kEpi, int TM, int TN, int KB, int DEPTH>
-void launch_cfg(const GemmArgs& a, hipStream_t st) {
-    const unsigned grid = (unsigned)(((((a.n_tiles + TN - 1) / TN) + 7) & ~7) * ((a.M + 64 * TM - 1) / (64 * TM)));
+void launch_cfg(GemmArgs a, hipStream_t st) {
+    const int n_wg = (a.n_tiles + TN - 1) / TN, m_wg = (a.M + 64 * TM - 1) / (64 * TM);
+    // XCD grid xm x xn = 8: every L2 reads its M tiles' rows of A and its N tiles' rows of
+    // W once; pick the split with the least total, counting the padding of the tile grid.
+    const double bytes_a = (double)a.M * a.K, bytes_w = (double)a.N * a.K * (kEpi == EPI_TERNARY ? 0.25 : 1.0);
+    double best = -1;
+    for (int xm = 1; xm <= 8; xm *= 2) {
+        const int xn = 8 / xm;
+        const long wgs = (long)((m_wg + xm - 1) / xm) * ((n_wg + xn - 1) / xn) * 8;
+        const double cost = (bytes_a * xn + bytes_w * xm) * (double)wgs / ((double)m_wg * n_wg);
+        if (best < 0 || cost < best) {
+            best = cost;
+            a.xm = xm;
+            a.xn = xn;
+        }
+    }
+    const unsigned grid = (unsigned)(((m_wg + a.xm - 1) / a.xm) * ((n_wg + a.xn - 1) / a.xn) * 8);
     gemm_kernel<T, kEpi, TM, TN, KB, DEPTH><<<grid, 256, 0, st>>>(a);
 }
 
