@@ -176,6 +176,13 @@ VLA_KAPI int vla_euler_step(float* x_t, const void* hn, const float* W_out, cons
 VLA_KAPI int vla_act_quant_bf16(const uint16_t* in, int8_t* out, float* scales, int32_t* rowsum, int M, int K,
                                 vla_stream_t stream);
 
+/* bitvla_rmsnorm_bf16 followed by vla_act_quant_bf16 in one launch (the pair that opens
+ * both halves of run_layer, src/kernels/bitvla/bitvla_lm_cuda.cu:422-486); the bf16
+ * intermediate is not written.  int8 rows, scales and row sums are bit-identical to the
+ * two separate calls.  K <= 4096. */
+VLA_KAPI int vla_rmsnorm_act_quant_bf16(const uint16_t* x, const uint16_t* w, int8_t* out, float* scales,
+                                        int32_t* rowsum, float eps, int M, int K, vla_stream_t stream);
+
 /* Ternary weight quantisation on the host (recover_ternary_and_scale,
  * src/models/bitvla.cpp:430-451). */
 VLA_KAPI int vla_ternary_quant_host(const float* W, int64_t n, int8_t* ternary, float* absmean);
@@ -199,6 +206,13 @@ VLA_KAPI int vla_ternary_repack_ladder_host(const uint8_t* ladder, int N, int K,
 VLA_KAPI int vla_ternary_gemm(const int8_t* A, const uint32_t* W_packed, uint16_t* out, int32_t* acc_out,
                               const float* s, const int32_t* rowsum, const float* ws, int ws_num, int M, int N,
                               int K, vla_stream_t stream);
+
+/* vla_ternary_gemm followed by bitvla_add_bf16 in one launch:
+ * out[m][n] = bf16(bf16(float(acc) / s[m] * ws[g]) + residual[m][n]); out may alias residual
+ * (the O projection + residual of run_layer, bitvla_lm_cuda.cu:480-486).  residual may be NULL. */
+VLA_KAPI int vla_ternary_gemm_add(const int8_t* A, const uint32_t* W_packed, uint16_t* out, const uint16_t* residual,
+                                  const float* s, const int32_t* rowsum, const float* ws, int ws_num, int M, int N,
+                                  int K, vla_stream_t stream);
 
 /* -------------------------------------- BitVLA layer helpers (same signatures
  * as src/kernels/bitvla/bitvla_lm_cuda.h:54-155 with hipStream_t / uint16_t) */

@@ -6,6 +6,7 @@ act-quant, ternary int32 accumulators and their bf16 epilogue); fp32 kernels
 within 1e-5 relative (max-abs error over max-abs value); bf16 kernels within
 2e-2 relative / 1e-2 absolute.
 """
+import ctypes
 import math
 
 import numpy as np
@@ -282,7 +283,7 @@ def test_attention_against_oracle(dtype, case):
     assert np.array_equal(host(out), host(out_m))
 
 
-@pytest.mark.parametrize("split", [1, 2, 5, 64])
+@pytest.mark.parametrize("split", [1, 2, 5, 8, 64])
 def test_attention_direct_kernel_key_slices_merge(monkeypatch, split):
     # Few query rows: any slicing of the keys across wavefronts (merged by the second
     # kernel) gives the same result as the oracle.
@@ -453,6 +454,75 @@ def test_ternary_gemm_prefill_shape_all_tilings_agree(monkeypatch):
     want_acc = orc.ternary_gemm_i32(A[rows], t)
     assert np.array_equal(host(res[0][0])[rows], want_acc)
     assert np.array_equal(host(res[0][1], np.uint16)[rows], orc.ternary_epilogue(want_acc, s[rows], ws))
+
+
+@pytest.mark.parametrize("M", [1, 8, 32])
+def test_ternary_gemv_decode_rows_bit_exact(M):
+    # At most 32 rows (single-token decode): the split-K GEMV kernel gives the oracle's
+    # accumulators and epilogue, and, with a residual, the bits of GEMM followed by add.
+    N, K, ws_num = 3840, 2560, 6
+    r = np.random.default_rng(900 + M)
+    A = r.integers(-127, 128, (M, K)).astype(np.int8)
+    t = r.integers(-1, 2, (N, K)).astype(np.int8)
+    s = (127.0 / np.abs(r.standard_normal(M) * 3 + 1e-3)).astype(np.float32)
+    ws = (0.01 + 0.001 * r.integers(0, 50, ws_num)).astype(np.float32)
+    res = orc.to_bf16(r.standard_normal((M, N)).astype(np.float32))
+    dA, dW, ds, dws = dev(A), dev(_pack_plain(t)), dev(s), dev(ws)
+    rowsum = dev(A.astype(np.int32).sum(1).astype(np.int32))
+    acc = torch.zeros((M, N), dtype=torch.int32, device="cuda")
+    out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+    pkg.call("vla_ternary_gemm", dA, dW, out, acc, ds, rowsum, dws, ws_num, M, N, K)
+    h = dev(res)
+    pkg.call("vla_ternary_gemm_add", dA, dW, h, h, ds, rowsum, dws, ws_num, M, N, K)  # in place, as the engine calls it
+    want_sum = torch.zeros_like(out)
+    pkg.call("bitvla_add_bf16", out, dev(res), want_sum, M * N)
+    sync()
+    want_acc = orc.ternary_gemm_i32(A, t)
+    assert np.array_equal(host(acc), want_acc)
+    assert np.array_equal(host(out, np.uint16), orc.ternary_epilogue(want_acc, s, ws))
+    assert np.array_equal(host(h), host(want_sum))
+
+
+@pytest.mark.parametrize("M,N,K,tile", [(300, 288, 256, 64), (300, 288, 256, 128), (515, 640, 384, 256)])
+def test_ternary_gemm_add_matches_gemm_then_add(monkeypatch, M, N, K, tile):
+    r = np.random.default_rng(M + tile)
+    A = r.integers(-127, 128, (M, K)).astype(np.int8)
+    t = r.integers(-1, 2, (N, K)).astype(np.int8)
+    s = (40.0 + r.integers(0, 100, M)).astype(np.float32)
+    ws = np.float32([0.02])
+    res = orc.to_bf16(r.standard_normal((M, N)).astype(np.float32))
+    dA, dW, ds, dws = dev(A), dev(_pack_plain(t)), dev(s), dev(ws)
+    rowsum = dev(A.astype(np.int32).sum(1).astype(np.int32))
+    monkeypatch.setenv("VLA_TERNARY_TILE", str(tile))
+    out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+    pkg.call("vla_ternary_gemm", dA, dW, out, None, ds, rowsum, dws, 1, M, N, K)
+    fused = torch.zeros_like(out)
+    pkg.call("vla_ternary_gemm_add", dA, dW, fused, dev(res), ds, rowsum, dws, 1, M, N, K)
+    want = torch.zeros_like(out)
+    pkg.call("bitvla_add_bf16", out, dev(res), want, M * N)
+    sync()
+    assert np.array_equal(host(fused), host(want))
+
+
+@pytest.mark.parametrize("M,K", [(8, 2560), (37, 720), (4, 4096)])
+def test_rmsnorm_act_quant_fused_is_the_pair(M, K):
+    r = np.random.default_rng(K + M)
+    x = orc.to_bf16((r.standard_normal((M, K)) * 3).astype(np.float32))
+    w = orc.to_bf16((1 + 0.1 * r.standard_normal(K)).astype(np.float32))
+    hn = torch.zeros((M, K), dtype=torch.int16, device="cuda")
+    q1, s1, r1 = (torch.zeros((M, K), dtype=torch.int8, device="cuda"), torch.zeros(M, device="cuda"),
+                  torch.zeros(M, dtype=torch.int32, device="cuda"))
+    q2, s2, r2 = torch.zeros_like(q1), torch.zeros_like(s1), torch.zeros_like(r1)
+    pkg.call("bitvla_rmsnorm_bf16", dev(x), dev(w), hn, 1e-5, M, K)
+    pkg.call("vla_act_quant_bf16", hn, q1, s1, r1, M, K)
+    pkg.call("vla_rmsnorm_act_quant_bf16", dev(x), dev(w), q2, s2, r2, 1e-5, M, K)
+    sync()
+    assert torch.equal(q1, q2) and torch.equal(s1, s2) and torch.equal(r1, r2)
+    # and the pair follows the oracle
+    n = orc.round_bf16(orc.rms_norm(orc.from_bf16(x), orc.from_bf16(w), 1e-5))
+    qo, so = orc.act_quant(n)
+    assert np.mean(host(q2) != qo) < 2e-3 and np.allclose(host(s2), so, rtol=1e-2)
+    assert pkg.lib().vla_rmsnorm_act_quant_bf16(0, 0, 0, 0, 0, ctypes.c_float(1e-5), 1, 8, 0) == pkg.VLA_K_ERR_ARG
 
 
 def test_ternary_pipeline_matches_cpu_twin():

@@ -22,11 +22,13 @@
 // MFMA formulation (transposed, so softmax statistics are per lane):
 //   S^T[key][row] = K . Q^T     A = K tile rows (lane r <-> key), B = Q rows
 //   O^T[d][row]  += V^T . P^T   A = V^T rows (lane r <-> d),      B = P^T
-// The 32x32 accumulator gives lane (g, r) the 16 keys 8j+4g+i of query row r,
+// The 32x32 accumulator gives lane (g, r) the 16 score rows 8j+4g+i of query row r,
 // so row max / sum are 15 in-lane ops plus one exchange with lane r+32, and the
-// probabilities are already in B-operand position for the second product: the
-// k-slot (g, e) of that product is bound to key 8(e/4)+4g+(e%4), and V^T is
-// fetched from LDS in the same order.  No score matrix is ever written
+// probabilities are already in B-operand position for the second product.  Which key
+// sits in score row x is free (it is just the K row a lane fetches): row 8j+4g+i holds
+// key 16(j/2) + 8g + 4(j%2) + i of the 32-key block, so that the 8 probabilities a lane
+// feeds to one output MFMA belong to 8 consecutive keys and its V^T fragment is a single
+// 16-byte run.  No score matrix is ever written
 // (the reference's explicit path writes and re-reads Hq*S*T scores).
 //
 // Few query rows (single-token decode, batch 1): the keys are split across
@@ -61,6 +63,13 @@ struct AttnArgs {
     float* part_o;   // [pair][split][r_pad][D]
     float* part_ml;  // [pair][split][r_pad][2]
 };
+
+// Key (within a 32-key block) held by score row x = 8j + 4h + i: 16(j/2) + 8h + 4(j%2) + i.
+__device__ __forceinline__ int key_of_score_row(int x) {
+    return 16 * (x >> 4) + 8 * ((x >> 2) & 1) + 4 * ((x >> 3) & 1) + (x & 3);
+}
+// Key of accumulator element e (= 4j + i) of a lane in half g.
+__device__ __forceinline__ int key_of_element(int e, int g) { return 16 * (e >> 3) + 8 * g + 4 * ((e >> 2) & 1) + (e & 3); }
 
 template <typename T> struct AT;
 template <> struct AT<bf16_t> {
@@ -245,7 +254,8 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
             for (int i = 0; i < 16; ++i) sc[i] = 0.f;
 #pragma unroll
             for (int c = 0; c < NQ; ++c) {
-                const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(ldsK + (kb * 32 + r) * KS + (c * CE + g * (CE / 2)) * EB);
+                const u32x4_t kf =
+                    *reinterpret_cast<const u32x4_t*>(ldsK + (kb * 32 + key_of_score_row(r)) * KS + (c * CE + g * (CE / 2)) * EB);
                 A::mma(sc, kf, qf[c]);
             }
 #pragma unroll
@@ -257,16 +267,16 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
                 for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        const int key = k0 + kb * 32 + 8 * (e >> 2) + 4 * g + (e & 3);
+                        const int key = k0 + kb * 32 + key_of_element(e, g);
                         p[kb][e] = key < a.n_keys ? p[kb][e] + a.mask[(long)s * a.n_keys + key] * LOG2E : -INFINITY;
                     }
             } else {
-                const int kl = k0 + 4 * g;
+                const int kl = k0 + 8 * g;
 #pragma unroll
                 for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
                     for (int e = 0; e < 16; ++e) {
-                        const int key = kl + kb * 32 + 8 * (e >> 2) + (e & 3);
+                        const int key = kl + kb * 32 + key_of_element(e, 0);
                         const bool visible = (key < hi) & !((key >= pad_lo) & (key < pad_hi));
                         p[kb][e] = visible ? p[kb][e] : -INFINITY;
                     }
@@ -325,13 +335,10 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
                         if (P2)
                             pl[e] = pack_bf2(pp[2 * e] - __uint_as_float(hi16 << 16), pp[2 * e + 1] - __uint_as_float(hi16 & 0xffff0000u));
                     }
-                    const int key_off = (kb * 32 + hh * 16 + 4 * g) * EB;
+                    const int key_off = (kb * 32 + hh * 16 + 8 * g) * EB;
 #pragma unroll
                     for (int db = 0; db < NDB; ++db) {
-                        const unsigned char* vr = ldsV + (db * 32 + r) * VS + key_off;
-                        const u32x2_t v0 = *reinterpret_cast<const u32x2_t*>(vr);
-                        const u32x2_t v1 = *reinterpret_cast<const u32x2_t*>(vr + 8 * EB);
-                        const u32x4_t vf = {v0[0], v0[1], v1[0], v1[1]};
+                        const u32x4_t vf = *reinterpret_cast<const u32x4_t*>(ldsV + (db * 32 + r) * VS + key_off);
                         A::mma(o[db], vf, pf);
                         if (P2) A::mma(o[db], vf, pl);
                     }
@@ -342,7 +349,7 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
                     const float* pp = &p[kb][4 * j];
                     const u32x4_t pf = {__float_as_uint(pp[0]), __float_as_uint(pp[1]), __float_as_uint(pp[2]),
                                         __float_as_uint(pp[3])};
-                    const int key_off = (kb * 32 + 8 * j + 4 * g) * EB;
+                    const int key_off = (kb * 32 + key_of_element(4 * j, g)) * EB;
 #pragma unroll
                     for (int db = 0; db < NDB; ++db) {
                         const u32x4_t vf = *reinterpret_cast<const u32x4_t*>(ldsV + (db * 32 + r) * VS + key_off);
@@ -443,15 +450,18 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
 // wavefront reads 16 bytes of key row r for the score product and two 8-byte runs of V^T
 // row r for the output product, exactly the fragments the LDS kernel would fetch.  A
 // wavefront owns one (pair, key slice) and keeps ST 32-key blocks of loads in flight.
-template <int D, bool P2, int ST>
-__global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attn_direct_kernel(AttnArgs a) {
+// MERGE: a workgroup is one pair and its wavefronts are the key slices; they combine
+// their partial (max, sum, output) through LDS, so sliced decode is one launch.
+template <int D, bool P2, int ST, bool MERGE>
+__global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 1) attn_direct_kernel(AttnArgs a) {
     constexpr int EB = 2, CE = 16;
     constexpr int NQ = D / CE, NDB = (D + 31) / 32;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 5, r = lane & 31;
-    const int unit = blockIdx.x * 4 + wave;
+    const int unit = MERGE ? blockIdx.x * a.n_split + wave : blockIdx.x * 4 + wave;
     const int pair = unit / a.n_split, split = unit % a.n_split;
-    if (pair >= a.batch * a.Hkv) return;  // whole wavefront; the kernel has no barriers
+    // whole wavefront (whole workgroup with MERGE); the main loop has no barriers
+    if (pair >= a.batch * a.Hkv) return;
     const int b = pair / a.Hkv, hk = pair % a.Hkv;
     const int grp = a.Hq / a.Hkv, R = grp * a.S;
     const bool row_valid = r < R;
@@ -483,47 +493,53 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attn_direct_kernel(AttnA
     const unsigned char* vbase = (const unsigned char*)a.vt_cache + ((long)b * a.Hkv + hk) * D * (long)a.t_max * EB;
 
     u32x4_t kr[ST][NQ];
-    u32x2_t vr[ST][NDB][2][2];  // [stage][32-row block of d][16-key half][8-byte run]
+    u32x4_t vr[ST][NDB][2];  // [stage][32-row block of d][16-key half]: 8 consecutive keys per lane
     // Rows of V^T past head_dim (D = 48: the upper half of the second 32-row block) are
     // read from row D-1 instead, so every lane loads valid memory; their outputs are dropped.
     const unsigned char* vrow[NDB];
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) vrow[db] = vbase + ((long)min(db * 32 + r, D - 1) * a.t_max + 4 * g) * EB;
+    for (int db = 0; db < NDB; ++db) vrow[db] = vbase + ((long)min(db * 32 + r, D - 1) * a.t_max + 8 * g) * EB;
+    const int krow = key_of_score_row(r);  // the key of the block this lane fetches for the score product
     auto load_full = [&](int st, int kb) __attribute__((always_inline)) {  // no checks at all
-        const unsigned char* kp = kbase + (long)(kb * 32 + r) * D * EB + g * 16;
+        const unsigned char* kp = kbase + (long)(kb * 32 + krow) * D * EB + g * 16;
 #pragma unroll
         for (int c = 0; c < NQ; ++c) kr[st][c] = *reinterpret_cast<const u32x4_t*>(kp + c * CE * EB);
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-                for (int q = 0; q < 2; ++q)
-                    vr[st][db][hh][q] = *reinterpret_cast<const u32x2_t*>(vrow[db] + (kb * 32 + hh * 16 + q * 8) * EB);
+            for (int hh = 0; hh < 2; ++hh) vr[st][db][hh] = *reinterpret_cast<const u32x4_t*>(vrow[db] + (kb * 32 + hh * 16) * EB);
     };
-    // A partial block: K rows past n_keys repeat the last key (their scores are masked);
-    // V^T elements past n_keys are zeroed so that stale cache contents (possibly NaN)
-    // cannot reach the accumulators.
+    // A partial block: K rows past n_keys repeat the last key (their scores are masked) and
+    // V^T runs past n_keys are not read.  mask_partial, called once the data is needed,
+    // zeroes the V^T elements past n_keys so that stale cache contents (possibly NaN)
+    // cannot reach the accumulators; keeping it apart from the loads keeps the wait for
+    // them out of the way of the loads issued next.
     auto load_partial = [&](int st, int kb) __attribute__((always_inline)) {
-        const int key = min(kb * 32 + r, a.n_keys - 1);
+        const int key = min(kb * 32 + krow, a.n_keys - 1);
         const unsigned char* kp = kbase + (long)key * D * EB + g * 16;
 #pragma unroll
         for (int c = 0; c < NQ; ++c) kr[st][c] = *reinterpret_cast<const u32x4_t*>(kp + c * CE * EB);
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh)
+            for (int hh = 0; hh < 2; ++hh) {
+                const int k8 = kb * 32 + hh * 16 + 8 * g;  // first of 8 consecutive keys
+                u32x4_t val = {0u, 0u, 0u, 0u};
+                // n_keys <= t_max and t_max is a multiple of 8: a group starting below n_keys is inside the row
+                if (k8 < a.n_keys) val = *reinterpret_cast<const u32x4_t*>(vrow[db] + (kb * 32 + hh * 16) * EB);
+                vr[st][db][hh] = val;
+            }
+    };
+    auto mask_partial = [&](int st, int kb) __attribute__((always_inline)) {
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const int k4 = kb * 32 + hh * 16 + q * 8 + 4 * g;  // first of 4 consecutive keys
-                    u32x2_t val = {0u, 0u};
-                    // n_keys <= t_max and t_max is a multiple of 8: a group starting below n_keys is inside the row
-                    if (k4 < a.n_keys) val = *reinterpret_cast<const u32x2_t*>(vrow[db] + (kb * 32 + hh * 16 + q * 8) * EB);
-                    const int nvalid = a.n_keys - k4;
-                    val[0] &= (nvalid > 0 ? 0xffffu : 0u) | (nvalid > 1 ? 0xffff0000u : 0u);
-                    val[1] &= (nvalid > 2 ? 0xffffu : 0u) | (nvalid > 3 ? 0xffff0000u : 0u);
-                    vr[st][db][hh][q] = val;
-                }
+        for (int hh = 0; hh < 2; ++hh) {
+            const int nvalid = a.n_keys - (kb * 32 + hh * 16 + 8 * g);  // real keys among this lane's 8, may be <= 0
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    vr[st][db][hh][e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+        }
     };
     // Per-row visibility of the generated masks, branch-free (see the LDS kernel).
     int hi = a.n_keys;
@@ -548,14 +564,14 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attn_direct_kernel(AttnA
             if (a.mask && live) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const int key = k0 + 8 * (e >> 2) + 4 * g + (e & 3);
+                    const int key = k0 + key_of_element(e, g);
                     p[e] = key < a.n_keys ? p[e] + a.mask[(long)s * a.n_keys + key] * LOG2E : -INFINITY;
                 }
             } else {
-                const int kl = k0 + 4 * g, hi_blk = live ? hi : 0;
+                const int kl = k0 + 8 * g, hi_blk = live ? hi : 0;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const int key = kl + 8 * (e >> 2) + (e & 3);
+                    const int key = kl + key_of_element(e, 0);
                     const bool visible = (key < hi_blk) & !((key >= pad_lo) & (key < pad_hi));
                     p[e] = visible ? p[e] : -INFINITY;
                 }
@@ -596,9 +612,8 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attn_direct_kernel(AttnA
             }
 #pragma unroll
             for (int db = 0; db < NDB; ++db) {
-                const u32x4_t vf = {vr[st][db][hh][0][0], vr[st][db][hh][0][1], vr[st][db][hh][1][0], vr[st][db][hh][1][1]};
-                AT<bf16_t>::mma(o[db], vf, pf);
-                if (P2) AT<bf16_t>::mma(o[db], vf, pl);
+                AT<bf16_t>::mma(o[db], vr[st][db][hh], pf);
+                if (P2) AT<bf16_t>::mma(o[db], vr[st][db][hh], pl);
             }
         }
     };
@@ -617,7 +632,10 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attn_direct_kernel(AttnA
 #pragma unroll
         for (int i = 0; i < ST - 1; ++i) load_full(i, min(kb0 + i, kbf - 1));
     }
-    if (has_partial) compute(ST - 1, kb1 - 1, true);
+    if (has_partial) {
+        mask_partial(ST - 1, kb1 - 1);
+        compute(ST - 1, kb1 - 1, true);
+    }
     if (n_full > 0) {
         const int groups = (n_full + ST - 1) / ST;
         for (int gi = 0; gi < groups; ++gi) {
@@ -631,6 +649,45 @@ __global__ void __launch_bounds__(256, D <= 64 ? 2 : 1) attn_direct_kernel(AttnA
         }
     }
 
+    if (MERGE) {
+        // LDS: [slice][row][D + 2] floats (unnormalised output, then max and sum), rows < R only
+        extern __shared__ float merge_buf[];
+        const int RS = D + 2;
+        if (row_valid) {
+            float* pr = merge_buf + ((long)split * R + r) * RS;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int d = db * 32 + 8 * j + 4 * g;
+                    if (d >= D) continue;
+                    const f32x4_t pk = {o[db][4 * j], o[db][4 * j + 1], o[db][4 * j + 2], o[db][4 * j + 3]};
+                    *reinterpret_cast<f32x4_t*>(pr + d) = pk;
+                }
+            if (g == 0) {
+                pr[D] = m_run;
+                pr[D + 1] = l_run;
+            }
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < R * D; i += blockDim.x) {
+            const int row = i / D, d = i % D;
+            float m = -INFINITY;
+            for (int sp = 0; sp < a.n_split; ++sp) m = fmaxf(m, merge_buf[((long)sp * R + row) * RS + D]);
+            float l = 0.f, acc = 0.f;
+            if (m > -INFINITY) {
+                for (int sp = 0; sp < a.n_split; ++sp) {
+                    const float* pr = merge_buf + ((long)sp * R + row) * RS;
+                    const float w = exp2f(pr[D] - m);
+                    l += pr[D + 1] * w;
+                    acc += pr[d] * w;
+                }
+            }
+            const int hh = hk * grp + row / a.S, ss = row % a.S;
+            ((bf16_t*)a.out)[(((long)b * a.S + ss) * a.Hq + hh) * D + d] = f2bf(l > 0.f ? acc / l : 0.f);
+        }
+        return;
+    }
     if (!row_valid) return;
     if (a.n_split > 1) {
         const long prow = ((long)pair * a.n_split + split) * a.r_pad + r;
@@ -732,6 +789,7 @@ template <int D>
 int launch_direct(AttnArgs& a, hipStream_t st) {
     constexpr int ST = D <= 64 ? 3 : 2;
     const int n_pairs = a.batch * a.Hkv;
+    const int R = (a.Hq / a.Hkv) * a.S;
     const int nb_total = (a.n_keys + 31) / 32;
     // Enough wavefronts to keep every CU's memory pipeline busy (8 per CU); a slice is
     // at least two 32-key blocks unless the whole sequence is shorter.
@@ -740,10 +798,24 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
     if (n_split > (nb_total + 1) / 2) n_split = (nb_total + 1) / 2;
     if (n_split < 1) n_split = 1;
     if (const char* e = getenv("VLA_ATTN_SPLIT")) n_split = atoi(e) > 0 ? (atoi(e) < nb_total ? atoi(e) : nb_total) : 1;
+    // Slices of one pair as the wavefronts of one workgroup (merged through LDS, one launch)
+    // when few enough; with fewer than 32 pairs more slices go through global partials and
+    // the merge kernel instead.
+    constexpr int MERGE_MAX = D <= 64 ? 8 : 4;  // wide heads need the registers of a 4-wavefront workgroup
+    const bool wg_merge = n_split > 1 && (n_split <= MERGE_MAX || n_pairs >= 32);
+    if (wg_merge && n_split > MERGE_MAX) n_split = MERGE_MAX;
     a.tiles_per_split = (nb_total + n_split - 1) / n_split;
     a.n_split = (nb_total + a.tiles_per_split - 1) / a.tiles_per_split;
     a.r_pad = 32;
     a.n_groups = 1;
+    if (wg_merge && a.n_split > 1) {
+        const size_t lds = (size_t)a.n_split * R * (D + 2) * sizeof(float);  // <= 8 * 32 * 130 * 4 = 133 KB; R is small in practice
+        if (lds <= 64 * 1024) {
+            if (a.p2) attn_direct_kernel<D, true, ST, true><<<n_pairs, a.n_split * 64, lds, st>>>(a);
+            else attn_direct_kernel<D, false, ST, true><<<n_pairs, a.n_split * 64, lds, st>>>(a);
+            return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+        }
+    }
     if (a.n_split > 1) {
         const size_t rows = (size_t)n_pairs * a.n_split * a.r_pad;
         float* ws = workspace(rows * (D + 2));
@@ -752,11 +824,10 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
         a.part_ml = ws + rows * D;
     }
     const unsigned grid = (unsigned)(((long)n_pairs * a.n_split + 3) / 4);
-    if (a.p2) attn_direct_kernel<D, true, ST><<<grid, 256, 0, st>>>(a);
-    else attn_direct_kernel<D, false, ST><<<grid, 256, 0, st>>>(a);
+    if (a.p2) attn_direct_kernel<D, true, ST, false><<<grid, 256, 0, st>>>(a);
+    else attn_direct_kernel<D, false, ST, false><<<grid, 256, 0, st>>>(a);
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     if (a.n_split > 1) {
-        const int R = (a.Hq / a.Hkv) * a.S;
         const long total = (long)n_pairs * R * D;
         attn_merge_kernel<bf16_t><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a.part_o, a.part_ml, (bf16_t*)a.out, n_pairs,
                                                                                    a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);

@@ -287,6 +287,62 @@ __global__ void act_quant_bf16_kernel(const bf16_t* __restrict__ in, int8_t* __r
     }
 }
 
+// RMSNorm (bf16 result) immediately quantised per row to int8: the pair
+// bitvla_rmsnorm_bf16 + act_quant in one pass, the row held in registers between the two.
+// Same thread <-> element assignment and the same reductions as the separate kernels, so
+// the int8 rows, scales and row sums are bit-identical to running them back to back.
+constexpr int RNAQ_MAX_PER_THREAD = 16;
+__global__ void rmsnorm_act_quant_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, int8_t* __restrict__ out,
+                                         float* __restrict__ scales, int32_t* __restrict__ rowsum, int K, float eps) {
+    __shared__ float red[16];
+    __shared__ int redi[16];
+    const bf16_t* xr = x + (long)blockIdx.x * K;
+    int8_t* qr = out + (long)blockIdx.x * K;
+    float v[RNAQ_MAX_PER_THREAD];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < RNAQ_MAX_PER_THREAD; ++i) {
+        const int k = threadIdx.x + i * blockDim.x;
+        v[i] = k < K ? bf2f(xr[k]) : 0.f;
+        ss += v[i] * v[i];
+    }
+    ss = block_sum(ss, red);
+    const float nscale = 1.0f / sqrtf(ss / (float)K + eps);
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < RNAQ_MAX_PER_THREAD; ++i) {
+        const int k = threadIdx.x + i * blockDim.x;
+        float n = v[i] * nscale;
+        if (w && k < K) n *= bf2f(w[k]);
+        v[i] = k < K ? bf2f(f2bf(n)) : 0.f;  // the normalised activation as the bf16 it would be stored as
+        amax = fmaxf(amax, fabsf(v[i]));
+    }
+    amax = block_max(amax, red);
+    if (amax < 1e-5f) amax = 1e-5f;
+    const float scale = 127.0f / amax;
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < RNAQ_MAX_PER_THREAD; ++i) {
+        const int k = threadIdx.x + i * blockDim.x;
+        if (k >= K) continue;
+        float q = rintf(v[i] * scale);
+        q = fminf(fmaxf(q, -128.0f), 127.0f);
+        const int qi = (int)q;
+        qr[k] = (int8_t)qi;
+        sum += qi;
+    }
+    sum = wave_sum_i(sum);
+    const int wv = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    if ((threadIdx.x & 63) == 0) redi[wv] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int t = 0;
+        for (int i = 0; i < nw; ++i) t += redi[i];
+        scales[blockIdx.x] = scale;
+        if (rowsum) rowsum[blockIdx.x] = t;
+    }
+}
+
 inline int row_threads(int K) { return K >= 2048 ? 256 : (K >= 512 ? 128 : 64); }
 
 }  // namespace
@@ -414,6 +470,16 @@ int vla_act_quant_bf16(const uint16_t* in, int8_t* out, float* scales, int32_t* 
     if (!in || !out || !scales || M < 0 || K <= 0) return VLA_K_ERR_ARG;
     if (M == 0) return VLA_K_OK;
     act_quant_bf16_kernel<<<M, 256, 0, (hipStream_t)stream>>>(in, out, scales, rowsum, K);
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_rmsnorm_act_quant_bf16(const uint16_t* x, const uint16_t* w, int8_t* out, float* scales, int32_t* rowsum, float eps,
+                               int M, int K, vla_stream_t stream) {
+    if (!x || !out || !scales || M < 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (M == 0) return VLA_K_OK;
+    const int th = row_threads(K);
+    if (K > th * RNAQ_MAX_PER_THREAD) return VLA_K_ERR_SHAPE;
+    rmsnorm_act_quant_kernel<<<M, th, 0, (hipStream_t)stream>>>(x, w, out, scales, rowsum, K, eps);
     return VLA_CHECK_LAUNCH();
 }
 

@@ -174,7 +174,11 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
                 if (n >= a.N) continue;
                 const int v = (int)crow[hlf * 32 + jg + e] - rs2;
                 if (a.acc_out) a.acc_out[(long)m * a.N + n] = v;
-                if (a.Y) ((bf16_t*)a.Y)[(long)m * a.N + n] = f2bf((float)v / sm * a.ws[n / group]);
+                if (a.Y) {
+                    bf16_t o = f2bf((float)v / sm * a.ws[n / group]);
+                    if (a.residual) o = f2bf(bf2f(o) + bf2f(((const bf16_t*)a.residual)[(long)m * a.N + n]));
+                    ((bf16_t*)a.Y)[(long)m * a.N + n] = o;
+                }
             }
         return;
     }
@@ -708,13 +712,88 @@ __global__ void __launch_bounds__(WM * 128, 2) ternary_gemm_big_kernel(GemmArgs 
             const int m = m0 + wm * 64 + i * 32 + row, n = n0 + c16 * 8;
             if (m >= a.M) continue;
             bf16_t* dst = (bf16_t*)a.Y + (long)m * a.N + n;
+            const bf16_t* res = a.residual ? (const bf16_t*)a.residual + (long)m * a.N + n : nullptr;
             if (vec_ok && n + 8 <= a.N) {
-                *reinterpret_cast<u32x4_t*>(dst) = v;
+                u32x4_t o = v;
+                if (res) {  // out = bf16(out + residual), both already bf16
+                    const u32x4_t rr = *reinterpret_cast<const u32x4_t*>(res);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        o[e] = pack_bf2(__uint_as_float(v[e] << 16) + __uint_as_float(rr[e] << 16),
+                                        __uint_as_float(v[e] & 0xffff0000u) + __uint_as_float(rr[e] & 0xffff0000u));
+                }
+                *reinterpret_cast<u32x4_t*>(dst) = o;
             } else {
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
-                    if (n + e < a.N) dst[e] = (bf16_t)(v[e >> 1] >> (16 * (e & 1)));
+                    if (n + e < a.N) {
+                        const bf16_t o = (bf16_t)(v[e >> 1] >> (16 * (e & 1)));
+                        dst[e] = res ? f2bf(bf2f(o) + bf2f(res[e])) : o;
+                    }
             }
+        }
+    }
+}
+
+// Ternary GEMV for a handful of rows (single-token decode, M <= 32).  A workgroup owns 32
+// output columns; its 8 wavefronts each take one eighth of K and multiply it with
+// v_mfma_i32_32x32x32_i8 as C[n][m] = sum_k W[n][k] * A[m][k] (weight fragment as the A
+// operand: one coalesced 256-byte load per 32 k; activation rows as the B operand, lanes
+// past M feed zeros).  Every load of a wavefront's slice is issued before the first is
+// used; the eight partial 32 x 32 int32 tiles are summed through LDS (exact) and the
+// epilogue of the tiled kernels follows, with an optional bf16 residual add.
+constexpr int GEMV_WAVES = 8;
+template <int MAXG>  // k groups of 32 per wavefront held in registers: K <= 256 * MAXG
+__global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_kernel(GemmArgs a) {
+    __shared__ int part[GEMV_WAVES][32][33];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 5, r = lane & 31;
+    const int nb = blockIdx.x;                       // 32-column block
+    const int kgroups = a.K / 32;
+    const int per_wave = (kgroups + GEMV_WAVES - 1) / GEMV_WAVES;
+    const int kg0 = wave * per_wave, kg1 = min(kgroups, kg0 + per_wave);
+    const uint32_t* wp = (const uint32_t*)a.W + (long)nb * kgroups * 64 + lane;
+    const bool row_ok = r < a.M;
+    const unsigned char* ap = (const unsigned char*)a.A + (long)(row_ok ? r : 0) * a.K + g * 16;
+
+    uint32_t wv[MAXG];
+    u32x4_t av[MAXG];
+#pragma unroll
+    for (int i = 0; i < MAXG; ++i) {
+        const int kg = min(kg0 + i, kgroups - 1);    // past the slice: a valid group, not multiplied
+        wv[i] = wp[(long)kg * 64];
+        av[i] = *reinterpret_cast<const u32x4_t*>(ap + kg * 32);
+    }
+    i32x16_t acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0;
+#pragma unroll
+    for (int i = 0; i < MAXG; ++i) {
+        if (kg0 + i < kg1) {                         // uniform
+            const uint32_t w = wv[i];
+            const u32x4_t fw = {w & 0x03030303u, (w >> 2) & 0x03030303u, (w >> 4) & 0x03030303u, (w >> 6) & 0x03030303u};
+            const u32x4_t z = {0u, 0u, 0u, 0u};
+            Traits<int8_t>::mma(acc, fw, row_ok ? av[i] : z);
+        }
+    }
+    // element 4j+i of lane (g, r) is C[n = 8j + 4g + i][m = r]
+#pragma unroll
+    for (int e = 0; e < 16; ++e) part[wave][8 * (e >> 2) + 4 * g + (e & 3)][r] = acc[e];
+    __syncthreads();
+    // thread -> (m, n): 512 threads cover 16 rows x 32 columns per pass, n fastest
+    const int group = a.N / a.ws_num;
+    for (int m = tid >> 5; m < a.M; m += GEMV_WAVES * 2) {
+        const int nl = tid & 31, n = nb * 32 + nl;
+        if (n >= a.N) continue;
+        int v = 0;
+#pragma unroll
+        for (int w = 0; w < GEMV_WAVES; ++w) v += part[w][nl][m];
+        v -= 2 * a.rowsum[m];
+        if (a.acc_out) a.acc_out[(long)m * a.N + n] = v;
+        if (a.Y) {
+            bf16_t o = f2bf((float)v / (a.s ? a.s[m] : 1.f) * a.ws[n / group]);
+            if (a.residual) o = f2bf(bf2f(o) + bf2f(((const bf16_t*)a.residual)[(long)m * a.N + n]));
+            ((bf16_t*)a.Y)[(long)m * a.N + n] = o;
         }
     }
 }
@@ -771,7 +850,12 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
         // CU (measured faster than one 256 x 256 workgroup: fewer wavefronts per barrier).
         const int n256 = (a.N + 255) / 256;
         const long wg128 = (long)((a.M + 127) / 128) * n256;
-        if (force == 256) {
+        const int gemv_groups = (a.K / 32 + GEMV_WAVES - 1) / GEMV_WAVES;  // k groups per wavefront
+        if (force == 0 && a.M <= 32 && gemv_groups <= 28) {
+            const unsigned grid = (unsigned)((a.N + 31) / 32);
+            if (gemv_groups <= 10) ternary_gemv_kernel<10><<<grid, GEMV_WAVES * 64, 0, st>>>(a);
+            else ternary_gemv_kernel<28><<<grid, GEMV_WAVES * 64, 0, st>>>(a);
+        } else if (force == 256) {
             const unsigned grid = (unsigned)(((((a.M + 255) / 256) + 7) & ~7) * n256);
             ternary_gemm_big_kernel<4><<<grid, 512, 0, st>>>(a);
         } else if (force == 128 || (force == 0 && wg128 >= 128)) {
@@ -859,6 +943,16 @@ int vla_ternary_gemm(const int8_t* A, const uint32_t* W_packed, uint16_t* out, i
     GemmArgs a = {};
     a.A = A; a.W = W_packed; a.M = M; a.N = N; a.K = K;
     a.Y = out; a.acc_out = acc_out; a.s = s; a.rowsum = rowsum; a.ws = ws; a.ws_num = ws_num > 0 ? ws_num : 1;
+    return launch<int8_t, EPI_TERNARY>(a, (N + BN - 1) / BN, stream);
+}
+
+int vla_ternary_gemm_add(const int8_t* A, const uint32_t* W_packed, uint16_t* out, const uint16_t* residual, const float* s,
+                         const int32_t* rowsum, const float* ws, int ws_num, int M, int N, int K, vla_stream_t stream) {
+    if (!A || !W_packed || !rowsum || !out || !s || !ws || ws_num <= 0 || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (K % 128 || N % ws_num) return VLA_K_ERR_SHAPE;
+    GemmArgs a = {};
+    a.A = A; a.W = W_packed; a.M = M; a.N = N; a.K = K;
+    a.Y = out; a.residual = residual; a.s = s; a.rowsum = rowsum; a.ws = ws; a.ws_num = ws_num;
     return launch<int8_t, EPI_TERNARY>(a, (N + BN - 1) / BN, stream);
 }
 
