@@ -144,17 +144,18 @@ def kernel_breakdown(pkg, cfg, B, P):
         kc, vc = kcs[0], vcs[0]
         cos, sin = torch.ones(T, D // 2, device=dev), torch.zeros(T, D // 2, device=dev)
         scale = 1.0 / np.sqrt(D)
-        add("rms_norm", lambda i: pkg.call("bitvla_rmsnorm_bf16", h, w1, hn, 1e-5, M, H), 2 * L + 1, "hbm", 2 * M * H * 2)
-        add("act_quant", lambda i: pkg.call("vla_act_quant_bf16", hn, q8, s, rs, M, H), 2 * L, "hbm", M * H * 3)
+        add("rmsnorm_act_quant", lambda i: pkg.call("vla_rmsnorm_act_quant_bf16", h, w1, q8, s, rs, 1e-5, M, H), 2 * L, "hbm",
+            M * H * 3)
         add("ternary_qkv_gemv", lambda i: pkg.call("vla_ternary_gemm", q8, wq, qkv, None, s, rs, ws, 6, M, N, H), L, "hbm",
             N * H // 4 + M * H + 2 * M * N)
         add("qkv_split_rope_append", lambda i: pkg.call("vla_qkv_split_rope_append", qkv, cos, sin, q, kc, vc, dt, M, 1, Hq,
                                                        Hkv, D, t_max, P), L, "hbm", 2 * M * N * 2)
-        add("attention_decode", lambda i: pkg.call("vla_attn_prefix_suffix", q, kcs[i % n_rot], vcs[i % n_rot], att, dt, B, 1, Hq, Hkv, D, t_max,
-                                                 T, scale, 0, T, 0, 0, None), L, "hbm", 2 * T * kvd * es * B)
-        add("ternary_o_gemv", lambda i: pkg.call("vla_ternary_gemm", q8, wo, hn, None, s, rs, ws, 1, M, H, H), L, "hbm",
-            H * H // 4 + M * H + 2 * M * H)
-        add("add_residual", lambda i: pkg.call("bitvla_add_bf16", h, hn, h, M * H), L, "hbm", 3 * M * H * 2)
+        add("attention_decode", lambda i: pkg.call("vla_attn_prefix_suffix", q, kcs[i % n_rot], vcs[i % n_rot], att,
+                                                 pkg.VLA_DT_BF16_P2, B, 1, Hq, Hkv, D, t_max, T, scale, 0, T, 0, 0, None),
+            L, "hbm", 2 * T * kvd * es * B)
+        add("ternary_o_gemv_add", lambda i: pkg.call("vla_ternary_gemm_add", q8, wo, h, h, s, rs, ws, 1, M, H, H), L, "hbm",
+            H * H // 4 + M * H + 4 * M * H)
+        add("final_rms_norm", lambda i: pkg.call("bitvla_rmsnorm_bf16", h, w1, hn, 1e-5, M, H), 1, "hbm", 2 * M * H * 2)
         # the prefill-shaped fused QKV GEMM (one launch per layer per observation batch)
         Mp = B * P
         q8p, sp, rsp = z(Mp, H, dtype=torch.int8), torch.ones(Mp, device=dev), z(Mp, dtype=torch.int32)

@@ -92,8 +92,14 @@ template <> struct AT<float> {
     __device__ static __forceinline__ float fexp2(float x) { return exp2f(x); }
 };
 
-template <typename T, int D, int NW, bool P2>
-__global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_kernel(AttnArgs a) {
+// NL > 0: producer / consumer wavefronts.  Wavefronts NW .. NW+NL-1 only move data: they
+// keep LOAD_AHEAD key tiles of global loads in flight in their own registers (they need
+// none for arithmetic) and store them into a double-buffered LDS tile pair; the NW compute
+// wavefronts never touch global memory inside the loop.  One barrier per tile.  Used for
+// wide heads, whose accumulators and query fragments leave the compute wavefronts no
+// registers to prefetch with, so that memory latency would be exposed once per tile.
+template <typename T, int D, int NW, bool P2, int NL>
+__global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_kernel(AttnArgs a) {
     typedef AT<T> A;
     constexpr int EB = A::EB, CE = A::CE;
     // Keys per staged tile: 64, or 32 for wide heads (rows of 512 bytes and more), whose
@@ -115,8 +121,10 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
     static_assert(D % CE == 0 && (D * EB) % 16 == 0, "head_dim must be whole MFMA groups and 16-byte rows");
     static_assert(NVEC == D * VV_PER_ROW, "K and V^T tiles hold the same number of vectors");
 
-    __shared__ __attribute__((aligned(16))) unsigned char ldsK[TK * KS];
-    __shared__ __attribute__((aligned(16))) unsigned char ldsV[DP * VS];
+    __shared__ __attribute__((aligned(16))) unsigned char ldsK_buf[NL ? 2 : 1][TK * KS];
+    __shared__ __attribute__((aligned(16))) unsigned char ldsV_buf[NL ? 2 : 1][DP * VS];
+    unsigned char* ldsK = ldsK_buf[0];
+    unsigned char* ldsV = ldsV_buf[0];
 
     // ---- XCD-aware decode of the linear workgroup id
     const int GS = a.n_groups * a.n_split;
@@ -132,8 +140,8 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
     const int grp = a.Hq / a.Hkv;
     const int R = grp * a.S;
     const int row = (group * NW + wave) * 32 + r;
-    const bool wave_active = (group * NW + wave) * 32 < R;
-    const bool row_valid = row < R;
+    const bool wave_active = wave < NW && (group * NW + wave) * 32 < R;
+    const bool row_valid = wave < NW && row < R;
     const int hg = row_valid ? row / a.S : 0;
     const int s = row_valid ? row % a.S : 0;
     const int h = hk * grp + hg;
@@ -249,17 +257,27 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
         float m_tile = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < NKB; ++kb) {
-            f32x16_t sc;
+            // the head_dim contraction runs as NA independent MFMA chains (a single chain of
+            // NQ dependent MFMAs is latency-bound for wide heads), summed at the end
+            constexpr int NA = (NQ >= 4 && NKB == 1) ? 2 : 1;
+            f32x16_t sc[NA];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+            for (int n = 0; n < NA; ++n)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) sc[n][i] = 0.f;
 #pragma unroll
             for (int c = 0; c < NQ; ++c) {
                 const u32x4_t kf =
                     *reinterpret_cast<const u32x4_t*>(ldsK + (kb * 32 + key_of_score_row(r)) * KS + (c * CE + g * (CE / 2)) * EB);
-                A::mma(sc, kf, qf[c]);
+                A::mma(sc[c % NA], kf, qf[c]);
             }
 #pragma unroll
-            for (int i = 0; i < 16; ++i) p[kb][i] = sc[i] * c2;
+            for (int i = 0; i < 16; ++i) {
+                float v = sc[0][i];
+#pragma unroll
+                for (int n = 1; n < NA; ++n) v += sc[n][i];
+                p[kb][i] = v * c2;
+            }
         }
         if (tile_masked) {
             if (a.mask) {  // mask given as data: additive, one fp32 per (query, key)
@@ -360,7 +378,69 @@ __global__ void __launch_bounds__(NW * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_
         }
     };
 
-    if (PREFETCH) {
+    if constexpr (NL > 0) {
+        constexpr int NTL = NL * 64, ITL = NVEC / NTL, LOAD_AHEAD = 3;
+        static_assert(NVEC % NTL == 0 && EB == 2, "loader wavefronts split a tile evenly; bf16 only");
+        const int n_t = (k_end - k_begin + TK - 1) / TK;
+        const int n_pad = (n_t + LOAD_AHEAD - 1) / LOAD_AHEAD * LOAD_AHEAD;  // both roles run n_pad + 1 barriers
+        if (wave >= NW) {
+            const int lt = tid - NW * 64;
+            u32x4_t kq[LOAD_AHEAD][ITL], vq[LOAD_AHEAD][ITL];
+            // Unconditional loads with clamped addresses (K rows past n_keys repeat the last
+            // key: their scores are masked; V^T runs are kept inside the row) so the loop body
+            // has no load under a branch; tiles past the last repeat it and are never read.
+            auto fetch = [&](int slot, int t) __attribute__((always_inline)) {
+                const int k0 = k_begin + max(min(t, n_t - 1), 0) * TK;
+#pragma unroll
+                for (int i = 0; i < ITL; ++i) {
+                    const int v = lt + i * NTL;
+                    const int key = min(k0 + v / KV_PER_ROW, a.n_keys - 1);
+                    kq[slot][i] = *reinterpret_cast<const u32x4_t*>(kbase + (long)key * D * EB + (v % KV_PER_ROW) * 16);
+                    const int key0 = min(k0 + (v % VV_PER_ROW) * EPV, a.t_max - EPV);
+                    vq[slot][i] = *reinterpret_cast<const u32x4_t*>(vbase + ((long)(v / VV_PER_ROW) * a.t_max + key0) * EB);
+                }
+            };
+            // V^T elements past n_keys are zeroed so that stale cache contents (possibly NaN)
+            // cannot reach the accumulators.
+            auto publish = [&](int slot, int t, int stage) __attribute__((always_inline)) {
+                const int k0 = k_begin + max(min(t, n_t - 1), 0) * TK;
+#pragma unroll
+                for (int i = 0; i < ITL; ++i) {
+                    const int v = lt + i * NTL;
+                    *reinterpret_cast<u32x4_t*>(ldsK_buf[stage] + (v / KV_PER_ROW) * KS + (v % KV_PER_ROW) * 16) = kq[slot][i];
+                    const int nvalid = a.n_keys - (k0 + (v % VV_PER_ROW) * EPV);  // real keys among the 8, may be <= 0
+                    u32x4_t val = vq[slot][i];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) val[e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+                    *reinterpret_cast<u32x4_t*>(ldsV_buf[stage] + (v / VV_PER_ROW) * VS + (v % VV_PER_ROW) * 16) = val;
+                }
+            };
+#pragma unroll
+            for (int sl = 0; sl < LOAD_AHEAD; ++sl) fetch(sl, sl);
+            publish(0, 0, 0);
+            __syncthreads();
+            for (int t0 = 0; t0 < n_pad; t0 += LOAD_AHEAD) {
+#pragma unroll
+                for (int sl = 0; sl < LOAD_AHEAD; ++sl) {
+                    const int t = t0 + sl;
+                    fetch(sl, t + LOAD_AHEAD);                       // slot sl held tile t, already published
+                    publish((sl + 1) % LOAD_AHEAD, t + 1, (t + 1) & 1);  // while the compute wavefronts read stage t & 1
+                    __syncthreads();
+                }
+            }
+            return;
+        }
+        __syncthreads();
+        for (int t = 0; t < n_pad; ++t) {
+            if (t < n_t && wave_active) {
+                ldsK = ldsK_buf[t & 1];
+                ldsV = ldsV_buf[t & 1];
+                scores_softmax(k_begin + t * TK);
+                output_product();
+            }
+            __syncthreads();
+        }
+    } else if (PREFETCH) {
         // Small tiles: the whole next tile waits in registers while the current one is used.
         if (k_begin < k_end) {
             load_k(k_begin);
@@ -769,10 +849,11 @@ int launch_nw(AttnArgs& a, hipStream_t st) {
     const int n_pairs = a.batch * a.Hkv;
     const int grid = (n_pairs + 7) / 8 * 8 * a.n_groups * a.n_split;
     if constexpr (sizeof(T) == 2) {
-        if (a.p2) attn_kernel<T, D, NW, true><<<grid, NW * 64, 0, st>>>(a);
-        else attn_kernel<T, D, NW, false><<<grid, NW * 64, 0, st>>>(a);
+        constexpr int NL = (D * sizeof(T) >= 512) ? 4 : 0;  // wide heads: four loader wavefronts
+        if (a.p2) attn_kernel<T, D, NW, true, NL><<<grid, (NW + NL) * 64, 0, st>>>(a);
+        else attn_kernel<T, D, NW, false, NL><<<grid, (NW + NL) * 64, 0, st>>>(a);
     } else {
-        attn_kernel<T, D, NW, false><<<grid, NW * 64, 0, st>>>(a);
+        attn_kernel<T, D, NW, false, 0><<<grid, NW * 64, 0, st>>>(a);
     }
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     if (a.n_split > 1) {
