@@ -849,7 +849,9 @@ int launch_nw(AttnArgs& a, hipStream_t st) {
     const int n_pairs = a.batch * a.Hkv;
     const int grid = (n_pairs + 7) / 8 * 8 * a.n_groups * a.n_split;
     if constexpr (sizeof(T) == 2) {
-        constexpr int NL = (D * sizeof(T) >= 512) ? 4 : 0;  // wide heads: four loader wavefronts
+        // Wide heads: four loader wavefronts.  Narrow heads prefetch in registers instead
+        // (with loader wavefronts a batch-32 SmolVLA launch no longer fits the chip in one round).
+        constexpr int NL = (D * sizeof(T) >= 512) ? 4 : 0;
         if (a.p2) attn_kernel<T, D, NW, true, NL><<<grid, (NW + NL) * 64, 0, st>>>(a);
         else attn_kernel<T, D, NW, false, NL><<<grid, (NW + NL) * 64, 0, st>>>(a);
     } else {
