@@ -319,9 +319,10 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     constexpr int VA = ROWS_A * VPR / 256, VW = ROWS_W * VPR / 256;  // vectors per thread
     static_assert(kEpi != EPI_TERNARY || (TM == 1 && TN == 1 && KB == 128), "ternary staging assumes 64x64x128 tiles");
 
-    __shared__ __attribute__((aligned(16))) unsigned char lds[(ROWS_A + ROWS_W) * STRIDE];
-    unsigned char* ldsA = lds;
-    unsigned char* ldsW = lds + ROWS_A * STRIDE;
+    // two operand buffers: tile kt is multiplied out of buffer kt & 1 while tile kt + 1 is
+    // being stored into the other one, so a k-tile costs one barrier
+    constexpr int BUF = (ROWS_A + ROWS_W) * STRIDE;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * BUF];
     static_assert(sizeof(float) * 64 * C_STRIDE <= sizeof(lds), "C sub-tile must fit in the operand buffers");
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -420,7 +421,9 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
                 }
         }
     };
-    auto store_tile = [&](int st) __attribute__((always_inline)) {
+    auto store_tile = [&](int st, int buf) __attribute__((always_inline)) {
+        unsigned char* ldsA = lds + buf * BUF;
+        unsigned char* ldsW = ldsA + ROWS_A * STRIDE;
 #pragma unroll
         for (int v = 0; v < VA; ++v) {
             const int idx = tid + v * 256;
@@ -449,7 +452,9 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
             }
         }
     };
-    auto multiply = [&]() __attribute__((always_inline)) {
+    auto multiply = [&](int buf) __attribute__((always_inline)) {
+        const unsigned char* ldsA = lds + buf * BUF;
+        const unsigned char* ldsW = ldsA + ROWS_A * STRIDE;
 #pragma unroll
         for (int ch = 0; ch < KB / TR::kChunkBytes; ++ch) {
             const int off = ch * TR::kChunkBytes + g * 16;
@@ -466,20 +471,25 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     };
 
     // Stage st of the ring holds tile kt with kt % DEPTH == st.  Main loop: whole groups
-    // of DEPTH full tiles, no branch in the body.  The remaining tiles (fewer than DEPTH
+    // of DEPTH full tiles, no branch around a load.  The remaining tiles (fewer than DEPTH
     // full ones and at most one partial) are already in flight when the main loop ends
-    // and are drained without further loads.
+    // and are drained without further loads.  The LDS store of tile kt + 1 follows the
+    // multiply of tile kt in program order, so it runs under the MFMAs still in flight.
 #pragma unroll
     for (int st = 0; st < DEPTH; ++st) load_tile(st, min(st, nkt - 1));
+    if (BK > a.K) mask_partial(0, 0);
+    store_tile(0, 0);
+    __syncthreads();
     const int n_main = (a.K / BK) / DEPTH;
     for (int gi = 0; gi < n_main; ++gi) {
 #pragma unroll
         for (int st = 0; st < DEPTH; ++st) {
-            store_tile(st);
-            __syncthreads();
-            load_tile(st, min(gi * DEPTH + st + DEPTH, nkt - 1));
-            __builtin_amdgcn_sched_barrier(0);  // the loads stay above the multiply they hide behind
-            multiply();
+            const int kt = gi * DEPTH + st;
+            load_tile(st, min(kt + DEPTH, nkt - 1));  // stage st held tile kt, already in LDS
+            __builtin_amdgcn_sched_barrier(0);        // the loads stay above the multiply they hide behind
+            multiply(kt & 1);
+            if ((kt + 2) * BK > a.K) mask_partial((st + 1) % DEPTH, kt + 1);  // uniform; only the last tile can be partial
+            store_tile((st + 1) % DEPTH, (kt + 1) & 1);  // past the last tile: a repeat of it, never read
             __syncthreads();
         }
     }
@@ -487,10 +497,11 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     for (int st = 0; st < DEPTH; ++st) {
         const int kt = n_main * DEPTH + st;
         if (kt < nkt) {  // uniform
-            if (kt * BK + BK > a.K) mask_partial(st, kt);
-            store_tile(st);
-            __syncthreads();
-            multiply();
+            multiply(kt & 1);
+            if (kt + 1 < nkt) {
+                if ((kt + 2) * BK > a.K) mask_partial((st + 1) % DEPTH, kt + 1);
+                store_tile((st + 1) % DEPTH, (kt + 1) & 1);
+            }
             __syncthreads();
         }
     }
