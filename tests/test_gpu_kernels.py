@@ -110,7 +110,7 @@ def test_bitvla_rope_head_major_bf16():
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("M,K", [(50, 720), (51, 1024), (17, 1536), (3, 2560)])
+@pytest.mark.parametrize("M,K", [(50, 720), (51, 1024), (17, 1536), (3, 2560), (1600, 720), (816, 1024), (1088, 1536), (200, 4096), (65, 724)])
 def test_rms_norm_and_adaln(dtype, M, K):
     r = np.random.default_rng(103)
     x = (r.standard_normal((M, K)) * 2 + 0.5).astype(np.float32)
@@ -456,11 +456,12 @@ def test_ternary_gemm_prefill_shape_all_tilings_agree(monkeypatch):
     assert np.array_equal(host(res[0][1], np.uint16)[rows], orc.ternary_epilogue(want_acc, s[rows], ws))
 
 
-@pytest.mark.parametrize("M", [1, 8, 32])
-def test_ternary_gemv_decode_rows_bit_exact(M):
+@pytest.mark.parametrize("M,N,K,ws_num", [(1, 3840, 2560, 6), (8, 3840, 2560, 6), (32, 3840, 2560, 6),
+                                          (5, 48, 128, 3), (3, 640, 6912, 1)])
+def test_ternary_gemv_decode_rows_bit_exact(M, N, K, ws_num):
     # At most 32 rows (single-token decode): the split-K GEMV kernel gives the oracle's
     # accumulators and epilogue, and, with a residual, the bits of GEMM followed by add.
-    N, K, ws_num = 3840, 2560, 6
+    # Ragged N (not a multiple of 32), a K of one 128-slice and the long-K variant included.
     r = np.random.default_rng(900 + M)
     A = r.integers(-127, 128, (M, K)).astype(np.int8)
     t = r.integers(-1, 2, (N, K)).astype(np.int8)
@@ -504,7 +505,7 @@ def test_ternary_gemm_add_matches_gemm_then_add(monkeypatch, M, N, K, tile):
     assert np.array_equal(host(fused), host(want))
 
 
-@pytest.mark.parametrize("M,K", [(8, 2560), (37, 720), (4, 4096)])
+@pytest.mark.parametrize("M,K", [(8, 2560), (37, 720), (4, 4096), (300, 2560), (129, 720), (70, 4096)])
 def test_rmsnorm_act_quant_fused_is_the_pair(M, K):
     r = np.random.default_rng(K + M)
     x = orc.to_bf16((r.standard_normal((M, K)) * 3).astype(np.float32))

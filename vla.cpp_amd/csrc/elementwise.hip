@@ -132,6 +132,145 @@ __global__ void adaln_kernel(const T* __restrict__ x, const float* __restrict__ 
     }
 }
 
+// Row normalisations, one wavefront per row (four rows per workgroup): the row is read once
+// with 16-byte loads and stays in registers, the reductions are wavefront shuffles, and there
+// is no LDS and no barrier.  RMS: y = x * rsqrt(mean(x^2) + eps) * w.  ADALN: LayerNorm
+// without affine, then y = xn * (1 + scale) + shift.  RMS_AQ: the RMS result, rounded to bf16
+// as it would be stored, quantised per row to int8 (scale 127 / max(amax, 1e-5), round half
+// even) with its row sum -- bitvla_rmsnorm_bf16 followed by act_quant without the round trip.
+enum { NORM_RMS = 0, NORM_ADALN = 1, NORM_RMS_AQ = 2 };
+template <typename T, int NV, int MODE>
+__global__ void __launch_bounds__(256) row_norm_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                       const float* __restrict__ sc, const float* __restrict__ sh,
+                                                       T* __restrict__ y, int8_t* __restrict__ q, float* __restrict__ scales,
+                                                       int32_t* __restrict__ rowsum, int M, int K, float eps) {
+    constexpr int EPV = 16 / sizeof(T);
+    const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const int nvec = K / EPV;
+    const T* xr = x + (long)row * K;
+    float v[NV][EPV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int vec = lane + 64 * i;
+        u32x4_t raw = {0u, 0u, 0u, 0u};
+        if (vec < nvec) raw = *reinterpret_cast<const u32x4_t*>(xr + (long)vec * EPV);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+            if (sizeof(T) == 2) v[i][e] = __uint_as_float((e & 1) ? (raw[e >> 1] & 0xffff0000u) : (raw[e >> 1] << 16));
+            else v[i][e] = __uint_as_float(raw[e]);
+        }
+    }
+    float mean = 0.f, inv;
+    if (MODE == NORM_ADALN) {
+        float s1 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) s1 += v[i][e];
+        mean = wave_sum(s1) / (float)K;
+        float s2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                const float d = (lane + 64 * i < nvec) ? v[i][e] - mean : 0.f;
+                s2 += d * d;
+            }
+        inv = 1.0f / sqrtf(wave_sum(s2) / (float)K + eps);
+    } else {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) ss += v[i][e] * v[i][e];
+        inv = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
+    }
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int vec = lane + 64 * i;
+        if (vec >= nvec) continue;
+        const int k0 = vec * EPV;
+        float o[EPV];
+        if (MODE == NORM_ADALN) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                const float xn = (v[i][e] - mean) * inv;
+                o[e] = xn + xn * sc[k0 + e] + sh[k0 + e];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                o[e] = v[i][e] * inv;
+                if (w) o[e] *= Elem<T>::load(w + k0 + e);
+            }
+        }
+        if (MODE == NORM_RMS_AQ) {
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                v[i][e] = bf2f(f2bf(o[e]));  // the activation as the bf16 it would be stored as
+                amax = fmaxf(amax, fabsf(v[i][e]));
+            }
+        } else if (sizeof(T) == 2) {
+            u32x4_t pk;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pk[e] = (uint32_t)f2bf(o[2 * e]) | ((uint32_t)f2bf(o[2 * e + 1]) << 16);
+            *reinterpret_cast<u32x4_t*>(y + (long)row * K + k0) = pk;
+        } else {
+            const u32x4_t pk = {__float_as_uint(o[0]), __float_as_uint(o[1]), __float_as_uint(o[2]), __float_as_uint(o[3])};
+            *reinterpret_cast<u32x4_t*>(y + (long)row * K + k0) = pk;
+        }
+    }
+    if (MODE == NORM_RMS_AQ) {
+        amax = wave_max(amax);
+        if (amax < 1e-5f) amax = 1e-5f;
+        const float scale = 127.0f / amax;
+        int sum = 0;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int vec = lane + 64 * i;
+            if (vec >= nvec) continue;
+            uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) {
+                float qf = rintf(v[i][e] * scale);
+                qf = fminf(fmaxf(qf, -128.0f), 127.0f);
+                const int qi = (int)qf;
+                sum += qi;
+                pk[e >> 2] |= (uint32_t)(qi & 0xff) << (8 * (e & 3));
+            }
+            *reinterpret_cast<u32x2_t*>(q + (long)row * K + (long)vec * EPV) = u32x2_t{pk[0], pk[1]};
+        }
+        sum = wave_sum_i(sum);
+        if (lane == 0) {
+            scales[row] = scale;
+            if (rowsum) rowsum[row] = sum;
+        }
+    }
+}
+
+// Launches row_norm_kernel when the row fits a wavefront's registers and the buffers allow
+// 16-byte accesses; returns false otherwise (the callers fall back to the scalar kernels).
+// The choice depends on the row length only, never on the number of rows, so an
+// observation's result does not depend on the batch it is run in.
+template <typename T, int MODE>
+bool launch_row_norm(const void* x, const void* w, const float* sc, const float* sh, void* y, int8_t* q, float* scales,
+                     int32_t* rowsum, int M, int K, float eps, hipStream_t st) {
+    constexpr int EPV = 16 / sizeof(T);
+    if (K % EPV || (((uintptr_t)x | (uintptr_t)y | (uintptr_t)q) & 15)) return false;
+    if (MODE == NORM_RMS_AQ && (K % 8)) return false;
+    const int nvec = K / EPV, blocks = (M + 3) / 4;
+#define VLA_ROW_NORM(NV) \
+    row_norm_kernel<T, NV, MODE><<<blocks, 256, 0, st>>>((const T*)x, (const T*)w, sc, sh, (T*)y, q, scales, rowsum, M, K, eps)
+    if (nvec <= 64 * 2) VLA_ROW_NORM(2);
+    else if (nvec <= 64 * 4) VLA_ROW_NORM(4);
+    else if (nvec <= 64 * 8) VLA_ROW_NORM(8);
+    else return false;
+#undef VLA_ROW_NORM
+    return true;
+}
+
 // ------------------------------------------------- flow-matching glue ---
 // One workgroup per EMB_ROWS consecutive (batch, token) rows.  The action rows and a
 // 64-column slab of W_in at a time sit in LDS (both read from HBM with contiguous,
@@ -407,6 +546,10 @@ int vla_rms_norm(const void* x, const void* w, void* y, int dtype, int M, int K,
     if (M == 0) return VLA_K_OK;
     hipStream_t st = (hipStream_t)stream;
     const int th = row_threads(K);
+    if (dtype == VLA_DT_F32 && launch_row_norm<float, NORM_RMS>(x, w, nullptr, nullptr, y, nullptr, nullptr, nullptr, M, K, eps, st))
+        return VLA_CHECK_LAUNCH();
+    if (dtype == VLA_DT_BF16 && launch_row_norm<bf16_t, NORM_RMS>(x, w, nullptr, nullptr, y, nullptr, nullptr, nullptr, M, K, eps, st))
+        return VLA_CHECK_LAUNCH();
     if (dtype == VLA_DT_F32)
         rms_norm_kernel<float><<<M, th, 0, st>>>((const float*)x, (const float*)w, (float*)y, K, eps);
     else if (dtype == VLA_DT_BF16)
@@ -422,6 +565,10 @@ int vla_adaln(const void* x, const float* sc, const float* sh, void* y, int dtyp
     if (M == 0) return VLA_K_OK;
     hipStream_t st = (hipStream_t)stream;
     const int th = row_threads(K);
+    if (dtype == VLA_DT_F32 && launch_row_norm<float, NORM_ADALN>(x, nullptr, sc, sh, y, nullptr, nullptr, nullptr, M, K, eps, st))
+        return VLA_CHECK_LAUNCH();
+    if (dtype == VLA_DT_BF16 && launch_row_norm<bf16_t, NORM_ADALN>(x, nullptr, sc, sh, y, nullptr, nullptr, nullptr, M, K, eps, st))
+        return VLA_CHECK_LAUNCH();
     if (dtype == VLA_DT_F32)
         adaln_kernel<float><<<M, th, 0, st>>>((const float*)x, sc, sh, (float*)y, K, eps);
     else if (dtype == VLA_DT_BF16)
@@ -477,6 +624,8 @@ int vla_rmsnorm_act_quant_bf16(const uint16_t* x, const uint16_t* w, int8_t* out
                                int M, int K, vla_stream_t stream) {
     if (!x || !out || !scales || M < 0 || K <= 0) return VLA_K_ERR_ARG;
     if (M == 0) return VLA_K_OK;
+    if (launch_row_norm<bf16_t, NORM_RMS_AQ>(x, w, nullptr, nullptr, nullptr, out, scales, rowsum, M, K, eps, (hipStream_t)stream))
+        return VLA_CHECK_LAUNCH();
     const int th = row_threads(K);
     if (K > th * RNAQ_MAX_PER_THREAD) return VLA_K_ERR_SHAPE;
     rmsnorm_act_quant_kernel<<<M, th, 0, (hipStream_t)stream>>>(x, w, out, scales, rowsum, K, eps);
