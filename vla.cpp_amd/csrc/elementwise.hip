@@ -272,11 +272,12 @@ bool launch_row_norm(const void* x, const void* w, const float* sc, const float*
 }
 
 // ------------------------------------------------- flow-matching glue ---
-// One workgroup per EMB_ROWS consecutive (batch, token) rows.  The action rows and a
-// 64-column slab of W_in at a time sit in LDS (both read from HBM with contiguous,
-// coalesced loads); thread (rr, c) then forms the dot products of rows rr, rr+4 with
-// column c, and stores are coalesced along the width.
-constexpr int EMB_ROWS = 8;
+// Workgroup (x, y) forms EMB_ROWS consecutive (batch, token) rows of column slab y (EMB_COLS
+// columns).  The action rows and the slab of W_in sit in LDS, both read with contiguous,
+// coalesced loads issued together; thread (rq, cl) then forms the dot products of rows
+// rq, rq+4, ... with column cl (summed over the action dimension in ascending order), and
+// stores are coalesced along the width.  One load round trip per workgroup.
+constexpr int EMB_ROWS = 32;
 constexpr int EMB_MAX_A = 64;
 constexpr int EMB_COLS = 64;
 template <typename T>
@@ -286,7 +287,8 @@ __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restri
                                                             int S, int n_lead, int A, int W) {
     __shared__ float xs[EMB_ROWS][EMB_MAX_A];
     __shared__ float ws[EMB_COLS][EMB_MAX_A + 1];
-    const int row0 = blockIdx.x * EMB_ROWS;
+    const int row0 = blockIdx.x * EMB_ROWS, c0 = blockIdx.y * EMB_COLS;
+    const int ncol = min(EMB_COLS, W - c0);
     for (int i = threadIdx.x; i < EMB_ROWS * A; i += blockDim.x) {
         const int rr = i / A, a = i % A, row = row0 + rr;
         float v = 0.f;
@@ -296,50 +298,75 @@ __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restri
         }
         xs[rr][a] = v;
     }
-    const int cl = threadIdx.x & 63, rq = threadIdx.x >> 6;  // column in slab, row quarter
-    for (int c0 = 0; c0 < W; c0 += EMB_COLS) {
-        __syncthreads();
-        const int ncol = min(EMB_COLS, W - c0);
-        for (int i = threadIdx.x; i < ncol * A; i += blockDim.x) ws[i / A][i % A] = W_in[(long)c0 * A + i];
-        __syncthreads();
-        const int c = c0 + cl;
-        if (c >= W) continue;
-        const float bias = bias_step[c];
+    for (int i = threadIdx.x; i < ncol * A; i += blockDim.x) ws[i / A][i % A] = W_in[(long)c0 * A + i];
+    const int cl = threadIdx.x & 63, rq = threadIdx.x >> 6;  // column in slab, row residue mod 4
+    const int c = c0 + cl;
+    const float bias = c < W ? bias_step[c] : 0.f;
+    __syncthreads();
+    if (c >= W) return;
 #pragma unroll
-        for (int k = 0; k < EMB_ROWS / 4; ++k) {
-            const int rr = rq + 4 * k, row = row0 + rr;
-            if (row >= n_rows) continue;
-            const int b = row / S, s = row % S;
-            float v;
-            if (s < n_lead) {
-                v = lead[((long)b * n_lead + s) * W + c];
-            } else {
-                float acc = 0.f;
-                for (int a = 0; a < A; ++a) acc += ws[cl][a] * xs[rr][a];
-                v = acc + bias;
-            }
-            Elem<T>::store(h + (long)row * W + c, v);
+    for (int k = 0; k < EMB_ROWS / 4; ++k) {
+        const int rr = rq + 4 * k, row = row0 + rr;
+        if (row >= n_rows) continue;
+        const int b = row / S, s = row % S;
+        float v;
+        if (s < n_lead) {
+            v = lead[((long)b * n_lead + s) * W + c];
+        } else {
+            float acc = 0.f;
+            for (int a = 0; a < A; ++a) acc += ws[cl][a] * xs[rr][a];
+            v = acc + bias;
         }
+        Elem<T>::store(h + (long)row * W + c, v);
     }
 }
 
-// grid (batch*(S - n_lead)), one wavefront per output column group.
-template <typename T>
-__global__ void euler_step_kernel(float* __restrict__ x_t, const T* __restrict__ hn, const float* __restrict__ W_out,
-                                  const float* __restrict__ b_out, int S, int n_lead, int A, int W, float dt) {
+// Workgroup (x, y): EUL_WAVES wavefronts, each owning ROWS action rows, all working on the
+// AU action outputs of group y.  A lane keeps elements lane, lane+64, ... of its rows in
+// registers (NC chunks cover the width); the chunk loads of the AU rows of W_out are
+// independent and issued together; the products are summed per lane in ascending k and then
+// across the wavefront, and lane (i, u) applies the update of row i, output u.
+constexpr int EUL_WAVES = 4;
+template <typename T, int NC, int AU, int ROWS>
+__global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __restrict__ x_t, const T* __restrict__ hn,
+                                                                    const float* __restrict__ W_out,
+                                                                    const float* __restrict__ b_out, int n_rows, int S,
+                                                                    int n_lead, int A, int W, float dt) {
     const int Sa = S - n_lead;
-    const int b = blockIdx.x / Sa, s = blockIdx.x % Sa;
-    const T* hr = hn + ((long)b * S + n_lead + s) * W;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
-    for (int a = wave; a < A; a += nw) {
-        const float* wr = W_out + (long)a * W;
-        float acc = 0.f;
-        for (int k = lane; k < W; k += 64) acc += wr[k] * Elem<T>::load(hr + k);
-        acc = wave_sum(acc);
-        if (lane == 0) {
-            float* xp = x_t + ((long)b * Sa + s) * A + a;
-            *xp = *xp + dt * (acc + (b_out ? b_out[a] : 0.f));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int r0 = (blockIdx.x * EUL_WAVES + wave) * ROWS, a0 = blockIdx.y * AU;
+    if (r0 >= n_rows) return;
+    float hv[ROWS][NC], wv[AU][NC];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        const int row = min(r0 + i, n_rows - 1);
+        const int b = row / Sa, s = row % Sa;
+        const T* hr = hn + ((long)b * S + n_lead + s) * W;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) hv[i][c] = Elem<T>::load(hr + min(lane + 64 * c, W - 1));
+    }
+#pragma unroll
+    for (int u = 0; u < AU; ++u) {
+        const float* wr = W_out + (long)min(a0 + u, A - 1) * W;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) wv[u][c] = wr[min(lane + 64 * c, W - 1)];
+    }
+    float mine = 0.f;
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i)
+#pragma unroll
+        for (int u = 0; u < AU; ++u) {
+            float acc = 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; ++c)
+                if (lane + 64 * c < W) acc += wv[u][c] * hv[i][c];
+            acc = wave_sum(acc);
+            if (lane == i * AU + u) mine = acc;
         }
+    const int i = lane / AU, a = a0 + lane % AU;
+    if (lane < ROWS * AU && r0 + i < n_rows && a < A) {
+        float* xp = x_t + (long)(r0 + i) * A + a;
+        *xp = *xp + dt * (mine + (b_out ? b_out[a] : 0.f));
     }
 }
 
@@ -586,7 +613,8 @@ int vla_embed_suffix(const float* x_t, const float* W_in, const float* bias_step
     if (A > EMB_MAX_A) return VLA_K_ERR_SHAPE;
     if (batch == 0) return VLA_K_OK;
     hipStream_t st = (hipStream_t)stream;
-    const int n_rows = batch * S, blocks = (n_rows + EMB_ROWS - 1) / EMB_ROWS;
+    const int n_rows = batch * S;
+    const dim3 blocks((n_rows + EMB_ROWS - 1) / EMB_ROWS, (W + EMB_COLS - 1) / EMB_COLS);
     if (out_dtype == VLA_DT_F32)
         embed_suffix_kernel<float><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W);
     else if (out_dtype == VLA_DT_BF16)
@@ -602,13 +630,28 @@ int vla_euler_step(float* x_t, const void* hn, const float* W_out, const float* 
         return VLA_K_ERR_ARG;
     if (batch == 0) return VLA_K_OK;
     hipStream_t st = (hipStream_t)stream;
-    const int blocks = batch * (S - n_lead);
+    if (dtype != VLA_DT_F32 && dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
+    if (W > 64 * 64) return VLA_K_ERR_SHAPE;
+    const int n_rows = batch * (S - n_lead);
+#define VLA_EULER(T, NC, AU, ROWS)                                                                                  \
+    euler_step_kernel<T, NC, AU, ROWS>                                                                              \
+        <<<dim3((n_rows + EUL_WAVES * ROWS - 1) / (EUL_WAVES * ROWS), (A + AU - 1) / AU), EUL_WAVES * 64, 0, st>>>(  \
+            x_t, (const T*)hn, W_out, b_out, n_rows, S, n_lead, A, W, dt)
+#define VLA_EULER_T(T)                                      \
+    do {                                                    \
+        if (W <= 64 * 8) VLA_EULER(T, 8, 8, 2);             \
+        else if (W <= 64 * 12) VLA_EULER(T, 12, 8, 2);      \
+        else if (W <= 64 * 16) VLA_EULER(T, 16, 8, 2);      \
+        else if (W <= 64 * 24) VLA_EULER(T, 24, 4, 2);      \
+        else if (W <= 64 * 32) VLA_EULER(T, 32, 4, 2);      \
+        else VLA_EULER(T, 64, 2, 1);                        \
+    } while (0)
     if (dtype == VLA_DT_F32)
-        euler_step_kernel<float><<<blocks, 256, 0, st>>>(x_t, (const float*)hn, W_out, b_out, S, n_lead, A, W, dt);
-    else if (dtype == VLA_DT_BF16)
-        euler_step_kernel<bf16_t><<<blocks, 256, 0, st>>>(x_t, (const bf16_t*)hn, W_out, b_out, S, n_lead, A, W, dt);
+        VLA_EULER_T(float);
     else
-        return VLA_K_ERR_ARG;
+        VLA_EULER_T(bf16_t);
+#undef VLA_EULER_T
+#undef VLA_EULER
     return VLA_CHECK_LAUNCH();
 }
 

@@ -24,6 +24,7 @@
 // (g, r), C[8j + 4g + i][r].
 
 #include <stdlib.h>
+#include <type_traits>
 
 #include "common.h"
 #include "vla_kernels.h"
@@ -386,24 +387,27 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
         wp[0] = (const unsigned char*)((const uint32_t*)a.W + tern_word_index(n, (tid & 3) * 2, a.K));
     }
     u32x4_t ra[DEPTH][VA], rw[DEPTH][VW];
-    auto load_tile = [&](int st, int kt) __attribute__((always_inline)) {
+    // Load vector i of tile kt into ring stage st; i runs over the VA vectors of A and then
+    // the VW vectors of W (the ternary staging has a single W entry of two words).
+    constexpr int NLOAD = VA + ((kEpi != EPI_TERNARY) ? VW : 1);
+    auto load_vec = [&](int st, int kt, int i) __attribute__((always_inline)) {
         const int k0 = kt * BK;
-#pragma unroll
-        for (int v = 0; v < VA; ++v) {
-            const int k = min(k0 + a_koff[v], a.K - EPV);
-            ra[st][v] = *reinterpret_cast<const u32x4_t*>(ap[v] + (long)k * EB);
-        }
-        if (kEpi != EPI_TERNARY) {
-#pragma unroll
-            for (int v = 0; v < VW; ++v) {
-                const int k = min(k0 + a_koff[v % VA], a.K - EPV);  // same column pattern as A (VPR | 256)
-                rw[st][v] = *reinterpret_cast<const u32x4_t*>(wp[v] + (long)k * EB);
-            }
+        if (i < VA) {
+            const int k = min(k0 + a_koff[i], a.K - EPV);
+            ra[st][i] = *reinterpret_cast<const u32x4_t*>(ap[i] + (long)k * EB);
+        } else if (kEpi != EPI_TERNARY) {
+            const int v = i - VA;
+            const int k = min(k0 + a_koff[v % VA], a.K - EPV);  // same column pattern as A (VPR | 256)
+            rw[st][v] = *reinterpret_cast<const u32x4_t*>(wp[v] + (long)k * EB);
         } else {
             const uint32_t* w = (const uint32_t*)wp[0] + (long)(k0 / 32) * 64;
             rw[st][0][0] = w[0];
             rw[st][0][1] = w[32];
         }
+    };
+    auto load_tile = [&](int st, int kt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NLOAD; ++i) load_vec(st, kt, i);
     };
     auto mask_partial = [&](int st, int kt) __attribute__((always_inline)) {  // zero what lies past K
 #pragma unroll
@@ -452,21 +456,39 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
             }
         }
     };
-    auto multiply = [&](int buf) __attribute__((always_inline)) {
+    // Multiplies the tile in LDS buffer buf.  With LOAD set, the loads of tile kt_load into
+    // ring stage st_load are issued a few per k-chunk between the MFMA groups instead of in
+    // one burst: a burst keeps every wavefront of the workgroup waiting at the texture
+    // unit's queue before any of them starts on the LDS reads, so load issue and multiply
+    // would run one after the other instead of side by side.
+    auto multiply = [&](int buf, auto do_load, int st_load, int kt_load) __attribute__((always_inline)) {
+        constexpr bool LOAD = decltype(do_load)::value;
+        constexpr int NCH = KB / TR::kChunkBytes;
         const unsigned char* ldsA = lds + buf * BUF;
         const unsigned char* ldsW = ldsA + ROWS_A * STRIDE;
-#pragma unroll
-        for (int ch = 0; ch < KB / TR::kChunkBytes; ++ch) {
+        // operand fragments are read one k-chunk ahead of the MFMAs that use them, so the
+        // LDS latency of chunk ch + 1 passes under the MFMAs of chunk ch
+        u32x4_t fa[2][TM], fw[2][TN];
+        auto read_frags = [&](int slot, int ch) __attribute__((always_inline)) {
             const int off = ch * TR::kChunkBytes + g * 16;
-            u32x4_t fa[TM], fw[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const u32x4_t*>(ldsA + ((wm + 2 * i) * 32 + r) * STRIDE + off);
+            for (int i = 0; i < TM; ++i) fa[slot][i] = *reinterpret_cast<const u32x4_t*>(ldsA + ((wm + 2 * i) * 32 + r) * STRIDE + off);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fw[j] = *reinterpret_cast<const u32x4_t*>(ldsW + ((wn + 2 * j) * 32 + r) * STRIDE + off);
+            for (int j = 0; j < TN; ++j) fw[slot][j] = *reinterpret_cast<const u32x4_t*>(ldsW + ((wn + 2 * j) * 32 + r) * STRIDE + off);
+        };
+        read_frags(0, 0);
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) {
+            if (ch + 1 < NCH) read_frags((ch + 1) & 1, ch + 1);
+            if (LOAD) {
+#pragma unroll
+                for (int i = ch * NLOAD / NCH; i < (ch + 1) * NLOAD / NCH; ++i) load_vec(st_load, kt_load, i);
+            }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
-                for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[i], fw[j]);
+                for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[ch & 1][i], fw[ch & 1][j]);
+            __builtin_amdgcn_sched_barrier(0);  // keeps the reads and loads where they were placed
         }
     };
 
@@ -485,9 +507,8 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
 #pragma unroll
         for (int st = 0; st < DEPTH; ++st) {
             const int kt = gi * DEPTH + st;
-            load_tile(st, min(kt + DEPTH, nkt - 1));  // stage st held tile kt, already in LDS
-            __builtin_amdgcn_sched_barrier(0);        // the loads stay above the multiply they hide behind
-            multiply(kt & 1);
+            // stage st held tile kt, already in LDS: refill it with tile kt + DEPTH
+            multiply(kt & 1, std::true_type{}, st, min(kt + DEPTH, nkt - 1));
             if ((kt + 2) * BK > a.K) mask_partial((st + 1) % DEPTH, kt + 1);  // uniform; only the last tile can be partial
             store_tile((st + 1) % DEPTH, (kt + 1) & 1);  // past the last tile: a repeat of it, never read
             __syncthreads();
@@ -497,7 +518,7 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     for (int st = 0; st < DEPTH; ++st) {
         const int kt = n_main * DEPTH + st;
         if (kt < nkt) {  // uniform
-            multiply(kt & 1);
+            multiply(kt & 1, std::false_type{}, 0, 0);
             if (kt + 1 < nkt) {
                 if ((kt + 2) * BK > a.K) mask_partial((st + 1) % DEPTH, kt + 1);
                 store_tile((st + 1) % DEPTH, (kt + 1) & 1);
