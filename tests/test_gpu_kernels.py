@@ -160,6 +160,36 @@ def test_linear_bias_residual(dtype, M, N, K):
         assert bf16_close(as_f32(y, dtype), want)
 
 
+@pytest.mark.parametrize("M,N,K", [(150, 720, 720), (333, 200, 1104), (64, 1600, 48)])
+def test_linear_bf16_every_kernel_and_tiling_gives_the_same_bits(monkeypatch, M, N, K):
+    """The direct-to-LDS kernel and the register-staged one, in every tile configuration, add
+    the products of a row in the same order (ascending k, 16 at a time): identical outputs,
+    including partial k-tiles (K not a multiple of 64 or 128) and ragged M and N."""
+    r = np.random.default_rng(1040 + M)
+    x = orc.round_bf16(r.standard_normal((M, K)).astype(np.float32))
+    W = orc.round_bf16((0.05 * r.standard_normal((N, K))).astype(np.float32))
+    res = orc.round_bf16(r.standard_normal((M, N)).astype(np.float32))
+    xd, Wd, rd = to_dev(x, BF16), to_dev(W, BF16), to_dev(res, BF16)
+    outs = {}
+    for dl in ("0", "1"):
+        for tile in ("0", "1", "2", "3", "4"):
+            monkeypatch.setenv("VLA_GEMM_DL", dl)
+            monkeypatch.setenv("VLA_GEMM_TILE", tile)
+            y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+            pkg.call("vla_linear", xd, Wd, None, None, y, BF16, F32, M, N, K)
+            yb = empty((M, N), BF16)
+            pkg.call("vla_linear", xd, Wd, None, rd, yb, BF16, BF16, M, N, K)
+            sync()
+            outs[(dl, tile)] = (host(y), host(yb))
+    want = orc.linear(x, W)
+    first = outs[("0", "0")]
+    assert rel_err(first[0], want) < 1e-5
+    assert bf16_close(orc.from_bf16(first[1].view(np.uint16)), want + res)
+    for key, (y, yb) in outs.items():
+        assert np.array_equal(y, first[0]), key
+        assert np.array_equal(yb.view(np.uint16), first[1].view(np.uint16)), key
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("name,B,S,Hq,Hkv,D,K,rope,bias,P", [
     ("smolvla-self", 2, 50, 15, 5, 64, 720, True, False, 241),

@@ -545,6 +545,176 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
         }
 }
 
+// ---- bf16 GEMM with operand tiles loaded straight into LDS --------------------------
+// s_waitcnt on the vector-memory counter alone (vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits
+// 15:14; the export and LDS/scalar counter fields at their maxima, i.e. not waited on).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+// One 16-byte load per lane from global memory straight into LDS, no register in between:
+// lane i's bytes land at lds_base + 16 i (lds_base wavefront-uniform, held in M0); the
+// per-lane global address is free.  Completion is tracked by vmcnt like any vector load.
+// Issued from inline assembly so that the wait counts stay under this file's control.
+__device__ __forceinline__ void load_to_lds16(const void* gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
+}
+
+// Same tiling, wavefront layout, XCD mapping and epilogues as gemm_kernel, for bf16
+// operands with K a multiple of 16.  A stage of the LDS ring holds one k-tile of A and W
+// rows, KB bytes per row and no padding: a load instruction of a wavefront fills 1 KiB of
+// consecutive LDS (1024 / KB rows).  Bank conflicts of the fragment reads are avoided by a
+// swizzle instead of padding: the 16-byte piece c of row `row` is kept at piece position
+// c ^ swz(row), swz = (row >> 1) & 7 for 128-byte rows and row & 15 for 256-byte rows (16
+// consecutive fragment rows then cover all 64 banks exactly once); the loading lane picks
+// the global piece that belongs in its LDS slot.  NS - 1 tiles of loads are in flight; a
+// k-tile costs one barrier, and no wavefront spends issue slots on LDS stores.
+template <int kEpi, int TM, int TN, int KB, int NS>
+__global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
+    typedef bf16_t T;
+    typedef Traits<bf16_t> TR;
+    constexpr int EB = 2, BK = KB / EB, EPV = 8;
+    constexpr int ROWS_A = 64 * TM, ROWS_W = 64 * TN;
+    constexpr int VPR = KB / 16;        // 16-byte pieces per row
+    constexpr int RPS = 256 / VPR;      // rows filled by one load per thread of the workgroup
+    constexpr int VA = ROWS_A / RPS, VW = ROWS_W / RPS, NLOAD = VA + VW;
+    constexpr int NCH = KB / 32;        // 16-k MFMA chunks per tile
+    constexpr int STAGE = (ROWS_A + ROWS_W) * KB;
+    constexpr int C_BYTES = 4 * 64 * C_STRIDE;
+    constexpr int LDS_BYTES = NS * STAGE > C_BYTES ? NS * STAGE : C_BYTES;
+    constexpr int IN_FLIGHT = (NS - 2) * NLOAD;  // loads younger than the tile about to be multiplied
+    static_assert(KB == 128 || KB == 256, "swizzle is defined for 128- and 256-byte rows");
+    static_assert(NS >= 2 && IN_FLIGHT <= 63, "ring depth exceeds the vector-memory counter");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int g = lane >> 5, r = lane & 31;
+    const int n_wg_tiles = (a.n_tiles + TN - 1) / TN, m_wg_tiles = (a.M + ROWS_A - 1) / ROWS_A;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int cn = (n_wg_tiles + a.xn - 1) / a.xn;
+    const int ntw = (local % cn) * a.xn + xcd % a.xn;
+    const int mtw = (local / cn) * a.xm + xcd / a.xn;
+    if (ntw >= n_wg_tiles || mtw >= m_wg_tiles) return;
+    const int m0 = mtw * ROWS_A;
+    TileCols tc[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) tc[j] = tile_cols<kEpi>(a, ntw * TN + j);
+
+    typename TR::Acc acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+    const int nkt = (a.K + BK - 1) / BK, nkt_full = a.K / BK;
+
+    // Loader side.  Thread tid fills LDS slot tid of each 256-slot slab; slab v of A holds
+    // rows v*RPS .. v*RPS+RPS-1.  The slot is piece position tid % VPR of row tid / VPR, so
+    // the lane fetches the logical piece (tid % VPR) ^ swz(row); swz only involves the low
+    // row bits, which do not depend on the slab.  Rows past M or N and k past K are
+    // redirected to valid addresses: their products land in outputs that are dropped, and
+    // k-chunks past K are never multiplied.
+    const int lrow = tid / VPR;
+    const int lsw = (KB == 128) ? ((lrow >> 1) & 7) : (lrow & 15);
+    const int koff = ((tid % VPR) ^ lsw) * EPV;
+    const unsigned char* ap[VA];
+#pragma unroll
+    for (int v = 0; v < VA; ++v) ap[v] = (const unsigned char*)a.A + (long)min(m0 + v * RPS + lrow, a.M - 1) * a.K * EB;
+    const unsigned char* wp[VW];
+#pragma unroll
+    for (int v = 0; v < VW; ++v) {
+        const int sub = (v * RPS) / 64, wr = (v * RPS + lrow) & 63;  // sub is compile-time per unrolled v
+        int n = (wr < 32) ? tc[sub].base0 + wr : tc[sub].base1 + wr - 32;
+        n = min(max(n, 0), a.N - 1);
+        wp[v] = (const unsigned char*)a.W + (long)n * a.K * EB;
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds + wave * 1024;  // low 32 bits of a shared-aperture address = LDS offset
+    auto issue = [&](int i, int kt, int stage) __attribute__((always_inline)) {
+        const long kb = (long)min(kt * BK + koff, a.K - EPV) * EB;
+        if (i < VA) load_to_lds16(ap[i] + kb, lds0 + stage * STAGE + i * 4096);
+        else load_to_lds16(wp[i - VA] + kb, lds0 + stage * STAGE + ROWS_A * KB + (i - VA) * 4096);
+    };
+
+    // Consumer side.  Fragment row r of any 32-row block has swz = (r >> 1) & 7 (or r & 15);
+    // the lane wants logical piece 2 ch + g, i.e. position (2 ch) ^ (g ^ swz).
+    const int fsw = (KB == 128) ? ((r >> 1) & 7) : (r & 15);
+    const int xo = (g ^ fsw) * 16;
+    const int fragA = (wm * 32 + r) * KB, fragW = ROWS_A * KB + (wn * 32 + r) * KB;
+    auto multiply = [&](int stage, auto do_load, int st_load, int kt_load, int n_chunks) __attribute__((always_inline)) {
+        constexpr bool LOAD = decltype(do_load)::value;
+        const unsigned char* base = lds + stage * STAGE;
+        u32x4_t fa[2][TM], fw[2][TN];
+        auto read_frags = [&](int slot, int ch) __attribute__((always_inline)) {
+            const int off = (ch * 32) ^ xo;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[slot][i] = *reinterpret_cast<const u32x4_t*>(base + fragA + i * 64 * KB + off);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fw[slot][j] = *reinterpret_cast<const u32x4_t*>(base + fragW + j * 64 * KB + off);
+        };
+        read_frags(0, 0);
+#pragma unroll
+        for (int ch = 0; ch < NCH; ++ch) {
+            if (ch + 1 < NCH) read_frags((ch + 1) & 1, ch + 1);
+            if (LOAD) {
+#pragma unroll
+                for (int i = ch * NLOAD / NCH; i < (ch + 1) * NLOAD / NCH; ++i) issue(i, kt_load, st_load);
+            }
+            if (LOAD || ch < n_chunks) {  // uniform; only the partial last tile has fewer chunks
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[ch & 1][i], fw[ch & 1][j]);
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keeps the reads and loads where they were placed
+        }
+    };
+
+    // Stage kt % NS holds tile kt.  Before tile kt is multiplied every wavefront waits for
+    // its own loads of that tile (the IN_FLIGHT younger ones may still be pending) and all
+    // meet at the barrier, which also tells that stage (kt - 1) % NS has been read by
+    // everyone: the loads of tile kt + NS - 1 go there.  Past the last tile the ring keeps
+    // re-fetching it into free stages, so the counts stay the same to the end.
+#pragma unroll
+    for (int t = 0; t < NS - 1; ++t)
+#pragma unroll
+        for (int i = 0; i < NLOAD; ++i) issue(i, min(t, nkt - 1), t);
+    int cs = 0, ls = NS - 1;
+    for (int kt = 0; kt < nkt_full; ++kt) {
+        wait_vmcnt<IN_FLIGHT>();
+        __syncthreads();
+        multiply(cs, std::true_type{}, ls, min(kt + NS - 1, nkt - 1), NCH);
+        cs = (cs + 1 == NS) ? 0 : cs + 1;
+        ls = (ls + 1 == NS) ? 0 : ls + 1;
+    }
+    if (nkt > nkt_full) {
+        wait_vmcnt<IN_FLIGHT>();
+        __syncthreads();
+        multiply(cs, std::false_type{}, 0, 0, (a.K - nkt_full * BK) / 16);
+    }
+    wait_vmcnt<0>();  // the re-fetches must have landed before the ring is reused for C
+    __syncthreads();
+
+    uint32_t* C = reinterpret_cast<uint32_t*>(lds);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            if (i + j > 0) __syncthreads();
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj)
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii)
+                    C[(wm * 32 + 8 * jj + 4 * g + ii) * C_STRIDE + wn * 32 + r] = acc_bits(acc[i][j][4 * jj + ii]);
+            __syncthreads();
+            const int nt_sub = ntw * TN + j;
+            if (nt_sub < a.n_tiles) epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid);
+        }
+}
+
 // Large-M ternary GEMM (BitVLA prefill: M = batch x prefix tokens).  Workgroup tile
 // (64*WM) x 256 with WM x 2 wavefronts, each owning 64 x 128 = 2 x 4 MFMA blocks (128
 // accumulator registers), so one 16-byte A fragment feeds four MFMAs and one weight
@@ -830,12 +1000,11 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_kernel(GemmArgs 
     }
 }
 
-template <typename T, int kEpi, int TM, int TN, int KB, int DEPTH>
-void launch_cfg(GemmArgs a, hipStream_t st) {
-    const int n_wg = (a.n_tiles + TN - 1) / TN, m_wg = (a.M + 64 * TM - 1) / (64 * TM);
-    // XCD grid xm x xn = 8: every L2 reads its M tiles' rows of A and its N tiles' rows of
-    // W once; pick the split with the least total, counting the padding of the tile grid.
-    const double bytes_a = (double)a.M * a.K, bytes_w = (double)a.N * a.K * (kEpi == EPI_TERNARY ? 0.25 : 1.0);
+// XCD grid xm x xn = 8 for a tile grid of m_wg x n_wg workgroup tiles: every L2 reads its M
+// tiles' rows of A and its N tiles' rows of W once; the split with the least total,
+// counting the padding of the tile grid.  Returns the grid size.
+unsigned xcd_split(GemmArgs& a, int m_wg, int n_wg, double w_bytes_per_elem) {
+    const double bytes_a = (double)a.M * a.K, bytes_w = (double)a.N * a.K * w_bytes_per_elem;
     double best = -1;
     for (int xm = 1; xm <= 8; xm *= 2) {
         const int xn = 8 / xm;
@@ -847,8 +1016,19 @@ void launch_cfg(GemmArgs a, hipStream_t st) {
             a.xn = xn;
         }
     }
-    const unsigned grid = (unsigned)(((m_wg + a.xm - 1) / a.xm) * ((n_wg + a.xn - 1) / a.xn) * 8);
+    return (unsigned)(((m_wg + a.xm - 1) / a.xm) * ((n_wg + a.xn - 1) / a.xn) * 8);
+}
+
+template <typename T, int kEpi, int TM, int TN, int KB, int DEPTH>
+void launch_cfg(GemmArgs a, hipStream_t st) {
+    const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, kEpi == EPI_TERNARY ? 0.25 : 1.0);
     gemm_kernel<T, kEpi, TM, TN, KB, DEPTH><<<grid, 256, 0, st>>>(a);
+}
+
+template <int kEpi, int TM, int TN, int KB, int NS>
+void launch_dl(GemmArgs a, hipStream_t st) {
+    const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, 1.0);
+    gemm_dl_kernel<kEpi, TM, TN, KB, NS><<<grid, 256, 0, st>>>(a);
 }
 
 template <typename T, int kEpi>
@@ -866,6 +1046,23 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             // 256-byte K rows (half the barriers per K).
             const long m128 = (a.M + 127) / 128;
             cfg = m128 * ((n_tiles + 1) / 2) >= 128 ? 0 : (m128 * n_tiles >= 150 ? 2 : 1);
+        }
+        // bf16 operands with 16-byte aligned rows and K a multiple of the MFMA depth take the
+        // direct-to-LDS kernel (VLA_GEMM_DL=0 pins the register-staged one).
+        bool dl = false;
+        if constexpr (std::is_same<T, bf16_t>::value) {
+            const char* e = getenv("VLA_GEMM_DL");
+            dl = !(e && atoi(e) == 0) && a.K % 16 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
+        }
+        if (dl) {
+            switch (cfg) {
+                case 0: launch_dl<kEpi, 2, 2, 128, 3>(a, st); break;
+                case 1: launch_dl<kEpi, 1, 1, 256, 4>(a, st); break;
+                case 2: launch_dl<kEpi, 2, 1, 128, 4>(a, st); break;
+                case 3: launch_dl<kEpi, 1, 2, 128, 4>(a, st); break;
+                default: launch_dl<kEpi, 1, 1, 128, 6>(a, st); break;
+            }
+            return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
         }
         switch (cfg) {
             case 0: launch_cfg<T, kEpi, 2, 2, 128, 3>(a, st); break;
