@@ -171,18 +171,19 @@ def test_linear_bf16_every_kernel_and_tiling_gives_the_same_bits(monkeypatch, M,
     res = orc.round_bf16(r.standard_normal((M, N)).astype(np.float32))
     xd, Wd, rd = to_dev(x, BF16), to_dev(W, BF16), to_dev(res, BF16)
     outs = {}
-    for dl in ("0", "1"):
-        for tile in ("0", "1", "2", "3", "4"):
+    for dl, tile, stages in [("0", t, "0") for t in "01234"] + [("1", t, ns) for t in "01234" for ns in "234"]:
+        if True:
             monkeypatch.setenv("VLA_GEMM_DL", dl)
             monkeypatch.setenv("VLA_GEMM_TILE", tile)
+            monkeypatch.setenv("VLA_GEMM_STAGES", stages)
             y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
             pkg.call("vla_linear", xd, Wd, None, None, y, BF16, F32, M, N, K)
             yb = empty((M, N), BF16)
             pkg.call("vla_linear", xd, Wd, None, rd, yb, BF16, BF16, M, N, K)
             sync()
-            outs[(dl, tile)] = (host(y), host(yb))
+            outs[(dl, tile, stages)] = (host(y), host(yb))
     want = orc.linear(x, W)
-    first = outs[("0", "0")]
+    first = outs[("0", "0", "0")]
     assert rel_err(first[0], want) < 1e-5
     assert bf16_close(orc.from_bf16(first[1].view(np.uint16)), want + res)
     for key, (y, yb) in outs.items():

@@ -157,7 +157,8 @@ __device__ __forceinline__ TileCols tile_cols(const GemmArgs& a, int nt) {
 // columns jg..jg+7 and 32+jg..32+jg+7 of the sub-tile.
 template <typename T, int kEpi>
 __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t* C, int m0, int nt, const TileCols& tc,
-                                               int tid) {
+                                               int tid, bool have_res = false, u32x4_t res_lo = u32x4_t{0u, 0u, 0u, 0u},
+                                               u32x4_t res_hi = u32x4_t{0u, 0u, 0u, 0u}) {
     const int erow = tid >> 2, jg = (tid & 3) * 8;
     const int m = m0 + erow;
     if (m >= a.M) return;
@@ -206,7 +207,9 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
             }
             if (full && a.out_bf16) {  // 8 consecutive bf16 = one 16-byte access each way
                 if (a.residual) {
-                    const u32x4_t rr = *reinterpret_cast<const u32x4_t*>((const bf16_t*)a.residual + o);
+                    // res_lo / res_hi: this thread's two residual vectors when fetched before the k loop
+                    u32x4_t rr = hlf ? res_hi : res_lo;
+                    if (!have_res) rr = *reinterpret_cast<const u32x4_t*>((const bf16_t*)a.residual + o);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         v[2 * e] += __uint_as_float(rr[e] << 16);
@@ -612,6 +615,24 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
 
     const int nkt = (a.K + BK - 1) / BK, nkt_full = a.K / BK;
 
+    // A bf16 residual is fetched now, ahead of every operand load, instead of in the
+    // epilogue where nothing is left to hide its latency (the epilogue thread layout:
+    // row tid / 4, columns 8 (tid % 4) .. +7 of each 32-column half of a 64x64 sub-tile).
+    u32x4_t res_pf[TM][TN][2] = {};
+    const bool pf = kEpi == EPI_PLAIN && a.residual != nullptr && a.out_bf16 && a.N % 8 == 0;
+    if (pf) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int hlf = 0; hlf < 2; ++hlf) {
+                    const int m = min(m0 + i * 64 + (tid >> 2), a.M - 1);
+                    const int n0 = min((ntw * TN + j) * BN + hlf * 32 + (tid & 3) * 8, a.N - 8);
+                    res_pf[i][j][hlf] = *reinterpret_cast<const u32x4_t*>((const bf16_t*)a.residual + (long)m * a.N + n0);
+                }
+    }
+
     // Loader side.  Thread tid fills LDS slot tid of each 256-slot slab; slab v of A holds
     // rows v*RPS .. v*RPS+RPS-1.  The slot is piece position tid % VPR of row tid / VPR, so
     // the lane fetches the logical piece (tid % VPR) ^ swz(row); swz only involves the low
@@ -711,7 +732,7 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
                     C[(wm * 32 + 8 * jj + 4 * g + ii) * C_STRIDE + wn * 32 + r] = acc_bits(acc[i][j][4 * jj + ii]);
             __syncthreads();
             const int nt_sub = ntw * TN + j;
-            if (nt_sub < a.n_tiles) epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid);
+            if (nt_sub < a.n_tiles) epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0], res_pf[i][j][1]);
         }
 }
 
@@ -1037,30 +1058,59 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
     a.n_tiles = n_tiles;
     hipStream_t st = (hipStream_t)stream;
     if constexpr (kEpi != EPI_TERNARY) {
-        // VLA_GEMM_TILE = 0..4 pins the tile configuration (tuning); unset = by shape.
+        // VLA_GEMM_TILE = 0..4 pins the tile configuration and VLA_GEMM_STAGES the ring depth
+        // of the direct-to-LDS kernel (tests and tuning); unset = by shape.
         const char* env = getenv("VLA_GEMM_TILE");
         int cfg = env ? atoi(env) : -1;
+        const long m128 = (a.M + 127) / 128, m64 = (a.M + 63) / 64;
+        const long wgs0 = m128 * ((n_tiles + 1) / 2), wgs2 = m128 * n_tiles, wgs4 = m64 * n_tiles;
         if (cfg < 0) {
             // Enough 128x128 tiles to occupy the chip: use them (half the LDS and L2 traffic
-            // per multiply); else 128x64 tiles if those fill it; else 64x64 tiles with
-            // 256-byte K rows (half the barriers per K).
-            const long m128 = (a.M + 127) / 128;
-            cfg = m128 * ((n_tiles + 1) / 2) >= 128 ? 0 : (m128 * n_tiles >= 150 ? 2 : 1);
+            // per multiply); else 128x64 tiles if those fill it; else 64x64 tiles, with
+            // 256-byte K rows (half the barriers per K) while one workgroup per CU covers them.
+            cfg = wgs0 >= 128 ? 0 : (wgs2 >= 150 ? 2 : (wgs4 <= 256 ? 1 : 4));
         }
         // bf16 operands with 16-byte aligned rows and K a multiple of the MFMA depth take the
-        // direct-to-LDS kernel (VLA_GEMM_DL=0 pins the register-staged one).
+        // direct-to-LDS kernel (VLA_GEMM_DL=0 pins the register-staged one).  Its ring depth
+        // trades loads in flight against LDS per workgroup: a workgroup is short-lived, so
+        // what matters first is that the whole grid is resident at once (160 KiB of LDS per
+        // CU, 256 CUs), and only then how far ahead each workgroup fetches.
         bool dl = false;
         if constexpr (std::is_same<T, bf16_t>::value) {
             const char* e = getenv("VLA_GEMM_DL");
             dl = !(e && atoi(e) == 0) && a.K % 16 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
         }
         if (dl) {
+            const char* es = getenv("VLA_GEMM_STAGES");
+            int ns = es ? atoi(es) : 0;
+            const long wgs = cfg == 0 ? wgs0 : (cfg == 2 || cfg == 3 ? wgs2 : wgs4);
             switch (cfg) {
-                case 0: launch_dl<kEpi, 2, 2, 128, 3>(a, st); break;
-                case 1: launch_dl<kEpi, 1, 1, 256, 4>(a, st); break;
-                case 2: launch_dl<kEpi, 2, 1, 128, 4>(a, st); break;
-                case 3: launch_dl<kEpi, 1, 2, 128, 4>(a, st); break;
-                default: launch_dl<kEpi, 1, 1, 128, 6>(a, st); break;
+                case 0:  // 32 KiB per stage
+                    if (ns == 0) ns = wgs <= 256 ? 3 : 2;
+                    if (ns <= 2) launch_dl<kEpi, 2, 2, 128, 2>(a, st);
+                    else launch_dl<kEpi, 2, 2, 128, 3>(a, st);
+                    break;
+                case 1:  // 32 KiB per stage
+                    if (ns == 0) ns = 4;
+                    if (ns <= 3) launch_dl<kEpi, 1, 1, 256, 3>(a, st);
+                    else launch_dl<kEpi, 1, 1, 256, 4>(a, st);
+                    break;
+                case 2:  // 24 KiB per stage
+                    if (ns == 0) ns = wgs <= 256 ? 4 : (wgs <= 512 ? 3 : 2);
+                    if (ns <= 2) launch_dl<kEpi, 2, 1, 128, 2>(a, st);
+                    else if (ns == 3) launch_dl<kEpi, 2, 1, 128, 3>(a, st);
+                    else launch_dl<kEpi, 2, 1, 128, 4>(a, st);
+                    break;
+                case 3:  // 24 KiB per stage
+                    if (ns == 0) ns = wgs <= 256 ? 4 : 3;
+                    if (ns <= 3) launch_dl<kEpi, 1, 2, 128, 3>(a, st);
+                    else launch_dl<kEpi, 1, 2, 128, 4>(a, st);
+                    break;
+                default:  // 16 KiB per stage
+                    if (ns == 0) ns = wgs <= 512 ? 4 : 3;
+                    if (ns <= 3) launch_dl<kEpi, 1, 1, 128, 3>(a, st);
+                    else launch_dl<kEpi, 1, 1, 128, 4>(a, st);
+                    break;
             }
             return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
         }
