@@ -125,6 +125,24 @@ VLA_KAPI int vla_attn_qkv_rope(const void* x, const void* W, const float* bias, 
                                const float* cos_tab, const float* sin_tab, void* q_out, void* k_cache,
                                void* vt_cache, int t_max, int tok_offset, vla_stream_t stream);
 
+/* The same launch with the layer's RMSNorm taken inside it: replaces build_norm ->
+ * mm_w(Wq/Wk/Wv) -> rope -> concat (src/models/smolvla.cpp:815-833,
+ * src/models/pi0.cpp:170-201).  x is the un-normalised residual stream; row m of
+ * the projection is scaled by rsqrt(mean_k x[m][k]^2 + rms_eps) before bias and
+ * rotation, and the norm weight is expected inside W_folded
+ * (W_folded[n][k] = W[n][k] * g[k], vla_fold_norm_weight_host).  bf16 only, K a
+ * multiple of 16 and 16-byte aligned operands; VLA_K_ERR_SHAPE otherwise (use
+ * vla_rms_norm + vla_attn_qkv_rope then). */
+VLA_KAPI int vla_rmsnorm_attn_qkv_rope(const void* x, const void* W_folded, const float* bias, int dtype, int M, int K,
+                                       int S, int n_q_heads, int n_kv_heads, int has_k, int has_v, int head_dim,
+                                       const float* cos_tab, const float* sin_tab, void* q_out, void* k_cache,
+                                       void* vt_cache, int t_max, int tok_offset, float rms_eps, vla_stream_t stream);
+
+/* Host helper for the call above: W_out[n][k] = W[n][k] * g[k] in `dtype` (bf16
+ * products rounded to nearest even; g is the RMSNorm weight ggml_mul applies after
+ * ggml_rms_norm, src/layers/norm.h:31-34).  W_out may alias W. */
+VLA_KAPI int vla_fold_norm_weight_host(const void* W, const void* g, int dtype, int N, int K, void* W_out);
+
 /* Unfused tail of the same step for a projection that already exists as a
  * [M][(n_q_heads + 2 n_kv_heads) * D] matrix (the BitVLA ternary GEMM output,
  * src/kernels/bitvla/bitvla_lm_cuda.cu:428-446: transposes, RoPE on Q and K,

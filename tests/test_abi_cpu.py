@@ -71,6 +71,22 @@ def test_ternary_quant_and_packers_against_oracle():
     assert lib.vla_ternary_repack_ladder_host(raw.ctypes.data, 24, K, rep.ctypes.data) == pkg.VLA_K_ERR_SHAPE
 
 
+def test_fold_norm_weight_host_rounds_products_to_nearest_even():
+    lib = pkg.lib()
+    r = np.random.default_rng(7)
+    N, K = 37, 48
+    W = orc.round_bf16(r.standard_normal((N, K)).astype(np.float32))
+    g = orc.round_bf16((1 + 0.5 * r.standard_normal(K)).astype(np.float32))
+    out = np.empty((N, K), np.uint16)
+    assert lib.vla_fold_norm_weight_host(orc.to_bf16(W).ctypes.data, orc.to_bf16(g).ctypes.data, pkg.VLA_DT_BF16, N, K,
+                                         out.ctypes.data) == pkg.VLA_K_OK
+    assert np.array_equal(out, orc.to_bf16(W * g[None, :]))  # products of bf16 values are exact in fp32: one rounding
+    out32 = np.empty((N, K), np.float32)
+    assert lib.vla_fold_norm_weight_host(W.ctypes.data, g.ctypes.data, pkg.VLA_DT_F32, N, K, out32.ctypes.data) == pkg.VLA_K_OK
+    assert np.array_equal(out32, W * g[None, :])
+    assert lib.vla_fold_norm_weight_host(None, g.ctypes.data, pkg.VLA_DT_F32, N, K, out32.ctypes.data) == pkg.VLA_K_ERR_ARG
+
+
 def test_null_and_shape_errors_are_reported_not_fatal():
     lib = pkg.lib()
     assert lib.vla_kv_append(None, None, None, None, 0, 1, 0, 64, 64, 0, 1, None) == pkg.VLA_K_ERR_ARG

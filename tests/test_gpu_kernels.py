@@ -234,6 +234,61 @@ def test_fused_qkv_rope_append(dtype, name, B, S, Hq, Hkv, D, K, rope, bias, P):
     assert not host(kc)[:, :, :P].any() and not host(vc)[:, :, :, :P].any()
 
 
+@pytest.mark.parametrize("name,B,S,Hq,Hkv,D,K,self_layer,P", [
+    ("smolvla-self", 2, 50, 15, 5, 64, 720, True, 241),
+    ("smolvla-cross-q", 3, 50, 15, 5, 64, 720, False, 0),
+    ("pi0", 1, 51, 8, 1, 256, 1024, True, 816),
+    ("one-partial-k-tile", 1, 5, 2, 1, 64, 48, True, 3),
+])
+def test_rmsnorm_inside_qkv_launch(name, B, S, Hq, Hkv, D, K, self_layer, P):
+    """Pre-norm taken inside the projection launch (norm weight folded into W on the host,
+    rows scaled by rsqrt(mean square + eps) in the epilogue) against the oracle's
+    rms_norm -> linear -> rope, and against the two-launch GPU path."""
+    r = np.random.default_rng(1105 + K)
+    M = B * S
+    nkv = Hkv if self_layer else 0
+    N = (Hq + 2 * nkv) * D
+    eps = 1e-5
+    x = orc.round_bf16((3.0 * r.standard_normal((M, K)) * (1.0 + r.random((M, 1)) * 4)).astype(np.float32))
+    g = orc.round_bf16((1.0 + 0.3 * r.standard_normal(K)).astype(np.float32))
+    W = orc.round_bf16((0.02 * r.standard_normal((N, K))).astype(np.float32))
+    c, s_ = orc.rope_tables(np.arange(S, dtype=np.int32) + P + 1, D, 10000.0)
+    t_max = (P + S + 63) // 64 * 64
+
+    def run(fused):
+        kc, vc = empty((B, Hkv, t_max, D), BF16), empty((B, Hkv, D, t_max), BF16)
+        q = empty((M, Hq * D), BF16)
+        if fused:
+            Wf = np.empty((N, K), np.uint16)
+            assert pkg.lib().vla_fold_norm_weight_host(orc.to_bf16(W).ctypes.data, orc.to_bf16(g).ctypes.data, BF16, N, K,
+                                                       Wf.ctypes.data) == 0
+            pkg.call("vla_rmsnorm_attn_qkv_rope", to_dev(x, BF16), dev(Wf), None, BF16, M, K, S, Hq, Hkv, int(self_layer),
+                     int(self_layer), D, dev(c), dev(s_), q, kc, vc, t_max, P, eps)
+        else:
+            hn = empty((M, K), BF16)
+            pkg.call("vla_rms_norm", to_dev(x, BF16), to_dev(g, BF16), hn, BF16, M, K, eps)
+            pkg.call("vla_attn_qkv_rope", hn, to_dev(W, BF16), None, BF16, M, K, S, Hq, Hkv, int(self_layer),
+                     int(self_layer), D, dev(c), dev(s_), q, kc, vc, t_max, P)
+        out = [as_f32(q, BF16).reshape(M, Hq, D)]
+        if self_layer:
+            kd, vd = empty((B, S, Hkv, D), BF16), empty((B, S, Hkv, D), BF16)
+            pkg.call("vla_kv_gather", kc, vc, kd, vd, BF16, B, Hkv, D, t_max, P, S)
+            out += [as_f32(kd, BF16).reshape(M, Hkv, D), as_f32(vd, BF16).reshape(M, Hkv, D)]
+        sync()
+        return out
+
+    y = orc.linear(orc.rms_norm(x, g, eps), W)
+    want = [y[:, :Hq * D].reshape(M, Hq, D)]
+    if self_layer:
+        want += [y[:, Hq * D:(Hq + Hkv) * D].reshape(M, Hkv, D), y[:, (Hq + Hkv) * D:].reshape(M, Hkv, D)]
+    for i in range(min(2, len(want))):  # Q and K are rotated, V is not
+        want[i] = np.concatenate([orc.rope_neox(want[i][b * S:(b + 1) * S], c, s_) for b in range(B)])
+    fused, pair = run(True), run(False)
+    for gf, gp, w in zip(fused, pair, want):
+        assert bf16_close(gf, w) and rel_err(gf, w) < 8e-3
+        assert rel_err(gf, gp) < 8e-3
+
+
 # ------------------------------------------------------------------ attention
 CASES = [
     # name, B, S, Hq, Hkv, D, P, mask kind, pad

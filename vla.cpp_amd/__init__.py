@@ -33,6 +33,8 @@ KERNEL_API = {
     "vla_adaln": [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _vp],
     "vla_linear": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "vla_attn_qkv_rope": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    "vla_rmsnorm_attn_qkv_rope": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp],
+    "vla_fold_norm_weight_host": [_vp, _vp, _i, _i, _i, _vp],
     "vla_qkv_split_rope_append": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "vla_attn_prefix_suffix": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp],
     "vla_embed_suffix": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],

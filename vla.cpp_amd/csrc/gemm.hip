@@ -24,6 +24,7 @@
 // (g, r), C[8j + 4g + i][r].
 
 #include <stdlib.h>
+#include <string.h>
 #include <type_traits>
 
 #include "common.h"
@@ -61,6 +62,8 @@ struct GemmArgs {
     const int32_t* rowsum;
     const float* ws;
     int ws_num;
+    // RMS statistics of the A rows taken inside the GEMM (direct-to-LDS kernel, kNorm)
+    float norm_eps;
 };
 
 template <typename T> struct Traits;
@@ -158,7 +161,8 @@ __device__ __forceinline__ TileCols tile_cols(const GemmArgs& a, int nt) {
 template <typename T, int kEpi>
 __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t* C, int m0, int nt, const TileCols& tc,
                                                int tid, bool have_res = false, u32x4_t res_lo = u32x4_t{0u, 0u, 0u, 0u},
-                                               u32x4_t res_hi = u32x4_t{0u, 0u, 0u, 0u}) {
+                                               u32x4_t res_hi = u32x4_t{0u, 0u, 0u, 0u}, bool scale_rows = false,
+                                               const float* row_scale = nullptr) {
     const int erow = tid >> 2, jg = (tid & 3) * 8;
     const int m = m0 + erow;
     if (m >= a.M) return;
@@ -190,6 +194,14 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
     for (int e = 0; e < 8; ++e) {
         lo[e] = __uint_as_float(crow[jg + e]);
         hi[e] = __uint_as_float(crow[32 + jg + e]);
+    }
+    if (scale_rows) {  // row_scale: one factor per row of the sub-tile (in LDS)
+        const float f = row_scale[erow];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            lo[e] *= f;
+            hi[e] *= f;
+        }
     }
 
     if (kEpi == EPI_PLAIN) {
@@ -548,6 +560,13 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
         }
 }
 
+// acc + lo^2 + hi^2 of the two bf16 values packed in u (taken by value: a bit_cast applied
+// directly to a vector element expression reads element 0).
+__device__ __forceinline__ float add_squares_bf16x2(uint32_t u, float acc) {
+    const bf16x2_t v = __builtin_bit_cast(bf16x2_t, u);
+    return __builtin_amdgcn_fdot2_f32_bf16(v, v, acc, false);
+}
+
 // ---- bf16 GEMM with operand tiles loaded straight into LDS --------------------------
 // s_waitcnt on the vector-memory counter alone (vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits
 // 15:14; the export and LDS/scalar counter fields at their maxima, i.e. not waited on).
@@ -573,7 +592,7 @@ __device__ __forceinline__ void load_to_lds16(const void* gptr, uint32_t lds_bas
 // consecutive fragment rows then cover all 64 banks exactly once); the loading lane picks
 // the global piece that belongs in its LDS slot.  NS - 1 tiles of loads are in flight; a
 // k-tile costs one barrier, and no wavefront spends issue slots on LDS stores.
-template <int kEpi, int TM, int TN, int KB, int NS>
+template <int kEpi, int TM, int TN, int KB, int NS, bool kNorm>
 __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     typedef bf16_t T;
     typedef Traits<bf16_t> TR;
@@ -585,7 +604,8 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     constexpr int NCH = KB / 32;        // 16-k MFMA chunks per tile
     constexpr int STAGE = (ROWS_A + ROWS_W) * KB;
     constexpr int C_BYTES = 4 * 64 * C_STRIDE;
-    constexpr int LDS_BYTES = NS * STAGE > C_BYTES ? NS * STAGE : C_BYTES;
+    constexpr int EPI_BYTES = C_BYTES + ROWS_A * 4;  // C sub-tile, then one scale per tile row (kNorm)
+    constexpr int LDS_BYTES = NS * STAGE > EPI_BYTES ? NS * STAGE : EPI_BYTES;
     constexpr int IN_FLIGHT = (NS - 2) * NLOAD;  // loads younger than the tile about to be multiplied
     static_assert(KB == 128 || KB == 256, "swizzle is defined for 128- and 256-byte rows");
     static_assert(NS >= 2 && IN_FLIGHT <= 63, "ring depth exceeds the vector-memory counter");
@@ -614,6 +634,13 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
     const int nkt = (a.K + BK - 1) / BK, nkt_full = a.K / BK;
+    // kNorm: the GEMM multiplies raw rows of A and scales row m of the result by
+    // rsqrt(mean_k A[m][k]^2 + eps); the squares are summed from the same LDS fragments
+    // the MFMAs read (lane (g, r) sees 8 of every 16 k of its rows; the two halves meet
+    // after the loop), two bf16 products per instruction.
+    float ssq[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) ssq[i] = 0.f;
 
     // A bf16 residual is fetched now, ahead of every operand load, instead of in the
     // epilogue where nothing is left to hide its latency (the epilogue thread layout:
@@ -689,6 +716,12 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[ch & 1][i], fw[ch & 1][j]);
+                if (kNorm) {
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) ssq[i] = add_squares_bf16x2(fa[ch & 1][i][e], ssq[i]);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);  // keeps the reads and loads where they were placed
         }
@@ -720,6 +753,15 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     __syncthreads();
 
     uint32_t* C = reinterpret_cast<uint32_t*>(lds);
+    float* row_scale = reinterpret_cast<float*>(lds + C_BYTES);
+    if (kNorm) {
+        const float inv_k = 1.0f / (float)a.K;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const float t = ssq[i] + __shfl_xor(ssq[i], 32, 64);
+            if (wn == 0 && g == 0) row_scale[(wm + 2 * i) * 32 + r] = rsqrtf(t * inv_k + a.norm_eps);
+        }
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -732,7 +774,9 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
                     C[(wm * 32 + 8 * jj + 4 * g + ii) * C_STRIDE + wn * 32 + r] = acc_bits(acc[i][j][4 * jj + ii]);
             __syncthreads();
             const int nt_sub = ntw * TN + j;
-            if (nt_sub < a.n_tiles) epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0], res_pf[i][j][1]);
+            if (nt_sub < a.n_tiles)
+                epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0], res_pf[i][j][1], kNorm,
+                                        row_scale + i * 64);
         }
 }
 
@@ -1049,7 +1093,13 @@ void launch_cfg(GemmArgs a, hipStream_t st) {
 template <int kEpi, int TM, int TN, int KB, int NS>
 void launch_dl(GemmArgs a, hipStream_t st) {
     const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, 1.0);
-    gemm_dl_kernel<kEpi, TM, TN, KB, NS><<<grid, 256, 0, st>>>(a);
+    if constexpr (kEpi == EPI_QKV) {
+        if (a.norm_eps >= 0.f) {
+            gemm_dl_kernel<kEpi, TM, TN, KB, NS, true><<<grid, 256, 0, st>>>(a);
+            return;
+        }
+    }
+    gemm_dl_kernel<kEpi, TM, TN, KB, NS, false><<<grid, 256, 0, st>>>(a);
 }
 
 template <typename T, int kEpi>
@@ -1080,6 +1130,7 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             const char* e = getenv("VLA_GEMM_DL");
             dl = !(e && atoi(e) == 0) && a.K % 16 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
         }
+        if (a.norm_eps >= 0.f && !(dl && kEpi == EPI_QKV)) return VLA_K_ERR_SHAPE;  // only that kernel takes the row statistics
         if (dl) {
             const char* es = getenv("VLA_GEMM_STAGES");
             int ns = es ? atoi(es) : 0;
@@ -1168,6 +1219,7 @@ int vla_linear(const void* x, const void* W, const float* bias, const void* resi
     if (!x || !W || !y || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
     if (out_dtype != VLA_DT_F32 && out_dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
     GemmArgs a = {};
+    a.norm_eps = -1.f;
     a.A = x; a.W = W; a.bias = bias; a.M = M; a.N = N; a.K = K;
     a.residual = residual; a.Y = y; a.out_bf16 = (out_dtype == VLA_DT_BF16);
     const int nt = (N + BN - 1) / BN;
@@ -1182,9 +1234,10 @@ int vla_linear(const void* x, const void* W, const float* bias, const void* resi
     return VLA_K_ERR_ARG;
 }
 
-int vla_attn_qkv_rope(const void* x, const void* W, const float* bias, int dtype, int M, int K, int S, int n_q_heads,
-                      int n_kv_heads, int has_k, int has_v, int head_dim, const float* cos_tab, const float* sin_tab,
-                      void* q_out, void* k_cache, void* vt_cache, int t_max, int tok_offset, vla_stream_t stream) {
+static int qkv_rope_impl(const void* x, const void* W, const float* bias, int dtype, int M, int K, int S, int n_q_heads,
+                         int n_kv_heads, int has_k, int has_v, int head_dim, const float* cos_tab, const float* sin_tab,
+                         void* q_out, void* k_cache, void* vt_cache, int t_max, int tok_offset, float rms_eps,
+                         vla_stream_t stream) {
     if (!x || !W || M < 0 || K <= 0 || S <= 0 || n_q_heads < 0 || n_kv_heads < 0 || head_dim <= 0) return VLA_K_ERR_ARG;
     const int nk = has_k ? n_kv_heads : 0, nv = has_v ? n_kv_heads : 0;
     if (n_q_heads > 0 && !q_out) return VLA_K_ERR_ARG;
@@ -1197,6 +1250,7 @@ int vla_attn_qkv_rope(const void* x, const void* W, const float* bias, int dtype
     if ((n_q_heads * D) % BN || (nk * D) % BN || (nv * D) % BN || D % 8) return VLA_K_ERR_SHAPE;
     if (cos_tab && D % BN) return VLA_K_ERR_SHAPE;  // rotation pairs both halves of a head inside one tile
     GemmArgs a = {};
+    a.norm_eps = rms_eps;
     a.A = x; a.W = W; a.bias = bias; a.M = M; a.K = K;
     a.N = (n_q_heads + nk + nv) * D;
     a.S = S; a.Hq = n_q_heads; a.nk = nk; a.nv = nv; a.D = D; a.Hkv = n_kv_heads;
@@ -1214,12 +1268,58 @@ int vla_attn_qkv_rope(const void* x, const void* W, const float* bias, int dtype
     return VLA_K_ERR_ARG;
 }
 
+int vla_attn_qkv_rope(const void* x, const void* W, const float* bias, int dtype, int M, int K, int S, int n_q_heads,
+                      int n_kv_heads, int has_k, int has_v, int head_dim, const float* cos_tab, const float* sin_tab,
+                      void* q_out, void* k_cache, void* vt_cache, int t_max, int tok_offset, vla_stream_t stream) {
+    return qkv_rope_impl(x, W, bias, dtype, M, K, S, n_q_heads, n_kv_heads, has_k, has_v, head_dim, cos_tab, sin_tab, q_out,
+                         k_cache, vt_cache, t_max, tok_offset, -1.f, stream);
+}
+
+int vla_rmsnorm_attn_qkv_rope(const void* x, const void* W_folded, const float* bias, int dtype, int M, int K, int S,
+                              int n_q_heads, int n_kv_heads, int has_k, int has_v, int head_dim, const float* cos_tab,
+                              const float* sin_tab, void* q_out, void* k_cache, void* vt_cache, int t_max, int tok_offset,
+                              float rms_eps, vla_stream_t stream) {
+    if (rms_eps < 0.f) return VLA_K_ERR_ARG;
+    if (dtype != VLA_DT_BF16) return VLA_K_ERR_SHAPE;
+    return qkv_rope_impl(x, W_folded, bias, dtype, M, K, S, n_q_heads, n_kv_heads, has_k, has_v, head_dim, cos_tab, sin_tab,
+                         q_out, k_cache, vt_cache, t_max, tok_offset, rms_eps, stream);
+}
+
+int vla_fold_norm_weight_host(const void* W, const void* g, int dtype, int N, int K, void* W_out) {
+    if (!W || !g || !W_out || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (dtype == VLA_DT_F32) {
+        for (long n = 0; n < N; ++n)
+            for (int k = 0; k < K; ++k) ((float*)W_out)[n * K + k] = ((const float*)W)[n * K + k] * ((const float*)g)[k];
+        return VLA_K_OK;
+    }
+    if (dtype == VLA_DT_BF16) {
+        const uint16_t* w = (const uint16_t*)W;
+        const uint16_t* gg = (const uint16_t*)g;
+        for (long n = 0; n < N; ++n)
+            for (int k = 0; k < K; ++k) {
+                uint32_t wb = (uint32_t)w[n * K + k] << 16, gb = (uint32_t)gg[k] << 16;
+                float wf, gf;
+                memcpy(&wf, &wb, 4);
+                memcpy(&gf, &gb, 4);
+                const float p = wf * gf;
+                uint32_t pb;
+                memcpy(&pb, &p, 4);
+                if ((pb & 0x7fffffffu) > 0x7f800000u) pb |= 0x00400000u;                // NaN stays NaN
+                else pb += 0x7fffu + ((pb >> 16) & 1u);                                  // round to nearest even
+                ((uint16_t*)W_out)[n * K + k] = (uint16_t)(pb >> 16);
+            }
+        return VLA_K_OK;
+    }
+    return VLA_K_ERR_ARG;
+}
+
 int vla_ternary_gemm(const int8_t* A, const uint32_t* W_packed, uint16_t* out, int32_t* acc_out, const float* s,
                      const int32_t* rowsum, const float* ws, int ws_num, int M, int N, int K, vla_stream_t stream) {
     if (!A || !W_packed || !rowsum || (!out && !acc_out) || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
     if (out && (!s || !ws || ws_num <= 0)) return VLA_K_ERR_ARG;
     if (K % 128 || (out && N % ws_num)) return VLA_K_ERR_SHAPE;
     GemmArgs a = {};
+    a.norm_eps = -1.f;
     a.A = A; a.W = W_packed; a.M = M; a.N = N; a.K = K;
     a.Y = out; a.acc_out = acc_out; a.s = s; a.rowsum = rowsum; a.ws = ws; a.ws_num = ws_num > 0 ? ws_num : 1;
     return launch<int8_t, EPI_TERNARY>(a, (N + BN - 1) / BN, stream);
@@ -1230,6 +1330,7 @@ int vla_ternary_gemm_add(const int8_t* A, const uint32_t* W_packed, uint16_t* ou
     if (!A || !W_packed || !rowsum || !out || !s || !ws || ws_num <= 0 || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
     if (K % 128 || N % ws_num) return VLA_K_ERR_SHAPE;
     GemmArgs a = {};
+    a.norm_eps = -1.f;
     a.A = A; a.W = W_packed; a.M = M; a.N = N; a.K = K;
     a.Y = out; a.residual = residual; a.s = s; a.rowsum = rowsum; a.ws = ws; a.ws_num = ws_num;
     return launch<int8_t, EPI_TERNARY>(a, (N + BN - 1) / BN, stream);

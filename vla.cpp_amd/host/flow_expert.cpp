@@ -51,6 +51,20 @@ DevBuf load_w(const Checkpoint& ck, const std::string& name, int dtype) {
 }
 DevBuf load_f32(const Checkpoint& ck, const std::string& name) { return load_w(ck, name, VLA_DT_F32); }
 
+// bf16 copy of weight `name` [N][K] with the RMSNorm weight `ln` [K] multiplied into its
+// columns, for the projection launch that takes the layer's pre-norm inside it.
+DevBuf load_folded_bf16(const Checkpoint& ck, const std::string& name, const std::string& ln) {
+    const std::vector<float> wf = ck.f32(name), gf = ck.f32(ln);
+    const size_t K = gf.size(), N = wf.size() / K;
+    std::vector<uint16_t> w(wf.size()), g(K);
+    for (size_t i = 0; i < wf.size(); ++i) w[i] = f32_to_bf16(wf[i]);
+    for (size_t k = 0; k < K; ++k) g[k] = f32_to_bf16(gf[k]);
+    VLA_K(vla_fold_norm_weight_host(w.data(), g.data(), VLA_DT_BF16, (int)N, (int)K, w.data()));
+    DevBuf b;
+    b.upload(w.data(), w.size() * sizeof(uint16_t));
+    return b;
+}
+
 // y = W x + b on the host, W [N][K] row-major, double accumulation.
 void host_linear(const float* W, const float* b, const float* x, float* y, int N, int K) {
     for (int n = 0; n < N; ++n) {
@@ -66,6 +80,7 @@ struct LayerW {
     bool is_self = true;
     DevBuf ln;                  // expert pre-norm weight (RMS archs)
     DevBuf Wqkv, bqkv;          // self: Q|K|V rows, cross: Q rows
+    DevBuf Wqkv_ln;             // the same rows with the pre-norm weight folded in (bf16 RMS archs)
     DevBuf Wo, bo;
     DevBuf vlm_ln, Wkv_pre, bkv_pre;  // prefix K|V producer
     DevBuf Wk_x, Wv_x;          // SmolVLA cross layers: re-projection of the cached prefix K / V
@@ -194,6 +209,8 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         w.needs_prefix = !(arch_ == Arch::GR00T && w.is_self);
         if (arch_ != Arch::GR00T) w.ln = load_w(ck, p + "ln", dt_);
         w.Wqkv = load_w(ck, p + (w.is_self ? "Wqkv" : "Wq"), dt_);
+        if (arch_ != Arch::GR00T && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
+            w.Wqkv_ln = load_folded_bf16(ck, p + (w.is_self ? "Wqkv" : "Wq"), p + "ln");
         if (ck.has(p + (w.is_self ? "bqkv" : "bq"))) w.bqkv = load_f32(ck, p + (w.is_self ? "bqkv" : "bq"));
         w.Wo = load_w(ck, p + "Wo", dt_);
         if (ck.has(p + "bo")) w.bo = load_f32(ck, p + "bo");
@@ -424,29 +441,31 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                                    n_lead_ ? lead_.as<float>() : nullptr, h.data, dt_, B, S_, n_lead_, A_, W_, C.stream));
             for (int l = 0; l < L_; ++l) {
                 LayerW& w = layers_[l];
-                if (arch_ == Arch::GR00T) {
-                    const float* sc = ada_.as<float>() + ((size_t)s * (L_ + 1) + l) * 2 * W_;
-                    adaln(C, h, sc, sc + W_, eps_, hn);
-                } else {
-                    rms_norm(C, h, w.ln.get(), eps_, hn);
-                }
                 const float* bq = w.bqkv ? w.bqkv.as<float>() : nullptr;
+                const int64_t n_rows_w = w.is_self ? (int64_t)(Hq_ + 2 * Hkv_) * D_ : (int64_t)Hq_ * D_;
+                const RopeTable* tab = rope_ ? (w.is_self ? &rope_self_ : &rope_cross_) : nullptr;
+                const int tok = w.is_self ? w.kv.n_prefix : 0;
+                // RMS archs in bf16: pre-norm, projection, rotation and append are one launch
+                bool done = false;
+                if (w.Wqkv_ln) {
+                    Tensor Wf = tensor_2d(w.Wqkv_ln.get(), dt_, W_, n_rows_w);
+                    done = rmsnorm_qkv_rope_append(C, h, Wf, bq, eps_, S_, Hq_, w.is_self, w.is_self, tab, Q.data, w.kv, tok);
+                }
+                if (!done) {
+                    if (arch_ == Arch::GR00T) {
+                        const float* sc = ada_.as<float>() + ((size_t)s * (L_ + 1) + l) * 2 * W_;
+                        adaln(C, h, sc, sc + W_, eps_, hn);
+                    } else {
+                        rms_norm(C, h, w.ln.get(), eps_, hn);
+                    }
+                    Tensor Wqkv = tensor_2d(w.Wqkv.get(), dt_, W_, n_rows_w);
+                    qkv_rope_append(C, hn, Wqkv, bq, S_, Hq_, w.is_self, w.is_self, tab, Q.data, w.kv, tok);
+                }
                 MaskSpec mask;
                 mask.pad_start = pad_start_;
                 mask.pad_end = pad_end_;
-                int n_keys;
-                if (w.is_self) {
-                    Tensor Wqkv = tensor_2d(w.Wqkv.get(), dt_, W_, (int64_t)(Hq_ + 2 * Hkv_) * D_);
-                    qkv_rope_append(C, hn, Wqkv, bq, S_, Hq_, true, true, rope_ ? &rope_self_ : nullptr, Q.data, w.kv,
-                                    w.kv.n_prefix);
-                    mask.kind = suffix_mask_;
-                    n_keys = w.kv.n_prefix + S_;
-                } else {
-                    Tensor Wq = tensor_2d(w.Wqkv.get(), dt_, W_, (int64_t)Hq_ * D_);
-                    qkv_rope_append(C, hn, Wq, bq, S_, Hq_, false, false, rope_ ? &rope_cross_ : nullptr, Q.data, w.kv, 0);
-                    mask.kind = VLA_MASK_NONE;
-                    n_keys = w.kv.n_prefix;
-                }
+                mask.kind = w.is_self ? suffix_mask_ : VLA_MASK_NONE;
+                const int n_keys = w.is_self ? w.kv.n_prefix + S_ : w.kv.n_prefix;
                 flash_attention(C, Q, w.kv, n_keys, mask, scale, att);
                 Tensor Wo = tensor_2d(w.Wo.get(), dt_, (int64_t)Hq_ * D_, W_);
                 linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
