@@ -193,23 +193,31 @@ def kernel_breakdown(pkg, cfg, B, P):
     mask_kind = cfg["suffix_mask"]
     add("embed_suffix", lambda i: pkg.call("vla_embed_suffix", xt, W_in, b_in, lead if n_lead else None, h, dt, B, S, n_lead, A, W),
         1, "hbm", M * W * es)
+    # bf16 RMS archs: the layer's pre-norm runs inside the projection launch (as the host
+    # layer does); only the final norm is a launch of its own
+    fused_norm = bf and not gr00t and W % 16 == 0
     if gr00t:
         add("adaln", lambda i: pkg.call("vla_adaln", h, scv, scv, hn, dt, M, W, 1e-5), L + 1, "hbm", 2 * M * W * es)
     else:
-        add("rms_norm", lambda i: pkg.call("vla_rms_norm", h, lnw, hn, dt, M, W, 1e-5), L + 1, "hbm", 2 * M * W * es)
+        add("rms_norm", lambda i: pkg.call("vla_rms_norm", h, lnw, hn, dt, M, W, 1e-5), 1 if fused_norm else L + 1, "hbm",
+            2 * M * W * es)
+
+    def proj(Wmat, has_kv, kc, vc, t_max, tok):
+        if fused_norm:
+            return lambda i: pkg.call("vla_rmsnorm_attn_qkv_rope", h, Wmat, None, dt, M, W, S, Hq, Hkv, has_kv, has_kv, D, rope,
+                                      sin, q, kc, vc, t_max, tok, 1e-5)
+        return lambda i: pkg.call("vla_attn_qkv_rope", hn, Wmat, None, dt, M, W, S, Hq, Hkv, has_kv, has_kv, D, rope,
+                                  None if gr00t else sin, q, kc, vc, t_max, tok)
+
     if n_self:
-        add("qkv_rope_append_self", lambda i: pkg.call("vla_attn_qkv_rope", hn, Wqkv, None, dt, M, W, S, Hq, Hkv, 1, 1, D, rope,
-                                                     None if gr00t else sin, q, kc_s, vc_s, t_self, P_self),
-            n_self, "mfma", 2.0 * M * (qd + 2 * kvd) * W)
+        add("qkv_rope_append_self", proj(Wqkv, 1, kc_s, vc_s, t_self, P_self), n_self, "mfma", 2.0 * M * (qd + 2 * kvd) * W)
         add("attention_self", lambda i: pkg.call("vla_attn_prefix_suffix", q, kcs_s[i % n_rot], vcs_s[i % n_rot], att, dt, B, S, Hq, Hkv, D, t_self,
                                                T_self, scale, mask_kind, P_self, 0, 0, None),
             n_self, "hbm", 2 * T_self * kvd * es * B)
     if n_cross:
         kcs_c, vcs_c = kv_set(n_rot, B, Hkv, t_cross, D), kv_set(n_rot, B, Hkv, D, t_cross)
         kc_c, vc_c = kcs_c[0], vcs_c[0]
-        add("q_rope_cross", lambda i: pkg.call("vla_attn_qkv_rope", hn, Wq, None, dt, M, W, S, Hq, Hkv, 0, 0, D, rope,
-                                             None if gr00t else sin, q, kc_c, vc_c, t_cross, 0),
-            n_cross, "mfma", 2.0 * M * qd * W)
+        add("q_rope_cross", proj(Wq, 0, kc_c, vc_c, t_cross, 0), n_cross, "mfma", 2.0 * M * qd * W)
         add("attention_cross", lambda i: pkg.call("vla_attn_prefix_suffix", q, kcs_c[i % n_rot], vcs_c[i % n_rot], att, dt, B, S, Hq, Hkv, D, t_cross,
                                                 P, scale, 0, P, 0, 0, None),
             n_cross, "hbm", 2 * P * kvd * es * B)

@@ -319,12 +319,26 @@ def _mask(kind, P, S, pad):
     return m, pkg.VLA_MASK_NONE, P + S
 
 
-@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("dtype,kernel", [(F32, "auto"), (BF16, "auto"), (BF16, "direct"), (BF16, "staged"), (BF16, "one-slice")],
+                         ids=["f32", "bf16", "bf16-direct", "bf16-staged", "bf16-one-slice"])
 @pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
-def test_attention_against_oracle(dtype, case):
+def test_attention_against_oracle(monkeypatch, dtype, kernel, case):
     name, B, S, Hq, Hkv, D, P, kind, pad = case
     if dtype == F32 and D == 256:
         pytest.skip("fp32 tiles for 256-wide heads are not built (LDS budget); pi0 runs in bf16")
+    if kernel == "direct":
+        # the register-direct kernel is the default up to 32 query rows per kv head; beyond
+        # that it walks 32-row blocks, exercised here on the cases that normally take the LDS kernel
+        if not (D <= 128 and 32 < (Hq // Hkv) * S <= 256):
+            pytest.skip("covered by the default dispatch")
+        monkeypatch.setenv("VLA_ATTN_DIRECT_ROWS", "256")
+    if kernel in ("staged", "one-slice"):
+        # 64-wide bf16 heads beyond 32 rows default to the direct-to-LDS variant of the LDS
+        # kernel (two key slices per row tile with 3+ key tiles); the
+        # register-staged variant and the unsliced one on the same cases
+        if not (D == 64 and (Hq // Hkv) * S > 32):
+            pytest.skip("covered by the default dispatch")
+        monkeypatch.setenv("VLA_ATTN_DL" if kernel == "staged" else "VLA_ATTN_SLICES", "0" if kernel == "staged" else "1")
     r = np.random.default_rng(106)
     mask, mkind, T = _mask(kind, P, S, pad)
     t_max = (T + 63) // 64 * 64

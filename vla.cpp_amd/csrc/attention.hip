@@ -60,6 +60,8 @@ struct AttnArgs {
     int mask_kind, n_prefix, pad_start, pad_end;
     const float* mask;
     int n_groups, n_split, tiles_per_split, r_pad, p2;
+    int n_rblocks;  // direct kernel: 32-row blocks per (batch, kv head)
+    int n_slices;   // LDS kernel, direct-to-LDS variant: key slices (wavefronts) per row tile
     float* part_o;   // [pair][split][r_pad][D]
     float* part_ml;  // [pair][split][r_pad][2]
 };
@@ -98,10 +100,20 @@ template <> struct AT<float> {
 // wavefronts never touch global memory inside the loop.  One barrier per tile.  Used for
 // wide heads, whose accumulators and query fragments leave the compute wavefronts no
 // registers to prefetch with, so that memory latency would be exposed once per tile.
-template <typename T, int D, int NW, bool P2, int NL>
-__global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_kernel(AttnArgs a) {
+//
+// NSL > 0 selects the direct-to-LDS variant (bf16, 128- or 256-byte K rows): tiles go from
+// the cache straight into an unpadded, swizzled LDS ring (16-byte piece c of row `row` at
+// piece position c ^ swz(row), swz = (row >> 1) & 7 for 128-byte rows, row & 15 for 256-byte
+// rows), one barrier per step and no staging registers or LDS stores.  The workgroup then
+// has NW x NSL wavefronts: NSL key slices per row tile, slice sl taking tiles sl, sl + NSL,
+// ... of the workgroup's key range; a step multiplies NSL tiles at once and the slices'
+// partial (max, sum, output) meet in LDS at the end.  RS step slots form the ring.
+template <typename T, int D, int NW, bool P2, int NL, int NSL = 0, int RS = 1>
+__global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_kernel(AttnArgs a) {
     typedef AT<T> A;
     constexpr int EB = A::EB, CE = A::CE;
+    constexpr bool DLOAD = NSL > 0;
+    static_assert(!DLOAD || (NL == 0 && EB == 2 && (D == 64 || D == 128)), "direct-to-LDS tiles: bf16, 128/256-byte K rows");
     // Keys per staged tile: 64, or 32 for wide heads (rows of 512 bytes and more), whose
     // accumulators and query fragments leave too few registers to stage 64 keys.
     constexpr int TK = (D * EB >= 512) ? 32 : SPLIT_KEYS;
@@ -121,8 +133,14 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
     static_assert(D % CE == 0 && (D * EB) % 16 == 0, "head_dim must be whole MFMA groups and 16-byte rows");
     static_assert(NVEC == D * VV_PER_ROW, "K and V^T tiles hold the same number of vectors");
 
-    __shared__ __attribute__((aligned(16))) unsigned char ldsK_buf[NL ? 2 : 1][TK * KS];
-    __shared__ __attribute__((aligned(16))) unsigned char ldsV_buf[NL ? 2 : 1][DP * VS];
+    constexpr int KROW = D * EB, VROW = TK * EB;          // unpadded row sizes of the direct-to-LDS ring
+    constexpr int KTILE = TK * KROW, VTILE = DP * VROW, STAGE = KTILE + VTILE;
+    constexpr int NWAVES = NW * (DLOAD ? NSL : 1);
+    constexpr int XCH = (NSL > 1) ? (NSL - 1) * NW * (NDB * 16 + 2) * 64 * 4 : 0;  // slice merge buffer
+    constexpr int RING = DLOAD ? (RS * NSL * STAGE > XCH ? RS * NSL * STAGE : XCH) : 16;
+    __shared__ __attribute__((aligned(16))) unsigned char ldsK_buf[NL ? 2 : 1][DLOAD ? 16 : TK * KS];
+    __shared__ __attribute__((aligned(16))) unsigned char ldsV_buf[NL ? 2 : 1][DLOAD ? 16 : DP * VS];
+    __shared__ __attribute__((aligned(1024))) unsigned char ring[RING];
     unsigned char* ldsK = ldsK_buf[0];
     unsigned char* ldsV = ldsV_buf[0];
 
@@ -139,9 +157,11 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
     const int g = lane >> 5, r = lane & 31;
     const int grp = a.Hq / a.Hkv;
     const int R = grp * a.S;
-    const int row = (group * NW + wave) * 32 + r;
-    const bool wave_active = wave < NW && (group * NW + wave) * 32 < R;
-    const bool row_valid = wave < NW && row < R;
+    const int rw = DLOAD ? wave % NW : wave;  // row tile of this wavefront
+    const int sl = DLOAD ? wave / NW : 0;     // key slice of this wavefront
+    const int row = (group * NW + rw) * 32 + r;
+    const bool wave_active = rw < NW && (group * NW + rw) * 32 < R;
+    const bool row_valid = rw < NW && row < R;
     const int hg = row_valid ? row / a.S : 0;
     const int s = row_valid ? row % a.S : 0;
     const int h = hk * grp + hg;
@@ -248,6 +268,16 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
         }
     };
 
+    // Direct-to-LDS ring: this lane's K fragment row and V^T fragment row inside a tile and
+    // the swizzle terms of its 16-byte pieces (piece 2c + g of a K row, piece 4kb + 2hh + g of
+    // a V^T row; the swizzle only involves the low row bits, which the 32-row block offsets
+    // leave alone).
+    const int krow_l = key_of_score_row(r);
+    const int kfrag = krow_l * KROW;
+    const int kx = g ^ (KROW == 128 ? ((krow_l >> 1) & 7) : (krow_l & 15));
+    const int vfrag = r * VROW;
+    const int vx = g ^ ((r >> 1) & 7);
+
     // Scores and online softmax of the staged K tile; leaves the probabilities in p.
     float p[NKB][16];
     auto scores_softmax = [&](int k0) __attribute__((always_inline)) {
@@ -267,8 +297,9 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
                 for (int i = 0; i < 16; ++i) sc[n][i] = 0.f;
 #pragma unroll
             for (int c = 0; c < NQ; ++c) {
-                const u32x4_t kf =
-                    *reinterpret_cast<const u32x4_t*>(ldsK + (kb * 32 + key_of_score_row(r)) * KS + (c * CE + g * (CE / 2)) * EB);
+                const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(
+                    DLOAD ? ldsK + kb * 32 * KROW + kfrag + (((2 * c) ^ kx) * 16)
+                          : ldsK + (kb * 32 + key_of_score_row(r)) * KS + (c * CE + g * (CE / 2)) * EB);
                 A::mma(sc[c % NA], kf, qf[c]);
             }
 #pragma unroll
@@ -334,7 +365,10 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
         l_run += psum;
     };
     // O^T += V^T . P^T from the staged V^T tile.
-    auto output_product = [&]() __attribute__((always_inline)) {
+    auto output_product = [&](int k0) __attribute__((always_inline)) {
+        // direct-to-LDS tiles arrive unfiltered: V^T elements past n_keys (stale cache
+        // contents, possibly NaN) are zeroed in the fragment registers of the last tile
+        const bool v_partial = DLOAD && k0 + TK > a.n_keys;  // uniform
 #pragma unroll
         for (int kb = 0; kb < NKB; ++kb) {
             if (EB == 2) {
@@ -354,9 +388,15 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
                             pl[e] = pack_bf2(pp[2 * e] - __uint_as_float(hi16 << 16), pp[2 * e + 1] - __uint_as_float(hi16 & 0xffff0000u));
                     }
                     const int key_off = (kb * 32 + hh * 16 + 8 * g) * EB;
+                    const int nvalid = a.n_keys - (k0 + kb * 32 + hh * 16 + 8 * g);  // real keys among this lane's 8
 #pragma unroll
                     for (int db = 0; db < NDB; ++db) {
-                        const u32x4_t vf = *reinterpret_cast<const u32x4_t*>(ldsV + (db * 32 + r) * VS + key_off);
+                        u32x4_t vf = *reinterpret_cast<const u32x4_t*>(
+                            DLOAD ? ldsV + db * 32 * VROW + vfrag + (((4 * kb + 2 * hh) ^ vx) * 16) : ldsV + (db * 32 + r) * VS + key_off);
+                        if (v_partial) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) vf[e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+                        }
                         A::mma(o[db], vf, pf);
                         if (P2) A::mma(o[db], vf, pl);
                     }
@@ -378,7 +418,102 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
         }
     };
 
-    if constexpr (NL > 0) {
+    if constexpr (DLOAD) {
+        constexpr int KI = KTILE / 1024, VI = VTILE / 1024;   // load instructions (1 KiB each) per K / V^T tile
+        constexpr int PER_STEP = NSL * (KI + VI);
+        constexpr int IPW = (PER_STEP + NWAVES - 1) / NWAVES;  // per wavefront and step, padded with repeats
+        constexpr int KRPI = 1024 / KROW;                      // K rows per load instruction (8 or 4)
+        static_assert(RS >= 2, "the ring needs a slot to load into while another is read");
+        constexpr int W0 = (RS - 1) * IPW < 63 ? (RS - 1) * IPW : 63;  // a smaller count only waits longer
+        constexpr int W1 = (RS - 2) * IPW < 63 ? (RS - 2) * IPW : 63;
+        const int n_t = (k_end - k_begin + TK - 1) / TK;
+        const int n_steps = (n_t + NSL - 1) / NSL;
+        const uint32_t ring0 = (uint32_t)(uintptr_t)ring;  // low 32 bits of a shared-aperture address = LDS offset
+        const int wv = __builtin_amdgcn_readfirstlane(wave);
+        // Step `st` goes into ring slot `slot`.  Instruction j of a step: tile j / (KI + VI)
+        // of the step, then K rows (j' < KI) or V^T rows.  Tiles past the last one repeat it
+        // and K rows past n_keys repeat the last key (their scores are masked); V^T runs are
+        // kept inside the cache row.  Repeats rewrite the same bytes, so the padding of the
+        // per-wavefront count is harmless.
+        auto issue_step = [&](int st, int slot) __attribute__((always_inline)) {
+#pragma unroll
+            for (int it = 0; it < IPW; ++it) {
+                const int j = (wv + it * NWAVES) % PER_STEP;  // wavefront-uniform
+                const int ts = j / (KI + VI), jj = j % (KI + VI);
+                const int t = min(st * NSL + ts, n_t - 1);
+                const int k0 = k_begin + t * TK;
+                const uint32_t base = ring0 + (slot * NSL + ts) * STAGE;
+                if (jj < KI) {
+                    const int rowi = jj * KRPI + lane / (KROW / 16), pos = lane % (KROW / 16);
+                    const int piece = pos ^ (KROW == 128 ? ((rowi >> 1) & 7) : (rowi & 15));
+                    const int key = min(k0 + rowi, a.n_keys - 1);
+                    load_to_lds16(kbase + (long)key * KROW + piece * 16, base + jj * 1024);
+                } else {
+                    const int rowi = (jj - KI) * 8 + lane / 8, pos = lane % 8;  // V^T rows are 128 bytes
+                    const int piece = pos ^ ((rowi >> 1) & 7);
+                    const int key0 = min(k0 + piece * 8, a.t_max - 8);
+                    load_to_lds16(vbase + ((long)min(rowi, D - 1) * a.t_max + key0) * EB, base + KTILE + (jj - KI) * 1024);
+                }
+            }
+        };
+        // The whole ring is requested up front (for short key ranges that is every tile: the
+        // kernel then pays the memory latency once); step st + RS - 1 follows at the start of
+        // step st into the slot step st - 1 has just been read from.
+#pragma unroll
+        for (int st = 0; st < RS; ++st) issue_step(st, st);
+        int slot = 0, lslot = RS - 1;
+        for (int st = 0; st < n_steps; ++st) {
+            // own loads of this step have landed (the younger ones may be pending) ...
+            if (st == 0) wait_vmcnt<W0>();
+            else wait_vmcnt<W1>();
+            __syncthreads();  // ... everyone's have, and the slot read in the previous step is free
+            if (st > 0) issue_step(st + RS - 1, lslot);
+            const int t = st * NSL + sl;
+            if (wave_active && t < n_t) {
+                ldsK = ring + (slot * NSL + sl) * STAGE;
+                ldsV = ldsK + KTILE;
+                scores_softmax(k_begin + t * TK);
+                output_product(k_begin + t * TK);
+            }
+            slot = (slot + 1 == RS) ? 0 : slot + 1;
+            lslot = (lslot + 1 == RS) ? 0 : lslot + 1;
+        }
+        wait_vmcnt<0>();  // the repeats must have landed before the ring is reused
+        __syncthreads();
+        if constexpr (NSL > 1) {
+            // slices 1.. leave their state in LDS, element-major with the lane innermost, so
+            // the wavefront of slice 0 with the same row tile finds each value under its own lane
+            constexpr int NE = NDB * 16 + 2;
+            float* xch = reinterpret_cast<float*>(ring);
+            if (sl > 0 && wave_active) {
+                float* px = xch + ((long)((sl - 1) * NW + rw) * NE) * 64 + lane;
+#pragma unroll
+                for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) px[(db * 16 + i) * 64] = o[db][i];
+                px[(NDB * 16) * 64] = m_run;
+                px[(NDB * 16 + 1) * 64] = l_run;
+            }
+            __syncthreads();
+            if (sl > 0) return;
+            if (wave_active) {
+#pragma unroll
+                for (int s2 = 1; s2 < NSL; ++s2) {
+                    const float* px = xch + ((long)((s2 - 1) * NW + rw) * NE) * 64 + lane;
+                    const float m2 = px[(NDB * 16) * 64], l2 = px[(NDB * 16 + 1) * 64];
+                    const float m_new = fmaxf(m_run, m2);
+                    const float mm = (m_new == -INFINITY) ? 0.f : m_new;
+                    const float w1 = A::fexp2(m_run - mm), w2 = A::fexp2(m2 - mm);  // 2^-inf = 0 for an empty side
+                    l_run = l_run * w1 + l2 * w2;
+                    m_run = m_new;
+#pragma unroll
+                    for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) o[db][i] = o[db][i] * w1 + px[(db * 16 + i) * 64] * w2;
+                }
+            }
+        }
+    } else if constexpr (NL > 0) {
         constexpr int NTL = NL * 64, ITL = NVEC / NTL, LOAD_AHEAD = 3;
         static_assert(NVEC % NTL == 0 && EB == 2, "loader wavefronts split a tile evenly; bf16 only");
         const int n_t = (k_end - k_begin + TK - 1) / TK;
@@ -436,7 +571,7 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
                 ldsK = ldsK_buf[t & 1];
                 ldsV = ldsV_buf[t & 1];
                 scores_softmax(k_begin + t * TK);
-                output_product();
+                output_product(k_begin + t * TK);
             }
             __syncthreads();
         }
@@ -460,7 +595,7 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
             __builtin_amdgcn_sched_barrier(0);
             if (wave_active) {
                 scores_softmax(k0);
-                output_product();
+                output_product(k0);
             }
         }
     } else {
@@ -480,7 +615,7 @@ __global__ void __launch_bounds__((NW + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1
             __syncthreads();
             if (k0 + TK < k_end) load_k(k0 + TK);
             __builtin_amdgcn_sched_barrier(0);
-            if (wave_active) output_product();
+            if (wave_active) output_product(k0);
         }
     }
 
@@ -539,13 +674,15 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 5, r = lane & 31;
     const int unit = MERGE ? blockIdx.x * a.n_split + wave : blockIdx.x * 4 + wave;
-    const int pair = unit / a.n_split, split = unit % a.n_split;
+    const int prb = unit / a.n_split, split = unit % a.n_split;  // (pair, 32-row block) and key slice
+    const int pair = prb / a.n_rblocks, rb = prb % a.n_rblocks;
     // whole wavefront (whole workgroup with MERGE); the main loop has no barriers
     if (pair >= a.batch * a.Hkv) return;
     const int b = pair / a.Hkv, hk = pair % a.Hkv;
     const int grp = a.Hq / a.Hkv, R = grp * a.S;
-    const bool row_valid = r < R;
-    const int hg = row_valid ? r / a.S : 0, s = row_valid ? r % a.S : 0;
+    const int row = rb * 32 + r;
+    const bool row_valid = row < R;
+    const int hg = row_valid ? row / a.S : 0, s = row_valid ? row % a.S : 0;
     const int h = hk * grp + hg;
 
     const int nb_total = (a.n_keys + 31) / 32;
@@ -730,11 +867,13 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
     }
 
     if (MERGE) {
-        // LDS: [slice][row][D + 2] floats (unnormalised output, then max and sum), rows < R only
+        // LDS: [slice][row of the block][D + 2] floats (unnormalised output, then max and sum)
         extern __shared__ float merge_buf[];
         const int RS = D + 2;
+        const int Rb = min(32, R - rb * 32);  // rows of this block
+        const int RB = min(32, R);            // rows per slice in the buffer
         if (row_valid) {
-            float* pr = merge_buf + ((long)split * R + r) * RS;
+            float* pr = merge_buf + ((long)split * RB + r) * RS;
 #pragma unroll
             for (int db = 0; db < NDB; ++db)
 #pragma unroll
@@ -750,27 +889,28 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
             }
         }
         __syncthreads();
-        for (int i = threadIdx.x; i < R * D; i += blockDim.x) {
-            const int row = i / D, d = i % D;
+        for (int i = threadIdx.x; i < Rb * D; i += blockDim.x) {
+            const int rl = i / D, d = i % D;
             float m = -INFINITY;
-            for (int sp = 0; sp < a.n_split; ++sp) m = fmaxf(m, merge_buf[((long)sp * R + row) * RS + D]);
+            for (int sp = 0; sp < a.n_split; ++sp) m = fmaxf(m, merge_buf[((long)sp * RB + rl) * RS + D]);
             float l = 0.f, acc = 0.f;
             if (m > -INFINITY) {
                 for (int sp = 0; sp < a.n_split; ++sp) {
-                    const float* pr = merge_buf + ((long)sp * R + row) * RS;
+                    const float* pr = merge_buf + ((long)sp * RB + rl) * RS;
                     const float w = exp2f(pr[D] - m);
                     l += pr[D + 1] * w;
                     acc += pr[d] * w;
                 }
             }
-            const int hh = hk * grp + row / a.S, ss = row % a.S;
+            const int grow = rb * 32 + rl;
+            const int hh = hk * grp + grow / a.S, ss = grow % a.S;
             ((bf16_t*)a.out)[(((long)b * a.S + ss) * a.Hq + hh) * D + d] = f2bf(l > 0.f ? acc / l : 0.f);
         }
         return;
     }
     if (!row_valid) return;
     if (a.n_split > 1) {
-        const long prow = ((long)pair * a.n_split + split) * a.r_pad + r;
+        const long prow = ((long)pair * a.n_split + split) * a.r_pad + row;
         if (g == 0) {
             a.part_ml[prow * 2] = m_run;
             a.part_ml[prow * 2 + 1] = l_run;
@@ -844,10 +984,47 @@ float* workspace(size_t floats) {
     return g_ws;
 }
 
+// Second launch of a key-split LDS-kernel call: combines the workgroups' partials.
+template <typename T, int D>
+int launch_merge(AttnArgs& a, hipStream_t st) {
+    if (a.n_split > 1) {
+        const int n_pairs = a.batch * a.Hkv;
+        const int R = (a.Hq / a.Hkv) * a.S;
+        const long total = (long)n_pairs * R * D;
+        attn_merge_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs,
+                                                                              a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
+        if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
+    }
+    return VLA_K_OK;
+}
+
 template <typename T, int D, int NW>
 int launch_nw(AttnArgs& a, hipStream_t st) {
     const int n_pairs = a.batch * a.Hkv;
     const int grid = (n_pairs + 7) / 8 * 8 * a.n_groups * a.n_split;
+    if constexpr (sizeof(T) == 2 && D == 64) {
+        // 64-wide bf16 heads: tiles go straight into a swizzled LDS ring (VLA_ATTN_DL=0 pins
+        // the register-staged path), and with three or more key tiles they are split over
+        // two wavefronts per row tile (VLA_ATTN_SLICES = 1 | 2 overrides).  The kernel also
+        // builds for 128-wide heads, where its register use makes it the slower choice.
+        const char* e = getenv("VLA_ATTN_DL");
+        if (!(e && atoi(e) == 0)) {
+            const int nsl = a.n_slices;
+            if constexpr (D == 64 && NW <= 2) {
+                if (nsl == 2) {
+                    if (a.p2) attn_kernel<T, D, NW, true, 0, 2, 2><<<grid, NW * 128, 0, st>>>(a);
+                    else attn_kernel<T, D, NW, false, 0, 2, 2><<<grid, NW * 128, 0, st>>>(a);
+                }
+            }
+            if (nsl == 2 && !(D == 64 && NW <= 2)) return VLA_K_ERR_SHAPE;  // launch_d never asks for this
+            if (nsl == 1) {
+                if (a.p2) attn_kernel<T, D, NW, true, 0, 1, 3><<<grid, NW * 64, 0, st>>>(a);
+                else attn_kernel<T, D, NW, false, 0, 1, 3><<<grid, NW * 64, 0, st>>>(a);
+            }
+            if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
+            return launch_merge<T, D>(a, st);
+        }
+    }
     if constexpr (sizeof(T) == 2) {
         // Wide heads: four loader wavefronts.  Narrow heads prefetch in registers instead
         // (with loader wavefronts a batch-32 SmolVLA launch no longer fits the chip in one round).
@@ -858,14 +1035,7 @@ int launch_nw(AttnArgs& a, hipStream_t st) {
         attn_kernel<T, D, NW, false, 0><<<grid, NW * 64, 0, st>>>(a);
     }
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
-    if (a.n_split > 1) {
-        const int R = (a.Hq / a.Hkv) * a.S;
-        const long total = (long)n_pairs * R * D;
-        attn_merge_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs,
-                                                                              a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
-        if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
-    }
-    return VLA_K_OK;
+    return launch_merge<T, D>(a, st);
 }
 
 template <int D>
@@ -873,11 +1043,13 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
     constexpr int ST = D <= 64 ? 3 : 2;
     const int n_pairs = a.batch * a.Hkv;
     const int R = (a.Hq / a.Hkv) * a.S;
+    a.n_rblocks = (R + 31) / 32;
+    const int n_units = n_pairs * a.n_rblocks;  // (pair, 32-row block)
     const int nb_total = (a.n_keys + 31) / 32;
     // Enough wavefronts to keep every CU's memory pipeline busy (8 per CU); a slice is
     // at least two 32-key blocks unless the whole sequence is shorter.
     int n_split = 1;
-    if (n_pairs < 2048) n_split = (2048 + n_pairs - 1) / n_pairs;
+    if (n_units < 2048) n_split = (2048 + n_units - 1) / n_units;
     if (n_split > (nb_total + 1) / 2) n_split = (nb_total + 1) / 2;
     if (n_split < 1) n_split = 1;
     if (const char* e = getenv("VLA_ATTN_SPLIT")) n_split = atoi(e) > 0 ? (atoi(e) < nb_total ? atoi(e) : nb_total) : 1;
@@ -885,17 +1057,17 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
     // when few enough; with fewer than 32 pairs more slices go through global partials and
     // the merge kernel instead.
     constexpr int MERGE_MAX = D <= 64 ? 8 : 4;  // wide heads need the registers of a 4-wavefront workgroup
-    const bool wg_merge = n_split > 1 && (n_split <= MERGE_MAX || n_pairs >= 32);
+    const bool wg_merge = n_split > 1 && (n_split <= MERGE_MAX || n_units >= 32);
     if (wg_merge && n_split > MERGE_MAX) n_split = MERGE_MAX;
     a.tiles_per_split = (nb_total + n_split - 1) / n_split;
     a.n_split = (nb_total + a.tiles_per_split - 1) / a.tiles_per_split;
-    a.r_pad = 32;
+    a.r_pad = a.n_rblocks * 32;
     a.n_groups = 1;
     if (wg_merge && a.n_split > 1) {
-        const size_t lds = (size_t)a.n_split * R * (D + 2) * sizeof(float);  // <= 8 * 32 * 130 * 4 = 133 KB; R is small in practice
+        const size_t lds = (size_t)a.n_split * (R < 32 ? R : 32) * (D + 2) * sizeof(float);  // at most 8 * 32 * 66 * 4 or 4 * 32 * 130 * 4 = 66 KB
         if (lds <= 64 * 1024) {
-            if (a.p2) attn_direct_kernel<D, true, ST, true><<<n_pairs, a.n_split * 64, lds, st>>>(a);
-            else attn_direct_kernel<D, false, ST, true><<<n_pairs, a.n_split * 64, lds, st>>>(a);
+            if (a.p2) attn_direct_kernel<D, true, ST, true><<<n_units, a.n_split * 64, lds, st>>>(a);
+            else attn_direct_kernel<D, false, ST, true><<<n_units, a.n_split * 64, lds, st>>>(a);
             return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
         }
     }
@@ -906,7 +1078,7 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
         a.part_o = ws;
         a.part_ml = ws + rows * D;
     }
-    const unsigned grid = (unsigned)(((long)n_pairs * a.n_split + 3) / 4);
+    const unsigned grid = (unsigned)(((long)n_units * a.n_split + 3) / 4);
     if (a.p2) attn_direct_kernel<D, true, ST, false><<<grid, 256, 0, st>>>(a);
     else attn_direct_kernel<D, false, ST, false><<<grid, 256, 0, st>>>(a);
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
@@ -921,14 +1093,31 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
 
 template <typename T, int D>
 int launch_d(AttnArgs& a, vla_stream_t stream) {
-    constexpr int NW_MAX = 4;  // at most one wavefront of a workgroup per SIMD
     const int R = (a.Hq / a.Hkv) * a.S;
     if constexpr (sizeof(T) == 2 && D <= 128) {
-        static const bool no_direct = getenv("VLA_ATTN_NO_DIRECT") != nullptr;
-        if (R <= 32 && !no_direct) return launch_direct<D>(a, (hipStream_t)stream);
+        // VLA_ATTN_NO_DIRECT pins the LDS kernel; VLA_ATTN_DIRECT_ROWS overrides the row limit
+        // of the register-direct one (tests and tuning).
+        const bool no_direct = getenv("VLA_ATTN_NO_DIRECT") != nullptr;
+        const char* er = getenv("VLA_ATTN_DIRECT_ROWS");
+        const int max_rows = er ? atoi(er) : 32;  // more rows: 16-byte runs per key row cost more than sharing tiles through LDS saves
+        if (R <= max_rows && !no_direct) return launch_direct<D>(a, (hipStream_t)stream);
     }
     const int n_tiles = (R + 31) / 32;
-    // One wavefront per row tile; more than NW_MAX tiles are spread evenly over groups.
+    // 64-wide bf16 heads with three or more key tiles: two key slices per row tile (the
+    // direct-to-LDS variant of the kernel; VLA_ATTN_DL=0 and VLA_ATTN_SLICES override).
+    // Two wavefronts per row tile then, and at most two row tiles per workgroup, so that a
+    // batch-32 launch stays resident at once (two 4-wavefront workgroups per CU).
+    a.n_slices = 1;
+    if constexpr (sizeof(T) == 2 && D == 64) {
+        const char* e = getenv("VLA_ATTN_DL");
+        if (!(e && atoi(e) == 0)) {
+            a.n_slices = (a.n_keys + SPLIT_KEYS - 1) / SPLIT_KEYS >= 3 ? 2 : 1;
+            if (const char* es = getenv("VLA_ATTN_SLICES")) a.n_slices = atoi(es) == 2 ? 2 : 1;
+        }
+    }
+    // One wavefront (per slice) per row tile, at most one wavefront of a workgroup per SIMD;
+    // more row tiles than that are spread evenly over groups.
+    const int NW_MAX = a.n_slices == 2 ? 2 : 4;
     a.n_groups = (n_tiles + NW_MAX - 1) / NW_MAX;
     const int nw = (n_tiles + a.n_groups - 1) / a.n_groups;
     a.r_pad = a.n_groups * nw * 32;

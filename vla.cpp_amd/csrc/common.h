@@ -91,4 +91,19 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return r;
 }
 
+// s_waitcnt on the vector-memory counter alone (vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits
+// 15:14; the export and LDS/scalar counter fields at their maxima, i.e. not waited on).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+// One 16-byte load per lane from global memory straight into LDS, no register in between:
+// lane i's bytes land at lds_base + 16 i (lds_base wavefront-uniform, held in M0); the
+// per-lane global address is free.  Completion is tracked by vmcnt like any vector load.
+// Issued from inline assembly so that the wait counts stay under this file's control.
+__device__ __forceinline__ void load_to_lds16(const void* gptr, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gptr) : "memory");
+}
+
 }  // namespace vk
