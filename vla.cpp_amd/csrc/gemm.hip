@@ -679,8 +679,12 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     const int fragA = (wm * 32 + r) * KB, fragW = ROWS_A * KB + (wn * 32 + r) * KB;
     auto multiply = [&](int stage, auto do_load, int st_load, int kt_load, int n_chunks) __attribute__((always_inline)) {
         constexpr bool LOAD = decltype(do_load)::value;
+        // fragments are read PF k-chunks ahead of the MFMAs that use them: one chunk of MFMAs
+        // is shorter than the LDS latency, so a single chunk of lookahead leaves every chunk
+        // waiting on its reads
+        constexpr int PF = NCH >= 4 ? 2 : 1, SLOTS = PF + 1;
         const unsigned char* base = lds + stage * STAGE;
-        u32x4_t fa[2][TM], fw[2][TN];
+        u32x4_t fa[SLOTS][TM], fw[SLOTS][TN];
         auto read_frags = [&](int slot, int ch) __attribute__((always_inline)) {
             const int off = (ch * 32) ^ xo;
 #pragma unroll
@@ -688,10 +692,11 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) fw[slot][j] = *reinterpret_cast<const u32x4_t*>(base + fragW + j * 64 * KB + off);
         };
-        read_frags(0, 0);
+#pragma unroll
+        for (int ch = 0; ch < PF; ++ch) read_frags(ch % SLOTS, ch);
 #pragma unroll
         for (int ch = 0; ch < NCH; ++ch) {
-            if (ch + 1 < NCH) read_frags((ch + 1) & 1, ch + 1);
+            if (ch + PF < NCH) read_frags((ch + PF) % SLOTS, ch + PF);
             if (LOAD) {
 #pragma unroll
                 for (int i = ch * NLOAD / NCH; i < (ch + 1) * NLOAD / NCH; ++i) issue(i, kt_load, st_load);
@@ -700,12 +705,12 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
 #pragma unroll
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[ch & 1][i], fw[ch & 1][j]);
+                    for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[ch % SLOTS][i], fw[ch % SLOTS][j]);
                 if (kNorm) {
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) ssq[i] = add_squares_bf16x2(fa[ch & 1][i][e], ssq[i]);
+                        for (int e = 0; e < 4; ++e) ssq[i] = add_squares_bf16x2(fa[ch % SLOTS][i][e], ssq[i]);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);  // keeps the reads and loads where they were placed
