@@ -108,6 +108,27 @@ VLA_KAPI int vla_adaln(const void* x, const float* sc, const float* sh, void* y,
 VLA_KAPI int vla_linear(const void* x, const void* W, const float* bias, const void* residual, void* y,
                         int dtype, int out_dtype, int M, int N, int K, vla_stream_t stream);
 
+/* Activations of the FFN halves (ggml_silu, ggml_gelu in its tanh form). */
+enum { VLA_ACT_NONE = 0, VLA_ACT_SILU = 1, VLA_ACT_GELU = 2 };
+
+/* vla_linear with an activation between the bias and the residual:
+ * y = act(x W^T + b) [+ residual]; the first half of ffn_gelu
+ * (src/layers/ffn.h:24-27, used by DitHead::block, src/modules/dit_head.cpp:133). */
+VLA_KAPI int vla_linear_act(const void* x, const void* W, const float* bias, const void* residual, void* y, int dtype,
+                            int out_dtype, int M, int N, int K, int act, vla_stream_t stream);
+
+/* Gated FFN input half in one launch: y[M][I] = act(x Wg^T + bg) * (x Wu^T + bu), replacing
+ * mm_w(Wgate) -> ggml_silu / ggml_gelu -> mm_w(Wup) -> ggml_mul (src/models/smolvla.cpp:845-847,
+ * src/models/pi0.cpp:227-230, src/layers/ffn.h:35-40).
+ *   W_gate_up [2 I][K]: the I gate rows, then the I up rows; bias fp32 [2 I] in the same order or NULL
+ *   I a multiple of 32
+ *   rms_eps >= 0: the RMSNorm in front of the FFN is taken inside the launch as in
+ *     vla_rmsnorm_attn_qkv_rope (rows scaled by rsqrt(mean x^2 + eps), norm weight folded
+ *     into both halves of W_gate_up with vla_fold_norm_weight_host; bf16, K % 16 == 0,
+ *     else VLA_K_ERR_SHAPE); rms_eps < 0: x is used as it is. */
+VLA_KAPI int vla_glu_linear(const void* x, const void* W_gate_up, const float* bias, void* y, int dtype, int out_dtype,
+                            int M, int I, int K, int act, float rms_eps, vla_stream_t stream);
+
 /* Fused QKV projection + RoPE + KV append for M = batch*S suffix (or prefix)
  * rows: replaces mm_w(Wq/Wk/Wv) -> reshape -> rope_q_or_k -> ggml_concat
  * (src/models/smolvla.cpp:821-833, src/models/pi0.cpp:174-201,

@@ -166,6 +166,26 @@ def silu(x):
     return (x / (1.0 + np.exp(-x.astype(np.float64)))).astype(np.float32)
 
 
+def gelu(x):
+    """ggml_gelu: the tanh form 0.5 x (1 + tanh(sqrt(2/pi) x (1 + 0.044715 x^2))), as the
+    reference's FFN halves use it (src/layers/ffn.h:24-27, src/models/pi0.cpp:229).  ggml's
+    CPU kernel reads a 16-bit lookup table for this function; the table is not reproduced
+    (parity unpinned at that level), the formula is."""
+    x = _f32(x).astype(np.float64)
+    return (0.5 * x * (1.0 + np.tanh(0.7978845608028654 * x * (1.0 + 0.044715 * x * x)))).astype(np.float32)
+
+
+def ffn_glu(x, Wg, Wu, Wd, act):
+    """Wd (act(Wg x) * (Wu x)): the gated FFN of the SmolVLA expert (act = silu,
+    src/models/smolvla.cpp:845-847) and of the Gemma expert (act = gelu, src/models/pi0.cpp:227-231)."""
+    return linear(act(linear(x, Wg)) * linear(x, Wu), Wd)
+
+
+def ffn_gelu(x, W1, b1, W2, b2):
+    """ffn_gelu (src/layers/ffn.h:24-27): W2 gelu(W1 x + b1) + b2."""
+    return linear(gelu(linear(x, W1, b1)), W2, b2)
+
+
 # ------------------------------------------------------------ concat / softmax
 def kv_concat(cache, suffix):
     """[P, ...] ++ [S, ...] along axis 0 into a fresh array (any dtype)."""

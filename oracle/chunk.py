@@ -182,6 +182,19 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
                 m = mask_cross if (pad[1] > pad[0]) else None
             att = rnd(orc.attention(q, K_full, V_full, m, scale))
             h = rnd(orc.linear(att, w[p + "Wo"], w.get(p + "bo")) + h)
+            if cfg.get("ffn_dim", 0) > 0:
+                # the FFN half of the layer (smolvla.cpp:845-848, pi0.cpp:227-232, dit_head.cpp:132-133)
+                I = cfg["ffn_dim"]
+                if gr00t:
+                    n3 = rnd(orc.layer_norm(h, None, None, eps))
+                    mid = rnd(orc.gelu(orc.linear(n3, w[p + "W1"], w[p + "b1"])))
+                    h = rnd(orc.linear(mid, w[p + "W2"], w[p + "b2"]) + h)
+                else:
+                    n2 = rnd(orc.rms_norm(h, w[p + "ln2"], eps))
+                    act = orc.silu if arch == "smolvla" else orc.gelu
+                    Wgu = w[p + "Wgu"]
+                    mid = rnd(act(orc.linear(n2, Wgu[:I])) * orc.linear(n2, Wgu[I:]))
+                    h = rnd(orc.linear(mid, w[p + "Wd"]) + h)
             if return_debug and s == 0 and l == 0:
                 debug["q0"], debug["att0"], debug["h0"] = q, att, h
         if gr00t:

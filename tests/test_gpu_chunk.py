@@ -126,6 +126,41 @@ def test_config3_gr00t_dit_bf16(tmp_path, n_layers, batch):
     m.close()
 
 
+@pytest.mark.parametrize("arch,dtype,n_layers,ffn_dim,batch", [
+    ("smolvla", "f32", 2, 256, 1),      # silu gate, fp32: 1e-5
+    ("smolvla", "bf16", 4, 2048, 2),    # the expert's real FFN width, pre-norm inside the gate/up launch
+    ("pi0", "bf16", 2, 4096, 1),        # gelu gate
+    ("gr00t", "bf16", 4, 6144, 2),      # LayerNorm -> ffn_gelu with biases
+])
+def test_whole_layers_with_the_ffn_half(tmp_path, arch, dtype, n_layers, ffn_dim, batch):
+    """The layers with their FFN half (not part of the BASELINE configurations, whose layers
+    stop after attention + Wo): post-attention norm, gated or plain FFN, residual."""
+    if arch == "smolvla":
+        cfg = ckpt.smolvla_config(n_layers=n_layers, dtype=dtype, suffix_mask=1)
+    elif arch == "pi0":
+        cfg = ckpt.pi0_config(n_layers=n_layers)
+    else:
+        cfg = ckpt.gr00t_config(n_layers=n_layers)
+    cfg["ffn_dim"] = ffn_dim
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 9)
+    r = np.random.default_rng(290 + ffn_dim)
+    obs = [make_obs(cfg, r, n_views=2) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "ffn_" + arch)
+    n_act = cfg["n_suffix"] - (0 if arch == "smolvla" else 1)
+    got = m.predict_batch(obs).reshape(batch, n_act, 32)
+    for b in range(batch):
+        if dtype == "f32":
+            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b])
+            assert rel_err(got[b], want) < 1e-5, rel_err(got[b], want)
+        else:
+            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+            assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    # without the FFN weights the same observation gives a different chunk: the half is really run
+    cfg0 = dict(cfg, ffn_dim=0)
+    assert not np.allclose(orc_chunk.flow_expert_chunk(cfg0, w, obs[0], emulate_bf16=dtype != "f32"), got[0], atol=1e-3)
+    m.close()
+
+
 @pytest.mark.parametrize("from_fp32", [False, True])
 def test_config4_bitvla_ternary_append(tmp_path, from_fp32):
     cfg = ckpt.bitvla_config(n_layers=2)

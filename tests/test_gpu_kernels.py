@@ -289,6 +289,56 @@ def test_rmsnorm_inside_qkv_launch(name, B, S, Hq, Hkv, D, K, self_layer, P):
         assert rel_err(gf, gp) < 8e-3
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("M,I,K,act,bias", [(50, 2048, 720, "silu", False), (130, 96, 72, "gelu", True), (1600, 256, 720, "silu", False),
+                                           (17, 6144, 1536, "gelu", True)])
+def test_glu_linear_and_linear_act(dtype, M, I, K, act, bias):
+    """Gate/up projection with the activation and the product in the epilogue, and the
+    activation between bias and residual of vla_linear_act, against the oracle."""
+    r = np.random.default_rng(1300 + M)
+    x = r.standard_normal((M, K)).astype(np.float32)
+    Wgu = (0.05 * r.standard_normal((2 * I, K))).astype(np.float32)
+    b = (0.1 * r.standard_normal(2 * I)).astype(np.float32) if bias else None
+    res = r.standard_normal((M, I)).astype(np.float32)
+    if dtype == BF16:
+        x, Wgu, res = orc.round_bf16(x), orc.round_bf16(Wgu), orc.round_bf16(res)
+    fact = orc.silu if act == "silu" else orc.gelu
+    code = pkg.VLA_ACT_SILU if act == "silu" else pkg.VLA_ACT_GELU
+    y = empty((M, I), dtype)
+    pkg.call("vla_glu_linear", to_dev(x, dtype), to_dev(Wgu, dtype), None if b is None else dev(b), y, dtype, dtype, M, I, K,
+             code, -1.0)
+    y2 = empty((M, I), dtype)
+    pkg.call("vla_linear_act", to_dev(x, dtype), to_dev(Wgu[:I], dtype), None if b is None else dev(b[:I]),
+             to_dev(res, dtype), y2, dtype, dtype, M, I, K, code)
+    sync()
+    gate = orc.linear(x, Wgu[:I], None if b is None else b[:I])
+    want = fact(gate) * orc.linear(x, Wgu[I:], None if b is None else b[I:])
+    want2 = fact(gate) + res
+    if dtype == F32:
+        assert rel_err(host(y), want) < FP32_TOL and rel_err(host(y2), want2) < FP32_TOL
+    else:
+        assert bf16_close(as_f32(y, dtype), want) and bf16_close(as_f32(y2, dtype), want2)
+    if dtype == BF16 and K % 16 == 0:
+        # the RMS pre-norm inside the launch (norm weight folded into both halves of the weights)
+        g = orc.round_bf16((1.0 + 0.3 * r.standard_normal(K)).astype(np.float32))
+        xs = orc.round_bf16(x * 3.0)
+        Wf = np.empty((2 * I, K), np.uint16)
+        assert pkg.lib().vla_fold_norm_weight_host(orc.to_bf16(Wgu).ctypes.data, orc.to_bf16(g).ctypes.data, BF16, 2 * I, K,
+                                                   Wf.ctypes.data) == 0
+        y3 = empty((M, I), BF16)
+        pkg.call("vla_glu_linear", to_dev(xs, BF16), dev(Wf), None, y3, BF16, BF16, M, I, K, code, 1e-5)
+        sync()
+        # exactly what the launch computes (unrounded normalised rows, weights folded and rounded once) ...
+        n0 = orc.rms_norm(xs, None, 1e-5)
+        Wfold = orc.from_bf16(Wf)
+        model = fact(orc.linear(n0, Wfold[:I])) * orc.linear(n0, Wfold[I:])
+        assert bf16_close(as_f32(y3, BF16), model)
+        # ... which stays within bf16 rounding of norm-then-project with the unfolded weights
+        n = orc.rms_norm(xs, g, 1e-5)
+        want3 = fact(orc.linear(n, Wgu[:I])) * orc.linear(n, Wgu[I:])
+        assert rel_err(as_f32(y3, BF16), want3) < 1e-2
+
+
 # ------------------------------------------------------------------ attention
 CASES = [
     # name, B, S, Hq, Hkv, D, P, mask kind, pad

@@ -180,6 +180,23 @@ def test_norms_against_torch():
     assert np.allclose(orc.adaln(x, sc, sh, 1e-5), xn * (1 + sc) + sh, rtol=1e-5, atol=1e-5)
     assert np.allclose(orc.silu(np.float32([0.0, 1.0, -2.0])),
                        torch.nn.functional.silu(torch.tensor([0.0, 1.0, -2.0])).numpy(), atol=1e-7)
+    # gelu, tanh form: known values, torch's tanh-approximate gelu, odd part x/2 (gelu(x) - gelu(-x) = x)
+    g = orc.gelu(np.float32([0.0, 1.0, -1.0, 3.0]))
+    assert np.allclose(g, [0.0, 0.8411919906, -0.1588080094, 2.9963626], atol=2e-7)
+    xs = np.linspace(-6, 6, 97).astype(np.float32)
+    assert np.allclose(orc.gelu(xs), torch.nn.functional.gelu(torch.tensor(xs), approximate="tanh").numpy(), atol=1e-6)
+    assert np.allclose(orc.gelu(xs) - orc.gelu(-xs), xs, atol=1e-6)
+    # the FFN compositions against a float64 evaluation of their definitions
+    xx = r.standard_normal((5, 24)).astype(np.float32)
+    Wg, Wu = r.standard_normal((32, 24)).astype(np.float32), r.standard_normal((32, 24)).astype(np.float32)
+    Wd, b1, b2 = r.standard_normal((24, 32)).astype(np.float32), r.standard_normal(32).astype(np.float32), r.standard_normal(24).astype(np.float32)
+    x64 = xx.astype(np.float64)
+    gate = x64 @ Wg.T.astype(np.float64)
+    want = ((gate / (1 + np.exp(-gate))) * (x64 @ Wu.T)) @ Wd.T.astype(np.float64)
+    assert np.allclose(orc.ffn_glu(xx, Wg, Wu, Wd, orc.silu), want, rtol=1e-5, atol=1e-4)
+    h = x64 @ Wg.T + b1
+    want = (0.5 * h * (1 + np.tanh(np.sqrt(2 / np.pi) * h * (1 + 0.044715 * h * h)))) @ Wd.T + b2
+    assert np.allclose(orc.ffn_gelu(xx, Wg, b1, Wd, b2), want, rtol=1e-5, atol=1e-4)
 
 
 # ---------------------------------------------------------- concat / softmax

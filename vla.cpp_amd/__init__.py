@@ -16,6 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libvla.so")
 
 VLA_DT_F32, VLA_DT_BF16, VLA_DT_BF16_P2 = 0, 1, 2
+VLA_ACT_NONE, VLA_ACT_SILU, VLA_ACT_GELU = 0, 1, 2
 VLA_MASK_NONE, VLA_MASK_CAUSAL_SUFFIX, VLA_MASK_PI0_STATE = 0, 1, 2
 VLA_K_OK, VLA_K_ERR_ARG, VLA_K_ERR_SHAPE, VLA_K_ERR_LAUNCH = 0, -1, -2, -3
 
@@ -32,6 +33,8 @@ KERNEL_API = {
     "vla_rms_norm": [_vp, _vp, _vp, _i, _i, _i, _f, _vp],
     "vla_adaln": [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _vp],
     "vla_linear": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "vla_linear_act": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "vla_glu_linear": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
     "vla_attn_qkv_rope": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
     "vla_rmsnorm_attn_qkv_rope": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _vp],
     "vla_fold_norm_weight_host": [_vp, _vp, _i, _i, _i, _vp],

@@ -172,6 +172,11 @@ def synth_weights(cfg, seed=0x5EED):
                 w[v + "bkv"] = vec(2 * kvd)
             w[p + "Wo"] = mat(W, qd)
             w[p + "bo"] = vec(W)
+            if cfg.get("ffn_dim", 0) > 0:  # ffn_gelu of the DiT block
+                w[p + "W1"] = mat(cfg["ffn_dim"], W)
+                w[p + "b1"] = vec(cfg["ffn_dim"])
+                w[p + "W2"] = mat(W, cfg["ffn_dim"])
+                w[p + "b2"] = vec(W)
             continue
         w[p + "ln"] = nrm(W)
         w[v + "ln"] = nrm(Wv)
@@ -183,6 +188,10 @@ def synth_weights(cfg, seed=0x5EED):
             w[p + "Wk_x"] = mat(kvd, kvd, 0.05)
             w[p + "Wv_x"] = mat(kvd, kvd, 0.05)
         w[p + "Wo"] = mat(W, qd)
+        if cfg.get("ffn_dim", 0) > 0:  # post-attention norm, [gate; up] rows, down
+            w[p + "ln2"] = nrm(W)
+            w[p + "Wgu"] = mat(2 * cfg["ffn_dim"], W)
+            w[p + "Wd"] = mat(W, cfg["ffn_dim"])
     return w
 
 
@@ -212,7 +221,7 @@ def write_synthetic(path, cfg, weights, ladder_pack=None, plain_pack=None):
             continue
         if name.endswith(".ws"):
             continue
-        small = name.startswith(_F32_NAMES) or name.endswith((".bqkv", ".bq", ".bo", ".bkv", ".adaln_b"))
+        small = name.startswith(_F32_NAMES) or name.endswith((".bqkv", ".bq", ".bo", ".bkv", ".adaln_b", ".b1", ".b2"))
         if cfg["arch"] == "bitvla" and name.endswith(("attn_norm", "sub_norm")):
             out[name] = BF16(t)
         elif bf and not small:

@@ -37,17 +37,18 @@ using namespace vk;
 constexpr int BN = 64;                     // epilogue sub-tile; column-tile unit of the N mapping
 constexpr int C_STRIDE = BN + 4;           // floats
 
-enum { EPI_PLAIN = 0, EPI_QKV = 1, EPI_TERNARY = 2 };
+enum { EPI_PLAIN = 0, EPI_QKV = 1, EPI_TERNARY = 2, EPI_GLU = 3 };
 
 struct GemmArgs {
     const void* A;
     const void* W;
     const float* bias;
     int M, N, K, n_tiles, xm, xn;
-    // PLAIN
+    // PLAIN, GLU
     const void* residual;
     void* Y;
     int out_bf16;
+    int act;  // VLA_ACT_*: PLAIN applies it after the bias, GLU to the gate
     // QKV
     int S, Hq, nk, nv, D;
     const float* cos_t;
@@ -109,6 +110,13 @@ __host__ __device__ __forceinline__ long tern_word_index(long n, int w, int K) {
 __device__ __forceinline__ uint32_t acc_bits(float v) { return __float_as_uint(v); }
 __device__ __forceinline__ uint32_t acc_bits(int v) { return (uint32_t)v; }
 
+// ggml_silu / ggml_gelu (tanh form), fp32 (src/layers/ffn.h:24-40).
+__device__ __forceinline__ float apply_act(float x, int act) {
+    if (act == VLA_ACT_SILU) return x / (1.0f + __expf(-x));
+    if (act == VLA_ACT_GELU) return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
+    return x;
+}
+
 // W-row bases of the two 32-column halves of output tile `nt`.
 struct TileCols {
     int base0, base1;  // rows of W feeding tile columns [0,32) and [32,64)
@@ -120,6 +128,15 @@ struct TileCols {
 template <int kEpi>
 __device__ __forceinline__ TileCols tile_cols(const GemmArgs& a, int nt) {
     TileCols t;
+    if (kEpi == EPI_GLU) {  // W = [gate rows; up rows]: the tile pairs 32 gate columns with their up columns
+        t.base0 = nt * 32;
+        t.base1 = a.N / 2 + nt * 32;
+        t.seg = 0;
+        t.col0 = t.base0;
+        t.col1 = t.base1;
+        t.rope = false;
+        return t;
+    }
     if (kEpi != EPI_QKV) {
         t.base0 = nt * BN;
         t.base1 = t.base0 + 32;
@@ -204,6 +221,33 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
         }
     }
 
+    if (kEpi == EPI_GLU) {
+        // lo = gate columns nt*32 + jg .. +7, hi = the up columns of the same outputs
+        const int I = a.N / 2, n0 = nt * 32 + jg;  // I is a multiple of 32: the 8 outputs are inside the row
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float gt = lo[e], up = hi[e];
+            if (a.bias) {
+                gt += a.bias[n0 + e];
+                up += a.bias[I + n0 + e];
+            }
+            v[e] = apply_act(gt, a.act) * up;
+        }
+        const long o = (long)m * I + n0;
+        if (a.out_bf16) {
+            const u32x4_t pk = {pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3]), pack_bf2(v[4], v[5]), pack_bf2(v[6], v[7])};
+            *reinterpret_cast<u32x4_t*>((bf16_t*)a.Y + o) = pk;
+        } else {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const f32x4_t pk = {v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+                *reinterpret_cast<f32x4_t*>((float*)a.Y + o + 4 * q) = pk;
+            }
+        }
+        return;
+    }
+
     if (kEpi == EPI_PLAIN) {
 #pragma unroll
         for (int hlf = 0; hlf < 2; ++hlf) {
@@ -216,6 +260,10 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
 #pragma unroll
                 for (int e = 0; e < 8; ++e)
                     if (n0 + e < a.N) v[e] += a.bias[n0 + e];
+            }
+            if (a.act != VLA_ACT_NONE) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = apply_act(v[e], a.act);
             }
             if (full && a.out_bf16) {  // 8 consecutive bf16 = one 16-byte access each way
                 if (a.residual) {
@@ -1083,7 +1131,7 @@ void launch_cfg(GemmArgs a, hipStream_t st) {
 template <int kEpi, int TM, int TN, int KB, int NS>
 void launch_dl(GemmArgs a, hipStream_t st) {
     const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, 1.0);
-    if constexpr (kEpi == EPI_QKV) {
+    if constexpr (kEpi == EPI_QKV || kEpi == EPI_GLU) {
         if (a.norm_eps >= 0.f) {
             gemm_dl_kernel<kEpi, TM, TN, KB, NS, true><<<grid, 256, 0, st>>>(a);
             return;
@@ -1120,7 +1168,7 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             const char* e = getenv("VLA_GEMM_DL");
             dl = !(e && atoi(e) == 0) && a.K % 16 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
         }
-        if (a.norm_eps >= 0.f && !(dl && kEpi == EPI_QKV)) return VLA_K_ERR_SHAPE;  // only that kernel takes the row statistics
+        if (a.norm_eps >= 0.f && !(dl && (kEpi == EPI_QKV || kEpi == EPI_GLU))) return VLA_K_ERR_SHAPE;  // only that kernel takes the row statistics
         if (dl) {
             const char* es = getenv("VLA_GEMM_STAGES");
             int ns = es ? atoi(es) : 0;
@@ -1263,6 +1311,49 @@ int vla_attn_qkv_rope(const void* x, const void* W, const float* bias, int dtype
                       void* q_out, void* k_cache, void* vt_cache, int t_max, int tok_offset, vla_stream_t stream) {
     return qkv_rope_impl(x, W, bias, dtype, M, K, S, n_q_heads, n_kv_heads, has_k, has_v, head_dim, cos_tab, sin_tab, q_out,
                          k_cache, vt_cache, t_max, tok_offset, -1.f, stream);
+}
+
+int vla_linear_act(const void* x, const void* W, const float* bias, const void* residual, void* y, int dtype,
+                   int out_dtype, int M, int N, int K, int act, vla_stream_t stream) {
+    if (!x || !W || !y || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (out_dtype != VLA_DT_F32 && out_dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
+    if (act < VLA_ACT_NONE || act > VLA_ACT_GELU) return VLA_K_ERR_ARG;
+    GemmArgs a = {};
+    a.norm_eps = -1.f;
+    a.A = x; a.W = W; a.bias = bias; a.M = M; a.N = N; a.K = K;
+    a.residual = residual; a.Y = y; a.out_bf16 = (out_dtype == VLA_DT_BF16); a.act = act;
+    const int nt = (N + BN - 1) / BN;
+    if (dtype == VLA_DT_BF16) {
+        if (K % 8) return VLA_K_ERR_SHAPE;
+        return launch<bf16_t, EPI_PLAIN>(a, nt, stream);
+    }
+    if (dtype == VLA_DT_F32) {
+        if (K % 4) return VLA_K_ERR_SHAPE;
+        return launch<float, EPI_PLAIN>(a, nt, stream);
+    }
+    return VLA_K_ERR_ARG;
+}
+
+int vla_glu_linear(const void* x, const void* W_gate_up, const float* bias, void* y, int dtype, int out_dtype, int M, int I,
+                   int K, int act, float rms_eps, vla_stream_t stream) {
+    if (!x || !W_gate_up || !y || M < 0 || I <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (out_dtype != VLA_DT_F32 && out_dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
+    if (act < VLA_ACT_NONE || act > VLA_ACT_GELU) return VLA_K_ERR_ARG;
+    if (I % 32) return VLA_K_ERR_SHAPE;  // a tile pairs 32 gate columns with their 32 up columns
+    GemmArgs a = {};
+    a.norm_eps = rms_eps >= 0.f ? rms_eps : -1.f;
+    a.A = x; a.W = W_gate_up; a.bias = bias; a.M = M; a.N = 2 * I; a.K = K;
+    a.Y = y; a.out_bf16 = (out_dtype == VLA_DT_BF16); a.act = act;
+    const int nt = I / 32;
+    if (dtype == VLA_DT_BF16) {
+        if (K % 8) return VLA_K_ERR_SHAPE;
+        return launch<bf16_t, EPI_GLU>(a, nt, stream);
+    }
+    if (dtype == VLA_DT_F32) {
+        if (K % 4) return VLA_K_ERR_SHAPE;
+        return launch<float, EPI_GLU>(a, nt, stream);
+    }
+    return VLA_K_ERR_ARG;
 }
 
 int vla_rmsnorm_attn_qkv_rope(const void* x, const void* W_folded, const float* bias, int dtype, int M, int K, int S,

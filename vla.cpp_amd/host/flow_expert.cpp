@@ -82,6 +82,8 @@ struct LayerW {
     DevBuf Wqkv, bqkv;          // self: Q|K|V rows, cross: Q rows
     DevBuf Wqkv_ln;             // the same rows with the pre-norm weight folded in (bf16 RMS archs)
     DevBuf Wo, bo;
+    DevBuf ln2, Wgu, Wgu_ln, Wd;      // FFN half of an RMS-norm layer: post-attention norm, [gate; up], down
+    DevBuf W1, b1, W2, b2;            // FFN half of a DiT block (ffn_gelu)
     DevBuf vlm_ln, Wkv_pre, bkv_pre;  // prefix K|V producer
     DevBuf Wk_x, Wv_x;          // SmolVLA cross layers: re-projection of the cached prefix K / V
     KVLayer kv;
@@ -109,6 +111,7 @@ class FlowExpert : public ModelArch {
     Arch arch_;
     int dt_ = VLA_DT_F32;
     int L_ = 0, Hq_ = 0, Hkv_ = 0, D_ = 0, W_ = 0, Wv_ = 0, A_ = 0, S_ = 0, n_lead_ = 0, steps_ = 0;
+    int I_ = 0;  // FFN width; 0 = the layers stop after the attention half
     int n_img_ = 0, n_lang_max_ = 0, max_views_ = 1, vocab_ = 0, max_state_ = 0;
     int suffix_mask_ = VLA_MASK_NONE;
     float eps_ = 1e-5f, final_eps_ = 1e-6f, dt_step_ = -0.1f;
@@ -124,7 +127,7 @@ class FlowExpert : public ModelArch {
     // per-call state
     int B_ = 0, P_ = 0, pad_start_ = 0, pad_end_ = 0;
     RopeTable rope_prefill_, rope_self_, rope_cross_;
-    DevBuf prefix_, prefix_n_, tmpk_, tmpv_, lead_, x0_, xt_, h_, hn_, q_, att_;
+    DevBuf prefix_, prefix_n_, tmpk_, tmpv_, lead_, x0_, xt_, h_, hn_, q_, att_, mid_;
     KVLayer tmp_kv_;
     std::mt19937 rng_{std::random_device{}()};
     hipStream_t last_stream_ = nullptr;
@@ -139,6 +142,7 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     Hkv_ = (int)ck.i64("n_kv_heads");
     D_ = (int)ck.i64("head_dim");
     W_ = (int)ck.i64("expert_h");
+    I_ = (int)ck.i64("ffn_dim", 0);
     Wv_ = (int)ck.i64("hidden");
     A_ = (int)ck.i64("max_action_dim");
     S_ = (int)ck.i64("n_suffix");
@@ -214,6 +218,18 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         if (ck.has(p + (w.is_self ? "bqkv" : "bq"))) w.bqkv = load_f32(ck, p + (w.is_self ? "bqkv" : "bq"));
         w.Wo = load_w(ck, p + "Wo", dt_);
         if (ck.has(p + "bo")) w.bo = load_f32(ck, p + "bo");
+        if (I_ > 0 && arch_ == Arch::GR00T) {
+            w.W1 = load_w(ck, p + "W1", dt_);
+            w.b1 = load_f32(ck, p + "b1");
+            w.W2 = load_w(ck, p + "W2", dt_);
+            w.b2 = load_f32(ck, p + "b2");
+        } else if (I_ > 0) {
+            w.ln2 = load_w(ck, p + "ln2", dt_);
+            w.Wgu = load_w(ck, p + "Wgu", dt_);
+            w.Wd = load_w(ck, p + "Wd", dt_);
+            if (dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
+                w.Wgu_ln = load_folded_bf16(ck, p + "Wgu", p + "ln2");
+        }
         if (w.needs_prefix) {
             const std::string v = "vlm." + std::to_string(l) + ".";
             if (arch_ != Arch::GR00T) w.vlm_ln = load_w(ck, v + "ln", dt_);
@@ -300,6 +316,7 @@ void FlowExpert::allocate(int B, int P) {
     hn_.alloc((size_t)B * S_ * W_ * es);
     q_.alloc((size_t)B * S_ * Hq_ * D_ * es);
     att_.alloc((size_t)B * S_ * Hq_ * D_ * es);
+    if (I_ > 0) mid_.alloc((size_t)B * S_ * I_ * es);
 }
 
 void FlowExpert::prefill(const Inputs* in, int batch) {
@@ -469,6 +486,29 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 flash_attention(C, Q, w.kv, n_keys, mask, scale, att);
                 Tensor Wo = tensor_2d(w.Wo.get(), dt_, (int64_t)Hq_ * D_, W_);
                 linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
+                if (I_ > 0) {
+                    // FFN half (smolvla.cpp:845-848, pi0.cpp:227-232, dit_head.cpp:132-133)
+                    Tensor mid = tensor_2d(mid_.get(), dt_, I_, M);
+                    if (arch_ == Arch::GR00T) {
+                        const float* z = ada_.as<float>() + ((size_t)s * (L_ + 1) + L_) * 2 * W_;  // zeros: plain LayerNorm
+                        adaln(C, h, z, z + W_, eps_, hn);
+                        Tensor W1 = tensor_2d(w.W1.get(), dt_, W_, I_), W2 = tensor_2d(w.W2.get(), dt_, I_, W_);
+                        ffn_gelu(C, W1, w.b1.as<float>(), W2, w.b2.as<float>(), hn, h.data, mid, h);
+                    } else {
+                        const int act = arch_ == Arch::SMOLVLA ? VLA_ACT_SILU : VLA_ACT_GELU;
+                        Tensor Wd = tensor_2d(w.Wd.get(), dt_, I_, W_);
+                        bool fused = false;
+                        if (w.Wgu_ln) {
+                            Tensor Wf = tensor_2d(w.Wgu_ln.get(), dt_, W_, 2 * (int64_t)I_);
+                            fused = ffn_glu(C, Wf, act, Wd, h, eps_, h.data, mid, h);
+                        }
+                        if (!fused) {
+                            rms_norm(C, h, w.ln2.get(), eps_, hn);
+                            Tensor Wgu = tensor_2d(w.Wgu.get(), dt_, W_, 2 * (int64_t)I_);
+                            ffn_glu(C, Wgu, act, Wd, hn, -1.f, h.data, mid, h);
+                        }
+                    }
+                }
             }
             if (arch_ == Arch::GR00T) {
                 const float* z = ada_.as<float>() + ((size_t)s * (L_ + 1) + L_) * 2 * W_;  // zeros: plain LayerNorm

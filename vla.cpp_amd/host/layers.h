@@ -86,6 +86,34 @@ inline void linear(Ctx& C, const Tensor& W, const float* b, const Tensor& x, con
                      C.stream));
 }
 
+// ffn.h:24-27 (ffn_gelu) with the residual add that follows it in DitHead::block
+// (src/modules/dit_head.cpp:133): y = residual + W2 gelu(W1 x + b1) + b2.  `mid` is scratch
+// for the activated intermediate [rows][W1 rows].
+inline void ffn_gelu(Ctx& C, const Tensor& W1, const float* b1, const Tensor& W2, const float* b2, const Tensor& x,
+                     const void* residual, Tensor& mid, Tensor& y) {
+    VLA_K(vla_linear_act(x.data, W1.data, b1, nullptr, mid.data, x.dtype, mid.dtype, (int)x.rows(), (int)W1.ne[1],
+                         (int)W1.ne[0], VLA_ACT_GELU, C.stream));
+    VLA_K(vla_linear(mid.data, W2.data, b2, residual, y.data, mid.dtype, y.dtype, (int)mid.rows(), (int)W2.ne[1],
+                     (int)W2.ne[0], C.stream));
+}
+
+// ffn.h:35-40 (ffn_swiglu) generalised over the gate activation (ggml_silu in the SmolVLA
+// expert, ggml_gelu in the Gemma expert), without biases, with the residual add that follows:
+// y = residual + Wd (act(Wg x) * (Wu x)).  Wgu holds the gate rows, then the up rows.  With
+// rms_eps >= 0, x is the un-normalised stream and Wgu carries the post-attention norm
+// weight (vla_fold_norm_weight_host); returns false, launching nothing, when the shapes do
+// not fit that fused launch.
+inline bool ffn_glu(Ctx& C, const Tensor& Wgu, int act, const Tensor& Wd, const Tensor& x, float rms_eps,
+                    const void* residual, Tensor& mid, Tensor& y) {
+    const int rc = vla_glu_linear(x.data, Wgu.data, nullptr, mid.data, x.dtype, mid.dtype, (int)x.rows(),
+                                  (int)(Wgu.ne[1] / 2), (int)Wgu.ne[0], act, rms_eps, C.stream);
+    if (rc == VLA_K_ERR_SHAPE && rms_eps >= 0.f) return false;
+    VLA_K(rc);
+    VLA_K(vla_linear(mid.data, Wd.data, nullptr, residual, y.data, mid.dtype, y.dtype, (int)mid.rows(), (int)Wd.ne[1],
+                     (int)Wd.ne[0], C.stream));
+    return true;
+}
+
 // norm.h:31-34.
 inline void rms_norm(Ctx& C, const Tensor& x, const void* w, float eps, Tensor& y) {
     VLA_K(vla_rms_norm(x.data, w, y.data, x.dtype, (int)x.rows(), (int)x.ne[0], eps, C.stream));
