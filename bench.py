@@ -43,6 +43,11 @@ def workloads():
         "cfg2_pi0_18layer_bf16_b16": dict(cfg=ck.pi0_config(18), B=16, views=3),
         "cfg3_gr00t_16dit_bf16_b1": dict(cfg=ck.gr00t_config(16), B=1, views=2),
         "cfg3_gr00t_16dit_bf16_b64": dict(cfg=ck.gr00t_config(16), B=64, views=2),
+        # beyond the BASELINE configurations: the same stacks with the FFN half of every layer
+        "whole_smolvla_16layer_bf16_b32": dict(cfg=dict(ck.smolvla_config(16, "bf16", 0), ffn_dim=2048), B=32, views=3),
+        "whole_smolvla_16layer_bf16_b1": dict(cfg=dict(ck.smolvla_config(16, "bf16", 0), ffn_dim=2048), B=1, views=3),
+        "whole_pi0_18layer_bf16_b16": dict(cfg=dict(ck.pi0_config(18), ffn_dim=4096), B=16, views=3),
+        "whole_gr00t_16dit_bf16_b64": dict(cfg=dict(ck.gr00t_config(16), ffn_dim=6144), B=64, views=2),
         "cfg4_bitvla_30layer_b1": dict(cfg=ck.bitvla_config(30), B=1, views=1),
         "cfg4_bitvla_30layer_b8": dict(cfg=ck.bitvla_config(30), B=8, views=1),
     }
@@ -222,6 +227,23 @@ def kernel_breakdown(pkg, cfg, B, P):
                                                 P, scale, 0, P, 0, 0, None),
             n_cross, "hbm", 2 * P * kvd * es * B)
     add("wo_residual", lambda i: pkg.call("vla_linear", att, Wo, None, h, h, dt, dt, M, W, qd), L, "mfma", 2.0 * M * W * qd)
+    I = cfg.get("ffn_dim", 0)
+    if I > 0:  # the FFN half of every layer (workloads beyond the BASELINE configurations)
+        mid = z(M, I)
+        if gr00t:
+            W1, W2, b1, b2 = rnd(I, W), rnd(W, I), torch.zeros(I, device=dev), torch.zeros(W, device=dev)
+            out["adaln"]["per_step"] += L
+            add("ffn_in_gelu", lambda i: pkg.call("vla_linear_act", hn, W1, b1, None, mid, dt, dt, M, I, W, pkg.VLA_ACT_GELU), L,
+                "mfma", 2.0 * M * I * W)
+            add("ffn_out_residual", lambda i: pkg.call("vla_linear", mid, W2, b2, h, h, dt, dt, M, W, I), L, "mfma", 2.0 * M * I * W)
+        else:
+            Wgu, Wd = rnd(2 * I, W), rnd(W, I)
+            act = pkg.VLA_ACT_SILU if arch == "smolvla" else pkg.VLA_ACT_GELU
+            if not fused_norm:
+                out["rms_norm"]["per_step"] += L
+            add("ffn_gate_up", lambda i: pkg.call("vla_glu_linear", h if fused_norm else hn, Wgu, None, mid, dt, dt, M, I, W, act,
+                                                  1e-5 if fused_norm else -1.0), L, "mfma", 4.0 * M * I * W)
+            add("ffn_down_residual", lambda i: pkg.call("vla_linear", mid, Wd, None, h, h, dt, dt, M, W, I), L, "mfma", 2.0 * M * I * W)
     add("euler_step", lambda i: pkg.call("vla_euler_step", xt, hn, W_out, b_out, dt, B, S, n_lead, A, W, -0.1), 1, "hbm",
         M * W * es)
     return out
