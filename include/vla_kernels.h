@@ -200,6 +200,20 @@ VLA_KAPI int vla_embed_suffix(const float* x_t, const float* W_in, const float* 
                               void* h, int out_dtype, int batch, int S, int n_lead, int A, int W,
                               vla_stream_t stream);
 
+/* The same with an activation on the projected rows (lead rows are copied as they are):
+ * the first projection of the action-time MLP of build_embed_suffix
+ * (src/models/smolvla.cpp:1397-1403, src/models/pi0.cpp:240-244) with the time half of its
+ * input folded into bias_step. */
+VLA_KAPI int vla_embed_suffix_act(const float* x_t, const float* W_in, const float* bias_step, const float* lead,
+                                  void* h, int out_dtype, int batch, int S, int n_lead, int A, int W, int act,
+                                  vla_stream_t stream);
+
+/* h[b][s][:] = lead[b][s][:] for s < n_lead, converted to `dtype`: the state-token rows
+ * of ggml_concat(state_emb, action_time_emb) (src/models/pi0.cpp:245-246) when the action
+ * rows were produced by a projection over all S rows of the suffix. */
+VLA_KAPI int vla_set_lead_rows(const float* lead, void* h, int dtype, int batch, int S, int n_lead, int W,
+                               vla_stream_t stream);
+
 /* Output projection + Euler update (src/models/smolvla.cpp:1416-1418,
  * src/models/pi0.cpp:577-587): x_t[b][s] += dt * (W_out . hn[b][n_lead + s] + b_out).
  *   hn [batch][S][W] in `dtype` (already normalised); W_out fp32 [A][W]. */

@@ -150,7 +150,16 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
         if not gr00t:
             t = np.float32(1.0) + np.float32(s) * dt32
             bias = bias + orc.sinusoidal_time_emb(float(t), W, cfg["min_period"], cfg["max_period"])
-        h = orc.linear(x, w["act.W_in"], bias)
+        if "act.W_at1" in w and not gr00t:
+            # action-time MLP (smolvla.cpp:1397-1403, pi0.cpp:240-244), in the reference's order
+            t = np.float32(1.0) + np.float32(s) * dt32
+            temb = orc.sinusoidal_time_emb(float(t), W, cfg["min_period"], cfg["max_period"])
+            action_emb = orc.linear(x, w["act.W_in"], w["act.b_in"])
+            cat = np.concatenate([action_emb, np.broadcast_to(temb, action_emb.shape)], 1)
+            mlp1 = orc.linear(cat, w["act.W_at1"], w["act.b_at1"])
+            h = orc.linear(orc.silu(mlp1), w["act.W_at2"], w["act.b_at2"])
+        else:
+            h = orc.linear(x, w["act.W_in"], bias)
         if n_lead:
             h = np.concatenate([lead, h], 0)
         h = rnd(h)

@@ -161,6 +161,30 @@ def test_whole_layers_with_the_ffn_half(tmp_path, arch, dtype, n_layers, ffn_dim
     m.close()
 
 
+@pytest.mark.parametrize("arch,dtype,batch", [("smolvla", "f32", 1), ("smolvla", "bf16", 3), ("pi0", "bf16", 2)])
+def test_suffix_embedding_with_the_action_time_mlp(tmp_path, arch, dtype, batch):
+    """The suffix embedding through its real action-time MLP (the BASELINE configurations use
+    W_in x + b + time embedding): the library folds the first two projections into one matrix
+    and a per-step bias, the oracle follows the reference's order."""
+    cfg = ckpt.smolvla_config(n_layers=2, dtype=dtype, suffix_mask=1) if arch == "smolvla" else ckpt.pi0_config(n_layers=2)
+    cfg["time_mlp"] = 1
+    cfg["ffn_dim"] = 256
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 11)
+    r = np.random.default_rng(300 + batch)
+    obs = [make_obs(cfg, r, n_views=2) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "tmlp_" + arch)
+    got = m.predict_batch(obs).reshape(batch, 50, 32)
+    for b in range(batch):
+        want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=dtype != "f32")
+        if dtype == "f32":
+            assert rel_err(got[b], want) < 1e-5, rel_err(got[b], want)
+        else:
+            assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    w0 = {k: v for k, v in w.items() if not k.startswith("act.W_at") and not k.startswith("act.b_at")}
+    assert not np.allclose(orc_chunk.flow_expert_chunk(cfg, w0, obs[0], emulate_bf16=dtype != "f32"), got[0], atol=1e-3)
+    m.close()
+
+
 @pytest.mark.parametrize("from_fp32", [False, True])
 def test_config4_bitvla_ternary_append(tmp_path, from_fp32):
     cfg = ckpt.bitvla_config(n_layers=2)

@@ -744,6 +744,18 @@ def test_embed_suffix_and_euler_step(out_dtype):
     want = np.concatenate([lead, (orc.linear(x_t.reshape(-1, A), W_in, bias)).reshape(B, S - n_lead, W)], axis=1)
     got = as_f32(h, out_dtype)
     assert rel_err(got, want) < (FP32_TOL if out_dtype == F32 else 8e-3)
+    # with an activation on the projected rows (lead rows are copied as they are), and the
+    # state-token rows written over a buffer afterwards
+    h2 = empty((B, S, W), out_dtype)
+    pkg.call("vla_embed_suffix_act", dev(x_t), dev(W_in), dev(bias), dev(lead), h2, out_dtype, B, S, n_lead, A, W, pkg.VLA_ACT_SILU)
+    h3 = empty((B, S, W), out_dtype)
+    pkg.call("vla_set_lead_rows", dev(lead), h3, out_dtype, B, S, n_lead, W)
+    sync()
+    want2 = want.copy()
+    want2[:, n_lead:] = orc.silu(want[:, n_lead:])
+    assert rel_err(as_f32(h2, out_dtype), want2) < (FP32_TOL if out_dtype == F32 else 8e-3)
+    got3 = as_f32(h3, out_dtype)
+    assert not got3[:, n_lead:].any() and rel_err(got3[:, :n_lead], lead) < (1e-7 if out_dtype == F32 else 8e-3)
     W_out = (0.05 * r.standard_normal((A, W))).astype(np.float32)
     b_out = r.standard_normal(A).astype(np.float32)
     xd = dev(x_t)

@@ -41,6 +41,8 @@ KERNEL_API = {
     "vla_qkv_split_rope_append": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "vla_attn_prefix_suffix": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp],
     "vla_embed_suffix": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "vla_embed_suffix_act": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "vla_set_lead_rows": [_vp, _vp, _i, _i, _i, _i, _i, _vp],
     "vla_euler_step": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
     "vla_act_quant_bf16": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "vla_ternary_quant_host": [_vp, _i64, _vp, _vp],

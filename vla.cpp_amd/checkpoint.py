@@ -151,6 +151,11 @@ def synth_weights(cfg, seed=0x5EED):
     w["act.b_out"] = vec(A)
     if arch != "gr00t_n1d5":
         w["act.norm"] = nrm(W)
+        if cfg.get("time_mlp", 0):  # action_time_mlp_in / _out of the suffix embedding
+            w["act.W_at1"] = (r.standard_normal((W, 2 * W)) / np.sqrt(2 * W)).astype(np.float32)
+            w["act.b_at1"] = vec(W, 0.1)
+            w["act.W_at2"] = (r.standard_normal((W, W)) / np.sqrt(W)).astype(np.float32)
+            w["act.b_at2"] = vec(W, 0.1)
     else:
         w["te.l1W"] = (0.05 * r.standard_normal((W, 256))).astype(np.float32)
         w["te.l1b"] = vec(W)

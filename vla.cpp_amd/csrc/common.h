@@ -1,6 +1,7 @@
 // Shared device helpers for the gfx950 kernels: bf16 bit conversions, vector
 // types, wavefront (64-lane) reductions and the MFMA fragment typedefs.
 #pragma once
+#include "vla_kernels.h"
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -89,6 +90,13 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     float r = 0.f;
     for (int i = 0; i < nw; ++i) r += red[i];
     return r;
+}
+
+// ggml_silu / ggml_gelu (tanh form), fp32 (src/layers/ffn.h:24-40).
+__device__ __forceinline__ float apply_act(float x, int act) {
+    if (act == VLA_ACT_SILU) return x / (1.0f + __expf(-x));
+    if (act == VLA_ACT_GELU) return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
+    return x;
 }
 
 // s_waitcnt on the vector-memory counter alone (vmcnt[3:0] in bits 3:0, vmcnt[5:4] in bits

@@ -284,7 +284,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restrict__ x_t, const float* __restrict__ W_in,
                                                             const float* __restrict__ bias_step,
                                                             const float* __restrict__ lead, T* __restrict__ h, int n_rows,
-                                                            int S, int n_lead, int A, int W) {
+                                                            int S, int n_lead, int A, int W, int act) {
     __shared__ float xs[EMB_ROWS][EMB_MAX_A];
     __shared__ float ws[EMB_COLS][EMB_MAX_A + 1];
     const int row0 = blockIdx.x * EMB_ROWS, c0 = blockIdx.y * EMB_COLS;
@@ -315,10 +315,23 @@ __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restri
         } else {
             float acc = 0.f;
             for (int a = 0; a < A; ++a) acc += ws[cl][a] * xs[rr][a];
-            v = acc + bias;
+            v = apply_act(acc + bias, act);
         }
         Elem<T>::store(h + (long)row * W + c, v);
     }
+}
+
+// h[b][s][:] = lead[b][s][:] for s < n_lead (the state token rows of a suffix whose action
+// rows came out of a projection over all rows).
+template <typename T>
+__global__ void lead_rows_kernel(const float* __restrict__ lead, T* __restrict__ h, long total, int S, int n_lead, int W) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int c = (int)(i % W);
+    const long bs = i / W;
+    const int s = (int)(bs % n_lead);
+    const long b = bs / n_lead;
+    Elem<T>::store(h + ((long)b * S + s) * W + c, lead[i]);
 }
 
 // Workgroup (x, y): EUL_WAVES wavefronts, each owning ROWS action rows, all working on the
@@ -607,8 +620,25 @@ int vla_adaln(const void* x, const float* sc, const float* sh, void* y, int dtyp
 
 int vla_embed_suffix(const float* x_t, const float* W_in, const float* bias_step, const float* lead, void* h,
                      int out_dtype, int batch, int S, int n_lead, int A, int W, vla_stream_t stream) {
+    return vla_embed_suffix_act(x_t, W_in, bias_step, lead, h, out_dtype, batch, S, n_lead, A, W, VLA_ACT_NONE, stream);
+}
+
+int vla_set_lead_rows(const float* lead, void* h, int dtype, int batch, int S, int n_lead, int W, vla_stream_t stream) {
+    if (!lead || !h || batch < 0 || S <= 0 || n_lead <= 0 || n_lead > S || W <= 0) return VLA_K_ERR_ARG;
+    if (batch == 0) return VLA_K_OK;
+    const long total = (long)batch * n_lead * W;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (dtype == VLA_DT_F32) lead_rows_kernel<float><<<blocks, 256, 0, (hipStream_t)stream>>>(lead, (float*)h, total, S, n_lead, W);
+    else if (dtype == VLA_DT_BF16) lead_rows_kernel<bf16_t><<<blocks, 256, 0, (hipStream_t)stream>>>(lead, (bf16_t*)h, total, S, n_lead, W);
+    else return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_embed_suffix_act(const float* x_t, const float* W_in, const float* bias_step, const float* lead, void* h,
+                         int out_dtype, int batch, int S, int n_lead, int A, int W, int act, vla_stream_t stream) {
     if (!x_t || !W_in || !bias_step || !h || batch < 0 || S <= 0 || n_lead < 0 || n_lead > S || A <= 0 || W <= 0)
         return VLA_K_ERR_ARG;
+    if (act < VLA_ACT_NONE || act > VLA_ACT_GELU) return VLA_K_ERR_ARG;
     if (n_lead > 0 && !lead) return VLA_K_ERR_ARG;
     if (A > EMB_MAX_A) return VLA_K_ERR_SHAPE;
     if (batch == 0) return VLA_K_OK;
@@ -616,9 +646,9 @@ int vla_embed_suffix(const float* x_t, const float* W_in, const float* bias_step
     const int n_rows = batch * S;
     const dim3 blocks((n_rows + EMB_ROWS - 1) / EMB_ROWS, (W + EMB_COLS - 1) / EMB_COLS);
     if (out_dtype == VLA_DT_F32)
-        embed_suffix_kernel<float><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W);
+        embed_suffix_kernel<float><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W, act);
     else if (out_dtype == VLA_DT_BF16)
-        embed_suffix_kernel<bf16_t><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W);
+        embed_suffix_kernel<bf16_t><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W, act);
     else
         return VLA_K_ERR_ARG;
     return VLA_CHECK_LAUNCH();

@@ -110,13 +110,6 @@ __host__ __device__ __forceinline__ long tern_word_index(long n, int w, int K) {
 __device__ __forceinline__ uint32_t acc_bits(float v) { return __float_as_uint(v); }
 __device__ __forceinline__ uint32_t acc_bits(int v) { return (uint32_t)v; }
 
-// ggml_silu / ggml_gelu (tanh form), fp32 (src/layers/ffn.h:24-40).
-__device__ __forceinline__ float apply_act(float x, int act) {
-    if (act == VLA_ACT_SILU) return x / (1.0f + __expf(-x));
-    if (act == VLA_ACT_GELU) return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
-    return x;
-}
-
 // W-row bases of the two 32-column halves of output tile `nt`.
 struct TileCols {
     int base0, base1;  // rows of W feeding tile columns [0,32) and [32,64)

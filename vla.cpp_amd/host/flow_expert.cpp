@@ -121,6 +121,8 @@ class FlowExpert : public ModelArch {
     // small fp32 tensors kept on the host for per-observation work
     std::vector<float> E_lang_, Wstate_, bstate_, W_sp_, b_sp_;
     DevBuf W_in_, W_out_, b_out_, final_norm_;
+    DevBuf W_at2_, b_at2_, m1_;  // action-time MLP: second projection, fp32 scratch [B*S][W]
+    bool time_mlp_ = false;
     DevBuf bias_step_;   // [steps][W] fp32: b_in (+ time embedding of the step)
     DevBuf ada_;         // GR00T: [steps][L+1][2][W] fp32 (scale, shift); slot L is the final norm (zeros)
 
@@ -246,13 +248,44 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     // so it is evaluated once here instead of inside every denoise step.
     const std::vector<float> b_in = ck.f32("act.b_in");
     std::vector<float> bias((size_t)steps_ * W_);
-    for (int s = 0; s < steps_; ++s) {
-        for (int c = 0; c < W_; ++c) bias[(size_t)s * W_ + c] = b_in[c];
-        if (arch_ != Arch::GR00T) {
-            // t = 1 + step*dt (src/models/pi0.cpp:654-656), embedding of src/layers/embed.h:61-73
+    time_mlp_ = arch_ != Arch::GR00T && ck.has("act.W_at1");
+    if (time_mlp_) {
+        // Action-time MLP (src/models/smolvla.cpp:1397-1403, src/models/pi0.cpp:240-244):
+        //   mlp1 = W_at1 . concat(W_in x + b_in, time_s) + b_at1,  suffix = W_at2 silu(mlp1) + b_at2.
+        // W_at1 = [Wa | Wt] by columns, so mlp1 = (Wa W_in) x + (Wa b_in + Wt time_s + b_at1):
+        // the first two projections collapse into one [W][A] matrix and a per-step bias,
+        // both formed here once (double accumulation), and the embed kernel applies the silu.
+        const std::vector<float> W_in = ck.f32("act.W_in"), W_at1 = ck.f32("act.W_at1"), b_at1 = ck.f32("act.b_at1");
+        std::vector<float> Wf((size_t)W_ * A_);
+        for (int r = 0; r < W_; ++r)
+            for (int a = 0; a < A_; ++a) {
+                double acc = 0.0;
+                for (int k = 0; k < W_; ++k) acc += (double)W_at1[(size_t)r * 2 * W_ + k] * (double)W_in[(size_t)k * A_ + a];
+                Wf[(size_t)r * A_ + a] = (float)acc;
+            }
+        W_in_.upload(Wf.data(), Wf.size() * sizeof(float));
+        for (int s = 0; s < steps_; ++s) {
             const float t = 1.0f + (float)s * dt_step_;
             const std::vector<float> te = sinusoidal_time_emb(t, W_, cfg.min_period, cfg.max_period);
-            for (int c = 0; c < W_; ++c) bias[(size_t)s * W_ + c] += te[c];
+            for (int r = 0; r < W_; ++r) {
+                double acc = (double)b_at1[r];
+                for (int k = 0; k < W_; ++k)
+                    acc += (double)W_at1[(size_t)r * 2 * W_ + k] * (double)b_in[k] +
+                           (double)W_at1[(size_t)r * 2 * W_ + W_ + k] * (double)te[k];
+                bias[(size_t)s * W_ + r] = (float)acc;
+            }
+        }
+        W_at2_ = load_f32(ck, "act.W_at2");
+        b_at2_ = load_f32(ck, "act.b_at2");
+    } else {
+        for (int s = 0; s < steps_; ++s) {
+            for (int c = 0; c < W_; ++c) bias[(size_t)s * W_ + c] = b_in[c];
+            if (arch_ != Arch::GR00T) {
+                // t = 1 + step*dt (src/models/pi0.cpp:654-656), embedding of src/layers/embed.h:61-73
+                const float t = 1.0f + (float)s * dt_step_;
+                const std::vector<float> te = sinusoidal_time_emb(t, W_, cfg.min_period, cfg.max_period);
+                for (int c = 0; c < W_; ++c) bias[(size_t)s * W_ + c] += te[c];
+            }
         }
     }
     bias_step_.upload(bias.data(), bias.size() * sizeof(float));
@@ -317,6 +350,7 @@ void FlowExpert::allocate(int B, int P) {
     q_.alloc((size_t)B * S_ * Hq_ * D_ * es);
     att_.alloc((size_t)B * S_ * Hq_ * D_ * es);
     if (I_ > 0) mid_.alloc((size_t)B * S_ * I_ * es);
+    if (time_mlp_) m1_.alloc((size_t)B * S_ * W_ * sizeof(float));
 }
 
 void FlowExpert::prefill(const Inputs* in, int batch) {
@@ -454,8 +488,17 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
         const int s = it % steps_;
         if (s == 0) VLA_HIP(hipMemcpyAsync(xt_.get(), x0_.get(), xbytes, hipMemcpyDeviceToDevice, C.stream));
         {
-            VLA_K(vla_embed_suffix(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
-                                   n_lead_ ? lead_.as<float>() : nullptr, h.data, dt_, B, S_, n_lead_, A_, W_, C.stream));
+            if (time_mlp_) {
+                VLA_K(vla_embed_suffix_act(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
+                                           n_lead_ ? lead_.as<float>() : nullptr, m1_.get(), VLA_DT_F32, B, S_, n_lead_, A_, W_,
+                                           VLA_ACT_SILU, C.stream));
+                VLA_K(vla_linear(m1_.get(), W_at2_.get(), b_at2_.as<float>(), nullptr, h.data, VLA_DT_F32, dt_, M, W_, W_,
+                                 C.stream));
+                if (n_lead_) VLA_K(vla_set_lead_rows(lead_.as<float>(), h.data, dt_, B, S_, n_lead_, W_, C.stream));
+            } else {
+                VLA_K(vla_embed_suffix(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
+                                       n_lead_ ? lead_.as<float>() : nullptr, h.data, dt_, B, S_, n_lead_, A_, W_, C.stream));
+            }
             for (int l = 0; l < L_; ++l) {
                 LayerW& w = layers_[l];
                 const float* bq = w.bqkv ? w.bqkv.as<float>() : nullptr;
