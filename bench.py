@@ -47,6 +47,7 @@ def workloads():
         "whole_smolvla_16layer_bf16_b32": dict(cfg=dict(ck.smolvla_config(16, "bf16", 0), ffn_dim=2048), B=32, views=3),
         "whole_smolvla_16layer_bf16_b1": dict(cfg=dict(ck.smolvla_config(16, "bf16", 0), ffn_dim=2048), B=1, views=3),
         "whole_pi0_18layer_bf16_b16": dict(cfg=dict(ck.pi0_config(18), ffn_dim=4096), B=16, views=3),
+        "whole_pi05_18layer_bf16_b16": dict(cfg=dict(ck.pi05_config(18), ffn_dim=4096), B=16, views=3),
         "whole_gr00t_16dit_bf16_b64": dict(cfg=dict(ck.gr00t_config(16), ffn_dim=6144), B=64, views=2),
         "cfg4_bitvla_30layer_b1": dict(cfg=ck.bitvla_config(30), B=1, views=1),
         "cfg4_bitvla_30layer_b8": dict(cfg=ck.bitvla_config(30), B=8, views=1),
@@ -55,7 +56,7 @@ def workloads():
 
 def make_obs(cfg, r, views):
     A = cfg["max_action_dim"]
-    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "bitvla") else 1)
+    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "bitvla", "pi05") else 1)
     img = r.standard_normal((views * cfg["n_img"], cfg["hidden"])).astype(np.float32)
     if cfg["arch"] == "smolvla":
         img /= np.sqrt(cfg["hidden"])
@@ -174,7 +175,7 @@ def kernel_breakdown(pkg, cfg, B, P):
     M = B * S
     qd, kvd = Hq * D, Hkv * D
     gr00t = arch == "gr00t_n1d5"
-    self_layers = [l for l in range(L) if (True if arch == "pi0" else (l % 2 == 0 if arch == "smolvla" else l % 2 == 1))]
+    self_layers = [l for l in range(L) if (True if arch in ("pi0", "pi05") else (l % 2 == 0 if arch == "smolvla" else l % 2 == 1))]
     n_self, n_cross = len(self_layers), L - len(self_layers)
     P_self = 0 if gr00t else P
     T_self = P_self + S
@@ -190,7 +191,8 @@ def kernel_breakdown(pkg, cfg, B, P):
     rope = None if gr00t else cos
     scale = 1.0 / np.sqrt(D)
     A = cfg["max_action_dim"]
-    n_lead = 0 if arch == "smolvla" else 1
+    pi05 = arch == "pi05"
+    n_lead = 0 if arch in ("smolvla", "pi05") else 1
     xt = torch.zeros(B, S - n_lead, A, device=dev)
     W_in, b_in = torch.randn(W, A, device=dev), torch.zeros(W, device=dev)
     lead = torch.zeros(B, max(n_lead, 1), W, device=dev)
@@ -200,8 +202,10 @@ def kernel_breakdown(pkg, cfg, B, P):
         1, "hbm", M * W * es)
     # bf16 RMS archs: the layer's pre-norm runs inside the projection launch (as the host
     # layer does); only the final norm is a launch of its own
-    fused_norm = bf and not gr00t and W % 16 == 0
-    if gr00t:
+    fused_norm = bf and not gr00t and not pi05 and W % 16 == 0
+    if pi05:  # adaRMS before the projections, before the FFN and before the Euler step
+        add("adarms", lambda i: pkg.call("vla_adarms", h, scv, scv, hn, dt, M, W, 1e-6), L + 1, "hbm", 2 * M * W * es)
+    elif gr00t:
         add("adaln", lambda i: pkg.call("vla_adaln", h, scv, scv, hn, dt, M, W, 1e-5), L + 1, "hbm", 2 * M * W * es)
     else:
         add("rms_norm", lambda i: pkg.call("vla_rms_norm", h, lnw, hn, dt, M, W, 1e-5), 1 if fused_norm else L + 1, "hbm",
@@ -226,7 +230,12 @@ def kernel_breakdown(pkg, cfg, B, P):
         add("attention_cross", lambda i: pkg.call("vla_attn_prefix_suffix", q, kcs_c[i % n_rot], vcs_c[i % n_rot], att, dt, B, S, Hq, Hkv, D, t_cross,
                                                 P, scale, 0, P, 0, 0, None),
             n_cross, "hbm", 2 * P * kvd * es * B)
-    add("wo_residual", lambda i: pkg.call("vla_linear", att, Wo, None, h, h, dt, dt, M, W, qd), L, "mfma", 2.0 * M * W * qd)
+    if pi05:
+        gatev = torch.ones(W, device=dev)
+        add("wo_gated_residual", lambda i: pkg.call("vla_linear_gated", att, Wo, None, gatev, h, h, dt, dt, M, W, qd), L, "mfma",
+            2.0 * M * W * qd)
+    else:
+        add("wo_residual", lambda i: pkg.call("vla_linear", att, Wo, None, h, h, dt, dt, M, W, qd), L, "mfma", 2.0 * M * W * qd)
     I = cfg.get("ffn_dim", 0)
     if I > 0:  # the FFN half of every layer (workloads beyond the BASELINE configurations)
         mid = z(M, I)
@@ -240,10 +249,15 @@ def kernel_breakdown(pkg, cfg, B, P):
             Wgu, Wd = rnd(2 * I, W), rnd(W, I)
             act = pkg.VLA_ACT_SILU if arch == "smolvla" else pkg.VLA_ACT_GELU
             if not fused_norm:
-                out["rms_norm"]["per_step"] += L
+                out["adarms" if pi05 else "rms_norm"]["per_step"] += L
             add("ffn_gate_up", lambda i: pkg.call("vla_glu_linear", h if fused_norm else hn, Wgu, None, mid, dt, dt, M, I, W, act,
                                                   1e-5 if fused_norm else -1.0), L, "mfma", 4.0 * M * I * W)
-            add("ffn_down_residual", lambda i: pkg.call("vla_linear", mid, Wd, None, h, h, dt, dt, M, W, I), L, "mfma", 2.0 * M * I * W)
+            if pi05:
+                add("ffn_down_gated_residual", lambda i: pkg.call("vla_linear_gated", mid, Wd, None, gatev, h, h, dt, dt, M, W, I), L,
+                    "mfma", 2.0 * M * I * W)
+            else:
+                add("ffn_down_residual", lambda i: pkg.call("vla_linear", mid, Wd, None, h, h, dt, dt, M, W, I), L, "mfma",
+                    2.0 * M * I * W)
     add("euler_step", lambda i: pkg.call("vla_euler_step", xt, hn, W_out, b_out, dt, B, S, n_lead, A, W, -0.1), 1, "hbm",
         M * W * es)
     return out
@@ -339,7 +353,7 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir):
     steps_per_chunk = cfg["n_suffix"] if cfg["arch"] == "bitvla" else cfg["num_steps"]
     if cfg["arch"] == "smolvla":
         P = views * cfg["n_img"] + cfg["n_lang"] + 1
-    elif cfg["arch"] == "pi0":
+    elif cfg["arch"] in ("pi0", "pi05"):
         P = views * cfg["n_img"] + cfg["n_lang"]
     elif cfg["arch"] == "bitvla":
         P = cfg["n_img"] + cfg["n_lang"]

@@ -99,6 +99,12 @@ VLA_KAPI int vla_rms_norm(const void* x, const void* w, void* y, int dtype, int 
 VLA_KAPI int vla_adaln(const void* x, const float* sc, const float* sh, void* y, int dtype, int M, int K,
                        float eps, vla_stream_t stream);
 
+/* build_adarms (src/models/pi05.cpp:208-223) with (scale, shift) already evaluated for the
+ * step: y = n + n * scale + shift, n = x * rsqrt(mean x^2 + eps) (no centring, no weight).
+ * scale, shift fp32 [K]. */
+VLA_KAPI int vla_adarms(const void* x, const float* sc, const float* sh, void* y, int dtype, int M, int K, float eps,
+                        vla_stream_t stream);
+
 /* ---------------------------------------------------------------- projections */
 
 /* y[M][N] = x[M][K] . W[N][K]^T (+ bias[N], fp32) (+ residual[M][N]), the
@@ -116,6 +122,13 @@ enum { VLA_ACT_NONE = 0, VLA_ACT_SILU = 1, VLA_ACT_GELU = 2 };
  * (src/layers/ffn.h:24-27, used by DitHead::block, src/modules/dit_head.cpp:133). */
 VLA_KAPI int vla_linear_act(const void* x, const void* W, const float* bias, const void* residual, void* y, int dtype,
                             int out_dtype, int M, int N, int K, int act, vla_stream_t stream);
+
+/* y = residual + col_gate * (x W^T + b): the gated residual adds of the adaRMS layers,
+ * h1 = x + o_out * gate_attn and h = h1 + mlp_out * gate_ffn (src/models/pi05.cpp:273, 281).
+ * col_gate fp32 [N] (one factor per output column, the same for every row). */
+VLA_KAPI int vla_linear_gated(const void* x, const void* W, const float* bias, const float* col_gate,
+                              const void* residual, void* y, int dtype, int out_dtype, int M, int N, int K,
+                              vla_stream_t stream);
 
 /* Gated FFN input half in one launch: y[M][I] = act(x Wg^T + bg) * (x Wu^T + bu), replacing
  * mm_w(Wgate) -> ggml_silu / ggml_gelu -> mm_w(Wup) -> ggml_mul (src/models/smolvla.cpp:845-847,

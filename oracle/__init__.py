@@ -161,6 +161,13 @@ def adaln(x, sc, sh, eps):
     return y
 
 
+def adarms(x, scale, shift, eps):
+    """adaRMS (build_adarms, src/models/pi05.cpp:208-224): n = rms_norm(x) without a weight,
+    then (n + n * scale) + shift in that order."""
+    n = rms_norm(x, None, eps)
+    return ((n + n * _f32(scale)) + _f32(shift)).astype(np.float32)
+
+
 def silu(x):
     x = _f32(x)
     return (x / (1.0 + np.exp(-x.astype(np.float64)))).astype(np.float32)

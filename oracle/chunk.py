@@ -27,7 +27,7 @@ def _rnd(emulate):
 
 
 def _is_self(cfg, l):
-    if cfg["arch"] == "pi0":
+    if cfg["arch"] in ("pi0", "pi05"):
         return True
     if cfg["arch"] == "smolvla":
         return l % cfg["self_attn_every_n"] == 0
@@ -43,13 +43,15 @@ def _split_heads(y, Hq, Hkv, D):
 
 
 def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
-    """SmolVLA / pi0 / GR00T N1.5 action chunk for one observation.
+    """SmolVLA / pi0 / pi0.5 / GR00T N1.5 action chunk for one observation.
 
     obs: img_emb [views*n_img, hidden], n_views, lang (int32 or None), state, noise
     [n_actions, max_action_dim].  Returns [n_actions, max_action_dim] fp32.
     Follows build_compute_graph (src/models/smolvla.cpp:1376-1419), the pi0 main
     graph (src/models/pi0.cpp:559-588) and the GR00T solver loop
-    (src/models/gr00tn1d5.cpp:359-381).
+    (src/models/gr00tn1d5.cpp:359-381).  pi0.5 is the pi0 schedule with adaRMS norms whose
+    (scale, shift, gate) come from the time embedding, gated residuals, no state token
+    and no suffix mask (src/models/pi05.cpp:208-283, 610-631).
     """
     arch = cfg["arch"]
     rnd = _rnd(emulate_bf16)
@@ -63,7 +65,8 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
     img = np.asarray(obs["img_emb"], np.float32).reshape(n_img_tot, Wv)
     state = np.zeros(cfg["max_state_dim"], np.float32) if obs.get("state") is None else np.asarray(obs["state"], np.float32)
     gr00t = arch == "gr00t_n1d5"
-    n_lead = 0 if arch == "smolvla" else 1
+    pi05 = arch == "pi05"
+    n_lead = 0 if arch in ("smolvla", "pi05") else 1
     Sa = S - n_lead
 
     # ---- prefix embeddings, positions, masks
@@ -147,7 +150,17 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
     debug = {}
     for s in range(steps):
         bias = w["act.b_in"].copy()
-        if not gr00t:
+        if pi05:
+            # the time only conditions the norms (pi05.cpp:619-622)
+            t = np.float32(1.0) + np.float32(s) * dt32
+            temb = orc.sinusoidal_time_emb(float(t), W, cfg["min_period"], cfg["max_period"])
+            c1 = orc.silu(orc.linear(temb[None, :], w["te.W_tin"], w["te.b_tin"]))
+            cond = orc.silu(orc.linear(c1, w["te.W_tout"], w["te.b_tout"]))
+
+            def adarms(x_, name):  # build_adarms, pi05.cpp:208-224
+                mod = orc.linear(cond, w[name + "_w"], w[name + "_b"])[0]
+                return orc.adarms(x_, mod[:W], mod[W:2 * W], eps), mod[2 * W:]
+        elif not gr00t:
             t = np.float32(1.0) + np.float32(s) * dt32
             bias = bias + orc.sinusoidal_time_emb(float(t), W, cfg["min_period"], cfg["max_period"])
         if "act.W_at1" in w and not gr00t:
@@ -166,7 +179,10 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
         for l in range(L):
             p = "ex.%d." % l
             self_l = _is_self(cfg, l)
-            if gr00t:
+            if pi05:
+                hn, gate_attn = adarms(h, p + "ada_in")
+                hn = rnd(hn)
+            elif gr00t:
                 c = ada[s][l]
                 hn = rnd(orc.adaln(h, c[:W], c[W:], eps))
             else:
@@ -190,6 +206,17 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
                 K_full, V_full = cacheK[l], cacheV[l]
                 m = mask_cross if (pad[1] > pad[0]) else None
             att = rnd(orc.attention(q, K_full, V_full, m, scale))
+            if pi05:
+                # gated residuals (pi05.cpp:273-282)
+                h = rnd(h + orc.linear(att, w[p + "Wo"]) * gate_attn)
+                if cfg.get("ffn_dim", 0) > 0:
+                    I = cfg["ffn_dim"]
+                    n2, gate_ffn = adarms(h, p + "ada_post")
+                    n2 = rnd(n2)
+                    Wgu = w[p + "Wgu"]
+                    mid = rnd(orc.gelu(orc.linear(n2, Wgu[:I])) * orc.linear(n2, Wgu[I:]))
+                    h = rnd(h + orc.linear(mid, w[p + "Wd"]) * gate_ffn)
+                continue
             h = rnd(orc.linear(att, w[p + "Wo"], w.get(p + "bo")) + h)
             if cfg.get("ffn_dim", 0) > 0:
                 # the FFN half of the layer (smolvla.cpp:845-848, pi0.cpp:227-232, dit_head.cpp:132-133)
@@ -206,7 +233,9 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
                     h = rnd(orc.linear(mid, w[p + "Wd"]) + h)
             if return_debug and s == 0 and l == 0:
                 debug["q0"], debug["att0"], debug["h0"] = q, att, h
-        if gr00t:
+        if pi05:
+            hn = rnd(adarms(h, "act.ada_final")[0])
+        elif gr00t:
             hn = rnd(orc.layer_norm(h, None, None, cfg.get("norm_out_eps", 1e-6)))
         else:
             hn = rnd(orc.rms_norm(h, w["act.norm"], eps))

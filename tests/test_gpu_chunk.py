@@ -27,7 +27,7 @@ def bf16_close(got, want):
 
 def make_obs(cfg, r, n_views, n_lang=None, bf16_inputs=False):
     A = cfg["max_action_dim"]
-    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "bitvla") else 1)
+    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "bitvla", "pi05") else 1)
     img = r.standard_normal((n_views * cfg["n_img"], cfg["hidden"])).astype(np.float32)
     if cfg["arch"] == "smolvla":
         img /= np.sqrt(cfg["hidden"])  # the prefix builder scales image rows by sqrt(hidden)
@@ -181,6 +181,35 @@ def test_suffix_embedding_with_the_action_time_mlp(tmp_path, arch, dtype, batch)
         else:
             assert bf16_close(got[b], want), np.abs(got[b] - want).max()
     w0 = {k: v for k, v in w.items() if not k.startswith("act.W_at") and not k.startswith("act.b_at")}
+    assert not np.allclose(orc_chunk.flow_expert_chunk(cfg, w0, obs[0], emulate_bf16=dtype != "f32"), got[0], atol=1e-3)
+    m.close()
+
+
+@pytest.mark.parametrize("dtype,n_layers,ffn_dim,batch", [
+    ("f32", 2, 256, 1),      # fp32: 1e-5
+    ("bf16", 3, 0, 2),       # attention half only
+    ("bf16", 4, 4096, 2),    # the expert's real FFN width
+])
+def test_pi05_adarms_layers(tmp_path, dtype, n_layers, ffn_dim, batch):
+    """pi0.5 (src/models/pi05.cpp:208-283, 610-631): adaRMS norms whose scale, shift and gate
+    come from the flow time, gated residuals, a suffix of action tokens only, no suffix mask."""
+    cfg = ckpt.pi05_config(n_layers=n_layers, dtype=dtype)
+    cfg["ffn_dim"] = ffn_dim
+    if dtype == "f32":
+        cfg["head_dim"] = 128  # 256-wide heads are built for bf16 only
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 13)
+    r = np.random.default_rng(310 + ffn_dim)
+    obs = [make_obs(cfg, r, n_views=2, n_lang=57) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "pi05")
+    got = m.predict_batch(obs).reshape(batch, 50, 32)
+    for b in range(batch):
+        want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=dtype != "f32")
+        if dtype == "f32":
+            assert rel_err(got[b], want) < 1e-5, rel_err(got[b], want)
+        else:
+            assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    # the modulation is live: a chunk computed with all gates at zero is a different chunk
+    w0 = {k: (np.zeros_like(v) if "ada_" in k else v) for k, v in w.items()}
     assert not np.allclose(orc_chunk.flow_expert_chunk(cfg, w0, obs[0], emulate_bf16=dtype != "f32"), got[0], atol=1e-3)
     m.close()
 

@@ -135,6 +135,40 @@ def test_rms_norm_and_adaln(dtype, M, K):
         assert np.array_equal(host(y3), host(y))
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("M,K,N", [(50, 1024, 1024), (800, 1024, 1024), (50, 4096, 1024), (7, 720, 200)])
+def test_adarms_and_gated_residual_projection(dtype, M, K, N):
+    """pi0.5's norm and its gated residual (src/models/pi05.cpp:208-224, 273-282):
+    y = rms(x) (1 + scale) + shift;  out = residual + (x W^T) * gate[column]."""
+    r = np.random.default_rng(140 + M)
+    x = (r.standard_normal((M, K)) * 2 + 0.5).astype(np.float32)
+    sc, sh = (0.2 * r.standard_normal(K)).astype(np.float32), (0.2 * r.standard_normal(K)).astype(np.float32)
+    W = (0.02 * r.standard_normal((N, K))).astype(np.float32)
+    gate = (1 + 0.2 * r.standard_normal(N)).astype(np.float32)
+    res = r.standard_normal((M, N)).astype(np.float32)
+    if dtype == BF16:
+        x, W, res = orc.round_bf16(x), orc.round_bf16(W), orc.round_bf16(res)
+    y = empty((M, K), dtype)
+    pkg.call("vla_adarms", to_dev(x, dtype), dev(sc), dev(sh), y, dtype, M, K, 1e-6)
+    out = empty((M, N), dtype)
+    pkg.call("vla_linear_gated", to_dev(x, dtype), to_dev(W, dtype), None, dev(gate), to_dev(res, dtype), out, dtype, dtype, M, N, K)
+    ones = torch.ones(N, dtype=torch.float32, device="cuda")
+    plain = empty((M, N), dtype)
+    pkg.call("vla_linear_gated", to_dev(x, dtype), to_dev(W, dtype), None, ones, to_dev(res, dtype), plain, dtype, dtype, M, N, K)
+    ref = empty((M, N), dtype)
+    pkg.call("vla_linear", to_dev(x, dtype), to_dev(W, dtype), None, to_dev(res, dtype), ref, dtype, dtype, M, N, K)
+    sync()
+    want_y = orc.adarms(x, sc, sh, 1e-6)
+    want = res + orc.linear(x, W) * gate
+    if dtype == F32:
+        assert rel_err(host(y), want_y) < FP32_TOL and rel_err(host(out), want) < FP32_TOL
+    else:
+        assert bf16_close(as_f32(y, dtype), want_y) and bf16_close(as_f32(out, dtype), want)
+    assert np.array_equal(host(plain), host(ref))  # a gate of ones: the plain projection, bit for bit
+    with pytest.raises(RuntimeError):  # the gate is not optional
+        pkg.call("vla_linear_gated", to_dev(x, dtype), to_dev(W, dtype), None, None, to_dev(res, dtype), plain, dtype, dtype, M, N, K)
+
+
 # ---------------------------------------------------------------- projections
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("M,N,K", [(50, 720, 960), (1, 64, 128), (130, 200, 72), (17, 1536, 1536), (64, 32, 720)])

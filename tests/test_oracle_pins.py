@@ -178,6 +178,12 @@ def test_norms_against_torch():
     sc, sh = r.standard_normal(96).astype(np.float32), r.standard_normal(96).astype(np.float32)
     xn = torch.nn.functional.layer_norm(xt, (96,), None, None, 1e-5).float().numpy()
     assert np.allclose(orc.adaln(x, sc, sh, 1e-5), xn * (1 + sc) + sh, rtol=1e-5, atol=1e-5)
+    # adaRMS: float64 evaluation of rms(x)*(1+scale)+shift; scale = -1 leaves the shift alone;
+    # a constant row normalises to its sign, so the output is sign*(1+scale)+shift
+    rn = (xt / torch.sqrt((xt * xt).mean(-1, keepdim=True) + 1e-6)).numpy()
+    assert np.allclose(orc.adarms(x, sc, sh, 1e-6), rn * (1 + sc.astype(np.float64)) + sh, rtol=1e-5, atol=1e-5)
+    assert np.allclose(orc.adarms(x, np.full(96, -1.0, np.float32), sh, 1e-6), np.broadcast_to(sh, x.shape), atol=1e-6)
+    assert np.allclose(orc.adarms(np.full((1, 96), -2.0, np.float32), sc, sh, 0.0), -(1 + sc) + sh, atol=1e-6)
     assert np.allclose(orc.silu(np.float32([0.0, 1.0, -2.0])),
                        torch.nn.functional.silu(torch.tensor([0.0, 1.0, -2.0])).numpy(), atol=1e-7)
     # gelu, tanh form: known values, torch's tanh-approximate gelu, odd part x/2 (gelu(x) - gelu(-x) = x)

@@ -33,6 +33,8 @@ KERNEL_API = {
     "vla_rms_norm": [_vp, _vp, _vp, _i, _i, _i, _f, _vp],
     "vla_adaln": [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _vp],
     "vla_linear": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "vla_adarms": [_vp, _vp, _vp, _vp, _i, _i, _i, _f, _vp],
+    "vla_linear_gated": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "vla_linear_act": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "vla_glu_linear": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
     "vla_attn_qkv_rope": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _vp],

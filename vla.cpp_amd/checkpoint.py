@@ -76,6 +76,15 @@ def pi0_config(n_layers=18, dtype="bf16", num_steps=10):
                 self_attn_every_n=1, min_period=4e-3, max_period=4.0, vocab=512, suffix_mask=2, max_views=3)
 
 
+def pi05_config(n_layers=18, dtype="bf16", num_steps=10):
+    """pi0.5 shape (src/models/pi05.cpp:292-328): the pi0 backbone and expert widths with
+    adaRMS norms conditioned on the flow time, no state token (suffix = 50 action tokens,
+    the state travels as text) and up to 200 text tokens."""
+    c = pi0_config(n_layers, dtype, num_steps)
+    c.update(arch="pi05", n_lang=200, n_suffix=50, suffix_mask=0)
+    return c
+
+
 def gr00t_config(n_layers=16, dtype="bf16", num_steps=4, n_suffix=17):
     """GR00T N1.5 DiT head (src/modules/dit_head.h:38-45): width 1536, 32 heads of 48,
     cross-attention on even layers onto 148 backbone tokens per view of width 2048,
@@ -96,7 +105,7 @@ def bitvla_config(n_layers=30):
 
 
 def _is_self(cfg, l):
-    if cfg["arch"] == "pi0":
+    if cfg["arch"] in ("pi0", "pi05"):
         return True
     if cfg["arch"] == "smolvla":
         return l % cfg["self_attn_every_n"] == 0
@@ -142,14 +151,24 @@ def synth_weights(cfg, seed=0x5EED):
     if arch == "smolvla":
         w["prefix.Wstate"] = (0.1 * r.standard_normal((Wv, cfg["max_state_dim"]))).astype(np.float32)
         w["prefix.bstate"] = vec(Wv, 0.1)
-    else:
+    elif arch != "pi05":
         w["act.W_sp"] = (0.1 * r.standard_normal((W, cfg["max_state_dim"]))).astype(np.float32)
         w["act.b_sp"] = vec(W, 0.1)
     w["act.W_in"] = (0.1 * r.standard_normal((W, A))).astype(np.float32)
     w["act.b_in"] = vec(W, 0.1)
     w["act.W_out"] = (0.02 * r.standard_normal((A, W))).astype(np.float32)
     w["act.b_out"] = vec(A)
-    if arch != "gr00t_n1d5":
+    # adaRMS modulation dense: rows [scale; shift; gate], the gate around 1 (pi05.cpp:208-224)
+    ada_w = lambda: (0.5 * r.standard_normal((3 * W, W)) / np.sqrt(W)).astype(np.float32)
+    ada_b = lambda: np.concatenate([vec(2 * W, 0.05), 1.0 + vec(W, 0.05)]).astype(np.float32)
+    if arch == "pi05":
+        w["te.W_tin"] = (r.standard_normal((W, W)) / np.sqrt(W)).astype(np.float32)
+        w["te.b_tin"] = vec(W, 0.1)
+        w["te.W_tout"] = (r.standard_normal((W, W)) / np.sqrt(W)).astype(np.float32)
+        w["te.b_tout"] = vec(W, 0.1)
+        w["act.ada_final_w"] = ada_w()
+        w["act.ada_final_b"] = ada_b()
+    elif arch != "gr00t_n1d5":
         w["act.norm"] = nrm(W)
         if cfg.get("time_mlp", 0):  # action_time_mlp_in / _out of the suffix embedding
             w["act.W_at1"] = (r.standard_normal((W, 2 * W)) / np.sqrt(2 * W)).astype(np.float32)
@@ -183,7 +202,12 @@ def synth_weights(cfg, seed=0x5EED):
                 w[p + "W2"] = mat(W, cfg["ffn_dim"])
                 w[p + "b2"] = vec(W)
             continue
-        w[p + "ln"] = nrm(W)
+        if arch == "pi05":
+            w[p + "ada_in_w"], w[p + "ada_in_b"] = ada_w(), ada_b()
+            if cfg.get("ffn_dim", 0) > 0:
+                w[p + "ada_post_w"], w[p + "ada_post_b"] = ada_w(), ada_b()
+        else:
+            w[p + "ln"] = nrm(W)
         w[v + "ln"] = nrm(Wv)
         w[v + "Wkv"] = mat(2 * kvd, Wv)
         if self_l:
@@ -194,7 +218,8 @@ def synth_weights(cfg, seed=0x5EED):
             w[p + "Wv_x"] = mat(kvd, kvd, 0.05)
         w[p + "Wo"] = mat(W, qd)
         if cfg.get("ffn_dim", 0) > 0:  # post-attention norm, [gate; up] rows, down
-            w[p + "ln2"] = nrm(W)
+            if arch != "pi05":
+                w[p + "ln2"] = nrm(W)
             w[p + "Wgu"] = mat(2 * cfg["ffn_dim"], W)
             w[p + "Wd"] = mat(W, cfg["ffn_dim"])
     return w
@@ -226,7 +251,8 @@ def write_synthetic(path, cfg, weights, ladder_pack=None, plain_pack=None):
             continue
         if name.endswith(".ws"):
             continue
-        small = name.startswith(_F32_NAMES) or name.endswith((".bqkv", ".bq", ".bo", ".bkv", ".adaln_b", ".b1", ".b2"))
+        small = name.startswith(_F32_NAMES) or name.endswith((".bqkv", ".bq", ".bo", ".bkv", ".adaln_b", ".b1", ".b2", ".ada_in_w", ".ada_in_b",
+                                                            ".ada_post_w", ".ada_post_b"))
         if cfg["arch"] == "bitvla" and name.endswith(("attn_norm", "sub_norm")):
             out[name] = BF16(t)
         elif bf and not small:

@@ -113,13 +113,13 @@ __global__ void rms_norm_kernel(const T* __restrict__ x, const T* __restrict__ w
 
 template <typename T>
 __global__ void adaln_kernel(const T* __restrict__ x, const float* __restrict__ sc, const float* __restrict__ sh,
-                             T* __restrict__ y, int K, float eps) {
+                             T* __restrict__ y, int K, float eps, int rms) {
     __shared__ float red[16];
     const T* xr = x + (long)blockIdx.x * K;
     T* yr = y + (long)blockIdx.x * K;
     float s1 = 0.f;
     for (int k = threadIdx.x; k < K; k += blockDim.x) s1 += Elem<T>::load(xr + k);
-    const float mean = block_sum(s1, red) / (float)K;
+    const float mean = rms ? 0.f : block_sum(s1, red) / (float)K;  // rms: no centring (build_adarms)
     float s2 = 0.f;
     for (int k = threadIdx.x; k < K; k += blockDim.x) {
         const float d = Elem<T>::load(xr + k) - mean;
@@ -138,7 +138,7 @@ __global__ void adaln_kernel(const T* __restrict__ x, const float* __restrict__ 
 // without affine, then y = xn * (1 + scale) + shift.  RMS_AQ: the RMS result, rounded to bf16
 // as it would be stored, quantised per row to int8 (scale 127 / max(amax, 1e-5), round half
 // even) with its row sum -- bitvla_rmsnorm_bf16 followed by act_quant without the round trip.
-enum { NORM_RMS = 0, NORM_ADALN = 1, NORM_RMS_AQ = 2 };
+enum { NORM_RMS = 0, NORM_ADALN = 1, NORM_RMS_AQ = 2, NORM_ADARMS = 3 };  // ADARMS: RMS statistics, then (1 + scale), shift
 template <typename T, int NV, int MODE>
 __global__ void __launch_bounds__(256) row_norm_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                        const float* __restrict__ sc, const float* __restrict__ sh,
@@ -193,10 +193,10 @@ __global__ void __launch_bounds__(256) row_norm_kernel(const T* __restrict__ x, 
         if (vec >= nvec) continue;
         const int k0 = vec * EPV;
         float o[EPV];
-        if (MODE == NORM_ADALN) {
+        if (MODE == NORM_ADALN || MODE == NORM_ADARMS) {
 #pragma unroll
             for (int e = 0; e < EPV; ++e) {
-                const float xn = (v[i][e] - mean) * inv;
+                const float xn = (v[i][e] - mean) * inv;  // mean stays 0 for ADARMS
                 o[e] = xn + xn * sc[k0 + e] + sh[k0 + e];
             }
         } else {
@@ -526,6 +526,30 @@ inline int row_threads(int K) { return K >= 2048 ? 256 : (K >= 512 ? 128 : 64); 
 
 }  // namespace
 
+namespace {
+template <int MODE>
+int mod_norm(const void* x, const float* sc, const float* sh, void* y, int dtype, int M, int K, float eps,
+                    vla_stream_t stream) {
+    if (!x || !y || !sc || !sh || M < 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (M == 0) return VLA_K_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int th = row_threads(K);
+    if (dtype == VLA_DT_F32 && launch_row_norm<float, MODE>(x, nullptr, sc, sh, y, nullptr, nullptr, nullptr, M, K, eps, st))
+        return VLA_CHECK_LAUNCH();
+    if (dtype == VLA_DT_BF16 && launch_row_norm<bf16_t, MODE>(x, nullptr, sc, sh, y, nullptr, nullptr, nullptr, M, K, eps, st))
+        return VLA_CHECK_LAUNCH();
+    const int rms = MODE == NORM_ADARMS;
+    if (dtype == VLA_DT_F32)
+        adaln_kernel<float><<<M, th, 0, st>>>((const float*)x, sc, sh, (float*)y, K, eps, rms);
+    else if (dtype == VLA_DT_BF16)
+        adaln_kernel<bf16_t><<<M, th, 0, st>>>((const bf16_t*)x, sc, sh, (bf16_t*)y, K, eps, rms);
+    else
+        return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
+}  // namespace
+
 extern "C" {
 
 int vla_rope_tables_host(const int32_t* pos, int n, int head_dim, double base, float* cos_tab, float* sin_tab) {
@@ -601,21 +625,12 @@ int vla_rms_norm(const void* x, const void* w, void* y, int dtype, int M, int K,
 
 int vla_adaln(const void* x, const float* sc, const float* sh, void* y, int dtype, int M, int K, float eps,
               vla_stream_t stream) {
-    if (!x || !y || !sc || !sh || M < 0 || K <= 0) return VLA_K_ERR_ARG;
-    if (M == 0) return VLA_K_OK;
-    hipStream_t st = (hipStream_t)stream;
-    const int th = row_threads(K);
-    if (dtype == VLA_DT_F32 && launch_row_norm<float, NORM_ADALN>(x, nullptr, sc, sh, y, nullptr, nullptr, nullptr, M, K, eps, st))
-        return VLA_CHECK_LAUNCH();
-    if (dtype == VLA_DT_BF16 && launch_row_norm<bf16_t, NORM_ADALN>(x, nullptr, sc, sh, y, nullptr, nullptr, nullptr, M, K, eps, st))
-        return VLA_CHECK_LAUNCH();
-    if (dtype == VLA_DT_F32)
-        adaln_kernel<float><<<M, th, 0, st>>>((const float*)x, sc, sh, (float*)y, K, eps);
-    else if (dtype == VLA_DT_BF16)
-        adaln_kernel<bf16_t><<<M, th, 0, st>>>((const bf16_t*)x, sc, sh, (bf16_t*)y, K, eps);
-    else
-        return VLA_K_ERR_ARG;
-    return VLA_CHECK_LAUNCH();
+    return mod_norm<NORM_ADALN>(x, sc, sh, y, dtype, M, K, eps, stream);
+}
+
+int vla_adarms(const void* x, const float* sc, const float* sh, void* y, int dtype, int M, int K, float eps,
+               vla_stream_t stream) {
+    return mod_norm<NORM_ADARMS>(x, sc, sh, y, dtype, M, K, eps, stream);
 }
 
 int vla_embed_suffix(const float* x_t, const float* W_in, const float* bias_step, const float* lead, void* h,

@@ -49,6 +49,7 @@ struct GemmArgs {
     void* Y;
     int out_bf16;
     int act;  // VLA_ACT_*: PLAIN applies it after the bias, GLU to the gate
+    const float* col_gate;  // PLAIN: fp32 [N] factor on the projection before the residual is added, or null
     // QKV
     int S, Hq, nk, nv, D;
     const float* cos_t;
@@ -257,6 +258,11 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
             if (a.act != VLA_ACT_NONE) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = apply_act(v[e], a.act);
+            }
+            if (a.col_gate) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (n0 + e < a.N) v[e] *= a.col_gate[n0 + e];
             }
             if (full && a.out_bf16) {  // 8 consecutive bf16 = one 16-byte access each way
                 if (a.residual) {
@@ -1315,6 +1321,26 @@ int vla_linear_act(const void* x, const void* W, const float* bias, const void* 
     a.norm_eps = -1.f;
     a.A = x; a.W = W; a.bias = bias; a.M = M; a.N = N; a.K = K;
     a.residual = residual; a.Y = y; a.out_bf16 = (out_dtype == VLA_DT_BF16); a.act = act;
+    const int nt = (N + BN - 1) / BN;
+    if (dtype == VLA_DT_BF16) {
+        if (K % 8) return VLA_K_ERR_SHAPE;
+        return launch<bf16_t, EPI_PLAIN>(a, nt, stream);
+    }
+    if (dtype == VLA_DT_F32) {
+        if (K % 4) return VLA_K_ERR_SHAPE;
+        return launch<float, EPI_PLAIN>(a, nt, stream);
+    }
+    return VLA_K_ERR_ARG;
+}
+
+int vla_linear_gated(const void* x, const void* W, const float* bias, const float* col_gate, const void* residual, void* y,
+                     int dtype, int out_dtype, int M, int N, int K, vla_stream_t stream) {
+    if (!x || !W || !y || !col_gate || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (out_dtype != VLA_DT_F32 && out_dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
+    GemmArgs a = {};
+    a.norm_eps = -1.f;
+    a.A = x; a.W = W; a.bias = bias; a.M = M; a.N = N; a.K = K;
+    a.residual = residual; a.Y = y; a.out_bf16 = (out_dtype == VLA_DT_BF16); a.col_gate = col_gate;
     const int nt = (N + BN - 1) / BN;
     if (dtype == VLA_DT_BF16) {
         if (K % 8) return VLA_K_ERR_SHAPE;

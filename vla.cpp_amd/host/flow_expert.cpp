@@ -123,6 +123,7 @@ class FlowExpert : public ModelArch {
     DevBuf W_in_, W_out_, b_out_, final_norm_;
     DevBuf W_at2_, b_at2_, m1_;  // action-time MLP: second projection, fp32 scratch [B*S][W]
     bool time_mlp_ = false;
+    bool adarms_ = false;  // pi0.5: ada_ holds [steps][2L+1][scale, shift, gate][W]
     DevBuf bias_step_;   // [steps][W] fp32: b_in (+ time embedding of the step)
     DevBuf ada_;         // GR00T: [steps][L+1][2][W] fp32 (scale, shift); slot L is the final norm (zeros)
 
@@ -137,7 +138,10 @@ class FlowExpert : public ModelArch {
 
 FlowExpert::FlowExpert(const Checkpoint& ck) {
     const std::string arch = ck.str("arch");
-    arch_ = arch == "smolvla" ? Arch::SMOLVLA : arch == "pi0" ? Arch::PI0 : Arch::GR00T;
+    // pi0.5 is the pi0 schedule with adaRMS norms, gated residuals, no state token in the
+    // suffix and no suffix mask (src/models/pi05.cpp:208-283, 610-631)
+    adarms_ = arch == "pi05";
+    arch_ = arch == "smolvla" ? Arch::SMOLVLA : (arch == "pi0" || adarms_) ? Arch::PI0 : Arch::GR00T;
     dt_ = ck.str("dtype") == "bf16" ? VLA_DT_BF16 : VLA_DT_F32;
     L_ = (int)ck.i64("n_layers");
     Hq_ = (int)ck.i64("n_q_heads");
@@ -156,10 +160,10 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     max_state_ = (int)ck.i64("max_state_dim", 32);
     eps_ = (float)ck.f64("rms_eps", arch_ == Arch::PI0 ? 1e-6 : 1e-5);
     final_eps_ = (float)ck.f64("norm_out_eps", 1e-6);
-    suffix_mask_ = (int)ck.i64("suffix_mask", arch_ == Arch::SMOLVLA ? VLA_MASK_CAUSAL_SUFFIX
-                                              : arch_ == Arch::PI0   ? VLA_MASK_PI0_STATE
-                                                                     : VLA_MASK_NONE);
-    n_lead_ = arch_ == Arch::SMOLVLA ? 0 : 1;
+    suffix_mask_ = (int)ck.i64("suffix_mask", arch_ == Arch::SMOLVLA            ? VLA_MASK_CAUSAL_SUFFIX
+                                              : (arch_ == Arch::PI0 && !adarms_) ? VLA_MASK_PI0_STATE
+                                                                                 : VLA_MASK_NONE);
+    n_lead_ = (arch_ == Arch::SMOLVLA || adarms_) ? 0 : 1;
     rope_ = arch_ != Arch::GR00T;
     dt_step_ = (arch_ == Arch::GR00T ? 1.0f : -1.0f) / (float)steps_;
     const int every = (int)ck.i64("self_attn_every_n", arch_ == Arch::PI0 ? 1 : 2);
@@ -196,14 +200,14 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     if (arch_ == Arch::SMOLVLA) {
         Wstate_ = ck.f32("prefix.Wstate");
         bstate_ = ck.f32("prefix.bstate");
-    } else {
+    } else if (n_lead_ > 0) {
         W_sp_ = ck.f32("act.W_sp");
         b_sp_ = ck.f32("act.b_sp");
     }
     W_in_ = load_f32(ck, "act.W_in");
     W_out_ = load_f32(ck, "act.W_out");
     b_out_ = load_f32(ck, "act.b_out");
-    if (arch_ != Arch::GR00T) final_norm_ = load_w(ck, "act.norm", dt_);
+    if (arch_ != Arch::GR00T && !adarms_) final_norm_ = load_w(ck, "act.norm", dt_);
 
     layers_.resize(L_);
     for (int l = 0; l < L_; ++l) {
@@ -213,9 +217,9 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         // cross on even, self on odd layers (src/models/gr00tn1d5.cpp:361-375).
         w.is_self = arch_ == Arch::PI0 ? true : arch_ == Arch::SMOLVLA ? (l % every == 0) : (l % 2 == 1);
         w.needs_prefix = !(arch_ == Arch::GR00T && w.is_self);
-        if (arch_ != Arch::GR00T) w.ln = load_w(ck, p + "ln", dt_);
+        if (arch_ != Arch::GR00T && !adarms_) w.ln = load_w(ck, p + "ln", dt_);
         w.Wqkv = load_w(ck, p + (w.is_self ? "Wqkv" : "Wq"), dt_);
-        if (arch_ != Arch::GR00T && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
+        if (arch_ != Arch::GR00T && !adarms_ && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
             w.Wqkv_ln = load_folded_bf16(ck, p + (w.is_self ? "Wqkv" : "Wq"), p + "ln");
         if (ck.has(p + (w.is_self ? "bqkv" : "bq"))) w.bqkv = load_f32(ck, p + (w.is_self ? "bqkv" : "bq"));
         w.Wo = load_w(ck, p + "Wo", dt_);
@@ -226,10 +230,10 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
             w.W2 = load_w(ck, p + "W2", dt_);
             w.b2 = load_f32(ck, p + "b2");
         } else if (I_ > 0) {
-            w.ln2 = load_w(ck, p + "ln2", dt_);
+            if (!adarms_) w.ln2 = load_w(ck, p + "ln2", dt_);
             w.Wgu = load_w(ck, p + "Wgu", dt_);
             w.Wd = load_w(ck, p + "Wd", dt_);
-            if (dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
+            if (!adarms_ && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
                 w.Wgu_ln = load_folded_bf16(ck, p + "Wgu", p + "ln2");
         }
         if (w.needs_prefix) {
@@ -248,7 +252,7 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     // so it is evaluated once here instead of inside every denoise step.
     const std::vector<float> b_in = ck.f32("act.b_in");
     std::vector<float> bias((size_t)steps_ * W_);
-    time_mlp_ = arch_ != Arch::GR00T && ck.has("act.W_at1");
+    time_mlp_ = arch_ != Arch::GR00T && !adarms_ && ck.has("act.W_at1");
     if (time_mlp_) {
         // Action-time MLP (src/models/smolvla.cpp:1397-1403, src/models/pi0.cpp:240-244):
         //   mlp1 = W_at1 . concat(W_in x + b_in, time_s) + b_at1,  suffix = W_at2 silu(mlp1) + b_at2.
@@ -280,7 +284,7 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     } else {
         for (int s = 0; s < steps_; ++s) {
             for (int c = 0; c < W_; ++c) bias[(size_t)s * W_ + c] = b_in[c];
-            if (arch_ != Arch::GR00T) {
+            if (arch_ != Arch::GR00T && !adarms_) {
                 // t = 1 + step*dt (src/models/pi0.cpp:654-656), embedding of src/layers/embed.h:61-73
                 const float t = 1.0f + (float)s * dt_step_;
                 const std::vector<float> te = sinusoidal_time_emb(t, W_, cfg.min_period, cfg.max_period);
@@ -289,6 +293,40 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         }
     }
     bias_step_.upload(bias.data(), bias.size() * sizeof(float));
+
+    if (adarms_) {
+        // cond_s = silu(W_tout silu(W_tin time_s + b_tin) + b_tout) (src/models/pi05.cpp:619-620);
+        // (scale, shift, gate) of a norm site = dense_w . cond + dense_b (build_adarms,
+        // pi05.cpp:212-215).  Sites per step: 2 per layer (attention, FFN), then the final norm.
+        const std::vector<float> Wt1 = ck.f32("te.W_tin"), bt1 = ck.f32("te.b_tin"), Wt2 = ck.f32("te.W_tout"),
+                                 bt2 = ck.f32("te.b_tout");
+        const int sites = 2 * L_ + 1;
+        std::vector<std::vector<float>> dw(sites), db(sites);
+        for (int l = 0; l < L_; ++l) {
+            const std::string p = "ex." + std::to_string(l) + ".";
+            dw[2 * l] = ck.f32(p + "ada_in_w");
+            db[2 * l] = ck.f32(p + "ada_in_b");
+            if (I_ > 0) {
+                dw[2 * l + 1] = ck.f32(p + "ada_post_w");
+                db[2 * l + 1] = ck.f32(p + "ada_post_b");
+            }
+        }
+        dw[2 * L_] = ck.f32("act.ada_final_w");
+        db[2 * L_] = ck.f32("act.ada_final_b");
+        std::vector<float> mod((size_t)steps_ * sites * 3 * W_);
+        std::vector<float> c1(W_), cond(W_);
+        for (int s = 0; s < steps_; ++s) {
+            const float t = 1.0f + (float)s * dt_step_;
+            const std::vector<float> te = sinusoidal_time_emb(t, W_, cfg.min_period, cfg.max_period);
+            host_linear(Wt1.data(), bt1.data(), te.data(), c1.data(), W_, W_);
+            for (auto& v : c1) v = host_silu(v);
+            host_linear(Wt2.data(), bt2.data(), c1.data(), cond.data(), W_, W_);
+            for (auto& v : cond) v = host_silu(v);
+            for (int k = 0; k < sites; ++k)
+                if (!dw[k].empty()) host_linear(dw[k].data(), db[k].data(), cond.data(), mod.data() + ((size_t)s * sites + k) * 3 * W_, 3 * W_, W_);
+        }
+        ada_.upload(mod.data(), mod.size() * sizeof(float));
+    }
 
     if (arch_ == Arch::GR00T) {
         // temb = l2(silu(l1(timesteps_proj(bucket)))) (DitHead::time_emb,
@@ -397,7 +435,7 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
         if (in[b].state) std::copy(in[b].state, in[b].state + max_state_, st.begin());
         if (arch_ == Arch::SMOLVLA) {
             host_linear(Wstate_.data(), bstate_.data(), st.data(), dst + (size_t)(P - 1) * Wv_, Wv_, max_state_);
-        } else {
+        } else if (n_lead_ > 0) {
             std::vector<float> ld(W_);
             host_linear(W_sp_.data(), b_sp_.data(), st.data(), ld.data(), W_, max_state_);
             VLA_HIP(hipMemcpy(lead_.as<float>() + (size_t)b * W_, ld.data(), W_ * sizeof(float), hipMemcpyHostToDevice));
@@ -505,9 +543,18 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 const int64_t n_rows_w = w.is_self ? (int64_t)(Hq_ + 2 * Hkv_) * D_ : (int64_t)Hq_ * D_;
                 const RopeTable* tab = rope_ ? (w.is_self ? &rope_self_ : &rope_cross_) : nullptr;
                 const int tok = w.is_self ? w.kv.n_prefix : 0;
+                // pi0.5: this step's (scale, shift, gate) of the layer's two norm sites
+                const float* mod_in = adarms_ ? ada_.as<float>() + ((size_t)s * (2 * L_ + 1) + 2 * l) * 3 * W_ : nullptr;
+                const float* mod_post = adarms_ ? mod_in + 3 * W_ : nullptr;
                 // RMS archs in bf16: pre-norm, projection, rotation and append are one launch
                 bool done = false;
-                if (w.Wqkv_ln) {
+                if (adarms_) {
+                    VLA_K(vla_adarms(h.data, mod_in, mod_in + W_, hn.data, dt_, M, W_, eps_, C.stream));
+                    Tensor Wqkv = tensor_2d(w.Wqkv.get(), dt_, W_, n_rows_w);
+                    qkv_rope_append(C, hn, Wqkv, bq, S_, Hq_, w.is_self, w.is_self, tab, Q.data, w.kv, tok);
+                    done = true;
+                }
+                if (!done && w.Wqkv_ln) {
                     Tensor Wf = tensor_2d(w.Wqkv_ln.get(), dt_, W_, n_rows_w);
                     done = rmsnorm_qkv_rope_append(C, h, Wf, bq, eps_, S_, Hq_, w.is_self, w.is_self, tab, Q.data, w.kv, tok);
                 }
@@ -528,6 +575,20 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 const int n_keys = w.is_self ? w.kv.n_prefix + S_ : w.kv.n_prefix;
                 flash_attention(C, Q, w.kv, n_keys, mask, scale, att);
                 Tensor Wo = tensor_2d(w.Wo.get(), dt_, (int64_t)Hq_ * D_, W_);
+                if (adarms_) {
+                    // h1 = x + o_out * gate_attn; h = h1 + mlp_out * gate_ffn (pi05.cpp:273-281)
+                    VLA_K(vla_linear_gated(att.data, Wo.data, nullptr, mod_in + 2 * W_, h.data, h.data, dt_, dt_, M, W_,
+                                           Hq_ * D_, C.stream));
+                    if (I_ > 0) {
+                        Tensor mid = tensor_2d(mid_.get(), dt_, I_, M);
+                        VLA_K(vla_adarms(h.data, mod_post, mod_post + W_, hn.data, dt_, M, W_, eps_, C.stream));
+                        VLA_K(vla_glu_linear(hn.data, w.Wgu.get(), nullptr, mid.data, dt_, dt_, M, I_, W_, VLA_ACT_GELU, -1.f,
+                                             C.stream));
+                        VLA_K(vla_linear_gated(mid.data, w.Wd.get(), nullptr, mod_post + 2 * W_, h.data, h.data, dt_, dt_, M, W_,
+                                               I_, C.stream));
+                    }
+                    continue;
+                }
                 linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
                 if (I_ > 0) {
                     // FFN half (smolvla.cpp:845-848, pi0.cpp:227-232, dit_head.cpp:132-133)
@@ -553,7 +614,10 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                     }
                 }
             }
-            if (arch_ == Arch::GR00T) {
+            if (adarms_) {
+                const float* mf = ada_.as<float>() + ((size_t)s * (2 * L_ + 1) + 2 * L_) * 3 * W_;  // gate unused (pi05.cpp:628)
+                VLA_K(vla_adarms(h.data, mf, mf + W_, hn.data, dt_, M, W_, eps_, C.stream));
+            } else if (arch_ == Arch::GR00T) {
                 const float* z = ada_.as<float>() + ((size_t)s * (L_ + 1) + L_) * 2 * W_;  // zeros: plain LayerNorm
                 adaln(C, h, z, z + W_, final_eps_, hn);
             } else {
