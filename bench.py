@@ -49,6 +49,7 @@ def workloads():
         "whole_pi0_18layer_bf16_b16": dict(cfg=dict(ck.pi0_config(18), ffn_dim=4096), B=16, views=3),
         "whole_pi05_18layer_bf16_b16": dict(cfg=dict(ck.pi05_config(18), ffn_dim=4096), B=16, views=3),
         "whole_gr00t_16dit_bf16_b64": dict(cfg=dict(ck.gr00t_config(16), ffn_dim=6144), B=64, views=2),
+        "whole_gr00t_n1d6_32dit_bf16_b64": dict(cfg=dict(ck.gr00t_n1d6_config(32), ffn_dim=6144), B=64, views=2),
         "cfg4_bitvla_30layer_b1": dict(cfg=ck.bitvla_config(30), B=1, views=1),
         "cfg4_bitvla_30layer_b8": dict(cfg=ck.bitvla_config(30), B=8, views=1),
     }
@@ -174,7 +175,7 @@ def kernel_breakdown(pkg, cfg, B, P):
     W, S = cfg["expert_h"], cfg["n_suffix"]
     M = B * S
     qd, kvd = Hq * D, Hkv * D
-    gr00t = arch == "gr00t_n1d5"
+    gr00t = arch in ("gr00t_n1d5", "gr00t_n1d6")
     self_layers = [l for l in range(L) if (True if arch in ("pi0", "pi05") else (l % 2 == 0 if arch == "smolvla" else l % 2 == 1))]
     n_self, n_cross = len(self_layers), L - len(self_layers)
     P_self = 0 if gr00t else P
@@ -227,9 +228,17 @@ def kernel_breakdown(pkg, cfg, B, P):
         kcs_c, vcs_c = kv_set(n_rot, B, Hkv, t_cross, D), kv_set(n_rot, B, Hkv, D, t_cross)
         kc_c, vc_c = kcs_c[0], vcs_c[0]
         add("q_rope_cross", proj(Wq, 0, kc_c, vc_c, t_cross, 0), n_cross, "mfma", 2.0 * M * qd * W)
+        # N1.6 / N1.7: every attend_text_every_n-th cross layer reads the (short) text K/V instead
+        n_txt = len([l for l in range(L) if l not in self_layers and l % (2 * cfg["attend_text_every_n"]) == 0]) \
+            if arch == "gr00t_n1d6" else 0
         add("attention_cross", lambda i: pkg.call("vla_attn_prefix_suffix", q, kcs_c[i % n_rot], vcs_c[i % n_rot], att, dt, B, S, Hq, Hkv, D, t_cross,
                                                 P, scale, 0, P, 0, 0, None),
-            n_cross, "hbm", 2 * P * kvd * es * B)
+            n_cross - n_txt, "hbm", 2 * P * kvd * es * B)
+        if n_txt:
+            Pt = cfg["n_lang"]
+            add("attention_cross_text", lambda i: pkg.call("vla_attn_prefix_suffix", q, kcs_c[i % n_rot], vcs_c[i % n_rot], att, dt, B, S, Hq,
+                                                         Hkv, D, t_cross, Pt, scale, 0, Pt, 0, 0, None),
+                n_txt, "hbm", 2 * Pt * kvd * es * B)
     if pi05:
         gatev = torch.ones(W, device=dev)
         add("wo_gated_residual", lambda i: pkg.call("vla_linear_gated", att, Wo, None, gatev, h, h, dt, dt, M, W, qd), L, "mfma",

@@ -31,7 +31,9 @@ def _is_self(cfg, l):
         return True
     if cfg["arch"] == "smolvla":
         return l % cfg["self_attn_every_n"] == 0
-    return l % 2 == 1
+    # GR00T DiT: cross on even, self on odd layers (gr00tn1d5.cpp:361-375); N1.6 / N1.7 only
+    # when dit_interleave is set (gr00tn1d6.cpp:449, 462)
+    return l % 2 == 1 and bool(cfg.get("dit_interleave", 1))
 
 
 def _split_heads(y, Hq, Hkv, D):
@@ -43,7 +45,7 @@ def _split_heads(y, Hq, Hkv, D):
 
 
 def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
-    """SmolVLA / pi0 / pi0.5 / GR00T N1.5 action chunk for one observation.
+    """SmolVLA / pi0 / pi0.5 / GR00T N1.5 / N1.6 action chunk for one observation.
 
     obs: img_emb [views*n_img, hidden], n_views, lang (int32 or None), state, noise
     [n_actions, max_action_dim].  Returns [n_actions, max_action_dim] fp32.
@@ -64,14 +66,24 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
     n_img_tot = views * cfg["n_img"]
     img = np.asarray(obs["img_emb"], np.float32).reshape(n_img_tot, Wv)
     state = np.zeros(cfg["max_state_dim"], np.float32) if obs.get("state") is None else np.asarray(obs["state"], np.float32)
-    gr00t = arch == "gr00t_n1d5"
+    gr00t = arch in ("gr00t_n1d5", "gr00t_n1d6")
+    alt_vl = arch == "gr00t_n1d6"
     pi05 = arch == "pi05"
     n_lead = 0 if arch in ("smolvla", "pi05") else 1
     Sa = S - n_lead
 
     # ---- prefix embeddings, positions, masks
     pad = (0, 0)
-    if gr00t:
+    if alt_vl:
+        # AlternateVLDiT (gr00tn1d6.cpp:440-467, gr00tn1d7.cpp:559-590): cross layer l attends to
+        # the text rows of the backbone features when l % (2 attend_text_every_n) == 0, else to
+        # the image rows; without text both are the image rows.  The text rows here are an
+        # embedding lookup standing in for the backbone's output at the text positions.
+        lang = np.asarray(obs["lang"], np.int32)
+        txt = w["prefix.E_lang"][lang] if lang.size else img
+        pe = img
+        P = n_img_tot
+    elif gr00t:
         pe = img
         P = n_img_tot
     else:
@@ -100,6 +112,8 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
         cs, ss = orc.rope_tables(pos_self, D, base)
         cc, sc_ = orc.rope_tables(pos_cross, D, base)
     pe = rnd(pe)
+    if alt_vl:
+        txt = rnd(txt)
 
     if cfg["suffix_mask"] == 1:
         mask_self = orc.mask_smolvla_full(P, S, pad[0], pad[1])
@@ -117,9 +131,10 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
         if gr00t:
             if self_l:
                 continue
-            kv = orc.linear(pe, w["vlm.%d.Wkv" % l], w["vlm.%d.bkv" % l])
-            cacheK[l] = rnd(kv[:, :kvd]).reshape(P, Hkv, D)
-            cacheV[l] = rnd(kv[:, kvd:]).reshape(P, Hkv, D)
+            src = txt if (alt_vl and l % (2 * cfg["attend_text_every_n"]) == 0) else pe
+            kv = orc.linear(src, w["vlm.%d.Wkv" % l], w["vlm.%d.bkv" % l])
+            cacheK[l] = rnd(kv[:, :kvd]).reshape(src.shape[0], Hkv, D)
+            cacheV[l] = rnd(kv[:, kvd:]).reshape(src.shape[0], Hkv, D)
             continue
         xn = rnd(orc.rms_norm(pe, w["vlm.%d.ln" % l], eps))
         kv = orc.linear(xn, w["vlm.%d.Wkv" % l])

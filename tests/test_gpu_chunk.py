@@ -214,6 +214,32 @@ def test_pi05_adarms_layers(tmp_path, dtype, n_layers, ffn_dim, batch):
     m.close()
 
 
+@pytest.mark.parametrize("n_layers,every,interleave,n_lang,batch", [
+    (8, 2, 1, 21, 2),     # N1.6 / N1.7 defaults: text on layers 0, 4; image on 2, 6; self on odd layers
+    (6, 1, 1, 33, 1),     # text on every cross layer
+    (4, 2, 0, 21, 2),     # no interleave: all layers cross, text on 0, image on 1, 2, 3
+    (4, 2, 1, 0, 1),      # no text rows: the text layers read the image rows
+    (32, 2, 1, 64, 1),    # the full depth
+])
+def test_gr00t_n1d6_alternating_text_and_image_cross_layers(tmp_path, n_layers, every, interleave, n_lang, batch):
+    """AlternateVLDiT (src/models/gr00tn1d6.cpp:445-467, src/models/gr00tn1d7.cpp:565-590): the cross
+    layers' resident K/V come from the text rows or the image rows of the backbone features."""
+    cfg = ckpt.gr00t_n1d6_config(n_layers=n_layers, attend_text_every_n=every, dit_interleave=interleave)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 17)
+    r = np.random.default_rng(320 + n_layers)
+    obs = [make_obs(cfg, r, n_views=2, n_lang=n_lang) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "n1d6")
+    got = m.predict_batch(obs).reshape(batch, 16, 32)
+    for b in range(batch):
+        want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+        assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    if n_lang:
+        # the text rows are really used: other tokens, another chunk
+        other = dict(obs[0], lang=(obs[0]["lang"] + 1) % cfg["vocab"])
+        assert not np.allclose(orc_chunk.flow_expert_chunk(cfg, w, other, emulate_bf16=True), got[0], atol=1e-3)
+    m.close()
+
+
 @pytest.mark.parametrize("from_fp32", [False, True])
 def test_config4_bitvla_ternary_append(tmp_path, from_fp32):
     cfg = ckpt.bitvla_config(n_layers=2)

@@ -95,6 +95,16 @@ def gr00t_config(n_layers=16, dtype="bf16", num_steps=4, n_suffix=17):
                 norm_out_eps=1e-6, rope_freq_base=10000.0, vocab=0, suffix_mask=0, max_views=2)
 
 
+def gr00t_n1d6_config(n_layers=32, dtype="bf16", num_steps=4, n_suffix=17, attend_text_every_n=2, dit_interleave=1):
+    """GR00T N1.6 / N1.7 DiT head (AlternateVLDiT, src/models/gr00tn1d6.cpp:85-86, 445-467;
+    src/models/gr00tn1d7.cpp:75, 565-590): the N1.5 block, 32 layers, whose cross layers
+    alternate between the text rows (layer % (2 attend_text_every_n) == 0) and the image rows
+    of the backbone features; up to 64 text rows (an embedding lookup stands in for them)."""
+    c = gr00t_config(n_layers, dtype, num_steps, n_suffix)
+    c.update(arch="gr00t_n1d6", n_lang=64, vocab=512, attend_text_every_n=attend_text_every_n, dit_interleave=dit_interleave)
+    return c
+
+
 def bitvla_config(n_layers=30):
     """BitVLA / BitNet b1.58 2B shape (src/models/bitvla.cpp:121-122): width 2560,
     20 query / 5 KV heads of 128, RoPE base 5e5; prefix 256 image + 256 text tokens,
@@ -109,7 +119,7 @@ def _is_self(cfg, l):
         return True
     if cfg["arch"] == "smolvla":
         return l % cfg["self_attn_every_n"] == 0
-    return l % 2 == 1  # gr00t: cross on even layers
+    return l % 2 == 1 and bool(cfg.get("dit_interleave", 1))  # gr00t: cross on even layers
 
 
 def synth_weights(cfg, seed=0x5EED):
@@ -147,7 +157,8 @@ def synth_weights(cfg, seed=0x5EED):
         return w
     W = cfg["expert_h"]
     if cfg.get("vocab", 0) > 0:
-        w["prefix.E_lang"] = (r.standard_normal((cfg["vocab"], Wv)) / np.sqrt(Wv)).astype(np.float32)
+        # N1.6: the rows stand for backbone features at the text positions, O(1) like the image rows
+        w["prefix.E_lang"] = (r.standard_normal((cfg["vocab"], Wv)) / (1.0 if arch == "gr00t_n1d6" else np.sqrt(Wv))).astype(np.float32)
     if arch == "smolvla":
         w["prefix.Wstate"] = (0.1 * r.standard_normal((Wv, cfg["max_state_dim"]))).astype(np.float32)
         w["prefix.bstate"] = vec(Wv, 0.1)
@@ -168,7 +179,7 @@ def synth_weights(cfg, seed=0x5EED):
         w["te.b_tout"] = vec(W, 0.1)
         w["act.ada_final_w"] = ada_w()
         w["act.ada_final_b"] = ada_b()
-    elif arch != "gr00t_n1d5":
+    elif arch not in ("gr00t_n1d5", "gr00t_n1d6"):
         w["act.norm"] = nrm(W)
         if cfg.get("time_mlp", 0):  # action_time_mlp_in / _out of the suffix embedding
             w["act.W_at1"] = (r.standard_normal((W, 2 * W)) / np.sqrt(2 * W)).astype(np.float32)
@@ -183,7 +194,7 @@ def synth_weights(cfg, seed=0x5EED):
     for l in range(cfg["n_layers"]):
         p, v = "ex.%d." % l, "vlm.%d." % l
         self_l = _is_self(cfg, l)
-        if arch == "gr00t_n1d5":
+        if arch in ("gr00t_n1d5", "gr00t_n1d6"):
             w[p + "adaln_w"] = mat(2 * W, W)
             w[p + "adaln_b"] = vec(2 * W)
             if self_l:

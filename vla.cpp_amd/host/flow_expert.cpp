@@ -88,6 +88,7 @@ struct LayerW {
     DevBuf Wk_x, Wv_x;          // SmolVLA cross layers: re-projection of the cached prefix K / V
     KVLayer kv;
     bool needs_prefix = true;
+    bool from_text = false;  // cross K/V from the text rows of the prefix (else image rows, or all rows)
 };
 
 class FlowExpert : public ModelArch {
@@ -105,7 +106,7 @@ class FlowExpert : public ModelArch {
     }
 
   private:
-    void allocate(int B, int P);
+    void allocate(int B, int P, int P_txt = 0);
     uint32_t alloc_gen_ = 0;
 
     Arch arch_;
@@ -123,6 +124,8 @@ class FlowExpert : public ModelArch {
     DevBuf W_in_, W_out_, b_out_, final_norm_;
     DevBuf W_at2_, b_at2_, m1_;  // action-time MLP: second projection, fp32 scratch [B*S][W]
     bool time_mlp_ = false;
+    bool alt_vl_ = false;   // GR00T N1.6 / N1.7: cross layers alternate text / image rows
+    int text_every_ = 2, P_txt_ = 0;
     bool adarms_ = false;  // pi0.5: ada_ holds [steps][2L+1][scale, shift, gate][W]
     DevBuf bias_step_;   // [steps][W] fp32: b_in (+ time embedding of the step)
     DevBuf ada_;         // GR00T: [steps][L+1][2][W] fp32 (scale, shift); slot L is the final norm (zeros)
@@ -142,6 +145,13 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     // suffix and no suffix mask (src/models/pi05.cpp:208-283, 610-631)
     adarms_ = arch == "pi05";
     arch_ = arch == "smolvla" ? Arch::SMOLVLA : (arch == "pi0" || adarms_) ? Arch::PI0 : Arch::GR00T;
+    // GR00T N1.6 / N1.7 (AlternateVLDiT): the cross layers alternate between the text rows and
+    // the image rows of the backbone features (src/models/gr00tn1d6.cpp:445-467,
+    // src/models/gr00tn1d7.cpp:565-590); N1.5 attends to all rows on every cross layer.
+    alt_vl_ = arch == "gr00t_n1d6";
+    text_every_ = (int)ck.i64("attend_text_every_n", 2);
+    const bool interleave = ck.i64("dit_interleave", 1) != 0;
+    if (alt_vl_ && text_every_ < 1) throw std::runtime_error("vla: attend_text_every_n must be >= 1");
     dt_ = ck.str("dtype") == "bf16" ? VLA_DT_BF16 : VLA_DT_F32;
     L_ = (int)ck.i64("n_layers");
     Hq_ = (int)ck.i64("n_q_heads");
@@ -215,8 +225,9 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         const std::string p = "ex." + std::to_string(l) + ".";
         // SmolVLA: self iff l % every == 0 (src/models/smolvla.cpp:1182); GR00T N1.5:
         // cross on even, self on odd layers (src/models/gr00tn1d5.cpp:361-375).
-        w.is_self = arch_ == Arch::PI0 ? true : arch_ == Arch::SMOLVLA ? (l % every == 0) : (l % 2 == 1);
+        w.is_self = arch_ == Arch::PI0 ? true : arch_ == Arch::SMOLVLA ? (l % every == 0) : (interleave && l % 2 == 1);
         w.needs_prefix = !(arch_ == Arch::GR00T && w.is_self);
+        w.from_text = alt_vl_ && w.needs_prefix && l % (2 * text_every_) == 0;
         if (arch_ != Arch::GR00T && !adarms_) w.ln = load_w(ck, p + "ln", dt_);
         w.Wqkv = load_w(ck, p + (w.is_self ? "Wqkv" : "Wq"), dt_);
         if (arch_ != Arch::GR00T && !adarms_ && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
@@ -361,14 +372,17 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     }
 }
 
-void FlowExpert::allocate(int B, int P) {
-    if (B == B_ && P == P_) return;
+void FlowExpert::allocate(int B, int P, int P_txt) {
+    if (B == B_ && P == P_ && P_txt == P_txt_) return;
     B_ = B;
     P_ = P;
+    P_txt_ = P_txt;
     ++alloc_gen_;
     const size_t es = dtype_size(dt_);
     for (LayerW& w : layers_) {
-        const int prefix = w.needs_prefix ? P : 0;
+        // alternating layers: text rows, or image rows (all rows when there is no text:
+        // vl_txt = vl_img then, gr00tn1d6.cpp:443)
+        const int prefix = !w.needs_prefix ? 0 : !alt_vl_ ? P : (w.from_text && P_txt > 0) ? P_txt : P - P_txt;
         const int tmax = round_up(prefix + (w.is_self ? S_ : 0), 64);
         w.kv.create(dt_, B, Hkv_, D_, tmax);
         w.kv.n_prefix = prefix;
@@ -393,12 +407,12 @@ void FlowExpert::allocate(int B, int P) {
 
 void FlowExpert::prefill(const Inputs* in, int batch) {
     if (!in || batch <= 0) throw std::invalid_argument("vla: prefill needs at least one observation");
-    const int views = in[0].n_img_views, n_lang = arch_ == Arch::GR00T ? 0 : in[0].n_lang;
+    const int views = in[0].n_img_views, n_lang = (arch_ == Arch::GR00T && !alt_vl_) ? 0 : in[0].n_lang;
     if (views < 1 || views > max_views_) throw std::invalid_argument("vla: n_img_views out of range");
     if (n_lang < 0 || n_lang > n_lang_max_) throw std::invalid_argument("vla: n_lang out of range");
     for (int b = 0; b < batch; ++b) {
         if (!in[b].precomputed_img_emb) throw std::invalid_argument("vla: precomputed_img_emb is required");
-        if (in[b].n_img_views != views || (arch_ != Arch::GR00T && in[b].n_lang != n_lang))
+        if (in[b].n_img_views != views || ((arch_ != Arch::GR00T || alt_vl_) && in[b].n_lang != n_lang))
             throw std::invalid_argument("vla: a batch shares one n_img_views and one n_lang");
         if (n_lang > 0 && !in[b].lang_tokens) throw std::invalid_argument("vla: lang_tokens missing");
         for (int i = 0; i < n_lang; ++i)
@@ -410,8 +424,9 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
     // (src/models/smolvla.cpp:1608-1612); pi0 uses the real length (pi0.cpp:526-528).
     const int P = arch_ == Arch::SMOLVLA ? n_img_tot + n_lang_max_ + 1
                   : arch_ == Arch::PI0   ? n_img_tot + n_lang
+                  : alt_vl_              ? n_img_tot + n_lang
                                          : n_img_tot;
-    allocate(batch, P);
+    allocate(batch, P, alt_vl_ ? n_lang : 0);
     const int B = batch;
     Ctx C;  // prefill runs on the default stream and is synchronous
 
@@ -420,15 +435,23 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
     const float lang_scale = std::sqrt((float)Wv_);
     for (int b = 0; b < B; ++b) {
         float* dst = pe.data() + (size_t)b * P * Wv_;
+        // alternating layers project the image rows and the text rows separately: all image
+        // rows of the batch first, then all text rows, each block [B][rows][Wv]
+        float* txt_dst = dst + (size_t)n_img_tot * Wv_;
+        if (alt_vl_) {
+            dst = pe.data() + (size_t)b * n_img_tot * Wv_;
+            txt_dst = pe.data() + ((size_t)B * n_img_tot + (size_t)b * n_lang) * Wv_;
+        }
         const float img_scale = arch_ == Arch::SMOLVLA ? lang_scale : 1.0f;  // smolvla.cpp:1363 vs pi0.cpp:554-555
         for (size_t i = 0; i < (size_t)n_img_tot * Wv_; ++i) dst[i] = in[b].precomputed_img_emb[i] * img_scale;
-        if (arch_ != Arch::GR00T) {
+        if (arch_ != Arch::GR00T || alt_vl_) {
             const int rows = arch_ == Arch::SMOLVLA ? n_lang_max_ : n_lang;
+            const float ls = alt_vl_ ? 1.0f : lang_scale;  // N1.6: the rows stand for backbone features, unscaled
             for (int i = 0; i < rows; ++i) {
                 const int tok = i < n_lang ? in[b].lang_tokens[i] : 0;  // zero-padded ids, smolvla.cpp:1628-1629
                 const float* e = E_lang_.data() + (size_t)tok * Wv_;
-                float* row = dst + (size_t)(n_img_tot + i) * Wv_;
-                for (int c = 0; c < Wv_; ++c) row[c] = e[c] * lang_scale;
+                float* row = txt_dst + (size_t)i * Wv_;
+                for (int c = 0; c < Wv_; ++c) row[c] = e[c] * ls;
             }
         }
         std::vector<float> st(max_state_, 0.f);
@@ -474,6 +497,14 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
         if (!w.needs_prefix) continue;
         Tensor Wkv = tensor_2d(w.Wkv_pre.get(), dt_, Wv_, 2 * kvd);
         const float* bkv = w.bkv_pre ? w.bkv_pre.as<float>() : nullptr;
+        if (alt_vl_) {
+            const bool txt = w.from_text && P_txt_ > 0;
+            const int rows = txt ? P_txt_ : P - P_txt_;
+            const char* base = (const char*)prefix_.get() + (txt ? (size_t)B * (P - P_txt_) * Wv_ * dtype_size(dt_) : 0);
+            Tensor xs = tensor_2d(const_cast<char*>(base), dt_, Wv_, (int64_t)B * rows);
+            qkv_rope_append(C, xs, Wkv, bkv, rows, 0, true, true, nullptr, nullptr, w.kv, 0);
+            continue;
+        }
         if (arch_ == Arch::GR00T) {
             qkv_rope_append(C, xp, Wkv, bkv, P, 0, true, true, nullptr, nullptr, w.kv, 0);
             continue;

@@ -98,7 +98,7 @@ Model* model_load(const std::string&, const std::string& ckpt_path, const std::s
     Checkpoint ck(ckpt_path);
     const std::string arch = ck.str("arch");
     ModelArch* a = nullptr;
-    if (arch == "smolvla" || arch == "pi0" || arch == "pi05" || arch == "gr00t_n1d5") a = flow_expert_create(ck);
+    if (arch == "smolvla" || arch == "pi0" || arch == "pi05" || arch == "gr00t_n1d5" || arch == "gr00t_n1d6") a = flow_expert_create(ck);
     else if (arch == "bitvla") a = bitvla_create(ck);
     else throw std::runtime_error("vla: unknown architecture '" + arch + "'");
     Model* m = new Model();
