@@ -1,0 +1,208 @@
+"""GGUF reader (include/vla_gguf.h) and GGUF checkpoints through vla_model_load.
+
+CPU part: the reader against a file assembled byte by byte from the container's published
+layout (independent of the package's writer), writer -> reader round trips, the
+conversions, and malformed files.  GPU part: the same synthetic weights loaded from a GGUF
+under the reference's tensor names and from the VLAW container give the same chunk, bit for bit.
+"""
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from util import declared_symbols, pkg
+
+from vla_cpp_amd import checkpoint as ckpt  # noqa: E402
+from vla_cpp_amd import gguf  # noqa: E402
+
+
+def gs(text):
+    return struct.pack("<Q", len(text)) + text.encode()
+
+
+def hand_made_file(version=3):
+    """magic, version, counts; 6 metadata records; 3 tensor records; padding to 64; data."""
+    f32_data = np.arange(6, dtype=np.float32).reshape(2, 3) - 2.5          # ne = [3, 2]
+    bf_vals = np.float32([1.0, -2.0, 0.5, 3.140625])                          # exact in bf16
+    bf_data = (bf_vals.view(np.uint32) >> 16).astype(np.uint16)               # ne = [4]
+    i8_data = np.int8([-1, 0, 1, 2, -128, 127, 5, 6])                         # ne = [8]
+    kv = b""
+    kv += gs("general.alignment") + struct.pack("<II", 4, 64)
+    kv += gs("smolvla.hidden") + struct.pack("<II", 4, 960)
+    kv += gs("some.eps") + struct.pack("<If", 6, 1e-6)
+    kv += gs("some.period") + struct.pack("<Id", 12, 4e-3)
+    kv += gs("general.name") + struct.pack("<I", 8) + gs("hand made")
+    kv += gs("tok.list") + struct.pack("<IIQ", 9, 8, 2) + gs("a") + gs("bc")
+    ti = b""
+    ti += gs("w.f32") + struct.pack("<IQQIQ", 2, 3, 2, 0, 0)
+    ti += gs("w.bf16") + struct.pack("<IQIQ", 1, 4, 30, 64)
+    ti += gs("w.i8") + struct.pack("<IQIQ", 1, 8, 24, 128)
+    head = b"GGUF" + struct.pack("<IQQ", version, 3, 6) + kv + ti
+    data_off = (len(head) + 63) // 64 * 64
+    blob = head + b"\0" * (data_off - len(head))
+    blob += f32_data.tobytes() + b"\0" * (64 - 24) + bf_data.tobytes() + b"\0" * (64 - 8) + i8_data.tobytes()
+    return blob, data_off, f32_data, bf_vals, i8_data
+
+
+def test_header_declares_and_library_exports_the_reader():
+    names = declared_symbols("vla_gguf.h")
+    assert len(names) == 18
+    for n in names:
+        assert hasattr(pkg.lib(), n), "libvla.so does not export %s" % n
+
+
+@pytest.mark.parametrize("version", [2, 3])
+def test_reader_on_a_hand_assembled_file(tmp_path, version):
+    blob, data_off, f32_data, bf_vals, i8_data = hand_made_file(version)
+    path = os.path.join(str(tmp_path), "hand.gguf")
+    open(path, "wb").write(blob)
+    with gguf.Reader(pkg.lib(), path) as g:
+        assert g.version == version and g.data_offset == data_off
+        assert g.has("smolvla.hidden") and not g.has("smolvla.missing")
+        assert g.u32("smolvla.hidden") == 960 and g.u32("general.alignment") == 64
+        assert g.f32("some.eps") == np.float32(1e-6) and g.f64("some.period") == 4e-3
+        assert g.str("general.name") == "hand made"
+        assert g.array_len("tok.list") == (2, gguf.STRING)
+        # a key of another type reads as the zero value (no abort), a missing one too
+        assert g.u32("some.eps") == 0 and g.f32("smolvla.hidden") == 0.0 and g.str("smolvla.hidden") == "" and g.u32("nope") == 0
+        assert g.key_type("some.period") == gguf.F64 and g.key_type("nope") == -1
+        assert g.tensor_names() == ["w.f32", "w.bf16", "w.i8"]
+        m = g.meta("w.f32")
+        assert m == dict(type=0, n_dims=2, ne=[3, 2, 1, 1], offset=0, nbytes=24)
+        assert g.meta("w.bf16")["nbytes"] == 8 and g.meta("w.i8")["offset"] == 128 and g.meta("absent") is None
+        assert np.array_equal(g.read_f32("w.f32"), f32_data)
+        assert np.array_equal(g.read_f32("w.bf16"), bf_vals)
+        assert g.read_f32("w.i8") is None                       # not a float tensor
+        assert np.array_equal(g.read_raw("w.i8", 8).view(np.int8), i8_data)
+        assert g.read_raw("w.i8", 7) is None and g.read_raw("absent", 8) is None   # cap must match
+        assert np.array_equal(g.fetch_rows_f32("w.f32", [1, 0, 1], 3), f32_data[[1, 0, 1]])
+        assert g.fetch_rows_f32("w.f32", [2], 3) is None and g.fetch_rows_f32("w.f32", [0], 2) is None
+        # conversions: bf16 -> f32 exact; f32 -> bf16 rounds to nearest even; the Gemma +1
+        assert np.array_equal(g.read_convert("w.bf16", gguf.T_F32).view(np.float32), bf_vals)
+        assert np.array_equal(g.read_convert("w.f32", gguf.T_BF16).view(np.uint16), orc.to_bf16(f32_data).ravel())
+        assert np.array_equal(g.read_convert("w.bf16", gguf.T_F32, gemma_norm=True).view(np.float32), bf_vals + 1)
+        assert np.array_equal(g.read_convert("w.i8", gguf.T_I8).view(np.int8), i8_data)
+        assert g.read_convert("w.i8", gguf.T_I8, gemma_norm=True) is None
+
+
+def test_writer_round_trip_types_alignment_and_half(tmp_path):
+    r = np.random.default_rng(7)
+    a = r.standard_normal((5, 7)).astype(np.float32)
+    h = np.float16([0.0, -0.0, 1.0, 65504.0, 6.1e-5, 5.96e-8, -2.5, np.inf])   # normal, max, subnormal, inf
+    b = r.standard_normal((3, 2, 4)).astype(np.float32)
+    kv = {"x.u32": (gguf.U32, 7), "x.i64": (gguf.I64, -5), "x.b": (gguf.BOOL, 1), "x.s": (gguf.STRING, "héllo"),
+          "x.arr": (gguf.ARRAY, (gguf.F32, [1.0, 2.0, 3.0]))}
+    for align in (32, 128):
+        path = os.path.join(str(tmp_path), "rt%d.gguf" % align)
+        gguf.write_gguf(path, kv, {"a": (gguf.T_F32, a), "h": (gguf.T_F16, h), "b": (gguf.T_BF16, gguf.bf16_bits(b)),
+                                   "one": (gguf.T_F32, np.float32([3.0]))}, alignment=align)
+        with gguf.Reader(pkg.lib(), path) as g:
+            assert g.data_offset % align == 0 and all(g.meta(n)["offset"] % align == 0 for n in g.tensor_names())
+            assert g.u32("x.u32") == 7 and g.str("x.s") == "héllo" and g.array_len("x.arr") == (3, gguf.F32)
+            assert np.array_equal(g.read_f32("a"), a)
+            assert np.array_equal(g.read_f32("h"), h.astype(np.float32))
+            assert np.array_equal(g.read_f32("b"), orc.round_bf16(b)) and g.meta("b")["ne"] == [4, 2, 3, 1]
+            assert np.array_equal(g.fetch_rows_f32("h", [0], 8)[0], h.astype(np.float32))
+    assert np.array_equal(gguf.bf16_bits(b), orc.to_bf16(b))
+
+
+def test_malformed_files_fail_to_open_instead_of_crashing(tmp_path):
+    blob, data_off, *_ = hand_made_file()
+    path = os.path.join(str(tmp_path), "bad.gguf")
+
+    def opens(data):
+        open(path, "wb").write(data)
+        try:
+            gguf.Reader(pkg.lib(), path).close()
+            return True
+        except RuntimeError:
+            return False
+
+    assert opens(blob)
+    assert not opens(b"GGML" + blob[4:]) and not opens(blob[:4] + struct.pack("<I", 1) + blob[8:])
+    # every truncation inside the header or the tensor data is refused
+    for cut in list(range(0, data_off, 7)) + [data_off, data_off + 64, len(blob) - 1]:
+        assert not opens(blob[:cut]), cut
+    # a string length, a record count or a tensor offset that points past the end
+    huge = struct.pack("<Q", 1 << 60)
+    assert not opens(blob[:24] + huge + blob[32:])            # first key's length
+    assert not opens(blob[:8] + huge + blob[16:]) and not opens(blob[:16] + huge + blob[24:])
+    i = blob.index(b"w.i8") + 4 + 4 + 8 + 4
+    assert not opens(blob[:i] + struct.pack("<Q", 1 << 20) + blob[i + 8:])   # offset beyond the file
+    assert not opens(blob[:i] + struct.pack("<Q", 130) + blob[i + 8:])       # misaligned offset
+    assert not os.path.exists(path + ".none") and not opens.__call__(b"")
+
+
+# ------------------------------------------------------------------ through vla_model_load
+def _chunk(path, obs, shape):
+    from vla_cpp_amd import ffi
+    m = ffi.Model(path)
+    out = m.predict_batch(obs).reshape(shape)
+    m.close()
+    return out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_smolvla_gguf_under_reference_names_equals_the_vlaw_checkpoint(tmp_path, monkeypatch, dtype):
+    from test_gpu_chunk import make_obs
+    cfg = ckpt.smolvla_config(n_layers=4, dtype=dtype, suffix_mask=1)
+    cfg.update(ffn_dim=512, time_mlp=1)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 21)
+    r = np.random.default_rng(330)
+    obs = [make_obs(cfg, r, n_views=2, n_lang=31) for _ in range(2)]
+    pv, pg = os.path.join(str(tmp_path), "m.vlaw"), os.path.join(str(tmp_path), "m.gguf")
+    ckpt.write_synthetic(pv, cfg, w)
+    gguf.write_synthetic_gguf(pg, cfg, w)
+    monkeypatch.setenv("VLA_WEIGHT_DTYPE", dtype)
+    want = _chunk(pv, obs, (2, 50, 32))
+    got = _chunk(pg, obs, (2, 50, 32))
+    assert np.array_equal(got, want) and np.abs(want).max() > 0.1
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("packed", [False, True])
+def test_bitvla_gguf_float_and_int2_packed_equal_the_vlaw_checkpoint(tmp_path, packed):
+    from test_gpu_chunk import make_obs
+    cfg = ckpt.bitvla_config(n_layers=2)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 22)
+    r = np.random.default_rng(331)
+    obs = [make_obs(cfg, r, n_views=1) for _ in range(2)]
+    pv, pg = os.path.join(str(tmp_path), "b.vlaw"), os.path.join(str(tmp_path), "b.gguf")
+    ckpt.write_synthetic(pv, cfg, w, ladder_pack=orc.pack_ladder_int2 if packed else None)
+    gguf.write_synthetic_gguf(pg, cfg, w, ladder_pack=orc.pack_ladder_int2 if packed else None)
+    want = _chunk(pv, obs, (2, 7, 32))
+    got = _chunk(pg, obs, (2, 7, 32))
+    assert np.array_equal(got, want) and np.abs(want).max() > 1e-3
+
+
+@pytest.mark.gpu
+def test_gguf_with_a_missing_or_misshapen_tensor_fails_to_load(tmp_path):
+    from vla_cpp_amd import ffi
+    cfg = ckpt.smolvla_config(n_layers=2, dtype="bf16", suffix_mask=1)
+    cfg.update(ffn_dim=256, time_mlp=1)
+    w = ckpt.synth_weights(cfg, seed=3)
+    for damage in ("drop", "shape", "arch"):
+        w2 = dict(w)
+        cfg2 = dict(cfg)
+        if damage == "drop":
+            del w2["ex.1.Wo"]
+        elif damage == "shape":
+            w2["ex.0.Wd"] = w2["ex.0.Wd"][:, :-8]
+        p = os.path.join(str(tmp_path), damage + ".gguf")
+        if damage == "drop":
+            with pytest.raises(KeyError):
+                gguf.write_synthetic_gguf(p, cfg2, w2)
+            w2["ex.1.Wo"] = w["ex.1.Wo"]
+            gguf.write_synthetic_gguf(p, cfg2, w2)
+            # cut the tensor out by renaming it inside the file (same length, so offsets hold)
+            data = open(p, "rb").read().replace(b"aex.blk.1.attn_o.weight", b"aex.blk.1.attn_x.weight")
+            open(p, "wb").write(data)
+        elif damage == "shape":
+            gguf.write_synthetic_gguf(p, cfg2, w2)
+        else:
+            gguf.write_gguf(p, {"general.architecture": (gguf.STRING, "llama")}, {"t": (gguf.T_F32, np.float32([1]))})
+        with pytest.raises(RuntimeError):
+            ffi.Model(p)

@@ -1,6 +1,7 @@
-// Reader for "VLAW" checkpoints: the flat container this library loads in place
-// of the reference's GGUF files (src/gguf_reader.h, src/loader.cpp; reading
-// GGUF is outside this library's scope).  Layout:
+// Weight container the model builders read.  Filled either from a "VLAW" file (the flat
+// container written by vla.cpp_amd/checkpoint.py) or in memory by the GGUF importer
+// (gguf_import.cpp), which maps the reference's tensor names (src/models/*.cpp) onto the
+// names used here.  VLAW layout:
 //
 //   bytes 0..7   "VLAW0001"
 //   bytes 8..15  header length H (little-endian uint64)
@@ -37,6 +38,31 @@ struct CkptTensor {
 
 class Checkpoint {
   public:
+    Checkpoint() = default;  // empty; filled with set_key / add_tensor
+
+    void set_key(const std::string& k, const std::string& v) { kv_[k] = v; }
+    void set_key(const std::string& k, int64_t v) { kv_[k] = std::to_string(v); }
+    void set_key(const std::string& k, double v) {
+        char buf[64];
+        std::snprintf(buf, sizeof(buf), "%.17g", v);
+        kv_[k] = buf;
+    }
+    // Appends a tensor (bytes copied, 64-byte aligned); dtype as in the VLAW header.
+    void add_tensor(const std::string& name, const std::string& dtype, const std::vector<int64_t>& shape, const void* bytes,
+                    size_t nbytes) {
+        CkptTensor t;
+        t.dtype = dtype;
+        t.shape = shape;
+        t.offset = (blob_.size() + 63) / 64 * 64;
+        t.nbytes = nbytes;
+        blob_.resize(t.offset + nbytes);
+        if (nbytes) std::memcpy(blob_.data() + t.offset, bytes, nbytes);
+        tensors_[name] = t;
+    }
+    void add_f32(const std::string& name, const std::vector<int64_t>& shape, const std::vector<float>& v) {
+        add_tensor(name, "f32", shape, v.data(), v.size() * sizeof(float));
+    }
+
     explicit Checkpoint(const std::string& path) {
         FILE* f = std::fopen(path.c_str(), "rb");
         if (!f) throw std::runtime_error("vla: cannot open checkpoint " + path);
@@ -120,5 +146,11 @@ class Checkpoint {
     std::map<std::string, std::string> kv_;
     std::map<std::string, CkptTensor> tensors_;
 };
+
+// GGUF input (gguf_import.cpp): true when the file starts with the GGUF magic; import_gguf
+// reads the tensors on the action-expert path under the reference's names and throws
+// std::runtime_error on a file it cannot use.
+bool is_gguf_file(const std::string& path);
+Checkpoint import_gguf(const std::string& path);
 
 }  // namespace vla

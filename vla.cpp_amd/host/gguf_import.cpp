@@ -1,0 +1,380 @@
+// GGUF checkpoints -> the in-memory weight container the model builders read.
+//
+// The reference's loaders read their tensors by the names its converters write
+// (SmolVLA: hf_to_gguf, src/models/smolvla.cpp:648-755 and the tensor list at 1099-1236;
+// BitVLA: src/models/bitvla.cpp:349-373, 640-700).  This file maps those names and metadata
+// keys onto the container's own names, fusing what the kernels want fused:
+//   [attn_q; attn_k; attn_v] rows -> Wqkv, [attn_k; attn_v] of a backbone layer -> Wkv,
+//   [ffn_gate; ffn_up] rows -> Wgu.
+// Only the tensors on the action-expert attention path (and the expert's FFN / embedding
+// MLPs around it) are read; vision tower, connector and backbone FFN tensors are ignored.
+// Also here: the C ABI over the reader itself (include/vla_gguf.h).
+#include <cstdlib>
+#include <memory>
+#include <stdexcept>
+
+#include "checkpoint.h"
+#include "gguf_reader.h"
+#include "vla_gguf.h"
+#include "vla_kernels.h"
+
+namespace vla {
+
+bool is_gguf_file(const std::string& path) {
+    FILE* f = std::fopen(path.c_str(), "rb");
+    if (!f) return false;
+    char m[4] = {0, 0, 0, 0};
+    const size_t n = std::fread(m, 1, 4, f);
+    std::fclose(f);
+    return n == 4 && std::memcmp(m, "GGUF", 4) == 0;
+}
+
+namespace {
+
+struct Importer {
+    gguf_reader& g;
+    Checkpoint& ck;
+    bool bf16;
+
+    // fp32 tensor `name` with exactly `rows` x `cols` elements (ne0 = cols)
+    std::vector<float> mat(const std::string& name, int64_t rows, int64_t cols) {
+        const gguf_tensor_meta* t = g.meta(name.c_str());
+        if (!t) throw std::runtime_error("vla: gguf has no tensor " + name);
+        const int64_t r = t->nelements() / t->ne[0];
+        if (t->ne[0] != cols || r != rows)
+            throw std::runtime_error("vla: gguf tensor " + name + " is [" + std::to_string(r) + " x " + std::to_string(t->ne[0]) +
+                                     "], expected [" + std::to_string(rows) + " x " + std::to_string(cols) + "]");
+        std::vector<float> v = g.read_f32(name.c_str());
+        if (v.empty()) throw std::runtime_error("vla: cannot read gguf tensor " + name);
+        return v;
+    }
+    std::vector<float> vec(const std::string& name, int64_t n) { return mat(name, 1, n); }
+
+    // matrices in the model's weight type, everything else fp32
+    void put_weight(const std::string& name, int64_t rows, int64_t cols, const std::vector<float>& v) {
+        if (!bf16) {
+            ck.add_f32(name, {rows, cols}, v);
+            return;
+        }
+        std::vector<uint16_t> h(v.size());
+        for (size_t i = 0; i < v.size(); ++i) h[i] = gguf_float_to_bf16(v[i]);
+        ck.add_tensor(name, "bf16", {rows, cols}, h.data(), h.size() * 2);
+    }
+    // rows of several gguf matrices stacked into one weight
+    void put_stacked(const std::string& name, const std::vector<std::string>& parts, const std::vector<int64_t>& rows, int64_t cols) {
+        std::vector<float> all;
+        int64_t total = 0;
+        for (size_t i = 0; i < parts.size(); ++i) {
+            const std::vector<float> p = mat(parts[i], rows[i], cols);
+            all.insert(all.end(), p.begin(), p.end());
+            total += rows[i];
+        }
+        put_weight(name, total, cols, all);
+    }
+};
+
+uint32_t need_u32(const gguf_reader& g, const char* k) {
+    if (!g.has(k)) throw std::runtime_error(std::string("vla: gguf missing key '") + k + "'");
+    return g.u32(k);
+}
+
+// SmolVLA: keys of load_config_from_gguf (src/models/smolvla.cpp:570-634), tensors of
+// smolvla_create (1099-1236) under their GGUF names (648-755).
+void import_smolvla(gguf_reader& g, Checkpoint& ck, bool bf16) {
+    if (g.str("smolvla.architecture") != "smolvla") throw std::runtime_error("vla: gguf architecture is not 'smolvla'");
+    const int64_t hidden = need_u32(g, "smolvla.hidden"), Hq = need_u32(g, "smolvla.n_q_heads"), Hkv = need_u32(g, "smolvla.n_kv_heads"),
+                  D = need_u32(g, "smolvla.head_dim"), L = need_u32(g, "smolvla.n_layers"), vocab = need_u32(g, "smolvla.vocab_size"),
+                  W = need_u32(g, "smolvla.expert_h"), I = need_u32(g, "smolvla.expert_inter"), S = need_u32(g, "smolvla.chunk_size"),
+                  steps = need_u32(g, "smolvla.num_steps"), sd = need_u32(g, "smolvla.max_state_dim"),
+                  ad = need_u32(g, "smolvla.max_action_dim"), every = need_u32(g, "smolvla.self_attn_every_n_layers"),
+                  n_lang = need_u32(g, "smolvla.tokenizer_max_length");
+    if (!g.has("smolvla.min_period") || !g.has("smolvla.max_period")) throw std::runtime_error("vla: gguf missing key 'smolvla.min_period/max_period'");
+    if (every < 1 || L < 1 || Hkv < 1 || Hq % Hkv) throw std::runtime_error("vla: gguf geometry is not usable");
+    const int64_t qd = Hq * D, kvd = Hkv * D;
+    ck.set_key("arch", "smolvla");
+    ck.set_key("dtype", bf16 ? "bf16" : "f32");
+    ck.set_key("n_layers", L);
+    ck.set_key("n_q_heads", Hq);
+    ck.set_key("n_kv_heads", Hkv);
+    ck.set_key("head_dim", D);
+    ck.set_key("hidden", hidden);
+    ck.set_key("expert_h", W);
+    ck.set_key("ffn_dim", I);
+    ck.set_key("n_img", (int64_t)(g.has("smolvla.n_img_tokens") ? g.u32("smolvla.n_img_tokens") : 64));
+    ck.set_key("n_lang", n_lang);
+    ck.set_key("n_suffix", S);
+    ck.set_key("max_action_dim", ad);
+    ck.set_key("max_state_dim", sd);
+    ck.set_key("real_action_dim", (int64_t)need_u32(g, "smolvla.real_action_dim"));
+    ck.set_key("real_state_dim", (int64_t)need_u32(g, "smolvla.real_state_dim"));
+    ck.set_key("num_steps", steps);
+    ck.set_key("rms_eps", 1e-5);                // fixed by the loader, smolvla.cpp:623-625
+    ck.set_key("rope_freq_base", 10000.0);
+    ck.set_key("self_attn_every_n", every);
+    ck.set_key("min_period", g.f64("smolvla.min_period"));
+    ck.set_key("max_period", g.f64("smolvla.max_period"));
+    ck.set_key("vocab", vocab);
+
+    Importer im{g, ck, bf16};
+    ck.add_f32("prefix.E_lang", {vocab, hidden}, im.mat("token_embd.weight", vocab, hidden));
+    ck.add_f32("prefix.Wstate", {hidden, sd}, im.mat("state_proj.weight", hidden, sd));
+    ck.add_f32("prefix.bstate", {hidden}, im.vec("state_proj.bias", hidden));
+    ck.add_f32("act.W_in", {W, ad}, im.mat("action_in_proj.weight", W, ad));
+    ck.add_f32("act.b_in", {W}, im.vec("action_in_proj.bias", W));
+    ck.add_f32("act.W_at1", {W, 2 * W}, im.mat("action_time_mlp_in.weight", W, 2 * W));
+    ck.add_f32("act.b_at1", {W}, im.vec("action_time_mlp_in.bias", W));
+    ck.add_f32("act.W_at2", {W, W}, im.mat("action_time_mlp_out.weight", W, W));
+    ck.add_f32("act.b_at2", {W}, im.vec("action_time_mlp_out.bias", W));
+    ck.add_f32("act.W_out", {ad, W}, im.mat("action_out_proj.weight", ad, W));
+    ck.add_f32("act.b_out", {ad}, im.vec("action_out_proj.bias", ad));
+    im.put_weight("act.norm", 1, W, im.vec("aex.output_norm.weight", W));
+    for (int64_t l = 0; l < L; ++l) {
+        const std::string a = "aex.blk." + std::to_string(l) + ".", v = "vlm.blk." + std::to_string(l) + ".";
+        const std::string e = "ex." + std::to_string(l) + ".", p = "vlm." + std::to_string(l) + ".";
+        const bool self = l % every == 0;
+        im.put_weight(e + "ln", 1, W, im.vec(a + "attn_norm.weight", W));
+        if (self) {
+            im.put_stacked(e + "Wqkv", {a + "attn_q.weight", a + "attn_k.weight", a + "attn_v.weight"}, {qd, kvd, kvd}, W);
+        } else {
+            // cross layers re-project the cached K and V: [kv_dim, kv_dim] (smolvla.cpp:1207-1208)
+            im.put_weight(e + "Wq", qd, W, im.mat(a + "attn_q.weight", qd, W));
+            im.put_weight(e + "Wk_x", kvd, kvd, im.mat(a + "attn_k.weight", kvd, kvd));
+            im.put_weight(e + "Wv_x", kvd, kvd, im.mat(a + "attn_v.weight", kvd, kvd));
+        }
+        im.put_weight(e + "Wo", W, qd, im.mat(a + "attn_o.weight", W, qd));
+        im.put_weight(e + "ln2", 1, W, im.vec(a + "ffn_norm.weight", W));
+        im.put_stacked(e + "Wgu", {a + "ffn_gate.weight", a + "ffn_up.weight"}, {I, I}, W);
+        im.put_weight(e + "Wd", W, I, im.mat(a + "ffn_down.weight", W, I));
+        im.put_weight(p + "ln", 1, hidden, im.vec(v + "attn_norm.weight", hidden));
+        im.put_stacked(p + "Wkv", {v + "attn_k.weight", v + "attn_v.weight"}, {kvd, kvd}, hidden);
+    }
+}
+
+// BitVLA language model: keys of load_config (src/models/bitvla.cpp:349-373), the ternary
+// projections of each block either as float tensors (quantised again at load, 430-451) or,
+// with bitvla.quant.int2_packed, as ladder-packed I8 tensors with a ".scale" sidecar
+// (728-747).  The action-token embeddings and the output projection this library's
+// token-by-token schedule uses have no counterpart in the reference's file; they are read
+// under this library's own names (act.emb, act.W_out, act.b_out) and must be present.
+void import_bitvla(gguf_reader& g, Checkpoint& ck) {
+    const int64_t H = need_u32(g, "bitvla.lm.hidden"), L = need_u32(g, "bitvla.lm.layers"), Hq = need_u32(g, "bitvla.lm.q_heads"),
+                  Hkv = need_u32(g, "bitvla.lm.kv_heads"), D = need_u32(g, "bitvla.lm.head_dim"),
+                  vocab = need_u32(g, "bitvla.lm.vocab_size");
+    if (Hkv < 1 || Hq % Hkv || Hq * D != H) throw std::runtime_error("vla: gguf lm q_heads x head_dim does not match hidden");
+    const bool packed = g.has("bitvla.quant.int2_packed") && g.u32("bitvla.quant.int2_packed") != 0;
+    const int64_t qd = Hq * D, kvd = Hkv * D;
+    const gguf_tensor_meta* emb = g.meta("act.emb");
+    const gguf_tensor_meta* wout = g.meta("act.W_out");
+    if (!emb || !wout) throw std::runtime_error("vla: bitvla gguf needs the act.emb / act.W_out / act.b_out tensors");
+    const int64_t n_act = emb->ne[1], A = wout->ne[1];
+    ck.set_key("arch", "bitvla");
+    ck.set_key("dtype", "bf16");
+    ck.set_key("n_layers", L);
+    ck.set_key("n_q_heads", Hq);
+    ck.set_key("n_kv_heads", Hkv);
+    ck.set_key("head_dim", D);
+    ck.set_key("hidden", H);
+    ck.set_key("n_img", (int64_t)(g.has("bitvla.vit.n_patches") ? g.u32("bitvla.vit.n_patches") : 256));
+    ck.set_key("n_lang", (int64_t)(g.has("bitvla.lm.max_text") ? g.u32("bitvla.lm.max_text") : 256));
+    ck.set_key("n_suffix", n_act);
+    ck.set_key("max_action_dim", A);
+    ck.set_key("real_action_dim", (int64_t)(g.has("bitvla.action.action_dim") ? g.u32("bitvla.action.action_dim") : A));
+    ck.set_key("rms_eps", (double)(g.has("bitvla.lm.rms_eps") ? g.f32("bitvla.lm.rms_eps") : 1e-5f));
+    ck.set_key("rope_freq_base", (double)(g.has("bitvla.lm.rope_theta") ? g.f32("bitvla.lm.rope_theta") : 500000.f));
+    ck.set_key("vocab", vocab);
+
+    Importer im{g, ck, false};
+    ck.add_f32("prefix.E_lang", {vocab, H}, im.mat("token_embd.weight", vocab, H));
+    ck.add_f32("act.emb", {n_act, H}, im.mat("act.emb", n_act, H));
+    ck.add_f32("act.W_out", {A, H}, im.mat("act.W_out", A, H));
+    ck.add_f32("act.b_out", {A}, im.vec("act.b_out", A));
+    ck.add_f32("act.norm", {H}, im.vec("lm.output_norm.weight", H));
+    for (int64_t l = 0; l < L; ++l) {
+        const std::string b = "lm.blk." + std::to_string(l) + ".", o = "lm." + std::to_string(l) + ".";
+        {
+            std::vector<float> n = im.vec(b + "attn_norm.weight", H), s = im.vec(b + "attn_sub_norm.weight", H);
+            std::vector<uint16_t> nh(H), sh(H);
+            for (int64_t i = 0; i < H; ++i) {
+                nh[i] = gguf_float_to_bf16(n[i]);
+                sh[i] = gguf_float_to_bf16(s[i]);
+            }
+            ck.add_tensor(o + "attn_norm", "bf16", {H}, nh.data(), nh.size() * 2);
+            ck.add_tensor(o + "sub_norm", "bf16", {H}, sh.data(), sh.size() * 2);
+        }
+        if (!packed) {
+            std::vector<float> all;
+            for (const auto& part : {std::make_pair("attn_q.weight", qd), std::make_pair("attn_k.weight", kvd), std::make_pair("attn_v.weight", kvd)}) {
+                const std::vector<float> p = im.mat(b + part.first, part.second, H);
+                all.insert(all.end(), p.begin(), p.end());
+            }
+            ck.add_f32(o + "Wqkv", {qd + 2 * kvd, H}, all);
+            ck.add_f32(o + "Wo", {H, qd}, im.mat(b + "attn_o.weight", H, qd));
+            continue;
+        }
+        // ladder-packed: each source tensor goes into the gfx950 word order on its own; that
+        // order is blocked by 32 output rows, so the fused tensor is the blocks back to back
+        if (qd % 32 || kvd % 32 || H % 128) throw std::runtime_error("vla: gguf int2 tensors need rows % 32 == 0 and K % 128 == 0");
+        std::vector<uint32_t> fused;
+        std::vector<float> ws;
+        for (const auto& part : {std::make_pair("attn_q", qd), std::make_pair("attn_k", kvd), std::make_pair("attn_v", kvd)}) {
+            const std::string name = b + part.first + ".weight";
+            std::vector<uint8_t> bytes = g.read_convert(name.c_str(), GGUF_T_I8);
+            if ((int64_t)bytes.size() != part.second * H / 4) throw std::runtime_error("vla: gguf int2 tensor " + name + " has the wrong size");
+            std::vector<uint32_t> words((size_t)vla_ternary_packed_words((int)part.second, (int)H));
+            if (vla_ternary_repack_ladder_host(bytes.data(), (int)part.second, (int)H, words.data()) != VLA_K_OK)
+                throw std::runtime_error("vla: cannot re-order gguf int2 tensor " + name);
+            fused.insert(fused.end(), words.begin(), words.end());
+            const std::vector<float> sc = g.read_f32((b + part.first + ".scale").c_str());
+            if (sc.empty()) throw std::runtime_error("vla: int2 tensor " + name + " has no .scale sidecar");
+            ws.push_back(sc[0]);
+        }
+        ck.add_tensor(o + "Wqkv.p2", "u8", {(int64_t)fused.size() * 4}, fused.data(), fused.size() * 4);
+        ck.add_f32(o + "Wqkv.ws", {3}, ws);
+        const std::string on = b + "attn_o.weight";
+        std::vector<uint8_t> ob = g.read_convert(on.c_str(), GGUF_T_I8);
+        if ((int64_t)ob.size() != H * qd / 4) throw std::runtime_error("vla: gguf int2 tensor " + on + " has the wrong size");
+        ck.add_tensor(o + "Wo.i2", "u8", {(int64_t)ob.size()}, ob.data(), ob.size());
+        const std::vector<float> osc = g.read_f32((b + "attn_o.scale").c_str());
+        if (osc.empty()) throw std::runtime_error("vla: int2 tensor " + on + " has no .scale sidecar");
+        ck.add_f32(o + "Wo.ws", {1}, {osc[0]});
+    }
+}
+
+}  // namespace
+
+// Weight type of the float architectures: bf16 unless VLA_WEIGHT_DTYPE=f32 (the reference's
+// default resident type is BF16 as well, src/models/smolvla.cpp:1965).
+Checkpoint import_gguf(const std::string& path) {
+    gguf_reader g("gguf");
+    if (!g.open(path)) throw std::runtime_error("vla: cannot read gguf " + path);
+    const char* wd = std::getenv("VLA_WEIGHT_DTYPE");
+    const bool bf16 = !(wd && std::string(wd) == "f32");
+    Checkpoint ck;
+    if (g.has("smolvla.architecture")) import_smolvla(g, ck, bf16);
+    else if (g.has("bitvla.architecture") || g.has("bitvla.lm.hidden")) import_bitvla(g, ck);
+    else throw std::runtime_error("vla: " + path + ": no importer for this gguf's architecture");
+    return ck;
+}
+
+}  // namespace vla
+
+// ---------------------------------------------------------------- C ABI over the reader
+struct vla_gguf {
+    vla::gguf_reader r{"gguf"};
+};
+
+extern "C" {
+
+vla_gguf* vla_gguf_open(const char* path) {
+    if (!path) return nullptr;
+    try {
+        std::unique_ptr<vla_gguf> g(new vla_gguf());
+        if (!g->r.open(path)) return nullptr;
+        return g.release();
+    } catch (...) {
+        return nullptr;
+    }
+}
+
+void vla_gguf_close(vla_gguf* g) { delete g; }
+
+int32_t vla_gguf_version(const vla_gguf* g) { return g ? (int32_t)g->r.version : 0; }
+int64_t vla_gguf_data_offset(const vla_gguf* g) { return g ? (int64_t)g->r.data_off : -1; }
+int32_t vla_gguf_has_key(const vla_gguf* g, const char* key) { return g && key && g->r.has(key) ? 1 : 0; }
+int32_t vla_gguf_key_type(const vla_gguf* g, const char* key) {
+    if (!g || !key) return -1;
+    auto it = g->r.kv.find(key);
+    return it == g->r.kv.end() ? -1 : (int32_t)it->second.type;
+}
+uint32_t vla_gguf_u32(const vla_gguf* g, const char* key) { return g && key ? g->r.u32(key) : 0u; }
+float vla_gguf_f32(const vla_gguf* g, const char* key) { return g && key ? g->r.f32(key) : 0.f; }
+double vla_gguf_f64(const vla_gguf* g, const char* key) { return g && key ? g->r.f64(key) : 0.0; }
+
+int64_t vla_gguf_str(const vla_gguf* g, const char* key, char* buf, int64_t cap) {
+    if (!g || !key) return -1;
+    const vla::gguf_kv* v = g->r.typed_key(key, vla::GGUF_KV_STRING);
+    if (!v) return -1;
+    if (buf && cap > 0) {
+        const size_t n = std::min((size_t)cap - 1, v->s.size());
+        std::memcpy(buf, v->s.data(), n);
+        buf[n] = 0;
+    }
+    return (int64_t)v->s.size();
+}
+
+int64_t vla_gguf_array_len(const vla_gguf* g, const char* key, int32_t* elem_type) {
+    if (!g || !key) return -1;
+    const vla::gguf_kv* v = g->r.typed_key(key, vla::GGUF_KV_ARRAY);
+    if (!v) return -1;
+    if (elem_type) *elem_type = (int32_t)v->elem_type;
+    return (int64_t)v->count;
+}
+
+int64_t vla_gguf_n_tensors(const vla_gguf* g) { return g ? (int64_t)g->r.tensors.size() : 0; }
+
+const char* vla_gguf_tensor_name(const vla_gguf* g, int64_t i) {
+    if (!g || i < 0 || i >= (int64_t)g->r.tensors.size()) return nullptr;
+    return g->r.tensors[(size_t)i].name.c_str();
+}
+
+int32_t vla_gguf_tensor_info(const vla_gguf* g, const char* name, int32_t* type, int32_t* n_dims, int64_t ne[4], int64_t* offset,
+                             int64_t* nbytes) {
+    if (!g || !name) return VLA_GGUF_ERR_ARG;
+    const vla::gguf_tensor_meta* t = g->r.meta(name);
+    if (!t) return VLA_GGUF_ERR_MISSING;
+    if (type) *type = (int32_t)t->type;
+    if (n_dims) *n_dims = t->n_dims;
+    if (ne)
+        for (int d = 0; d < 4; ++d) ne[d] = t->ne[d];
+    if (offset) *offset = (int64_t)t->offset;
+    if (nbytes) *nbytes = (int64_t)t->nbytes;
+    return VLA_GGUF_OK;
+}
+
+int32_t vla_gguf_read_raw(vla_gguf* g, const char* name, void* buf, int64_t cap) {
+    if (!g || !name || !buf || cap < 0) return VLA_GGUF_ERR_ARG;
+    if (!g->r.meta(name)) return VLA_GGUF_ERR_MISSING;
+    return g->r.read_raw(name, buf, (size_t)cap) ? VLA_GGUF_OK : VLA_GGUF_ERR_READ;
+}
+
+int32_t vla_gguf_read_f32(vla_gguf* g, const char* name, float* out, int64_t n) {
+    if (!g || !name || !out) return VLA_GGUF_ERR_ARG;
+    const vla::gguf_tensor_meta* t = g->r.meta(name);
+    if (!t) return VLA_GGUF_ERR_MISSING;
+    if (t->nelements() != n) return VLA_GGUF_ERR_ARG;
+    try {
+        const std::vector<float> v = g->r.read_f32(name);
+        if (v.empty()) return VLA_GGUF_ERR_READ;
+        std::memcpy(out, v.data(), v.size() * sizeof(float));
+        return VLA_GGUF_OK;
+    } catch (...) {
+        return VLA_GGUF_ERR_READ;
+    }
+}
+
+int32_t vla_gguf_read_convert(vla_gguf* g, const char* name, int32_t target_type, int32_t gemma_norm, void* out, int64_t cap) {
+    if (!g || !name || !out || cap < 0) return VLA_GGUF_ERR_ARG;
+    if (!g->r.meta(name)) return VLA_GGUF_ERR_MISSING;
+    try {
+        const std::vector<uint8_t> v = g->r.read_convert(name, (uint32_t)target_type, gemma_norm != 0);
+        if (v.empty()) return VLA_GGUF_ERR_READ;
+        if ((int64_t)v.size() != cap) return VLA_GGUF_ERR_ARG;
+        std::memcpy(out, v.data(), v.size());
+        return VLA_GGUF_OK;
+    } catch (...) {
+        return VLA_GGUF_ERR_READ;
+    }
+}
+
+int32_t vla_gguf_fetch_rows_f32(vla_gguf* g, const char* name, const int32_t* row_ids, int64_t n_rows, float* dst, int64_t cols) {
+    if (!g || !name || (!row_ids && n_rows > 0) || !dst || n_rows < 0 || cols <= 0) return VLA_GGUF_ERR_ARG;
+    if (!g->r.meta(name)) return VLA_GGUF_ERR_MISSING;
+    try {
+        const std::vector<int32_t> ids(row_ids, row_ids + n_rows);
+        return g->r.fetch_rows_f32(name, ids, dst, cols) ? VLA_GGUF_OK : VLA_GGUF_ERR_READ;
+    } catch (...) {
+        return VLA_GGUF_ERR_READ;
+    }
+}
+
+}  // extern "C"

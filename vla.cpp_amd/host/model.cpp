@@ -94,8 +94,10 @@ bool config_is_sane(const Config& c) {
            c.real_state_dim >= 0;
 }
 
+// ckpt_path: a GGUF written by the reference's converters (the tensors on the action-expert
+// path are taken from it, gguf_import.cpp) or this library's VLAW container.
 Model* model_load(const std::string&, const std::string& ckpt_path, const std::string&) {
-    Checkpoint ck(ckpt_path);
+    const Checkpoint ck = is_gguf_file(ckpt_path) ? import_gguf(ckpt_path) : Checkpoint(ckpt_path);
     const std::string arch = ck.str("arch");
     ModelArch* a = nullptr;
     if (arch == "smolvla" || arch == "pi0" || arch == "pi05" || arch == "gr00t_n1d5" || arch == "gr00t_n1d6") a = flow_expert_create(ck);
