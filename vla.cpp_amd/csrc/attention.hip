@@ -763,29 +763,27 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
     if (a.mask_kind == VLA_MASK_CAUSAL_SUFFIX) hi = min(a.n_keys, a.n_prefix + s + 1);
     else if (a.mask_kind == VLA_MASK_PI0_STATE && s == 0) hi = min(a.n_keys, a.n_prefix + 1);
     const int pad_lo = a.pad_start, pad_hi = min(a.pad_end, a.n_prefix);
-    // `live` = false: a phantom block past the slice (the pipeline is padded to whole groups
-    // of ST blocks); every key is hidden, so it leaves the state untouched.
-    auto compute = [&](int st, int kb, bool live) __attribute__((always_inline)) {
+    auto compute = [&](int st, int kb) __attribute__((always_inline)) {
         const int k0 = kb * 32;
         f32x16_t sc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) sc[i] = 0.f;
 #pragma unroll
         for (int c = 0; c < NQ; ++c) AT<bf16_t>::mma(sc, kr[st][c], qf[c]);
-        const bool blk_masked = !live || a.mask != nullptr || k0 + 32 > a.n_keys || (k0 < pad_hi && k0 + 32 > pad_lo) ||
+        const bool blk_masked = a.mask != nullptr || k0 + 32 > a.n_keys || (k0 < pad_hi && k0 + 32 > pad_lo) ||
                                 (a.mask_kind != VLA_MASK_NONE && k0 + 32 > a.n_prefix);
         float p[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) p[i] = sc[i] * c2;
         if (blk_masked) {
-            if (a.mask && live) {
+            if (a.mask) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int key = k0 + key_of_element(e, g);
                     p[e] = key < a.n_keys ? p[e] + a.mask[(long)s * a.n_keys + key] * LOG2E : -INFINITY;
                 }
             } else {
-                const int kl = k0 + 8 * g, hi_blk = live ? hi : 0;
+                const int kl = k0 + 8 * g, hi_blk = hi;
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int key = kl + key_of_element(e, 0);
@@ -835,33 +833,28 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
         }
     };
 
-    // Software pipeline over the slice's full blocks [kb0, kbf): ST - 1 blocks of loads
-    // stay in flight ahead of the block being multiplied.  The loop body is branch-free:
-    // the block count is padded to whole groups of ST, loads past the last full block
-    // re-read it, and the padded blocks are multiplied as phantoms.  A trailing partial
-    // block (only the slice that reaches n_keys has one) is loaded first, into the stage
-    // the pipeline needs last, and consumed while the first pipeline loads are in flight.
-    const bool has_partial = kb1 * 32 > a.n_keys;  // uniform
-    const int kbf = has_partial ? kb1 - 1 : kb1;
-    const int n_full = kbf - kb0;
-    if (has_partial) load_partial(ST - 1, kb1 - 1);
-    if (n_full > 0) {
+    // Software pipeline over the slice's blocks [kb0, kb1) in key order: ST - 1 blocks of
+    // loads stay in flight ahead of the block being multiplied.  Only the slice that reaches
+    // n_keys can end in a partial block; it takes the checked loads and, being last, shares
+    // its V^T cache lines with the full block fetched just before it.  The conditions in
+    // the loop are uniform over the wavefront (scalar branches).
+    const bool has_partial = kb1 * 32 > a.n_keys;
+    const int kbp = has_partial ? kb1 - 1 : -1;  // the partial block, if any
+    auto load_any = [&](int st, int kb) __attribute__((always_inline)) {
+        if (kb == kbp) load_partial(st, kb);
+        else if (kb < kb1) load_full(st, kb);
+    };
 #pragma unroll
-        for (int i = 0; i < ST - 1; ++i) load_full(i, min(kb0 + i, kbf - 1));
-    }
-    if (has_partial) {
-        mask_partial(ST - 1, kb1 - 1);
-        compute(ST - 1, kb1 - 1, true);
-    }
-    if (n_full > 0) {
-        const int groups = (n_full + ST - 1) / ST;
-        for (int gi = 0; gi < groups; ++gi) {
+    for (int i = 0; i < ST - 1; ++i) load_any(i, kb0 + i);
+    for (int base = kb0; base < kb1; base += ST) {
 #pragma unroll
-            for (int st = 0; st < ST; ++st) {
-                const int cur = kb0 + gi * ST + st;
-                load_full((st + ST - 1) % ST, min(cur + ST - 1, kbf - 1));
-                __builtin_amdgcn_sched_barrier(0);  // loads stay above the math they hide behind
-                compute(st, cur, cur < kbf);
+        for (int st = 0; st < ST; ++st) {
+            const int cur = base + st;
+            load_any((st + ST - 1) % ST, cur + ST - 1);
+            __builtin_amdgcn_sched_barrier(0);  // loads stay above the math they hide behind
+            if (cur < kb1) {
+                if (cur == kbp) mask_partial(st, cur);
+                compute(st, cur);
             }
         }
     }
