@@ -163,6 +163,27 @@ def test_smolvla_gguf_under_reference_names_equals_the_vlaw_checkpoint(tmp_path,
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("arch", ["pi0", "pi05"])
+def test_gemma_expert_gguf_equals_the_vlaw_checkpoint(tmp_path, arch):
+    """pi0 / pi0.5 files (src/models/pi0.cpp:427-437, src/models/pi05.cpp:459-485): norm weights
+    stored minus one, the adaRMS dense in the norm slots, the time MLP."""
+    from test_gpu_chunk import make_obs
+    cfg = ckpt.pi0_config(n_layers=3) if arch == "pi0" else ckpt.pi05_config(n_layers=3)
+    cfg.update(ffn_dim=512)
+    if arch == "pi0":
+        cfg.update(time_mlp=1)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 23)
+    r = np.random.default_rng(332)
+    obs = [make_obs(cfg, r, n_views=2, n_lang=29) for _ in range(2)]
+    pv, pg = os.path.join(str(tmp_path), "g.vlaw"), os.path.join(str(tmp_path), "g.gguf")
+    ckpt.write_synthetic(pv, cfg, w)
+    gguf.write_synthetic_gguf(pg, cfg, w)
+    want = _chunk(pv, obs, (2, 50, 32))
+    got = _chunk(pg, obs, (2, 50, 32))
+    assert np.array_equal(got, want) and np.abs(want).max() > 0.1
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("packed", [False, True])
 def test_bitvla_gguf_float_and_int2_packed_equal_the_vlaw_checkpoint(tmp_path, packed):
     from test_gpu_chunk import make_obs

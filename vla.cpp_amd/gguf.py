@@ -194,39 +194,61 @@ def _wt(cfg, a):
 
 def write_synthetic_gguf(path, cfg, w, ladder_pack=None):
     """The synthetic weights of checkpoint.synth_weights under the reference's GGUF names
-    and metadata keys: SmolVLA (src/models/smolvla.cpp:570-634, 648-755, 1099-1236; needs
-    cfg["ffn_dim"] and cfg["time_mlp"]) and the BitVLA language model
+    and metadata keys: SmolVLA (src/models/smolvla.cpp:570-634, 648-755, 1099-1236), pi0
+    (src/models/pi0.cpp:252-297, 427-437), pi0.5 (src/models/pi05.cpp:292-328, 459-485) --
+    these need cfg["ffn_dim"] and, except pi0.5, cfg["time_mlp"] -- and the BitVLA language model
     (src/models/bitvla.cpp:349-373, 640-700; ladder_pack(int8 [N, K]) -> bytes writes the
     int2-packed form with ".scale" sidecars, else float tensors the loader quantises)."""
     f32 = lambda a: (T_F32, np.ascontiguousarray(a, np.float32))
     L, Hq, Hkv, D = cfg["n_layers"], cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"]
     qd, kvd = Hq * D, Hkv * D
     kv, t = {}, {}
-    if cfg["arch"] == "smolvla":
-        I = cfg["ffn_dim"]
-        u = lambda k, v: kv.__setitem__("smolvla." + k, (U32, int(v)))
-        kv["smolvla.architecture"] = (STRING, "smolvla")
+    if cfg["arch"] in ("smolvla", "pi0", "pi05"):
+        arch = cfg["arch"]
+        smol, pi05 = arch == "smolvla", arch == "pi05"
+        I, W = cfg["ffn_dim"], cfg["expert_h"]
+        u = lambda k, v: kv.__setitem__(arch + "." + k, (U32, int(v)))
+        # Gemma norm weights are stored minus one (the loader adds it back); exact for the
+        # synthetic weights, which lie in [0.5, 2)
+        nrm = (lambda a: f32(a)) if smol else (lambda a: f32(np.asarray(a, np.float32) - np.float32(1)))
+        kv[arch + ".architecture"] = (STRING, arch)
+        chunk = cfg["n_suffix"] - (1 if arch == "pi0" else 0)
         for k, v in (("hidden", cfg["hidden"]), ("intermediate", 4 * cfg["hidden"]), ("n_q_heads", Hq), ("n_kv_heads", Hkv),
-                     ("head_dim", D), ("n_layers", L), ("vocab_size", cfg["vocab"]), ("expert_h", cfg["expert_h"]),
-                     ("expert_inter", I), ("chunk_size", cfg["n_suffix"]), ("num_steps", cfg["num_steps"]),
-                     ("max_state_dim", cfg["max_state_dim"]), ("max_action_dim", cfg["max_action_dim"]),
-                     ("real_state_dim", cfg["real_state_dim"]), ("real_action_dim", cfg["real_action_dim"]),
-                     ("self_attn_every_n_layers", cfg["self_attn_every_n"]), ("tokenizer_max_length", cfg["n_lang"]),
+                     ("head_dim", D), ("n_layers", L), ("expert_h", W), ("expert_inter", I), ("chunk_size", chunk),
+                     ("num_steps", cfg["num_steps"]), ("max_state_dim", cfg["max_state_dim"]),
+                     ("max_action_dim", cfg["max_action_dim"]), ("real_state_dim", cfg["real_state_dim"]),
+                     ("real_action_dim", cfg["real_action_dim"]), ("tokenizer_max_length", cfg["n_lang"]),
                      ("n_img_tokens", cfg["n_img"])):
             u(k, v)
-        kv["smolvla.min_period"] = (F64, float(cfg["min_period"]))
-        kv["smolvla.max_period"] = (F64, float(cfg["max_period"]))
+        if smol:
+            u("vocab_size", cfg["vocab"])
+            u("self_attn_every_n_layers", cfg["self_attn_every_n"])
+        kv[arch + ".min_period"] = (F64, float(cfg["min_period"]))
+        kv[arch + ".max_period"] = (F64, float(cfg["max_period"]))
         t["token_embd.weight"] = f32(w["prefix.E_lang"])
-        t["state_proj.weight"], t["state_proj.bias"] = f32(w["prefix.Wstate"]), f32(w["prefix.bstate"])
+        if smol:
+            t["state_proj.weight"], t["state_proj.bias"] = f32(w["prefix.Wstate"]), f32(w["prefix.bstate"])
+        elif not pi05:
+            t["state_proj.weight"], t["state_proj.bias"] = f32(w["act.W_sp"]), f32(w["act.b_sp"])
         t["action_in_proj.weight"], t["action_in_proj.bias"] = f32(w["act.W_in"]), f32(w["act.b_in"])
-        t["action_time_mlp_in.weight"], t["action_time_mlp_in.bias"] = f32(w["act.W_at1"]), f32(w["act.b_at1"])
-        t["action_time_mlp_out.weight"], t["action_time_mlp_out.bias"] = f32(w["act.W_at2"]), f32(w["act.b_at2"])
         t["action_out_proj.weight"], t["action_out_proj.bias"] = f32(w["act.W_out"]), f32(w["act.b_out"])
-        t["aex.output_norm.weight"] = f32(w["act.norm"])
+        if pi05:
+            t["time_mlp_in.weight"], t["time_mlp_in.bias"] = f32(w["te.W_tin"]), f32(w["te.b_tin"])
+            t["time_mlp_out.weight"], t["time_mlp_out.bias"] = f32(w["te.W_tout"]), f32(w["te.b_tout"])
+            t["aex.output_norm.weight"], t["aex.output_norm.bias"] = f32(w["act.ada_final_w"]), f32(w["act.ada_final_b"])
+        else:
+            t["action_time_mlp_in.weight"], t["action_time_mlp_in.bias"] = f32(w["act.W_at1"]), f32(w["act.b_at1"])
+            t["action_time_mlp_out.weight"], t["action_time_mlp_out.bias"] = f32(w["act.W_at2"]), f32(w["act.b_at2"])
+            t["aex.output_norm.weight"] = nrm(w["act.norm"])
+        every = cfg["self_attn_every_n"] if smol else 1
         for l in range(L):
             a, v, e, p = "aex.blk.%d." % l, "vlm.blk.%d." % l, "ex.%d." % l, "vlm.%d." % l
-            t[a + "attn_norm.weight"] = f32(w[e + "ln"])
-            if l % cfg["self_attn_every_n"] == 0:
+            if pi05:
+                t[a + "attn_norm.weight"], t[a + "attn_norm.bias"] = f32(w[e + "ada_in_w"]), f32(w[e + "ada_in_b"])
+                t[a + "ffn_norm.weight"], t[a + "ffn_norm.bias"] = f32(w[e + "ada_post_w"]), f32(w[e + "ada_post_b"])
+            else:
+                t[a + "attn_norm.weight"], t[a + "ffn_norm.weight"] = nrm(w[e + "ln"]), nrm(w[e + "ln2"])
+            if l % every == 0:
                 Wqkv = w[e + "Wqkv"]
                 t[a + "attn_q.weight"], t[a + "attn_k.weight"] = _wt(cfg, Wqkv[:qd]), _wt(cfg, Wqkv[qd:qd + kvd])
                 t[a + "attn_v.weight"] = _wt(cfg, Wqkv[qd + kvd:])
@@ -234,10 +256,9 @@ def write_synthetic_gguf(path, cfg, w, ladder_pack=None):
                 t[a + "attn_q.weight"], t[a + "attn_k.weight"] = _wt(cfg, w[e + "Wq"]), _wt(cfg, w[e + "Wk_x"])
                 t[a + "attn_v.weight"] = _wt(cfg, w[e + "Wv_x"])
             t[a + "attn_o.weight"] = _wt(cfg, w[e + "Wo"])
-            t[a + "ffn_norm.weight"] = f32(w[e + "ln2"])
             t[a + "ffn_gate.weight"], t[a + "ffn_up.weight"] = _wt(cfg, w[e + "Wgu"][:I]), _wt(cfg, w[e + "Wgu"][I:])
             t[a + "ffn_down.weight"] = _wt(cfg, w[e + "Wd"])
-            t[v + "attn_norm.weight"] = f32(w[p + "ln"])
+            t[v + "attn_norm.weight"] = nrm(w[p + "ln"])
             t[v + "attn_k.weight"], t[v + "attn_v.weight"] = _wt(cfg, w[p + "Wkv"][:kvd]), _wt(cfg, w[p + "Wkv"][kvd:])
             # tensors of the file that are not on the path; the importer must skip them
             t[v + "attn_q.weight"] = _wt(cfg, np.zeros((8, cfg["hidden"]), np.float32))

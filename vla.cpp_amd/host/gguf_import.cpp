@@ -2,7 +2,8 @@
 //
 // The reference's loaders read their tensors by the names its converters write
 // (SmolVLA: hf_to_gguf, src/models/smolvla.cpp:648-755 and the tensor list at 1099-1236;
-// BitVLA: src/models/bitvla.cpp:349-373, 640-700).  This file maps those names and metadata
+// pi0: src/models/pi0.cpp:427-437 with src/modules/gemma_expert.h:46-62; pi0.5:
+// src/models/pi05.cpp:459-485; BitVLA: src/models/bitvla.cpp:349-373, 640-700).  This file maps those names and metadata
 // keys onto the container's own names, fusing what the kernels want fused:
 //   [attn_q; attn_k; attn_v] rows -> Wqkv, [attn_k; attn_v] of a backbone layer -> Wkv,
 //   [ffn_gate; ffn_up] rows -> Wgu.
@@ -78,20 +79,36 @@ uint32_t need_u32(const gguf_reader& g, const char* k) {
     return g.u32(k);
 }
 
-// SmolVLA: keys of load_config_from_gguf (src/models/smolvla.cpp:570-634), tensors of
-// smolvla_create (1099-1236) under their GGUF names (648-755).
-void import_smolvla(gguf_reader& g, Checkpoint& ck, bool bf16) {
-    if (g.str("smolvla.architecture") != "smolvla") throw std::runtime_error("vla: gguf architecture is not 'smolvla'");
-    const int64_t hidden = need_u32(g, "smolvla.hidden"), Hq = need_u32(g, "smolvla.n_q_heads"), Hkv = need_u32(g, "smolvla.n_kv_heads"),
-                  D = need_u32(g, "smolvla.head_dim"), L = need_u32(g, "smolvla.n_layers"), vocab = need_u32(g, "smolvla.vocab_size"),
-                  W = need_u32(g, "smolvla.expert_h"), I = need_u32(g, "smolvla.expert_inter"), S = need_u32(g, "smolvla.chunk_size"),
-                  steps = need_u32(g, "smolvla.num_steps"), sd = need_u32(g, "smolvla.max_state_dim"),
-                  ad = need_u32(g, "smolvla.max_action_dim"), every = need_u32(g, "smolvla.self_attn_every_n_layers"),
-                  n_lang = need_u32(g, "smolvla.tokenizer_max_length");
-    if (!g.has("smolvla.min_period") || !g.has("smolvla.max_period")) throw std::runtime_error("vla: gguf missing key 'smolvla.min_period/max_period'");
+// SmolVLA, pi0 and pi0.5 share one layout: metadata under "<arch>.", backbone layers
+// "vlm.blk.N.", expert layers "aex.blk.N.", the action projections at the top level.
+//   SmolVLA: keys of load_config_from_gguf (src/models/smolvla.cpp:570-634), tensors of
+//            smolvla_create (1099-1236) under their GGUF names (648-755); cross layers every
+//            self_attn_every_n_layers re-project the cached K / V ([kv_dim, kv_dim]).
+//   pi0:     keys src/models/pi0.cpp:252-297, tensors 427-437 and GemmaExpert::declare
+//            (src/modules/gemma_expert.h:46-62); Gemma norm weights are stored minus one
+//            (f32_gemma_norm adds it back, src/gguf_reader.h:151-181).
+//   pi0.5:   keys src/models/pi05.cpp:292-328, tensors 459-485: the expert's norm slots hold
+//            the adaRMS modulation dense ([3 expert_h, expert_h] weight and [3 expert_h]
+//            bias), the time MLP replaces the action-time MLP, there is no state projection.
+void import_flow(gguf_reader& g, Checkpoint& ck, bool bf16, const std::string& arch) {
+    const bool smol = arch == "smolvla", pi05 = arch == "pi05", gemma = !smol;
+    const std::string kp = arch + ".";
+    auto key = [&](const char* k) { return kp + k; };
+    auto u = [&](const char* k) { return (int64_t)need_u32(g, key(k).c_str()); };
+    if (g.str(key("architecture").c_str()) != arch) throw std::runtime_error("vla: gguf architecture is not '" + arch + "'");
+    const int64_t hidden = u("hidden"), Hq = u("n_q_heads"), Hkv = u("n_kv_heads"), D = u("head_dim"), L = u("n_layers"),
+                  W = u("expert_h"), I = u("expert_inter"), S = u("chunk_size"), steps = u("num_steps"), sd = u("max_state_dim"),
+                  ad = u("max_action_dim"), n_lang = u("tokenizer_max_length");
+    const int64_t every = smol ? u("self_attn_every_n_layers") : 1;
+    if (!g.has(key("min_period").c_str()) || !g.has(key("max_period").c_str()))
+        throw std::runtime_error("vla: gguf missing key '" + kp + "min_period/max_period'");
     if (every < 1 || L < 1 || Hkv < 1 || Hq % Hkv) throw std::runtime_error("vla: gguf geometry is not usable");
+    const gguf_tensor_meta* emb = g.meta("token_embd.weight");
+    if (!emb || emb->ne[0] != hidden) throw std::runtime_error("vla: gguf token_embd.weight is missing or has the wrong width");
+    const int64_t vocab = smol ? u("vocab_size") : emb->ne[1];
     const int64_t qd = Hq * D, kvd = Hkv * D;
-    ck.set_key("arch", "smolvla");
+    auto f32_or = [&](const char* k, double dflt) { return g.has(key(k).c_str()) ? (double)g.f32(key(k).c_str()) : dflt; };
+    ck.set_key("arch", arch);
     ck.set_key("dtype", bf16 ? "bf16" : "f32");
     ck.set_key("n_layers", L);
     ck.set_key("n_q_heads", Hq);
@@ -100,39 +117,67 @@ void import_smolvla(gguf_reader& g, Checkpoint& ck, bool bf16) {
     ck.set_key("hidden", hidden);
     ck.set_key("expert_h", W);
     ck.set_key("ffn_dim", I);
-    ck.set_key("n_img", (int64_t)(g.has("smolvla.n_img_tokens") ? g.u32("smolvla.n_img_tokens") : 64));
+    ck.set_key("n_img", (int64_t)(g.has(key("n_img_tokens").c_str()) ? g.u32(key("n_img_tokens").c_str()) : (smol ? 64 : 256)));
     ck.set_key("n_lang", n_lang);
-    ck.set_key("n_suffix", S);
+    ck.set_key("n_suffix", smol || pi05 ? S : S + 1);  // pi0: the state token leads the action chunk (pi0.cpp:526-528)
     ck.set_key("max_action_dim", ad);
     ck.set_key("max_state_dim", sd);
-    ck.set_key("real_action_dim", (int64_t)need_u32(g, "smolvla.real_action_dim"));
-    ck.set_key("real_state_dim", (int64_t)need_u32(g, "smolvla.real_state_dim"));
+    ck.set_key("real_action_dim", u("real_action_dim"));
+    ck.set_key("real_state_dim", u("real_state_dim"));
     ck.set_key("num_steps", steps);
-    ck.set_key("rms_eps", 1e-5);                // fixed by the loader, smolvla.cpp:623-625
-    ck.set_key("rope_freq_base", 10000.0);
+    ck.set_key("rms_eps", smol ? 1e-5 : f32_or("rms_norm_eps", 1e-6));  // smolvla.cpp:623-625, pi0.cpp:290
+    ck.set_key("rope_freq_base", gemma && g.has(key("rope_theta").c_str()) ? g.f64(key("rope_theta").c_str()) : 10000.0);
     ck.set_key("self_attn_every_n", every);
-    ck.set_key("min_period", g.f64("smolvla.min_period"));
-    ck.set_key("max_period", g.f64("smolvla.max_period"));
+    ck.set_key("min_period", g.f64(key("min_period").c_str()));
+    ck.set_key("max_period", g.f64(key("max_period").c_str()));
     ck.set_key("vocab", vocab);
 
     Importer im{g, ck, bf16};
+    auto norm = [&](const std::string& name, int64_t n) {  // Gemma stores norm weights minus one
+        std::vector<float> v = im.vec(name, n);
+        if (gemma)
+            for (float& x : v) x += 1.0f;
+        return v;
+    };
     ck.add_f32("prefix.E_lang", {vocab, hidden}, im.mat("token_embd.weight", vocab, hidden));
-    ck.add_f32("prefix.Wstate", {hidden, sd}, im.mat("state_proj.weight", hidden, sd));
-    ck.add_f32("prefix.bstate", {hidden}, im.vec("state_proj.bias", hidden));
+    if (smol) {
+        ck.add_f32("prefix.Wstate", {hidden, sd}, im.mat("state_proj.weight", hidden, sd));
+        ck.add_f32("prefix.bstate", {hidden}, im.vec("state_proj.bias", hidden));
+    } else if (!pi05) {
+        ck.add_f32("act.W_sp", {W, sd}, im.mat("state_proj.weight", W, sd));
+        ck.add_f32("act.b_sp", {W}, im.vec("state_proj.bias", W));
+    }
     ck.add_f32("act.W_in", {W, ad}, im.mat("action_in_proj.weight", W, ad));
     ck.add_f32("act.b_in", {W}, im.vec("action_in_proj.bias", W));
-    ck.add_f32("act.W_at1", {W, 2 * W}, im.mat("action_time_mlp_in.weight", W, 2 * W));
-    ck.add_f32("act.b_at1", {W}, im.vec("action_time_mlp_in.bias", W));
-    ck.add_f32("act.W_at2", {W, W}, im.mat("action_time_mlp_out.weight", W, W));
-    ck.add_f32("act.b_at2", {W}, im.vec("action_time_mlp_out.bias", W));
     ck.add_f32("act.W_out", {ad, W}, im.mat("action_out_proj.weight", ad, W));
     ck.add_f32("act.b_out", {ad}, im.vec("action_out_proj.bias", ad));
-    im.put_weight("act.norm", 1, W, im.vec("aex.output_norm.weight", W));
+    if (pi05) {
+        ck.add_f32("te.W_tin", {W, W}, im.mat("time_mlp_in.weight", W, W));
+        ck.add_f32("te.b_tin", {W}, im.vec("time_mlp_in.bias", W));
+        ck.add_f32("te.W_tout", {W, W}, im.mat("time_mlp_out.weight", W, W));
+        ck.add_f32("te.b_tout", {W}, im.vec("time_mlp_out.bias", W));
+        ck.add_f32("act.ada_final_w", {3 * W, W}, im.mat("aex.output_norm.weight", 3 * W, W));
+        ck.add_f32("act.ada_final_b", {3 * W}, im.vec("aex.output_norm.bias", 3 * W));
+    } else {
+        ck.add_f32("act.W_at1", {W, 2 * W}, im.mat("action_time_mlp_in.weight", W, 2 * W));
+        ck.add_f32("act.b_at1", {W}, im.vec("action_time_mlp_in.bias", W));
+        ck.add_f32("act.W_at2", {W, W}, im.mat("action_time_mlp_out.weight", W, W));
+        ck.add_f32("act.b_at2", {W}, im.vec("action_time_mlp_out.bias", W));
+        im.put_weight("act.norm", 1, W, norm("aex.output_norm.weight", W));
+    }
     for (int64_t l = 0; l < L; ++l) {
         const std::string a = "aex.blk." + std::to_string(l) + ".", v = "vlm.blk." + std::to_string(l) + ".";
         const std::string e = "ex." + std::to_string(l) + ".", p = "vlm." + std::to_string(l) + ".";
         const bool self = l % every == 0;
-        im.put_weight(e + "ln", 1, W, im.vec(a + "attn_norm.weight", W));
+        if (pi05) {
+            ck.add_f32(e + "ada_in_w", {3 * W, W}, im.mat(a + "attn_norm.weight", 3 * W, W));
+            ck.add_f32(e + "ada_in_b", {3 * W}, im.vec(a + "attn_norm.bias", 3 * W));
+            ck.add_f32(e + "ada_post_w", {3 * W, W}, im.mat(a + "ffn_norm.weight", 3 * W, W));
+            ck.add_f32(e + "ada_post_b", {3 * W}, im.vec(a + "ffn_norm.bias", 3 * W));
+        } else {
+            im.put_weight(e + "ln", 1, W, norm(a + "attn_norm.weight", W));
+            im.put_weight(e + "ln2", 1, W, norm(a + "ffn_norm.weight", W));
+        }
         if (self) {
             im.put_stacked(e + "Wqkv", {a + "attn_q.weight", a + "attn_k.weight", a + "attn_v.weight"}, {qd, kvd, kvd}, W);
         } else {
@@ -142,10 +187,9 @@ void import_smolvla(gguf_reader& g, Checkpoint& ck, bool bf16) {
             im.put_weight(e + "Wv_x", kvd, kvd, im.mat(a + "attn_v.weight", kvd, kvd));
         }
         im.put_weight(e + "Wo", W, qd, im.mat(a + "attn_o.weight", W, qd));
-        im.put_weight(e + "ln2", 1, W, im.vec(a + "ffn_norm.weight", W));
         im.put_stacked(e + "Wgu", {a + "ffn_gate.weight", a + "ffn_up.weight"}, {I, I}, W);
         im.put_weight(e + "Wd", W, I, im.mat(a + "ffn_down.weight", W, I));
-        im.put_weight(p + "ln", 1, hidden, im.vec(v + "attn_norm.weight", hidden));
+        im.put_weight(p + "ln", 1, hidden, norm(v + "attn_norm.weight", hidden));
         im.put_stacked(p + "Wkv", {v + "attn_k.weight", v + "attn_v.weight"}, {kvd, kvd}, hidden);
     }
 }
@@ -250,7 +294,9 @@ Checkpoint import_gguf(const std::string& path) {
     const char* wd = std::getenv("VLA_WEIGHT_DTYPE");
     const bool bf16 = !(wd && std::string(wd) == "f32");
     Checkpoint ck;
-    if (g.has("smolvla.architecture")) import_smolvla(g, ck, bf16);
+    if (g.has("smolvla.architecture")) import_flow(g, ck, bf16, "smolvla");
+    else if (g.has("pi05.architecture")) import_flow(g, ck, bf16, "pi05");
+    else if (g.has("pi0.architecture")) import_flow(g, ck, bf16, "pi0");
     else if (g.has("bitvla.architecture") || g.has("bitvla.lm.hidden")) import_bitvla(g, ck);
     else throw std::runtime_error("vla: " + path + ": no importer for this gguf's architecture");
     return ck;
