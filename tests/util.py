@@ -42,4 +42,4 @@ def rel_err(got, want):
 def declared_symbols(header):
     text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(?:VLA_KAPI|VLA_API|VLA_GGUF_API)\s+[\w\s\*]+?\b(\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(?:VLA_KAPI|VLA_API|VLA_GGUF_API|VLA_SERVE_API)\s+[\w\s\*]+?\b(\w+)\s*\(", text)))

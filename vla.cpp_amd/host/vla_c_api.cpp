@@ -5,6 +5,7 @@
 // callers may free() them).
 
 #include "vla.h"
+#include "vla_serve.h"
 
 #include <cstdio>
 #include <cstdlib>
@@ -201,6 +202,11 @@ int32_t vla_predict_batch(vla_model* h, const vla_inputs* in, int32_t batch, flo
     rc = vla_denoise_async(h, 1, nullptr);
     if (rc != VLA_OK) return rc;
     return vla_fetch_actions(h, out_actions, out_n);
+}
+
+int64_t vla_model_n_actions(const vla_model* h) {
+    if (!h || !h->m) return 0;
+    return h->m->arch->n_actions();
 }
 
 }  // extern "C"
