@@ -6,9 +6,9 @@
  * the reference's bindings/python/vla_cpp/_ffi.py:124-163 binds these) and the
  * same seven entry points, so a program linked against the reference's libvla
  * can be pointed at this library.  Behaviour behind the ABI: the handle drives
- * the MI355X action-expert attention path on one GPU; checkpoints are the flat
- * "VLAW" files written by vla.cpp_amd/checkpoint.py (a GGUF reader is outside
- * this library's scope).
+ * the MI355X action-expert attention path on one GPU; checkpoints are the
+ * reference's GGUF files (the tensors on the path are taken from them) or the
+ * flat "VLAW" files written by vla.cpp_amd/checkpoint.py.
  *
  * Ownership rules are the reference's: load pairs with free, predict pairs with
  * vla_free_actions, every pointer inside vla_inputs is only borrowed for the
@@ -29,102 +29,60 @@ extern "C" {
 
 typedef struct vla_model vla_model;
 
-typedef enum {
-    VLA_OK = 0,
-    VLA_ERR_ARG = -1,       /* null handle / malformed inputs */
-    VLA_ERR_PREDICT = -2,   /* the engine produced no actions */
-    VLA_ERR_EXCEPTION = -3, /* a C++ exception stopped at the boundary */
-} vla_status;
+/* Status codes, pixel formats and timing detail: the reference's values (include/vla.h:41-57). */
+typedef enum { VLA_OK = 0, VLA_ERR_ARG = -1, VLA_ERR_PREDICT = -2, VLA_ERR_EXCEPTION = -3 } vla_status;
+/* VLA_ERR_ARG: null handle or malformed inputs; VLA_ERR_PREDICT: the engine produced no actions;
+ * VLA_ERR_EXCEPTION: a C++ exception stopped at the boundary. */
+typedef enum { VLA_PIXEL_U8 = 0, VLA_PIXEL_F32_RGB_01 = 1 } vla_pixel_format;
+typedef enum { VLA_TIMING_NONE = 0, VLA_TIMING_PHASE = 1 } vla_timing_detail;
 
-typedef enum {
-    VLA_PIXEL_U8 = 0,
-    VLA_PIXEL_F32_RGB_01 = 1,
-} vla_pixel_format;
-
-typedef enum {
-    VLA_TIMING_NONE = 0,
-    VLA_TIMING_PHASE = 1,
-} vla_timing_detail;
-
-/* Resolved hyper-parameters (reference: vla::Config, src/model.h:48-87). */
+/* Resolved hyper-parameters (reference: vla::Config, src/model.h:48-87).  Field order and
+ * types are the ABI; fields of one type that follow each other share a declaration. */
 typedef struct {
-    int64_t n_img;
-    int64_t n_lang;
-    int64_t n_state;
-    int64_t n_prefix;
-    int64_t n_suffix;
-    int64_t n_full;
-
-    int64_t hidden;
-    int64_t expert_h;
-    int64_t intermediate;
-    int64_t expert_inter;
-    int64_t n_q_heads;
-    int64_t n_kv_heads;
-    int64_t head_dim;
-    int64_t q_full_dim;
-    int64_t kv_full_dim;
-    int64_t n_layers;
+    int64_t n_img, n_lang, n_state, n_prefix, n_suffix, n_full;                 /* token counts */
+    int64_t hidden, expert_h, intermediate, expert_inter;                        /* widths */
+    int64_t n_q_heads, n_kv_heads, head_dim, q_full_dim, kv_full_dim, n_layers;  /* attention geometry */
     int32_t self_attn_every_n;
-
-    int64_t max_state_dim;
-    int64_t max_action_dim;
-    int64_t real_state_dim;
-    int64_t real_action_dim;
-    float   norm_eps;
-    double  min_period;
-    double  max_period;
+    int64_t max_state_dim, max_action_dim, real_state_dim, real_action_dim;
+    float norm_eps;
+    double min_period, max_period; /* sinusoidal time embedding */
     int32_t num_steps;
-
-    float   rms_eps;
-    int32_t rope_n_dims;
-    int32_t rope_mode;
-    float   rope_freq_base;
-
+    float rms_eps;
+    int32_t rope_n_dims, rope_mode;
+    float rope_freq_base;
     int32_t denormalized;
 } vla_config;
 
 typedef struct {
-    const void * data;
-    int32_t      w;
-    int32_t      h;
-    int32_t      format;
+    const void* data;
+    int32_t w, h, format; /* format: vla_pixel_format */
 } vla_image;
 
 /* One observation.  This library has no vision tower: precomputed_img_emb
  * ([n_img_views * n_img, hidden] floats) is required and `images` is ignored. */
 typedef struct {
-    const vla_image * images;
-    int32_t           n_images;
-
-    const float *     precomputed_img_emb;
-    int32_t           n_img_views;
-
-    const int32_t *   lang_tokens;
-    int32_t           n_lang;
-
-    const float *     state; /* max_state_dim floats, or NULL for zeros */
-    const float *     noise; /* n_suffix * max_action_dim floats, or NULL to sample */
-
-    const int32_t *   attention_mask;
-    int32_t           attention_mask_n;
-
-    int32_t           timing_detail;
+    const vla_image* images;
+    int32_t n_images;
+    const float* precomputed_img_emb;
+    int32_t n_img_views;
+    const int32_t* lang_tokens;
+    int32_t n_lang;
+    const float* state; /* max_state_dim floats, or NULL for zeros */
+    const float* noise; /* n_actions * max_action_dim floats, or NULL to sample */
+    const int32_t* attention_mask;
+    int32_t attention_mask_n;
+    int32_t timing_detail; /* vla_timing_detail */
 } vla_inputs;
 
-/* Milliseconds; phase fields stay zero unless VLA_TIMING_PHASE was asked for. */
+/* Milliseconds; the phase fields stay zero unless VLA_TIMING_PHASE was asked for. */
 typedef struct {
-    float ms_total;
-    float ms_vision;
-    float ms_inference;
-    float ms_prefill;
-    float ms_denoise;
+    float ms_total, ms_vision, ms_inference, ms_prefill, ms_denoise;
 } vla_stats;
 
 VLA_API int32_t vla_abi_version(void);
 
-/* mmproj_path and config_path are accepted and ignored; ckpt_path names a VLAW
- * file.  NULL on any failure. */
+/* mmproj_path and config_path are accepted and ignored; ckpt_path names a GGUF
+ * or VLAW file.  NULL on any failure. */
 VLA_API vla_model * vla_model_load(const char * mmproj_path, const char * ckpt_path, const char * config_path);
 
 VLA_API void vla_model_free(vla_model * m);
