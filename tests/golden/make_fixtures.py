@@ -54,6 +54,20 @@ def build():
     h = r.standard_normal((6, 96)).astype(np.float32)
     w = (1 + 0.1 * r.standard_normal(96)).astype(np.float32)
     out.update(norm_x=h, norm_w=w, norm_out=orc.rms_norm(h, w, 1e-5))
+    # --- the widened layer pieces: gated FFN (silu and gelu), biased GELU FFN, adaRMS, gated residual
+    r = np.random.default_rng(0xFF4)
+    x = r.standard_normal((6, 96)).astype(np.float32)
+    Wg, Wu = (0.1 * r.standard_normal((128, 96))).astype(np.float32), (0.1 * r.standard_normal((128, 96))).astype(np.float32)
+    Wd = (0.1 * r.standard_normal((96, 128))).astype(np.float32)
+    b1, b2 = (0.1 * r.standard_normal(128)).astype(np.float32), (0.1 * r.standard_normal(96)).astype(np.float32)
+    sc, sh = (0.2 * r.standard_normal(96)).astype(np.float32), (0.2 * r.standard_normal(96)).astype(np.float32)
+    gate = (1 + 0.2 * r.standard_normal(96)).astype(np.float32)
+    Wo = (0.1 * r.standard_normal((96, 96))).astype(np.float32)
+    out.update(ffn_x=x, ffn_wg=Wg, ffn_wu=Wu, ffn_wd=Wd, ffn_b1=b1, ffn_b2=b2,
+               ffn_glu_silu=orc.ffn_glu(x, Wg, Wu, Wd, orc.silu), ffn_glu_gelu=orc.ffn_glu(x, Wg, Wu, Wd, orc.gelu),
+               ffn_gelu=orc.ffn_gelu(x, Wg, b1, Wd, b2),
+               ada_scale=sc, ada_shift=sh, ada_out=orc.adarms(x, sc, sh, 1e-6),
+               gated_w=Wo, gated_gate=gate, gated_out=(x + orc.linear(x, Wo) * gate).astype(np.float32))
     return out
 
 

@@ -122,3 +122,26 @@ def test_hip_path_against_committed_fixtures():
     pkg.call("vla_rms_norm", dev(fx["norm_x"]), dev(fx["norm_w"]), y, F32, Mn, Kn, 1e-5)
     torch.cuda.synchronize()
     assert rel_err(host(y), fx["norm_out"]) < 1e-6
+    # the widened layer pieces: gated FFN through the GLU epilogue, biased GELU FFN, adaRMS, gated residual
+    x, Wg, Wu, Wd = fx["ffn_x"], fx["ffn_wg"], fx["ffn_wu"], fx["ffn_wd"]
+    M, K = x.shape
+    I = Wg.shape[0]
+    Wgu = dev(np.concatenate([Wg, Wu], 0))
+    for act, want in ((pkg.VLA_ACT_SILU, fx["ffn_glu_silu"]), (pkg.VLA_ACT_GELU, fx["ffn_glu_gelu"])):
+        mid = torch.zeros((M, I), device="cuda")
+        y = torch.zeros((M, K), device="cuda")
+        pkg.call("vla_glu_linear", dev(x), Wgu, None, mid, F32, F32, M, I, K, act, -1.0)
+        pkg.call("vla_linear", mid, dev(Wd), None, None, y, F32, F32, M, K, I)
+        torch.cuda.synchronize()
+        assert rel_err(host(y), want) < 1e-5
+    mid = torch.zeros((M, I), device="cuda")
+    y = torch.zeros((M, K), device="cuda")
+    pkg.call("vla_linear_act", dev(x), dev(Wg), dev(fx["ffn_b1"]), None, mid, F32, F32, M, I, K, pkg.VLA_ACT_GELU)
+    pkg.call("vla_linear", mid, dev(Wd), dev(fx["ffn_b2"]), None, y, F32, F32, M, K, I)
+    ya = torch.zeros((M, K), device="cuda")
+    pkg.call("vla_adarms", dev(x), dev(fx["ada_scale"]), dev(fx["ada_shift"]), ya, F32, M, K, 1e-6)
+    yg = torch.zeros((M, K), device="cuda")
+    pkg.call("vla_linear_gated", dev(x), dev(fx["gated_w"]), None, dev(fx["gated_gate"]), dev(x), yg, F32, F32, M, K, K)
+    torch.cuda.synchronize()
+    assert rel_err(host(y), fx["ffn_gelu"]) < 1e-5 and rel_err(host(ya), fx["ada_out"]) < 1e-6
+    assert rel_err(host(yg), fx["gated_out"]) < 1e-5
