@@ -491,6 +491,38 @@ def test_attention_direct_kernel_key_slices_merge(monkeypatch, split):
     assert np.isfinite(got).all() and bf16_close(got, want) and rel_err(got, want) < 1e-2
 
 
+@pytest.mark.parametrize("B", [1, 4])
+def test_attention_wide_heads_key_slices_and_partial_formats(monkeypatch, B):
+    # pi0's 256-wide MQA heads: with few workgroups the keys are walked in slices whose partial
+    # outputs travel as fp16 (normalised per slice) to a merge launch.  Unsliced, fp32 partials
+    # and fp16 partials all meet the oracle; the fp16 partials cost less than the output rounding.
+    r = np.random.default_rng(130 + B)
+    S, Hq, Hkv, D, P = 51, 8, 1, 256, 816
+    T, t_max = P + S, 896
+    Q = orc.round_bf16(r.standard_normal((B, S, Hq, D)).astype(np.float32))
+    K = orc.round_bf16(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    V = orc.round_bf16(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    kc = torch.full((B, Hkv, t_max, D), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
+    vc = torch.full((B, Hkv, D, t_max), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
+    pkg.call("vla_kv_append", kc, vc, to_dev(K, BF16), to_dev(V, BF16), BF16, B, Hkv, D, t_max, 0, T)
+    mask = orc.mask_pi0_full(P, S)
+    want = np.stack([orc.attention(Q[b], K[b], V[b], mask, 1.0 / 16) for b in range(B)])
+    got = {}
+    for name, env in (("sliced-fp16", {}), ("sliced-fp32", {"VLA_ATTN_PART_F32": "1"}), ("unsliced", {"VLA_ATTN_SPLIT": "1"})):
+        for k in ("VLA_ATTN_PART_F32", "VLA_ATTN_SPLIT"):
+            monkeypatch.delenv(k, raising=False)
+        for k, v in env.items():
+            monkeypatch.setenv(k, v)
+        out = empty((B, S, Hq * D), BF16)
+        pkg.call("vla_attn_prefix_suffix", to_dev(Q, BF16), kc, vc, out, BF16, B, S, Hq, Hkv, D, t_max, T, 1.0 / 16,
+                 pkg.VLA_MASK_PI0_STATE, P, 0, 0, None)
+        sync()
+        got[name] = as_f32(out, BF16)
+        assert np.isfinite(got[name]).all() and bf16_close(got[name], want) and rel_err(got[name], want) < 1e-2, name
+    assert rel_err(got["sliced-fp16"], want) <= rel_err(got["unsliced"], want) * 1.25 + 1e-4
+    assert rel_err(got["sliced-fp16"], got["sliced-fp32"]) < 1e-2
+
+
 def test_attention_special_cases_fp32():
     # all-zero Q -> mean of the visible V rows; permuting keys changes nothing
     r = np.random.default_rng(107)

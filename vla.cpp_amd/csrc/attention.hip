@@ -62,8 +62,9 @@ struct AttnArgs {
     int n_groups, n_split, tiles_per_split, r_pad, p2;
     int n_rblocks;  // direct kernel: 32-row blocks per (batch, kv head)
     int n_slices;   // LDS kernel, direct-to-LDS variant: key slices (wavefronts) per row tile
-    float* part_o;   // [pair][split][r_pad][D]
+    float* part_o;   // [pair][split][r_pad][D] fp32 unnormalised, or fp16 normalised (part_half)
     float* part_ml;  // [pair][split][r_pad][2]
+    int part_half;   // partial outputs stored as o / l in fp16 (half the bytes; wide heads)
 };
 
 // Key (within a 32-key block) held by score row x = 8j + 4h + i: 16(j/2) + 8h + 4(j%2) + i.
@@ -72,6 +73,43 @@ __device__ __forceinline__ int key_of_score_row(int x) {
 }
 // Key of accumulator element e (= 4j + i) of a lane in half g.
 __device__ __forceinline__ int key_of_element(int e, int g) { return 16 * (e >> 3) + 8 * g + 4 * ((e >> 2) & 1) + (e & 3); }
+
+// One output row from its key slices' partials, by one wavefront: the slices' (max, sum) pairs
+// are read by every lane (one address per slice: a broadcast), the weights 2^(m_slice - m) are
+// formed once, and each lane combines four consecutive elements per 256-element stretch.
+// prow0 = the row's index in slice 0; slice sp lies sp * r_pad rows further.  HALF: the
+// partial outputs are fp16 and normalised by their slice's sum.
+template <typename T, bool HALF>
+__device__ __forceinline__ void merge_row(const float* __restrict__ part_o, const float* __restrict__ part_ml, T* __restrict__ orow,
+                                          long prow0, int n_split, int r_pad, int D, int lane) {
+    float m = -INFINITY;
+    for (int sp = 0; sp < n_split; ++sp) m = fmaxf(m, part_ml[(prow0 + (long)sp * r_pad) * 2]);
+    for (int d0 = lane * 4; d0 < D; d0 += 256) {
+        float l = 0.f;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        if (m > -INFINITY) {
+            for (int sp = 0; sp < n_split; ++sp) {
+                const long prow = prow0 + (long)sp * r_pad;
+                const float w = exp2f(part_ml[prow * 2] - m);
+                if (HALF) {
+                    typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+                    const float wl = part_ml[prow * 2 + 1] * w;
+                    l += wl;
+                    const h4_t po = *reinterpret_cast<const h4_t*>(reinterpret_cast<const _Float16*>(part_o) + prow * D + d0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] += (float)po[e] * wl;
+                } else {
+                    l += part_ml[prow * 2 + 1] * w;
+                    const f32x4_t po = *reinterpret_cast<const f32x4_t*>(part_o + prow * D + d0);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[e] += po[e] * w;
+                }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) Elem<T>::store(orow + d0 + e, l > 0.f ? acc[e] / l : 0.f);
+    }
+}
 
 template <typename T> struct AT;
 template <> struct AT<bf16_t> {
@@ -563,17 +601,18 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
                     __syncthreads();
                 }
             }
-            return;
-        }
-        __syncthreads();
-        for (int t = 0; t < n_pad; ++t) {
-            if (t < n_t && wave_active) {
-                ldsK = ldsK_buf[t & 1];
-                ldsV = ldsV_buf[t & 1];
-                scores_softmax(k_begin + t * TK);
-                output_product(k_begin + t * TK);
-            }
+            // the loader wavefronts own no rows: they go on to the tail and leave there
+        } else {
             __syncthreads();
+            for (int t = 0; t < n_pad; ++t) {
+                if (t < n_t && wave_active) {
+                    ldsK = ldsK_buf[t & 1];
+                    ldsV = ldsV_buf[t & 1];
+                    scores_softmax(k_begin + t * TK);
+                    output_product(k_begin + t * TK);
+                }
+                __syncthreads();
+            }
         }
     } else if (PREFETCH) {
         // Small tiles: the whole next tile waits in registers while the current one is used.
@@ -626,6 +665,24 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         if (g == 0) {
             a.part_ml[prow * 2] = m_run;
             a.part_ml[prow * 2 + 1] = l_run;
+        }
+        if (a.part_half) {
+            // normalised by the slice's own sum, so the values are averages of V rows (safe in
+            // fp16's range) and carry 11 bits; the merge weights them with l * 2^(m - m_all)
+            typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+            const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+            _Float16* ph = reinterpret_cast<_Float16*>(a.part_o) + prow * D;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int d = db * 32 + 8 * j + 4 * g;
+                    if (d >= D) continue;
+                    const h4_t pk = {(_Float16)(o[db][4 * j] * inv_l), (_Float16)(o[db][4 * j + 1] * inv_l),
+                                     (_Float16)(o[db][4 * j + 2] * inv_l), (_Float16)(o[db][4 * j + 3] * inv_l)};
+                    *reinterpret_cast<h4_t*>(ph + d) = pk;
+                }
+            return;
         }
         float* po = a.part_o + prow * D;
 #pragma unroll
@@ -934,30 +991,19 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
         }
 }
 
-// Merge of key-split partials: one thread per (pair, row, d).
-template <typename T>
-__global__ void attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, T* __restrict__ out,
-                                  int n_pairs, int n_split, int r_pad, int R, int S, int Hq, int Hkv, int D) {
-    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    const long total = (long)n_pairs * R * D;
-    if (i >= total) return;
-    const int d = (int)(i % D);
-    const int row = (int)((i / D) % R);
-    const int pair = (int)(i / ((long)D * R));
-    float m = -INFINITY;
-    for (int sp = 0; sp < n_split; ++sp) m = fmaxf(m, part_ml[(((long)pair * n_split + sp) * r_pad + row) * 2]);
-    float l = 0.f, acc = 0.f;
-    if (m > -INFINITY) {
-        for (int sp = 0; sp < n_split; ++sp) {
-            const long prow = ((long)pair * n_split + sp) * r_pad + row;
-            const float w = exp2f(part_ml[prow * 2] - m);
-            l += part_ml[prow * 2 + 1] * w;
-            acc += part_o[prow * D + d] * w;
-        }
-    }
+// Merge of key-split partials as a launch of its own: one wavefront per (pair, row).
+template <typename T, bool HALF>
+__global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                                         T* __restrict__ out, int n_pairs, int n_split, int r_pad, int R, int S,
+                                                         int Hq, int Hkv, int D) {
+    const int lane = threadIdx.x & 63;
+    const int ridx = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (ridx >= n_pairs * R) return;  // whole wavefront
+    const int pair = ridx / R, row = ridx % R;
     const int grp = Hq / Hkv, b = pair / Hkv, hk = pair % Hkv;
     const int h = hk * grp + row / S, s = row % S;
-    Elem<T>::store(out + (((long)b * S + s) * Hq + h) * D + d, l > 0.f ? acc / l : 0.f);
+    merge_row<T, HALF>(part_o, part_ml, out + (((long)b * S + s) * Hq + h) * D, (long)pair * n_split * r_pad + row, n_split, r_pad, D,
+                       lane);
 }
 
 // Workspace for key-split partials, grown on demand (never under stream capture:
@@ -983,9 +1029,11 @@ int launch_merge(AttnArgs& a, hipStream_t st) {
     if (a.n_split > 1) {
         const int n_pairs = a.batch * a.Hkv;
         const int R = (a.Hq / a.Hkv) * a.S;
-        const long total = (long)n_pairs * R * D;
-        attn_merge_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs,
-                                                                              a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
+        const unsigned mgrid = (unsigned)(((long)n_pairs * R + 3) / 4);
+        if (a.part_half)
+            attn_merge_kernel<T, true><<<mgrid, 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
+        else
+            attn_merge_kernel<T, false><<<mgrid, 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
         if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     }
     return VLA_K_OK;
@@ -1076,9 +1124,9 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
     else attn_direct_kernel<D, false, ST, false><<<grid, 256, 0, st>>>(a);
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     if (a.n_split > 1) {
-        const long total = (long)n_pairs * R * D;
-        attn_merge_kernel<bf16_t><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a.part_o, a.part_ml, (bf16_t*)a.out, n_pairs,
-                                                                                   a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
+        attn_merge_kernel<bf16_t, false><<<(unsigned)(((long)n_pairs * R + 3) / 4), 256, 0, st>>>(a.part_o, a.part_ml, (bf16_t*)a.out,
+                                                                                           n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq,
+                                                                                           a.Hkv, D);
         if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     }
     return VLA_K_OK;
@@ -1126,6 +1174,18 @@ int launch_d(AttnArgs& a, vla_stream_t stream) {
         if (want > key_tiles) want = key_tiles;
         if (want > 32) want = 32;
         a.n_split = want;
+    } else if (D * sizeof(T) >= 512 && wgs <= 128 && key_tiles >= 4) {
+        // Wide heads (pi0's 256): a workgroup spends ~2.7 us per key tile whatever the batch, so
+        // a 14-tile walk costs 40 us on a quarter of the chip.  Slices of at least two tiles,
+        // as many as still fit the chip in one round; the partial outputs travel as fp16
+        // (normalised per slice: 1.7 MB per slice at batch 16) and the merge pass costs less
+        // than the tiles it removes from the critical path.
+        int want = (int)(256 / wgs);
+        if (want > key_tiles / 2) want = key_tiles / 2;
+        if (want >= 2) {
+            a.n_split = want;
+            a.part_half = getenv("VLA_ATTN_PART_F32") ? 0 : 1;  // the env keeps fp32 partials (tests)
+        }
     }
     if (const char* e = getenv("VLA_ATTN_SPLIT")) a.n_split = atoi(e) > 0 ? (atoi(e) < key_tiles ? atoi(e) : key_tiles) : 1;
     a.tiles_per_split = (key_tiles + a.n_split - 1) / a.n_split;
