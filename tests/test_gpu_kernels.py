@@ -205,7 +205,7 @@ def test_linear_bf16_every_kernel_and_tiling_gives_the_same_bits(monkeypatch, M,
     res = orc.round_bf16(r.standard_normal((M, N)).astype(np.float32))
     xd, Wd, rd = to_dev(x, BF16), to_dev(W, BF16), to_dev(res, BF16)
     outs = {}
-    for dl, tile, stages in [("0", t, "0") for t in "01234"] + [("1", t, ns) for t in "01234" for ns in "234"]:
+    for dl, tile, stages in [("0", t, "0") for t in "01234"] + [("1", t, ns) for t in "01234" for ns in "234"] + [("1", "5", "0")]:
         if True:
             monkeypatch.setenv("VLA_GEMM_DL", dl)
             monkeypatch.setenv("VLA_GEMM_TILE", tile)

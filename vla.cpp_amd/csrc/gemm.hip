@@ -1145,7 +1145,7 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
     a.n_tiles = n_tiles;
     hipStream_t st = (hipStream_t)stream;
     if constexpr (kEpi != EPI_TERNARY) {
-        // VLA_GEMM_TILE = 0..4 pins the tile configuration and VLA_GEMM_STAGES the ring depth
+        // VLA_GEMM_TILE = 0..5 pins the tile configuration and VLA_GEMM_STAGES the ring depth
         // of the direct-to-LDS kernel (tests and tuning); unset = by shape.
         const char* env = getenv("VLA_GEMM_TILE");
         int cfg = env ? atoi(env) : -1;
@@ -1156,6 +1156,11 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             // per multiply); else 128x64 tiles if those fill it; else 64x64 tiles, with
             // 256-byte K rows (half the barriers per K) while one workgroup per CU covers them.
             cfg = wgs0 >= 128 ? 0 : (wgs2 >= 150 ? 2 : (wgs4 <= 256 ? 1 : 4));
+            // Between one and one and a half rounds of 128x128 tiles, some CUs would run two
+            // workgroups while the rest run one; 128x192 tiles cover the same grid in a single
+            // round of 1.5x workgroups (GR00T's fused QKV: 324 -> 216 workgroups).
+            const long wgs5 = m128 * ((n_tiles + 2) / 3);
+            if (cfg == 0 && wgs0 > 256 && wgs0 <= 384 && wgs5 <= 256) cfg = 5;
         }
         // bf16 operands with 16-byte aligned rows and K a multiple of the MFMA depth take the
         // direct-to-LDS kernel (VLA_GEMM_DL=0 pins the register-staged one).  Its ring depth
@@ -1173,6 +1178,9 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             int ns = es ? atoi(es) : 0;
             const long wgs = cfg == 0 ? wgs0 : (cfg == 2 || cfg == 3 ? wgs2 : wgs4);
             switch (cfg) {
+                case 5:  // 40 KiB per stage, one workgroup per CU
+                    launch_dl<kEpi, 2, 3, 128, 3>(a, st);
+                    break;
                 case 0:  // 32 KiB per stage
                     if (ns == 0) ns = wgs <= 256 ? 3 : 2;
                     if (ns <= 2) launch_dl<kEpi, 2, 2, 128, 2>(a, st);
@@ -1207,6 +1215,7 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             case 1: launch_cfg<T, kEpi, 1, 1, 256, 4>(a, st); break;
             case 2: launch_cfg<T, kEpi, 2, 1, 128, 4>(a, st); break;
             case 3: launch_cfg<T, kEpi, 1, 2, 128, 4>(a, st); break;
+            case 5: launch_cfg<T, kEpi, 2, 2, 128, 3>(a, st); break;  // the register-staged kernel has no 192-column tile
             default: launch_cfg<T, kEpi, 1, 1, 128, 6>(a, st); break;
         }
     } else {
