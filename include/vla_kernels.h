@@ -280,6 +280,16 @@ VLA_KAPI int vla_ternary_gemm_add(const int8_t* A, const uint32_t* W_packed, uin
                                   const float* s, const int32_t* rowsum, const float* ws, int ws_num, int M, int N,
                                   int K, vla_stream_t stream);
 
+/* The decode step's norm -> quantise -> projection chain in one launch, for M <= 8 rows:
+ * vla_rmsnorm_act_quant_bf16(x, norm_w, eps) feeding vla_ternary_gemm_add, with the int8
+ * rows, scales and row sums kept on chip (run_layer's attn_norm + QKV and sub_norm + O
+ * pairs, bitvla_lm_cuda.cu:421-486, at S = 1).  Same bits as the two calls.  out may alias
+ * residual, never x (every workgroup reads whole rows of x while others write out).
+ * VLA_K_ERR_SHAPE when M > 8, K > 4096 or K % 128: callers fall back to the pair. */
+VLA_KAPI int vla_rmsnorm_ternary_gemv(const uint16_t* x, const uint16_t* norm_w, float eps, const uint32_t* W_packed,
+                                      uint16_t* out, const uint16_t* residual, const float* ws, int ws_num, int M,
+                                      int N, int K, vla_stream_t stream);
+
 /* -------------------------------------- BitVLA layer helpers (same signatures
  * as src/kernels/bitvla/bitvla_lm_cuda.h:54-155 with hipStream_t / uint16_t) */
 VLA_KAPI int bitvla_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* out, float eps, int M, int K,

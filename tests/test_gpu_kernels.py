@@ -742,6 +742,51 @@ def test_rmsnorm_act_quant_fused_is_the_pair(M, K):
     assert pkg.lib().vla_rmsnorm_act_quant_bf16(0, 0, 0, 0, 0, ctypes.c_float(1e-5), 1, 8, 0) == pkg.VLA_K_ERR_ARG
 
 
+@pytest.mark.parametrize("M,N,K,ws_num", [(1, 3840, 2560, 3), (8, 3840, 2560, 3), (8, 2560, 2560, 1), (3, 48, 128, 3),
+                                          (5, 640, 4096, 1), (7, 100, 1024, 1)])
+def test_rmsnorm_ternary_gemv_one_launch_is_the_chain(M, N, K, ws_num):
+    # Decode rows: norm + quantisation inside the GEMV launch gives the bits of
+    # vla_rmsnorm_act_quant_bf16 -> vla_ternary_gemm_add, with and without the residual
+    # (written in place, as the engine's O projection does).  Two calls in a row on
+    # different rows: nothing of the first survives in the second.
+    r = np.random.default_rng(77 * M + K)
+    t = r.integers(-1, 2, (N, K)).astype(np.int8)
+    ws = (0.01 + 0.001 * r.integers(0, 50, ws_num)).astype(np.float32)
+    w = orc.to_bf16((1 + 0.1 * r.standard_normal(K)).astype(np.float32))
+    dW, dws, dw = dev(_pack_plain(t)), dev(ws), dev(w)
+    for rep in range(2):
+        x = orc.to_bf16((r.standard_normal((M, K)) * (3 if rep == 0 else 0.2)).astype(np.float32))
+        res = orc.to_bf16(r.standard_normal((M, N)).astype(np.float32))
+        q, sc, rs = (torch.zeros((M, K), dtype=torch.int8, device="cuda"), torch.zeros(M, device="cuda"),
+                     torch.zeros(M, dtype=torch.int32, device="cuda"))
+        pkg.call("vla_rmsnorm_act_quant_bf16", dev(x), dw, q, sc, rs, 1e-5, M, K)
+        want, want_res = torch.zeros((M, N), dtype=torch.int16, device="cuda"), dev(res)
+        pkg.call("vla_ternary_gemm", q, dW, want, None, sc, rs, dws, ws_num, M, N, K)
+        pkg.call("vla_ternary_gemm_add", q, dW, want_res, want_res, sc, rs, dws, ws_num, M, N, K)
+        got, got_res = torch.zeros_like(want), dev(res)
+        pkg.call("vla_rmsnorm_ternary_gemv", dev(x), dw, 1e-5, dW, got, None, dws, ws_num, M, N, K)
+        pkg.call("vla_rmsnorm_ternary_gemv", dev(x), dw, 1e-5, dW, got_res, got_res, dws, ws_num, M, N, K)
+        sync()
+        assert torch.equal(got, want) and torch.equal(got_res, want_res)
+    # and the chain follows the oracle: norm -> bf16 -> quantise -> int32 GEMM -> epilogue
+    n = orc.round_bf16(orc.rms_norm(orc.from_bf16(x), orc.from_bf16(w), 1e-5))
+    qo, so = orc.act_quant(n)
+    ref = orc.from_bf16(orc.ternary_epilogue(orc.ternary_gemm_i32(qo, t), so, ws))
+    assert rel_err(orc.from_bf16(host(got, np.uint16)), ref) < 2e-2
+
+
+def test_rmsnorm_ternary_gemv_rejects_what_it_cannot_hold():
+    lib, f = pkg.lib(), ctypes.c_float(1e-5)
+    buf = torch.zeros(16 * 8192, dtype=torch.int16, device="cuda")
+    p = buf.data_ptr()
+    assert lib.vla_rmsnorm_ternary_gemv(p, p, f, p, p, 0, p, 1, 9, 64, 256, 0) == pkg.VLA_K_ERR_SHAPE   # rows
+    assert lib.vla_rmsnorm_ternary_gemv(p, p, f, p, p, 0, p, 1, 4, 64, 8192, 0) == pkg.VLA_K_ERR_SHAPE  # row length
+    assert lib.vla_rmsnorm_ternary_gemv(p, p, f, p, p, 0, p, 1, 4, 64, 200, 0) == pkg.VLA_K_ERR_SHAPE
+    assert lib.vla_rmsnorm_ternary_gemv(p, p, f, p, p, 0, p, 3, 4, 64, 256, 0) == pkg.VLA_K_ERR_SHAPE   # N % ws_num
+    assert lib.vla_rmsnorm_ternary_gemv(0, p, f, p, p, 0, p, 1, 4, 64, 256, 0) == pkg.VLA_K_ERR_ARG
+    assert lib.vla_rmsnorm_ternary_gemv(p, p, f, p, p, 0, p, 1, 0, 64, 256, 0) == pkg.VLA_K_OK
+
+
 def test_ternary_pipeline_matches_cpu_twin():
     # act-quant + ternary GEMM + epilogue against the reference's CPU formulation
     # (fp32 fake-quant GEMM, src/models/bitvla.cpp:173-176): same number up to bf16 rounding.

@@ -92,6 +92,82 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return r;
 }
 
+// One bf16 row through RMSNorm and the per-row int8 quantisation of the BitNet activations,
+// by one wavefront (bitvla_rmsnorm_bf16 then act_quant, src/kernels/bitnet_kernels.h:49-54,
+// without the round trip): lane L holds the 16-byte vectors L, L + 64, ... of the row, NV of
+// them.  y = x * rsqrt(mean(x^2) + eps) * w is rounded to bf16 as it would be stored; the
+// scale is 127 / max(amax, 1e-5); q = clamp(round-half-even(y * scale)).  The int8 row goes
+// to qrow (global or LDS, 8 bytes per vector); scale and the sum of the row's int8 values
+// are returned in every lane.  K % 8 == 0 and K <= 512 NV.
+template <int NV>
+__device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr, const bf16_t* __restrict__ w, int K,
+                                                  float eps, int lane, int8_t* qrow, float& scale_out, int& sum_out) {
+    const int nvec = K / 8;
+    float v[NV][8];
+    u32x4_t wraw[NV];  // the weight's vectors, requested with the row's so that one round trip covers both
+    const bool w_vec = w && !((uintptr_t)w & 15);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int vec = lane + 64 * i;
+        u32x4_t raw = {0u, 0u, 0u, 0u};
+        wraw[i] = raw;
+        if (vec < nvec) {
+            raw = *reinterpret_cast<const u32x4_t*>(xr + (long)vec * 8);
+            if (w_vec) wraw[i] = *reinterpret_cast<const u32x4_t*>(w + (long)vec * 8);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[i][e] = __uint_as_float((e & 1) ? (raw[e >> 1] & 0xffff0000u) : (raw[e >> 1] << 16));
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int vec = lane + 64 * i;
+        if (vec >= nvec) continue;
+        const int k0 = vec * 8;
+        float o[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            o[e] = v[i][e] * inv;
+            if (w_vec) o[e] *= __uint_as_float((e & 1) ? (wraw[i][e >> 1] & 0xffff0000u) : (wraw[i][e >> 1] << 16));
+            else if (w) o[e] *= bf2f(w[k0 + e]);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {  // the activation as the bf16 it would be stored as
+            const uint32_t pr = pack_bf2(o[e], o[e + 1]);
+            v[i][e] = __uint_as_float(pr << 16);
+            v[i][e + 1] = __uint_as_float(pr & 0xffff0000u);
+            amax = fmaxf(amax, fmaxf(fabsf(v[i][e]), fabsf(v[i][e + 1])));
+        }
+    }
+    amax = wave_max(amax);
+    if (amax < 1e-5f) amax = 1e-5f;
+    const float scale = 127.0f / amax;
+    int sum = 0;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int vec = lane + 64 * i;
+        if (vec >= nvec) continue;
+        uint32_t pk[2] = {0u, 0u};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float qf = rintf(v[i][e] * scale);
+            qf = fminf(fmaxf(qf, -128.0f), 127.0f);
+            pk[e >> 2] |= (uint32_t)((int)qf & 0xff) << (8 * (e & 3));
+        }
+        sum = __builtin_amdgcn_sdot4((int)pk[0], 0x01010101, sum, false);  // + the four signed bytes
+        sum = __builtin_amdgcn_sdot4((int)pk[1], 0x01010101, sum, false);
+        *reinterpret_cast<u32x2_t*>(qrow + (long)vec * 8) = u32x2_t{pk[0], pk[1]};
+    }
+    scale_out = scale;
+    sum_out = wave_sum_i(sum);
+}
+
 // ggml_silu / ggml_gelu (tanh form), fp32 (src/layers/ffn.h:24-40).
 __device__ __forceinline__ float apply_act(float x, int act) {
     if (act == VLA_ACT_SILU) return x / (1.0f + __expf(-x));

@@ -147,6 +147,16 @@ __global__ void __launch_bounds__(256) row_norm_kernel(const T* __restrict__ x, 
     constexpr int EPV = 16 / sizeof(T);
     const int lane = threadIdx.x & 63, row = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= M) return;
+    if constexpr (MODE == NORM_RMS_AQ && sizeof(T) == 2) {
+        float scale;
+        int sum;
+        rms_act_quant_row<NV>((const bf16_t*)x + (long)row * K, (const bf16_t*)w, K, eps, lane, q + (long)row * K, scale, sum);
+        if (lane == 0) {
+            scales[row] = scale;
+            if (rowsum) rowsum[row] = sum;
+        }
+        return;
+    }
     const int nvec = K / EPV;
     const T* xr = x + (long)row * K;
     float v[NV][EPV];

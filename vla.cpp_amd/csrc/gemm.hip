@@ -66,6 +66,7 @@ struct GemmArgs {
     int ws_num;
     // RMS statistics of the A rows taken inside the GEMM (direct-to-LDS kernel, kNorm)
     float norm_eps;
+    const void* norm_w;  // ternary GEMV with the RMSNorm and quantisation of its rows inside: A is bf16, this the norm weight
 };
 
 template <typename T> struct Traits;
@@ -1102,6 +1103,79 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_kernel(GemmArgs 
     }
 }
 
+// The same GEMV with the producer of its activations inside: A holds the bf16 rows before
+// RMSNorm, and wavefront w of every workgroup normalises and quantises row w (the code of
+// the stand-alone kernel, so the bits are the same) into LDS while the weight loads are in
+// flight.  Saves the separate norm + quantise launch in front of each decode projection
+// (bitvla.cpp's attn_norm -> QKV and sub_norm -> O pairs).  M <= GEMV_WAVES, K <= 512 NV.
+constexpr int GEMV_FUSED_MAX_K = 4096;
+template <int MAXG, int NV>
+__global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(GemmArgs a) {
+    // int8 rows (stride K + 32 bytes: eight rows' 16-byte fragments fall on distinct banks),
+    // later the partial accumulator tiles
+    constexpr int kPartBytes = GEMV_WAVES * 32 * 33 * 4, kRowBytes = GEMV_WAVES * (GEMV_FUSED_MAX_K + 32);
+    __shared__ __align__(16) unsigned char smem[kPartBytes > kRowBytes ? kPartBytes : kRowBytes];
+    __shared__ float s_sh[GEMV_WAVES];
+    __shared__ int rs_sh[GEMV_WAVES];
+    int (*part)[32][33] = reinterpret_cast<int (*)[32][33]>(smem);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int g = lane >> 5, r = lane & 31;
+    const int nb = blockIdx.x;
+    const int kgroups = a.K / 32;
+    const int per_wave = (kgroups + GEMV_WAVES - 1) / GEMV_WAVES;
+    const int kg0 = wave * per_wave, kg1 = min(kgroups, kg0 + per_wave);
+    const uint32_t* wp = (const uint32_t*)a.W + (long)nb * kgroups * 64 + lane;
+    const int stride = a.K + 32;
+
+    uint32_t wv[MAXG];
+#pragma unroll
+    for (int i = 0; i < MAXG; ++i) wv[i] = wp[(long)min(kg0 + i, kgroups - 1) * 64];
+    if (wave < a.M) {  // uniform per wavefront
+        float scale;
+        int sum;
+        rms_act_quant_row<NV>((const bf16_t*)a.A + (long)wave * a.K, (const bf16_t*)a.norm_w, a.K, a.norm_eps, lane,
+                              (int8_t*)smem + wave * stride, scale, sum);
+        if (lane == 0) {
+            s_sh[wave] = scale;
+            rs_sh[wave] = sum;
+        }
+    }
+    __syncthreads();
+    const bool row_ok = r < a.M;
+    const unsigned char* ap = smem + (row_ok ? r : 0) * stride + g * 16;
+    u32x4_t av[MAXG];
+#pragma unroll
+    for (int i = 0; i < MAXG; ++i) av[i] = *reinterpret_cast<const u32x4_t*>(ap + min(kg0 + i, kgroups - 1) * 32);
+    __syncthreads();  // the rows are in registers: the partial tiles may overwrite them
+    i32x16_t acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0;
+#pragma unroll
+    for (int i = 0; i < MAXG; ++i) {
+        if (kg0 + i < kg1) {
+            const uint32_t w = wv[i];
+            const u32x4_t fw = {w & 0x03030303u, (w >> 2) & 0x03030303u, (w >> 4) & 0x03030303u, (w >> 6) & 0x03030303u};
+            const u32x4_t z = {0u, 0u, 0u, 0u};
+            Traits<int8_t>::mma(acc, fw, row_ok ? av[i] : z);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) part[wave][8 * (e >> 2) + 4 * g + (e & 3)][r] = acc[e];
+    __syncthreads();
+    const int group = a.N / a.ws_num;
+    for (int m = tid >> 5; m < a.M; m += GEMV_WAVES * 2) {
+        const int nl = tid & 31, n = nb * 32 + nl;
+        if (n >= a.N) continue;
+        int v = 0;
+#pragma unroll
+        for (int w = 0; w < GEMV_WAVES; ++w) v += part[w][nl][m];
+        v -= 2 * rs_sh[m];
+        bf16_t o = f2bf((float)v / s_sh[m] * a.ws[n / group]);
+        if (a.residual) o = f2bf(bf2f(o) + bf2f(((const bf16_t*)a.residual)[(long)m * a.N + n]));
+        ((bf16_t*)a.Y)[(long)m * a.N + n] = o;
+    }
+}
+
 // XCD grid xm x xn = 8 for a tile grid of m_wg x n_wg workgroup tiles: every L2 reads its M
 // tiles' rows of A and its N tiles' rows of W once; the split with the least total,
 // counting the padding of the tile grid.  Returns the grid size.
@@ -1443,6 +1517,30 @@ int vla_ternary_gemm_add(const int8_t* A, const uint32_t* W_packed, uint16_t* ou
     a.A = A; a.W = W_packed; a.M = M; a.N = N; a.K = K;
     a.Y = out; a.residual = residual; a.s = s; a.rowsum = rowsum; a.ws = ws; a.ws_num = ws_num;
     return launch<int8_t, EPI_TERNARY>(a, (N + BN - 1) / BN, stream);
+}
+
+int vla_rmsnorm_ternary_gemv(const uint16_t* x, const uint16_t* norm_w, float eps, const uint32_t* W_packed, uint16_t* out,
+                             const uint16_t* residual, const float* ws, int ws_num, int M, int N, int K,
+                             vla_stream_t stream) {
+    if (!x || !W_packed || !out || !ws || ws_num <= 0 || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (M > GEMV_WAVES || K > GEMV_FUSED_MAX_K || K % 128 || N % ws_num || (((uintptr_t)x) & 15)) return VLA_K_ERR_SHAPE;
+    if (M == 0) return VLA_K_OK;
+    GemmArgs a = {};
+    a.A = x; a.norm_w = norm_w; a.norm_eps = eps; a.W = W_packed; a.M = M; a.N = N; a.K = K;
+    a.Y = out; a.residual = residual; a.ws = ws; a.ws_num = ws_num;
+    const unsigned grid = (unsigned)((N + 31) / 32);
+    const int groups = (K / 32 + GEMV_WAVES - 1) / GEMV_WAVES, nvec = K / 8;
+    hipStream_t st = (hipStream_t)stream;
+#define VLA_GEMV_NORM(G, NV) ternary_gemv_norm_kernel<G, NV><<<grid, GEMV_WAVES * 64, 0, st>>>(a)
+    if (groups <= 10) {
+        if (nvec <= 128) VLA_GEMV_NORM(10, 2);
+        else if (nvec <= 256) VLA_GEMV_NORM(10, 4);
+        else VLA_GEMV_NORM(10, 8);
+    } else {
+        VLA_GEMV_NORM(16, 8);
+    }
+#undef VLA_GEMV_NORM
+    return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
 }
 
 static int bitvla_ws_num(int N, int K) {  // the reference's per-shape table, bitnet_kernels.cu:31-116

@@ -207,20 +207,36 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
     const float scale = 1.0f / std::sqrt((float)D_);
     const float* cos_t = rope_.cos.as<float>() + (size_t)tok_offset * half;
     const float* sin_t = rope_.sin.as<float>() + (size_t)tok_offset * half;
+    // a handful of rows (token-by-token decode): norm, quantisation and projection in one launch
+    const bool fused = M <= 8 && H_ <= 4096 && H_ % 128 == 0;
     for (LmLayer& w : layers_) {
-        VLA_K(vla_rmsnorm_act_quant_bf16(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
-                                         rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
-        VLA_K(vla_ternary_gemm(q8_.as<int8_t>(), w.Wqkv.packed.as<uint32_t>(), qkv_.as<uint16_t>(), nullptr, s_.as<float>(),
-                               rowsum_.as<int32_t>(), w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_, C.stream));
+        if (fused) {
+            VLA_K(vla_rmsnorm_ternary_gemv(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), eps_, w.Wqkv.packed.as<uint32_t>(),
+                                           qkv_.as<uint16_t>(), nullptr, w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_,
+                                           C.stream));
+        } else {
+            VLA_K(vla_rmsnorm_act_quant_bf16(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
+                                             rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
+            VLA_K(vla_ternary_gemm(q8_.as<int8_t>(), w.Wqkv.packed.as<uint32_t>(), qkv_.as<uint16_t>(), nullptr,
+                                   s_.as<float>(), rowsum_.as<int32_t>(), w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_,
+                                   C.stream));
+        }
         VLA_K(vla_qkv_split_rope_append(qkv_.get(), cos_t, sin_t, q_.get(), w.kv.k.get(), w.kv.vt.get(), VLA_DT_BF16, M, S,
                                         Hq_, Hkv_, D_, w.kv.t_max, tok_offset, C.stream));
         VLA_K(vla_attn_prefix_suffix(q_.get(), w.kv.k.get(), w.kv.vt.get(), att_.get(), VLA_DT_BF16_P2, M / S, S, Hq_, Hkv_,
                                      D_, w.kv.t_max, n_keys, scale, VLA_MASK_NONE, n_keys, 0, 0, nullptr, C.stream));
-        VLA_K(vla_rmsnorm_act_quant_bf16(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
-                                         rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
         // O projection and the residual add of the hidden stream in one launch
-        VLA_K(vla_ternary_gemm_add(q8_.as<int8_t>(), w.Wo.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
-                                   s_.as<float>(), rowsum_.as<int32_t>(), w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_, C.stream));
+        if (fused) {
+            VLA_K(vla_rmsnorm_ternary_gemv(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), eps_, w.Wo.packed.as<uint32_t>(),
+                                           h_.as<uint16_t>(), h_.as<uint16_t>(), w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_,
+                                           C.stream));
+        } else {
+            VLA_K(vla_rmsnorm_act_quant_bf16(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
+                                             rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
+            VLA_K(vla_ternary_gemm_add(q8_.as<int8_t>(), w.Wo.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
+                                       s_.as<float>(), rowsum_.as<int32_t>(), w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_,
+                                       C.stream));
+        }
     }
 }
 
