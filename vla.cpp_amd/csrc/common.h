@@ -22,14 +22,10 @@ typedef uint16_t u16x8_t __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
 
-// bf16 <-> f32, round to nearest even, NaN quieted.
+// bf16 <-> f32, round to nearest even, NaN quieted: the hardware converter (v_cvt_pk_bf16_f32),
+// one instruction where the integer formulation takes seven.
 __device__ __forceinline__ float bf2f(bf16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
-__device__ __forceinline__ bf16_t f2bf(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (bf16_t)(u >> 16);
-}
+__device__ __forceinline__ bf16_t f2bf(float f) { return __builtin_bit_cast(bf16_t, (__bf16)f); }
 // Two floats -> packed bf16 pair with the hardware converter (v_cvt_pk_bf16_f32,
 // round to nearest even).
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
