@@ -159,12 +159,13 @@ def kernel_breakdown(pkg, cfg, B, P):
         add("ternary_qkv_gemv", lambda i: pkg.call("vla_ternary_gemm", q8, wq, qkv, None, s, rs, ws, 6, M, N, H),
             0 if fused else L, "hbm", N * H // 4 + M * H + 2 * M * N)
         if fused:
-            add("norm_quant_ternary_qkv_gemv", lambda i: pkg.call("vla_rmsnorm_ternary_gemv", h, w1, 1e-5, wq, qkv, None, ws, 6,
-                                                                  M, N, H), L, "hbm", N * H // 4 + 2 * M * H + 2 * M * N)
+            add("norm_quant_ternary_qkv_gemv_rope_append",
+                lambda i: pkg.call("vla_rmsnorm_ternary_gemv_rope_append", h, w1, 1e-5, wq, ws, 6, cos, sin, q, kc, vc, M, Hq, Hkv,
+                                   D, H, t_max, P), L, "hbm", N * H // 4 + 2 * M * H + 2 * M * N)
             add("norm_quant_ternary_o_gemv_add", lambda i: pkg.call("vla_rmsnorm_ternary_gemv", att, w1, 1e-5, wo, h, h, ws, 1,
                                                                     M, H, H), L, "hbm", H * H // 4 + 2 * M * H + 4 * M * H)
         add("qkv_split_rope_append", lambda i: pkg.call("vla_qkv_split_rope_append", qkv, cos, sin, q, kc, vc, dt, M, 1, Hq,
-                                                       Hkv, D, t_max, P), L, "hbm", 2 * M * N * 2)
+                                                       Hkv, D, t_max, P), 0 if fused else L, "hbm", 2 * M * N * 2)
         add("attention_decode", lambda i: pkg.call("vla_attn_prefix_suffix", q, kcs[i % n_rot], vcs[i % n_rot], att,
                                                  pkg.VLA_DT_BF16_P2, B, 1, Hq, Hkv, D, t_max, T, scale, 0, T, 0, 0, None),
             L, "hbm", 2 * T * kvd * es * B)

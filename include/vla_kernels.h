@@ -290,6 +290,27 @@ VLA_KAPI int vla_rmsnorm_ternary_gemv(const uint16_t* x, const uint16_t* norm_w,
                                       uint16_t* out, const uint16_t* residual, const float* ws, int ws_num, int M,
                                       int N, int K, vla_stream_t stream);
 
+/* The same launch for the fused Q | K | V projection of one appended token per batch row,
+ * with vla_qkv_split_rope_append (S = 1) in its epilogue: Q rotated to q_out [batch][Hq][D],
+ * K rotated into k_cache at slot tok_offset, V into vt_cache (attn_norm -> QKV -> RoPE ->
+ * cache of run_layer, bitvla_lm_cuda.cu:421-460).  cos_row / sin_row: the D/2 table entries
+ * of the token's position.  W_paired: the packed weight with its rows reordered by
+ * vla_ternary_pair_rope_rows_host (a rotation pair in one 32-row block).  Same bits as
+ * vla_rmsnorm_ternary_gemv + vla_qkv_split_rope_append.  N = (Hq + 2 Hkv) D;
+ * VLA_K_ERR_SHAPE when batch > 8, K > 4096, K % 128, D % 32 or a scale group (N / ws_num)
+ * is not whole heads. */
+VLA_KAPI int vla_rmsnorm_ternary_gemv_rope_append(const uint16_t* x, const uint16_t* norm_w, float eps,
+                                                  const uint32_t* W_paired, const float* ws, int ws_num,
+                                                  const float* cos_row, const float* sin_row, uint16_t* q_out,
+                                                  uint16_t* k_cache, uint16_t* vt_cache, int batch, int n_q_heads,
+                                                  int n_kv_heads, int head_dim, int K, int t_max, int tok_offset,
+                                                  vla_stream_t stream);
+/* paired = packed with row n of every Q and K head taken from row
+ * (n < 16 ? 16 b + n : D/2 + 16 b + n - 16) of 32-row block b of that head; V rows unchanged.
+ * Host memory, vla_ternary_packed_words(N, K) words each, no overlap. */
+VLA_KAPI int vla_ternary_pair_rope_rows_host(const uint32_t* packed, int n_q_heads, int n_kv_heads, int head_dim,
+                                             int K, uint32_t* paired);
+
 /* -------------------------------------- BitVLA layer helpers (same signatures
  * as src/kernels/bitvla/bitvla_lm_cuda.h:54-155 with hipStream_t / uint16_t) */
 VLA_KAPI int bitvla_rmsnorm_bf16(const uint16_t* x, const uint16_t* w, uint16_t* out, float eps, int M, int K,

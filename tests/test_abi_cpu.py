@@ -71,6 +71,29 @@ def test_ternary_quant_and_packers_against_oracle():
     assert lib.vla_ternary_repack_ladder_host(raw.ctypes.data, 24, K, rep.ctypes.data) == pkg.VLA_K_ERR_SHAPE
 
 
+def test_pair_rope_rows_host_is_the_row_permutation_the_decode_epilogue_assumes():
+    # Packing the permuted ternary matrix equals permuting the packed words: inside Q and K heads
+    # 32-row block b holds rows 16b..16b+15 then D/2+16b..D/2+16b+15; V rows stay.
+    lib = pkg.lib()
+    Hq, Hkv, D, K = 3, 1, 64, 128
+    N = (Hq + 2 * Hkv) * D
+    r = np.random.default_rng(5)
+    t = r.integers(-1, 2, (N, K)).astype(np.int8)
+    src = np.arange(N)
+    for n in range((Hq + Hkv) * D):
+        rr, nl = n % D, n % 32
+        src[n] = n - rr + (16 * (rr // 32) + nl if nl < 16 else D // 2 + 16 * (rr // 32) + nl - 16)
+    assert sorted(src) == list(range(N))
+    packed, want, got = (np.empty(N * K // 16, np.uint32) for _ in range(3))
+    assert lib.vla_ternary_pack_host(t.ctypes.data, N, K, packed.ctypes.data) == 0
+    tp = np.ascontiguousarray(t[src])
+    assert lib.vla_ternary_pack_host(tp.ctypes.data, N, K, want.ctypes.data) == 0
+    assert lib.vla_ternary_pair_rope_rows_host(packed.ctypes.data, Hq, Hkv, D, K, got.ctypes.data) == 0
+    assert np.array_equal(got, want)
+    assert lib.vla_ternary_pair_rope_rows_host(packed.ctypes.data, Hq, Hkv, 48, K, got.ctypes.data) == pkg.VLA_K_ERR_SHAPE
+    assert lib.vla_ternary_pair_rope_rows_host(packed.ctypes.data, Hq, Hkv, D, K, packed.ctypes.data) == pkg.VLA_K_ERR_ARG
+
+
 def test_fold_norm_weight_host_rounds_products_to_nearest_even():
     lib = pkg.lib()
     r = np.random.default_rng(7)

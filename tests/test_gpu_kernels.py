@@ -775,6 +775,44 @@ def test_rmsnorm_ternary_gemv_one_launch_is_the_chain(M, N, K, ws_num):
     assert rel_err(orc.from_bf16(host(got, np.uint16)), ref) < 2e-2
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,D,K,ws_num", [(8, 20, 5, 128, 2560, 6), (1, 20, 5, 128, 2560, 6), (3, 4, 2, 64, 256, 2),
+                                                 (5, 2, 2, 32, 128, 1)])
+def test_rmsnorm_ternary_gemv_rope_append_one_launch_is_the_chain(B, Hq, Hkv, D, K, ws_num):
+    # One appended token per batch row: norm + quantisation + QKV GEMV + split + RoPE + cache
+    # append in one launch (paired weight rows) gives the bits of the three-launch chain, in Q
+    # and in the written cache slot, and touches nothing else of the cache.
+    r = np.random.default_rng(31 * B + D)
+    N, t_max, pos = (Hq + 2 * Hkv) * D, 64, 37
+    t = r.integers(-1, 2, (N, K)).astype(np.int8)
+    ws = (0.01 + 0.001 * r.integers(0, 50, ws_num)).astype(np.float32)
+    w = orc.to_bf16((1 + 0.1 * r.standard_normal(K)).astype(np.float32))
+    x = orc.to_bf16((r.standard_normal((B, K)) * 2).astype(np.float32))
+    cos, sin = orc.rope_tables(np.int32([pos]), D, 10000.0)
+    packed = _pack_plain(t)
+    paired = np.empty_like(packed)
+    assert pkg.lib().vla_ternary_pair_rope_rows_host(packed.ctypes.data, Hq, Hkv, D, K, paired.ctypes.data) == 0
+    dws, dw, dx, dcos, dsin = dev(ws), dev(w), dev(x), dev(cos.astype(np.float32)), dev(sin.astype(np.float32))
+    fill = r.integers(0, 65536, (2, B, Hkv, t_max * D)).astype(np.uint16)
+    kc1, vc1, kc2, vc2 = dev(fill[0]), dev(fill[1]), dev(fill[0]), dev(fill[1])
+    q1 = torch.zeros((B, Hq * D), dtype=torch.int16, device="cuda")
+    q2 = torch.zeros_like(q1)
+    qkv = torch.zeros((B, N), dtype=torch.int16, device="cuda")
+    pkg.call("vla_rmsnorm_ternary_gemv", dx, dw, 1e-5, dev(packed), qkv, None, dws, ws_num, B, N, K)
+    pkg.call("vla_qkv_split_rope_append", qkv, dcos, dsin, q1, kc1, vc1, pkg.VLA_DT_BF16, B, 1, Hq, Hkv, D, t_max, pos)
+    pkg.call("vla_rmsnorm_ternary_gemv_rope_append", dx, dw, 1e-5, dev(paired), dws, ws_num, dcos, dsin, q2, kc2, vc2, B, Hq, Hkv,
+             D, K, t_max, pos)
+    sync()
+    assert torch.equal(q1, q2) and torch.equal(kc1, kc2) and torch.equal(vc1, vc2)
+    assert not np.array_equal(host(kc2, np.uint16), fill[0]) and not np.array_equal(host(vc2, np.uint16), fill[1])
+    lib, f, p = pkg.lib(), ctypes.c_float(1e-5), qkv.data_ptr()
+    bad = lambda *a: lib.vla_rmsnorm_ternary_gemv_rope_append(p, p, f, p, p, a[0], p, p, p, p, p, a[1], a[2], a[3], a[4], a[5], 64, a[6], 0)
+    assert bad(1, 9, 2, 2, 32, 128, 0) == pkg.VLA_K_ERR_SHAPE      # rows
+    assert bad(1, 4, 2, 2, 48, 128, 0) == pkg.VLA_K_ERR_SHAPE      # head width not whole 32-row blocks
+    assert bad(4, 4, 2, 2, 32, 128, 0) == pkg.VLA_K_ERR_SHAPE      # scale group of 48 columns cuts a head
+    assert bad(1, 4, 2, 2, 32, 128, 64) == pkg.VLA_K_ERR_SHAPE     # slot past the cache
+    assert bad(1, 0, 2, 2, 32, 128, 0) == pkg.VLA_K_OK
+
+
 def test_rmsnorm_ternary_gemv_rejects_what_it_cannot_hold():
     lib, f = pkg.lib(), ctypes.c_float(1e-5)
     buf = torch.zeros(16 * 8192, dtype=torch.int16, device="cuda")

@@ -1108,8 +1108,15 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_kernel(GemmArgs 
 // the stand-alone kernel, so the bits are the same) into LDS while the weight loads are in
 // flight.  Saves the separate norm + quantise launch in front of each decode projection
 // (bitvla.cpp's attn_norm -> QKV and sub_norm -> O pairs).  M <= GEMV_WAVES, K <= 512 NV.
+//
+// ROPE: the fused Q | K | V projection of one appended token per batch row, with the split,
+// the NeoX rotation and the cache append of qkv_split_rope_append_kernel in the epilogue.  The
+// weight rows are in "paired" order (vla_ternary_pair_rope_rows_host): inside the Q and K
+// columns every 32-row block holds 16 rotation pairs, d in lanes 0-15 and d + D/2 in lanes
+// 16-31, so a pair meets through one shuffle.  The projection is rounded to bf16 before the
+// rotation, as the stand-alone chain stores it.
 constexpr int GEMV_FUSED_MAX_K = 4096;
-template <int MAXG, int NV>
+template <int MAXG, int NV, bool ROPE>
 __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(GemmArgs a) {
     // int8 rows (stride K + 32 bytes: eight rows' 16-byte fragments fall on distinct banks),
     // later the partial accumulator tiles
@@ -1171,8 +1178,27 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
         for (int w = 0; w < GEMV_WAVES; ++w) v += part[w][nl][m];
         v -= 2 * rs_sh[m];
         bf16_t o = f2bf((float)v / s_sh[m] * a.ws[n / group]);
-        if (a.residual) o = f2bf(bf2f(o) + bf2f(((const bf16_t*)a.residual)[(long)m * a.N + n]));
-        ((bf16_t*)a.Y)[(long)m * a.N + n] = o;
+        if constexpr (ROPE) {  // N is a multiple of 32 here: no lane of a half-wavefront is missing
+            const float own = bf2f(o);
+            const float other = __shfl_xor(own, 16, 64);
+            const int hh = n / a.D, r = n % a.D, half = a.D >> 1;
+            if (hh < a.Hq + a.Hkv) {
+                const bool lower = nl < 16;
+                const int pi = 16 * (r >> 5) + (nl & 15);
+                const float c = a.cos_t[pi], sn = a.sin_t[pi];
+                const float x0 = lower ? own : other, x1 = lower ? other : own;
+                const float lo = x0 * c - x1 * sn, hi = x1 * c + x0 * sn;
+                const int d = lower ? pi : pi + half;
+                const bf16_t rot = f2bf(lower ? lo : hi);
+                if (hh < a.Hq) ((bf16_t*)a.q_out)[((long)m * a.Hq + hh) * a.D + d] = rot;
+                else ((bf16_t*)a.k_cache)[(((long)m * a.Hkv + (hh - a.Hq)) * a.t_max + a.tok_offset) * a.D + d] = rot;
+            } else {
+                ((bf16_t*)a.vt_cache)[(((long)m * a.Hkv + (hh - a.Hq - a.Hkv)) * a.D + r) * (long)a.t_max + a.tok_offset] = o;
+            }
+        } else {
+            if (a.residual) o = f2bf(bf2f(o) + bf2f(((const bf16_t*)a.residual)[(long)m * a.N + n]));
+            ((bf16_t*)a.Y)[(long)m * a.N + n] = o;
+        }
     }
 }
 
@@ -1329,6 +1355,23 @@ __global__ void rowsum_i8_kernel(const int8_t* __restrict__ A, int32_t* __restri
 
 int32_t* g_rowsum = nullptr;
 int g_rowsum_cap = 0;
+
+template <bool ROPE>
+int launch_gemv_norm(const GemmArgs& a, vla_stream_t stream) {
+    const unsigned grid = (unsigned)((a.N + 31) / 32);
+    const int groups = (a.K / 32 + GEMV_WAVES - 1) / GEMV_WAVES, nvec = a.K / 8;
+    hipStream_t st = (hipStream_t)stream;
+#define VLA_GEMV_NORM(G, NV) ternary_gemv_norm_kernel<G, NV, ROPE><<<grid, GEMV_WAVES * 64, 0, st>>>(a)
+    if (groups <= 10) {
+        if (nvec <= 128) VLA_GEMV_NORM(10, 2);
+        else if (nvec <= 256) VLA_GEMV_NORM(10, 4);
+        else VLA_GEMV_NORM(10, 8);
+    } else {
+        VLA_GEMV_NORM(16, 8);
+    }
+#undef VLA_GEMV_NORM
+    return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+}
 
 }  // namespace
 
@@ -1528,19 +1571,46 @@ int vla_rmsnorm_ternary_gemv(const uint16_t* x, const uint16_t* norm_w, float ep
     GemmArgs a = {};
     a.A = x; a.norm_w = norm_w; a.norm_eps = eps; a.W = W_packed; a.M = M; a.N = N; a.K = K;
     a.Y = out; a.residual = residual; a.ws = ws; a.ws_num = ws_num;
-    const unsigned grid = (unsigned)((N + 31) / 32);
-    const int groups = (K / 32 + GEMV_WAVES - 1) / GEMV_WAVES, nvec = K / 8;
-    hipStream_t st = (hipStream_t)stream;
-#define VLA_GEMV_NORM(G, NV) ternary_gemv_norm_kernel<G, NV><<<grid, GEMV_WAVES * 64, 0, st>>>(a)
-    if (groups <= 10) {
-        if (nvec <= 128) VLA_GEMV_NORM(10, 2);
-        else if (nvec <= 256) VLA_GEMV_NORM(10, 4);
-        else VLA_GEMV_NORM(10, 8);
-    } else {
-        VLA_GEMV_NORM(16, 8);
+    return launch_gemv_norm<false>(a, stream);
+}
+
+int vla_rmsnorm_ternary_gemv_rope_append(const uint16_t* x, const uint16_t* norm_w, float eps, const uint32_t* W_paired,
+                                         const float* ws, int ws_num, const float* cos_row, const float* sin_row,
+                                         uint16_t* q_out, uint16_t* k_cache, uint16_t* vt_cache, int batch, int n_q_heads,
+                                         int n_kv_heads, int head_dim, int K, int t_max, int tok_offset,
+                                         vla_stream_t stream) {
+    if (!x || !W_paired || !ws || !cos_row || !sin_row || !q_out || !k_cache || !vt_cache || ws_num <= 0 || batch < 0 ||
+        n_q_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || K <= 0)
+        return VLA_K_ERR_ARG;
+    const int N = (n_q_heads + 2 * n_kv_heads) * head_dim;
+    if (batch > GEMV_WAVES || K > GEMV_FUSED_MAX_K || K % 128 || head_dim % 32 || N % ws_num || (N / ws_num) % head_dim ||
+        tok_offset < 0 || tok_offset >= t_max || (((uintptr_t)x) & 15))
+        return VLA_K_ERR_SHAPE;
+    if (batch == 0) return VLA_K_OK;
+    GemmArgs a = {};
+    a.A = x; a.norm_w = norm_w; a.norm_eps = eps; a.W = W_paired; a.M = batch; a.N = N; a.K = K;
+    a.ws = ws; a.ws_num = ws_num; a.cos_t = cos_row; a.sin_t = sin_row;
+    a.q_out = q_out; a.k_cache = k_cache; a.vt_cache = vt_cache;
+    a.Hq = n_q_heads; a.Hkv = n_kv_heads; a.D = head_dim; a.t_max = t_max; a.tok_offset = tok_offset; a.S = 1;
+    return launch_gemv_norm<true>(a, stream);
+}
+
+int vla_ternary_pair_rope_rows_host(const uint32_t* packed, int n_q_heads, int n_kv_heads, int head_dim, int K,
+                                    uint32_t* paired) {
+    if (!packed || !paired || packed == paired || n_q_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || K <= 0)
+        return VLA_K_ERR_ARG;
+    if (head_dim % 32 || K % 32) return VLA_K_ERR_SHAPE;
+    const int half = head_dim / 2, kw = K / 16;
+    const long rope_rows = (long)(n_q_heads + n_kv_heads) * head_dim, N = rope_rows + (long)n_kv_heads * head_dim;
+    for (long n = 0; n < N; ++n) {
+        long src = n;
+        if (n < rope_rows) {
+            const int r = (int)(n % head_dim), nl = r % 32;
+            src = n - r + (nl < 16 ? 16 * (r / 32) + nl : half + 16 * (r / 32) + (nl - 16));
+        }
+        for (int w = 0; w < kw; ++w) paired[tern_word_index(n, w, K)] = packed[tern_word_index(src, w, K)];
     }
-#undef VLA_GEMV_NORM
-    return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+    return VLA_K_OK;
 }
 
 static int bitvla_ws_num(int N, int K) {  // the reference's per-shape table, bitnet_kernels.cu:31-116

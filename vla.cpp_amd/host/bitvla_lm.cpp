@@ -35,12 +35,15 @@ int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
 struct TernaryW {
     DevBuf packed;  // [N][K/16] words
+    DevBuf paired;  // fused QKV only: the same words with rotation pairs in one 32-row block (decode launch)
     DevBuf ws;      // fp32 [ws_num]
     int N = 0, K = 0, ws_num = 1;
 };
 
 // `parts` = row counts of the tensors fused into `name` (one absmean each).
-TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::vector<int>& parts, int K, int ws_group) {
+// pair_q / pair_kv / pair_d > 0: also keep the row order of vla_ternary_pair_rope_rows_host.
+TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::vector<int>& parts, int K, int ws_group,
+                      int pair_q = 0, int pair_kv = 0, int pair_d = 0) {
     TernaryW w;
     w.K = K;
     for (int n : parts) w.N += n;
@@ -74,6 +77,11 @@ TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::
     w.ws_num = (int)ws.size();
     w.packed.upload(packed.data(), packed.size() * 4);
     w.ws.upload(ws.data(), ws.size() * 4);
+    if (pair_d > 0 && pair_d % 32 == 0 && K % 32 == 0 && ws_group % pair_d == 0 && w.N == (pair_q + 2 * pair_kv) * pair_d) {
+        std::vector<uint32_t> paired(packed.size());
+        VLA_K(vla_ternary_pair_rope_rows_host(packed.data(), pair_q, pair_kv, pair_d, K, paired.data()));
+        w.paired.upload(paired.data(), paired.size() * 4);
+    }
     return w;
 }
 
@@ -145,7 +153,7 @@ BitvlaLm::BitvlaLm(const Checkpoint& ck) {
         std::vector<float> a = ck.f32(p + "attn_norm"), s = ck.f32(p + "sub_norm");
         upload_as(w.attn_norm, a.data(), a.size(), VLA_DT_BF16);
         upload_as(w.sub_norm, s.data(), s.size(), VLA_DT_BF16);
-        w.Wqkv = load_ternary(ck, p + "Wqkv", {H_, kvd, kvd}, H_, kvd);
+        w.Wqkv = load_ternary(ck, p + "Wqkv", {H_, kvd, kvd}, H_, kvd, Hq_, Hkv_, D_);
         w.Wo = load_ternary(ck, p + "Wo", {H_}, H_, H_);
     }
 }
@@ -210,7 +218,14 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
     // a handful of rows (token-by-token decode): norm, quantisation and projection in one launch
     const bool fused = M <= 8 && H_ <= 4096 && H_ % 128 == 0;
     for (LmLayer& w : layers_) {
-        if (fused) {
+        if (fused && S == 1 && w.Wqkv.paired.get()) {
+            // ... and the split, rotation and cache append as well
+            VLA_K(vla_rmsnorm_ternary_gemv_rope_append(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), eps_,
+                                                       w.Wqkv.paired.as<uint32_t>(), w.Wqkv.ws.as<float>(), w.Wqkv.ws_num,
+                                                       cos_t, sin_t, q_.as<uint16_t>(), w.kv.k.as<uint16_t>(),
+                                                       w.kv.vt.as<uint16_t>(), M, Hq_, Hkv_, D_, H_, w.kv.t_max, tok_offset,
+                                                       C.stream));
+        } else if (fused) {
             VLA_K(vla_rmsnorm_ternary_gemv(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), eps_, w.Wqkv.packed.as<uint32_t>(),
                                            qkv_.as<uint16_t>(), nullptr, w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_,
                                            C.stream));
@@ -221,8 +236,9 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
                                    s_.as<float>(), rowsum_.as<int32_t>(), w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_,
                                    C.stream));
         }
-        VLA_K(vla_qkv_split_rope_append(qkv_.get(), cos_t, sin_t, q_.get(), w.kv.k.get(), w.kv.vt.get(), VLA_DT_BF16, M, S,
-                                        Hq_, Hkv_, D_, w.kv.t_max, tok_offset, C.stream));
+        if (!(fused && S == 1 && w.Wqkv.paired.get()))
+            VLA_K(vla_qkv_split_rope_append(qkv_.get(), cos_t, sin_t, q_.get(), w.kv.k.get(), w.kv.vt.get(), VLA_DT_BF16, M, S,
+                                            Hq_, Hkv_, D_, w.kv.t_max, tok_offset, C.stream));
         VLA_K(vla_attn_prefix_suffix(q_.get(), w.kv.k.get(), w.kv.vt.get(), att_.get(), VLA_DT_BF16_P2, M / S, S, Hq_, Hkv_,
                                      D_, w.kv.t_max, n_keys, scale, VLA_MASK_NONE, n_keys, 0, 0, nullptr, C.stream));
         // O projection and the residual add of the hidden stream in one launch
