@@ -286,13 +286,13 @@ def kernel_breakdown(pkg, cfg, B, P):
 # 256 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the per-kernel tables and
 # the commands are in profiles/*_pmc.txt.  Kernels without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg1_smolvla_16layer_bf16_b32", "wo_residual"): int((7817.0 * 2 + 2250.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "qkv_rope_append_self"): int((6963.5 * 2 + 5400.2) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "q_rope_cross"): int((5082.0 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "attention_self"): int((7731.1 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "attention_cross"): int((6588.5 * 2 + 3000.0) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "attention_cross"): int((62782.4 * 2 + 3345.6) * 1024),
-    ("cfg4_bitvla_30layer_b8", "ternary_qkv_gemm_prefill"): int((16939.8 * 2 + 30720.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "wo_residual"): int((7821.0 * 2 + 2250.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "qkv_rope_append_self"): int((6934.0 * 2 + 5400.1) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "q_rope_cross"): int((5072.5 * 2 + 3000.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "attention_self"): int((7734.6 * 2 + 3000.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "attention_cross"): int((6592.0 * 2 + 3000.0) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "attention_cross"): int((62789.0 * 2 + 3351.8) * 1024),
+    ("cfg4_bitvla_30layer_b8", "ternary_qkv_gemm_prefill"): int((16895.0 * 2 + 30720.0) * 1024),
 }
 
 
