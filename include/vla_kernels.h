@@ -338,6 +338,49 @@ VLA_KAPI int bitlinear_int8xint2_m(int8_t* A, int8_t* B, uint16_t* out, float* s
 VLA_KAPI int bitlinear_int8xint2(int8_t* A, int8_t* B, uint16_t* out, float* s, float* ws, int M, int N, int K,
                                  vla_stream_t stream);
 
+/* out[s][k] = bf16(relu(gate[s][k])^2 * up[s][k]) on a fused [seq][gate(ffn) | up(ffn)] projection
+ * (gate_up_fused_sqrelu_mul_bf16, src/kernels/bitvla/bitvla_lm_cuda.cu:525-548). */
+VLA_KAPI int gate_up_fused_sqrelu_mul_bf16(const uint16_t* gu, uint16_t* out, int seq, int ffn, vla_stream_t stream);
+
+/* The context form of the BitVLA language model (bitvla_lm_layer_cuda and
+ * bitvla_lm_cuda_{init,set_layer,set_output_norm,forward,free},
+ * src/kernels/bitvla/bitvla_lm_cuda.h:211-286; run_layer,
+ * src/kernels/bitvla/bitvla_lm_cuda.cu:395-522): same fields, arguments and meaning, device
+ * pointers owned by the caller.  Differences: *_packed weights are in the gfx950 word order
+ * (vla_ternary_pack_host / vla_ternary_repack_ladder_host, one buffer of
+ * vla_ternary_packed_words(N, K) words per tensor); *_ws hold one fp32 scale per tensor, two for
+ * gate_up (gate, up); attention runs as one fused kernel with fp32 scores instead of bf16
+ * scores between two library GEMMs.  forward() copies d_in, runs every layer over all `seq`
+ * tokens (no mask, positions 0..seq-1) and writes the output-normed hidden states; it launches
+ * on `stream` without synchronising and returns 0, or -1 for seq > max_seq, an unbound layer
+ * or a failed launch.  One forward at a time per context. */
+typedef struct {
+    uint16_t* attn_norm_w;
+    uint16_t* attn_sub_norm_w;
+    uint16_t* ffn_norm_w;
+    uint16_t* ffn_sub_norm_w;
+    int8_t* q_packed;
+    float* q_ws;
+    int8_t* k_packed;
+    float* k_ws;
+    int8_t* v_packed;
+    float* v_ws;
+    int8_t* o_packed;
+    float* o_ws;
+    int8_t* gate_up_packed;
+    float* gate_up_ws;
+    int8_t* down_packed;
+    float* down_ws;
+} bitvla_lm_layer_hip;
+typedef struct bitvla_lm_hip_ctx bitvla_lm_hip_ctx;
+VLA_KAPI bitvla_lm_hip_ctx* bitvla_lm_hip_init(int hidden, int n_q, int n_kv, int head_dim, int ffn, int n_layers,
+                                               float rope_base, float rms_eps, int max_seq);
+VLA_KAPI void bitvla_lm_hip_free(bitvla_lm_hip_ctx* ctx);
+VLA_KAPI void bitvla_lm_hip_set_layer(bitvla_lm_hip_ctx* ctx, int L, const bitvla_lm_layer_hip* layer);
+VLA_KAPI void bitvla_lm_hip_set_output_norm(bitvla_lm_hip_ctx* ctx, const uint16_t* w);
+VLA_KAPI int bitvla_lm_hip_forward(bitvla_lm_hip_ctx* ctx, const uint16_t* d_in, uint16_t* d_out, int seq,
+                                   vla_stream_t stream);
+
 /* Library identification, for a loader that wants to check what it bound. */
 VLA_KAPI const char* vla_kernels_arch(void); /* "gfx950" */
 

@@ -337,3 +337,45 @@ def bitvla_chunk(cfg, w, obs, from_fp32=False):
     x = orc.linear(hf, w["act.W_out"], w["act.b_out"])
     x[:, cfg["real_action_dim"]:] = 0
     return x, acc0[0]
+
+
+def sqrelu_mul(gu, ffn):
+    """gate_up_fused_sqrelu_mul_bf16 (src/kernels/bitvla/bitvla_lm_cuda.cu:525-548): relu(gate)^2 * up
+    on a fused [seq, gate(ffn) | up(ffn)] projection, fp32 products, one rounding to bf16."""
+    gu = np.asarray(gu, np.float32)
+    g = np.maximum(gu[:, :ffn], np.float32(0))
+    return orc.round_bf16((g * g) * gu[:, ffn:2 * ffn])
+
+
+def bitvla_lm_forward(x, layers, out_norm, n_q, n_kv, D, eps, rope_base):
+    """bitvla_lm_cuda_forward (src/kernels/bitvla/bitvla_lm_cuda.cu:668-724): every layer of run_layer
+    (395-522) over all seq tokens, no mask, positions 0..seq-1, then the output RMSNorm.
+
+    x [seq, hidden] (bf16 values); layers: dicts with attn_norm, sub_norm, ffn_norm, ffn_sub_norm
+    (fp32 vectors of bf16 values) and q, k, v, o, gate_up, down = (ternary int8 [N, K], scales) with one
+    scale per tensor, two for gate_up.  Every stored intermediate is rounded to bf16 as the kernels
+    store it; scores and softmax are exact (the reference keeps bf16 scores between two GEMMs)."""
+    rb = orc.round_bf16
+    seq = x.shape[0]
+    cos_t, sin_t = orc.rope_tables(np.arange(seq, dtype=np.int32), D, rope_base)
+    scale = 1.0 / math.sqrt(D)
+
+    def bitlinear(x_bf, tw):
+        t, ws = tw
+        q, s = orc.act_quant(x_bf)
+        return orc.from_bf16(orc.ternary_epilogue(orc.ternary_gemm_i32(q, t), s, np.asarray(ws, np.float32)))
+
+    h = rb(x)
+    for w in layers:
+        hn = rb(orc.rms_norm(h, w["attn_norm"], eps))
+        q = bitlinear(hn, w["q"]).reshape(seq, n_q, D)
+        k = bitlinear(hn, w["k"]).reshape(seq, n_kv, D)
+        v = bitlinear(hn, w["v"]).reshape(seq, n_kv, D)
+        q, k = rb(orc.rope_neox(q, cos_t, sin_t)), rb(orc.rope_neox(k, cos_t, sin_t))
+        att = rb(orc.attention(q, k, v, None, scale)).reshape(seq, n_q * D)
+        h = rb(h + bitlinear(rb(orc.rms_norm(att, w["sub_norm"], eps)), w["o"]))
+        gu = bitlinear(rb(orc.rms_norm(h, w["ffn_norm"], eps)), w["gate_up"])
+        ffn = gu.shape[1] // 2
+        act = sqrelu_mul(gu, ffn)
+        h = rb(h + bitlinear(rb(orc.rms_norm(act, w["ffn_sub_norm"], eps)), w["down"]))
+    return rb(orc.rms_norm(h, out_norm, eps))

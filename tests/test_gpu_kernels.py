@@ -845,6 +845,86 @@ def test_ternary_pipeline_matches_cpu_twin():
     assert bf16_close(got, want) and rel_err(got, want) < 5e-3
 
 
+# ------------------------------------------------------- BitVLA LM context
+class _LmLayer(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in (
+        "attn_norm_w", "attn_sub_norm_w", "ffn_norm_w", "ffn_sub_norm_w", "q_packed", "q_ws", "k_packed", "k_ws", "v_packed",
+        "v_ws", "o_packed", "o_ws", "gate_up_packed", "gate_up_ws", "down_packed", "down_ws")]
+
+
+def test_bitvla_lm_context_forward_follows_the_oracle():
+    # init / set_layer / set_output_norm / forward / free with the reference's argument meaning:
+    # two full layers (attention and squared-ReLU GLU halves) over 37 tokens against the CPU
+    # restatement of run_layer; plus the error returns (sequence too long, unbound layer).
+    import oracle.chunk as orc_chunk
+    lib = pkg.lib()
+    H, n_q, n_kv, D, F, L, seq, eps, base = 256, 4, 2, 64, 384, 2, 37, 1e-5, 500000.0
+    r = np.random.default_rng(0xB17)
+    keep, layers_o = [], []
+
+    def tern(N, K, n_ws):
+        t = r.choice(np.int8([-1, 0, 0, 1]), (N, K))
+        ws = (0.02 + 0.01 * r.random(n_ws)).astype(np.float32)
+        dp, dws = dev(_pack_plain(t)), dev(ws)
+        keep.extend([dp, dws])
+        return (t, ws), dp.data_ptr(), dws.data_ptr()
+
+    def norm(K):
+        wv = orc.to_bf16((1 + 0.1 * r.standard_normal(K)).astype(np.float32))
+        d = dev(wv)
+        keep.append(d)
+        return orc.from_bf16(wv), d.data_ptr()
+
+    assert lib.bitvla_lm_hip_init(H, n_q, n_kv, D, F, L, base, eps, 0) is None        # no sequence
+    assert lib.bitvla_lm_hip_init(200, n_q, n_kv, D, F, L, base, eps, 48) is None      # K not a multiple of 128
+    ctx = lib.bitvla_lm_hip_init(H, n_q, n_kv, D, F, L, base, eps, 48)
+    assert ctx
+    x = orc.to_bf16(r.standard_normal((seq, H)).astype(np.float32))
+    d_in, d_out = dev(x), torch.zeros((seq, H), dtype=torch.int16, device="cuda")
+    on_o, on_p = norm(H)
+    lib.bitvla_lm_hip_set_output_norm(ctx, on_p)
+    assert lib.bitvla_lm_hip_forward(ctx, d_in.data_ptr(), d_out.data_ptr(), seq, None) == -1   # layers not bound
+    for l in range(L):
+        st, lo = _LmLayer(), {}
+        for name, K in (("attn_norm", H), ("sub_norm", n_q * D), ("ffn_norm", H), ("ffn_sub_norm", F)):
+            lo[name], p = norm(K)
+            setattr(st, {"sub_norm": "attn_sub_norm_w"}.get(name, name + "_w"), p)
+        for name, N, K, n_ws in (("q", n_q * D, H, 1), ("k", n_kv * D, H, 1), ("v", n_kv * D, H, 1), ("o", H, n_q * D, 1),
+                                 ("gate_up", 2 * F, H, 2), ("down", H, F, 1)):
+            lo[name], pp, pw = tern(N, K, n_ws)
+            setattr(st, name + "_packed", pp)
+            setattr(st, name + "_ws", pw)
+        lib.bitvla_lm_hip_set_layer(ctx, l, ctypes.byref(st))
+        layers_o.append(lo)
+    assert lib.bitvla_lm_hip_forward(ctx, d_in.data_ptr(), d_out.data_ptr(), 49, None) == -1    # longer than max_seq
+    assert lib.bitvla_lm_hip_forward(ctx, d_in.data_ptr(), d_out.data_ptr(), seq, None) == 0
+    sync()
+    got = orc.from_bf16(host(d_out, np.uint16))
+    want = orc_chunk.bitvla_lm_forward(orc.from_bf16(x), layers_o, on_o, n_q, n_kv, D, eps, base)
+    # a one-ulp difference before a quantisation can flip an int8 code, so a few elements may sit
+    # outside the per-element bar; the bulk and the worst case are both bounded
+    bad = np.abs(got - want) > 1e-2 + 2e-2 * np.abs(want)
+    assert bad.mean() < 5e-3 and rel_err(got, want) < 3e-2, (bad.mean(), rel_err(got, want))
+    # a second forward on a shorter sequence reuses the workspace
+    assert lib.bitvla_lm_hip_forward(ctx, d_in.data_ptr(), d_out.data_ptr(), 5, None) == 0
+    sync()
+    want5 = orc_chunk.bitvla_lm_forward(orc.from_bf16(x[:5]), layers_o, on_o, n_q, n_kv, D, eps, base)
+    assert rel_err(orc.from_bf16(host(d_out, np.uint16))[:5], want5) < 3e-2
+    lib.bitvla_lm_hip_free(ctx)
+    lib.bitvla_lm_hip_free(None)
+
+
+def test_gate_up_squared_relu_bit_exact():
+    import oracle.chunk as orc_chunk
+    r = np.random.default_rng(77)
+    for seq, ffn in ((5, 384), (3, 20)):   # vector and scalar paths
+        gu = orc.to_bf16((r.standard_normal((seq, 2 * ffn)) * 3).astype(np.float32))
+        out = torch.zeros((seq, ffn), dtype=torch.int16, device="cuda")
+        pkg.call("gate_up_fused_sqrelu_mul_bf16", dev(gu), out, seq, ffn)
+        sync()
+        assert np.array_equal(host(out, np.uint16), orc.to_bf16(orc_chunk.sqrelu_mul(orc.from_bf16(gu), ffn)))
+
+
 # ------------------------------------------------------- BitVLA layer helpers
 def test_bitvla_layout_helpers_and_softmax():
     r = np.random.default_rng(110)

@@ -442,3 +442,11 @@ def test_layout_helpers():
     assert np.array_equal(rep, np.repeat(t[:2], 3, axis=0))  # kv_h = q_h * n_kv / n_q
     ids = np.int32([3, 3, 0, 6])
     assert np.array_equal(orc.gather_rows(x, ids), x[ids])
+
+
+def test_squared_relu_glu_hand_values():
+    # relu(gate)^2 * up on [gate | up]: negative gates give 0 whatever up is; 1.5^2 * -2 = -4.5;
+    # the product is rounded to bf16 once (3^2 * 1.0078125 = 9.0703125 -> 9.0625)
+    import oracle.chunk as orc_chunk
+    gu = np.float32([[-1.0, 1.5, 3.0, 0.0, 7.0, -2.0, 1.0078125, 5.0]])
+    assert list(orc_chunk.sqrelu_mul(gu, 4)[0]) == [0.0, -4.5, 9.0625, 0.0]

@@ -62,6 +62,12 @@ KERNEL_API = {
     "bitvla_rope_neox_bf16": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "bitvla_softmax_scaled_bf16": [_vp, _f, _i, _i, _vp],
     "bitvla_add_bf16": [_vp, _vp, _vp, _i, _vp],
+    "gate_up_fused_sqrelu_mul_bf16": [_vp, _vp, _i, _i, _vp],
+    "bitvla_lm_hip_init": [_i, _i, _i, _i, _i, _i, _f, _f, _i],
+    "bitvla_lm_hip_free": [_vp],
+    "bitvla_lm_hip_set_layer": [_vp, _i, _vp],
+    "bitvla_lm_hip_set_output_norm": [_vp, _vp],
+    "bitvla_lm_hip_forward": [_vp, _vp, _vp, _i, _vp],
     "bitvla_repeat_kv_bf16": [_vp, _vp, _i, _i, _i, _i, _vp],
     "bitvla_transpose_sNhd_to_NshHd_bf16": [_vp, _vp, _i, _i, _i, _vp],
     "bitvla_transpose_NshHd_to_sNhd_bf16": [_vp, _vp, _i, _i, _i, _vp],
@@ -71,7 +77,9 @@ KERNEL_API = {
     "bitlinear_int8xint2": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "vla_kernels_arch": [],
 }
-_RESTYPES = {"vla_kernels_arch": ctypes.c_char_p, "vla_ternary_packed_words": ctypes.c_long}
+_RESTYPES = {"vla_kernels_arch": ctypes.c_char_p, "vla_ternary_packed_words": ctypes.c_long,
+             "bitvla_lm_hip_init": ctypes.c_void_p, "bitvla_lm_hip_free": None, "bitvla_lm_hip_set_layer": None,
+             "bitvla_lm_hip_set_output_norm": None}
 
 
 def tern_word_index(n, w, K):

@@ -408,6 +408,39 @@ __global__ void softmax_scaled_bf16_kernel(bf16_t* __restrict__ inout, float sca
     for (int i = threadIdx.x; i < S; i += blockDim.x) r[i] = f2bf(expf(bf2f(r[i]) * scale - mx) * inv);
 }
 
+// BitNet FFN activation on a fused [gate | up] projection (gate_up_fused_sqrelu_mul_bf16,
+// src/kernels/bitvla/bitvla_lm_cuda.cu:525-548): out[s][k] = relu(gate)^2 * up, rounded once.
+// One thread per 8 columns when ffn allows 16-byte accesses.
+__global__ void sqrelu_mul_bf16_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int ffn, long total8) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total8) return;
+    const int per_row = ffn / 8;
+    const long s = i / per_row;
+    const int k = (int)(i % per_row) * 8;
+    const u32x4_t g = *reinterpret_cast<const u32x4_t*>(gu + s * 2 * ffn + k);
+    const u32x4_t u = *reinterpret_cast<const u32x4_t*>(gu + s * 2 * ffn + ffn + k);
+    u32x4_t o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        float g0 = __uint_as_float(g[e] << 16), g1 = __uint_as_float(g[e] & 0xffff0000u);
+        const float u0 = __uint_as_float(u[e] << 16), u1 = __uint_as_float(u[e] & 0xffff0000u);
+        if (g0 < 0.f) g0 = 0.f;
+        if (g1 < 0.f) g1 = 0.f;
+        o[e] = (uint32_t)f2bf(g0 * g0 * u0) | ((uint32_t)f2bf(g1 * g1 * u1) << 16);
+    }
+    *reinterpret_cast<u32x4_t*>(out + s * ffn + k) = o;
+}
+__global__ void sqrelu_mul_bf16_scalar_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int ffn, long total) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const long s = i / ffn;
+    const int k = (int)(i % ffn);
+    float g = bf2f(gu[s * 2 * ffn + k]);
+    const float u = bf2f(gu[s * 2 * ffn + ffn + k]);
+    if (g < 0.f) g = 0.f;
+    out[i] = f2bf(g * g * u);
+}
+
 __global__ void add_bf16_kernel(const bf16_t* a, const bf16_t* b, bf16_t* out, int N) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < N) out[i] = f2bf(bf2f(a[i]) + bf2f(b[i]));
@@ -760,6 +793,17 @@ int bitvla_add_bf16(const uint16_t* a, const uint16_t* b, uint16_t* out, int N, 
     if (!a || !b || !out || N < 0) return VLA_K_ERR_ARG;
     if (N == 0) return VLA_K_OK;
     add_bf16_kernel<<<(N + 255) / 256, 256, 0, (hipStream_t)stream>>>(a, b, out, N);
+    return VLA_CHECK_LAUNCH();
+}
+
+int gate_up_fused_sqrelu_mul_bf16(const uint16_t* gu, uint16_t* out, int seq, int ffn, vla_stream_t stream) {
+    if (!gu || !out || seq < 0 || ffn <= 0) return VLA_K_ERR_ARG;
+    if (seq == 0) return VLA_K_OK;
+    const long total = (long)seq * ffn;
+    if (ffn % 8 == 0 && !(((uintptr_t)gu | (uintptr_t)out) & 15))
+        sqrelu_mul_bf16_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, (hipStream_t)stream>>>(gu, out, ffn, total / 8);
+    else
+        sqrelu_mul_bf16_scalar_kernel<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(gu, out, ffn, total);
     return VLA_CHECK_LAUNCH();
 }
 
