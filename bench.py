@@ -52,6 +52,7 @@ def workloads():
         "whole_gr00t_n1d6_32dit_bf16_b64": dict(cfg=dict(ck.gr00t_n1d6_config(32), ffn_dim=6144), B=64, views=2),
         "cfg4_bitvla_30layer_b1": dict(cfg=ck.bitvla_config(30), B=1, views=1),
         "cfg4_bitvla_30layer_b8": dict(cfg=ck.bitvla_config(30), B=8, views=1),
+        "whole_bitvla_30layer_b8": dict(cfg=dict(ck.bitvla_config(30), ffn_dim=6912), B=8, views=1),
     }
 
 
@@ -172,6 +173,23 @@ def kernel_breakdown(pkg, cfg, B, P):
         add("ternary_o_gemv_add", lambda i: pkg.call("vla_ternary_gemm_add", q8, wo, h, h, s, rs, ws, 1, M, H, H),
             0 if fused else L, "hbm", H * H // 4 + M * H + 4 * M * H)
         add("final_rms_norm", lambda i: pkg.call("bitvla_rmsnorm_bf16", h, w1, hn, 1e-5, M, H), 1, "hbm", 2 * M * H * 2)
+        F = cfg.get("ffn_dim", 0)
+        if F > 0:  # the squared-ReLU GLU half of every layer
+            wgu = torch.randint(0, 2 ** 31 - 1, (2 * F, H // 16), dtype=torch.int32, device=dev)
+            wd = torch.randint(0, 2 ** 31 - 1, (H, F // 16), dtype=torch.int32, device=dev)
+            gu, actv, wf = rnd(M, 2 * F), rnd(M, F), rnd(F)
+            q8f = z(M, F, dtype=torch.int8)
+            if fused:
+                add("norm_quant_ternary_gate_up_gemv", lambda i: pkg.call("vla_rmsnorm_ternary_gemv", h, w1, 1e-5, wgu, gu, None, ws, 2,
+                                                                          M, 2 * F, H), L, "hbm", 2 * F * H // 4 + 2 * M * H + 4 * M * F)
+            else:
+                add("ternary_gate_up_gemm", lambda i: pkg.call("vla_ternary_gemm", q8, wgu, gu, None, s, rs, ws, 2, M, 2 * F, H), L,
+                    "hbm", 2 * F * H // 4 + M * H + 4 * M * F)
+            add("sqrelu_mul", lambda i: pkg.call("gate_up_fused_sqrelu_mul_bf16", gu, actv, M, F), L, "hbm", 6 * M * F)
+            add("ffn_subnorm_act_quant", lambda i: pkg.call("vla_rmsnorm_act_quant_bf16", actv, wf, q8f, s, rs, 1e-5, M, F), L, "hbm",
+                3 * M * F)
+            add("ternary_down_gemv_add", lambda i: pkg.call("vla_ternary_gemm_add", q8f, wd, h, h, s, rs, ws, 1, M, H, F), L, "hbm",
+                H * F // 4 + M * F + 4 * M * H)
         # the prefill-shaped fused QKV GEMM (one launch per layer per observation batch)
         Mp = B * P
         q8p, sp, rsp = z(Mp, H, dtype=torch.int8), torch.ones(Mp, device=dev), z(Mp, dtype=torch.int32)

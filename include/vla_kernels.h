@@ -285,10 +285,17 @@ VLA_KAPI int vla_ternary_gemm_add(const int8_t* A, const uint32_t* W_packed, uin
  * rows, scales and row sums kept on chip (run_layer's attn_norm + QKV and sub_norm + O
  * pairs, bitvla_lm_cuda.cu:421-486, at S = 1).  Same bits as the two calls.  out may alias
  * residual, never x (every workgroup reads whole rows of x while others write out).
- * VLA_K_ERR_SHAPE when M > 8, K > 4096 or K % 128: callers fall back to the pair. */
+ * VLA_K_ERR_SHAPE when M > 8, K > 7168 or K % 128: callers fall back to the pair. */
 VLA_KAPI int vla_rmsnorm_ternary_gemv(const uint16_t* x, const uint16_t* norm_w, float eps, const uint32_t* W_packed,
                                       uint16_t* out, const uint16_t* residual, const float* ws, int ws_num, int M,
                                       int N, int K, vla_stream_t stream);
+/* The same with x formed on the fly from a fused [M][gate(K) | up(K)] projection,
+ * x = bf16(relu(gate)^2 * up): gate_up_fused_sqrelu_mul_bf16 -> ffn sub-norm -> act_quant ->
+ * down projection (+ residual) of run_layer (bitvla_lm_cuda.cu:503-520) in one launch, same
+ * bits as those calls. */
+VLA_KAPI int vla_sqrelu_rmsnorm_ternary_gemv(const uint16_t* gate_up, const uint16_t* norm_w, float eps,
+                                             const uint32_t* W_packed, uint16_t* out, const uint16_t* residual,
+                                             const float* ws, int ws_num, int M, int N, int K, vla_stream_t stream);
 
 /* The same launch for the fused Q | K | V projection of one appended token per batch row,
  * with vla_qkv_split_rope_append (S = 1) in its epilogue: Q rotated to q_out [batch][Hq][D],

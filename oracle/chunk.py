@@ -264,8 +264,8 @@ def bitvla_ternary(cfg, w, name, from_fp32):
     """(ternary int8 [N,K], per-row-group scales expanded to ws groups) as the loader derives them."""
     kvd = cfg["n_kv_heads"] * cfg["head_dim"]
     t = w[name + ".t"]
-    parts = [cfg["hidden"], kvd, kvd] if name.endswith("Wqkv") else [t.shape[0]]
-    group = kvd if name.endswith("Wqkv") else t.shape[0]
+    parts = [cfg["hidden"], kvd, kvd] if name.endswith("Wqkv") else ([t.shape[0] // 2] * 2 if name.endswith("Wgu") else [t.shape[0]])
+    group = kvd if name.endswith("Wqkv") else parts[0]
     if from_fp32:
         scales, row, tt = [], 0, np.empty_like(t)
         for n, s in zip(parts, w[name + ".ws"]):
@@ -286,7 +286,9 @@ def bitvla_chunk(cfg, w, obs, from_fp32=False):
 
     One layer = run_layer's attention half (src/kernels/bitvla/bitvla_lm_cuda.cu:422-486):
     bf16 rmsnorm -> act-quant -> ternary GEMM (int32, bf16 out) -> RoPE(Q,K) ->
-    attention -> bf16 sub-norm -> act-quant -> ternary O GEMM -> bf16 add.
+    attention -> bf16 sub-norm -> act-quant -> ternary O GEMM -> bf16 add; with cfg["ffn_dim"]
+    also its squared-ReLU GLU half (488-520): ffn norm -> act-quant -> fused gate|up GEMM ->
+    relu(gate)^2 * up -> ffn sub-norm -> act-quant -> down GEMM -> bf16 add.
     Returns (actions [n_act, A], int32 accumulators of layer 0's QKV GEMM over the prefix).
     """
     L, Hq, Hkv, D, H = cfg["n_layers"], cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["hidden"]
@@ -296,6 +298,9 @@ def bitvla_chunk(cfg, w, obs, from_fp32=False):
     rb = orc.round_bf16
     tern = [(bitvla_ternary(cfg, w, "lm.%d.Wqkv" % l, from_fp32), bitvla_ternary(cfg, w, "lm.%d.Wo" % l, from_fp32))
             for l in range(L)]
+    F = cfg.get("ffn_dim", 0)
+    tern_ffn = [(bitvla_ternary(cfg, w, "lm.%d.Wgu" % l, from_fp32), bitvla_ternary(cfg, w, "lm.%d.Wd" % l, from_fp32))
+                for l in range(L)] if F > 0 else None
     cos_t, sin_t = orc.rope_tables(np.arange(P + n_act, dtype=np.int32), D, cfg["rope_freq_base"])
     cacheK, cacheV = [None] * L, [None] * L
     acc0 = [None]
@@ -324,6 +329,11 @@ def bitvla_chunk(cfg, w, obs, from_fp32=False):
             sub = rb(orc.rms_norm(att, w["lm.%d.sub_norm" % l], eps))
             o = bitlinear(sub, to, wso)
             h = rb(h + o)
+            if F > 0:
+                (tg, wsg), (td, wsd) = tern_ffn[l]
+                gu = bitlinear(rb(orc.rms_norm(h, w["lm.%d.ffn_norm" % l], eps)), tg, wsg)
+                act = sqrelu_mul(gu, F)
+                h = rb(h + bitlinear(rb(orc.rms_norm(act, w["lm.%d.ffn_sub_norm" % l], eps)), td, wsd))
         return h
 
     emb = np.concatenate([np.asarray(obs["img_emb"], np.float32).reshape(cfg["n_img"], H),

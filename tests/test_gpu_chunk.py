@@ -240,9 +240,13 @@ def test_gr00t_n1d6_alternating_text_and_image_cross_layers(tmp_path, n_layers, 
     m.close()
 
 
-@pytest.mark.parametrize("from_fp32", [False, True])
-def test_config4_bitvla_ternary_append(tmp_path, from_fp32):
+@pytest.mark.parametrize("from_fp32,ffn_dim", [(False, 0), (True, 0), (False, 768), (True, 6912)])
+def test_config4_bitvla_ternary_append(tmp_path, from_fp32, ffn_dim):
+    # ffn_dim > 0: the layers also run their squared-ReLU GLU half (768: the down projection of
+    # the decode rows takes the one-launch norm + GEMV; 6912, the model's width: the two-launch pair)
     cfg = ckpt.bitvla_config(n_layers=2)
+    if ffn_dim:
+        cfg["ffn_dim"] = ffn_dim
     w = ckpt.synth_weights(cfg, seed=0x5EED + 5)
     r = np.random.default_rng(250)
     obs = [make_obs(cfg, r, n_views=1) for _ in range(2)]
@@ -250,7 +254,14 @@ def test_config4_bitvla_ternary_append(tmp_path, from_fp32):
     got = m.predict_batch(obs).reshape(2, 7, 32)
     for b in range(2):
         want, _ = orc_chunk.bitvla_chunk(cfg, w, obs[b], from_fp32=from_fp32)
-        assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+        if ffn_dim == 0:
+            assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+        else:
+            # Two more quantisations and a squaring per layer: when 1 % of its bf16 inputs change
+            # by one ulp the oracle itself moves by 0.03 (max) at width 768 and by 0.05 (max),
+            # 0.013-0.015 (mean) at width 6912, outputs up to 2.9, so the per-element bar does
+            # not apply; the distance to the oracle stays at that scale.
+            assert rel_err(got[b], want) < 3e-2 and np.abs(got[b] - want).mean() < 2e-2, np.abs(got[b] - want).max()
     m.close()
 
 

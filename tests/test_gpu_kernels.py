@@ -721,7 +721,7 @@ def test_ternary_gemm_add_matches_gemm_then_add(monkeypatch, M, N, K, tile):
     assert np.array_equal(host(fused), host(want))
 
 
-@pytest.mark.parametrize("M,K", [(8, 2560), (37, 720), (4, 4096), (300, 2560), (129, 720), (70, 4096)])
+@pytest.mark.parametrize("M,K", [(8, 2560), (37, 720), (4, 4096), (300, 2560), (129, 720), (70, 4096), (9, 6912), (3, 16384)])
 def test_rmsnorm_act_quant_fused_is_the_pair(M, K):
     r = np.random.default_rng(K + M)
     x = orc.to_bf16((r.standard_normal((M, K)) * 3).astype(np.float32))
@@ -734,12 +734,21 @@ def test_rmsnorm_act_quant_fused_is_the_pair(M, K):
     pkg.call("vla_act_quant_bf16", hn, q1, s1, r1, M, K)
     pkg.call("vla_rmsnorm_act_quant_bf16", dev(x), dev(w), q2, s2, r2, 1e-5, M, K)
     sync()
-    assert torch.equal(q1, q2) and torch.equal(s1, s2) and torch.equal(r1, r2)
+    if K <= 4096:  # longer rows: the two paths sum the squares in different orders, so only the oracle check below applies
+        assert torch.equal(q1, q2) and torch.equal(s1, s2) and torch.equal(r1, r2)
+    assert np.array_equal(host(r2), host(q2).astype(np.int32).sum(1))
     # and the pair follows the oracle
     n = orc.round_bf16(orc.rms_norm(orc.from_bf16(x), orc.from_bf16(w), 1e-5))
     qo, so = orc.act_quant(n)
     assert np.mean(host(q2) != qo) < 2e-3 and np.allclose(host(s2), so, rtol=1e-2)
     assert pkg.lib().vla_rmsnorm_act_quant_bf16(0, 0, 0, 0, 0, ctypes.c_float(1e-5), 1, 8, 0) == pkg.VLA_K_ERR_ARG
+    # a norm weight that is not 16-byte aligned takes element loads: same bits
+    wpad = torch.zeros(K + 8, dtype=torch.int16, device="cuda")
+    wpad[1:K + 1] = dev(w)
+    q3, s3, r3 = torch.zeros_like(q1), torch.zeros_like(s1), torch.zeros_like(r1)
+    pkg.call("vla_rmsnorm_act_quant_bf16", dev(x), wpad[1:K + 1], q3, s3, r3, 1e-5, M, K)
+    sync()
+    assert torch.equal(q3, q2) and torch.equal(s3, s2) and torch.equal(r3, r2)
 
 
 @pytest.mark.parametrize("M,N,K,ws_num", [(1, 3840, 2560, 3), (8, 3840, 2560, 3), (8, 2560, 2560, 1), (3, 48, 128, 3),
@@ -811,6 +820,34 @@ def test_rmsnorm_ternary_gemv_rope_append_one_launch_is_the_chain(B, Hq, Hkv, D,
     assert bad(4, 4, 2, 2, 32, 128, 0) == pkg.VLA_K_ERR_SHAPE      # scale group of 48 columns cuts a head
     assert bad(1, 4, 2, 2, 32, 128, 64) == pkg.VLA_K_ERR_SHAPE     # slot past the cache
     assert bad(1, 0, 2, 2, 32, 128, 0) == pkg.VLA_K_OK
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 2560, 6912), (1, 2560, 6912), (5, 96, 768), (3, 64, 4096)])
+def test_sqrelu_rmsnorm_ternary_gemv_one_launch_is_the_chain(M, N, K):
+    # The FFN's second half on decode rows: relu(gate)^2 * up -> sub-norm -> quantisation -> down
+    # projection + residual in one launch against the three stand-alone launches; and the long
+    # rows alone (no activation) through vla_rmsnorm_ternary_gemv.
+    r = np.random.default_rng(13 * M + K)
+    t = r.integers(-1, 2, (N, K)).astype(np.int8)
+    ws = np.float32([0.017])
+    w = orc.to_bf16((1 + 0.1 * r.standard_normal(K)).astype(np.float32))
+    gu = orc.to_bf16((r.standard_normal((M, 2 * K)) * 1.5).astype(np.float32))
+    res = orc.to_bf16(r.standard_normal((M, N)).astype(np.float32))
+    dW, dws, dw, dgu = dev(_pack_plain(t)), dev(ws), dev(w), dev(gu)
+    act = torch.zeros((M, K), dtype=torch.int16, device="cuda")
+    q, sc, rs = (torch.zeros((M, K), dtype=torch.int8, device="cuda"), torch.zeros(M, device="cuda"),
+                 torch.zeros(M, dtype=torch.int32, device="cuda"))
+    pkg.call("gate_up_fused_sqrelu_mul_bf16", dgu, act, M, K)
+    pkg.call("vla_rmsnorm_act_quant_bf16", act, dw, q, sc, rs, 1e-5, M, K)
+    want = dev(res)
+    pkg.call("vla_ternary_gemm_add", q, dW, want, want, sc, rs, dws, 1, M, N, K)
+    got, got2 = dev(res), dev(res)
+    pkg.call("vla_sqrelu_rmsnorm_ternary_gemv", dgu, dw, 1e-5, dW, got, got, dws, 1, M, N, K)
+    pkg.call("vla_rmsnorm_ternary_gemv", act, dw, 1e-5, dW, got2, got2, dws, 1, M, N, K)
+    sync()
+    assert torch.equal(got, want) and torch.equal(got2, want)
+    assert pkg.lib().vla_sqrelu_rmsnorm_ternary_gemv(dgu.data_ptr(), dw.data_ptr(), ctypes.c_float(1e-5), dW.data_ptr(),
+                                                     got.data_ptr(), 0, dws.data_ptr(), 1, 9, N, K, 0) == pkg.VLA_K_ERR_SHAPE
 
 
 def test_rmsnorm_ternary_gemv_rejects_what_it_cannot_hold():

@@ -154,6 +154,14 @@ def synth_weights(cfg, seed=0x5EED):
             w[p + "Wqkv.ws"] = (0.02 * np.sqrt(2 / np.pi) * r.uniform(0.9, 1.1, 3)).astype(np.float32)
             w[p + "Wo.t"] = r.choice(np.int8([-1, 0, 0, 1]), size=(H, qd)).astype(np.int8)
             w[p + "Wo.ws"] = (0.02 * np.sqrt(2 / np.pi) * r.uniform(0.9, 1.1, 1)).astype(np.float32)
+            F = cfg.get("ffn_dim", 0)
+            if F > 0:  # the squared-ReLU GLU half of run_layer (bitvla_lm_cuda.cu:488-520): [gate; up] rows, down
+                w[p + "ffn_norm"] = bf16_round((1.0 + 0.05 * r.standard_normal(H)).astype(np.float32))
+                w[p + "ffn_sub_norm"] = bf16_round((1.0 + 0.05 * r.standard_normal(F)).astype(np.float32))
+                w[p + "Wgu.t"] = r.choice(np.int8([-1, 0, 0, 1]), size=(2 * F, H)).astype(np.int8)
+                w[p + "Wgu.ws"] = (0.02 * np.sqrt(2 / np.pi) * r.uniform(0.9, 1.1, 2)).astype(np.float32)
+                w[p + "Wd.t"] = r.choice(np.int8([-1, 0, 0, 1]), size=(H, F)).astype(np.int8)
+                w[p + "Wd.ws"] = (0.02 * np.sqrt(2 / np.pi) * r.uniform(0.9, 1.1, 1)).astype(np.float32)
         return w
     W = cfg["expert_h"]
     if cfg.get("vocab", 0) > 0:
@@ -264,7 +272,7 @@ def write_synthetic(path, cfg, weights, ladder_pack=None, plain_pack=None):
             continue
         small = name.startswith(_F32_NAMES) or name.endswith((".bqkv", ".bq", ".bo", ".bkv", ".adaln_b", ".b1", ".b2", ".ada_in_w", ".ada_in_b",
                                                             ".ada_post_w", ".ada_post_b"))
-        if cfg["arch"] == "bitvla" and name.endswith(("attn_norm", "sub_norm")):
+        if cfg["arch"] == "bitvla" and name.endswith(("attn_norm", "sub_norm", "ffn_norm")):
             out[name] = BF16(t)
         elif bf and not small:
             out[name] = BF16(t)
@@ -277,7 +285,7 @@ def write_synthetic(path, cfg, weights, ladder_pack=None, plain_pack=None):
 
 def _dequant_sources(cfg, base, t, ws):
     kvd = cfg["n_kv_heads"] * cfg["head_dim"]
-    parts = [cfg["hidden"], kvd, kvd] if base.endswith("Wqkv") else [t.shape[0]]
+    parts = [cfg["hidden"], kvd, kvd] if base.endswith("Wqkv") else ([t.shape[0] // 2] * 2 if base.endswith("Wgu") else [t.shape[0]])
     out = np.empty(t.shape, np.float32)
     row = 0
     for n, s in zip(parts, ws):

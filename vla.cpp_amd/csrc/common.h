@@ -95,55 +95,84 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // scale is 127 / max(amax, 1e-5); q = clamp(round-half-even(y * scale)).  The int8 row goes
 // to qrow (global or LDS, 8 bytes per vector); scale and the sum of the row's int8 values
 // are returned in every lane.  K % 8 == 0 and K <= 512 NV.
-template <int NV>
+// GLU: the row is formed on the fly from a fused projection, x[k] = bf16(relu(gate[k])^2 * up[k])
+// with gate = xr and up = xr + K (gate_up_fused_sqrelu_mul_bf16, src/kernels/bitvla/bitvla_lm_cuda.cu:525-548).
+template <int NV, bool GLU = false>
 __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr, const bf16_t* __restrict__ w, int K,
                                                   float eps, int lane, int8_t* qrow, float& scale_out, int& sum_out) {
     const int nvec = K / 8;
-    float v[NV][8];
+    // Every value kept between the passes is a bf16 (the input, then the rounded normalised
+    // row), so the row stays packed: 4 registers per 16-byte vector.
+    u32x4_t xp[NV];
     u32x4_t wraw[NV];  // the weight's vectors, requested with the row's so that one round trip covers both
     const bool w_vec = w && !((uintptr_t)w & 15);
+    auto lo = [](uint32_t u) { return __uint_as_float(u << 16); };
+    auto hi = [](uint32_t u) { return __uint_as_float(u & 0xffff0000u); };
+    float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int vec = lane + 64 * i;
-        u32x4_t raw = {0u, 0u, 0u, 0u};
+        u32x4_t raw = {0u, 0u, 0u, 0u}, upr = {0u, 0u, 0u, 0u};
         wraw[i] = raw;
         if (vec < nvec) {
             raw = *reinterpret_cast<const u32x4_t*>(xr + (long)vec * 8);
+            if (GLU) upr = *reinterpret_cast<const u32x4_t*>(xr + K + (long)vec * 8);
             if (w_vec) wraw[i] = *reinterpret_cast<const u32x4_t*>(w + (long)vec * 8);
         }
+        if (GLU) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[i][e] = __uint_as_float((e & 1) ? (raw[e >> 1] & 0xffff0000u) : (raw[e >> 1] << 16));
+            for (int e = 0; e < 4; ++e) {
+                float g0 = lo(raw[e]), g1 = hi(raw[e]);
+                if (g0 < 0.f) g0 = 0.f;
+                if (g1 < 0.f) g1 = 0.f;
+                raw[e] = pack_bf2(g0 * g0 * lo(upr[e]), g1 * g1 * hi(upr[e]));
+            }
+        }
+        xp[i] = raw;
     }
-    float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) ss += v[i][e] * v[i][e];
+        for (int e = 0; e < 4; ++e) {
+            const float a = lo(xp[i][e]), b = hi(xp[i][e]);
+            ss += a * a;
+            ss += b * b;
+        }
     const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
+    // the packed words are opaque from here on, or the compiler keeps the first pass's unpacked
+    // floats alive across the reduction (8 registers per vector instead of 4)
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) asm volatile("" : "+v"(xp[i][e]));
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int vec = lane + 64 * i;
         if (vec >= nvec) continue;
         const int k0 = vec * 8;
-        float o[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            o[e] = v[i][e] * inv;
-            if (w_vec) o[e] *= __uint_as_float((e & 1) ? (wraw[i][e >> 1] & 0xffff0000u) : (wraw[i][e >> 1] << 16));
-            else if (w) o[e] *= bf2f(w[k0 + e]);
-        }
-#pragma unroll
-        for (int e = 0; e < 8; e += 2) {  // the activation as the bf16 it would be stored as
-            const uint32_t pr = pack_bf2(o[e], o[e + 1]);
-            v[i][e] = __uint_as_float(pr << 16);
-            v[i][e + 1] = __uint_as_float(pr & 0xffff0000u);
-            amax = fmaxf(amax, fmaxf(fabsf(v[i][e]), fabsf(v[i][e + 1])));
+        for (int e = 0; e < 4; ++e) {
+            float o0 = lo(xp[i][e]) * inv, o1 = hi(xp[i][e]) * inv;
+            if (w_vec) {
+                o0 *= lo(wraw[i][e]);
+                o1 *= hi(wraw[i][e]);
+            } else if (w) {
+                o0 *= bf2f(w[k0 + 2 * e]);
+                o1 *= bf2f(w[k0 + 2 * e + 1]);
+            }
+            const uint32_t pr = pack_bf2(o0, o1);  // the activation as the bf16 it would be stored as
+            xp[i][e] = pr;
+            amax = fmaxf(amax, fmaxf(fabsf(lo(pr)), fabsf(hi(pr))));
         }
     }
     amax = wave_max(amax);
     if (amax < 1e-5f) amax = 1e-5f;
     const float scale = 127.0f / amax;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) asm volatile("" : "+v"(xp[i][e]));
     int sum = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
@@ -152,7 +181,8 @@ __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr,
         uint32_t pk[2] = {0u, 0u};
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            float qf = rintf(v[i][e] * scale);
+            const uint32_t u = xp[i][e >> 1];
+            float qf = rintf(((e & 1) ? hi(u) : lo(u)) * scale);
             qf = fminf(fmaxf(qf, -128.0f), 127.0f);
             pk[e >> 2] |= (uint32_t)((int)qf & 0xff) << (8 * (e & 3));
         }

@@ -276,7 +276,12 @@ bool launch_row_norm(const void* x, const void* w, const float* sc, const float*
     if (nvec <= 64 * 2) VLA_ROW_NORM(2);
     else if (nvec <= 64 * 4) VLA_ROW_NORM(4);
     else if (nvec <= 64 * 8) VLA_ROW_NORM(8);
-    else return false;
+    else if constexpr (MODE == NORM_RMS_AQ && sizeof(T) == 2) {  // the 6912-wide BitNet FFN rows
+        if (nvec > 64 * 16) return false;
+        VLA_ROW_NORM(16);
+    } else {
+        return false;
+    }
 #undef VLA_ROW_NORM
     return true;
 }
@@ -757,7 +762,8 @@ int vla_rmsnorm_act_quant_bf16(const uint16_t* x, const uint16_t* w, int8_t* out
     if (M == 0) return VLA_K_OK;
     if (launch_row_norm<bf16_t, NORM_RMS_AQ>(x, w, nullptr, nullptr, nullptr, out, scales, rowsum, M, K, eps, (hipStream_t)stream))
         return VLA_CHECK_LAUNCH();
-    const int th = row_threads(K);
+    int th = row_threads(K);
+    while (K > th * RNAQ_MAX_PER_THREAD && th < 1024) th *= 2;  // long rows (the 6912-wide BitNet FFN): up to 16 wavefronts
     if (K > th * RNAQ_MAX_PER_THREAD) return VLA_K_ERR_SHAPE;
     rmsnorm_act_quant_kernel<<<M, th, 0, (hipStream_t)stream>>>(x, w, out, scales, rowsum, K, eps);
     return VLA_CHECK_LAUNCH();

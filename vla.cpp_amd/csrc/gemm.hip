@@ -1115,12 +1115,16 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_kernel(GemmArgs 
 // columns every 32-row block holds 16 rotation pairs, d in lanes 0-15 and d + D/2 in lanes
 // 16-31, so a pair meets through one shuffle.  The projection is rounded to bf16 before the
 // rotation, as the stand-alone chain stores it.
-constexpr int GEMV_FUSED_MAX_K = 4096;
-template <int MAXG, int NV, bool ROPE>
+//
+// GLU: A is a fused [gate | up] projection of 2 K columns and the rows are relu(gate)^2 * up
+// (the FFN's sub-norm -> down projection step, bitvla_lm_cuda.cu:505-517).
+constexpr int GEMV_FUSED_MAX_K = 7168;
+template <int MAXG, int NV, bool ROPE, bool GLU = false>
 __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(GemmArgs a) {
     // int8 rows (stride K + 32 bytes: eight rows' 16-byte fragments fall on distinct banks),
     // later the partial accumulator tiles
-    constexpr int kPartBytes = GEMV_WAVES * 32 * 33 * 4, kRowBytes = GEMV_WAVES * (GEMV_FUSED_MAX_K + 32);
+    constexpr int KMAX = NV * 512 < GEMV_FUSED_MAX_K ? NV * 512 : GEMV_FUSED_MAX_K;
+    constexpr int kPartBytes = GEMV_WAVES * 32 * 33 * 4, kRowBytes = GEMV_WAVES * (KMAX + 32);
     __shared__ __align__(16) unsigned char smem[kPartBytes > kRowBytes ? kPartBytes : kRowBytes];
     __shared__ float s_sh[GEMV_WAVES];
     __shared__ int rs_sh[GEMV_WAVES];
@@ -1140,8 +1144,8 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
     if (wave < a.M) {  // uniform per wavefront
         float scale;
         int sum;
-        rms_act_quant_row<NV>((const bf16_t*)a.A + (long)wave * a.K, (const bf16_t*)a.norm_w, a.K, a.norm_eps, lane,
-                              (int8_t*)smem + wave * stride, scale, sum);
+        rms_act_quant_row<NV, GLU>((const bf16_t*)a.A + (long)wave * a.K * (GLU ? 2 : 1), (const bf16_t*)a.norm_w, a.K,
+                                   a.norm_eps, lane, (int8_t*)smem + wave * stride, scale, sum);
         if (lane == 0) {
             s_sh[wave] = scale;
             rs_sh[wave] = sum;
@@ -1356,18 +1360,21 @@ __global__ void rowsum_i8_kernel(const int8_t* __restrict__ A, int32_t* __restri
 int32_t* g_rowsum = nullptr;
 int g_rowsum_cap = 0;
 
-template <bool ROPE>
+template <bool ROPE, bool GLU = false>
 int launch_gemv_norm(const GemmArgs& a, vla_stream_t stream) {
     const unsigned grid = (unsigned)((a.N + 31) / 32);
     const int groups = (a.K / 32 + GEMV_WAVES - 1) / GEMV_WAVES, nvec = a.K / 8;
     hipStream_t st = (hipStream_t)stream;
-#define VLA_GEMV_NORM(G, NV) ternary_gemv_norm_kernel<G, NV, ROPE><<<grid, GEMV_WAVES * 64, 0, st>>>(a)
+#define VLA_GEMV_NORM(G, NV) ternary_gemv_norm_kernel<G, NV, ROPE, GLU><<<grid, GEMV_WAVES * 64, 0, st>>>(a)
     if (groups <= 10) {
         if (nvec <= 128) VLA_GEMV_NORM(10, 2);
         else if (nvec <= 256) VLA_GEMV_NORM(10, 4);
         else VLA_GEMV_NORM(10, 8);
-    } else {
+    } else if (groups <= 16) {
         VLA_GEMV_NORM(16, 8);
+    } else {
+        if constexpr (ROPE) return VLA_K_ERR_SHAPE;  // the QKV projection's K is the model width, never that long
+        else VLA_GEMV_NORM(28, 16);
     }
 #undef VLA_GEMV_NORM
     return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
@@ -1574,6 +1581,18 @@ int vla_rmsnorm_ternary_gemv(const uint16_t* x, const uint16_t* norm_w, float ep
     return launch_gemv_norm<false>(a, stream);
 }
 
+int vla_sqrelu_rmsnorm_ternary_gemv(const uint16_t* gate_up, const uint16_t* norm_w, float eps, const uint32_t* W_packed,
+                                    uint16_t* out, const uint16_t* residual, const float* ws, int ws_num, int M, int N, int K,
+                                    vla_stream_t stream) {
+    if (!gate_up || !W_packed || !out || !ws || ws_num <= 0 || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (M > GEMV_WAVES || K > GEMV_FUSED_MAX_K || K % 128 || N % ws_num || (((uintptr_t)gate_up) & 15)) return VLA_K_ERR_SHAPE;
+    if (M == 0) return VLA_K_OK;
+    GemmArgs a = {};
+    a.A = gate_up; a.norm_w = norm_w; a.norm_eps = eps; a.W = W_packed; a.M = M; a.N = N; a.K = K;
+    a.Y = out; a.residual = residual; a.ws = ws; a.ws_num = ws_num;
+    return launch_gemv_norm<false, true>(a, stream);
+}
+
 int vla_rmsnorm_ternary_gemv_rope_append(const uint16_t* x, const uint16_t* norm_w, float eps, const uint32_t* W_paired,
                                          const float* ws, int ws_num, const float* cos_row, const float* sin_row,
                                          uint16_t* q_out, uint16_t* k_cache, uint16_t* vt_cache, int batch, int n_q_heads,
@@ -1583,7 +1602,7 @@ int vla_rmsnorm_ternary_gemv_rope_append(const uint16_t* x, const uint16_t* norm
         n_q_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || K <= 0)
         return VLA_K_ERR_ARG;
     const int N = (n_q_heads + 2 * n_kv_heads) * head_dim;
-    if (batch > GEMV_WAVES || K > GEMV_FUSED_MAX_K || K % 128 || head_dim % 32 || N % ws_num || (N / ws_num) % head_dim ||
+    if (batch > GEMV_WAVES || K > 4096 || K % 128 || head_dim % 32 || N % ws_num || (N / ws_num) % head_dim ||
         tok_offset < 0 || tok_offset >= t_max || (((uintptr_t)x) & 15))
         return VLA_K_ERR_SHAPE;
     if (batch == 0) return VLA_K_OK;

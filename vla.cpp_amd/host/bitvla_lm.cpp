@@ -88,6 +88,8 @@ TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::
 struct LmLayer {
     DevBuf attn_norm, sub_norm;
     TernaryW Wqkv, Wo;
+    DevBuf ffn_norm, ffn_sub_norm;  // the GLU half, present when the checkpoint carries ffn_dim
+    TernaryW Wgu, Wd;
     KVLayer kv;
 };
 
@@ -107,13 +109,13 @@ class BitvlaLm : public ModelArch {
     uint32_t alloc_gen_ = 0;
     DevBuf zeros_;
     void run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys);
-    int L_, Hq_, Hkv_, D_, H_, A_, n_act_, n_img_, n_lang_, vocab_, P_ = 0, B_ = 0;
+    int L_, Hq_, Hkv_, D_, H_, A_, n_act_, n_img_, n_lang_, vocab_, F_ = 0, P_ = 0, B_ = 0;
     float eps_;
     std::vector<LmLayer> layers_;
     std::vector<float> E_lang_, act_emb_;
     DevBuf out_norm_, W_out_, b_out_;
     RopeTable rope_;
-    DevBuf h_, hn_, q8_, s_, rowsum_, qkv_, q_, att_, o_, emb_bcast_, hfin_, x_;
+    DevBuf h_, hn_, q8_, s_, rowsum_, qkv_, q_, att_, o_, emb_bcast_, hfin_, x_, gu_, act_;
     hipStream_t last_stream_ = nullptr;
 };
 
@@ -129,6 +131,8 @@ BitvlaLm::BitvlaLm(const Checkpoint& ck) {
     n_lang_ = (int)ck.i64("n_lang");
     vocab_ = (int)ck.i64("vocab");
     eps_ = (float)ck.f64("rms_eps", 1e-5);
+    F_ = (int)ck.i64("ffn_dim", 0);
+    if (F_ % 128) throw std::runtime_error("vla(bitvla): ffn_dim must be a multiple of 128");
     if (Hq_ * D_ != H_) throw std::runtime_error("vla(bitvla): n_q_heads * head_dim must equal hidden");
     cfg.n_img = n_img_; cfg.n_lang = n_lang_; cfg.n_prefix = n_img_ + n_lang_; cfg.n_suffix = n_act_;
     cfg.n_full = cfg.n_prefix + n_act_;
@@ -155,6 +159,13 @@ BitvlaLm::BitvlaLm(const Checkpoint& ck) {
         upload_as(w.sub_norm, s.data(), s.size(), VLA_DT_BF16);
         w.Wqkv = load_ternary(ck, p + "Wqkv", {H_, kvd, kvd}, H_, kvd, Hq_, Hkv_, D_);
         w.Wo = load_ternary(ck, p + "Wo", {H_}, H_, H_);
+        if (F_ > 0) {
+            std::vector<float> fn = ck.f32(p + "ffn_norm"), fs = ck.f32(p + "ffn_sub_norm");
+            upload_as(w.ffn_norm, fn.data(), fn.size(), VLA_DT_BF16);
+            upload_as(w.ffn_sub_norm, fs.data(), fs.size(), VLA_DT_BF16);
+            w.Wgu = load_ternary(ck, p + "Wgu", {F_, F_}, H_, F_);
+            w.Wd = load_ternary(ck, p + "Wd", {H_}, F_, H_);
+        }
     }
 }
 
@@ -176,7 +187,8 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
             w.kv.create(VLA_DT_BF16, B, Hkv_, D_, t_max);
             w.kv.n_prefix = P;
         }
-        h_.alloc(M * H_ * 2); hn_.alloc(M * H_ * 2); q8_.alloc(M * H_); s_.alloc(M * 4); rowsum_.alloc(M * 4);
+        h_.alloc(M * H_ * 2); hn_.alloc(M * H_ * 2); q8_.alloc(M * (size_t)(F_ > H_ ? F_ : H_)); s_.alloc(M * 4); rowsum_.alloc(M * 4);
+        if (F_ > 0) { gu_.alloc(M * 2 * F_ * 2); act_.alloc(M * F_ * 2); }
         qkv_.alloc(M * (H_ + 2 * Hkv_ * D_) * 2); q_.alloc(M * H_ * 2); att_.alloc(M * H_ * 2); o_.alloc(M * H_ * 2);
         hfin_.alloc((size_t)n_act_ * B * H_ * 2);
         x_.alloc((size_t)n_act_ * B * A_ * 4);
@@ -251,6 +263,30 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
                                              rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
             VLA_K(vla_ternary_gemm_add(q8_.as<int8_t>(), w.Wo.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
                                        s_.as<float>(), rowsum_.as<int32_t>(), w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_,
+                                       C.stream));
+        }
+        if (F_ == 0) continue;
+        // the GLU half: ffn norm -> [gate | up] -> relu(gate)^2 * up -> sub-norm -> down + residual
+        if (fused) {
+            VLA_K(vla_rmsnorm_ternary_gemv(h_.as<uint16_t>(), w.ffn_norm.as<uint16_t>(), eps_, w.Wgu.packed.as<uint32_t>(),
+                                           gu_.as<uint16_t>(), nullptr, w.Wgu.ws.as<float>(), w.Wgu.ws_num, M, 2 * F_, H_,
+                                           C.stream));
+        } else {
+            VLA_K(vla_rmsnorm_act_quant_bf16(h_.as<uint16_t>(), w.ffn_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
+                                             rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
+            VLA_K(vla_ternary_gemm(q8_.as<int8_t>(), w.Wgu.packed.as<uint32_t>(), gu_.as<uint16_t>(), nullptr, s_.as<float>(),
+                                   rowsum_.as<int32_t>(), w.Wgu.ws.as<float>(), w.Wgu.ws_num, M, 2 * F_, H_, C.stream));
+        }
+        if (fused && F_ <= 7168) {  // activation, sub-norm, quantisation and down projection in one launch
+            VLA_K(vla_sqrelu_rmsnorm_ternary_gemv(gu_.as<uint16_t>(), w.ffn_sub_norm.as<uint16_t>(), eps_,
+                                                  w.Wd.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
+                                                  w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_, C.stream));
+        } else {
+            VLA_K(gate_up_fused_sqrelu_mul_bf16(gu_.as<uint16_t>(), act_.as<uint16_t>(), M, F_, C.stream));
+            VLA_K(vla_rmsnorm_act_quant_bf16(act_.as<uint16_t>(), w.ffn_sub_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
+                                             rowsum_.as<int32_t>(), eps_, M, F_, C.stream));
+            VLA_K(vla_ternary_gemm_add(q8_.as<int8_t>(), w.Wd.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
+                                       s_.as<float>(), rowsum_.as<int32_t>(), w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_,
                                        C.stream));
         }
     }
