@@ -185,11 +185,17 @@ def kernel_breakdown(pkg, cfg, B, P):
             else:
                 add("ternary_gate_up_gemm", lambda i: pkg.call("vla_ternary_gemm", q8, wgu, gu, None, s, rs, ws, 2, M, 2 * F, H), L,
                     "hbm", 2 * F * H // 4 + M * H + 4 * M * F)
-            add("sqrelu_mul", lambda i: pkg.call("gate_up_fused_sqrelu_mul_bf16", gu, actv, M, F), L, "hbm", 6 * M * F)
-            add("ffn_subnorm_act_quant", lambda i: pkg.call("vla_rmsnorm_act_quant_bf16", actv, wf, q8f, s, rs, 1e-5, M, F), L, "hbm",
-                3 * M * F)
-            add("ternary_down_gemv_add", lambda i: pkg.call("vla_ternary_gemm_add", q8f, wd, h, h, s, rs, ws, 1, M, H, F), L, "hbm",
-                H * F // 4 + M * F + 4 * M * H)
+            one = fused and F <= 4096  # activation, sub-norm, quantisation and down projection in one launch
+            add("sqrelu_norm_quant_ternary_down_gemv_add",
+                lambda i: pkg.call("vla_sqrelu_rmsnorm_ternary_gemv", gu, wf, 1e-5, wd, h, h, ws, 1, M, H, F), L if one else 0, "hbm",
+                H * F // 4 + 4 * M * F + 4 * M * H)
+            add("sqrelu_norm_act_quant", lambda i: pkg.call("vla_sqrelu_rmsnorm_act_quant_bf16", gu, wf, q8f, s, rs, 1e-5, M, F),
+                0 if one else L, "hbm", 5 * M * F)
+            add("sqrelu_mul", lambda i: pkg.call("gate_up_fused_sqrelu_mul_bf16", gu, actv, M, F), 0, "hbm", 6 * M * F)
+            add("ffn_subnorm_act_quant", lambda i: pkg.call("vla_rmsnorm_act_quant_bf16", actv, wf, q8f, s, rs, 1e-5, M, F),
+                0, "hbm", 3 * M * F)
+            add("ternary_down_gemv_add", lambda i: pkg.call("vla_ternary_gemm_add", q8f, wd, h, h, s, rs, ws, 1, M, H, F),
+                0 if one else L, "hbm", H * F // 4 + M * F + 4 * M * H)
         # the prefill-shaped fused QKV GEMM (one launch per layer per observation batch)
         Mp = B * P
         q8p, sp, rsp = z(Mp, H, dtype=torch.int8), torch.ones(Mp, device=dev), z(Mp, dtype=torch.int32)

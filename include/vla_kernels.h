@@ -245,9 +245,16 @@ VLA_KAPI int vla_act_quant_bf16(const uint16_t* in, int8_t* out, float* scales, 
 /* bitvla_rmsnorm_bf16 followed by vla_act_quant_bf16 in one launch (the pair that opens
  * both halves of run_layer, src/kernels/bitvla/bitvla_lm_cuda.cu:422-486); the bf16
  * intermediate is not written.  int8 rows, scales and row sums are bit-identical to the
- * two separate calls.  K <= 4096. */
+ * two separate calls for K <= 4096 (longer rows add the squares in another order). */
 VLA_KAPI int vla_rmsnorm_act_quant_bf16(const uint16_t* x, const uint16_t* w, int8_t* out, float* scales,
                                         int32_t* rowsum, float eps, int M, int K, vla_stream_t stream);
+/* The same on rows formed on the fly from a fused [M][gate(K) | up(K)] projection,
+ * x = bf16(relu(gate)^2 * up): gate_up_fused_sqrelu_mul_bf16 -> ffn sub-norm -> act_quant of
+ * run_layer (bitvla_lm_cuda.cu:503-513) in one launch, same bits as those calls; the
+ * activation is not written.  VLA_K_ERR_SHAPE when K % 8, K > 8192 or a buffer is not
+ * 16-byte aligned: callers fall back to the separate calls. */
+VLA_KAPI int vla_sqrelu_rmsnorm_act_quant_bf16(const uint16_t* gate_up, const uint16_t* w, int8_t* out, float* scales,
+                                               int32_t* rowsum, float eps, int M, int K, vla_stream_t stream);
 
 /* Ternary weight quantisation on the host (recover_ternary_and_scale,
  * src/models/bitvla.cpp:430-451). */

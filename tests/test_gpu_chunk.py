@@ -243,7 +243,7 @@ def test_gr00t_n1d6_alternating_text_and_image_cross_layers(tmp_path, n_layers, 
 @pytest.mark.parametrize("from_fp32,ffn_dim", [(False, 0), (True, 0), (False, 768), (True, 6912)])
 def test_config4_bitvla_ternary_append(tmp_path, from_fp32, ffn_dim):
     # ffn_dim > 0: the layers also run their squared-ReLU GLU half (768: the down projection of
-    # the decode rows takes the one-launch norm + GEMV; 6912, the model's width: the two-launch pair)
+    # the decode rows takes the one-launch activation + norm + GEMV; 6912, the model's width: activation + norm + quantisation in one launch, then the GEMV)
     cfg = ckpt.bitvla_config(n_layers=2)
     if ffn_dim:
         cfg["ffn_dim"] = ffn_dim

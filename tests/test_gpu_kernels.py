@@ -850,6 +850,32 @@ def test_sqrelu_rmsnorm_ternary_gemv_one_launch_is_the_chain(M, N, K):
                                                      got.data_ptr(), 0, dws.data_ptr(), 1, 9, N, K, 0) == pkg.VLA_K_ERR_SHAPE
 
 
+@pytest.mark.parametrize("M,K", [(8, 6912), (300, 6912), (5, 768), (37, 4096), (2, 8192)])
+def test_sqrelu_rmsnorm_act_quant_one_launch_is_the_pair(M, K):
+    # relu(gate)^2 * up -> sub-norm -> quantisation in one launch (the activation never written)
+    # against gate_up_fused_sqrelu_mul_bf16 followed by vla_rmsnorm_act_quant_bf16: same bits.
+    r = np.random.default_rng(7 * M + K)
+    gu = dev(orc.to_bf16((r.standard_normal((M, 2 * K)) * 1.5).astype(np.float32)))
+    w = dev(orc.to_bf16((1 + 0.1 * r.standard_normal(K)).astype(np.float32)))
+    act = torch.zeros((M, K), dtype=torch.int16, device="cuda")
+    q1, s1, r1 = (torch.zeros((M, K), dtype=torch.int8, device="cuda"), torch.zeros(M, device="cuda"),
+                  torch.zeros(M, dtype=torch.int32, device="cuda"))
+    q2, s2, r2 = torch.zeros_like(q1), torch.zeros_like(s1), torch.zeros_like(r1)
+    pkg.call("gate_up_fused_sqrelu_mul_bf16", gu, act, M, K)
+    pkg.call("vla_rmsnorm_act_quant_bf16", act, w, q1, s1, r1, 1e-5, M, K)
+    pkg.call("vla_sqrelu_rmsnorm_act_quant_bf16", gu, w, q2, s2, r2, 1e-5, M, K)
+    sync()
+    assert torch.equal(q1, q2) and torch.equal(s1, s2) and torch.equal(r1, r2)
+    assert np.array_equal(host(r2), host(q2).astype(np.int32).sum(1))
+    lib, f = pkg.lib(), ctypes.c_float(1e-5)
+    p = [t.data_ptr() for t in (gu, w, q2, s2, r2)]
+    assert lib.vla_sqrelu_rmsnorm_act_quant_bf16(0, p[1], p[2], p[3], p[4], f, M, K, 0) == pkg.VLA_K_ERR_ARG
+    assert lib.vla_sqrelu_rmsnorm_act_quant_bf16(p[0], p[1], p[2], p[3], p[4], f, 1, 8200, 0) == pkg.VLA_K_ERR_SHAPE
+    assert lib.vla_sqrelu_rmsnorm_act_quant_bf16(p[0], p[1], p[2], p[3], p[4], f, 1, 100, 0) == pkg.VLA_K_ERR_SHAPE
+    assert lib.vla_sqrelu_rmsnorm_act_quant_bf16(p[0] + 2, p[1], p[2], p[3], p[4], f, 1, 64, 0) == pkg.VLA_K_ERR_SHAPE
+    assert lib.vla_sqrelu_rmsnorm_act_quant_bf16(p[0], p[1], p[2], p[3], p[4], f, 0, K, 0) == pkg.VLA_K_OK
+
+
 def test_rmsnorm_ternary_gemv_rejects_what_it_cannot_hold():
     lib, f = pkg.lib(), ctypes.c_float(1e-5)
     buf = torch.zeros(16 * 8192, dtype=torch.int16, device="cuda")

@@ -54,6 +54,7 @@ KERNEL_API = {
     "vla_ternary_gemm": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "vla_ternary_gemm_add": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "vla_rmsnorm_act_quant_bf16": [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _vp],
+    "vla_sqrelu_rmsnorm_act_quant_bf16": [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _vp],
     "vla_rmsnorm_ternary_gemv": [_vp, _vp, _f, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "vla_sqrelu_rmsnorm_ternary_gemv": [_vp, _vp, _f, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "vla_rmsnorm_ternary_gemv_rope_append": [_vp, _vp, _f, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i,

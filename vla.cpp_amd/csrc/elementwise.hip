@@ -139,7 +139,7 @@ __global__ void adaln_kernel(const T* __restrict__ x, const float* __restrict__ 
 // as it would be stored, quantised per row to int8 (scale 127 / max(amax, 1e-5), round half
 // even) with its row sum -- bitvla_rmsnorm_bf16 followed by act_quant without the round trip.
 enum { NORM_RMS = 0, NORM_ADALN = 1, NORM_RMS_AQ = 2, NORM_ADARMS = 3 };  // ADARMS: RMS statistics, then (1 + scale), shift
-template <typename T, int NV, int MODE>
+template <typename T, int NV, int MODE, bool GLU = false>
 __global__ void __launch_bounds__(256) row_norm_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                        const float* __restrict__ sc, const float* __restrict__ sh,
                                                        T* __restrict__ y, int8_t* __restrict__ q, float* __restrict__ scales,
@@ -150,7 +150,9 @@ __global__ void __launch_bounds__(256) row_norm_kernel(const T* __restrict__ x, 
     if constexpr (MODE == NORM_RMS_AQ && sizeof(T) == 2) {
         float scale;
         int sum;
-        rms_act_quant_row<NV>((const bf16_t*)x + (long)row * K, (const bf16_t*)w, K, eps, lane, q + (long)row * K, scale, sum);
+        // GLU: x holds [gate(K) | up(K)] rows and the row normalised is relu(gate)^2 * up
+        rms_act_quant_row<NV, GLU>((const bf16_t*)x + (long)row * K * (GLU ? 2 : 1), (const bf16_t*)w, K, eps, lane,
+                                   q + (long)row * K, scale, sum);
         if (lane == 0) {
             scales[row] = scale;
             if (rowsum) rowsum[row] = sum;
@@ -264,7 +266,7 @@ __global__ void __launch_bounds__(256) row_norm_kernel(const T* __restrict__ x, 
 // 16-byte accesses; returns false otherwise (the callers fall back to the scalar kernels).
 // The choice depends on the row length only, never on the number of rows, so an
 // observation's result does not depend on the batch it is run in.
-template <typename T, int MODE>
+template <typename T, int MODE, bool GLU = false>
 bool launch_row_norm(const void* x, const void* w, const float* sc, const float* sh, void* y, int8_t* q, float* scales,
                      int32_t* rowsum, int M, int K, float eps, hipStream_t st) {
     constexpr int EPV = 16 / sizeof(T);
@@ -272,7 +274,7 @@ bool launch_row_norm(const void* x, const void* w, const float* sc, const float*
     if (MODE == NORM_RMS_AQ && (K % 8)) return false;
     const int nvec = K / EPV, blocks = (M + 3) / 4;
 #define VLA_ROW_NORM(NV) \
-    row_norm_kernel<T, NV, MODE><<<blocks, 256, 0, st>>>((const T*)x, (const T*)w, sc, sh, (T*)y, q, scales, rowsum, M, K, eps)
+    row_norm_kernel<T, NV, MODE, GLU><<<blocks, 256, 0, st>>>((const T*)x, (const T*)w, sc, sh, (T*)y, q, scales, rowsum, M, K, eps)
     if (nvec <= 64 * 2) VLA_ROW_NORM(2);
     else if (nvec <= 64 * 4) VLA_ROW_NORM(4);
     else if (nvec <= 64 * 8) VLA_ROW_NORM(8);
@@ -766,6 +768,16 @@ int vla_rmsnorm_act_quant_bf16(const uint16_t* x, const uint16_t* w, int8_t* out
     while (K > th * RNAQ_MAX_PER_THREAD && th < 1024) th *= 2;  // long rows (the 6912-wide BitNet FFN): up to 16 wavefronts
     if (K > th * RNAQ_MAX_PER_THREAD) return VLA_K_ERR_SHAPE;
     rmsnorm_act_quant_kernel<<<M, th, 0, (hipStream_t)stream>>>(x, w, out, scales, rowsum, K, eps);
+    return VLA_CHECK_LAUNCH();
+}
+
+int vla_sqrelu_rmsnorm_act_quant_bf16(const uint16_t* gate_up, const uint16_t* w, int8_t* out, float* scales, int32_t* rowsum,
+                                      float eps, int M, int K, vla_stream_t stream) {
+    if (!gate_up || !out || !scales || M < 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (M == 0) return VLA_K_OK;
+    if (!launch_row_norm<bf16_t, NORM_RMS_AQ, true>(gate_up, w, nullptr, nullptr, nullptr, out, scales, rowsum, M, K, eps,
+                                                    (hipStream_t)stream))
+        return VLA_K_ERR_SHAPE;
     return VLA_CHECK_LAUNCH();
 }
 

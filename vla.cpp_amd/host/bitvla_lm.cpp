@@ -277,18 +277,26 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
             VLA_K(vla_ternary_gemm(q8_.as<int8_t>(), w.Wgu.packed.as<uint32_t>(), gu_.as<uint16_t>(), nullptr, s_.as<float>(),
                                    rowsum_.as<int32_t>(), w.Wgu.ws.as<float>(), w.Wgu.ws_num, M, 2 * F_, H_, C.stream));
         }
-        if (fused && F_ <= 7168) {  // activation, sub-norm, quantisation and down projection in one launch
+        if (fused && F_ <= 4096) {  // activation, sub-norm, quantisation and down projection in one launch
             VLA_K(vla_sqrelu_rmsnorm_ternary_gemv(gu_.as<uint16_t>(), w.ffn_sub_norm.as<uint16_t>(), eps_,
                                                   w.Wd.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
                                                   w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_, C.stream));
-        } else {
+            continue;
+        }
+        // Longer rows (the model's 6912): every 32-column workgroup of the one-launch form would
+        // repeat the rows' activation and norm, which costs more than a launch; the activation
+        // still stays on chip, inside the norm + quantisation launch.
+        const int rc = vla_sqrelu_rmsnorm_act_quant_bf16(gu_.as<uint16_t>(), w.ffn_sub_norm.as<uint16_t>(), q8_.as<int8_t>(),
+                                                         s_.as<float>(), rowsum_.as<int32_t>(), eps_, M, F_, C.stream);
+        if (rc != VLA_K_ERR_SHAPE) VLA_K(rc);
+        else {  // rows the one-wavefront kernel does not hold
             VLA_K(gate_up_fused_sqrelu_mul_bf16(gu_.as<uint16_t>(), act_.as<uint16_t>(), M, F_, C.stream));
             VLA_K(vla_rmsnorm_act_quant_bf16(act_.as<uint16_t>(), w.ffn_sub_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
                                              rowsum_.as<int32_t>(), eps_, M, F_, C.stream));
-            VLA_K(vla_ternary_gemm_add(q8_.as<int8_t>(), w.Wd.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
-                                       s_.as<float>(), rowsum_.as<int32_t>(), w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_,
-                                       C.stream));
         }
+        VLA_K(vla_ternary_gemm_add(q8_.as<int8_t>(), w.Wd.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
+                                   s_.as<float>(), rowsum_.as<int32_t>(), w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_,
+                                   C.stream));
     }
 }
 

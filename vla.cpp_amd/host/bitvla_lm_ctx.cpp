@@ -54,8 +54,13 @@ int run(bitvla_lm_hip_ctx* c, const uint16_t* d_in, uint16_t* d_out, int seq, hi
         VLA_K(vla_rmsnorm_act_quant_bf16(h, w.ffn_norm_w, q8, s, rs, c->rms_eps, seq, H, st));
         VLA_K(vla_ternary_gemm(q8, (const uint32_t*)w.gate_up_packed, c->gate_up.as<uint16_t>(), nullptr, s, rs, w.gate_up_ws, 2, seq,
                                2 * F, H, st));
-        VLA_K(gate_up_fused_sqrelu_mul_bf16(c->gate_up.as<uint16_t>(), c->act.as<uint16_t>(), seq, F, st));
-        VLA_K(vla_rmsnorm_act_quant_bf16(c->act.as<uint16_t>(), w.ffn_sub_norm_w, q8, s, rs, c->rms_eps, seq, F, st));
+        // activation, sub-norm and quantisation in one launch (same bits as the two below it)
+        const int rc = vla_sqrelu_rmsnorm_act_quant_bf16(c->gate_up.as<uint16_t>(), w.ffn_sub_norm_w, q8, s, rs, c->rms_eps, seq, F, st);
+        if (rc != VLA_K_ERR_SHAPE) VLA_K(rc);
+        else {
+            VLA_K(gate_up_fused_sqrelu_mul_bf16(c->gate_up.as<uint16_t>(), c->act.as<uint16_t>(), seq, F, st));
+            VLA_K(vla_rmsnorm_act_quant_bf16(c->act.as<uint16_t>(), w.ffn_sub_norm_w, q8, s, rs, c->rms_eps, seq, F, st));
+        }
         VLA_K(vla_ternary_gemm_add(q8, (const uint32_t*)w.down_packed, h, h, s, rs, w.down_ws, 1, seq, H, F, st));
     }
     VLA_K(bitvla_rmsnorm_bf16(h, c->out_norm, d_out, c->rms_eps, seq, H, st));
