@@ -491,6 +491,40 @@ def test_attention_direct_kernel_key_slices_merge(monkeypatch, split):
     assert np.isfinite(got).all() and bf16_close(got, want) and rel_err(got, want) < 1e-2
 
 
+@pytest.mark.parametrize("B,S,Hq,Hkv,T", [(8, 1, 20, 5, 519), (1, 1, 20, 5, 513), (3, 2, 8, 2, 519), (1, 1, 28, 4, 1000), (3, 2, 8, 2, 300), (2, 1, 4, 4, 97),
+                                          (8, 1, 20, 5, 33)])
+def test_attention_decode_slices_merged_by_the_last_to_arrive(monkeypatch, B, S, Hq, Hkv, T):
+    # 128-wide heads, a few rows per kv head (single-token decode): the keys are sliced over
+    # single-wavefront workgroups and the slice that arrives last merges them inside the launch.
+    # Same tolerance against the oracle as the one-workgroup form, repeatable bit for bit
+    # (the counters return to zero), and close to that form.
+    D, t_max = 128, (T + 15) // 16 * 16 + 16
+    r = np.random.default_rng(1000 * B + T)
+    Q = orc.round_bf16(r.standard_normal((B, S, Hq, D)).astype(np.float32))
+    K = orc.round_bf16(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    V = orc.round_bf16(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    kc = torch.full((B, Hkv, t_max, D), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
+    vc = torch.full((B, Hkv, D, t_max), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
+    pkg.call("vla_kv_append", kc, vc, to_dev(K, BF16), to_dev(V, BF16), BF16, B, Hkv, D, t_max, 0, T)
+    scale = 1.0 / np.sqrt(D)
+
+    def run():
+        out = empty((B, S, Hq * D), BF16)
+        pkg.call("vla_attn_prefix_suffix", to_dev(Q, BF16), kc, vc, out, pkg.VLA_DT_BF16_P2, B, S, Hq, Hkv, D, t_max, T, scale,
+                 pkg.VLA_MASK_NONE, T, 0, 0, None)
+        sync()
+        return as_f32(out, BF16)
+
+    got = [run() for _ in range(3)]
+    monkeypatch.setenv("VLA_ATTN_NO_ARRIVE", "1")
+    ref = run()
+    mask = np.zeros((S, T), np.float32)
+    want = np.stack([orc.attention(Q[b], K[b], V[b], mask, scale) for b in range(B)]).reshape(B, S, Hq * D)
+    assert np.isfinite(got[0]).all() and np.array_equal(got[0], got[1]) and np.array_equal(got[0], got[2])
+    assert bf16_close(got[0], want) and rel_err(got[0], want) < 1e-2
+    assert bf16_close(ref, want) and rel_err(got[0], ref) < 1e-2
+
+
 @pytest.mark.parametrize("B", [1, 4])
 def test_attention_wide_heads_key_slices_and_partial_formats(monkeypatch, B):
     # pi0's 256-wide MQA heads: with few workgroups the keys are walked in slices whose partial

@@ -65,6 +65,7 @@ struct AttnArgs {
     float* part_o;   // [pair][split][r_pad][D] fp32 unnormalised, or fp16 normalised (part_half)
     float* part_ml;  // [pair][split][r_pad][2]
     int part_half;   // partial outputs stored as o / l in fp16 (half the bytes; wide heads)
+    int* arrive;     // direct kernel: one counter per (pair, row block); the slice that arrives last merges (zero between launches)
 };
 
 // Key (within a 32-key block) held by score row x = 8j + 4h + i: 16(j/2) + 8h + 4(j%2) + i.
@@ -716,6 +717,96 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         }
 }
 
+// Key slices of one (pair, row block) as wavefronts of different workgroups, merged without a
+// second launch: every slice writes its unnormalised partial rows and (max, sum), then counts
+// itself in; the one that finds all others counted combines them and writes the output.  No
+// wavefront waits for another.  The partials cross between the per-XCD L2s as device-scope
+// relaxed atomic accesses (write-through stores, loads served from memory) and the count is
+// taken only after the wavefront's stores have been acknowledged, so neither side needs a
+// cache-wide write-back or invalidate.  The arithmetic order is fixed by the slice index, not
+// by who arrives last.  At most ARRIVE_MAX_T (row, slice) pairs per block, 128-wide heads.
+constexpr int ARRIVE_MAX_T = 48, ARRIVE_MAX_UNITS = 16384;
+__device__ __forceinline__ void st_dev64(float* p, float x, float y) {
+    const unsigned long long v = (unsigned long long)__float_as_uint(x) | ((unsigned long long)__float_as_uint(y) << 32);
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long ld_dev64(const float* p) {
+    return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void arrive_merge(const AttnArgs& a, const f32x16_t (&o)[4], float m_run, float l_run, int pair, int prb,
+                                             int split, int row, bool row_valid, int b, int hk, int grp, int R, int lane, int g) {
+    constexpr int D = 128;
+    if (row_valid) {
+        const long prow = ((long)pair * a.n_split + split) * a.r_pad + row;
+        if (g == 0) st_dev64(a.part_ml + prow * 2, m_run, l_run);
+        float* po = a.part_o + prow * D;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int d = db * 32 + 8 * j + 4 * g;
+                st_dev64(po + d, o[db][4 * j], o[db][4 * j + 1]);
+                st_dev64(po + d + 2, o[db][4 * j + 2], o[db][4 * j + 3]);
+            }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's partials are in memory before it is counted
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(a.arrive + prb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __builtin_amdgcn_readfirstlane(old);
+    if (old != a.n_split - 1) return;
+    if (lane == 0) __hip_atomic_store(a.arrive + prb, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+
+    // Lane t = rl * n_split + sp holds (max, sum) of row rl in slice sp, then its weight
+    // 2^(max - row max) and the reciprocal of the row's combined sum.
+    const int Rb = min(32, R);  // one row block only
+    const int T = Rb * a.n_split;
+    const long prow0 = (long)pair * a.n_split * a.r_pad;
+    float mt = -INFINITY, lt = 0.f;
+    if (lane < T) {
+        const unsigned long long v = ld_dev64(a.part_ml + (prow0 + (long)(lane % a.n_split) * a.r_pad + lane / a.n_split) * 2);
+        mt = __uint_as_float((uint32_t)v);
+        lt = __uint_as_float((uint32_t)(v >> 32));
+    }
+    unsigned long long pv[ARRIVE_MAX_T];
+    {
+        int lsp = 0, lrl = 0;  // slice and row of t, kept by counting (no divisions in the unrolled body)
+#pragma unroll
+        for (int t = 0; t < ARRIVE_MAX_T; ++t) {
+            pv[t] = 0ull;
+            if (t < T) pv[t] = ld_dev64(a.part_o + (prow0 + (long)lsp * a.r_pad + lrl) * D + lane * 2);
+            if (++lsp == a.n_split) {
+                lsp = 0;
+                ++lrl;
+            }
+        }
+    }
+    const int t0 = lane < T ? (lane / a.n_split) * a.n_split : 0;
+    float mrow = -INFINITY;
+    for (int sp = 0; sp < a.n_split; ++sp) mrow = fmaxf(mrow, __shfl(mt, t0 + sp, 64));
+    const float wt = (lane < T && mrow > -INFINITY) ? exp2f(mt - mrow) : 0.f;
+    float lrow = 0.f;
+    for (int sp = 0; sp < a.n_split; ++sp) lrow += __shfl(lt * wt, t0 + sp, 64);
+    const float inv = lrow > 0.f ? 1.0f / lrow : 0.f;
+    float a0 = 0.f, a1 = 0.f;
+    int sp = 0, rl = 0;
+#pragma unroll
+    for (int t = 0; t < ARRIVE_MAX_T; ++t) {
+        if (t < T) {  // uniform
+            const float w = __shfl(wt, t, 64);
+            a0 += __uint_as_float((uint32_t)pv[t]) * w;
+            a1 += __uint_as_float((uint32_t)(pv[t] >> 32)) * w;
+            if (++sp == a.n_split) {
+                const float iv = __shfl(inv, t, 64);
+                const int hh = hk * grp + rl / a.S, ss = rl % a.S;
+                reinterpret_cast<uint32_t*>((bf16_t*)a.out + (((long)b * a.S + ss) * a.Hq + hh) * D)[lane] = pack_bf2(a0 * iv, a1 * iv);
+                a0 = a1 = 0.f;
+                sp = 0;
+                ++rl;
+            }
+        }
+    }
+}
+
 // Few query rows per (batch, kv head) -- at most one 32-row tile: GR00T's 17 DiT tokens,
 // single-token decode.  Nothing is shared between wavefronts then, so K and V^T go straight
 // from the cache into MFMA operand registers (no LDS, no barriers): lane (g, r) of a
@@ -730,7 +821,7 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
     constexpr int NQ = D / CE, NDB = (D + 31) / 32;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int g = lane >> 5, r = lane & 31;
-    const int unit = MERGE ? blockIdx.x * a.n_split + wave : blockIdx.x * 4 + wave;
+    const int unit = MERGE ? blockIdx.x * a.n_split + wave : blockIdx.x * (int)(blockDim.x >> 6) + wave;
     const int prb = unit / a.n_split, split = unit % a.n_split;  // (pair, 32-row block) and key slice
     const int pair = prb / a.n_rblocks, rb = prb % a.n_rblocks;
     // whole wavefront (whole workgroup with MERGE); the main loop has no barriers
@@ -958,6 +1049,12 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
         }
         return;
     }
+    if constexpr (D == 128) {
+        if (a.arrive) {  // uniform over the launch
+            arrive_merge(a, o, m_run, l_run, pair, prb, split, row, row_valid, b, hk, grp, R, lane, g);
+            return;
+        }
+    }
     if (!row_valid) return;
     if (a.n_split > 1) {
         const long prow = ((long)pair * a.n_split + split) * a.r_pad + row;
@@ -1010,6 +1107,21 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
 // run the shape once before capturing it).
 float* g_ws = nullptr;
 size_t g_ws_floats = 0;
+
+// Arrival counters of the direct kernel's in-launch merge: allocated and zeroed once, left at
+// zero by every launch that uses them.  Launches that overlap on the device must not share
+// them (nor the partial workspace): one attention launch at a time per process.
+int* g_arrive = nullptr;
+int* arrive_counters() {
+    if (!g_arrive) {
+        if (hipMalloc((void**)&g_arrive, ARRIVE_MAX_UNITS * sizeof(int)) != hipSuccess) return g_arrive = nullptr;
+        if (hipMemset(g_arrive, 0, ARRIVE_MAX_UNITS * sizeof(int)) != hipSuccess) {
+            (void)hipFree(g_arrive);
+            return g_arrive = nullptr;
+        }
+    }
+    return g_arrive;
+}
 
 float* workspace(size_t floats) {
     if (floats > g_ws_floats) {
@@ -1098,7 +1210,21 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
     // when few enough; with fewer than 32 pairs more slices go through global partials and
     // the merge kernel instead.
     constexpr int MERGE_MAX = D <= 64 ? 8 : 4;  // wide heads need the registers of a 4-wavefront workgroup
-    const bool wg_merge = n_split > 1 && (n_split <= MERGE_MAX || n_units >= 32);
+    bool wg_merge = n_split > 1 && (n_split <= MERGE_MAX || n_units >= 32);
+    // 128-wide heads with few rows (single-token decode): more slices than one workgroup holds,
+    // as single-wavefront workgroups over more CUs, merged by the slice that arrives last.
+    // Slices of three blocks there: each slice costs the merging wavefront a row of loads, and the
+    // hand-over is three dependent trips to memory whatever the count (519 keys, batch 8: six
+    // slices 13.6 us, nine 14.7 us, one workgroup of four 13.5 us alone and 1.4 us slower in sequence).
+    const int Rb = R < 32 ? R : 32;
+    int n_arrive = n_split < (nb_total + 2) / 3 || getenv("VLA_ATTN_SPLIT") ? n_split : (nb_total + 2) / 3;
+    if (n_arrive * Rb > ARRIVE_MAX_T) n_arrive = ARRIVE_MAX_T / Rb;
+    bool arrive = D == 128 && n_arrive > MERGE_MAX && a.n_rblocks == 1 && n_units <= ARRIVE_MAX_UNITS &&
+                  !getenv("VLA_ATTN_NO_ARRIVE") && arrive_counters();
+    if (arrive) {
+        n_split = n_arrive;
+        wg_merge = false;
+    }
     if (wg_merge && n_split > MERGE_MAX) n_split = MERGE_MAX;
     a.tiles_per_split = (nb_total + n_split - 1) / n_split;
     a.n_split = (nb_total + a.tiles_per_split - 1) / a.tiles_per_split;
@@ -1119,11 +1245,14 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
         a.part_o = ws;
         a.part_ml = ws + rows * D;
     }
-    const unsigned grid = (unsigned)(((long)n_units * a.n_split + 3) / 4);
-    if (a.p2) attn_direct_kernel<D, true, ST, false><<<grid, 256, 0, st>>>(a);
-    else attn_direct_kernel<D, false, ST, false><<<grid, 256, 0, st>>>(a);
+    arrive = arrive && a.n_split > 1 && a.n_split * Rb <= ARRIVE_MAX_T;
+    a.arrive = arrive ? g_arrive : nullptr;
+    const int wgw = arrive ? 1 : 4;  // wavefronts per workgroup
+    const unsigned grid = (unsigned)(((long)n_units * a.n_split + wgw - 1) / wgw);
+    if (a.p2) attn_direct_kernel<D, true, ST, false><<<grid, wgw * 64, 0, st>>>(a);
+    else attn_direct_kernel<D, false, ST, false><<<grid, wgw * 64, 0, st>>>(a);
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
-    if (a.n_split > 1) {
+    if (a.n_split > 1 && !arrive) {
         attn_merge_kernel<bf16_t, false><<<(unsigned)(((long)n_pairs * R + 3) / 4), 256, 0, st>>>(a.part_o, a.part_ml, (bf16_t*)a.out,
                                                                                            n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq,
                                                                                            a.Hkv, D);
