@@ -317,6 +317,7 @@ MEASURED_TRAFFIC_BYTES = {
     ("cfg1_smolvla_16layer_bf16_b32", "attention_cross"): int((6592.0 * 2 + 3000.0) * 1024),
     ("cfg3_gr00t_16dit_bf16_b64", "attention_cross"): int((62789.0 * 2 + 3351.8) * 1024),
     ("cfg4_bitvla_30layer_b8", "ternary_qkv_gemm_prefill"): int((16895.0 * 2 + 30720.0) * 1024),
+    ("cfg4_bitvla_30layer_b8", "attention_decode"): int((7005.5 * 2 + 1016.2) * 1024),
 }
 
 
