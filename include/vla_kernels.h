@@ -195,7 +195,11 @@ VLA_KAPI int vla_qkv_split_rope_append(const void* qkv, const float* cos_tab, co
  * src/kernels/bitvla/bitvla_lm_cuda.cu:446-486.
  *   q   [batch][S][n_q_heads][D] token-major, out [batch][S][n_q_heads*D]
  *   mask: additive fp32 [S][n_keys] shared by heads and batch, or NULL to use
- *   the generated mask (mask_kind, n_prefix, pad_start, pad_end). */
+ *   the generated mask (mask_kind, n_prefix, pad_start, pad_end).
+ * Shapes whose keys are sliced across workgroups use a partial-result workspace and arrival
+ * counters owned by the library (allocated on first use, outside any stream capture): calls
+ * that may overlap on the device -- different streams -- must be serialised by the caller,
+ * as one vla_predict at a time per handle already is (include/vla.h:18-19 of the reference). */
 VLA_KAPI int vla_attn_prefix_suffix(const void* q, const void* k_cache, const void* vt_cache, void* out,
                                     int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
                                     int t_max, int n_keys, float scale, int mask_kind, int n_prefix,
