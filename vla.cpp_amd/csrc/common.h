@@ -97,9 +97,15 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 // are returned in every lane.  K % 8 == 0 and K <= 512 NV.
 // GLU: the row is formed on the fly from a fused projection, x[k] = bf16(relu(gate[k])^2 * up[k])
 // with gate = xr and up = xr + K (gate_up_fused_sqrelu_mul_bf16, src/kernels/bitvla/bitvla_lm_cuda.cu:525-548).
-template <int NV, bool GLU = false>
+// WAVES > 1: the row is shared by the WAVES wavefronts of a workgroup (`lane` = the thread's
+// index in it, vectors lane, lane + 64 WAVES, ...; `red` = 16 floats of LDS for the three
+// reductions; every thread of the workgroup calls).  The squares are then added in another
+// order than by one wavefront, so the two forms agree to rounding, not bit for bit.
+template <int NV, bool GLU = false, int WAVES = 1>
 __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr, const bf16_t* __restrict__ w, int K,
-                                                  float eps, int lane, int8_t* qrow, float& scale_out, int& sum_out) {
+                                                  float eps, int lane, int8_t* qrow, float& scale_out, int& sum_out,
+                                                  float* red = nullptr) {
+    constexpr int LS = 64 * WAVES;  // vectors per pass over the row
     const int nvec = K / 8;
     // Every value kept between the passes is a bf16 (the input, then the rounded normalised
     // row), so the row stays packed: 4 registers per 16-byte vector.
@@ -111,7 +117,7 @@ __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr,
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int vec = lane + 64 * i;
+        const int vec = lane + LS * i;
         u32x4_t raw = {0u, 0u, 0u, 0u}, upr = {0u, 0u, 0u, 0u};
         wraw[i] = raw;
         if (vec < nvec) {
@@ -138,7 +144,7 @@ __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr,
             ss += a * a;
             ss += b * b;
         }
-    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)K + eps);
+    const float inv = 1.0f / sqrtf((WAVES > 1 ? block_sum(ss, red) : wave_sum(ss)) / (float)K + eps);
     // the packed words are opaque from here on, or the compiler keeps the first pass's unpacked
     // floats alive across the reduction (8 registers per vector instead of 4)
 #pragma unroll
@@ -148,7 +154,7 @@ __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr,
     float amax = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int vec = lane + 64 * i;
+        const int vec = lane + LS * i;
         if (vec >= nvec) continue;
         const int k0 = vec * 8;
 #pragma unroll
@@ -166,7 +172,7 @@ __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr,
             amax = fmaxf(amax, fmaxf(fabsf(lo(pr)), fabsf(hi(pr))));
         }
     }
-    amax = wave_max(amax);
+    amax = WAVES > 1 ? block_max(amax, red) : wave_max(amax);
     if (amax < 1e-5f) amax = 1e-5f;
     const float scale = 127.0f / amax;
 #pragma unroll
@@ -176,7 +182,7 @@ __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr,
     int sum = 0;
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        const int vec = lane + 64 * i;
+        const int vec = lane + LS * i;
         if (vec >= nvec) continue;
         uint32_t pk[2] = {0u, 0u};
 #pragma unroll
@@ -191,7 +197,16 @@ __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr,
         *reinterpret_cast<u32x2_t*>(qrow + (long)vec * 8) = u32x2_t{pk[0], pk[1]};
     }
     scale_out = scale;
-    sum_out = wave_sum_i(sum);
+    sum = wave_sum_i(sum);
+    if (WAVES > 1) {  // exact in any order
+        int* redi = reinterpret_cast<int*>(red);
+        __syncthreads();
+        if ((lane & 63) == 0) redi[lane >> 6] = sum;
+        __syncthreads();
+        sum = 0;
+        for (int i = 0; i < WAVES; ++i) sum += redi[i];
+    }
+    sum_out = sum;
 }
 
 // ggml_silu / ggml_gelu (tanh form), fp32 (src/layers/ffn.h:24-40).

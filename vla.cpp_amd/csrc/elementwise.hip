@@ -262,6 +262,24 @@ __global__ void __launch_bounds__(256) row_norm_kernel(const T* __restrict__ x, 
     }
 }
 
+// Rows longer than 4096 (the 6912-wide BitNet FFN) through RMSNorm + int8 quantisation: one
+// workgroup of four wavefronts per row, four vectors per lane at most (a single wavefront
+// would hold sixteen and spend its time in the arithmetic of 128 elements per lane).
+template <bool GLU>
+__global__ void __launch_bounds__(256) row_norm_wide_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                            int8_t* __restrict__ q, float* __restrict__ scales,
+                                                            int32_t* __restrict__ rowsum, int K, float eps) {
+    __shared__ float red[16];
+    const int row = blockIdx.x;
+    float scale;
+    int sum;
+    rms_act_quant_row<4, GLU, 4>(x + (long)row * K * (GLU ? 2 : 1), w, K, eps, threadIdx.x, q + (long)row * K, scale, sum, red);
+    if (threadIdx.x == 0) {
+        scales[row] = scale;
+        if (rowsum) rowsum[row] = sum;
+    }
+}
+
 // Launches row_norm_kernel when the row fits a wavefront's registers and the buffers allow
 // 16-byte accesses; returns false otherwise (the callers fall back to the scalar kernels).
 // The choice depends on the row length only, never on the number of rows, so an
@@ -280,7 +298,7 @@ bool launch_row_norm(const void* x, const void* w, const float* sc, const float*
     else if (nvec <= 64 * 8) VLA_ROW_NORM(8);
     else if constexpr (MODE == NORM_RMS_AQ && sizeof(T) == 2) {  // the 6912-wide BitNet FFN rows
         if (nvec > 64 * 16) return false;
-        VLA_ROW_NORM(16);
+        row_norm_wide_kernel<GLU><<<M, 256, 0, st>>>((const bf16_t*)x, (const bf16_t*)w, q, scales, rowsum, K, eps);
     } else {
         return false;
     }
