@@ -249,7 +249,8 @@ VLA_KAPI int vla_act_quant_bf16(const uint16_t* in, int8_t* out, float* scales, 
 /* bitvla_rmsnorm_bf16 followed by vla_act_quant_bf16 in one launch (the pair that opens
  * both halves of run_layer, src/kernels/bitvla/bitvla_lm_cuda.cu:422-486); the bf16
  * intermediate is not written.  int8 rows, scales and row sums are bit-identical to the
- * two separate calls for K <= 4096 (longer rows add the squares in another order). */
+ * two separate calls for K <= 4096 (longer rows are shared by four wavefronts, which add
+ * the squares in another order than the separate RMSNorm: results agree to rounding). */
 VLA_KAPI int vla_rmsnorm_act_quant_bf16(const uint16_t* x, const uint16_t* w, int8_t* out, float* scales,
                                         int32_t* rowsum, float eps, int M, int K, vla_stream_t stream);
 /* The same on rows formed on the fly from a fused [M][gate(K) | up(K)] projection,
@@ -303,7 +304,7 @@ VLA_KAPI int vla_rmsnorm_ternary_gemv(const uint16_t* x, const uint16_t* norm_w,
 /* The same with x formed on the fly from a fused [M][gate(K) | up(K)] projection,
  * x = bf16(relu(gate)^2 * up): gate_up_fused_sqrelu_mul_bf16 -> ffn sub-norm -> act_quant ->
  * down projection (+ residual) of run_layer (bitvla_lm_cuda.cu:503-520) in one launch, same
- * bits as those calls. */
+ * bits as those calls for K <= 4096, equal to rounding beyond. */
 VLA_KAPI int vla_sqrelu_rmsnorm_ternary_gemv(const uint16_t* gate_up, const uint16_t* norm_w, float eps,
                                              const uint32_t* W_packed, uint16_t* out, const uint16_t* residual,
                                              const float* ws, int ws_num, int M, int N, int K, vla_stream_t stream);
