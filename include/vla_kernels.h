@@ -21,6 +21,7 @@
 #ifndef VLA_KERNELS_H
 #define VLA_KERNELS_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -41,6 +42,7 @@ typedef enum {
     VLA_K_ERR_ARG = -1,    /* null pointer or negative size */
     VLA_K_ERR_SHAPE = -2,  /* a size the kernels do not support (alignment, head_dim, ...) */
     VLA_K_ERR_LAUNCH = -3, /* hipGetLastError() after the launch */
+    VLA_K_ERR_WORKSPACE = -4, /* the workspace handed in (or the fixed one) is too small for the shape */
 } vla_kstatus;
 
 /* Suffix-block mask generated inside the attention kernel (the reference builds
@@ -196,14 +198,32 @@ VLA_KAPI int vla_qkv_split_rope_append(const void* qkv, const float* cos_tab, co
  *   q   [batch][S][n_q_heads][D] token-major, out [batch][S][n_q_heads*D]
  *   mask: additive fp32 [S][n_keys] shared by heads and batch, or NULL to use
  *   the generated mask (mask_kind, n_prefix, pad_start, pad_end).
- * Shapes whose keys are sliced across workgroups use a partial-result workspace and arrival
- * counters owned by the library (allocated on first use, outside any stream capture): calls
- * that may overlap on the device -- different streams -- must be serialised by the caller,
- * as one vla_predict at a time per handle already is (include/vla.h:18-19 of the reference). */
+ * Shapes whose keys are sliced across workgroups need scratch memory (the slices' partial
+ * rows and arrival counters).  This entry point takes it from blocks the library keeps per
+ * (device, stream): grown on demand with hipMalloc -- so a shape must have run once on a
+ * stream before that stream is captured -- and never freed before the process ends, so a
+ * captured graph keeps pointing at live memory.  Calls on one stream are ordered and may
+ * share a block; calls on different streams never do. */
 VLA_KAPI int vla_attn_prefix_suffix(const void* q, const void* k_cache, const void* vt_cache, void* out,
                                     int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
                                     int t_max, int n_keys, float scale, int mask_kind, int n_prefix,
                                     int pad_start, int pad_end, const float* mask, vla_stream_t stream);
+
+/* The same call with the scratch memory owned by the caller -- what a model handle uses, so
+ * that the reference's rule "one vla_predict at a time per handle" (include/vla.h:18-19) is
+ * all a caller has to keep: handles never share scratch.
+ *   vla_attn_workspace_bytes: bytes the shape needs, 0 when it needs none (or is not
+ *     supported); depends on the shape only, not on pointers.
+ *   workspace: device memory of at least that many bytes, 16-byte aligned, zero-filled once
+ *     before its first use (every launch leaves the part that must stay zero at zero);
+ *     NULL is accepted when the shape needs none.  VLA_K_ERR_WORKSPACE if it is too small. */
+VLA_KAPI size_t vla_attn_workspace_bytes(int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
+                                         int n_keys);
+VLA_KAPI int vla_attn_prefix_suffix_ws(const void* q, const void* k_cache, const void* vt_cache, void* out,
+                                       int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
+                                       int t_max, int n_keys, float scale, int mask_kind, int n_prefix,
+                                       int pad_start, int pad_end, const float* mask, void* workspace,
+                                       size_t workspace_bytes, vla_stream_t stream);
 
 /* --------------------------------------------------------- flow-matching glue */
 
@@ -402,6 +422,13 @@ VLA_KAPI int bitvla_lm_hip_forward(bitvla_lm_hip_ctx* ctx, const uint16_t* d_in,
 
 /* Library identification, for a loader that wants to check what it bound. */
 VLA_KAPI const char* vla_kernels_arch(void); /* "gfx950" */
+
+/* Optional set-up for the current device, so that no later call has to do it lazily: reads
+ * the tuning overrides from the environment.  0 or a vla_kstatus. */
+VLA_KAPI int vla_kernels_init(void);
+/* Reads the tuning overrides (VLA_ATTN_*, VLA_GEMM_*, VLA_TERNARY_TILE; tests and tuning
+ * only) from the environment again.  No launch path reads the environment. */
+VLA_KAPI void vla_kernels_reload_env(void);
 
 #ifdef __cplusplus
 }

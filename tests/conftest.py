@@ -41,3 +41,26 @@ def mt19937_raw(seed, n):
 @pytest.fixture
 def rng():
     return np.random.default_rng(0x5EED)
+
+
+@pytest.fixture
+def tune(monkeypatch):
+    """Tuning overrides of the kernel library (VLA_ATTN_*, VLA_GEMM_*, VLA_TERNARY_TILE).
+
+    The library reads them from the environment once, never on a launch path, so a test that
+    changes one asks it to read them again; everything is restored when the test ends."""
+    from util import pkg
+
+    class Tune:
+        def set(self, key, value):
+            monkeypatch.setenv(key, str(value))
+            pkg.lib().vla_kernels_reload_env()
+
+        def clear(self, *keys):
+            for k in keys:
+                monkeypatch.delenv(k, raising=False)
+            pkg.lib().vla_kernels_reload_env()
+
+    yield Tune()
+    monkeypatch.undo()
+    pkg.lib().vla_kernels_reload_env()

@@ -195,7 +195,7 @@ def test_linear_bias_residual(dtype, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(150, 720, 720), (333, 200, 1104), (64, 1600, 48)])
-def test_linear_bf16_every_kernel_and_tiling_gives_the_same_bits(monkeypatch, M, N, K):
+def test_linear_bf16_every_kernel_and_tiling_gives_the_same_bits(tune, M, N, K):
     """The direct-to-LDS kernel and the register-staged one, in every tile configuration, add
     the products of a row in the same order (ascending k, 16 at a time): identical outputs,
     including partial k-tiles (K not a multiple of 64 or 128) and ragged M and N."""
@@ -207,9 +207,9 @@ def test_linear_bf16_every_kernel_and_tiling_gives_the_same_bits(monkeypatch, M,
     outs = {}
     for dl, tile, stages in [("0", t, "0") for t in "01234"] + [("1", t, ns) for t in "01234" for ns in "234"] + [("1", "5", "0")]:
         if True:
-            monkeypatch.setenv("VLA_GEMM_DL", dl)
-            monkeypatch.setenv("VLA_GEMM_TILE", tile)
-            monkeypatch.setenv("VLA_GEMM_STAGES", stages)
+            tune.set("VLA_GEMM_DL", dl)
+            tune.set("VLA_GEMM_TILE", tile)
+            tune.set("VLA_GEMM_STAGES", stages)
             y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
             pkg.call("vla_linear", xd, Wd, None, None, y, BF16, F32, M, N, K)
             yb = empty((M, N), BF16)
@@ -406,7 +406,7 @@ def _mask(kind, P, S, pad):
 @pytest.mark.parametrize("dtype,kernel", [(F32, "auto"), (BF16, "auto"), (BF16, "direct"), (BF16, "staged"), (BF16, "one-slice")],
                          ids=["f32", "bf16", "bf16-direct", "bf16-staged", "bf16-one-slice"])
 @pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
-def test_attention_against_oracle(monkeypatch, dtype, kernel, case):
+def test_attention_against_oracle(tune, dtype, kernel, case):
     name, B, S, Hq, Hkv, D, P, kind, pad = case
     if dtype == F32 and D == 256:
         pytest.skip("fp32 tiles for 256-wide heads are not built (LDS budget); pi0 runs in bf16")
@@ -415,14 +415,14 @@ def test_attention_against_oracle(monkeypatch, dtype, kernel, case):
         # that it walks 32-row blocks, exercised here on the cases that normally take the LDS kernel
         if not (D <= 128 and 32 < (Hq // Hkv) * S <= 256):
             pytest.skip("covered by the default dispatch")
-        monkeypatch.setenv("VLA_ATTN_DIRECT_ROWS", "256")
+        tune.set("VLA_ATTN_DIRECT_ROWS", "256")
     if kernel in ("staged", "one-slice"):
         # 64-wide bf16 heads beyond 32 rows default to the direct-to-LDS variant of the LDS
         # kernel (two key slices per row tile with 3+ key tiles); the
         # register-staged variant and the unsliced one on the same cases
         if not (D == 64 and (Hq // Hkv) * S > 32):
             pytest.skip("covered by the default dispatch")
-        monkeypatch.setenv("VLA_ATTN_DL" if kernel == "staged" else "VLA_ATTN_SLICES", "0" if kernel == "staged" else "1")
+        tune.set("VLA_ATTN_DL" if kernel == "staged" else "VLA_ATTN_SLICES", "0" if kernel == "staged" else "1")
     r = np.random.default_rng(106)
     mask, mkind, T = _mask(kind, P, S, pad)
     t_max = (T + 63) // 64 * 64
@@ -468,7 +468,7 @@ def test_attention_against_oracle(monkeypatch, dtype, kernel, case):
 
 
 @pytest.mark.parametrize("split", [1, 2, 5, 8, 64])
-def test_attention_direct_kernel_key_slices_merge(monkeypatch, split):
+def test_attention_direct_kernel_key_slices_merge(tune, split):
     # Few query rows: any slicing of the keys across wavefronts (merged by the second
     # kernel) gives the same result as the oracle.
     r = np.random.default_rng(120 + split)
@@ -480,7 +480,7 @@ def test_attention_direct_kernel_key_slices_merge(monkeypatch, split):
     kc = torch.full((B, Hkv, t_max, D), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
     vc = torch.full((B, Hkv, D, t_max), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
     pkg.call("vla_kv_append", kc, vc, to_dev(K, BF16), to_dev(V, BF16), BF16, B, Hkv, D, t_max, 0, T)
-    monkeypatch.setenv("VLA_ATTN_SPLIT", str(split))
+    tune.set("VLA_ATTN_SPLIT", str(split))
     out = empty((B, S, Hq * D), BF16)
     pkg.call("vla_attn_prefix_suffix", to_dev(Q, BF16), kc, vc, out, BF16, B, S, Hq, Hkv, D, t_max, T, 0.125,
              pkg.VLA_MASK_CAUSAL_SUFFIX, T - S, 100, 120, None)
@@ -493,7 +493,7 @@ def test_attention_direct_kernel_key_slices_merge(monkeypatch, split):
 
 @pytest.mark.parametrize("B,S,Hq,Hkv,T", [(8, 1, 20, 5, 519), (1, 1, 20, 5, 513), (3, 2, 8, 2, 519), (1, 1, 28, 4, 1000), (3, 2, 8, 2, 300), (2, 1, 4, 4, 97),
                                           (8, 1, 20, 5, 33)])
-def test_attention_decode_slices_merged_by_the_last_to_arrive(monkeypatch, B, S, Hq, Hkv, T):
+def test_attention_decode_slices_merged_by_the_last_to_arrive(tune, B, S, Hq, Hkv, T):
     # 128-wide heads, a few rows per kv head (single-token decode): the keys are sliced over
     # single-wavefront workgroups and the slice that arrives last merges them inside the launch.
     # Same tolerance against the oracle as the one-workgroup form, repeatable bit for bit
@@ -516,7 +516,7 @@ def test_attention_decode_slices_merged_by_the_last_to_arrive(monkeypatch, B, S,
         return as_f32(out, BF16)
 
     got = [run() for _ in range(3)]
-    monkeypatch.setenv("VLA_ATTN_NO_ARRIVE", "1")
+    tune.set("VLA_ATTN_NO_ARRIVE", "1")
     ref = run()
     mask = np.zeros((S, T), np.float32)
     want = np.stack([orc.attention(Q[b], K[b], V[b], mask, scale) for b in range(B)]).reshape(B, S, Hq * D)
@@ -526,7 +526,7 @@ def test_attention_decode_slices_merged_by_the_last_to_arrive(monkeypatch, B, S,
 
 
 @pytest.mark.parametrize("B", [1, 4])
-def test_attention_wide_heads_key_slices_and_partial_formats(monkeypatch, B):
+def test_attention_wide_heads_key_slices_and_partial_formats(tune, B):
     # pi0's 256-wide MQA heads: with few workgroups the keys are walked in slices whose partial
     # outputs travel as fp16 (normalised per slice) to a merge launch.  Unsliced, fp32 partials
     # and fp16 partials all meet the oracle; the fp16 partials cost less than the output rounding.
@@ -544,9 +544,9 @@ def test_attention_wide_heads_key_slices_and_partial_formats(monkeypatch, B):
     got = {}
     for name, env in (("sliced-fp16", {}), ("sliced-fp32", {"VLA_ATTN_PART_F32": "1"}), ("unsliced", {"VLA_ATTN_SPLIT": "1"})):
         for k in ("VLA_ATTN_PART_F32", "VLA_ATTN_SPLIT"):
-            monkeypatch.delenv(k, raising=False)
+            tune.clear(k)
         for k, v in env.items():
-            monkeypatch.setenv(k, v)
+            tune.set(k, v)
         out = empty((B, S, Hq * D), BF16)
         pkg.call("vla_attn_prefix_suffix", to_dev(Q, BF16), kc, vc, out, BF16, B, S, Hq, Hkv, D, t_max, T, 1.0 / 16,
                  pkg.VLA_MASK_PI0_STATE, P, 0, 0, None)
@@ -649,7 +649,7 @@ def test_ternary_gemm_accumulators_and_epilogue_bit_exact(M, N, K, ws_num):
 
 @pytest.mark.parametrize("tile", [128, 256])
 @pytest.mark.parametrize("M,N,K", [(300, 288, 256), (515, 640, 384), (64, 48, 128)])
-def test_ternary_gemm_large_tile_kernels_bit_exact(monkeypatch, tile, M, N, K):
+def test_ternary_gemm_large_tile_kernels_bit_exact(tune, tile, M, N, K):
     # The large-M kernels (weights read straight from the fragment-major layout), pinned
     # by VLA_TERNARY_TILE, on ragged M and N: same int32 accumulators and bf16 epilogue.
     r = np.random.default_rng(tile + M)
@@ -667,7 +667,7 @@ def test_ternary_gemm_large_tile_kernels_bit_exact(monkeypatch, tile, M, N, K):
     acc = torch.zeros((M, N), dtype=torch.int32, device="cuda")
     out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
     rowsum = dev(A.astype(np.int32).sum(1).astype(np.int32))
-    monkeypatch.setenv("VLA_TERNARY_TILE", str(tile))
+    tune.set("VLA_TERNARY_TILE", str(tile))
     pkg.call("vla_ternary_gemm", dev(A), dev(packed), out, acc, dev(s), rowsum, dev(ws), ws_num, M, N, K)
     sync()
     want_acc = orc.ternary_gemm_i32(A, Wt)
@@ -675,7 +675,7 @@ def test_ternary_gemm_large_tile_kernels_bit_exact(monkeypatch, tile, M, N, K):
     assert np.array_equal(host(out, np.uint16), orc.ternary_epilogue(want_acc, s, ws))
 
 
-def test_ternary_gemm_prefill_shape_all_tilings_agree(monkeypatch):
+def test_ternary_gemm_prefill_shape_all_tilings_agree(tune):
     # BitVLA prefill QKV at full size (M = 8 x 512 tokens): the shape-selected kernel and
     # both pinned tilings give identical accumulators and outputs; a sample of rows is
     # checked against the oracle.
@@ -690,9 +690,9 @@ def test_ternary_gemm_prefill_shape_all_tilings_agree(monkeypatch):
     res = []
     for tile in (None, 64, 128, 256):
         if tile is None:
-            monkeypatch.delenv("VLA_TERNARY_TILE", raising=False)
+            tune.clear("VLA_TERNARY_TILE")
         else:
-            monkeypatch.setenv("VLA_TERNARY_TILE", str(tile))
+            tune.set("VLA_TERNARY_TILE", str(tile))
         acc = torch.zeros((M, N), dtype=torch.int32, device="cuda")
         out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
         pkg.call("vla_ternary_gemm", dA, dW, out, acc, ds, rowsum, dws, ws_num, M, N, K)
@@ -735,7 +735,7 @@ def test_ternary_gemv_decode_rows_bit_exact(M, N, K, ws_num):
 
 
 @pytest.mark.parametrize("M,N,K,tile", [(300, 288, 256, 64), (300, 288, 256, 128), (515, 640, 384, 256)])
-def test_ternary_gemm_add_matches_gemm_then_add(monkeypatch, M, N, K, tile):
+def test_ternary_gemm_add_matches_gemm_then_add(tune, M, N, K, tile):
     r = np.random.default_rng(M + tile)
     A = r.integers(-127, 128, (M, K)).astype(np.int8)
     t = r.integers(-1, 2, (N, K)).astype(np.int8)
@@ -744,7 +744,7 @@ def test_ternary_gemm_add_matches_gemm_then_add(monkeypatch, M, N, K, tile):
     res = orc.to_bf16(r.standard_normal((M, N)).astype(np.float32))
     dA, dW, ds, dws = dev(A), dev(_pack_plain(t)), dev(s), dev(ws)
     rowsum = dev(A.astype(np.int32).sum(1).astype(np.int32))
-    monkeypatch.setenv("VLA_TERNARY_TILE", str(tile))
+    tune.set("VLA_TERNARY_TILE", str(tile))
     out = torch.zeros((M, N), dtype=torch.int16, device="cuda")
     pkg.call("vla_ternary_gemm", dA, dW, out, None, ds, rowsum, dws, 1, M, N, K)
     fused = torch.zeros_like(out)

@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(HERE, "libvla.so")
 VLA_DT_F32, VLA_DT_BF16, VLA_DT_BF16_P2 = 0, 1, 2
 VLA_ACT_NONE, VLA_ACT_SILU, VLA_ACT_GELU = 0, 1, 2
 VLA_MASK_NONE, VLA_MASK_CAUSAL_SUFFIX, VLA_MASK_PI0_STATE = 0, 1, 2
-VLA_K_OK, VLA_K_ERR_ARG, VLA_K_ERR_SHAPE, VLA_K_ERR_LAUNCH = 0, -1, -2, -3
+VLA_K_OK, VLA_K_ERR_ARG, VLA_K_ERR_SHAPE, VLA_K_ERR_LAUNCH, VLA_K_ERR_WORKSPACE = 0, -1, -2, -3, -4
 
 _lib = None
 
@@ -42,6 +42,9 @@ KERNEL_API = {
     "vla_fold_norm_weight_host": [_vp, _vp, _i, _i, _i, _vp],
     "vla_qkv_split_rope_append": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "vla_attn_prefix_suffix": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp],
+    "vla_attn_prefix_suffix_ws": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp,
+                                  ctypes.c_size_t, _vp],
+    "vla_attn_workspace_bytes": [_i, _i, _i, _i, _i, _i, _i],
     "vla_embed_suffix": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "vla_embed_suffix_act": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "vla_set_lead_rows": [_vp, _vp, _i, _i, _i, _i, _i, _vp],
@@ -78,8 +81,11 @@ KERNEL_API = {
     "bitlinear_int8xint2_m": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "bitlinear_int8xint2": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "vla_kernels_arch": [],
+    "vla_kernels_init": [],
+    "vla_kernels_reload_env": [],
 }
-_RESTYPES = {"vla_kernels_arch": ctypes.c_char_p, "vla_ternary_packed_words": ctypes.c_long,
+_RESTYPES = {"vla_kernels_arch": ctypes.c_char_p, "vla_attn_workspace_bytes": ctypes.c_size_t,
+             "vla_kernels_reload_env": None, "vla_ternary_packed_words": ctypes.c_long,
              "bitvla_lm_hip_init": ctypes.c_void_p, "bitvla_lm_hip_free": None, "bitvla_lm_hip_set_layer": None,
              "bitvla_lm_hip_set_output_norm": None}
 

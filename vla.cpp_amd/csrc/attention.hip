@@ -749,11 +749,22 @@ __device__ __forceinline__ void arrive_merge(const AttnArgs& a, const f32x16_t (
                 st_dev64(po + d + 2, o[db][4 * j + 2], o[db][4 * j + 3]);
             }
     }
+    // Ordering.  Hardware (gfx950, which this file is compiled for and nothing else -- see the
+    // #error in common.h): the partials above are device-scope atomic stores, i.e. written
+    // through to memory, and vmcnt counts a store only once memory has acknowledged it; the
+    // merger's device-scope atomic loads below are served from memory, not from its XCD's L2.
+    // So once vmcnt is zero the partials are visible to every XCD, and the counter's value
+    // tells the last slice that every other slice got that far.  Compiler: the two
+    // workgroup-scope fences forbid moving the stores below the count and the merger's loads
+    // above it; at workgroup scope they cost no cache maintenance (an agent-scope release
+    // would write back the whole L2: 121 us per launch, measured).
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's partials are in memory before it is counted
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     int old = 0;
     if (lane == 0) old = __hip_atomic_fetch_add(a.arrive + prb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     old = __builtin_amdgcn_readfirstlane(old);
     if (old != a.n_split - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     if (lane == 0) __hip_atomic_store(a.arrive + prb, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
 
     // Lane t = rl * n_split + sp holds (max, sum) of row rl in slice sp, then its weight
@@ -1103,36 +1114,43 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
                        lane);
 }
 
-// Workspace for key-split partials, grown on demand (never under stream capture:
-// run the shape once before capturing it).
-float* g_ws = nullptr;
-size_t g_ws_floats = 0;
+// ---- scratch memory of a call ---------------------------------------------------------
+// Shapes whose keys are sliced across workgroups need device memory beyond the inputs and
+// outputs: the slices' partial (max, sum, output) rows and, for the in-launch merge, one
+// arrival counter per (pair, row block).  One block holds both:
+//     [0, ARRIVE_BYTES)      int counters, zero between launches (a new block is zero-filled,
+//                            every launch that uses them leaves them at zero)
+//     [ARRIVE_BYTES, ...)    partials, rows x (D + 2) floats
+// It comes from the library's per-stream blocks (vla_attn_prefix_suffix), from the caller
+// (vla_attn_prefix_suffix_ws);
+// a dry run only reports the size (vla_attn_workspace_bytes).
+constexpr size_t ARRIVE_BYTES = (size_t)ARRIVE_MAX_UNITS * sizeof(int);
+struct Scratch {
+    enum Kind { LIBRARY, CALLER, DRY };
+    Kind kind = LIBRARY;
+    unsigned char* base = nullptr;  // CALLER: the block handed in
+    size_t bytes = 0;
+    size_t need = 0;  // bytes the shape asked for (every kind)
+};
+size_t scratch_bytes(size_t rows, int D) { return ARRIVE_BYTES + (rows * (size_t)(D + 2) * sizeof(float) + 255) / 256 * 256; }
 
-// Arrival counters of the direct kernel's in-launch merge: allocated and zeroed once, left at
-// zero by every launch that uses them.  Launches that overlap on the device must not share
-// them (nor the partial workspace): one attention launch at a time per process.
-int* g_arrive = nullptr;
-int* arrive_counters() {
-    if (!g_arrive) {
-        if (hipMalloc((void**)&g_arrive, ARRIVE_MAX_UNITS * sizeof(int)) != hipSuccess) return g_arrive = nullptr;
-        if (hipMemset(g_arrive, 0, ARRIVE_MAX_UNITS * sizeof(int)) != hipSuccess) {
-            (void)hipFree(g_arrive);
-            return g_arrive = nullptr;
-        }
+// Binds the partial rows (and the counters) of a sliced call.  Returns VLA_K_OK with
+// a.part_o == nullptr on a dry run: the caller then returns without launching.
+int bind_scratch(AttnArgs& a, Scratch& sc, hipStream_t st, size_t rows, int D) {
+    sc.need = scratch_bytes(rows, D);
+    a.part_o = nullptr;
+    if (sc.kind == Scratch::DRY) return VLA_K_OK;
+    unsigned char* base = sc.base;
+    if (sc.kind == Scratch::LIBRARY) {
+        base = (unsigned char*)stream_scratch(SCRATCH_ATTN, st, sc.need);
+        if (!base) return VLA_K_ERR_LAUNCH;
+    } else if (!base || sc.bytes < sc.need || ((uintptr_t)base & 15)) {
+        return VLA_K_ERR_WORKSPACE;
     }
-    return g_arrive;
-}
-
-float* workspace(size_t floats) {
-    if (floats > g_ws_floats) {
-        if (g_ws) (void)hipFree(g_ws);
-        g_ws = nullptr;
-        g_ws_floats = 0;
-        const size_t want = floats < (1u << 20) ? (1u << 20) : floats;
-        if (hipMalloc((void**)&g_ws, want * sizeof(float)) != hipSuccess) return nullptr;
-        g_ws_floats = want;
-    }
-    return g_ws;
+    a.arrive = reinterpret_cast<int*>(base);
+    a.part_o = reinterpret_cast<float*>(base + ARRIVE_BYTES);
+    a.part_ml = a.part_o + rows * D;
+    return VLA_K_OK;
 }
 
 // Second launch of a key-split LDS-kernel call: combines the workgroups' partials.
@@ -1156,12 +1174,11 @@ int launch_nw(AttnArgs& a, hipStream_t st) {
     const int n_pairs = a.batch * a.Hkv;
     const int grid = (n_pairs + 7) / 8 * 8 * a.n_groups * a.n_split;
     if constexpr (sizeof(T) == 2 && D == 64) {
-        // 64-wide bf16 heads: tiles go straight into a swizzled LDS ring (VLA_ATTN_DL=0 pins
-        // the register-staged path), and with three or more key tiles they are split over
-        // two wavefronts per row tile (VLA_ATTN_SLICES = 1 | 2 overrides).  The kernel also
-        // builds for 128-wide heads, where its register use makes it the slower choice.
-        const char* e = getenv("VLA_ATTN_DL");
-        if (!(e && atoi(e) == 0)) {
+        // 64-wide bf16 heads: tiles go straight into a swizzled LDS ring (the tuning override
+        // attn_dl = 0 pins the register-staged path), and with three or more key tiles they
+        // are split over two wavefronts per row tile (attn_slices = 1 | 2 overrides).  The
+        // kernel also builds for 128-wide heads, where its register use makes it the slower choice.
+        if (tuning().attn_dl != 0) {
             const int nsl = a.n_slices;
             if constexpr (D == 64 && NW <= 2) {
                 if (nsl == 2) {
@@ -1192,8 +1209,9 @@ int launch_nw(AttnArgs& a, hipStream_t st) {
 }
 
 template <int D>
-int launch_direct(AttnArgs& a, hipStream_t st) {
+int launch_direct(AttnArgs& a, hipStream_t st, Scratch& sc) {
     constexpr int ST = D <= 64 ? 3 : 2;
+    const Tuning& tn = tuning();
     const int n_pairs = a.batch * a.Hkv;
     const int R = (a.Hq / a.Hkv) * a.S;
     a.n_rblocks = (R + 31) / 32;
@@ -1205,7 +1223,7 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
     if (n_units < 2048) n_split = (2048 + n_units - 1) / n_units;
     if (n_split > (nb_total + 1) / 2) n_split = (nb_total + 1) / 2;
     if (n_split < 1) n_split = 1;
-    if (const char* e = getenv("VLA_ATTN_SPLIT")) n_split = atoi(e) > 0 ? (atoi(e) < nb_total ? atoi(e) : nb_total) : 1;
+    if (tn.attn_split_set) n_split = tn.attn_split > 0 ? (tn.attn_split < nb_total ? tn.attn_split : nb_total) : 1;
     // Slices of one pair as the wavefronts of one workgroup (merged through LDS, one launch)
     // when few enough; with fewer than 32 pairs more slices go through global partials and
     // the merge kernel instead.
@@ -1217,10 +1235,9 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
     // hand-over is three dependent trips to memory whatever the count (519 keys, batch 8: six
     // slices 13.6 us, nine 14.7 us, one workgroup of four 13.5 us alone and 1.4 us slower in sequence).
     const int Rb = R < 32 ? R : 32;
-    int n_arrive = n_split < (nb_total + 2) / 3 || getenv("VLA_ATTN_SPLIT") ? n_split : (nb_total + 2) / 3;
+    int n_arrive = n_split < (nb_total + 2) / 3 || tn.attn_split_set ? n_split : (nb_total + 2) / 3;
     if (n_arrive * Rb > ARRIVE_MAX_T) n_arrive = ARRIVE_MAX_T / Rb;
-    bool arrive = D == 128 && n_arrive > MERGE_MAX && a.n_rblocks == 1 && n_units <= ARRIVE_MAX_UNITS &&
-                  !getenv("VLA_ATTN_NO_ARRIVE") && arrive_counters();
+    bool arrive = D == 128 && n_arrive > MERGE_MAX && a.n_rblocks == 1 && n_units <= ARRIVE_MAX_UNITS && !tn.attn_no_arrive;
     if (arrive) {
         n_split = n_arrive;
         wg_merge = false;
@@ -1230,23 +1247,23 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
     a.n_split = (nb_total + a.tiles_per_split - 1) / a.tiles_per_split;
     a.r_pad = a.n_rblocks * 32;
     a.n_groups = 1;
+    a.arrive = nullptr;
     if (wg_merge && a.n_split > 1) {
         const size_t lds = (size_t)a.n_split * (R < 32 ? R : 32) * (D + 2) * sizeof(float);  // at most 8 * 32 * 66 * 4 or 4 * 32 * 130 * 4 = 66 KB
         if (lds <= 64 * 1024) {
+            if (sc.kind == Scratch::DRY) return VLA_K_OK;
             if (a.p2) attn_direct_kernel<D, true, ST, true><<<n_units, a.n_split * 64, lds, st>>>(a);
             else attn_direct_kernel<D, false, ST, true><<<n_units, a.n_split * 64, lds, st>>>(a);
             return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
         }
     }
     if (a.n_split > 1) {
-        const size_t rows = (size_t)n_pairs * a.n_split * a.r_pad;
-        float* ws = workspace(rows * (D + 2));
-        if (!ws) return VLA_K_ERR_LAUNCH;
-        a.part_o = ws;
-        a.part_ml = ws + rows * D;
+        const int rc = bind_scratch(a, sc, st, (size_t)n_pairs * a.n_split * a.r_pad, D);
+        if (rc != VLA_K_OK) return rc;
     }
+    if (sc.kind == Scratch::DRY) return VLA_K_OK;
     arrive = arrive && a.n_split > 1 && a.n_split * Rb <= ARRIVE_MAX_T;
-    a.arrive = arrive ? g_arrive : nullptr;
+    if (!arrive) a.arrive = nullptr;
     const int wgw = arrive ? 1 : 4;  // wavefronts per workgroup
     const unsigned grid = (unsigned)(((long)n_units * a.n_split + wgw - 1) / wgw);
     if (a.p2) attn_direct_kernel<D, true, ST, false><<<grid, wgw * 64, 0, st>>>(a);
@@ -1262,27 +1279,25 @@ int launch_direct(AttnArgs& a, hipStream_t st) {
 }
 
 template <typename T, int D>
-int launch_d(AttnArgs& a, vla_stream_t stream) {
+int launch_d(AttnArgs& a, vla_stream_t stream, Scratch& sc) {
+    const Tuning& tn = tuning();
+    hipStream_t st = (hipStream_t)stream;
     const int R = (a.Hq / a.Hkv) * a.S;
     if constexpr (sizeof(T) == 2 && D <= 128) {
-        // VLA_ATTN_NO_DIRECT pins the LDS kernel; VLA_ATTN_DIRECT_ROWS overrides the row limit
-        // of the register-direct one (tests and tuning).
-        const bool no_direct = getenv("VLA_ATTN_NO_DIRECT") != nullptr;
-        const char* er = getenv("VLA_ATTN_DIRECT_ROWS");
-        const int max_rows = er ? atoi(er) : 32;  // more rows: 16-byte runs per key row cost more than sharing tiles through LDS saves
-        if (R <= max_rows && !no_direct) return launch_direct<D>(a, (hipStream_t)stream);
+        // At most attn_direct_rows (32) rows per kv head: the register-direct kernel.  With more
+        // rows, 16-byte runs per key row cost more than sharing tiles through LDS saves.
+        if (R <= tn.attn_direct_rows && !tn.attn_no_direct) return launch_direct<D>(a, st, sc);
     }
     const int n_tiles = (R + 31) / 32;
     // 64-wide bf16 heads with three or more key tiles: two key slices per row tile (the
-    // direct-to-LDS variant of the kernel; VLA_ATTN_DL=0 and VLA_ATTN_SLICES override).
-    // Two wavefronts per row tile then, and at most two row tiles per workgroup, so that a
-    // batch-32 launch stays resident at once (two 4-wavefront workgroups per CU).
+    // direct-to-LDS variant of the kernel).  Two wavefronts per row tile then, and at most
+    // two row tiles per workgroup, so that a batch-32 launch stays resident at once (two
+    // 4-wavefront workgroups per CU).
     a.n_slices = 1;
     if constexpr (sizeof(T) == 2 && D == 64) {
-        const char* e = getenv("VLA_ATTN_DL");
-        if (!(e && atoi(e) == 0)) {
+        if (tn.attn_dl != 0) {
             a.n_slices = (a.n_keys + SPLIT_KEYS - 1) / SPLIT_KEYS >= 3 ? 2 : 1;
-            if (const char* es = getenv("VLA_ATTN_SLICES")) a.n_slices = atoi(es) == 2 ? 2 : 1;
+            if (tn.attn_slices) a.n_slices = tn.attn_slices == 2 ? 2 : 1;
         }
     }
     // One wavefront (per slice) per row tile, at most one wavefront of a workgroup per SIMD;
@@ -1313,20 +1328,18 @@ int launch_d(AttnArgs& a, vla_stream_t stream) {
         if (want > key_tiles / 2) want = key_tiles / 2;
         if (want >= 2) {
             a.n_split = want;
-            a.part_half = getenv("VLA_ATTN_PART_F32") ? 0 : 1;  // the env keeps fp32 partials (tests)
+            a.part_half = (tn.attn_part_f32 || sizeof(T) != 2) ? 0 : 1;
         }
     }
-    if (const char* e = getenv("VLA_ATTN_SPLIT")) a.n_split = atoi(e) > 0 ? (atoi(e) < key_tiles ? atoi(e) : key_tiles) : 1;
+    if (tn.attn_split_set) a.n_split = tn.attn_split > 0 ? (tn.attn_split < key_tiles ? tn.attn_split : key_tiles) : 1;
     a.tiles_per_split = (key_tiles + a.n_split - 1) / a.n_split;
     a.n_split = (key_tiles + a.tiles_per_split - 1) / a.tiles_per_split;  // no empty slices
     if (a.n_split > 1) {
-        const size_t rows = (size_t)a.batch * a.Hkv * a.n_split * a.r_pad;
-        float* ws = workspace(rows * (D + 2));
-        if (!ws) return VLA_K_ERR_LAUNCH;
-        a.part_o = ws;
-        a.part_ml = ws + rows * D;
+        const int rc = bind_scratch(a, sc, st, (size_t)a.batch * a.Hkv * a.n_split * a.r_pad, D);
+        if (rc != VLA_K_OK) return rc;
     }
-    hipStream_t st = (hipStream_t)stream;
+    if (sc.kind == Scratch::DRY) return VLA_K_OK;
+    a.arrive = nullptr;
     switch (nw) {
         case 1: return launch_nw<T, D, 1>(a, st);
         case 2: return launch_nw<T, D, 2>(a, st);
@@ -1338,26 +1351,24 @@ int launch_d(AttnArgs& a, vla_stream_t stream) {
 }
 
 template <typename T>
-int launch_t(AttnArgs& a, int D, vla_stream_t stream) {
+int launch_t(AttnArgs& a, int D, vla_stream_t stream, Scratch& sc) {
     switch (D) {
-        case 48: return launch_d<T, 48>(a, stream);
-        case 64: return launch_d<T, 64>(a, stream);
-        case 128: return launch_d<T, 128>(a, stream);
+        case 48: return launch_d<T, 48>(a, stream, sc);
+        case 64: return launch_d<T, 64>(a, stream, sc);
+        case 128: return launch_d<T, 128>(a, stream, sc);
         case 256:
             // fp32 tiles of 256-wide heads would not fit the LDS budget; only bf16 is built.
-            if constexpr (sizeof(T) == 2) return launch_d<T, 256>(a, stream);
+            if constexpr (sizeof(T) == 2) return launch_d<T, 256>(a, stream, sc);
             else return VLA_K_ERR_SHAPE;
         default: return VLA_K_ERR_SHAPE;
     }
 }
 
-}  // namespace
-
-extern "C" int vla_attn_prefix_suffix(const void* q, const void* k_cache, const void* vt_cache, void* out, int dtype,
-                                      int batch, int S, int n_q_heads, int n_kv_heads, int head_dim, int t_max,
-                                      int n_keys, float scale, int mask_kind, int n_prefix, int pad_start, int pad_end,
-                                      const float* mask, vla_stream_t stream) {
-    if (!q || !k_cache || !vt_cache || !out || batch < 0 || S <= 0 || n_q_heads <= 0 || n_kv_heads <= 0)
+int attn_entry(const void* q, const void* k_cache, const void* vt_cache, void* out, int dtype, int batch, int S, int n_q_heads,
+               int n_kv_heads, int head_dim, int t_max, int n_keys, float scale, int mask_kind, int n_prefix, int pad_start,
+               int pad_end, const float* mask, vla_stream_t stream, Scratch& sc) {
+    const bool dry = sc.kind == Scratch::DRY;
+    if ((!dry && (!q || !k_cache || !vt_cache || !out)) || batch < 0 || S <= 0 || n_q_heads <= 0 || n_kv_heads <= 0)
         return VLA_K_ERR_ARG;
     if (n_q_heads % n_kv_heads || t_max % 8 || n_keys <= 0 || n_keys > t_max) return VLA_K_ERR_SHAPE;
     if (mask_kind < VLA_MASK_NONE || mask_kind > VLA_MASK_PI0_STATE) return VLA_K_ERR_ARG;
@@ -1369,7 +1380,47 @@ extern "C" int vla_attn_prefix_suffix(const void* q, const void* k_cache, const 
     a.n_prefix = n_prefix < 0 ? 0 : (n_prefix > n_keys ? n_keys : n_prefix);
     a.pad_start = pad_start; a.pad_end = pad_end; a.mask = mask;
     a.p2 = dtype == VLA_DT_BF16_P2;
-    if (dtype == VLA_DT_BF16 || dtype == VLA_DT_BF16_P2) return launch_t<bf16_t>(a, head_dim, stream);
-    if (dtype == VLA_DT_F32) return launch_t<float>(a, head_dim, stream);
+    if (dtype == VLA_DT_BF16 || dtype == VLA_DT_BF16_P2) return launch_t<bf16_t>(a, head_dim, stream, sc);
+    if (dtype == VLA_DT_F32) return launch_t<float>(a, head_dim, stream, sc);
     return VLA_K_ERR_ARG;
+}
+
+}  // namespace
+
+extern "C" int vla_attn_prefix_suffix(const void* q, const void* k_cache, const void* vt_cache, void* out, int dtype,
+                                      int batch, int S, int n_q_heads, int n_kv_heads, int head_dim, int t_max,
+                                      int n_keys, float scale, int mask_kind, int n_prefix, int pad_start, int pad_end,
+                                      const float* mask, vla_stream_t stream) {
+    Scratch sc;
+    sc.kind = Scratch::LIBRARY;
+    return attn_entry(q, k_cache, vt_cache, out, dtype, batch, S, n_q_heads, n_kv_heads, head_dim, t_max, n_keys, scale,
+                      mask_kind, n_prefix, pad_start, pad_end, mask, stream, sc);
+}
+
+extern "C" size_t vla_attn_workspace_bytes(int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
+                                           int n_keys) {
+    Scratch sc;
+    sc.kind = Scratch::DRY;
+    const int t_max = (n_keys + 7) / 8 * 8;
+    const int rc = attn_entry(nullptr, nullptr, nullptr, nullptr, dtype, batch, S, n_q_heads, n_kv_heads, head_dim, t_max,
+                              n_keys, 1.0f, VLA_MASK_NONE, 0, 0, 0, nullptr, nullptr, sc);
+    return rc == VLA_K_OK ? sc.need : 0;
+}
+
+extern "C" int vla_attn_prefix_suffix_ws(const void* q, const void* k_cache, const void* vt_cache, void* out, int dtype,
+                                         int batch, int S, int n_q_heads, int n_kv_heads, int head_dim, int t_max,
+                                         int n_keys, float scale, int mask_kind, int n_prefix, int pad_start,
+                                         int pad_end, const float* mask, void* workspace, size_t workspace_bytes,
+                                         vla_stream_t stream) {
+    Scratch sc;
+    sc.kind = Scratch::CALLER;
+    sc.base = (unsigned char*)workspace;
+    sc.bytes = workspace ? workspace_bytes : 0;
+    return attn_entry(q, k_cache, vt_cache, out, dtype, batch, S, n_q_heads, n_kv_heads, head_dim, t_max, n_keys, scale,
+                      mask_kind, n_prefix, pad_start, pad_end, mask, stream, sc);
+}
+
+extern "C" int vla_kernels_init(void) {
+    (void)tuning();
+    return VLA_K_OK;
 }

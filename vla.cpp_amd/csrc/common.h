@@ -8,7 +8,39 @@
 
 #define VLA_WAVE 64
 
+#if defined(__HIP_DEVICE_COMPILE__) && !defined(__gfx950__)
+#error "these kernels are written for gfx950 (MI355X) only"
+#endif
+
 namespace vk {
+
+// Overrides of the by-shape kernel selection, for tests and tuning.  Read from the
+// environment once (vla_kernels_init, or the first launch that asks) and again only by
+// vla_kernels_reload_env: no launch path calls getenv.
+struct Tuning {
+    int attn_dl = -1;           // VLA_ATTN_DL: 0 pins the register-staged LDS kernel for 64-wide bf16 heads
+    int attn_slices = 0;        // VLA_ATTN_SLICES: 1 | 2 key slices per row tile in the direct-to-LDS kernel
+    int attn_split = -1;        // VLA_ATTN_SPLIT: key slices across workgroups (<= 0 pins one)
+    bool attn_split_set = false;
+    bool attn_part_f32 = false;  // VLA_ATTN_PART_F32: fp32 partials where fp16 would be used
+    bool attn_no_arrive = false; // VLA_ATTN_NO_ARRIVE: no in-launch merge by the last slice to arrive
+    bool attn_no_direct = false; // VLA_ATTN_NO_DIRECT: never the register-direct kernel
+    int attn_direct_rows = 32;   // VLA_ATTN_DIRECT_ROWS: row limit of the register-direct kernel
+    int gemm_tile = -1;          // VLA_GEMM_TILE: 0..5
+    int gemm_dl = -1;            // VLA_GEMM_DL: 0 pins the register-staged GEMM
+    int gemm_stages = 0;         // VLA_GEMM_STAGES: ring depth of the direct-to-LDS GEMM
+    int ternary_tile = 0;        // VLA_TERNARY_TILE: 64 | 128 | 256
+};
+const Tuning& tuning();
+
+// Scratch memory the library owns on behalf of entry points whose signature has no
+// workspace argument: one block per (purpose, device, stream), grown on demand and never
+// freed before the process ends, so a captured graph that holds an older block keeps
+// pointing at live memory and calls on different streams never share a block.  New blocks
+// are zero-filled.  Allocates (never under stream capture: run a shape once before
+// capturing it).  Returns nullptr when the allocation fails.
+enum { SCRATCH_ATTN = 0, SCRATCH_ROWSUM = 1 };
+void* stream_scratch(int purpose, hipStream_t stream, size_t bytes);
 
 typedef uint16_t bf16_t;  // raw bf16 bits
 

@@ -873,6 +873,4 @@ int bitvla_gather_rows_bf16(const uint16_t* in, uint16_t* out, const int32_t* ro
     return VLA_CHECK_LAUNCH();
 }
 
-const char* vla_kernels_arch(void) { return "gfx950"; }
-
 }  // extern "C"

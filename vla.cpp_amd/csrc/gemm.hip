@@ -1251,8 +1251,7 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
     if constexpr (kEpi != EPI_TERNARY) {
         // VLA_GEMM_TILE = 0..5 pins the tile configuration and VLA_GEMM_STAGES the ring depth
         // of the direct-to-LDS kernel (tests and tuning); unset = by shape.
-        const char* env = getenv("VLA_GEMM_TILE");
-        int cfg = env ? atoi(env) : -1;
+        int cfg = tuning().gemm_tile;
         const long m128 = (a.M + 127) / 128, m64 = (a.M + 63) / 64;
         const long wgs0 = m128 * ((n_tiles + 1) / 2), wgs2 = m128 * n_tiles, wgs4 = m64 * n_tiles;
         if (cfg < 0) {
@@ -1273,13 +1272,11 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
         // CU, 256 CUs), and only then how far ahead each workgroup fetches.
         bool dl = false;
         if constexpr (std::is_same<T, bf16_t>::value) {
-            const char* e = getenv("VLA_GEMM_DL");
-            dl = !(e && atoi(e) == 0) && a.K % 16 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
+            dl = tuning().gemm_dl != 0 && a.K % 16 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
         }
         if (a.norm_eps >= 0.f && !(dl && (kEpi == EPI_QKV || kEpi == EPI_GLU))) return VLA_K_ERR_SHAPE;  // only that kernel takes the row statistics
         if (dl) {
-            const char* es = getenv("VLA_GEMM_STAGES");
-            int ns = es ? atoi(es) : 0;
+            int ns = tuning().gemm_stages;
             const long wgs = cfg == 0 ? wgs0 : (cfg == 2 || cfg == 3 ? wgs2 : wgs4);
             switch (cfg) {
                 case 5:  // 40 KiB per stage, one workgroup per CU
@@ -1324,8 +1321,7 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
         }
     } else {
         // VLA_TERNARY_TILE = 64 | 128 | 256 pins the tile (tests and tuning); unset = by shape.
-        const char* env = getenv("VLA_TERNARY_TILE");
-        const int force = env ? atoi(env) : 0;
+        const int force = tuning().ternary_tile;
         // Enough 128 x 256 tiles for half the chip: the large-M kernel, two workgroups per
         // CU (measured faster than one 256 x 256 workgroup: fewer wavefronts per barrier).
         const int n256 = (a.N + 255) / 256;
@@ -1356,9 +1352,6 @@ __global__ void rowsum_i8_kernel(const int8_t* __restrict__ A, int32_t* __restri
     s = wave_sum_i(s);
     if (threadIdx.x == 0) rowsum[blockIdx.x] = s;
 }
-
-int32_t* g_rowsum = nullptr;
-int g_rowsum_cap = 0;
 
 template <bool ROPE, bool GLU = false>
 int launch_gemv_norm(const GemmArgs& a, vla_stream_t stream) {
@@ -1644,16 +1637,12 @@ int bitlinear_int8xint2_m(int8_t* A, int8_t* B, uint16_t* out, float* s, float* 
                           vla_stream_t stream) {
     if (!A || !B || !out || !s || !ws || M < 0) return VLA_K_ERR_ARG;
     if (M == 0) return VLA_K_OK;
-    if (M > g_rowsum_cap) {
-        if (g_rowsum) (void)hipFree(g_rowsum);
-        g_rowsum = nullptr;
-        g_rowsum_cap = 0;
-        const int cap = M < 4096 ? 4096 : M;
-        if (hipMalloc((void**)&g_rowsum, (size_t)cap * sizeof(int32_t)) != hipSuccess) return VLA_K_ERR_LAUNCH;
-        g_rowsum_cap = cap;
-    }
-    rowsum_i8_kernel<<<M, 64, 0, (hipStream_t)stream>>>(A, g_rowsum, K);
-    return vla_ternary_gemm(A, (const uint32_t*)B, out, nullptr, s, g_rowsum, ws, bitvla_ws_num(N, K), M, N, K, stream);
+    // the reference's signature carries no row sums: they go into a block the library keeps
+    // for this stream (calls on one stream are ordered, other streams have their own block)
+    int32_t* rowsum = (int32_t*)stream_scratch(SCRATCH_ROWSUM, (hipStream_t)stream, (size_t)M * sizeof(int32_t));
+    if (!rowsum) return VLA_K_ERR_LAUNCH;
+    rowsum_i8_kernel<<<M, 64, 0, (hipStream_t)stream>>>(A, rowsum, K);
+    return vla_ternary_gemm(A, (const uint32_t*)B, out, nullptr, s, rowsum, ws, bitvla_ws_num(N, K), M, N, K, stream);
 }
 
 int bitlinear_int8xint2(int8_t* A, int8_t* B, uint16_t* out, float* s, float* ws, int M, int N, int K,

@@ -115,6 +115,7 @@ class BitvlaLm : public ModelArch {
     std::vector<float> E_lang_, act_emb_;
     DevBuf out_norm_, W_out_, b_out_;
     RopeTable rope_;
+    AttnWorkspace attn_ws_;
     DevBuf h_, hn_, q8_, s_, rowsum_, qkv_, q_, att_, o_, emb_bcast_, hfin_, x_, gu_, act_;
     hipStream_t last_stream_ = nullptr;
 };
@@ -194,6 +195,10 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
         x_.alloc((size_t)n_act_ * B * A_ * 4);
         zeros_.alloc((size_t)n_act_ * B * A_ * 4);
         zeros_.zero();
+        attn_ws_.reset();
+        attn_ws_.plan(VLA_DT_BF16_P2, B, P, Hq_, Hkv_, D_, P);  // prefill
+        for (int t = 0; t < n_act_; ++t) attn_ws_.plan(VLA_DT_BF16_P2, B, 1, Hq_, Hkv_, D_, P + t + 1);  // appended tokens
+        attn_ws_.commit();
         ++alloc_gen_;
         std::vector<int32_t> pos(P + n_act_);
         for (int i = 0; i < P + n_act_; ++i) pos[i] = i;  // src/models/bitvla.cpp positions 0..seq-1
@@ -251,8 +256,9 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
         if (!(fused && S == 1 && w.Wqkv.paired.get()))
             VLA_K(vla_qkv_split_rope_append(qkv_.get(), cos_t, sin_t, q_.get(), w.kv.k.get(), w.kv.vt.get(), VLA_DT_BF16, M, S,
                                             Hq_, Hkv_, D_, w.kv.t_max, tok_offset, C.stream));
-        VLA_K(vla_attn_prefix_suffix(q_.get(), w.kv.k.get(), w.kv.vt.get(), att_.get(), VLA_DT_BF16_P2, M / S, S, Hq_, Hkv_,
-                                     D_, w.kv.t_max, n_keys, scale, VLA_MASK_NONE, n_keys, 0, 0, nullptr, C.stream));
+        VLA_K(vla_attn_prefix_suffix_ws(q_.get(), w.kv.k.get(), w.kv.vt.get(), att_.get(), VLA_DT_BF16_P2, M / S, S, Hq_, Hkv_,
+                                        D_, w.kv.t_max, n_keys, scale, VLA_MASK_NONE, n_keys, 0, 0, nullptr, attn_ws_.buf.get(),
+                                        attn_ws_.buf.bytes(), C.stream));
         // O projection and the residual add of the hidden stream in one launch
         if (fused) {
             VLA_K(vla_rmsnorm_ternary_gemv(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), eps_, w.Wo.packed.as<uint32_t>(),

@@ -24,7 +24,7 @@ struct bitvla_lm_hip_ctx {
     std::vector<bitvla_lm_layer_hip> layers;
     std::vector<char> bound;
     const uint16_t* out_norm = nullptr;
-    vla::DevBuf cos, sin, h, q8, s, rowsum, q, k, v, kc, vtc, att, gate_up, act;
+    vla::DevBuf cos, sin, h, q8, s, rowsum, q, k, v, kc, vtc, att, gate_up, act, attn_ws;
 };
 
 namespace {
@@ -47,8 +47,9 @@ int run(bitvla_lm_hip_ctx* c, const uint16_t* d_in, uint16_t* d_out, int seq, hi
         VLA_K(vla_rope_neox(c->q.get(), c->cos.as<float>(), c->sin.as<float>(), VLA_DT_BF16, seq, seq, c->n_q, c->hd, st));
         VLA_K(vla_rope_neox(c->k.get(), c->cos.as<float>(), c->sin.as<float>(), VLA_DT_BF16, seq, seq, c->n_kv, c->hd, st));
         VLA_K(vla_kv_append(c->kc.get(), c->vtc.get(), c->k.get(), c->v.get(), VLA_DT_BF16, 1, c->n_kv, c->hd, c->t_max, 0, seq, st));
-        VLA_K(vla_attn_prefix_suffix(c->q.get(), c->kc.get(), c->vtc.get(), c->att.get(), VLA_DT_BF16_P2, 1, seq, c->n_q, c->n_kv,
-                                     c->hd, c->t_max, seq, scale, VLA_MASK_NONE, seq, 0, 0, nullptr, st));
+        VLA_K(vla_attn_prefix_suffix_ws(c->q.get(), c->kc.get(), c->vtc.get(), c->att.get(), VLA_DT_BF16_P2, 1, seq, c->n_q, c->n_kv,
+                                        c->hd, c->t_max, seq, scale, VLA_MASK_NONE, seq, 0, 0, nullptr, c->attn_ws.get(),
+                                        c->attn_ws.bytes(), st));
         VLA_K(vla_rmsnorm_act_quant_bf16(c->att.as<uint16_t>(), w.attn_sub_norm_w, q8, s, rs, c->rms_eps, seq, hq, st));
         VLA_K(vla_ternary_gemm_add(q8, (const uint32_t*)w.o_packed, h, h, s, rs, w.o_ws, 1, seq, H, hq, st));
         VLA_K(vla_rmsnorm_act_quant_bf16(h, w.ffn_norm_w, q8, s, rs, c->rms_eps, seq, H, st));
@@ -107,6 +108,14 @@ bitvla_lm_hip_ctx* bitvla_lm_hip_init(int hidden, int n_q, int n_kv, int head_di
         c->att.alloc(S * hq * 2);
         c->gate_up.alloc(S * 2 * ffn * 2);
         c->act.alloc(S * ffn * 2);
+        // attention scratch for the most demanding sequence length, so forward() never allocates
+        size_t ws = 0;
+        for (int seq = 1; seq <= max_seq; ++seq) {
+            const size_t b = vla_attn_workspace_bytes(VLA_DT_BF16_P2, 1, seq, n_q, n_kv, head_dim, seq);
+            if (b > ws) ws = b;
+        }
+        c->attn_ws.alloc(ws);
+        c->attn_ws.zero();
         return c;
     } catch (const std::exception& e) {
         std::fprintf(stderr, "vla(bitvla_lm_hip): init failed: %s\n", e.what());

@@ -135,6 +135,7 @@ class FlowExpert : public ModelArch {
     RopeTable rope_prefill_, rope_self_, rope_cross_;
     DevBuf prefix_, prefix_n_, tmpk_, tmpv_, lead_, x0_, xt_, h_, hn_, q_, att_, mid_;
     KVLayer tmp_kv_;
+    AttnWorkspace attn_ws_;
     std::mt19937 rng_{std::random_device{}()};
     hipStream_t last_stream_ = nullptr;
 };
@@ -379,6 +380,7 @@ void FlowExpert::allocate(int B, int P, int P_txt) {
     P_txt_ = P_txt;
     ++alloc_gen_;
     const size_t es = dtype_size(dt_);
+    attn_ws_.reset();
     for (LayerW& w : layers_) {
         // alternating layers: text rows, or image rows (all rows when there is no text:
         // vl_txt = vl_img then, gr00tn1d6.cpp:443)
@@ -386,7 +388,9 @@ void FlowExpert::allocate(int B, int P, int P_txt) {
         const int tmax = round_up(prefix + (w.is_self ? S_ : 0), 64);
         w.kv.create(dt_, B, Hkv_, D_, tmax);
         w.kv.n_prefix = prefix;
+        attn_ws_.plan(dt_, B, S_, Hq_, Hkv_, D_, prefix + (w.is_self ? S_ : 0));
     }
+    attn_ws_.commit();
     if (arch_ == Arch::SMOLVLA) {
         tmp_kv_.create(dt_, B, Hkv_, D_, round_up(P, 64));
         tmpk_.alloc((size_t)B * P * Hkv_ * D_ * es);
@@ -604,7 +608,7 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 mask.pad_end = pad_end_;
                 mask.kind = w.is_self ? suffix_mask_ : VLA_MASK_NONE;
                 const int n_keys = w.is_self ? w.kv.n_prefix + S_ : w.kv.n_prefix;
-                flash_attention(C, Q, w.kv, n_keys, mask, scale, att);
+                flash_attention(C, Q, w.kv, n_keys, mask, scale, att, attn_ws_);
                 Tensor Wo = tensor_2d(w.Wo.get(), dt_, (int64_t)Hq_ * D_, W_);
                 if (adarms_) {
                     // h1 = x + o_out * gate_attn; h = h1 + mlp_out * gate_ffn (pi05.cpp:273-281)

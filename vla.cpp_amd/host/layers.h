@@ -72,6 +72,25 @@ struct KVLayer {
     }
 };
 
+// Scratch memory of a handle's attention launches (key-slice partials and arrival counters):
+// owned by the handle, so that handles never share any -- the reference's contract is one
+// call at a time per handle (include/vla.h:18-19), not per process.  plan() every shape the
+// handle will launch, then commit() (allocates and zero-fills; invalidates captured graphs
+// that hold the old block, so the owner bumps its launch key).
+struct AttnWorkspace {
+    DevBuf buf;
+    size_t need = 0;
+    void reset() { need = 0; }
+    void plan(int dtype, int batch, int S, int Hq, int Hkv, int D, int n_keys) {
+        const size_t b = vla_attn_workspace_bytes(dtype, batch, S, Hq, Hkv, D, n_keys);
+        if (b > need) need = b;
+    }
+    void commit() {
+        buf.alloc(need);
+        buf.zero();
+    }
+};
+
 // Mask as the attention kernel generates it (masks are data in the reference:
 // src/models/smolvla.cpp:1651-1669, src/models/pi0.cpp:638-653).
 struct MaskSpec {
@@ -159,10 +178,11 @@ inline bool rmsnorm_qkv_rope_append(Ctx& C, const Tensor& x, const Tensor& W_fol
 // attn.h:48-58 (flash_attention) over the resident cache: Q [D, Hq, S, B]
 // token-major, keys [0, n_keys).
 inline void flash_attention(Ctx& C, const Tensor& Q, const KVLayer& kv, int n_keys, const MaskSpec& mask, float scale,
-                            Tensor& out) {
-    VLA_K(vla_attn_prefix_suffix(Q.data, kv.k.get(), kv.vt.get(), out.data, Q.dtype, (int)Q.ne[3], (int)Q.ne[2],
-                                 (int)Q.ne[1], kv.n_kv_heads, (int)Q.ne[0], kv.t_max, n_keys, scale, mask.kind,
-                                 kv.n_prefix, mask.pad_start, mask.pad_end, nullptr, C.stream));
+                            Tensor& out, const AttnWorkspace& ws) {
+    VLA_K(vla_attn_prefix_suffix_ws(Q.data, kv.k.get(), kv.vt.get(), out.data, Q.dtype, (int)Q.ne[3], (int)Q.ne[2],
+                                    (int)Q.ne[1], kv.n_kv_heads, (int)Q.ne[0], kv.t_max, n_keys, scale, mask.kind,
+                                    kv.n_prefix, mask.pad_start, mask.pad_end, nullptr, ws.buf.get(), ws.buf.bytes(),
+                                    C.stream));
 }
 
 // embed.h:61-73, log-spaced periods, sin first.
