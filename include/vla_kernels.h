@@ -225,6 +225,22 @@ VLA_KAPI int vla_attn_prefix_suffix_ws(const void* q, const void* k_cache, const
                                        int pad_start, int pad_end, const float* mask, void* workspace,
                                        size_t workspace_bytes, vla_stream_t stream);
 
+/* vla_attn_prefix_suffix for callers that cannot allocate.  It has no counterpart in the
+ * reference; it is for code under HIP graph capture, tight serving loops and harnesses that
+ * forbid hipMalloc.  Same arguments, same results (bit for bit), but the scratch memory is a
+ * fixed device array inside the library (VLA_ATTN_NOALLOC_SCRATCH_BYTES per GPU, held until
+ * the process ends) and no allocating call is made; a shape that needs more returns
+ * VLA_K_ERR_WORKSPACE and launches nothing (vla_attn_workspace_bytes tells in advance).
+ * Every call on a GPU uses that GPU's one array: calls that may overlap on the device
+ * (different streams) race and must be serialised by the caller.  The array's address is
+ * looked up on the first call per device; vla_kernels_init() does it ahead of time. */
+#define VLA_ATTN_NOALLOC_SCRATCH_BYTES ((size_t)(64u << 10) + ((size_t)16u << 20))
+VLA_KAPI int vla_attn_prefix_suffix_noalloc(const void* q, const void* k_cache, const void* vt_cache, void* out,
+                                            int dtype, int batch, int S, int n_q_heads, int n_kv_heads,
+                                            int head_dim, int t_max, int n_keys, float scale, int mask_kind,
+                                            int n_prefix, int pad_start, int pad_end, const float* mask,
+                                            vla_stream_t stream);
+
 /* --------------------------------------------------------- flow-matching glue */
 
 /* Suffix embedding h[b][s][:] for one denoise step (stand-in for
@@ -424,7 +440,8 @@ VLA_KAPI int bitvla_lm_hip_forward(bitvla_lm_hip_ctx* ctx, const uint16_t* d_in,
 VLA_KAPI const char* vla_kernels_arch(void); /* "gfx950" */
 
 /* Optional set-up for the current device, so that no later call has to do it lazily: reads
- * the tuning overrides from the environment.  0 or a vla_kstatus. */
+ * the tuning overrides from the environment and resolves the fixed scratch array of
+ * vla_attn_prefix_suffix_noalloc.  0 or a vla_kstatus. */
 VLA_KAPI int vla_kernels_init(void);
 /* Reads the tuning overrides (VLA_ATTN_*, VLA_GEMM_*, VLA_TERNARY_TILE; tests and tuning
  * only) from the environment again.  No launch path reads the environment. */

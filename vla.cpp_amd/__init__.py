@@ -42,6 +42,7 @@ KERNEL_API = {
     "vla_fold_norm_weight_host": [_vp, _vp, _i, _i, _i, _vp],
     "vla_qkv_split_rope_append": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp],
     "vla_attn_prefix_suffix": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp],
+    "vla_attn_prefix_suffix_noalloc": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp],
     "vla_attn_prefix_suffix_ws": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp,
                                   ctypes.c_size_t, _vp],
     "vla_attn_workspace_bytes": [_i, _i, _i, _i, _i, _i, _i],

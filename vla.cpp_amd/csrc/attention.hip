@@ -38,6 +38,7 @@
 #include <math.h>
 #include <stdlib.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -1122,7 +1123,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
 //                            every launch that uses them leaves them at zero)
 //     [ARRIVE_BYTES, ...)    partials, rows x (D + 2) floats
 // It comes from the library's per-stream blocks (vla_attn_prefix_suffix), from the caller
-// (vla_attn_prefix_suffix_ws);
+// (vla_attn_prefix_suffix_ws) or from a static device array (vla_attn_prefix_suffix_noalloc);
 // a dry run only reports the size (vla_attn_workspace_bytes).
 constexpr size_t ARRIVE_BYTES = (size_t)ARRIVE_MAX_UNITS * sizeof(int);
 struct Scratch {
@@ -1387,6 +1388,32 @@ int attn_entry(const void* q, const void* k_cache, const void* vt_cache, void* o
 
 }  // namespace
 
+// The no-allocation entry point's scratch: the block a sliced call needs, as a static device
+// array (zero-initialised when the code object is loaded; every GPU the library runs on holds
+// its own copy until the process ends).  In host code the name is only a handle for
+// hipGetSymbolAddress: the address kernels and copies use is looked up once per device.
+static __device__ __align__(256) unsigned char scratch[VLA_ATTN_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+unsigned char* g_scratch_ptr[MAX_DEVICES] = {};
+std::mutex g_scratch_ptr_mu;
+
+// The current device's copy of `scratch`, looked up on first use with that device current.
+int noalloc_scratch(unsigned char** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return VLA_K_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lk(g_scratch_ptr_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return VLA_K_ERR_LAUNCH;
+        g_scratch_ptr[dev] = (unsigned char*)p;
+    }
+    *out = g_scratch_ptr[dev];
+    return VLA_K_OK;
+}
+}  // namespace
+
 extern "C" int vla_attn_prefix_suffix(const void* q, const void* k_cache, const void* vt_cache, void* out, int dtype,
                                       int batch, int S, int n_q_heads, int n_kv_heads, int head_dim, int t_max,
                                       int n_keys, float scale, int mask_kind, int n_prefix, int pad_start, int pad_end,
@@ -1420,7 +1447,21 @@ extern "C" int vla_attn_prefix_suffix_ws(const void* q, const void* k_cache, con
                       mask_kind, n_prefix, pad_start, pad_end, mask, stream, sc);
 }
 
+extern "C" int vla_attn_prefix_suffix_noalloc(const void* q, const void* k_cache, const void* vt_cache, void* out,
+                                              int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
+                                              int t_max, int n_keys, float scale, int mask_kind, int n_prefix,
+                                              int pad_start, int pad_end, const float* mask, vla_stream_t stream) {
+    Scratch sc;
+    sc.kind = Scratch::CALLER;
+    const int rc = noalloc_scratch(&sc.base);
+    if (rc != VLA_K_OK) return rc;
+    sc.bytes = VLA_ATTN_NOALLOC_SCRATCH_BYTES;
+    return attn_entry(q, k_cache, vt_cache, out, dtype, batch, S, n_q_heads, n_kv_heads, head_dim, t_max, n_keys, scale,
+                      mask_kind, n_prefix, pad_start, pad_end, mask, stream, sc);
+}
+
 extern "C" int vla_kernels_init(void) {
     (void)tuning();
-    return VLA_K_OK;
+    unsigned char* p = nullptr;
+    return noalloc_scratch(&p);
 }
