@@ -1,0 +1,289 @@
+"""Pins for oracle/chunk.py: the composition of the pinned primitives into whole action chunks.
+
+oracle/chunk.py decides what the primitives cannot: which layers are self / cross layers, the
+position bases of prefix, suffix and cross queries, the masks, the sign and size of dt, the time
+fed to each step, where the state token sits, which rows feed the Euler update.  Three kinds of
+checks hold it, none of which re-types its code:
+
+  1. tests/chunk_restatement.py, an independent float64 torch statement of every architecture
+     written from the reference's graph builders, at tiny dimensions;
+  2. closed forms: with Wo = 0 (and W_down = 0) the layers are the identity on the residual
+     stream, so x_T = x_0 + dt * sum_s W_out norm(W_in x_s + b_in + time(t_s)) + b_out -- a few
+     lines of numpy that know nothing about attention;
+  3. sensitivity: the mistakes this file exists to catch (self / cross parity, a position base
+     off by one, dt's sign, the causal block, the state row) each move the restatement's result
+     by orders of magnitude more than the tolerance, so the comparison in 1 can see them.
+
+BitVLA (bitvla_chunk: prefill + token-by-token append) is integer arithmetic between bf16
+roundings, so its pin is exact: the same chunk as ONE pass over prefix + action tokens with a
+prefix-LM mask, composed here from the pinned primitives in another order (no cache, no
+incremental positions), must give the same bits.
+"""
+import copy
+import math
+
+import numpy as np
+import pytest
+
+import oracle as orc
+from oracle import chunk as orc_chunk
+
+import chunk_restatement as ref
+from util import pkg
+
+from vla_cpp_amd import checkpoint as ckpt  # noqa: E402
+
+TOL = 2e-5  # fp32 oracle (fp64 accumulation inside a product, fp32 between ops) vs float64 throughout
+
+
+def tiny(arch, **kw):
+    """Few layers, narrow heads, a handful of tokens; every structural feature kept."""
+    if arch == "smolvla":
+        c = ckpt.smolvla_config(n_layers=4, dtype="f32", suffix_mask=kw.pop("suffix_mask", 1), num_steps=3)
+        c.update(n_q_heads=6, n_kv_heads=2, head_dim=8, hidden=24, expert_h=20, n_img=2, n_lang=4, n_suffix=5,
+                 max_action_dim=6, max_state_dim=5, real_action_dim=5, real_state_dim=5, vocab=11)
+    elif arch == "pi0":
+        c = ckpt.pi0_config(n_layers=3, dtype="f32", num_steps=3)
+        c.update(n_q_heads=4, n_kv_heads=1, head_dim=16, hidden=24, expert_h=16, n_img=3, n_lang=3, n_suffix=5,
+                 max_action_dim=6, max_state_dim=5, real_action_dim=6, real_state_dim=5, vocab=11)
+    elif arch == "pi05":
+        c = ckpt.pi05_config(n_layers=3, dtype="f32", num_steps=3)
+        c.update(n_q_heads=4, n_kv_heads=1, head_dim=16, hidden=24, expert_h=16, n_img=3, n_lang=5, n_suffix=4,
+                 max_action_dim=6, max_state_dim=5, real_action_dim=6, real_state_dim=5, vocab=11)
+    elif arch == "gr00t_n1d5":
+        c = ckpt.gr00t_config(n_layers=4, dtype="f32", num_steps=3, n_suffix=5)
+        c.update(n_q_heads=3, n_kv_heads=3, head_dim=8, hidden=20, expert_h=24, n_img=4, max_action_dim=6,
+                 max_state_dim=7, real_action_dim=6, real_state_dim=7)
+    else:
+        c = ckpt.gr00t_n1d6_config(n_layers=8, dtype="f32", num_steps=2, n_suffix=5, attend_text_every_n=kw.pop("every", 2),
+                                   dit_interleave=kw.pop("interleave", 1))
+        c.update(n_q_heads=3, n_kv_heads=3, head_dim=8, hidden=20, expert_h=24, n_img=4, n_lang=3, max_action_dim=6,
+                 max_state_dim=7, real_action_dim=6, real_state_dim=7, vocab=11)
+    c.update(kw)
+    return c
+
+
+def obs_for(cfg, r, n_views=2, n_lang=None):
+    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "pi05") else 1)
+    o = dict(img_emb=r.standard_normal((n_views * cfg["n_img"], cfg["hidden"])).astype(np.float32), n_views=n_views,
+             noise=r.standard_normal((n_act, cfg["max_action_dim"])).astype(np.float32),
+             state=r.standard_normal(cfg["max_state_dim"]).astype(np.float32))
+    if cfg.get("vocab", 0) > 0:
+        o["lang"] = r.integers(0, cfg["vocab"], cfg["n_lang"] if n_lang is None else n_lang).astype(np.int32)
+    return o
+
+
+def big_weights(cfg, seed):
+    """Synthetic weights scaled up so that attention, rotation and masks matter to the output
+    (with N(0, 0.02) projections a tiny model's softmax is nearly uniform)."""
+    w = ckpt.synth_weights(cfg, seed=seed)
+    for k in list(w):
+        if k.endswith(("Wqkv", "Wq", "Wkv", "Wk_x", "Wv_x", "Wo", "W_out", "Wgu", "Wd", "W1", "W2")):
+            w[k] = (w[k] * np.float32(12.0)).astype(np.float32)
+    return w
+
+
+def rel(a, b):
+    return float(np.abs(np.asarray(a, np.float64) - b).max() / np.abs(b).max())
+
+
+CASES = [("smolvla", {}), ("smolvla", dict(suffix_mask=0)), ("smolvla", dict(ffn_dim=12, time_mlp=1)), ("pi0", {}),
+         ("pi0", dict(ffn_dim=12, time_mlp=1)), ("pi05", {}), ("pi05", dict(ffn_dim=12)), ("gr00t_n1d5", {}),
+         ("gr00t_n1d5", dict(ffn_dim=12)), ("gr00t_n1d6", {}), ("gr00t_n1d6", dict(every=1)),
+         ("gr00t_n1d6", dict(interleave=0, ffn_dim=12))]
+
+
+@pytest.mark.parametrize("arch,kw", CASES, ids=["%s-%s" % (a, "-".join("%s%s" % i for i in k.items()) or "base") for a, k in CASES])
+def test_chunk_oracle_against_the_float64_restatement(arch, kw):
+    cfg = tiny(arch, **dict(kw))
+    w = big_weights(cfg, seed=900 + len(kw))
+    r = np.random.default_rng(901)
+    # SmolVLA: fewer real text tokens than the capacity, so the padded range and the state position differ
+    o = obs_for(cfg, r, n_views=2, n_lang=2 if arch == "smolvla" else None)
+    got = orc_chunk.flow_expert_chunk(cfg, w, o)
+    want = ref.chunk(cfg, w, o)
+    assert got.shape == want.shape and np.isfinite(want).all()
+    assert rel(got, want) < TOL, rel(got, want)
+    assert np.all(got[:, cfg["real_action_dim"]:] == 0)
+
+
+def _mutants(arch, cfg):
+    """(name, cfg', weights -> weights', obs -> obs'): one structural mistake each, expressed on
+    the restatement's inputs or definition, never by editing the oracle."""
+    m = []
+    if arch == "smolvla":
+        m.append(("self/cross parity", dict(self_attn_every_n=1), None))   # every layer self
+        m.append(("causal block", dict(suffix_mask=0), None))
+    if arch == "gr00t_n1d6":
+        m.append(("text/image alternation", dict(attend_text_every_n=1), None))
+        m.append(("interleave", dict(dit_interleave=0), None))
+    m.append(("steps", dict(num_steps=cfg["num_steps"] + 1), None))
+    return m
+
+
+@pytest.mark.parametrize("arch", ["smolvla", "gr00t_n1d6", "pi0"])
+def test_structural_mistakes_are_far_outside_the_tolerance(arch):
+    # What the comparison above can see: changing the structure moves the chunk by >> TOL.
+    cfg = tiny(arch)
+    w = big_weights(cfg, seed=910)
+    o = obs_for(cfg, np.random.default_rng(911), n_lang=2 if arch == "smolvla" else None)
+    base = ref.chunk(cfg, w, o)
+    for name, delta, _ in _mutants(arch, cfg):
+        c2 = dict(cfg)
+        c2.update(delta)
+        w2 = w
+        if "self_attn_every_n" in delta or "dit_interleave" in delta:  # layers change kind: give them the weights they need
+            w2 = dict(big_weights(c2, seed=910))
+            for k in w:
+                if k in w2 and w2[k].shape == w[k].shape:
+                    w2[k] = w[k]
+        moved = rel(ref.chunk(c2, w2, o), base)
+        assert moved > 100 * TOL, (name, moved)
+    # positions: the suffix one slot further, the state row swapped for an action row
+    import chunk_restatement as R
+    keep = R.rope_neox
+    try:
+        R.rope_neox = lambda x, pos, base_: keep(x, [p + (1 if len(pos) == cfg["n_suffix"] else 0) for p in pos], base_)
+        if arch != "gr00t_n1d6":
+            assert rel(ref.chunk(cfg, w, o), base) > 100 * TOL
+    finally:
+        R.rope_neox = keep
+
+
+@pytest.mark.parametrize("arch", ["smolvla", "pi0", "gr00t_n1d5"])
+def test_zero_output_projections_give_the_closed_form(arch):
+    # Wo = 0 (and no FFN): every layer leaves the residual stream alone, attention included, so
+    # one step is v = W_out norm(h0) + b_out with h0 = W_in x + b_in + time(t) and x += dt v.
+    cfg = tiny(arch)
+    w = big_weights(cfg, seed=920)
+    for k in list(w):
+        if k.endswith(".Wo"):
+            w[k] = np.zeros_like(w[k])
+        if k.endswith(".bo"):
+            w[k] = np.zeros_like(w[k])
+    o = obs_for(cfg, np.random.default_rng(921), n_lang=3 if arch == "smolvla" else None)
+    got = orc_chunk.flow_expert_chunk(cfg, w, o)
+
+    W, steps = cfg["expert_h"], cfg["num_steps"]
+    x = o["noise"].astype(np.float64)
+    gr = arch == "gr00t_n1d5"
+    dt = (1.0 if gr else -1.0) / steps
+    for s in range(steps):
+        h = x @ w["act.W_in"].astype(np.float64).T + w["act.b_in"]
+        if not gr:
+            t = 1.0 + s * dt
+            half = W // 2
+            period = cfg["min_period"] * (cfg["max_period"] / cfg["min_period"]) ** (np.arange(half) / (half - 1))
+            h = h + np.concatenate([np.sin(2 * math.pi / period * t), np.cos(2 * math.pi / period * t)])
+            hn = h / np.sqrt((h * h).mean(-1, keepdims=True) + cfg["rms_eps"]) * w["act.norm"]
+        else:
+            mu = h.mean(-1, keepdims=True)
+            hn = (h - mu) / np.sqrt(((h - mu) ** 2).mean(-1, keepdims=True) + cfg["norm_out_eps"])
+        x = x + dt * (hn @ w["act.W_out"].astype(np.float64).T + w["act.b_out"])
+    x[:, cfg["real_action_dim"]:] = 0
+    assert rel(got, x) < TOL, rel(got, x)
+
+
+# ------------------------------------------------------------------ BitVLA: exact
+
+def _bitvla_tiny(ffn):
+    c = ckpt.bitvla_config(n_layers=2)
+    c.update(n_q_heads=4, n_kv_heads=2, head_dim=8, hidden=32, n_img=3, n_lang=4, n_suffix=3, max_action_dim=5,
+             real_action_dim=4, vocab=9)
+    if ffn:
+        c["ffn_dim"] = ffn
+    return c
+
+
+def _bitvla_one_pass(cfg, w, o):
+    """The chunk as a single pass over [prefix ; action tokens] under a prefix-LM mask: prefix rows
+    see the prefix, action row t sees the prefix and action rows <= t.  Per-row operations
+    (norms, quantisation, projections) do not depend on which other rows are present, and a key
+    hidden by -inf contributes an exact zero, so this must equal prefill + append bit for bit.
+    Layer sequence from run_layer, src/kernels/bitvla/bitvla_lm_cuda.cu:422-520."""
+    L, Hq, Hkv, D, H = cfg["n_layers"], cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"], cfg["hidden"]
+    P, n_act = cfg["n_img"] + cfg["n_lang"], cfg["n_suffix"]
+    N = P + n_act
+    F = cfg.get("ffn_dim", 0)
+    rb = orc.round_bf16
+    mask = np.zeros((N, N), np.float32)
+    for i in range(N):
+        for j in range(N):
+            if j >= P and j > i:
+                mask[i, j] = -np.inf
+    cos_t, sin_t = orc.rope_tables(np.arange(N, dtype=np.int32), D, cfg["rope_freq_base"])
+
+    def bl(x_bf, name):
+        t, ws = orc_chunk.bitvla_ternary(cfg, w, name, False)
+        q, s = orc.act_quant(x_bf)
+        return orc.from_bf16(orc.ternary_epilogue(orc.ternary_gemm_i32(q, t), s, ws))
+
+    h = rb(np.concatenate([o["img_emb"].reshape(cfg["n_img"], H), w["prefix.E_lang"][o["lang"]], w["act.emb"][:n_act]], 0))
+    for l in range(L):
+        p = "lm.%d." % l
+        y = bl(rb(orc.rms_norm(h, w[p + "attn_norm"], cfg["rms_eps"])), p + "Wqkv")
+        q = y[:, :Hq * D].reshape(N, Hq, D)
+        k = y[:, Hq * D:(Hq + Hkv) * D].reshape(N, Hkv, D)
+        v = y[:, (Hq + Hkv) * D:].reshape(N, Hkv, D)
+        q, k = rb(orc.rope_neox(q, cos_t, sin_t)), rb(orc.rope_neox(k, cos_t, sin_t))
+        att = rb(orc.attention(q, k, v, mask, 1.0 / math.sqrt(D)))
+        h = rb(h + bl(rb(orc.rms_norm(att, w[p + "sub_norm"], cfg["rms_eps"])), p + "Wo"))
+        if F:
+            gu = bl(rb(orc.rms_norm(h, w[p + "ffn_norm"], cfg["rms_eps"])), p + "Wgu")
+            g = np.maximum(gu[:, :F], 0)
+            act = rb((g * g) * gu[:, F:])
+            h = rb(h + bl(rb(orc.rms_norm(act, w[p + "ffn_sub_norm"], cfg["rms_eps"])), p + "Wd"))
+    hf = rb(orc.rms_norm(h[P:], w["act.norm"], cfg["rms_eps"]))
+    x = orc.linear(hf, w["act.W_out"], w["act.b_out"])
+    x[:, cfg["real_action_dim"]:] = 0
+    return x
+
+
+@pytest.mark.parametrize("ffn", [0, 16])
+def test_bitvla_prefill_and_append_is_one_pass_under_a_prefix_lm_mask(ffn):
+    cfg = _bitvla_tiny(ffn)
+    w = ckpt.synth_weights(cfg, seed=930)
+    r = np.random.default_rng(931)
+    o = dict(img_emb=r.standard_normal((cfg["n_img"], cfg["hidden"])).astype(np.float32), n_views=1,
+             lang=r.integers(0, cfg["vocab"], cfg["n_lang"]).astype(np.int32))
+    got, _ = orc_chunk.bitvla_chunk(cfg, w, o)
+    want = _bitvla_one_pass(cfg, w, o)
+    assert np.array_equal(got, want)
+    # and the pass is sensitive to what the chunk decides: the appended tokens one position
+    # further (a common shift of all positions would cancel in the rotation) changes the bits
+    keep = orc.rope_tables
+    P = cfg["n_img"] + cfg["n_lang"]
+    try:
+        orc.rope_tables = lambda pos, D, base: keep(np.asarray(pos) + (np.arange(len(pos)) >= P), D, base)
+        assert not np.array_equal(_bitvla_one_pass(cfg, w, o), want)
+    finally:
+        orc.rope_tables = keep
+
+
+def test_bitvla_lm_forward_is_the_chunk_without_a_cache():
+    # One layer, no appended tokens' influence on the prefix: bitvla_lm_forward over
+    # [prefix ; action tokens 0..t] (bidirectional) gives, in its last row, what the chunk's
+    # token t sees only if t is the last token; with one layer the prefix K/V do not depend on
+    # later tokens, so row P + t of the forward over P + t + 1 tokens equals the chunk's token t.
+    cfg = _bitvla_tiny(16)
+    cfg["n_layers"] = 1
+    w = ckpt.synth_weights(cfg, seed=940)
+    r = np.random.default_rng(941)
+    o = dict(img_emb=r.standard_normal((cfg["n_img"], cfg["hidden"])).astype(np.float32), n_views=1,
+             lang=r.integers(0, cfg["vocab"], cfg["n_lang"]).astype(np.int32))
+    got, _ = orc_chunk.bitvla_chunk(cfg, w, o)
+    H, P, D = cfg["hidden"], cfg["n_img"] + cfg["n_lang"], cfg["head_dim"]
+    kvd = cfg["n_kv_heads"] * D
+    tq, wq = orc_chunk.bitvla_ternary(cfg, w, "lm.0.Wqkv", False)
+    layer = dict(attn_norm=w["lm.0.attn_norm"], sub_norm=w["lm.0.sub_norm"], ffn_norm=w["lm.0.ffn_norm"],
+                 ffn_sub_norm=w["lm.0.ffn_sub_norm"], q=(tq[:H], w["lm.0.Wqkv.ws"][:1]), k=(tq[H:H + kvd], w["lm.0.Wqkv.ws"][1:2]),
+                 v=(tq[H + kvd:], w["lm.0.Wqkv.ws"][2:3]), o=orc_chunk.bitvla_ternary(cfg, w, "lm.0.Wo", False),
+                 gate_up=orc_chunk.bitvla_ternary(cfg, w, "lm.0.Wgu", False), down=orc_chunk.bitvla_ternary(cfg, w, "lm.0.Wd", False))
+    emb = np.concatenate([o["img_emb"].reshape(cfg["n_img"], H), w["prefix.E_lang"][o["lang"]]], 0)
+    for t in range(cfg["n_suffix"]):
+        x = np.concatenate([emb, w["act.emb"][:t + 1]], 0)
+        hf = orc_chunk.bitvla_lm_forward(orc.round_bf16(x), [layer], w["act.norm"], cfg["n_q_heads"], cfg["n_kv_heads"], D,
+                                         cfg["rms_eps"], cfg["rope_freq_base"])
+        row = orc.linear(hf[P + t:P + t + 1], w["act.W_out"], w["act.b_out"])[0]
+        row[cfg["real_action_dim"]:] = 0
+        assert np.array_equal(row, got[t]), t
