@@ -19,7 +19,6 @@ roundings, so its pin is exact: the same chunk as ONE pass over prefix + action 
 prefix-LM mask, composed here from the pinned primitives in another order (no cache, no
 incremental positions), must give the same bits.
 """
-import copy
 import math
 
 import numpy as np
@@ -29,7 +28,7 @@ import oracle as orc
 from oracle import chunk as orc_chunk
 
 import chunk_restatement as ref
-from util import pkg
+from util import one_ulp_noise, pkg  # noqa: F401  (makes the package importable as vla_cpp_amd)
 
 from vla_cpp_amd import checkpoint as ckpt  # noqa: E402
 
@@ -287,3 +286,30 @@ def test_bitvla_lm_forward_is_the_chunk_without_a_cache():
         row = orc.linear(hf[P + t:P + t + 1], w["act.W_out"], w["act.b_out"])[0]
         row[cfg["real_action_dim"]:] = 0
         assert np.array_equal(row, got[t]), t
+
+
+def test_bitvla_chunk_amplifies_one_ulp_input_noise_with_depth():
+    # Why the 30-layer BitVLA chunk is not held to the per-element bf16 bar end to end: every
+    # layer re-quantises its activations to int8 twice, so a one-ulp change of a bf16 input
+    # flips integer codes now and then and the difference grows with depth and width.  Measured
+    # on the oracle alone (no GPU involved): the chunk output under 1 % one-ulp input noise moves
+    # more at 12 layers than at 1, and at 12 layers of width 512 some outputs already leave the
+    # 2e-2 relative / 1e-2 absolute bar.  The GPU test of the full configuration derives its
+    # end-to-end bound from this same measurement on its own weights.
+    def moved(L, H, Hq, Hkv, D):
+        cfg = ckpt.bitvla_config(n_layers=L)
+        cfg.update(hidden=H, n_q_heads=Hq, n_kv_heads=Hkv, head_dim=D, n_img=24, n_lang=24)
+        w = ckpt.synth_weights(cfg, seed=5)
+        r = np.random.default_rng(7)
+        o = dict(img_emb=orc.round_bf16(r.standard_normal((24, H)).astype(np.float32)), n_views=1,
+                 lang=r.integers(0, cfg["vocab"], 24).astype(np.int32))
+        a, _ = orc_chunk.bitvla_chunk(cfg, w, o)
+        b, _ = orc_chunk.bitvla_chunk(cfg, w, dict(o, img_emb=one_ulp_noise(o["img_emb"], r)))
+        d = np.abs(a - b)
+        return d.mean(), d.max(), float((d > 1e-2 + 2e-2 * np.abs(a)).mean())
+
+    shallow = moved(1, 512, 4, 1, 128)
+    deep = moved(12, 512, 4, 1, 128)
+    assert shallow[2] == 0.0                      # one layer: inside the bar
+    assert deep[0] > 2.5 * shallow[0] and deep[1] > 2.5 * shallow[1]
+    assert deep[2] > 0.0                          # twelve layers: the oracle disagrees with itself beyond the bar

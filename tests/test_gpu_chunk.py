@@ -12,7 +12,7 @@ import pytest
 
 import oracle as orc
 from oracle import chunk as orc_chunk
-from util import pkg, rel_err
+from util import one_ulp_noise, pkg, rel_err
 
 pytestmark = pytest.mark.gpu
 
@@ -109,6 +109,9 @@ def test_config2_pi0_mqa_bf16(tmp_path, n_layers, batch):
     for b in range(batch):
         want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
         assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+        if b == 0:  # and the pure fp32 CPU reference, which is what the tolerance is quoted against
+            want32 = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=False)
+            assert bf16_close(got[b], want32), np.abs(got[b] - want32).max()
     m.close()
 
 
@@ -123,6 +126,9 @@ def test_config3_gr00t_dit_bf16(tmp_path, n_layers, batch):
     for b in range(batch):
         want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
         assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+        if b == 0:  # and the pure fp32 CPU reference, which is what the tolerance is quoted against
+            want32 = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=False)
+            assert bf16_close(got[b], want32), np.abs(got[b] - want32).max()
     m.close()
 
 
@@ -257,11 +263,14 @@ def test_config4_bitvla_ternary_append(tmp_path, from_fp32, ffn_dim):
         if ffn_dim == 0:
             assert bf16_close(got[b], want), np.abs(got[b] - want).max()
         else:
-            # Two more quantisations and a squaring per layer: when 1 % of its bf16 inputs change
-            # by one ulp the oracle itself moves by 0.03 (max) at width 768 and by 0.05 (max),
-            # 0.013-0.015 (mean) at width 6912, outputs up to 2.9, so the per-element bar does
-            # not apply; the distance to the oracle stays at that scale.
-            assert rel_err(got[b], want) < 3e-2 and np.abs(got[b] - want).mean() < 2e-2, np.abs(got[b] - want).max()
+            # Two more quantisations and a squaring per layer: a one-ulp bf16 difference can flip
+            # int8 codes, so the per-element bar does not apply end to end (it does stage by stage:
+            # test_gpu_full_configs.py).  The bound is the oracle's own distance to itself when
+            # 1 % of its bf16 inputs move by one ulp, measured here on the same weights.
+            noisy, _ = orc_chunk.bitvla_chunk(cfg, w, dict(obs[b], img_emb=one_ulp_noise(obs[b]["img_emb"], r)), from_fp32=from_fp32)
+            d_self, d_gpu = np.abs(noisy - want), np.abs(got[b] - want)
+            assert d_gpu.max() <= 1.5 * d_self.max() + 1e-2 and d_gpu.mean() <= 1.5 * d_self.mean() + 2e-3, (
+                d_gpu.max(), d_gpu.mean(), d_self.max(), d_self.mean())
     m.close()
 
 

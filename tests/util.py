@@ -43,3 +43,15 @@ def declared_symbols(header):
     text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(?:VLA_KAPI|VLA_API|VLA_GGUF_API|VLA_SERVE_API)\s+[\w\s\*]+?\b(\w+)\s*\(", text)))
+
+
+def one_ulp_noise(x, r, frac=0.01):
+    """x (fp32 values that are bf16-representable) with `frac` of its elements moved to a
+    neighbouring bf16 value: the probe that measures how far a quantised network moves under
+    the smallest possible input difference.  Stays finite; zero moves to the smallest positive."""
+    import oracle as orc
+    b = orc.to_bf16(x).astype(np.int32).ravel()
+    idx = r.choice(b.size, max(1, int(frac * b.size)), replace=False)
+    mag = np.clip((b[idx] & 0x7fff) + r.choice(np.int32([-1, 1]), idx.size), 0, 0x7f7f)
+    b[idx] = (b[idx] & 0x8000) | mag
+    return orc.from_bf16(b.astype(np.uint16).reshape(np.shape(x)))
