@@ -5,17 +5,26 @@ One "step" is one denoise step (every expert layer: pre-norm, fused QKV + RoPE +
 KV append, masked prefix+suffix attention, Wo + residual, then the Euler update)
 over one batch of synthetic observations whose prefix KV is already resident in
 HBM; for the BitVLA workload a step is one appended action token through every
-layer.  The timed region is exactly K steps on one stream, bracketed by device
-synchronisation, launched through the model-level C ABI (vla_denoise_steps_async).
+layer.  Launched through the model-level C ABI (vla_denoise_steps_async).
+
+Timed region: exactly K steps on one stream, bracketed by device synchronisation, in
+steady state -- before it, three whole chunks always run (the first eagerly, the second
+is captured into a HIP graph, the third replays it) and then the W warm-up steps.
+
+Per-kernel figures are measured live, in the step's own sequence: after the timed region
+one more chunk runs with a HIP event recorded after every launch on the launch stream
+(vla_profile_begin / vla_profile_end), so a kernel's time is taken with the caches as
+its predecessors left them and includes the gap to the launch before it.  The events'
+own cost (the marked chunk minus a replayed one, per mark) is subtracted.
 
 Prints ONE JSON line with the contract fields plus
-  roofline      the dominant kernel of the step (by measured time), timed in
-                isolation with HIP events on the launch stream
-  roofline_kv   the attention kernel's prefix-KV read rate (same method)
-  cpu_baseline  the CPU oracle (restated reference op sequence, with the
-                reference's per-step concat copies) timed on this host
-  kernels       per-kernel average microseconds and launches per step
-  other_configs the same summary for further BASELINE configurations (--all)
+  roofline      the step's dominant kernel (largest share of the step's time)
+  roofline_kv   the attention launch that reads the most prefix KV
+  cpu_baseline  the CPU oracle (restated reference op sequence, with the reference's
+                per-step concat copies, fp32 SIMD-style accumulation) timed on this host
+                with the reference's thread rule and timing recipe
+  kernels       per launch site: average microseconds, launches per step, roofline fraction
+  other_configs the same summary for every other BASELINE configuration
 """
 import argparse
 import json
@@ -81,6 +90,14 @@ def plain_pack(t):
     return out.view(np.uint8).reshape(-1)
 
 
+def cpu_threads():
+    """The reference's rule (src/arch.h:43-53): VLA_N_THREADS if set, else min(hardware threads, 16)."""
+    e = os.environ.get("VLA_N_THREADS")
+    if e and e.isdigit() and 0 < int(e) <= 1024:
+        return int(e)
+    return min(os.cpu_count() or 4, 16)
+
+
 def time_events(fn, iters, warm=3):
     """Average device microseconds of one fn() call.  fn(i) launches on the current
     torch stream; `iters` calls are captured into one HIP graph and the graph is
@@ -106,7 +123,7 @@ def time_events(fn, iters, warm=3):
 
 
 def kernel_breakdown(pkg, cfg, B, P):
-    """Times every kernel of one step in isolation at the workload's shapes.
+    """(--isolated) Times every kernel of one step in isolation at the workload's shapes.
     Returns {name: dict(us, per_step, bound, work)} with work = algorithmic bytes
     (bound hbm) or flops (bound mfma) per launch."""
     import torch
@@ -307,65 +324,171 @@ def kernel_breakdown(pkg, cfg, B, P):
 
 # HBM-side bytes per launch (L2 misses) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # on this command, KiB per dispatch, each scaled by what the same counter reads for a plain
-# 256 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); the per-kernel tables and
-# the commands are in profiles/*_pmc.txt.  Kernels without a measurement report null.
+# 256 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Counters cannot be read from
+# inside the process, so these are the figures of profiles/*_pmc.txt (which give the commands);
+# launch sites without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg1_smolvla_16layer_bf16_b32", "wo_residual"): int((7821.0 * 2 + 2250.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "qkv_rope_append_self"): int((6934.0 * 2 + 5400.1) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "q_rope_cross"): int((5072.5 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "attention_self"): int((7734.6 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "attention_cross"): int((6592.0 * 2 + 3000.0) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "attention_cross"): int((62789.0 * 2 + 3351.8) * 1024),
-    ("cfg4_bitvla_30layer_b8", "ternary_qkv_gemm_prefill"): int((16895.0 * 2 + 30720.0) * 1024),
-    ("cfg4_bitvla_30layer_b8", "attention_decode"): int((7005.5 * 2 + 1016.2) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.wo_residual"): int((7821.0 * 2 + 2250.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.qkv_rope_append_self"): int((6934.0 * 2 + 5400.1) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.q_rope_cross"): int((5072.5 * 2 + 3000.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_self"): int((7734.6 * 2 + 3000.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_cross"): int((6592.0 * 2 + 3000.0) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "step.attention_cross"): int((62789.0 * 2 + 3351.8) * 1024),
+    ("cfg4_bitvla_30layer_b8", "prefill.ternary_qkv_gemm"): int((16895.0 * 2 + 30720.0) * 1024),
+    ("cfg4_bitvla_30layer_b8", "step.attention"): int((7005.5 * 2 + 1016.2) * 1024),
 }
 
 
-def roofline_of(name, k, workload=None):
-    if k["bound"] == "hbm":
-        achieved = k["work"] / (k["us"] * 1e-6) / 1e9
+def prefix_tokens(cfg, views):
+    if cfg["arch"] == "smolvla":
+        return views * cfg["n_img"] + cfg["n_lang"] + 1
+    if cfg["arch"] in ("pi0", "pi05"):
+        return views * cfg["n_img"] + cfg["n_lang"]
+    if cfg["arch"] == "bitvla":
+        return cfg["n_img"] + cfg["n_lang"]
+    return views * cfg["n_img"]
+
+
+def algorithmic_work(cfg, B, P):
+    """{launch-site label: (bound, algorithmic bytes or flops per launch, peak key)}: the per-unit
+    figures of the path (K/V read once per launch, 2 M N K per projection) at this workload."""
+    arch = cfg["arch"]
+    bf = cfg["dtype"] == "bf16"
+    es = 2 if bf else 4
+    mf = "bf16" if bf else "f32"
+    Hq, Hkv, D = cfg["n_q_heads"], cfg["n_kv_heads"], cfg["head_dim"]
+    qd, kvd = Hq * D, Hkv * D
+    w = {}
+    if arch == "bitvla":
+        H, n_act, F = cfg["hidden"], cfg["n_suffix"], cfg.get("ffn_dim", 0)
+        N, M, Mp = H + 2 * kvd, B, B * P
+        T = P + (n_act + 1) / 2.0  # keys seen by an appended token, averaged over the chunk
+        w["step.token_embedding"] = ("hbm", 2 * M * H * 2, "hbm")
+        w["step.norm_quant_qkv_gemv_rope_append"] = ("hbm", N * H // 4 + 2 * M * H + 2 * M * N, "hbm")
+        w["step.attention"] = ("hbm", 2 * T * kvd * 2 * B, "hbm")
+        w["step.norm_quant_o_gemv_add"] = ("hbm", H * H // 4 + 2 * M * H + 4 * M * H, "hbm")
+        w["step.final_norm"] = ("hbm", 2 * M * H * 2, "hbm")
+        w["step.action_head"] = ("hbm", n_act * M * H * 2, "hbm")
+        w["prefill.norm_quant"] = ("hbm", 3 * Mp * H, "hbm")
+        w["prefill.ternary_qkv_gemm"] = ("mfma", 2.0 * Mp * N * H, "i8")
+        w["prefill.qkv_split_rope_append"] = ("hbm", 2 * Mp * N * 2, "hbm")
+        w["prefill.attention"] = ("mfma", 4.0 * Hq * P * P * D * B, "bf16")
+        w["prefill.ternary_o_gemm_add"] = ("mfma", 2.0 * Mp * H * H, "i8")
+        if F:
+            w["step.norm_quant_gate_up_gemv"] = ("hbm", 2 * F * H // 4 + 2 * M * H + 4 * M * F, "hbm")
+            w["step.sqrelu_norm_quant_down_gemv_add"] = ("hbm", H * F // 4 + 4 * M * F + 4 * M * H, "hbm")
+            w["step.sqrelu_norm_quant"] = ("hbm", 5 * M * F, "hbm")
+            w["step.ternary_down_gemm_add"] = ("hbm", H * F // 4 + M * F + 4 * M * H, "hbm")
+            w["prefill.ternary_gate_up_gemm"] = ("mfma", 4.0 * Mp * F * H, "i8")
+            w["prefill.sqrelu_norm_quant"] = ("hbm", 5 * Mp * F, "hbm")
+            w["prefill.ternary_down_gemm_add"] = ("mfma", 2.0 * Mp * H * F, "i8")
+        return w
+    W, Wv, S, A, I = cfg["expert_h"], cfg["hidden"], cfg["n_suffix"], cfg["max_action_dim"], cfg.get("ffn_dim", 0)
+    M = B * S
+    gr00t = arch in ("gr00t_n1d5", "gr00t_n1d6")
+    P_self = 0 if gr00t else P
+    n_lead = 0 if arch in ("smolvla", "pi05") else 1
+    w["step.stage_noise"] = ("hbm", 2 * B * (S - n_lead) * A * 4, "hbm")
+    w["step.embed_suffix"] = ("hbm", M * W * es, "hbm")
+    for k in ("step.pre_norm", "step.final_norm", "step.ffn_norm"):
+        w[k] = ("hbm", 2 * M * W * es, "hbm")
+    w["step.qkv_rope_append_self"] = ("mfma", 2.0 * M * (qd + 2 * kvd) * W, mf)
+    w["step.q_rope_cross"] = ("mfma", 2.0 * M * qd * W, mf)
+    w["step.attention_self"] = ("hbm", 2 * (P_self + S) * kvd * es * B, "hbm")
+    w["step.attention_cross"] = ("hbm", 2 * P * kvd * es * B, "hbm")
+    if arch == "gr00t_n1d6":
+        w["step.attention_cross_text"] = ("hbm", 2 * cfg["n_lang"] * kvd * es * B, "hbm")
+        w["step.attention_cross"] = ("hbm", 2 * (P - 0) * kvd * es * B, "hbm")
+    w["step.wo_residual"] = ("mfma", 2.0 * M * W * qd, mf)
+    w["step.ffn_gate_up"] = ("mfma", 4.0 * M * I * W, mf)
+    w["step.ffn_down_residual"] = ("mfma", 2.0 * M * I * W, mf)
+    w["step.ffn_gate_up_down"] = ("mfma", 6.0 * M * I * W, mf)
+    w["step.ffn_in_out"] = ("mfma", 4.0 * M * I * W, mf)
+    w["step.euler_step"] = ("hbm", M * W * es, "hbm")
+    w["prefill.prefix_norm"] = ("hbm", 2 * B * P * Wv * es, "hbm")
+    w["prefill.prefix_kv_proj"] = ("mfma", 2.0 * B * P * 2 * kvd * Wv, mf)
+    w["prefill.prefix_kv_proj_and_cross_reprojection"] = ("mfma", 2.0 * B * P * 2 * kvd * (Wv + kvd), mf)
+    return w
+
+
+def roofline_entry(label, us, work, workload=None):
+    bound, amount, peak_key = work
+    if bound == "hbm":
+        achieved = amount / (us * 1e-6) / 1e9
         peak, unit = HBM_PEAK_GBS, "GB/s"
     else:
-        achieved = k["work"] / (k["us"] * 1e-6) / 1e12
-        peak, unit = PEAK_TFLOPS[k["peak_key"]], "TFLOP/s"
-    return dict(kernel=name, bound=k["bound"], achieved=round(achieved, 3), peak=peak, unit=unit,
-                frac=round(achieved / peak, 5), traffic=MEASURED_TRAFFIC_BYTES.get((workload, name)),
-                avg_us=round(k["us"], 3),
-                algorithmic_work_per_launch=k["work"])
+        achieved = amount / (us * 1e-6) / 1e12
+        peak, unit = PEAK_TFLOPS[peak_key], "TFLOP/s" if peak_key != "i8" else "TOP/s"
+    return dict(kernel=label, bound=bound, achieved=round(achieved, 3), peak=peak, unit=unit,
+                frac=round(achieved / peak, 5), traffic=MEASURED_TRAFFIC_BYTES.get((workload, label)),
+                avg_us=round(us, 3), algorithmic_work_per_launch=amount,
+                timing="HIP events on the launch stream, in the step's own sequence, less the events' own cost")
+
+
+def pct(xs, q):
+    xs = sorted(xs)
+    return xs[min(len(xs) - 1, int(round(q * (len(xs) - 1))))]
 
 
 def cpu_baseline(cfg, w, obs, B):
-    """The CPU oracle on a bounded sample: one observation, a few denoise steps; the
-    per-step figure is scaled by the batch (observations are independent and the
-    restated reference handles one at a time, as the reference's server does)."""
+    """The CPU oracle on a bounded sample: one observation, denoise steps only (the prefix K/V
+    build is excluded, as on the GPU side), timed with the reference's recipe -- warm-ups, then
+    repetitions, min / p50 / p90 (src/serving/vla-bench.cpp:159-195) -- on the reference's thread
+    count (src/arch.h:43-53).  The per-step figure is scaled by the batch: observations are
+    independent and the reference serves one at a time (src/serving/server.cpp:340-558)."""
     import oracle as orc
     from oracle import chunk as oc
-    if cfg["arch"] == "bitvla":
-        small = dict(cfg, n_layers=2)
-        t0 = time.perf_counter()
-        oc.bitvla_chunk(small, w, obs)
-        t_all = time.perf_counter() - t0
-        # prefill dominates; time the decode tokens alone through a second run is not
-        # separable here, so report whole-chunk (prefill + 7 tokens) per token for 2 of L layers, scaled
-        per_step = t_all / cfg["n_suffix"] * (cfg["n_layers"] / 2.0)
-        return dict(value=round(per_step * 1e6 * B, 1), unit="us per appended token (batch of %d)" % B,
-                    cores=orc.num_threads(), kind="port",
-                    sample="1 observation, 2 of %d layers, prefix prefill + 7 tokens, scaled by layers and batch; "
-                           "includes the prefill the GPU figure excludes" % cfg["n_layers"])
-    n1, n2 = 1, 3
-    ts = []
-    for n in (n1, n2):
-        c = dict(cfg, num_steps=n)
-        t0 = time.perf_counter()
-        oc.flow_expert_chunk(c, w, obs, emulate_bf16=False)
-        ts.append(time.perf_counter() - t0)
-    per_step = (ts[1] - ts[0]) / (n2 - n1)
-    return dict(value=round(per_step * 1e6 * B, 1), unit="us per denoise step (batch of %d)" % B,
-                cores=orc.num_threads(), kind="port",
-                sample="restated CPU reference (not ggml): 1 observation, steps 2-3 of a 3-step run, scaled by batch %d" % B)
+    threads = cpu_threads()
+    orc.set_num_threads(threads)
+    orc.set_default_accumulation(False)  # fp32 accumulation with SIMD-style partial sums, not the parity oracle's double
+    try:
+        if cfg["arch"] == "bitvla":
+            small = dict(cfg, n_layers=2)
+            run = lambda: oc.bitvla_chunk(small, w, obs)
+            scale_layers, n_units, what = cfg["n_layers"] / 2.0, cfg["n_suffix"], "appended token"
+            budget = 12.0
+            t0 = time.perf_counter()
+            run()
+            first = time.perf_counter() - t0
+            reps = int(max(3, min(20, budget / max(first, 1e-3))))
+            ts = []
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                run()
+                ts.append(time.perf_counter() - t0)
+            per = [t / n_units * scale_layers * 1e6 * B for t in ts]
+            sample = ("restated CPU reference (not ggml): 1 observation, 2 of %d layers, prefix prefill + 7 tokens per run "
+                      "(the prefill is included: the restated reference has no cache to skip it with), 1 warm-up + %d "
+                      "repetitions, scaled by layers and batch %d" % (cfg["n_layers"], reps, B))
+        else:
+            n1, n2 = 1, 1 + cfg["num_steps"]
+            run = lambda n: oc.flow_expert_chunk(dict(cfg, num_steps=n), w, obs, emulate_bf16=False)
+            t0 = time.perf_counter()
+            run(n2)
+            first = time.perf_counter() - t0
+            reps = int(max(3, min(20, 15.0 / max(first * 1.2, 1e-3))))
+            for _ in range(2):
+                run(n2)
+            short, full = [], []
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                run(n1)
+                short.append(time.perf_counter() - t0)
+                t0 = time.perf_counter()
+                run(n2)
+                full.append(time.perf_counter() - t0)
+            base = pct(short, 0.5)  # prefix build + one step
+            per = [(t - base) / (n2 - n1) * 1e6 * B for t in full]
+            what = "denoise step"
+            sample = ("restated CPU reference (not ggml): 1 observation, (chunk of %d steps - chunk of 1 step) / %d, 3 warm-ups + "
+                      "%d repetitions, scaled by batch %d" % (n2, n2 - n1, reps, B))
+    finally:
+        orc.set_default_accumulation(True)
+    return dict(value=round(pct(per, 0.5), 1), unit="us per %s (batch of %d)" % (what, B), cores=threads, kind="port",
+                min=round(min(per), 1), p50=round(pct(per, 0.5), 1), p90=round(pct(per, 0.9), 1), sample=sample)
 
 
-def run_workload(name, spec, steps, warmup, with_cpu, tmpdir):
+def run_workload(name, spec, steps, warmup, with_cpu, tmpdir, isolated=False):
     import torch
     import __graft_entry__ as entry
     pkg = entry.load_package()
@@ -378,11 +501,18 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir):
     m = ffi.Model(path)
     r = np.random.default_rng(0x5EED)
     obs = [make_obs(cfg, r, views) for _ in range(B)]
+    spc = cfg["n_suffix"] if cfg["arch"] == "bitvla" else cfg["num_steps"]  # steps per chunk
+    m.prefill_batch(obs)  # allocates
+    m.profile_begin()
     t0 = time.perf_counter()
     m.prefill_batch(obs)
     prefill_ms = (time.perf_counter() - t0) * 1e3
+    prof_prefill = m.profile_end()
     stream = torch.cuda.current_stream().cuda_stream
-    m.denoise_steps_async(warmup, stream)
+    # steady state first: eager chunk, captured chunk, one replay -- whatever W is
+    m.denoise_steps_async(3 * spc, stream)
+    if warmup > 0:
+        m.denoise_steps_async(warmup, stream)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -392,31 +522,49 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir):
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     dev_ms = e0.elapsed_time(e1)
-    ms_per_step = max(dev_ms, wall_ms) / steps  # the host-inclusive figure is the honest one for an eager launch loop
-    steps_per_chunk = cfg["n_suffix"] if cfg["arch"] == "bitvla" else cfg["num_steps"]
-    if cfg["arch"] == "smolvla":
-        P = views * cfg["n_img"] + cfg["n_lang"] + 1
-    elif cfg["arch"] in ("pi0", "pi05"):
-        P = views * cfg["n_img"] + cfg["n_lang"]
-    elif cfg["arch"] == "bitvla":
-        P = cfg["n_img"] + cfg["n_lang"]
-    else:
-        P = views * cfg["n_img"]
-    kern = kernel_breakdown(pkg, cfg, B, P)
-    step_kern = {k: v for k, v in kern.items() if v["per_step"] > 0}
-    dominant = max(step_kern, key=lambda k: step_kern[k]["us"] * step_kern[k]["per_step"])
-    attn = [k for k in kern if k.startswith("attention")]
-    kv_name = max(attn, key=lambda k: kern[k]["work"])
+    ms_per_step = max(dev_ms, wall_ms) / steps  # the host-inclusive figure when the host is the slower side
+    # one more chunk with an event after every launch
+    m.profile_begin()
+    m.denoise_steps_async(spc, stream)
+    prof = m.profile_end()
+    P = prefix_tokens(cfg, views)
+    work = algorithmic_work(cfg, B, P)
+    # An event between two launches costs stream time of its own: the marked chunk takes longer
+    # than a replayed one.  The difference, spread evenly over the marks, is taken off every
+    # launch, so that the per-launch figures add up to the step as it was timed above.
+    n_marks = sum(v["launches"] for v in prof.values())
+    marked_us = sum(v["us"] * v["launches"] for v in prof.values())
+    event_us = max(0.0, (marked_us - dev_ms * 1e3 / steps * spc) / max(n_marks, 1))
+    prof = {k: dict(us=max(v["us"] - event_us, 0.05), launches=v["launches"], us_marked=v["us"]) for k, v in prof.items()}
+    kernels, best, best_kv, best_t = {}, None, None, 0.0
+    for label, v in sorted(prof.items()):
+        per_step = v["launches"] / float(spc)
+        k = dict(us=round(v["us"], 2), per_step=round(per_step, 3))
+        if label in work:
+            rf = roofline_entry(label, v["us"], work[label], name)
+            k.update(bound=rf["bound"], frac=rf["frac"])
+            if v["us"] * per_step > best_t:
+                best, best_t = rf, v["us"] * per_step
+            if label.startswith("step.attention") and (best_kv is None or work[label][1] > best_kv["algorithmic_work_per_launch"]):
+                best_kv = rf
+        kernels[label] = k
     res = dict(
         workload=name, batch=B, us_per_denoise_step=round(ms_per_step * 1e3, 2),
-        us_per_action_chunk=round(ms_per_step * 1e3 * steps_per_chunk, 1), steps_per_chunk=steps_per_chunk,
-        device_us_per_step=round(dev_ms * 1e3 / steps, 2), prefix_kv_build_ms=round(prefill_ms, 2),
-        sum_kernel_us_per_step=round(sum(v["us"] * v["per_step"] for v in step_kern.values()), 2),
-        roofline=roofline_of(dominant, kern[dominant], name), roofline_kv=roofline_of(kv_name, kern[kv_name], name),
-        kernels={k: dict(us=round(v["us"], 2), per_step=v["per_step"]) for k, v in kern.items()},
+        us_per_action_chunk=round(ms_per_step * 1e3 * spc, 1), steps_per_chunk=spc, timed_steps=steps,
+        device_us_per_step=round(dev_ms * 1e3 / steps, 2), host_us_per_step=round(wall_ms * 1e3 / steps, 2),
+        prefix_kv_build_ms=round(prefill_ms, 2),
+        sum_launch_us_per_step=round(sum(v["us"] * v["launches"] for v in prof.values()) / spc, 2),
+        event_overhead_us_per_launch=round(event_us, 3),
+        launches_per_step=round(sum(v["launches"] for v in prof.values()) / float(spc), 1),
+        roofline=best, roofline_kv=best_kv, kernels=kernels,
+        prefill_kernels={k: dict(us=round(v["us"], 2), launches=v["launches"]) for k, v in sorted(prof_prefill.items())},
     )
-    if "ternary_qkv_gemm_prefill" in kern:
-        res["roofline_ternary_prefill"] = roofline_of("ternary_qkv_gemm_prefill", kern["ternary_qkv_gemm_prefill"], name)
+    if "prefill.ternary_qkv_gemm" in prof_prefill:
+        res["roofline_ternary_prefill"] = roofline_entry("prefill.ternary_qkv_gemm", prof_prefill["prefill.ternary_qkv_gemm"]["us"],
+                                                         work["prefill.ternary_qkv_gemm"], name)
+    if isolated:
+        kern = kernel_breakdown(pkg, cfg, B, P)
+        res["kernels_isolated"] = {k: dict(us=round(v["us"], 2), per_step=v["per_step"]) for k, v in kern.items()}
     if with_cpu:
         res["cpu_baseline"] = cpu_baseline(cfg, w, obs[0], B)
     m.close()
@@ -424,16 +572,24 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir):
     return res, ms_per_step
 
 
+BASELINE_WORKLOADS = ["cfg0_smolvla_1layer_f32_b1", "cfg1_smolvla_16layer_bf16_b1", "cfg1_smolvla_16layer_bf16_b32",
+                      "cfg2_pi0_18layer_bf16_b1", "cfg2_pi0_18layer_bf16_b16", "cfg3_gr00t_16dit_bf16_b1",
+                      "cfg3_gr00t_16dit_bf16_b64", "cfg4_bitvla_30layer_b1", "cfg4_bitvla_30layer_b8"]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="cfg1_smolvla_16layer_bf16_b32")
-    ap.add_argument("--all", action="store_true", help="also run every other BASELINE configuration")
-    ap.add_argument("--others", default="cfg3_gr00t_16dit_bf16_b64,cfg4_bitvla_30layer_b8",
-                    help="comma-separated extra workloads reported under other_configs")
+    # the headline workload: the largest single-GPU configuration of the BASELINE set, GR00T
+    # N1.5-shape DiT at batch 64 -- the largest prefix-KV read per step (931 MB)
+    ap.add_argument("--config", default="cfg3_gr00t_16dit_bf16_b64")
+    ap.add_argument("--others", default="baseline",
+                    help="'baseline' = every other BASELINE configuration (both batch sizes), 'all' = every workload, "
+                         "'none', or a comma-separated list; reported under other_configs")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--isolated", action="store_true", help="also time every kernel alone (replayed, warm caches)")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="only run plain device copies of a known size (reference for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -460,13 +616,24 @@ def main():
     if args.config not in wl:
         print("unknown --config; choose from: " + ", ".join(wl), file=sys.stderr)
         sys.exit(2)
+    if args.others == "baseline":
+        names = [n for n in BASELINE_WORKLOADS if n != args.config]
+    elif args.others == "all":
+        names = [n for n in wl if n != args.config]
+    elif args.others == "none":
+        names = []
+    else:
+        names = [n for n in args.others.split(",") if n and n != args.config]
     with tempfile.TemporaryDirectory() as tmp:
-        main_res, ms_per_step = run_workload(args.config, wl[args.config], args.steps, args.warmup, not args.no_cpu, tmp)
+        main_res, ms_per_step = run_workload(args.config, wl[args.config], args.steps, args.warmup, not args.no_cpu, tmp,
+                                             args.isolated)
         others = []
-        names = [n for n in wl if n != args.config] if args.all else [n for n in args.others.split(",") if n and n != args.config]
         for n in names:
-            steps = args.steps if "bitvla" not in n else max(7, args.steps // 7 * 7 // 2)
-            r, _ = run_workload(n, wl[n], steps, min(args.warmup, steps), False, tmp)
+            c = wl[n]["cfg"]
+            spc = c["n_suffix"] if c["arch"] == "bitvla" else c["num_steps"]
+            r, _ = run_workload(n, wl[n], 3 * spc, 0, False, tmp, args.isolated)  # whole chunks: graph replays only
+            for k in ("kernels", "prefill_kernels"):  # the headline carries the full tables; keep the line readable
+                r[k] = {a: b for a, b in r[k].items() if "attention" in a or "gemm" in a or "gemv" in a or "qkv" in a or "wo_" in a}
             others.append(r)
     cfg = wl[args.config]["cfg"]
     line = {
@@ -475,15 +642,22 @@ def main():
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if cfg["dtype"] == "bf16" else "f32", "data": "synthetic",
         "config": {"workload": args.config, "batch": wl[args.config]["B"], "n_layers": cfg["n_layers"],
-                   "prefix_tokens_resident": True, "step": "one denoise step over all expert layers"},
+                   "prefix_tokens_resident": True, "step": "one denoise step over all expert layers",
+                   "timed_region": "graph replays in steady state (3 whole chunks + warmup steps run before it)"},
         "us_per_action_chunk": main_res["us_per_action_chunk"],
         "roofline": main_res["roofline"], "roofline_kv": main_res["roofline_kv"],
         "cpu_baseline": main_res.get("cpu_baseline"),
-        "kernels": main_res["kernels"], "device_us_per_step": main_res["device_us_per_step"],
-        "sum_kernel_us_per_step": main_res["sum_kernel_us_per_step"],
+        "kernels": main_res["kernels"], "prefill_kernels": main_res["prefill_kernels"],
+        "device_us_per_step": main_res["device_us_per_step"], "host_us_per_step": main_res["host_us_per_step"],
+        "sum_launch_us_per_step": main_res["sum_launch_us_per_step"], "launches_per_step": main_res["launches_per_step"],
+        "event_overhead_us_per_launch": main_res["event_overhead_us_per_launch"],
         "prefix_kv_build_ms": main_res["prefix_kv_build_ms"],
         "other_configs": others,
     }
+    if "roofline_ternary_prefill" in main_res:
+        line["roofline_ternary_prefill"] = main_res["roofline_ternary_prefill"]
+    if "kernels_isolated" in main_res:
+        line["kernels_isolated"] = main_res["kernels_isolated"]
     print(json.dumps(line))
 
 

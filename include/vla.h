@@ -119,6 +119,17 @@ VLA_API int32_t vla_fetch_actions(vla_model * m, float ** out_actions, int64_t *
 VLA_API int32_t vla_predict_batch(vla_model * m, const vla_inputs * in, int32_t batch, float ** out_actions,
                                   int64_t * out_n);
 
+/* Per-launch timing for benchmarks (no counterpart in the reference, whose vla-bench times
+ * whole predict() calls, src/serving/vla-bench.cpp:159-195).  Between begin and end, prefill
+ * and denoise calls record a HIP event after every kernel launch and denoise launches eagerly
+ * instead of replaying its graph.  vla_profile_end synchronises, disarms and writes a JSON
+ * object {"phase.label": {"us": average, "launches": count}, ...} -- the time from the
+ * previous launch's end to this launch's end on the stream, i.e. the launch in its real
+ * sequence, cold caches and dependent-launch gap included.  Returns the string length, or the
+ * negated size needed when cap is too small, or a vla_status. */
+VLA_API int32_t vla_profile_begin(vla_model * m);
+VLA_API int64_t vla_profile_end(vla_model * m, char * json_out, int64_t cap);
+
 #ifdef __cplusplus
 }
 #endif

@@ -63,6 +63,21 @@ def num_threads():
     return int(_lib.orc_num_threads())
 
 
+def set_num_threads(n):
+    _lib.orc_set_num_threads(int(n))
+
+
+# Accumulation of linear() and attention() when the caller does not say: double for parity
+# checks (the default, never changed by tests); the benchmark's CPU-baseline leg switches to
+# fp32 SIMD-style accumulation, which is what a CPU inference engine runs.
+_DEFAULT_ACC64 = True
+
+
+def set_default_accumulation(acc64):
+    global _DEFAULT_ACC64
+    _DEFAULT_ACC64 = bool(acc64)
+
+
 # ---------------------------------------------------------------- bf16 helpers
 def to_bf16(x):
     """fp32 array -> uint16 array of bf16 bit patterns (round to nearest even)."""
@@ -123,7 +138,8 @@ def rotate_half(x):
 
 
 # ---------------------------------------------------------------- linear, norm
-def linear(x, W, b=None, acc64=True):
+def linear(x, W, b=None, acc64=None):
+    acc64 = _DEFAULT_ACC64 if acc64 is None else acc64
     x, W = _f32(x), _f32(W)
     M, K = x.shape
     N, K2 = W.shape
@@ -223,8 +239,9 @@ def softmax_scaled_bf16(u16, scale):
     return y
 
 
-def attention(Q, K, V, mask, scale, acc64=True):
+def attention(Q, K, V, mask, scale, acc64=None):
     """Q [S,Hq,D], K/V [T,Hkv,D] token-major, mask [S,T] additive or None -> [S, Hq*D]."""
+    acc64 = _DEFAULT_ACC64 if acc64 is None else acc64
     Q, K, V = _f32(Q), _f32(K), _f32(V)
     S, Hq, D = Q.shape
     T, Hkv, D2 = K.shape

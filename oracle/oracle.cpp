@@ -141,11 +141,26 @@ void orc_rotate_half(const float* x, float* out, int D) {
 // src/models/smolvla.cpp:771-776,821-823, src/models/pi0.cpp:174-176,
 // src/layers/linear.h:24-27.  acc64 != 0 accumulates in double.
 // ----------------------------------------------------------------------------
+// fp32 dot product the way a SIMD CPU kernel forms it (ggml's vec_dot keeps several vector
+// accumulators): 32 independent partial sums with fused multiply-add, combined at the end.
+// Used only when acc64 == 0, i.e. by the timed CPU baseline; the parity oracle accumulates
+// in double.
+static inline float dot_f32_lanes(const float* a, const float* b, int n) {
+    float acc[32] = {0.f};
+    int k = 0;
+    for (; k + 32 <= n; k += 32)
+        for (int j = 0; j < 32; ++j) acc[j] = __builtin_fmaf(a[k + j], b[k + j], acc[j]);
+    for (; k < n; ++k) acc[k & 31] = __builtin_fmaf(a[k], b[k], acc[k & 31]);
+    for (int w = 16; w > 0; w >>= 1)
+        for (int j = 0; j < w; ++j) acc[j] += acc[j + w];
+    return acc[0];
+}
+
 void orc_linear(const float* x, const float* W, const float* b, float* y, int M, int N, int K, int acc64) {
-#pragma omp parallel for schedule(static)
+#pragma omp parallel for schedule(static) collapse(2)
     for (int m = 0; m < M; ++m) {
-        const float* xr = x + (size_t)m * K;
         for (int n = 0; n < N; ++n) {
+            const float* xr = x + (size_t)m * K;
             const float* wr = W + (size_t)n * K;
             float out;
             if (acc64) {
@@ -153,9 +168,7 @@ void orc_linear(const float* x, const float* W, const float* b, float* y, int M,
                 for (int k = 0; k < K; ++k) a += (double)wr[k] * (double)xr[k];
                 out = (float)(a + (b ? (double)b[n] : 0.0));
             } else {
-                float a = 0.f;
-                for (int k = 0; k < K; ++k) a += wr[k] * xr[k];
-                out = a + (b ? b[n] : 0.f);
+                out = dot_f32_lanes(wr, xr, K) + (b ? b[n] : 0.f);
             }
             y[(size_t)m * N + n] = out;
         }
@@ -290,22 +303,23 @@ void orc_attention(const float* Q, const float* K, const float* V, const float* 
                     for (int d = 0; d < D; ++d) a += (double)q[d] * (double)k[d];
                     sc[t] = (float)a;
                 } else {
-                    float a = 0.f;
-                    for (int d = 0; d < D; ++d) a += q[d] * k[d];
-                    sc[t] = a;
+                    sc[t] = dot_f32_lanes(q, k, D);
                 }
             }
             orc_softmax_ext(sc.data(), mask ? mask + (size_t)s * T : nullptr, scale, 1, T);
             float* o = out + ((size_t)s * Hq + h) * D;
-            for (int d = 0; d < D; ++d) {
-                if (acc64) {
+            if (acc64) {
+                for (int d = 0; d < D; ++d) {
                     double a = 0.0;
                     for (int t = 0; t < T; ++t) a += (double)sc[t] * (double)V[((size_t)t * Hkv + hk) * D + d];
                     o[d] = (float)a;
-                } else {
-                    float a = 0.f;
-                    for (int t = 0; t < T; ++t) a += sc[t] * V[((size_t)t * Hkv + hk) * D + d];
-                    o[d] = a;
+                }
+            } else {  // keys outermost: every V row is read once, contiguously
+                for (int d = 0; d < D; ++d) o[d] = 0.f;
+                for (int t = 0; t < T; ++t) {
+                    const float* v = V + ((size_t)t * Hkv + hk) * D;
+                    const float p = sc[t];
+                    for (int d = 0; d < D; ++d) o[d] = __builtin_fmaf(p, v[d], o[d]);
                 }
             }
         }
@@ -581,6 +595,14 @@ void orc_transpose_Hsd_to_sHd_u16(const uint16_t* in, uint16_t* out, int H, int 
 }
 void orc_gather_rows_u16(const uint16_t* in, uint16_t* out, const int32_t* ids, int n_rows, int K) {
     for (int m = 0; m < n_rows; ++m) std::memcpy(out + (size_t)m * K, in + (size_t)ids[m] * K, (size_t)K * 2);
+}
+
+void orc_set_num_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void)n;
+#endif
 }
 
 int orc_num_threads(void) {

@@ -73,6 +73,9 @@ def _bind():
     L.vla_fetch_actions.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.POINTER(_f32)), ctypes.POINTER(_i64)]
     L.vla_predict_batch.argtypes = [ctypes.c_void_p, ctypes.POINTER(Inputs), _i32,
                                     ctypes.POINTER(ctypes.POINTER(_f32)), ctypes.POINTER(_i64)]
+    L.vla_profile_begin.argtypes = [ctypes.c_void_p]
+    L.vla_profile_end.argtypes = [ctypes.c_void_p, ctypes.c_char_p, _i64]
+    L.vla_profile_end.restype = _i64
     _bound = True
     return L
 
@@ -164,6 +167,18 @@ class Model:
         if rc != VLA_OK:
             raise RuntimeError("vla_fetch_actions returned %d" % rc)
         return self._take(p, n)
+
+    def profile_begin(self):
+        assert self._L.vla_profile_begin(self._h) == VLA_OK
+
+    def profile_end(self):
+        """{"phase.label": {"us": ..., "launches": ...}} for the launches since profile_begin()."""
+        import json
+        buf = ctypes.create_string_buffer(1 << 16)
+        n = self._L.vla_profile_end(self._h, buf, len(buf))
+        if n < 0:
+            raise RuntimeError("vla_profile_end returned %d" % n)
+        return json.loads(buf.value.decode())
 
     def predict_batch(self, obs_list):
         self.prefill_batch(obs_list)

@@ -220,6 +220,7 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
     }
     h_.upload(emb.data(), emb.size() * 2);
     Ctx C;
+    prof_start("prefill", C.stream);
     run_layers(C, B * P, P, 0, P);
     VLA_HIP(hipDeviceSynchronize());
 }
@@ -242,34 +243,44 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
                                                        cos_t, sin_t, q_.as<uint16_t>(), w.kv.k.as<uint16_t>(),
                                                        w.kv.vt.as<uint16_t>(), M, Hq_, Hkv_, D_, H_, w.kv.t_max, tok_offset,
                                                        C.stream));
+            prof_mark("norm_quant_qkv_gemv_rope_append");
         } else if (fused) {
             VLA_K(vla_rmsnorm_ternary_gemv(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), eps_, w.Wqkv.packed.as<uint32_t>(),
                                            qkv_.as<uint16_t>(), nullptr, w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_,
                                            C.stream));
+            prof_mark("norm_quant_qkv_gemv");
         } else {
             VLA_K(vla_rmsnorm_act_quant_bf16(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
                                              rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
+            prof_mark("norm_quant");
             VLA_K(vla_ternary_gemm(q8_.as<int8_t>(), w.Wqkv.packed.as<uint32_t>(), qkv_.as<uint16_t>(), nullptr,
                                    s_.as<float>(), rowsum_.as<int32_t>(), w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_,
                                    C.stream));
+            prof_mark("ternary_qkv_gemm");
         }
-        if (!(fused && S == 1 && w.Wqkv.paired.get()))
+        if (!(fused && S == 1 && w.Wqkv.paired.get())) {
             VLA_K(vla_qkv_split_rope_append(qkv_.get(), cos_t, sin_t, q_.get(), w.kv.k.get(), w.kv.vt.get(), VLA_DT_BF16, M, S,
                                             Hq_, Hkv_, D_, w.kv.t_max, tok_offset, C.stream));
+            prof_mark("qkv_split_rope_append");
+        }
         VLA_K(vla_attn_prefix_suffix_ws(q_.get(), w.kv.k.get(), w.kv.vt.get(), att_.get(), VLA_DT_BF16_P2, M / S, S, Hq_, Hkv_,
                                         D_, w.kv.t_max, n_keys, scale, VLA_MASK_NONE, n_keys, 0, 0, nullptr, attn_ws_.buf.get(),
                                         attn_ws_.buf.bytes(), C.stream));
+        prof_mark("attention");
         // O projection and the residual add of the hidden stream in one launch
         if (fused) {
             VLA_K(vla_rmsnorm_ternary_gemv(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), eps_, w.Wo.packed.as<uint32_t>(),
                                            h_.as<uint16_t>(), h_.as<uint16_t>(), w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_,
                                            C.stream));
+            prof_mark("norm_quant_o_gemv_add");
         } else {
             VLA_K(vla_rmsnorm_act_quant_bf16(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
                                              rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
+            prof_mark("norm_quant");
             VLA_K(vla_ternary_gemm_add(q8_.as<int8_t>(), w.Wo.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
                                        s_.as<float>(), rowsum_.as<int32_t>(), w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_,
                                        C.stream));
+            prof_mark("ternary_o_gemm_add");
         }
         if (F_ == 0) continue;
         // the GLU half: ffn norm -> [gate | up] -> relu(gate)^2 * up -> sub-norm -> down + residual
@@ -277,16 +288,20 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
             VLA_K(vla_rmsnorm_ternary_gemv(h_.as<uint16_t>(), w.ffn_norm.as<uint16_t>(), eps_, w.Wgu.packed.as<uint32_t>(),
                                            gu_.as<uint16_t>(), nullptr, w.Wgu.ws.as<float>(), w.Wgu.ws_num, M, 2 * F_, H_,
                                            C.stream));
+            prof_mark("norm_quant_gate_up_gemv");
         } else {
             VLA_K(vla_rmsnorm_act_quant_bf16(h_.as<uint16_t>(), w.ffn_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
                                              rowsum_.as<int32_t>(), eps_, M, H_, C.stream));
+            prof_mark("norm_quant");
             VLA_K(vla_ternary_gemm(q8_.as<int8_t>(), w.Wgu.packed.as<uint32_t>(), gu_.as<uint16_t>(), nullptr, s_.as<float>(),
                                    rowsum_.as<int32_t>(), w.Wgu.ws.as<float>(), w.Wgu.ws_num, M, 2 * F_, H_, C.stream));
+            prof_mark("ternary_gate_up_gemm");
         }
         if (fused && F_ <= 4096) {  // activation, sub-norm, quantisation and down projection in one launch
             VLA_K(vla_sqrelu_rmsnorm_ternary_gemv(gu_.as<uint16_t>(), w.ffn_sub_norm.as<uint16_t>(), eps_,
                                                   w.Wd.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
                                                   w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_, C.stream));
+            prof_mark("sqrelu_norm_quant_down_gemv_add");
             continue;
         }
         // Longer rows (the model's 6912): every 32-column workgroup of the one-launch form would
@@ -300,9 +315,11 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
             VLA_K(vla_rmsnorm_act_quant_bf16(act_.as<uint16_t>(), w.ffn_sub_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
                                              rowsum_.as<int32_t>(), eps_, M, F_, C.stream));
         }
+        prof_mark("sqrelu_norm_quant");
         VLA_K(vla_ternary_gemm_add(q8_.as<int8_t>(), w.Wd.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
                                    s_.as<float>(), rowsum_.as<int32_t>(), w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_,
                                    C.stream));
+        prof_mark("ternary_down_gemm_add");
     }
 }
 
@@ -315,19 +332,23 @@ void BitvlaLm::run_steps(int n_steps, void* stream) {
     const size_t row = (size_t)B * H_;
     // one step = one appended action token through every layer; the action head runs
     // when the last token of a chunk is done
+    prof_start("step", C.stream);
     for (int it = 0; it < n_steps; ++it) {
         const int t = it % n_act_;
         VLA_HIP(hipMemcpyAsync(h_.get(), emb_bcast_.as<uint16_t>() + (size_t)t * row, row * 2, hipMemcpyDeviceToDevice,
                                C.stream));
+        prof_mark("token_embedding");
         run_layers(C, B, 1, P_ + t, P_ + t + 1);
         VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), out_norm_.as<uint16_t>(), hfin_.as<uint16_t>() + (size_t)t * row, eps_, B,
                                   H_, C.stream));
+        prof_mark("final_norm");
         if (t == n_act_ - 1) {
             // cleared by a copy node: memset nodes are kept out of captured graphs
             VLA_HIP(hipMemcpyAsync(x_.get(), zeros_.get(), (size_t)n_act_ * B * A_ * 4, hipMemcpyDeviceToDevice, C.stream));
             // x[t][b] = W_out . hfin[t][b] + b_out (batch' = n_act, rows = B, unit step)
             VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B,
                                  0, A_, H_, 1.0f, C.stream));
+            prof_mark("action_head");
         }
     }
 }

@@ -497,6 +497,7 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
     Tensor xp = tensor_2d(prefix_.get(), dt_, Wv_, (int64_t)B * P);
     Tensor xn = tensor_2d(prefix_n_.get(), dt_, Wv_, (int64_t)B * P);
     const int kvd = Hkv_ * D_;
+    prof_start("prefill", C.stream);
     for (LayerW& w : layers_) {
         if (!w.needs_prefix) continue;
         Tensor Wkv = tensor_2d(w.Wkv_pre.get(), dt_, Wv_, 2 * kvd);
@@ -507,13 +508,16 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
             const char* base = (const char*)prefix_.get() + (txt ? (size_t)B * (P - P_txt_) * Wv_ * dtype_size(dt_) : 0);
             Tensor xs = tensor_2d(const_cast<char*>(base), dt_, Wv_, (int64_t)B * rows);
             qkv_rope_append(C, xs, Wkv, bkv, rows, 0, true, true, nullptr, nullptr, w.kv, 0);
+            prof_mark("prefix_kv_proj");
             continue;
         }
         if (arch_ == Arch::GR00T) {
             qkv_rope_append(C, xp, Wkv, bkv, P, 0, true, true, nullptr, nullptr, w.kv, 0);
+            prof_mark("prefix_kv_proj");
             continue;
         }
         rms_norm(C, xp, w.vlm_ln.get(), eps_, xn);
+        prof_mark("prefix_norm");
         if (arch_ == Arch::SMOLVLA && !w.is_self) {
             // expert_cross_kv: K = Wk_x . cachedK_flat, V = Wv_x . cachedV_flat, no second rotation
             qkv_rope_append(C, xn, Wkv, bkv, P, 0, true, true, &rope_prefill_, nullptr, tmp_kv_, 0);
@@ -523,8 +527,10 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
             Tensor Wkx = tensor_2d(w.Wk_x.get(), dt_, kvd, kvd), Wvx = tensor_2d(w.Wv_x.get(), dt_, kvd, kvd);
             qkv_rope_append(C, tk, Wkx, nullptr, P, 0, true, false, nullptr, nullptr, w.kv, 0);
             qkv_rope_append(C, tv, Wvx, nullptr, P, 0, false, true, nullptr, nullptr, w.kv, 0);
+            prof_mark("prefix_kv_proj_and_cross_reprojection");
         } else {
             qkv_rope_append(C, xn, Wkv, bkv, P, 0, true, true, &rope_prefill_, nullptr, w.kv, 0);
+            prof_mark("prefix_kv_proj");
         }
     }
 
@@ -557,9 +563,13 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
     Q.dtype = dt_;
     Q.ne[0] = D_; Q.ne[1] = Hq_; Q.ne[2] = S_; Q.ne[3] = B;
     const size_t xbytes = (size_t)B * (S_ - n_lead_) * A_ * sizeof(float);
+    prof_start("step", C.stream);
     for (int it = 0; it < n_steps; ++it) {
         const int s = it % steps_;
-        if (s == 0) VLA_HIP(hipMemcpyAsync(xt_.get(), x0_.get(), xbytes, hipMemcpyDeviceToDevice, C.stream));
+        if (s == 0) {
+            VLA_HIP(hipMemcpyAsync(xt_.get(), x0_.get(), xbytes, hipMemcpyDeviceToDevice, C.stream));
+            prof_mark("stage_noise");
+        }
         {
             if (time_mlp_) {
                 VLA_K(vla_embed_suffix_act(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
@@ -572,6 +582,7 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 VLA_K(vla_embed_suffix(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
                                        n_lead_ ? lead_.as<float>() : nullptr, h.data, dt_, B, S_, n_lead_, A_, W_, C.stream));
             }
+            prof_mark("embed_suffix");
             for (int l = 0; l < L_; ++l) {
                 LayerW& w = layers_[l];
                 const float* bq = w.bqkv ? w.bqkv.as<float>() : nullptr;
@@ -585,6 +596,7 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 bool done = false;
                 if (adarms_) {
                     VLA_K(vla_adarms(h.data, mod_in, mod_in + W_, hn.data, dt_, M, W_, eps_, C.stream));
+                    prof_mark("pre_norm");
                     Tensor Wqkv = tensor_2d(w.Wqkv.get(), dt_, W_, n_rows_w);
                     qkv_rope_append(C, hn, Wqkv, bq, S_, Hq_, w.is_self, w.is_self, tab, Q.data, w.kv, tok);
                     done = true;
@@ -600,39 +612,49 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                     } else {
                         rms_norm(C, h, w.ln.get(), eps_, hn);
                     }
+                    prof_mark("pre_norm");
                     Tensor Wqkv = tensor_2d(w.Wqkv.get(), dt_, W_, n_rows_w);
                     qkv_rope_append(C, hn, Wqkv, bq, S_, Hq_, w.is_self, w.is_self, tab, Q.data, w.kv, tok);
                 }
+                prof_mark(w.is_self ? "qkv_rope_append_self" : "q_rope_cross");
                 MaskSpec mask;
                 mask.pad_start = pad_start_;
                 mask.pad_end = pad_end_;
                 mask.kind = w.is_self ? suffix_mask_ : VLA_MASK_NONE;
                 const int n_keys = w.is_self ? w.kv.n_prefix + S_ : w.kv.n_prefix;
                 flash_attention(C, Q, w.kv, n_keys, mask, scale, att, attn_ws_);
+                prof_mark(w.is_self ? "attention_self" : (w.from_text && P_txt_ > 0) ? "attention_cross_text" : "attention_cross");
                 Tensor Wo = tensor_2d(w.Wo.get(), dt_, (int64_t)Hq_ * D_, W_);
                 if (adarms_) {
                     // h1 = x + o_out * gate_attn; h = h1 + mlp_out * gate_ffn (pi05.cpp:273-281)
                     VLA_K(vla_linear_gated(att.data, Wo.data, nullptr, mod_in + 2 * W_, h.data, h.data, dt_, dt_, M, W_,
                                            Hq_ * D_, C.stream));
+                    prof_mark("wo_residual");
                     if (I_ > 0) {
                         Tensor mid = tensor_2d(mid_.get(), dt_, I_, M);
                         VLA_K(vla_adarms(h.data, mod_post, mod_post + W_, hn.data, dt_, M, W_, eps_, C.stream));
+                        prof_mark("ffn_norm");
                         VLA_K(vla_glu_linear(hn.data, w.Wgu.get(), nullptr, mid.data, dt_, dt_, M, I_, W_, VLA_ACT_GELU, -1.f,
                                              C.stream));
+                        prof_mark("ffn_gate_up");
                         VLA_K(vla_linear_gated(mid.data, w.Wd.get(), nullptr, mod_post + 2 * W_, h.data, h.data, dt_, dt_, M, W_,
                                                I_, C.stream));
+                        prof_mark("ffn_down_residual");
                     }
                     continue;
                 }
                 linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
+                prof_mark("wo_residual");
                 if (I_ > 0) {
                     // FFN half (smolvla.cpp:845-848, pi0.cpp:227-232, dit_head.cpp:132-133)
                     Tensor mid = tensor_2d(mid_.get(), dt_, I_, M);
                     if (arch_ == Arch::GR00T) {
                         const float* z = ada_.as<float>() + ((size_t)s * (L_ + 1) + L_) * 2 * W_;  // zeros: plain LayerNorm
                         adaln(C, h, z, z + W_, eps_, hn);
+                        prof_mark("ffn_norm");
                         Tensor W1 = tensor_2d(w.W1.get(), dt_, W_, I_), W2 = tensor_2d(w.W2.get(), dt_, I_, W_);
                         ffn_gelu(C, W1, w.b1.as<float>(), W2, w.b2.as<float>(), hn, h.data, mid, h);
+                        prof_mark("ffn_in_out");
                     } else {
                         const int act = arch_ == Arch::SMOLVLA ? VLA_ACT_SILU : VLA_ACT_GELU;
                         Tensor Wd = tensor_2d(w.Wd.get(), dt_, I_, W_);
@@ -646,6 +668,7 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                             Tensor Wgu = tensor_2d(w.Wgu.get(), dt_, W_, 2 * (int64_t)I_);
                             ffn_glu(C, Wgu, act, Wd, hn, -1.f, h.data, mid, h);
                         }
+                        prof_mark("ffn_gate_up_down");
                     }
                 }
             }
@@ -658,8 +681,10 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
             } else {
                 rms_norm(C, h, final_norm_.get(), eps_, hn);
             }
+            prof_mark("final_norm");
             VLA_K(vla_euler_step(xt_.as<float>(), hn.data, W_out_.as<float>(), b_out_.as<float>(), dt_, B, S_, n_lead_,
                                  A_, W_, dt_step_, C.stream));
+            prof_mark("euler_step");
         }
     }
 }

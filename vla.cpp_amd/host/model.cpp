@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cstdlib>
+#include <map>
 #include <thread>
 
 #include "checkpoint.h"
@@ -36,6 +37,73 @@ struct ModelArch::GraphState {
     bool warmed = false;  // the shape has run eagerly once (lazy workspaces exist)
 };
 
+// ---- per-launch timing ------------------------------------------------------
+struct ModelArch::Profiler {
+    std::string phase;
+    hipStream_t stream = nullptr;
+    struct Mark {
+        std::string label;  // empty: the opening event of a sequence
+        hipEvent_t ev;
+    };
+    std::vector<Mark> marks;
+    ~Profiler() {
+        for (Mark& m : marks) (void)hipEventDestroy(m.ev);
+    }
+    void add(const std::string& label) {
+        Mark m;
+        m.label = label;
+        VLA_HIP(hipEventCreate(&m.ev));
+        VLA_HIP(hipEventRecord(m.ev, stream));
+        marks.push_back(m);
+    }
+};
+
+ModelArch::~ModelArch() {
+    drop_graph();
+    delete prof_;
+}
+
+void ModelArch::profile_begin() {
+    delete prof_;
+    prof_ = new Profiler();
+}
+
+void ModelArch::prof_start(const char* phase, void* stream) {
+    if (!prof_) return;
+    prof_->phase = phase;
+    prof_->stream = (hipStream_t)stream;
+    prof_->add("");
+}
+
+void ModelArch::prof_mark(const char* label) {
+    if (!prof_) return;
+    prof_->add(prof_->phase + "." + label);
+}
+
+std::string ModelArch::profile_end() {
+    if (!prof_) return "{}";
+    VLA_HIP(hipDeviceSynchronize());
+    std::map<std::string, std::pair<double, long>> acc;
+    for (size_t i = 1; i < prof_->marks.size(); ++i) {
+        if (prof_->marks[i].label.empty()) continue;
+        float ms = 0.f;
+        VLA_HIP(hipEventElapsedTime(&ms, prof_->marks[i - 1].ev, prof_->marks[i].ev));
+        auto& a = acc[prof_->marks[i].label];
+        a.first += (double)ms * 1e3;
+        a.second += 1;
+    }
+    delete prof_;
+    prof_ = nullptr;
+    std::string out = "{";
+    char buf[256];
+    for (const auto& kv : acc) {
+        std::snprintf(buf, sizeof(buf), "%s\"%s\": {\"us\": %.4f, \"launches\": %ld}", out.size() > 1 ? ", " : "", kv.first.c_str(),
+                      kv.second.first / (double)kv.second.second, kv.second.second);
+        out += buf;
+    }
+    return out + "}";
+}
+
 void ModelArch::drop_graph() {
     if (!graph_) return;
     if (graph_->exec) (void)hipGraphExecDestroy(graph_->exec);
@@ -51,6 +119,10 @@ void ModelArch::denoise_steps(int n_steps, void* stream) {
     int chunks = n_steps / spc;
     const int rem = n_steps % spc;
     hipStream_t st = (hipStream_t)stream;
+    if (prof_) {  // timing every launch: eager, one sequence
+        run_steps(n_steps, stream);
+        return;
+    }
     if (!graph_) graph_ = new GraphState();
     GraphState& g = *graph_;
     const uint64_t key = launch_key();

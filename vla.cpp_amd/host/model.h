@@ -46,7 +46,7 @@ struct Stats {
 // per handle (the reference's rule, src/arch.h:85-87).
 class ModelArch {
   public:
-    virtual ~ModelArch() { drop_graph(); }
+    virtual ~ModelArch();
     Config cfg;
     Stats stats;
     // Builds the prefix KV for `batch` observations and stages state / noise.
@@ -66,12 +66,26 @@ class ModelArch {
     // Changes whenever anything baked into the launches changes (buffers, shapes, masks).
     virtual uint64_t launch_key() const = 0;
 
+    // Per-launch timing for benchmarks.  While armed, prefill and run_steps record a HIP event
+    // after every launch (prof_mark names what was launched since the previous mark) and
+    // denoise launches eagerly instead of replaying its graph.
+    void prof_start(const char* phase, void* stream);
+    void prof_mark(const char* label);
+
   private:
     struct GraphState;
     GraphState* graph_ = nullptr;
+    struct Profiler;
+    Profiler* prof_ = nullptr;
 
   public:
     void drop_graph();
+    // Arms the per-launch timing / synchronises, disarms and returns a JSON object
+    // {"phase.label": {"us": average microseconds between the previous mark and this one,
+    // "launches": marks recorded}, ...}.  The time between two marks is the launch's duration
+    // plus the gap to its predecessor on the stream.
+    void profile_begin();
+    std::string profile_end();
     // Synchronises and returns [batch, n_actions, max_action_dim].
     virtual std::vector<float> fetch() = 0;
     virtual int64_t n_actions() const = 0;

@@ -204,6 +204,31 @@ int32_t vla_predict_batch(vla_model* h, const vla_inputs* in, int32_t batch, flo
     return vla_fetch_actions(h, out_actions, out_n);
 }
 
+int32_t vla_profile_begin(vla_model* h) {
+    if (!h || !h->m) return VLA_ERR_ARG;
+    try {
+        h->m->arch->profile_begin();
+        return VLA_OK;
+    } catch (...) {
+        return VLA_ERR_EXCEPTION;
+    }
+}
+
+int64_t vla_profile_end(vla_model* h, char* json_out, int64_t cap) {
+    if (!h || !h->m || !json_out || cap <= 0) return VLA_ERR_ARG;
+    try {
+        const std::string s = h->m->arch->profile_end();
+        if ((int64_t)s.size() + 1 > cap) return -(int64_t)(s.size() + 1);
+        std::memcpy(json_out, s.c_str(), s.size() + 1);
+        return (int64_t)s.size();
+    } catch (const std::exception& e) {
+        std::fprintf(stderr, "vla: profile failed: %s\n", e.what());
+        return VLA_ERR_EXCEPTION;
+    } catch (...) {
+        return VLA_ERR_EXCEPTION;
+    }
+}
+
 int64_t vla_model_n_actions(const vla_model* h) {
     if (!h || !h->m) return 0;
     return h->m->arch->n_actions();
