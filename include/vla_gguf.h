@@ -69,6 +69,15 @@ VLA_GGUF_API int32_t vla_gguf_read_convert(vla_gguf* g, const char* name, int32_
 VLA_GGUF_API int32_t vla_gguf_fetch_rows_f32(vla_gguf* g, const char* name, const int32_t* row_ids, int64_t n_rows, float* dst,
                                              int64_t cols);
 
+/* Runs the checkpoint import that vla_model_load would run on a GGUF file (host only, no GPU
+ * state, nothing kept) and writes the names of the GGUF tensors it read, one per line in
+ * reading order, NUL-terminated: the importer's view of the reference's tensor names
+ * (src/models/smolvla.cpp:648-755, src/models/pi0.cpp:427-437, src/models/pi05.cpp:459-485,
+ * src/modules/dit_head.cpp:29-85, src/modules/action_expert.cpp:20-39, src/models/bitvla.cpp:640-700).
+ * Returns the length, VLA_GGUF_ERR_READ when the file cannot be imported (the reason goes to
+ * stderr), or a value below -16 when cap is too small. */
+VLA_GGUF_API int64_t vla_gguf_import_trace(const char* path, char* out, int64_t cap);
+
 #ifdef __cplusplus
 }
 #endif

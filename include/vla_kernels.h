@@ -116,8 +116,9 @@ VLA_KAPI int vla_adarms(const void* x, const float* sc, const float* sh, void* y
 VLA_KAPI int vla_linear(const void* x, const void* W, const float* bias, const void* residual, void* y,
                         int dtype, int out_dtype, int M, int N, int K, vla_stream_t stream);
 
-/* Activations of the FFN halves (ggml_silu, ggml_gelu in its tanh form). */
-enum { VLA_ACT_NONE = 0, VLA_ACT_SILU = 1, VLA_ACT_GELU = 2 };
+/* Activations of the FFN halves (ggml_silu, ggml_gelu in its tanh form) and of the DiT head's
+ * state encoder / action decoder (ggml_relu, src/modules/action_expert.cpp:41-59). */
+enum { VLA_ACT_NONE = 0, VLA_ACT_SILU = 1, VLA_ACT_GELU = 2, VLA_ACT_RELU = 3 };
 
 /* vla_linear with an activation between the bias and the residual:
  * y = act(x W^T + b) [+ residual]; the first half of ffn_gelu
@@ -266,6 +267,15 @@ VLA_KAPI int vla_embed_suffix_act(const float* x_t, const float* W_in, const flo
  * rows were produced by a projection over all S rows of the suffix. */
 VLA_KAPI int vla_set_lead_rows(const float* lead, void* h, int dtype, int batch, int S, int n_lead, int W,
                                vla_stream_t stream);
+
+/* h[b][s][:] = lead[b][s][:] for s < n_lead, else acc[b][s][:] + row_table[s - n_lead][:],
+ * converted to `dtype`: the tail of ActionExpert::encode_action
+ * (src/modules/action_expert.cpp:46-52: W3 . silu(..) + bias, plus the learned position rows)
+ * and of the concat with the state / future-token rows (src/models/gr00tn1d5.cpp:371) when
+ * the action rows came out of an fp32 projection over all S rows.  acc fp32 [batch][S][W];
+ * row_table fp32 [S - n_lead][W] or NULL; lead fp32 [batch][n_lead][W]. */
+VLA_KAPI int vla_finish_suffix_rows(const float* acc, const float* row_table, const float* lead, void* h, int dtype,
+                                    int batch, int S, int n_lead, int W, vla_stream_t stream);
 
 /* Output projection + Euler update (src/models/smolvla.cpp:1416-1418,
  * src/models/pi0.cpp:577-587): x_t[b][s] += dt * (W_out . hn[b][n_lead + s] + b_out).

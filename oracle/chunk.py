@@ -69,7 +69,9 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
     gr00t = arch in ("gr00t_n1d5", "gr00t_n1d6")
     alt_vl = arch == "gr00t_n1d6"
     pi05 = arch == "pi05"
-    n_lead = 0 if arch in ("smolvla", "pi05") else 1
+    # the DiT head's own MLPs: state + future tokens lead, encode_action / proj_out + decode
+    head_io = gr00t and bool(cfg.get("head_io", 0))
+    n_lead = 0 if arch in ("smolvla", "pi05") else (1 + cfg["num_future"] if head_io else 1)
     Sa = S - n_lead
 
     # ---- prefix embeddings, positions, masks
@@ -150,21 +152,28 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
     dt = (1.0 if gr00t else -1.0) / steps
     dt32 = np.float32(dt)
     if gr00t:
-        ada = []
+        ada, po_mod = [], []
+        n_buckets = cfg.get("num_buckets", 1000)
         for s in range(steps):
-            tp = orc.timesteps_proj(int(s / steps * 1000.0))
+            tp = orc.timesteps_proj(int(s / steps * n_buckets))
             t1 = orc.silu(orc.linear(tp[None, :], w["te.l1W"], w["te.l1b"]))
             temb = orc.linear(t1, w["te.l2W"], w["te.l2b"])
             st = orc.silu(temb)
             ada.append([orc.linear(st, w["ex.%d.adaln_w" % l], w["ex.%d.adaln_b" % l])[0] for l in range(L)])
+            if head_io:  # DitHead::proj_out's dense: (shift, scale), dit_head.cpp:140-142
+                po_mod.append(orc.linear(st, w["aex.po1W"], w["aex.po1b"])[0])
     lead = None
-    if n_lead:
+    if head_io:
+        # ActionExpert::encode_state (action_expert.cpp:41-44), then the learned future tokens (gr00tn1d5.cpp:371)
+        se = np.maximum(orc.linear(state[None, :], w["aex.se_l1W"], w["aex.se_l1b"]), 0)
+        lead = np.concatenate([orc.linear(se, w["aex.se_l2W"], w["aex.se_l2b"]), w["aex.future_tokens"]], 0)
+    elif n_lead:
         lead = orc.linear(state[None, :], w["act.W_sp"], w["act.b_sp"])
 
     x = np.asarray(obs["noise"], np.float32).reshape(Sa, A).copy()
     debug = {}
     for s in range(steps):
-        bias = w["act.b_in"].copy()
+        bias = None if head_io else w["act.b_in"].copy()
         if pi05:
             # the time only conditions the norms (pi05.cpp:619-622)
             t = np.float32(1.0) + np.float32(s) * dt32
@@ -178,7 +187,13 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
         elif not gr00t:
             t = np.float32(1.0) + np.float32(s) * dt32
             bias = bias + orc.sinusoidal_time_emb(float(t), W, cfg["min_period"], cfg["max_period"])
-        if "act.W_at1" in w and not gr00t:
+        if head_io:
+            # ActionExpert::encode_action (action_expert.cpp:46-52) with tau = action_sinusoid(bucket)
+            tau = orc.action_sinusoid(int(s / steps * n_buckets), W, Sa)
+            a_emb = orc.linear(x, w["aex.ae_W1"], w["aex.ae_b1"])
+            m = orc.silu(orc.linear(np.concatenate([a_emb, tau], 1), w["aex.ae_W2"], w["aex.ae_b2"]))
+            h = orc.linear(m, w["aex.ae_W3"], w["aex.ae_b3"]) + w["aex.pos_embd"][:Sa]
+        elif "act.W_at1" in w and not gr00t:
             # action-time MLP (smolvla.cpp:1397-1403, pi0.cpp:240-244), in the reference's order
             t = np.float32(1.0) + np.float32(s) * dt32
             temb = orc.sinusoidal_time_emb(float(t), W, cfg["min_period"], cfg["max_period"])
@@ -250,6 +265,15 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
                 debug["q0"], debug["att0"], debug["h0"] = q, att, h
         if pi05:
             hn = rnd(adarms(h, "act.ada_final")[0])
+        elif head_io:
+            # DitHead::proj_out (dit_head.cpp:139-147) then ActionExpert::decode (action_expert.cpp:54-57)
+            sh, sc = po_mod[s][:W], po_mod[s][W:]
+            hn = rnd(orc.adaln(h, sc, sh, cfg.get("norm_out_eps", 1e-6)))
+            d1 = rnd(orc.linear(hn, w["aex.po2W"], w["aex.po2b"]))
+            d2 = rnd(np.maximum(orc.linear(d1, w["aex.ad_l1W"], w["aex.ad_l1b"]), 0))
+            v_t = orc.linear(d2[n_lead:], w["aex.ad_l2W"], w["aex.ad_l2b"])
+            x = (x + dt32 * v_t).astype(np.float32)
+            continue
         elif gr00t:
             hn = rnd(orc.layer_norm(h, None, None, cfg.get("norm_out_eps", 1e-6)))
         else:

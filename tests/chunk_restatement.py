@@ -272,13 +272,29 @@ def gr00t(cfg, w, obs):
         kv = mm(w["vlm.%d.Wkv" % l], src, w["vlm.%d.bkv" % l])
         Kc[l], Vc[l] = kv[:, :kvd].reshape(-1, H, D), kv[:, kvd:].reshape(-1, H, D)
     state = T(obs["state"]) if obs.get("state") is not None else torch.zeros(cfg["max_state_dim"], dtype=F64)
-    lead = mm(w["act.W_sp"], state[None], w["act.b_sp"])
+    head_io = bool(cfg.get("head_io", 0))
+    if head_io:  # encode_state, then the learned future tokens: 1 + num_future leading rows
+        lead = torch.cat([mm(w["aex.se_l2W"], F.relu(mm(w["aex.se_l1W"], state[None], w["aex.se_l1b"])), w["aex.se_l2b"]),
+                          T(w["aex.future_tokens"])], 0)
+    else:
+        lead = mm(w["act.W_sp"], state[None], w["act.b_sp"])
+    n_lead = lead.shape[0]
+    AH = S - n_lead
     dt = 1.0 / steps
-    x = T(obs["noise"]).reshape(S - 1, cfg["max_action_dim"])
+    x = T(obs["noise"]).reshape(AH, cfg["max_action_dim"])
     for s in range(steps):
-        bucket = int(s / steps * 1000.0)
+        bucket = int(s / steps * cfg.get("num_buckets", 1000))
         temb = mm(w["te.l2W"], F.silu(mm(w["te.l1W"], timesteps_proj(bucket)[None], w["te.l1b"])), w["te.l2b"])
-        h = torch.cat([lead, mm(w["act.W_in"], x, w["act.b_in"])], 0)
+        if head_io:
+            # encode_action: W3 silu(W2 [W1 x + b1 ; tau] + b2) + b3 + pos, tau = sin | cos of bucket * 10000^(-i / half)
+            half = W // 2
+            ang = float(bucket) * torch.exp(-torch.arange(half, dtype=F64) * (math.log(10000.0) / half))
+            tau = torch.cat([torch.sin(ang), torch.cos(ang)])[None].expand(AH, W)
+            a = mm(w["aex.ae_W1"], x, w["aex.ae_b1"])
+            act_rows = mm(w["aex.ae_W3"], F.silu(mm(w["aex.ae_W2"], torch.cat([a, tau], 1), w["aex.ae_b2"])), w["aex.ae_b3"])
+            h = torch.cat([lead, act_rows + T(w["aex.pos_embd"])[:AH]], 0)
+        else:
+            h = torch.cat([lead, mm(w["act.W_in"], x, w["act.b_in"])], 0)
         for l in range(L):
             p = "ex.%d." % l
             cond = mm(w[p + "adaln_w"], F.silu(temb), w[p + "adaln_b"])[0]
@@ -295,7 +311,15 @@ def gr00t(cfg, w, obs):
                 n3 = F.layer_norm(h, (W,), eps=eps)
                 h = h + mm(w[p + "W2"], F.gelu(mm(w[p + "W1"], n3, w[p + "b1"]), approximate="tanh"), w[p + "b2"])
         hn = F.layer_norm(h, (W,), eps=cfg.get("norm_out_eps", 1e-6))
-        x = x + dt * mm(w["act.W_out"], hn[1:], w["act.b_out"])
+        if head_io:
+            # proj_out: the dense on silu(temb) yields (shift, scale); then decode's relu MLP; the
+            # velocity is the last AH rows
+            po = mm(w["aex.po1W"], F.silu(temb), w["aex.po1b"])[0]
+            hm = hn + hn * po[W:] + po[:W]
+            pred = mm(w["aex.ad_l2W"], F.relu(mm(w["aex.ad_l1W"], mm(w["aex.po2W"], hm, w["aex.po2b"]), w["aex.ad_l1b"])), w["aex.ad_l2b"])
+            x = x + dt * pred[-AH:]
+        else:
+            x = x + dt * mm(w["act.W_out"], hn[1:], w["act.b_out"])
     return _finish(cfg, x)
 
 

@@ -49,6 +49,11 @@ def tiny(arch, **kw):
         c = ckpt.pi05_config(n_layers=3, dtype="f32", num_steps=3)
         c.update(n_q_heads=4, n_kv_heads=1, head_dim=16, hidden=24, expert_h=16, n_img=3, n_lang=5, n_suffix=4,
                  max_action_dim=6, max_state_dim=5, real_action_dim=6, real_state_dim=5, vocab=11)
+    elif arch == "gr00t_head_io":
+        c = ckpt.gr00t_head_io_config(n_layers=4, dtype="f32", num_steps=3, ffn_dim=12)
+        c.update(n_q_heads=3, n_kv_heads=3, head_dim=8, hidden=20, expert_h=24, n_img=4, max_action_dim=6, max_state_dim=7,
+                 real_action_dim=6, real_state_dim=7, num_future=2, n_suffix=1 + 2 + 3, dit_out_dim=10, dec_hidden=14,
+                 state_hidden=9, max_pos=8)
     elif arch == "gr00t_n1d5":
         c = ckpt.gr00t_config(n_layers=4, dtype="f32", num_steps=3, n_suffix=5)
         c.update(n_q_heads=3, n_kv_heads=3, head_dim=8, hidden=20, expert_h=24, n_img=4, max_action_dim=6,
@@ -63,7 +68,7 @@ def tiny(arch, **kw):
 
 
 def obs_for(cfg, r, n_views=2, n_lang=None):
-    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "pi05") else 1)
+    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "pi05") else 1 + cfg.get("num_future", 0) * cfg.get("head_io", 0))
     o = dict(img_emb=r.standard_normal((n_views * cfg["n_img"], cfg["hidden"])).astype(np.float32), n_views=n_views,
              noise=r.standard_normal((n_act, cfg["max_action_dim"])).astype(np.float32),
              state=r.standard_normal(cfg["max_state_dim"]).astype(np.float32))
@@ -77,7 +82,7 @@ def big_weights(cfg, seed):
     (with N(0, 0.02) projections a tiny model's softmax is nearly uniform)."""
     w = ckpt.synth_weights(cfg, seed=seed)
     for k in list(w):
-        if k.endswith(("Wqkv", "Wq", "Wkv", "Wk_x", "Wv_x", "Wo", "W_out", "Wgu", "Wd", "W1", "W2")):
+        if k.endswith(("Wqkv", "Wq", "Wkv", "Wk_x", "Wv_x", "Wo", "W_out", "Wgu", "Wd", ".W1", ".W2", "po1W", "po2W", "ad_l1W", "ad_l2W")):
             w[k] = (w[k] * np.float32(12.0)).astype(np.float32)
     return w
 
@@ -89,7 +94,7 @@ def rel(a, b):
 CASES = [("smolvla", {}), ("smolvla", dict(suffix_mask=0)), ("smolvla", dict(ffn_dim=12, time_mlp=1)), ("pi0", {}),
          ("pi0", dict(ffn_dim=12, time_mlp=1)), ("pi05", {}), ("pi05", dict(ffn_dim=12)), ("gr00t_n1d5", {}),
          ("gr00t_n1d5", dict(ffn_dim=12)), ("gr00t_n1d6", {}), ("gr00t_n1d6", dict(every=1)),
-         ("gr00t_n1d6", dict(interleave=0, ffn_dim=12))]
+         ("gr00t_n1d6", dict(interleave=0, ffn_dim=12)), ("gr00t_head_io", {})]
 
 
 @pytest.mark.parametrize("arch,kw", CASES, ids=["%s-%s" % (a, "-".join("%s%s" % i for i in k.items()) or "base") for a, k in CASES])

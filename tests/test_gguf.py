@@ -48,7 +48,7 @@ def hand_made_file(version=3):
 
 def test_header_declares_and_library_exports_the_reader():
     names = declared_symbols("vla_gguf.h")
-    assert len(names) == 18
+    assert len(names) == 19
     for n in names:
         assert hasattr(pkg.lib(), n), "libvla.so does not export %s" % n
 
@@ -184,6 +184,62 @@ def test_gemma_expert_gguf_equals_the_vlaw_checkpoint(tmp_path, arch):
 
 
 @pytest.mark.gpu
+def test_gr00t_head_gguf_equals_the_vlaw_checkpoint(tmp_path, monkeypatch):
+    """GR00T N1.5 action head under the reference's names (src/modules/dit_head.cpp:29-85,
+    src/modules/action_expert.cpp:20-39): per-embodiment stacks with the wanted row at id 24
+    (the default) and noise elsewhere; the tag of embodiment_tag_mapping selects the same row."""
+    from test_gpu_chunk import make_obs
+    cfg = ckpt.gr00t_head_io_config(n_layers=4, ffn_dim=512)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 24)
+    r = np.random.default_rng(333)
+    obs = [make_obs(cfg, r, n_views=2) for _ in range(2)]
+    pv, pg = os.path.join(str(tmp_path), "g.vlaw"), os.path.join(str(tmp_path), "g.gguf")
+    ckpt.write_synthetic(pv, cfg, w)
+    gguf.write_synthetic_gguf(pg, cfg, w)
+    want = _chunk(pv, obs, (2, 16, 32))
+    assert np.array_equal(_chunk(pg, obs, (2, 16, 32)), want) and np.abs(want).max() > 0.1
+    monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "gr1")
+    assert np.array_equal(_chunk(pg, obs, (2, 16, 32)), want)
+    monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "3")  # another row of the stacks: other weights
+    assert not np.array_equal(_chunk(pg, obs, (2, 16, 32)), want)
+    monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "no_such_tag")
+    from vla_cpp_amd import ffi
+    with pytest.raises(RuntimeError):
+        ffi.Model(pg)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("arch", ["pi0", "bitvla"])
+def test_token_embedding_rows_fetched_from_the_file_give_the_resident_result(tmp_path, monkeypatch, arch):
+    """Large vocabularies stay on disk and each request reads its rows (fetch_rows_f32,
+    src/models/pi0.cpp:530-534); forced here on a small file, the chunk is bit-identical."""
+    from test_gpu_chunk import make_obs
+    if arch == "pi0":
+        cfg = ckpt.pi0_config(n_layers=2)
+        cfg.update(ffn_dim=256, time_mlp=1)
+        shape = (2, 50, 32)
+    else:
+        cfg = ckpt.bitvla_config(n_layers=1)
+        shape = (2, 7, 32)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 25)
+    r = np.random.default_rng(334)
+    obs = [make_obs(cfg, r, n_views=1 if arch == "bitvla" else 2) for _ in range(2)]
+    pg = os.path.join(str(tmp_path), "rows.gguf")
+    gguf.write_synthetic_gguf(pg, cfg, w)
+    monkeypatch.setenv("VLA_EMBED_ON_DEMAND", "0")
+    want = _chunk(pg, obs, shape)
+    monkeypatch.setenv("VLA_EMBED_ON_DEMAND", "1")
+    from vla_cpp_amd import ffi
+    m = ffi.Model(pg)
+    got = m.predict_batch(obs).reshape(shape)
+    assert np.array_equal(got, want)
+    bad = dict(obs[0], lang=np.full_like(obs[0]["lang"], cfg["vocab"] + 3))
+    with pytest.raises(RuntimeError, match="-1"):
+        m.predict(bad)
+    m.close()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("packed", [False, True])
 def test_bitvla_gguf_float_and_int2_packed_equal_the_vlaw_checkpoint(tmp_path, packed):
     from test_gpu_chunk import make_obs
@@ -227,3 +283,112 @@ def test_gguf_with_a_missing_or_misshapen_tensor_fails_to_load(tmp_path):
             gguf.write_gguf(p, {"general.architecture": (gguf.STRING, "llama")}, {"t": (gguf.T_F32, np.float32([1]))})
         with pytest.raises(RuntimeError):
             ffi.Model(p)
+
+
+# ------------------------------------------------------------------ the importer's name map
+def _fixture_names():
+    import json
+    with open(os.path.join(os.path.dirname(__file__), "golden", "gguf_tensor_names.json")) as f:
+        return json.load(f)
+
+
+def _tiny(arch):
+    if arch == "gr00t":
+        cfg = ckpt.gr00t_head_io_config(n_layers=3, ffn_dim=256)
+        cfg.update(n_q_heads=4, n_kv_heads=4, head_dim=16, hidden=96, expert_h=64, n_img=8, max_action_dim=8, real_action_dim=8,
+                   max_state_dim=8, real_state_dim=8, num_future=3, n_suffix=1 + 3 + 4, dit_out_dim=32, dec_hidden=48,
+                   state_hidden=40, max_pos=16)
+        return cfg
+    cfg = {"smolvla": ckpt.smolvla_config, "pi0": ckpt.pi0_config, "pi05": ckpt.pi05_config}[arch](n_layers=3)
+    cfg.update(n_q_heads=4, n_kv_heads=2, head_dim=16, hidden=96, expert_h=64, n_img=8, n_lang=6, max_action_dim=8, real_action_dim=8,
+               max_state_dim=8, real_state_dim=8, vocab=40, ffn_dim=128)
+    if arch != "pi05":
+        cfg["time_mlp"] = 1
+    return cfg
+
+
+@pytest.mark.parametrize("arch", ["smolvla", "pi0", "pi05", "gr00t"])
+def test_importer_reads_the_tensor_names_the_reference_converters_write(tmp_path, arch):
+    """The per-block GGUF names the importer asks for are held against the name lists the
+    reference's own converter tests keep as data (tests/golden/gguf_tensor_names.json, from
+    tests/py/test_converters.py:102-111, 178-184), not against this package's writer: the import is
+    traced on the host (vla_gguf_import_trace) and every block-level name it read must be one the
+    reference writes; the blocks on the path must be read completely."""
+    import re
+    fx = _fixture_names()
+    cfg = _tiny(arch)
+    w = ckpt.synth_weights(cfg, seed=5)
+    p = os.path.join(str(tmp_path), arch + ".gguf")
+    gguf.write_synthetic_gguf(p, cfg, w)
+    read = gguf.import_trace(pkg.lib(), p)
+    assert len(read) == len(set(read)), "a tensor was read twice"
+    L = cfg["n_layers"]
+    if arch == "gr00t":
+        for i in range(L):
+            want = {n.format(i=i) for n in fx["dit_block"]["names"]}
+            got = {n for n in read if re.match(r"aex\.dit\.%d\." % i, n)}
+            assert got == want, (i, sorted(got ^ want))
+        # nothing but the DiT head is read: no vision tower, backbone or VL self-attention tensor
+        assert not [n for n in read if n.startswith(("vit.", "vlm.", "mm.", "aex.vlsa", "aex.vlln", "token_embd"))]
+        return
+    allowed = {n.format(p=pfx, i=i) for pfx in fx["decoder_block"]["prefixes"] for i in range(L) for n in fx["decoder_block"]["names"]}
+    block_level = [n for n in read if re.match(r"(vlm|aex)\.blk\.\d+\.", n)]
+    if arch == "pi05":  # the adaRMS dense sits in the norm slots with a bias beside the weight (src/models/pi05.cpp:459-485)
+        block_level = [n for n in block_level if not re.search(r"(attn_norm|ffn_norm)\.bias$", n)]
+    assert block_level and set(block_level) <= allowed, sorted(set(block_level) - allowed)
+    for i in range(L):
+        # expert blocks are read whole; of a backbone block only the pre-norm and the K / V projections are on the path
+        assert {n.format(p="aex", i=i) for n in fx["decoder_block"]["names"]} <= set(read)
+        assert {n for n in read if n.startswith("vlm.blk.%d." % i)} == {
+            "vlm.blk.%d.%s.weight" % (i, s) for s in ("attn_norm", "attn_k", "attn_v")}
+    assert "token_embd.weight" in read and fx["qwen3_lm"]["names"][0] == "token_embd.weight"
+
+
+def test_embedding_rows_left_on_disk_are_traced_not_read(tmp_path, monkeypatch):
+    cfg = _tiny("pi0")
+    w = ckpt.synth_weights(cfg, seed=6)
+    p = os.path.join(str(tmp_path), "lazy.gguf")
+    gguf.write_synthetic_gguf(p, cfg, w)
+    monkeypatch.setenv("VLA_EMBED_ON_DEMAND", "1")
+    assert "token_embd.weight" in gguf.import_trace(pkg.lib(), p)
+
+
+def test_malformed_vlaw_files_are_refused_at_load(tmp_path, capfd):
+    """The flat container's header is checked before anything is uploaded: a record whose byte
+    count does not match its shape and type, a shape that overflows, more than 8 dimensions, an
+    offset or size past the end of the file (also when offset + size wraps around)."""
+    from vla_cpp_amd import ffi
+    cfg = ckpt.smolvla_config(n_layers=1, dtype="f32")
+    w = ckpt.synth_weights(cfg, seed=4)
+    good = os.path.join(str(tmp_path), "good.vlaw")
+    ckpt.write_synthetic(good, cfg, w)
+    blob = open(good, "rb").read()
+    hlen = struct.unpack("<Q", blob[8:16])[0]
+    header = blob[16:16 + hlen].decode()
+    line = next(l for l in header.split("\n") if l.startswith("T ex.0.Wo "))
+    f = line.split()  # T name dtype ndim d0 d1 offset nbytes
+
+    def damaged(new_line):
+        h = header.replace(line, new_line).encode()
+        pad = (-(16 + len(h))) % 64
+        return blob[:8] + struct.pack("<Q", len(h)) + h + b"\0" * pad + blob[(16 + hlen + 63) // 64 * 64:]
+
+    cases = {
+        "bytes do not match the shape": " ".join(f[:7] + [str(int(f[7]) - 4)]),
+        "overflowing shape": " ".join(f[:4] + [str(1 << 62), f[5]] + f[6:]),
+        "too many dimensions": " ".join(f[:3] + ["9"] + ["1"] * 9 + f[6:]),
+        "offset past the end": " ".join(f[:6] + [str(1 << 40), f[7]]),
+        "offset + size wraps": " ".join(f[:6] + [str((1 << 64) - 64), f[7]]),
+        "negative dimension": " ".join(f[:4] + ["-720", f[5]] + f[6:]),
+    }
+    for name, new_line in cases.items():
+        p = os.path.join(str(tmp_path), "bad.vlaw")
+        open(p, "wb").write(damaged(new_line))
+        with pytest.raises(RuntimeError):
+            ffi.Model(p)
+        err = capfd.readouterr().err
+        assert "ex.0.Wo" in err, (name, err)
+    open(os.path.join(str(tmp_path), "cut.vlaw"), "wb").write(blob[:len(blob) // 2])
+    with pytest.raises(RuntimeError):
+        ffi.Model(os.path.join(str(tmp_path), "cut.vlaw"))
+    assert "outside the checkpoint" in capfd.readouterr().err

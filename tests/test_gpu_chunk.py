@@ -27,7 +27,7 @@ def bf16_close(got, want):
 
 def make_obs(cfg, r, n_views, n_lang=None, bf16_inputs=False):
     A = cfg["max_action_dim"]
-    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "bitvla", "pi05") else 1)
+    n_act = cfg["n_suffix"] - (0 if cfg["arch"] in ("smolvla", "bitvla", "pi05") else 1 + cfg.get("num_future", 0) * cfg.get("head_io", 0))
     img = r.standard_normal((n_views * cfg["n_img"], cfg["hidden"])).astype(np.float32)
     if cfg["arch"] == "smolvla":
         img /= np.sqrt(cfg["hidden"])  # the prefix builder scales image rows by sqrt(hidden)
@@ -129,6 +129,36 @@ def test_config3_gr00t_dit_bf16(tmp_path, n_layers, batch):
         if b == 0:  # and the pure fp32 CPU reference, which is what the tolerance is quoted against
             want32 = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=False)
             assert bf16_close(got[b], want32), np.abs(got[b] - want32).max()
+    m.close()
+
+
+@pytest.mark.parametrize("dtype,n_layers,batch", [("f32", 2, 1), ("bf16", 4, 2), ("bf16", 16, 1)])
+def test_gr00t_with_the_dit_heads_own_input_and_output_mlps(tmp_path, dtype, n_layers, batch):
+    # The real GR00T N1.5 head (src/models/gr00tn1d5.cpp:366-381): state token from encode_state,
+    # 32 learned future tokens, 16 action tokens from encode_action (step sinusoid, learned
+    # positions), 49 tokens through DiT blocks with their FFN, velocity = decode(proj_out(h)).
+    cfg = ckpt.gr00t_head_io_config(n_layers=n_layers, dtype=dtype, ffn_dim=1024 if n_layers < 16 else 6144)
+    if dtype == "f32":
+        cfg.update(head_dim=64, n_q_heads=8, n_kv_heads=8, expert_h=512, dit_out_dim=256, dec_hidden=256, state_hidden=256)  # fp32 heads of 48 are not built
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 31)
+    r = np.random.default_rng(310 + n_layers)
+    obs = [make_obs(cfg, r, n_views=2) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "gr00t_io")
+    got = m.predict_batch(obs).reshape(batch, 16, 32)
+    assert m.config().n_suffix == 49
+    for b in range(batch):
+        if dtype == "f32":
+            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b])
+            assert rel_err(got[b], want) < 1e-5, rel_err(got[b], want)
+        else:
+            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+            assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+            if b == 0:
+                want32 = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=False)
+                assert bf16_close(got[b], want32), np.abs(got[b] - want32).max()
+    # the state really enters through encode_state: another state, another chunk
+    other = dict(obs[0], state=obs[0]["state"] + 1.0)
+    assert np.abs(m.predict(other).reshape(16, 32) - got[0]).max() > 1e-4
     m.close()
 
 
@@ -321,3 +351,16 @@ def test_bad_inputs_are_argument_errors_not_crashes(tmp_path):
     m.close()
     with pytest.raises(RuntimeError):
         ffi.Model(os.path.join(str(tmp_path), "missing.vlaw"))
+    # a file whose tensors do not match its own configuration fails at load, whichever tensor it is
+    for name, cut in (("ex.0.Wo", (slice(None), slice(0, -16))), ("vlm.0.Wkv", (slice(0, -64), slice(None))), ("act.W_out", (slice(0, -1), slice(None))),
+                      ("ex.0.ln", (slice(0, -8),))):
+        w2 = dict(w)
+        w2[name] = np.ascontiguousarray(w[name][cut])
+        with pytest.raises(RuntimeError):
+            load(tmp_path, cfg, w2, "misshapen")
+    cfg4 = ckpt.bitvla_config(n_layers=1)
+    w4 = ckpt.synth_weights(cfg4, seed=1)
+    w4["lm.0.Wo.t"] = w4["lm.0.Wo.t"][:-32]
+    for pack in (None, orc.pack_ladder_int2):
+        with pytest.raises(RuntimeError):
+            load(tmp_path, cfg4, w4, "misshapen4", ladder_pack=pack)

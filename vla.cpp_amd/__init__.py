@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libvla.so")
 
 VLA_DT_F32, VLA_DT_BF16, VLA_DT_BF16_P2 = 0, 1, 2
-VLA_ACT_NONE, VLA_ACT_SILU, VLA_ACT_GELU = 0, 1, 2
+VLA_ACT_NONE, VLA_ACT_SILU, VLA_ACT_GELU, VLA_ACT_RELU = 0, 1, 2, 3
 VLA_MASK_NONE, VLA_MASK_CAUSAL_SUFFIX, VLA_MASK_PI0_STATE = 0, 1, 2
 VLA_K_OK, VLA_K_ERR_ARG, VLA_K_ERR_SHAPE, VLA_K_ERR_LAUNCH, VLA_K_ERR_WORKSPACE = 0, -1, -2, -3, -4
 
@@ -48,6 +48,7 @@ KERNEL_API = {
     "vla_attn_workspace_bytes": [_i, _i, _i, _i, _i, _i, _i],
     "vla_embed_suffix": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "vla_embed_suffix_act": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "vla_finish_suffix_rows": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "vla_set_lead_rows": [_vp, _vp, _i, _i, _i, _i, _i, _vp],
     "vla_euler_step": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
     "vla_act_quant_bf16": [_vp, _vp, _vp, _vp, _i, _i, _vp],

@@ -95,6 +95,18 @@ def gr00t_config(n_layers=16, dtype="bf16", num_steps=4, n_suffix=17):
                 norm_out_eps=1e-6, rope_freq_base=10000.0, vocab=0, suffix_mask=0, max_views=2)
 
 
+def gr00t_head_io_config(n_layers=16, dtype="bf16", num_steps=4, ffn_dim=6144):
+    """GR00T N1.5 with the DiT head's own input / output MLPs (src/models/gr00tn1d5.cpp:281, 366-381;
+    src/modules/action_expert.cpp:41-59; src/modules/dit_head.cpp:139-147): the sequence is
+    1 state token (encode_state) + 32 learned future tokens + 16 action tokens (encode_action with
+    the step's sinusoid and learned positions), every block has its FFN, and the velocity is
+    decode(proj_out(h)) on the action rows."""
+    c = gr00t_config(n_layers, dtype, num_steps, n_suffix=1 + 32 + 16)
+    c.update(head_io=1, num_future=32, dit_out_dim=1024, dec_hidden=1024, state_hidden=1024, ffn_dim=ffn_dim,
+             num_buckets=1000, max_pos=1024)
+    return c
+
+
 def gr00t_n1d6_config(n_layers=32, dtype="bf16", num_steps=4, n_suffix=17, attend_text_every_n=2, dit_interleave=1):
     """GR00T N1.6 / N1.7 DiT head (AlternateVLDiT, src/models/gr00tn1d6.cpp:85-86, 445-467;
     src/models/gr00tn1d7.cpp:75, 565-590): the N1.5 block, 32 layers, whose cross layers
@@ -173,10 +185,26 @@ def synth_weights(cfg, seed=0x5EED):
     elif arch != "pi05":
         w["act.W_sp"] = (0.1 * r.standard_normal((W, cfg["max_state_dim"]))).astype(np.float32)
         w["act.b_sp"] = vec(W, 0.1)
-    w["act.W_in"] = (0.1 * r.standard_normal((W, A))).astype(np.float32)
-    w["act.b_in"] = vec(W, 0.1)
-    w["act.W_out"] = (0.02 * r.standard_normal((A, W))).astype(np.float32)
-    w["act.b_out"] = vec(A)
+    if cfg.get("head_io", 0):
+        del w["act.W_sp"], w["act.b_sp"]
+        Hs, Hd, O, NF = cfg["state_hidden"], cfg["dec_hidden"], cfg["dit_out_dim"], cfg["num_future"]
+        f32m = lambda n, k, s_: (s_ * r.standard_normal((n, k))).astype(np.float32)
+        w["aex.se_l1W"], w["aex.se_l1b"] = f32m(Hs, cfg["max_state_dim"], 0.1), vec(Hs, 0.1)
+        w["aex.se_l2W"], w["aex.se_l2b"] = f32m(W, Hs, 1.0 / np.sqrt(Hs)), vec(W, 0.1)
+        w["aex.ae_W1"], w["aex.ae_b1"] = f32m(W, A, 0.1), vec(W, 0.1)
+        w["aex.ae_W2"], w["aex.ae_b2"] = f32m(W, 2 * W, 1.0 / np.sqrt(2 * W)), vec(W, 0.1)
+        w["aex.ae_W3"], w["aex.ae_b3"] = f32m(W, W, 1.0 / np.sqrt(W)), vec(W, 0.1)
+        w["aex.pos_embd"] = f32m(cfg.get("max_pos", 64), W, 0.02)
+        w["aex.future_tokens"] = f32m(NF, W, 0.5)
+        w["aex.po1W"], w["aex.po1b"] = f32m(2 * W, W, 0.02), vec(2 * W)
+        w["aex.po2W"], w["aex.po2b"] = mat(O, W), vec(O)
+        w["aex.ad_l1W"], w["aex.ad_l1b"] = mat(Hd, O), vec(Hd)
+        w["aex.ad_l2W"], w["aex.ad_l2b"] = f32m(A, Hd, 0.02), vec(A)
+    else:
+        w["act.W_in"] = (0.1 * r.standard_normal((W, A))).astype(np.float32)
+        w["act.b_in"] = vec(W, 0.1)
+        w["act.W_out"] = (0.02 * r.standard_normal((A, W))).astype(np.float32)
+        w["act.b_out"] = vec(A)
     # adaRMS modulation dense: rows [scale; shift; gate], the gate around 1 (pi05.cpp:208-224)
     ada_w = lambda: (0.5 * r.standard_normal((3 * W, W)) / np.sqrt(W)).astype(np.float32)
     ada_b = lambda: np.concatenate([vec(2 * W, 0.05), 1.0 + vec(W, 0.05)]).astype(np.float32)
@@ -244,7 +272,7 @@ def synth_weights(cfg, seed=0x5EED):
     return w
 
 
-_F32_NAMES = ("prefix.", "act.", "te.")
+_F32_NAMES = ("prefix.", "act.", "te.", "aex.")
 
 
 def write_synthetic(path, cfg, weights, ladder_pack=None, plain_pack=None):

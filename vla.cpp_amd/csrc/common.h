@@ -241,10 +241,11 @@ __device__ __forceinline__ void rms_act_quant_row(const bf16_t* __restrict__ xr,
     sum_out = sum;
 }
 
-// ggml_silu / ggml_gelu (tanh form), fp32 (src/layers/ffn.h:24-40).
+// ggml_silu / ggml_gelu (tanh form) / ggml_relu, fp32 (src/layers/ffn.h:24-40, src/modules/action_expert.cpp:41-59).
 __device__ __forceinline__ float apply_act(float x, int act) {
     if (act == VLA_ACT_SILU) return x / (1.0f + __expf(-x));
     if (act == VLA_ACT_GELU) return 0.5f * x * (1.0f + tanhf(0.79788456080286535588f * x * (1.0f + 0.044715f * x * x)));
+    if (act == VLA_ACT_RELU) return x > 0.f ? x : 0.f;
     return x;
 }
 

@@ -369,6 +369,24 @@ __global__ void lead_rows_kernel(const float* __restrict__ lead, T* __restrict__
     Elem<T>::store(h + ((long)b * S + s) * W + c, lead[i]);
 }
 
+// h[b][s][:] = lead[b][s][:] for s < n_lead, else acc[b][s][:] + table[s - n_lead][:], converted
+// to T: the last step of a suffix embedding whose action rows came out of an fp32 projection
+// over all rows and carry a learned per-position term.
+template <typename T>
+__global__ void finish_suffix_rows_kernel(const float* __restrict__ acc, const float* __restrict__ table,
+                                          const float* __restrict__ lead, T* __restrict__ h, long total, int S, int n_lead, int W) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int c = (int)(i % W);
+    const long bs = i / W;
+    const int s = (int)(bs % S);
+    const long b = bs / S;
+    float v;
+    if (s < n_lead) v = lead[((long)b * n_lead + s) * W + c];
+    else v = acc[i] + (table ? table[(long)(s - n_lead) * W + c] : 0.f);
+    Elem<T>::store(h + i, v);
+}
+
 // Workgroup (x, y): EUL_WAVES wavefronts, each owning ROWS action rows, all working on the
 // AU action outputs of group y.  A lane keeps elements lane, lane+64, ... of its rows in
 // registers (NC chunks cover the width); the chunk loads of the AU rows of W_out are
@@ -717,11 +735,26 @@ int vla_set_lead_rows(const float* lead, void* h, int dtype, int batch, int S, i
     return VLA_CHECK_LAUNCH();
 }
 
+int vla_finish_suffix_rows(const float* acc, const float* row_table, const float* lead, void* h, int dtype, int batch, int S,
+                           int n_lead, int W, vla_stream_t stream) {
+    if (!acc || !h || batch < 0 || S <= 0 || n_lead < 0 || n_lead > S || W <= 0 || (n_lead > 0 && !lead)) return VLA_K_ERR_ARG;
+    if (batch == 0) return VLA_K_OK;
+    const long total = (long)batch * S * W;
+    const unsigned blocks = (unsigned)((total + 255) / 256);
+    if (dtype == VLA_DT_F32)
+        finish_suffix_rows_kernel<float><<<blocks, 256, 0, (hipStream_t)stream>>>(acc, row_table, lead, (float*)h, total, S, n_lead, W);
+    else if (dtype == VLA_DT_BF16)
+        finish_suffix_rows_kernel<bf16_t><<<blocks, 256, 0, (hipStream_t)stream>>>(acc, row_table, lead, (bf16_t*)h, total, S, n_lead, W);
+    else
+        return VLA_K_ERR_ARG;
+    return VLA_CHECK_LAUNCH();
+}
+
 int vla_embed_suffix_act(const float* x_t, const float* W_in, const float* bias_step, const float* lead, void* h,
                          int out_dtype, int batch, int S, int n_lead, int A, int W, int act, vla_stream_t stream) {
     if (!x_t || !W_in || !bias_step || !h || batch < 0 || S <= 0 || n_lead < 0 || n_lead > S || A <= 0 || W <= 0)
         return VLA_K_ERR_ARG;
-    if (act < VLA_ACT_NONE || act > VLA_ACT_GELU) return VLA_K_ERR_ARG;
+    if (act < VLA_ACT_NONE || act > VLA_ACT_RELU) return VLA_K_ERR_ARG;
     if (n_lead > 0 && !lead) return VLA_K_ERR_ARG;
     if (A > EMB_MAX_A) return VLA_K_ERR_SHAPE;
     if (batch == 0) return VLA_K_OK;

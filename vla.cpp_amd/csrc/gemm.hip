@@ -1442,7 +1442,7 @@ int vla_linear_act(const void* x, const void* W, const float* bias, const void* 
                    int out_dtype, int M, int N, int K, int act, vla_stream_t stream) {
     if (!x || !W || !y || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
     if (out_dtype != VLA_DT_F32 && out_dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
-    if (act < VLA_ACT_NONE || act > VLA_ACT_GELU) return VLA_K_ERR_ARG;
+    if (act < VLA_ACT_NONE || act > VLA_ACT_RELU) return VLA_K_ERR_ARG;
     GemmArgs a = {};
     a.norm_eps = -1.f;
     a.A = x; a.W = W; a.bias = bias; a.M = M; a.N = N; a.K = K;
@@ -1483,7 +1483,7 @@ int vla_glu_linear(const void* x, const void* W_gate_up, const float* bias, void
                    int K, int act, float rms_eps, vla_stream_t stream) {
     if (!x || !W_gate_up || !y || M < 0 || I <= 0 || K <= 0) return VLA_K_ERR_ARG;
     if (out_dtype != VLA_DT_F32 && out_dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
-    if (act < VLA_ACT_NONE || act > VLA_ACT_GELU) return VLA_K_ERR_ARG;
+    if (act < VLA_ACT_NONE || act > VLA_ACT_RELU) return VLA_K_ERR_ARG;
     if (I % 32) return VLA_K_ERR_SHAPE;  // a tile pairs 32 gate columns with their 32 up columns
     GemmArgs a = {};
     a.norm_eps = rms_eps >= 0.f ? rms_eps : -1.f;

@@ -287,6 +287,70 @@ def write_synthetic_gguf(path, cfg, w, ladder_pack=None):
                 else:
                     # floats whose absmean quantisation gives back (tern, scale): see checkpoint._dequant_sources
                     t[b + name + ".weight"] = f32(tern.astype(np.float32) * np.float32(scale))
+    elif cfg["arch"] == "gr00t_n1d5" and cfg.get("head_io", 0):
+        # GR00T N1.5 action head (src/models/gr00tn1d5.cpp:92-147; src/modules/dit_head.cpp:29-85;
+        # src/modules/action_expert.cpp:20-39): the head's MLPs are cat_linear stacks, one
+        # [in][out] matrix per embodiment (ggml ne = [out, in, n]); the synthetic weights go into
+        # row `embodiment`, the other rows hold noise that must not be read.
+        W, Wv, I, A = cfg["expert_h"], cfg["hidden"], cfg["ffn_dim"], cfg["max_action_dim"]
+        n_emb, emb = cfg.get("max_embodiments", 32), cfg.get("embodiment", 24)
+        rr = np.random.default_rng(99)
+        kv["gr00t_n1_5.architecture"] = (STRING, "gr00t_n1_5")
+        for k, v in (("backbone_embedding_dim", Wv), ("input_embedding_dim", W), ("dit_hidden", W), ("dit_heads", Hq),
+                     ("dit_head_dim", D), ("dit_layers", L), ("dit_interleave", cfg.get("dit_interleave", 1)),
+                     ("num_target_vision_tokens", cfg["num_future"]), ("action_horizon", cfg["n_suffix"] - 1 - cfg["num_future"]),
+                     ("action_dim", A), ("max_state_dim", cfg["max_state_dim"]), ("num_inference_timesteps", cfg["num_steps"]),
+                     ("num_timestep_buckets", cfg.get("num_buckets", 1000)), ("max_num_embodiments", n_emb),
+                     ("n_img_tokens", cfg["n_img"])):
+            kv["gr00t_n1_5." + k] = (U32, int(v))
+        kv["gr00t_n1_5.ln_eps"] = (F32, float(cfg["rms_eps"]))
+        kv["gr00t_n1_5.norm_out_eps"] = (F32, float(cfg["norm_out_eps"]))
+        kv["gr00t_n1_5.embodiment_tag_mapping"] = (STRING, '{"new_embodiment":31,"gr1":%d}' % emb)
+
+        def cat(wm, b):  # [out][in] weight, [out] bias -> per-embodiment stacks
+            wm, b = np.asarray(wm, np.float32), np.asarray(b, np.float32)
+            W3 = rr.standard_normal((n_emb, wm.shape[1], wm.shape[0])).astype(np.float32)
+            B2 = rr.standard_normal((n_emb, wm.shape[0])).astype(np.float32)
+            W3[emb], B2[emb] = wm.T, b
+            return f32(W3), f32(B2)
+
+        # (the synthetic time-embedding weights are not bf16 values: kept F32 so the file equals the VLAW container)
+        t["aex.dit.time_emb.l1.weight"], t["aex.dit.time_emb.l1.bias"] = f32(w["te.l1W"]), f32(w["te.l1b"])
+        t["aex.dit.time_emb.l2.weight"], t["aex.dit.time_emb.l2.bias"] = f32(w["te.l2W"]), f32(w["te.l2b"])
+        t["aex.dit.proj_out1.weight"], t["aex.dit.proj_out1.bias"] = f32(w["aex.po1W"]), f32(w["aex.po1b"])
+        t["aex.dit.proj_out2.weight"], t["aex.dit.proj_out2.bias"] = _wt(cfg, w["aex.po2W"]), f32(w["aex.po2b"])
+        for g_name, wn, bn in (("state_enc.l1", "se_l1W", "se_l1b"), ("state_enc.l2", "se_l2W", "se_l2b"), ("act_enc.W1", "ae_W1", "ae_b1"),
+                               ("act_enc.W2", "ae_W2", "ae_b2"), ("act_enc.W3", "ae_W3", "ae_b3"), ("act_dec.l1", "ad_l1W", "ad_l1b"),
+                               ("act_dec.l2", "ad_l2W", "ad_l2b")):
+            t["aex.%s.W" % g_name], t["aex.%s.b" % g_name] = cat(w["aex." + wn], w["aex." + bn])
+        t["aex.pos_embd"], t["aex.future_tokens"] = f32(w["aex.pos_embd"]), f32(w["aex.future_tokens"])
+        interleave = bool(cfg.get("dit_interleave", 1))
+        for l in range(L):
+            a, e, p = "aex.dit.%d." % l, "ex.%d." % l, "vlm.%d." % l
+            t[a + "adaln.weight"], t[a + "adaln.bias"] = _wt(cfg, w[e + "adaln_w"]), f32(w[e + "adaln_b"])
+            if interleave and l % 2 == 1:
+                Wqkv, bqkv = w[e + "Wqkv"], w[e + "bqkv"]
+                parts = ((Wqkv[:W], bqkv[:W]), (Wqkv[W:2 * W], bqkv[W:2 * W]), (Wqkv[2 * W:], bqkv[2 * W:]))
+            else:
+                Wkv, bkv = w[p + "Wkv"], w[p + "bkv"]
+                parts = ((w[e + "Wq"], w[e + "bq"]), (Wkv[:W], bkv[:W]), (Wkv[W:], bkv[W:]))
+            for nm, (wm, bm) in zip(("attn_q", "attn_k", "attn_v"), parts):
+                t[a + nm + ".weight"], t[a + nm + ".bias"] = _wt(cfg, wm), f32(bm)
+            t[a + "attn_o.weight"], t[a + "attn_o.bias"] = _wt(cfg, w[e + "Wo"]), f32(w[e + "bo"])
+            t[a + "ff0.weight"], t[a + "ff0.bias"] = _wt(cfg, w[e + "W1"]), f32(w[e + "b1"])
+            t[a + "ff2.weight"], t[a + "ff2.bias"] = _wt(cfg, w[e + "W2"]), f32(w[e + "b2"])
     else:
         raise ValueError("no GGUF layout for arch %r" % cfg["arch"])
     write_gguf(path, kv, t)
+
+
+def import_trace(lib, path):
+    """Names of the GGUF tensors the library's checkpoint import reads from `path`, in order
+    (vla_gguf_import_trace); raises when the file cannot be imported."""
+    lib.vla_gguf_import_trace.restype = ctypes.c_int64
+    lib.vla_gguf_import_trace.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int64]
+    buf = ctypes.create_string_buffer(1 << 20)
+    n = lib.vla_gguf_import_trace(path.encode(), buf, len(buf))
+    if n < 0:
+        raise RuntimeError("vla_gguf_import_trace returned %d" % n)
+    return buf.value.decode().split("\n")[:-1]

@@ -50,6 +50,8 @@ TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::
     std::vector<uint32_t> packed((size_t)vla_ternary_packed_words(w.N, K));
     std::vector<float> scales;
     if (ck.has(name + ".i2")) {
+        if (ck.info(name + ".i2").nbytes != (size_t)w.N * K / 4 || w.N % 16 || K % 128)
+            throw std::runtime_error("vla: " + name + ".i2 does not hold " + std::to_string(w.N) + " x " + std::to_string(K) + " ladder-packed weights");
         VLA_K(vla_ternary_repack_ladder_host((const uint8_t*)ck.data(name + ".i2"), w.N, K, packed.data()));
         scales = ck.f32(name + ".ws");
         if (scales.size() != parts.size()) throw std::runtime_error("vla: " + name + ".ws has the wrong length");
@@ -59,6 +61,7 @@ TernaryW load_ternary(const Checkpoint& ck, const std::string& name, const std::
         scales = ck.f32(name + ".ws");
         if (scales.size() != parts.size()) throw std::runtime_error("vla: " + name + ".ws has the wrong length");
     } else {
+        ck.expect(name, {(int64_t)w.N, (int64_t)K});
         const std::vector<float> W = ck.f32(name);
         std::vector<int8_t> tern((size_t)w.N * K);
         size_t row = 0;
@@ -113,6 +116,7 @@ class BitvlaLm : public ModelArch {
     float eps_;
     std::vector<LmLayer> layers_;
     std::vector<float> E_lang_, act_emb_;
+    std::shared_ptr<RowSource> lang_rows_;
     DevBuf out_norm_, W_out_, b_out_;
     RopeTable rope_;
     AttnWorkspace attn_ws_;
@@ -144,7 +148,17 @@ BitvlaLm::BitvlaLm(const Checkpoint& ck) {
     cfg.num_steps = n_act_; cfg.rms_eps = eps_; cfg.rope_n_dims = D_;
     cfg.rope_freq_base = (float)ck.f64("rope_freq_base", 500000.0);
 
-    E_lang_ = ck.f32("prefix.E_lang");
+    lang_rows_ = ck.row_source("prefix.E_lang");  // a large vocabulary stays on disk
+    if (lang_rows_) {
+        if (lang_rows_->rows != vocab_ || lang_rows_->cols != H_) throw std::runtime_error("vla: token embedding matrix does not match vocab x hidden");
+    } else {
+        ck.expect("prefix.E_lang", {(int64_t)vocab_, (int64_t)H_});
+        E_lang_ = ck.f32("prefix.E_lang");
+    }
+    ck.expect("act.emb", {(int64_t)n_act_, (int64_t)H_});
+    ck.expect("act.norm", {(int64_t)H_});
+    ck.expect("act.W_out", {(int64_t)A_, (int64_t)H_});
+    ck.expect("act.b_out", {(int64_t)A_});
     act_emb_ = ck.f32("act.emb");
     std::vector<float> nf = ck.f32("act.norm");
     upload_as(out_norm_, nf.data(), nf.size(), VLA_DT_BF16);
@@ -155,12 +169,16 @@ BitvlaLm::BitvlaLm(const Checkpoint& ck) {
     for (int l = 0; l < L_; ++l) {
         const std::string p = "lm." + std::to_string(l) + ".";
         LmLayer& w = layers_[l];
+        ck.expect(p + "attn_norm", {(int64_t)H_});
+        ck.expect(p + "sub_norm", {(int64_t)H_});
         std::vector<float> a = ck.f32(p + "attn_norm"), s = ck.f32(p + "sub_norm");
         upload_as(w.attn_norm, a.data(), a.size(), VLA_DT_BF16);
         upload_as(w.sub_norm, s.data(), s.size(), VLA_DT_BF16);
         w.Wqkv = load_ternary(ck, p + "Wqkv", {H_, kvd, kvd}, H_, kvd, Hq_, Hkv_, D_);
         w.Wo = load_ternary(ck, p + "Wo", {H_}, H_, H_);
         if (F_ > 0) {
+            ck.expect(p + "ffn_norm", {(int64_t)H_});
+            ck.expect(p + "ffn_sub_norm", {(int64_t)F_});
             std::vector<float> fn = ck.f32(p + "ffn_norm"), fs = ck.f32(p + "ffn_sub_norm");
             upload_as(w.ffn_norm, fn.data(), fn.size(), VLA_DT_BF16);
             upload_as(w.ffn_sub_norm, fs.data(), fs.size(), VLA_DT_BF16);
@@ -213,8 +231,14 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
     for (int b = 0; b < B; ++b) {
         uint16_t* dst = emb.data() + (size_t)b * P * H_;
         for (size_t i = 0; i < (size_t)n_img_ * H_; ++i) dst[i] = f32_to_bf16(in[b].precomputed_img_emb[i]);
+        std::vector<float> fetched;
+        if (lang_rows_) {
+            fetched.resize((size_t)n_lang_ * H_);
+            const std::vector<int32_t> ids(in[b].lang_tokens, in[b].lang_tokens + n_lang_);
+            if (n_lang_ > 0 && !lang_rows_->fetch(ids, fetched.data())) throw std::runtime_error("vla: cannot read token embedding rows");
+        }
         for (int i = 0; i < n_lang_; ++i) {
-            const float* e = E_lang_.data() + (size_t)in[b].lang_tokens[i] * H_;
+            const float* e = lang_rows_ ? fetched.data() + (size_t)i * H_ : E_lang_.data() + (size_t)in[b].lang_tokens[i] * H_;
             for (int c = 0; c < H_; ++c) dst[(size_t)(n_img_ + i) * H_ + c] = f32_to_bf16(e[c]);
         }
     }

@@ -18,12 +18,30 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <sstream>
 #include <stdexcept>
 #include <string>
 #include <vector>
 
 namespace vla {
+
+// Rows of a matrix that stays on disk and is read per request: the token embeddings of a
+// 257k-row vocabulary are 2 GB as fp32, and one observation uses a few dozen rows (the
+// reference fetches them the same way, fetch_rows_f32, src/models/pi0.cpp:530-534).
+struct RowSource {
+    int64_t rows = 0, cols = 0;
+    virtual ~RowSource() = default;
+    // dst receives ids.size() x cols floats; false on an id outside [0, rows) or a read error
+    virtual bool fetch(const std::vector<int32_t>& ids, float* dst) = 0;
+};
+
+inline size_t ckpt_dtype_size(const std::string& dt) {
+    if (dt == "f32" || dt == "i32") return 4;
+    if (dt == "bf16") return 2;
+    if (dt == "i8" || dt == "u8") return 1;
+    return 0;
+}
 
 struct CkptTensor {
     std::string dtype;
@@ -76,8 +94,9 @@ class Checkpoint {
             throw std::runtime_error("vla: " + path + " is not a VLAW0001 checkpoint");
         uint64_t hlen = 0;
         std::memcpy(&hlen, blob_.data() + 8, 8);
-        if (16 + hlen > (uint64_t)sz) throw std::runtime_error("vla: truncated checkpoint header");
+        if (hlen > (uint64_t)sz - 16) throw std::runtime_error("vla: truncated checkpoint header");
         data_ = (16 + (size_t)hlen + 63) / 64 * 64;
+        if (data_ > blob_.size()) data_ = blob_.size();
         std::istringstream hs(std::string(blob_.data() + 16, (size_t)hlen));
         std::string line;
         while (std::getline(hs, line)) {
@@ -93,11 +112,23 @@ class Checkpoint {
                 CkptTensor t;
                 int ndim = 0;
                 ls >> name >> t.dtype >> ndim;
-                t.shape.resize(ndim);
-                for (int i = 0; i < ndim; ++i) ls >> t.shape[i];
+                if (!ls || ndim < 0 || ndim > 8) throw std::runtime_error("vla: tensor " + name + " has a malformed record");
+                t.shape.resize((size_t)ndim);
+                int64_t numel = 1;
+                for (int i = 0; i < ndim; ++i) {
+                    ls >> t.shape[i];
+                    if (!ls || t.shape[i] <= 0 || t.shape[i] > ((int64_t)1 << 40) / numel)
+                        throw std::runtime_error("vla: tensor " + name + " has a malformed shape");
+                    numel *= t.shape[i];
+                }
                 ls >> t.offset >> t.nbytes;
-                if (!ls || data_ + t.offset + t.nbytes > blob_.size())
+                const size_t room = blob_.size() - data_;  // data_ <= blob_.size() was checked above
+                const size_t es = ckpt_dtype_size(t.dtype);
+                if (!ls || es == 0 || t.offset > room || t.nbytes > room - t.offset)
                     throw std::runtime_error("vla: tensor " + name + " lies outside the checkpoint");
+                if (t.nbytes != (size_t)numel * es)
+                    throw std::runtime_error("vla: tensor " + name + " declares " + std::to_string(t.nbytes) + " bytes for " +
+                                             std::to_string(numel) + " " + t.dtype + " elements");
                 tensors_[name] = t;
             }
         }
@@ -110,6 +141,33 @@ class Checkpoint {
         return it->second;
     }
     const void* data(const std::string& name) const { return blob_.data() + data_ + info(name).offset; }
+    // info(name), after checking that the tensor has exactly this shape: a file whose tensors
+    // do not match its own configuration must fail at load, not as an out-of-bounds read on
+    // the device.
+    const CkptTensor& expect(const std::string& name, const std::vector<int64_t>& shape) const {
+        const CkptTensor& t = info(name);
+        auto squeeze = [](const std::vector<int64_t>& v) {  // [1, W] and [W] name the same vector
+            std::vector<int64_t> o;
+            for (int64_t d : v)
+                if (d != 1) o.push_back(d);
+            return o;
+        };
+        if (squeeze(t.shape) != squeeze(shape)) {
+            std::string got, want;
+            for (int64_t d : t.shape) got += (got.empty() ? "" : " x ") + std::to_string(d);
+            for (int64_t d : shape) want += (want.empty() ? "" : " x ") + std::to_string(d);
+            throw std::runtime_error("vla: checkpoint tensor " + name + " is [" + got + "], expected [" + want + "]");
+        }
+        return t;
+    }
+
+    // A matrix left on disk (see RowSource); the model keeps the pointer after the
+    // checkpoint object is gone.
+    void set_row_source(const std::string& name, std::shared_ptr<RowSource> src) { rows_[name] = std::move(src); }
+    std::shared_ptr<RowSource> row_source(const std::string& name) const {
+        auto it = rows_.find(name);
+        return it == rows_.end() ? nullptr : it->second;
+    }
 
     // Tensor as fp32 on the host (bf16 widened exactly).
     std::vector<float> f32(const std::string& name) const {
@@ -145,6 +203,7 @@ class Checkpoint {
     size_t data_ = 0;
     std::map<std::string, std::string> kv_;
     std::map<std::string, CkptTensor> tensors_;
+    std::map<std::string, std::shared_ptr<RowSource>> rows_;
 };
 
 // GGUF input (gguf_import.cpp): true when the file starts with the GGUF magic; import_gguf

@@ -38,8 +38,11 @@ enum class Arch { SMOLVLA, PI0, GR00T };
 
 int round_up(int x, int m) { return (x + m - 1) / m * m; }
 
-DevBuf load_w(const Checkpoint& ck, const std::string& name, int dtype) {
-    const CkptTensor& t = ck.info(name);
+// Every load names the shape the configuration implies: a file whose tensors do not match its
+// own keys fails here, not as a device read past a buffer.
+using Shape = std::vector<int64_t>;
+DevBuf load_w(const Checkpoint& ck, const std::string& name, int dtype, const Shape& shape) {
+    const CkptTensor& t = ck.expect(name, shape);
     DevBuf b;
     if ((dtype == VLA_DT_F32 && t.dtype == "f32") || (dtype == VLA_DT_BF16 && t.dtype == "bf16")) {
         b.upload(ck.data(name), t.nbytes);
@@ -49,12 +52,16 @@ DevBuf load_w(const Checkpoint& ck, const std::string& name, int dtype) {
     }
     return b;
 }
-DevBuf load_f32(const Checkpoint& ck, const std::string& name) { return load_w(ck, name, VLA_DT_F32); }
+DevBuf load_f32(const Checkpoint& ck, const std::string& name, const Shape& shape) { return load_w(ck, name, VLA_DT_F32, shape); }
+std::vector<float> host_f32(const Checkpoint& ck, const std::string& name, const Shape& shape) {
+    ck.expect(name, shape);
+    return ck.f32(name);
+}
 
 // bf16 copy of weight `name` [N][K] with the RMSNorm weight `ln` [K] multiplied into its
 // columns, for the projection launch that takes the layer's pre-norm inside it.
-DevBuf load_folded_bf16(const Checkpoint& ck, const std::string& name, const std::string& ln) {
-    const std::vector<float> wf = ck.f32(name), gf = ck.f32(ln);
+DevBuf load_folded_bf16(const Checkpoint& ck, const std::string& name, const std::string& ln, int64_t rows, int64_t cols) {
+    const std::vector<float> wf = host_f32(ck, name, {rows, cols}), gf = host_f32(ck, ln, {cols});
     const size_t K = gf.size(), N = wf.size() / K;
     std::vector<uint16_t> w(wf.size()), g(K);
     for (size_t i = 0; i < wf.size(); ++i) w[i] = f32_to_bf16(wf[i]);
@@ -124,6 +131,13 @@ class FlowExpert : public ModelArch {
     DevBuf W_in_, W_out_, b_out_, final_norm_;
     DevBuf W_at2_, b_at2_, m1_;  // action-time MLP: second projection, fp32 scratch [B*S][W]
     bool time_mlp_ = false;
+    // GR00T with the DiT head's own input / output MLPs (ActionExpert::encode_state / encode_action /
+    // decode, src/modules/action_expert.cpp:41-59; DitHead::proj_out, src/modules/dit_head.cpp:139-147)
+    bool head_io_ = false;
+    int n_future_ = 0, O_ = 0, Hd_ = 0, Hs_ = 0;  // future tokens, DiT output width, decoder / state-encoder hidden widths
+    std::vector<float> se_l1W_, se_l1b_, se_l2W_, se_l2b_, future_;
+    DevBuf W3_, b3_, pos_, m2_, po2W_, po2b_, ad1W_, ad1b_, d1_, d2_;
+    std::shared_ptr<RowSource> lang_rows_;  // token embeddings left on disk (large vocabularies)
     bool alt_vl_ = false;   // GR00T N1.6 / N1.7: cross layers alternate text / image rows
     int text_every_ = 2, P_txt_ = 0;
     bool adarms_ = false;  // pi0.5: ada_ holds [steps][2L+1][scale, shift, gate][W]
@@ -174,7 +188,9 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     suffix_mask_ = (int)ck.i64("suffix_mask", arch_ == Arch::SMOLVLA            ? VLA_MASK_CAUSAL_SUFFIX
                                               : (arch_ == Arch::PI0 && !adarms_) ? VLA_MASK_PI0_STATE
                                                                                  : VLA_MASK_NONE);
-    n_lead_ = (arch_ == Arch::SMOLVLA || adarms_) ? 0 : 1;
+    head_io_ = arch_ == Arch::GR00T && ck.i64("head_io", 0) != 0;
+    n_future_ = head_io_ ? (int)ck.i64("num_future") : 0;
+    n_lead_ = (arch_ == Arch::SMOLVLA || adarms_) ? 0 : 1 + n_future_;
     rope_ = arch_ != Arch::GR00T;
     dt_step_ = (arch_ == Arch::GR00T ? 1.0f : -1.0f) / (float)steps_;
     const int every = (int)ck.i64("self_attn_every_n", arch_ == Arch::PI0 ? 1 : 2);
@@ -207,19 +223,56 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     cfg.n_full = cfg.n_prefix + S_;
     if (!config_is_sane(cfg)) throw std::runtime_error("vla: real_* dims exceed max_* dims");
 
-    if (vocab_ > 0) E_lang_ = ck.f32("prefix.E_lang");
-    if (arch_ == Arch::SMOLVLA) {
-        Wstate_ = ck.f32("prefix.Wstate");
-        bstate_ = ck.f32("prefix.bstate");
-    } else if (n_lead_ > 0) {
-        W_sp_ = ck.f32("act.W_sp");
-        b_sp_ = ck.f32("act.b_sp");
+    if (S_ <= n_lead_) throw std::runtime_error("vla: n_suffix leaves no action rows");
+    const int64_t qd = (int64_t)Hq_ * D_, kvd = (int64_t)Hkv_ * D_;
+    if (vocab_ > 0) {
+        lang_rows_ = ck.row_source("prefix.E_lang");
+        if (lang_rows_) {
+            if (lang_rows_->rows != vocab_ || lang_rows_->cols != Wv_) throw std::runtime_error("vla: token embedding matrix does not match vocab x hidden");
+        } else {
+            E_lang_ = host_f32(ck, "prefix.E_lang", {vocab_, Wv_});
+        }
     }
-    W_in_ = load_f32(ck, "act.W_in");
-    W_out_ = load_f32(ck, "act.W_out");
-    b_out_ = load_f32(ck, "act.b_out");
-    if (arch_ != Arch::GR00T && !adarms_) final_norm_ = load_w(ck, "act.norm", dt_);
+    if (arch_ == Arch::SMOLVLA) {
+        Wstate_ = host_f32(ck, "prefix.Wstate", {Wv_, max_state_});
+        bstate_ = host_f32(ck, "prefix.bstate", {Wv_});
+    } else if (head_io_) {
+        O_ = (int)ck.i64("dit_out_dim");
+        Hd_ = (int)ck.i64("dec_hidden");
+        Hs_ = (int)ck.i64("state_hidden");
+        se_l1W_ = host_f32(ck, "aex.se_l1W", {Hs_, max_state_});
+        se_l1b_ = host_f32(ck, "aex.se_l1b", {Hs_});
+        se_l2W_ = host_f32(ck, "aex.se_l2W", {W_, Hs_});
+        se_l2b_ = host_f32(ck, "aex.se_l2b", {W_});
+        future_ = host_f32(ck, "aex.future_tokens", {n_future_, W_});
+    } else if (n_lead_ > 0) {
+        W_sp_ = host_f32(ck, "act.W_sp", {W_, max_state_});
+        b_sp_ = host_f32(ck, "act.b_sp", {W_});
+    }
+    if (head_io_) {
+        // decode's second projection plays the part of W_out in the Euler launch
+        W_out_ = load_f32(ck, "aex.ad_l2W", {A_, Hd_});
+        b_out_ = load_f32(ck, "aex.ad_l2b", {A_});
+        W3_ = load_f32(ck, "aex.ae_W3", {W_, W_});
+        b3_ = load_f32(ck, "aex.ae_b3", {W_});
+        const int Sa = S_ - n_lead_;
+        const CkptTensor& pe = ck.info("aex.pos_embd");
+        if (pe.shape.size() != 2 || pe.shape[1] != W_ || pe.shape[0] < Sa) throw std::runtime_error("vla: aex.pos_embd does not cover the action horizon");
+        std::vector<float> pos = ck.f32("aex.pos_embd");
+        pos.resize((size_t)Sa * W_);  // rows [0, horizon) (action_expert.cpp:50)
+        pos_.upload(pos.data(), pos.size() * sizeof(float));
+        po2W_ = load_w(ck, "aex.po2W", dt_, {O_, W_});
+        po2b_ = load_f32(ck, "aex.po2b", {O_});
+        ad1W_ = load_w(ck, "aex.ad_l1W", dt_, {Hd_, O_});
+        ad1b_ = load_f32(ck, "aex.ad_l1b", {Hd_});
+    } else {
+        W_in_ = load_f32(ck, "act.W_in", {W_, A_});
+        W_out_ = load_f32(ck, "act.W_out", {A_, W_});
+        b_out_ = load_f32(ck, "act.b_out", {A_});
+    }
+    if (arch_ != Arch::GR00T && !adarms_) final_norm_ = load_w(ck, "act.norm", dt_, {W_});
 
+    const bool no_norm_fusion = std::getenv("VLA_NO_NORM_FUSION") != nullptr;  // read once, at load
     layers_.resize(L_);
     for (int l = 0; l < L_; ++l) {
         LayerW& w = layers_[l];
@@ -229,49 +282,84 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         w.is_self = arch_ == Arch::PI0 ? true : arch_ == Arch::SMOLVLA ? (l % every == 0) : (interleave && l % 2 == 1);
         w.needs_prefix = !(arch_ == Arch::GR00T && w.is_self);
         w.from_text = alt_vl_ && w.needs_prefix && l % (2 * text_every_) == 0;
-        if (arch_ != Arch::GR00T && !adarms_) w.ln = load_w(ck, p + "ln", dt_);
-        w.Wqkv = load_w(ck, p + (w.is_self ? "Wqkv" : "Wq"), dt_);
-        if (arch_ != Arch::GR00T && !adarms_ && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
-            w.Wqkv_ln = load_folded_bf16(ck, p + (w.is_self ? "Wqkv" : "Wq"), p + "ln");
-        if (ck.has(p + (w.is_self ? "bqkv" : "bq"))) w.bqkv = load_f32(ck, p + (w.is_self ? "bqkv" : "bq"));
-        w.Wo = load_w(ck, p + "Wo", dt_);
-        if (ck.has(p + "bo")) w.bo = load_f32(ck, p + "bo");
+        const int64_t n_proj = w.is_self ? qd + 2 * kvd : qd;
+        if (arch_ != Arch::GR00T && !adarms_) w.ln = load_w(ck, p + "ln", dt_, {W_});
+        w.Wqkv = load_w(ck, p + (w.is_self ? "Wqkv" : "Wq"), dt_, {n_proj, W_});
+        if (arch_ != Arch::GR00T && !adarms_ && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !no_norm_fusion)
+            w.Wqkv_ln = load_folded_bf16(ck, p + (w.is_self ? "Wqkv" : "Wq"), p + "ln", n_proj, W_);
+        if (ck.has(p + (w.is_self ? "bqkv" : "bq"))) w.bqkv = load_f32(ck, p + (w.is_self ? "bqkv" : "bq"), {n_proj});
+        w.Wo = load_w(ck, p + "Wo", dt_, {W_, qd});
+        if (ck.has(p + "bo")) w.bo = load_f32(ck, p + "bo", {W_});
         if (I_ > 0 && arch_ == Arch::GR00T) {
-            w.W1 = load_w(ck, p + "W1", dt_);
-            w.b1 = load_f32(ck, p + "b1");
-            w.W2 = load_w(ck, p + "W2", dt_);
-            w.b2 = load_f32(ck, p + "b2");
+            w.W1 = load_w(ck, p + "W1", dt_, {I_, W_});
+            w.b1 = load_f32(ck, p + "b1", {I_});
+            w.W2 = load_w(ck, p + "W2", dt_, {W_, I_});
+            w.b2 = load_f32(ck, p + "b2", {W_});
         } else if (I_ > 0) {
-            if (!adarms_) w.ln2 = load_w(ck, p + "ln2", dt_);
-            w.Wgu = load_w(ck, p + "Wgu", dt_);
-            w.Wd = load_w(ck, p + "Wd", dt_);
-            if (!adarms_ && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !getenv("VLA_NO_NORM_FUSION"))
-                w.Wgu_ln = load_folded_bf16(ck, p + "Wgu", p + "ln2");
+            if (!adarms_) w.ln2 = load_w(ck, p + "ln2", dt_, {W_});
+            w.Wgu = load_w(ck, p + "Wgu", dt_, {2 * (int64_t)I_, W_});
+            w.Wd = load_w(ck, p + "Wd", dt_, {W_, I_});
+            if (!adarms_ && dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !no_norm_fusion)
+                w.Wgu_ln = load_folded_bf16(ck, p + "Wgu", p + "ln2", 2 * (int64_t)I_, W_);
         }
         if (w.needs_prefix) {
             const std::string v = "vlm." + std::to_string(l) + ".";
-            if (arch_ != Arch::GR00T) w.vlm_ln = load_w(ck, v + "ln", dt_);
-            w.Wkv_pre = load_w(ck, v + "Wkv", dt_);
-            if (ck.has(v + "bkv")) w.bkv_pre = load_f32(ck, v + "bkv");
+            if (arch_ != Arch::GR00T) w.vlm_ln = load_w(ck, v + "ln", dt_, {Wv_});
+            w.Wkv_pre = load_w(ck, v + "Wkv", dt_, {2 * kvd, Wv_});
+            if (ck.has(v + "bkv")) w.bkv_pre = load_f32(ck, v + "bkv", {2 * kvd});
         }
         if (arch_ == Arch::SMOLVLA && !w.is_self) {
-            w.Wk_x = load_w(ck, p + "Wk_x", dt_);
-            w.Wv_x = load_w(ck, p + "Wv_x", dt_);
+            w.Wk_x = load_w(ck, p + "Wk_x", dt_, {kvd, kvd});
+            w.Wv_x = load_w(ck, p + "Wv_x", dt_, {kvd, kvd});
         }
     }
 
     // Per-step constants.  The time conditioning depends on the step index only,
     // so it is evaluated once here instead of inside every denoise step.
-    const std::vector<float> b_in = ck.f32("act.b_in");
     std::vector<float> bias((size_t)steps_ * W_);
     time_mlp_ = arch_ != Arch::GR00T && !adarms_ && ck.has("act.W_at1");
-    if (time_mlp_) {
+    if (head_io_) {
+        // encode_action (action_expert.cpp:46-52): a = W1 x + b1; m = silu(W2 [a ; tau] + b2);
+        // out = W3 m + b3 + pos.  W2 = [W2a | W2t] by columns, tau depends on the step only, so
+        // m = silu((W2a W1) x + (W2a b1 + W2t tau_s + b2)): one [W][A] matrix and a per-step bias.
+        const std::vector<float> W1 = host_f32(ck, "aex.ae_W1", {W_, A_}), b1 = host_f32(ck, "aex.ae_b1", {W_}),
+                                 W2 = host_f32(ck, "aex.ae_W2", {W_, 2 * (int64_t)W_}), b2 = host_f32(ck, "aex.ae_b2", {W_});
+        std::vector<float> Wf((size_t)W_ * A_);
+        for (int r = 0; r < W_; ++r)
+            for (int a = 0; a < A_; ++a) {
+                double acc = 0.0;
+                for (int k = 0; k < W_; ++k) acc += (double)W2[(size_t)r * 2 * W_ + k] * (double)W1[(size_t)k * A_ + a];
+                Wf[(size_t)r * A_ + a] = (float)acc;
+            }
+        W_in_.upload(Wf.data(), Wf.size() * sizeof(float));
+        const int64_t n_buckets = ck.i64("num_buckets", 1000);
+        for (int s = 0; s < steps_; ++s) {
+            // action_sinusoid(bucket, E, ...): sin first, then cos, the same row for every token (embed.h:47-59)
+            const int64_t bucket = (int64_t)((double)s / (double)steps_ * (double)n_buckets);
+            const int half = W_ / 2;
+            const float stp = std::log(10000.0f) / (float)half, tb = (float)bucket;
+            std::vector<float> tau(W_, 0.f);
+            for (int i = 0; i < half; ++i) {
+                const float e = tb * std::exp(-(float)i * stp);
+                tau[i] = std::sin(e);
+                tau[half + i] = std::cos(e);
+            }
+            for (int r = 0; r < W_; ++r) {
+                double acc = (double)b2[r];
+                for (int k = 0; k < W_; ++k)
+                    acc += (double)W2[(size_t)r * 2 * W_ + k] * (double)b1[k] + (double)W2[(size_t)r * 2 * W_ + W_ + k] * (double)tau[k];
+                bias[(size_t)s * W_ + r] = (float)acc;
+            }
+        }
+    } else if (time_mlp_) {
+        const std::vector<float> b_in = host_f32(ck, "act.b_in", {W_});
         // Action-time MLP (src/models/smolvla.cpp:1397-1403, src/models/pi0.cpp:240-244):
         //   mlp1 = W_at1 . concat(W_in x + b_in, time_s) + b_at1,  suffix = W_at2 silu(mlp1) + b_at2.
         // W_at1 = [Wa | Wt] by columns, so mlp1 = (Wa W_in) x + (Wa b_in + Wt time_s + b_at1):
         // the first two projections collapse into one [W][A] matrix and a per-step bias,
         // both formed here once (double accumulation), and the embed kernel applies the silu.
-        const std::vector<float> W_in = ck.f32("act.W_in"), W_at1 = ck.f32("act.W_at1"), b_at1 = ck.f32("act.b_at1");
+        const std::vector<float> W_in = ck.f32("act.W_in"), W_at1 = host_f32(ck, "act.W_at1", {W_, 2 * (int64_t)W_}),
+                                 b_at1 = host_f32(ck, "act.b_at1", {W_});
         std::vector<float> Wf((size_t)W_ * A_);
         for (int r = 0; r < W_; ++r)
             for (int a = 0; a < A_; ++a) {
@@ -291,9 +379,10 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
                 bias[(size_t)s * W_ + r] = (float)acc;
             }
         }
-        W_at2_ = load_f32(ck, "act.W_at2");
-        b_at2_ = load_f32(ck, "act.b_at2");
+        W_at2_ = load_f32(ck, "act.W_at2", {W_, W_});
+        b_at2_ = load_f32(ck, "act.b_at2", {W_});
     } else {
+        const std::vector<float> b_in = host_f32(ck, "act.b_in", {W_});
         for (int s = 0; s < steps_; ++s) {
             for (int c = 0; c < W_; ++c) bias[(size_t)s * W_ + c] = b_in[c];
             if (arch_ != Arch::GR00T && !adarms_) {
@@ -310,21 +399,21 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         // cond_s = silu(W_tout silu(W_tin time_s + b_tin) + b_tout) (src/models/pi05.cpp:619-620);
         // (scale, shift, gate) of a norm site = dense_w . cond + dense_b (build_adarms,
         // pi05.cpp:212-215).  Sites per step: 2 per layer (attention, FFN), then the final norm.
-        const std::vector<float> Wt1 = ck.f32("te.W_tin"), bt1 = ck.f32("te.b_tin"), Wt2 = ck.f32("te.W_tout"),
-                                 bt2 = ck.f32("te.b_tout");
+        const std::vector<float> Wt1 = host_f32(ck, "te.W_tin", {W_, W_}), bt1 = host_f32(ck, "te.b_tin", {W_}),
+                                 Wt2 = host_f32(ck, "te.W_tout", {W_, W_}), bt2 = host_f32(ck, "te.b_tout", {W_});
         const int sites = 2 * L_ + 1;
         std::vector<std::vector<float>> dw(sites), db(sites);
         for (int l = 0; l < L_; ++l) {
             const std::string p = "ex." + std::to_string(l) + ".";
-            dw[2 * l] = ck.f32(p + "ada_in_w");
-            db[2 * l] = ck.f32(p + "ada_in_b");
+            dw[2 * l] = host_f32(ck, p + "ada_in_w", {3 * (int64_t)W_, W_});
+            db[2 * l] = host_f32(ck, p + "ada_in_b", {3 * (int64_t)W_});
             if (I_ > 0) {
-                dw[2 * l + 1] = ck.f32(p + "ada_post_w");
-                db[2 * l + 1] = ck.f32(p + "ada_post_b");
+                dw[2 * l + 1] = host_f32(ck, p + "ada_post_w", {3 * (int64_t)W_, W_});
+                db[2 * l + 1] = host_f32(ck, p + "ada_post_b", {3 * (int64_t)W_});
             }
         }
-        dw[2 * L_] = ck.f32("act.ada_final_w");
-        db[2 * L_] = ck.f32("act.ada_final_b");
+        dw[2 * L_] = host_f32(ck, "act.ada_final_w", {3 * (int64_t)W_, W_});
+        db[2 * L_] = host_f32(ck, "act.ada_final_b", {3 * (int64_t)W_});
         std::vector<float> mod((size_t)steps_ * sites * 3 * W_);
         std::vector<float> c1(W_), cond(W_);
         for (int s = 0; s < steps_; ++s) {
@@ -344,17 +433,25 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         // temb = l2(silu(l1(timesteps_proj(bucket)))) (DitHead::time_emb,
         // src/modules/dit_head.cpp:135-137); per layer (scale, shift) =
         // adaln_w . silu(temb) + adaln_b (src/layers/norm.h:39-41).
-        const std::vector<float> l1W = ck.f32("te.l1W"), l1b = ck.f32("te.l1b"), l2W = ck.f32("te.l2W"),
-                                 l2b = ck.f32("te.l2b");
-        std::vector<float> ada((size_t)steps_ * (L_ + 1) * 2 * W_, 0.f);
+        const std::vector<float> l1W = host_f32(ck, "te.l1W", {W_, 256}), l1b = host_f32(ck, "te.l1b", {W_}),
+                                 l2W = host_f32(ck, "te.l2W", {W_, W_}), l2b = host_f32(ck, "te.l2b", {W_});
+        // per step: L layer slots (scale, shift), slot L = zeros (a plain LayerNorm), slot L + 1 =
+        // the output modulation of DitHead::proj_out when the head's own MLPs are present
+        std::vector<float> ada((size_t)steps_ * (L_ + 2) * 2 * W_, 0.f);
         std::vector<std::vector<float>> aw(L_), ab(L_);
         for (int l = 0; l < L_; ++l) {
-            aw[l] = ck.f32("ex." + std::to_string(l) + ".adaln_w");
-            ab[l] = ck.f32("ex." + std::to_string(l) + ".adaln_b");
+            aw[l] = host_f32(ck, "ex." + std::to_string(l) + ".adaln_w", {2 * (int64_t)W_, W_});
+            ab[l] = host_f32(ck, "ex." + std::to_string(l) + ".adaln_b", {2 * (int64_t)W_});
         }
+        std::vector<float> po1W, po1b;
+        if (head_io_) {
+            po1W = host_f32(ck, "aex.po1W", {2 * (int64_t)W_, W_});
+            po1b = host_f32(ck, "aex.po1b", {2 * (int64_t)W_});
+        }
+        const int64_t n_buckets = ck.i64("num_buckets", 1000);
         for (int s = 0; s < steps_; ++s) {
             std::vector<float> tp, t1(W_), temb(W_), st(W_);
-            timesteps_proj((int64_t)((double)s / (double)steps_ * 1000.0), tp);
+            timesteps_proj((int64_t)((double)s / (double)steps_ * (double)n_buckets), tp);
             host_linear(l1W.data(), l1b.data(), tp.data(), t1.data(), W_, 256);
             for (auto& v : t1) v = host_silu(v);
             host_linear(l2W.data(), l2b.data(), t1.data(), temb.data(), W_, W_);
@@ -365,9 +462,18 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
                 pool.emplace_back([&, t]() {
                     for (int l = t; l < L_; l += nthr)
                         host_linear(aw[l].data(), ab[l].data(), st.data(),
-                                    ada.data() + ((size_t)s * (L_ + 1) + l) * 2 * W_, 2 * W_, W_);
+                                    ada.data() + ((size_t)s * (L_ + 2) + l) * 2 * W_, 2 * W_, W_);
                 });
             for (auto& th : pool) th.join();
+            if (head_io_) {
+                // proj_out's dense gives (shift, scale) in that order (dit_head.cpp:140-142, norm.h:36);
+                // the norm launch takes (scale, shift)
+                std::vector<float> po(2 * (size_t)W_);
+                host_linear(po1W.data(), po1b.data(), st.data(), po.data(), 2 * W_, W_);
+                float* slot = ada.data() + ((size_t)s * (L_ + 2) + L_ + 1) * 2 * W_;
+                std::copy(po.begin() + W_, po.end(), slot);
+                std::copy(po.begin(), po.begin() + W_, slot + W_);
+            }
         }
         ada_.upload(ada.data(), ada.size() * sizeof(float));
     }
@@ -406,7 +512,12 @@ void FlowExpert::allocate(int B, int P, int P_txt) {
     q_.alloc((size_t)B * S_ * Hq_ * D_ * es);
     att_.alloc((size_t)B * S_ * Hq_ * D_ * es);
     if (I_ > 0) mid_.alloc((size_t)B * S_ * I_ * es);
-    if (time_mlp_) m1_.alloc((size_t)B * S_ * W_ * sizeof(float));
+    if (time_mlp_ || head_io_) m1_.alloc((size_t)B * S_ * W_ * sizeof(float));
+    if (head_io_) {
+        m2_.alloc((size_t)B * S_ * W_ * sizeof(float));
+        d1_.alloc((size_t)B * S_ * O_ * es);
+        d2_.alloc((size_t)B * S_ * Hd_ * es);
+    }
 }
 
 void FlowExpert::prefill(const Inputs* in, int batch) {
@@ -451,9 +562,16 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
         if (arch_ != Arch::GR00T || alt_vl_) {
             const int rows = arch_ == Arch::SMOLVLA ? n_lang_max_ : n_lang;
             const float ls = alt_vl_ ? 1.0f : lang_scale;  // N1.6: the rows stand for backbone features, unscaled
+            std::vector<float> fetched;
+            if (lang_rows_) {  // the rows this observation needs, read from the file
+                std::vector<int32_t> ids((size_t)rows, 0);
+                for (int i = 0; i < n_lang; ++i) ids[i] = in[b].lang_tokens[i];
+                fetched.resize((size_t)rows * Wv_);
+                if (rows > 0 && !lang_rows_->fetch(ids, fetched.data())) throw std::runtime_error("vla: cannot read token embedding rows");
+            }
             for (int i = 0; i < rows; ++i) {
                 const int tok = i < n_lang ? in[b].lang_tokens[i] : 0;  // zero-padded ids, smolvla.cpp:1628-1629
-                const float* e = E_lang_.data() + (size_t)tok * Wv_;
+                const float* e = lang_rows_ ? fetched.data() + (size_t)i * Wv_ : E_lang_.data() + (size_t)tok * Wv_;
                 float* row = txt_dst + (size_t)i * Wv_;
                 for (int c = 0; c < Wv_; ++c) row[c] = e[c] * ls;
             }
@@ -462,6 +580,14 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
         if (in[b].state) std::copy(in[b].state, in[b].state + max_state_, st.begin());
         if (arch_ == Arch::SMOLVLA) {
             host_linear(Wstate_.data(), bstate_.data(), st.data(), dst + (size_t)(P - 1) * Wv_, Wv_, max_state_);
+        } else if (head_io_) {
+            // encode_state (relu between the two projections), then the learned future tokens
+            std::vector<float> h1(Hs_), ld((size_t)n_lead_ * W_);
+            host_linear(se_l1W_.data(), se_l1b_.data(), st.data(), h1.data(), Hs_, max_state_);
+            for (float& v : h1) v = v > 0.f ? v : 0.f;
+            host_linear(se_l2W_.data(), se_l2b_.data(), h1.data(), ld.data(), W_, Hs_);
+            std::copy(future_.begin(), future_.end(), ld.begin() + W_);
+            VLA_HIP(hipMemcpy(lead_.as<float>() + (size_t)b * n_lead_ * W_, ld.data(), ld.size() * sizeof(float), hipMemcpyHostToDevice));
         } else if (n_lead_ > 0) {
             std::vector<float> ld(W_);
             host_linear(W_sp_.data(), b_sp_.data(), st.data(), ld.data(), W_, max_state_);
@@ -571,7 +697,14 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
             prof_mark("stage_noise");
         }
         {
-            if (time_mlp_) {
+            if (head_io_) {
+                VLA_K(vla_embed_suffix_act(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
+                                           lead_.as<float>(), m1_.get(), VLA_DT_F32, B, S_, n_lead_, A_, W_, VLA_ACT_SILU, C.stream));
+                VLA_K(vla_linear(m1_.get(), W3_.get(), b3_.as<float>(), nullptr, m2_.get(), VLA_DT_F32, VLA_DT_F32, M, W_, W_,
+                                 C.stream));
+                VLA_K(vla_finish_suffix_rows(m2_.as<float>(), pos_.as<float>(), lead_.as<float>(), h.data, dt_, B, S_, n_lead_, W_,
+                                             C.stream));
+            } else if (time_mlp_) {
                 VLA_K(vla_embed_suffix_act(xt_.as<float>(), W_in_.as<float>(), bias_step_.as<float>() + (size_t)s * W_,
                                            n_lead_ ? lead_.as<float>() : nullptr, m1_.get(), VLA_DT_F32, B, S_, n_lead_, A_, W_,
                                            VLA_ACT_SILU, C.stream));
@@ -607,7 +740,7 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 }
                 if (!done) {
                     if (arch_ == Arch::GR00T) {
-                        const float* sc = ada_.as<float>() + ((size_t)s * (L_ + 1) + l) * 2 * W_;
+                        const float* sc = ada_.as<float>() + ((size_t)s * (L_ + 2) + l) * 2 * W_;
                         adaln(C, h, sc, sc + W_, eps_, hn);
                     } else {
                         rms_norm(C, h, w.ln.get(), eps_, hn);
@@ -649,7 +782,7 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                     // FFN half (smolvla.cpp:845-848, pi0.cpp:227-232, dit_head.cpp:132-133)
                     Tensor mid = tensor_2d(mid_.get(), dt_, I_, M);
                     if (arch_ == Arch::GR00T) {
-                        const float* z = ada_.as<float>() + ((size_t)s * (L_ + 1) + L_) * 2 * W_;  // zeros: plain LayerNorm
+                        const float* z = ada_.as<float>() + ((size_t)s * (L_ + 2) + L_) * 2 * W_;  // zeros: plain LayerNorm
                         adaln(C, h, z, z + W_, eps_, hn);
                         prof_mark("ffn_norm");
                         Tensor W1 = tensor_2d(w.W1.get(), dt_, W_, I_), W2 = tensor_2d(w.W2.get(), dt_, I_, W_);
@@ -675,8 +808,21 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
             if (adarms_) {
                 const float* mf = ada_.as<float>() + ((size_t)s * (2 * L_ + 1) + 2 * L_) * 3 * W_;  // gate unused (pi05.cpp:628)
                 VLA_K(vla_adarms(h.data, mf, mf + W_, hn.data, dt_, M, W_, eps_, C.stream));
+            } else if (head_io_) {
+                // DitHead::proj_out then ActionExpert::decode; its last projection is the Euler launch's
+                const float* po = ada_.as<float>() + ((size_t)s * (L_ + 2) + L_ + 1) * 2 * W_;
+                adaln(C, h, po, po + W_, final_eps_, hn);
+                prof_mark("final_norm");
+                VLA_K(vla_linear(hn.data, po2W_.get(), po2b_.as<float>(), nullptr, d1_.get(), dt_, dt_, M, O_, W_, C.stream));
+                VLA_K(vla_linear_act(d1_.get(), ad1W_.get(), ad1b_.as<float>(), nullptr, d2_.get(), dt_, dt_, M, Hd_, O_, VLA_ACT_RELU,
+                                     C.stream));
+                prof_mark("head_decode");
+                VLA_K(vla_euler_step(xt_.as<float>(), d2_.get(), W_out_.as<float>(), b_out_.as<float>(), dt_, B, S_, n_lead_, A_, Hd_,
+                                     dt_step_, C.stream));
+                prof_mark("euler_step");
+                continue;
             } else if (arch_ == Arch::GR00T) {
-                const float* z = ada_.as<float>() + ((size_t)s * (L_ + 1) + L_) * 2 * W_;  // zeros: plain LayerNorm
+                const float* z = ada_.as<float>() + ((size_t)s * (L_ + 2) + L_) * 2 * W_;  // zeros: plain LayerNorm
                 adaln(C, h, z, z + W_, final_eps_, hn);
             } else {
                 rms_norm(C, h, final_norm_.get(), eps_, hn);

@@ -11,6 +11,7 @@
 // MLPs around it) are read; vision tower, connector and backbone FFN tensors are ignored.
 // Also here: the C ABI over the reader itself (include/vla_gguf.h).
 #include <cstdlib>
+#include <functional>
 #include <memory>
 #include <stdexcept>
 
@@ -32,6 +33,43 @@ bool is_gguf_file(const std::string& path) {
 
 namespace {
 
+// Names of the gguf tensors an import read (or left on disk for row fetches), in order: what
+// vla_gguf_import_trace reports, so that the name map can be checked against name lists kept
+// as data (the reference's converter tests hold them, tests/py/test_converters.py).
+thread_local std::vector<std::string>* g_trace = nullptr;
+void trace(const std::string& name) {
+    if (g_trace) g_trace->push_back(name);
+}
+
+// Token embeddings read per request from the file (RowSource); owns its own reader.
+struct GgufRows : RowSource {
+    gguf_reader r{"gguf"};
+    std::string name;
+    bool fetch(const std::vector<int32_t>& ids, float* dst) override { return r.fetch_rows_f32(name.c_str(), ids, dst, cols); }
+};
+
+// prefix.E_lang from `name`: resident when small, left on disk when the matrix is large
+// (VLA_EMBED_ON_DEMAND=1 / 0 forces either; read at load).  The reference fetches the rows
+// of every request from the file (fetch_rows_f32, src/models/pi0.cpp:530-534).
+void put_token_embeddings(const std::string& path, gguf_reader& g, Checkpoint& ck, const std::string& name, int64_t vocab,
+                          int64_t hidden, const std::function<std::vector<float>()>& whole) {
+    const char* e = std::getenv("VLA_EMBED_ON_DEMAND");
+    const bool lazy = e ? std::atoi(e) != 0 : vocab * hidden * 4 > ((int64_t)256 << 20);
+    if (!lazy) {
+        ck.add_f32("prefix.E_lang", {vocab, hidden}, whole());
+        return;
+    }
+    const gguf_tensor_meta* t = g.meta(name.c_str());
+    if (!t || t->ne[0] != hidden || t->ne[1] != vocab) throw std::runtime_error("vla: gguf tensor " + name + " is not [vocab x hidden]");
+    auto rows = std::make_shared<GgufRows>();
+    if (!rows->r.open(path)) throw std::runtime_error("vla: cannot reopen " + path + " for row fetches");
+    rows->name = name;
+    rows->rows = vocab;
+    rows->cols = hidden;
+    trace(name);
+    ck.set_row_source("prefix.E_lang", rows);
+}
+
 struct Importer {
     gguf_reader& g;
     Checkpoint& ck;
@@ -47,7 +85,34 @@ struct Importer {
                                      "], expected [" + std::to_string(rows) + " x " + std::to_string(cols) + "]");
         std::vector<float> v = g.read_f32(name.c_str());
         if (v.empty()) throw std::runtime_error("vla: cannot read gguf tensor " + name);
+        trace(name);
         return v;
+    }
+    // Row `id` of a cat_linear weight (src/layers/linear.h:30-37): ggml [out, in, n] holds one
+    // [in][out] matrix per embodiment; returned transposed, [out][in], as every projection here
+    // stores its weight.  The bias [out, n] gives row `id`.
+    std::vector<float> cat_w(const std::string& name, int64_t id, int64_t out, int64_t in) {
+        const gguf_tensor_meta* t = g.meta(name.c_str());
+        if (!t) throw std::runtime_error("vla: gguf has no tensor " + name);
+        if (t->ne[0] != out || t->ne[1] != in || id < 0 || id >= t->ne[2])
+            throw std::runtime_error("vla: gguf tensor " + name + " is not [n][" + std::to_string(in) + "][" + std::to_string(out) +
+                                     "] with embodiment " + std::to_string(id));
+        const std::vector<float> all = g.read_f32(name.c_str());
+        if (all.empty()) throw std::runtime_error("vla: cannot read gguf tensor " + name);
+        trace(name);
+        std::vector<float> w((size_t)out * in);
+        const float* src = all.data() + (size_t)id * in * out;
+        for (int64_t i = 0; i < in; ++i)
+            for (int64_t o = 0; o < out; ++o) w[(size_t)o * in + i] = src[(size_t)i * out + o];
+        return w;
+    }
+    std::vector<float> cat_b(const std::string& name, int64_t id, int64_t out) {
+        const gguf_tensor_meta* t = g.meta(name.c_str());
+        if (!t || t->ne[0] != out || id < 0 || id >= t->ne[1]) throw std::runtime_error("vla: gguf tensor " + name + " is missing or misshapen");
+        const std::vector<float> all = g.read_f32(name.c_str());
+        if (all.empty()) throw std::runtime_error("vla: cannot read gguf tensor " + name);
+        trace(name);
+        return std::vector<float>(all.begin() + id * out, all.begin() + (id + 1) * out);
     }
     std::vector<float> vec(const std::string& name, int64_t n) { return mat(name, 1, n); }
 
@@ -90,7 +155,7 @@ uint32_t need_u32(const gguf_reader& g, const char* k) {
 //   pi0.5:   keys src/models/pi05.cpp:292-328, tensors 459-485: the expert's norm slots hold
 //            the adaRMS modulation dense ([3 expert_h, expert_h] weight and [3 expert_h]
 //            bias), the time MLP replaces the action-time MLP, there is no state projection.
-void import_flow(gguf_reader& g, Checkpoint& ck, bool bf16, const std::string& arch) {
+void import_flow(const std::string& path, gguf_reader& g, Checkpoint& ck, bool bf16, const std::string& arch) {
     const bool smol = arch == "smolvla", pi05 = arch == "pi05", gemma = !smol;
     const std::string kp = arch + ".";
     auto key = [&](const char* k) { return kp + k; };
@@ -139,7 +204,7 @@ void import_flow(gguf_reader& g, Checkpoint& ck, bool bf16, const std::string& a
             for (float& x : v) x += 1.0f;
         return v;
     };
-    ck.add_f32("prefix.E_lang", {vocab, hidden}, im.mat("token_embd.weight", vocab, hidden));
+    put_token_embeddings(path, g, ck, "token_embd.weight", vocab, hidden, [&]() { return im.mat("token_embd.weight", vocab, hidden); });
     if (smol) {
         ck.add_f32("prefix.Wstate", {hidden, sd}, im.mat("state_proj.weight", hidden, sd));
         ck.add_f32("prefix.bstate", {hidden}, im.vec("state_proj.bias", hidden));
@@ -200,7 +265,133 @@ void import_flow(gguf_reader& g, Checkpoint& ck, bool bf16, const std::string& a
 // (728-747).  The action-token embeddings and the output projection this library's
 // token-by-token schedule uses have no counterpart in the reference's file; they are read
 // under this library's own names (act.emb, act.W_out, act.b_out) and must be present.
-void import_bitvla(gguf_reader& g, Checkpoint& ck) {
+// GR00T N1.5 action head: keys of load_config (src/models/gr00tn1d5.cpp:92-147), DiT tensors of
+// DitHead::declare (src/modules/dit_head.cpp:29-85; GGUF names "aex.dit.N.{adaln, attn_q,
+// attn_k, attn_v, attn_o, ff0, ff2}.{weight, bias}", the list the reference's converter test
+// holds, tests/py/test_converters.py:178-184), the head's own MLPs of ActionExpert::declare
+// (src/modules/action_expert.cpp:20-39) with the embodiment's row selected here (id 24 unless
+// VLA_GR00T_EMBODIMENT gives a number or a tag of gr00t_n1_5.embodiment_tag_mapping,
+// gr00tn1d5.cpp:149-167), "aex.future_tokens" and "aex.pos_embd".  Cross layers (even, or all
+// without dit_interleave) take K / V from the backbone features ([inner, backbone_embedding_dim]),
+// self layers fuse [q; k; v].  The backbone (vision tower, Qwen3 layers, VL self-attention) is
+// not read: precomputed_img_emb stands for its output rows.
+void import_gr00t(gguf_reader& g, Checkpoint& ck, bool bf16) {
+    auto key = [](const char* k) { return std::string("gr00t_n1_5.") + k; };
+    auto u = [&](const char* k) { return (int64_t)need_u32(g, key(k).c_str()); };
+    auto u_or = [&](const char* k, int64_t d) { return g.has(key(k).c_str()) ? (int64_t)g.u32(key(k).c_str()) : d; };
+    auto f_or = [&](const char* k, double d) { return g.has(key(k).c_str()) ? (double)g.f32(key(k).c_str()) : d; };
+    const int64_t Wv = u_or("backbone_embedding_dim", 2048), E = u_or("input_embedding_dim", 1536), W = u("dit_hidden"),
+                  H = u("dit_heads"), D = u("dit_head_dim"), L = u("dit_layers"), interleave = u_or("dit_interleave", 1),
+                  NF = u_or("num_target_vision_tokens", 32), AH = u_or("action_horizon", 16), A = u_or("action_dim", 32),
+                  sd = u_or("max_state_dim", 64), steps = u_or("num_inference_timesteps", 4),
+                  buckets = u_or("num_timestep_buckets", 1000), n_emb = u_or("max_num_embodiments", 32);
+    if (H < 1 || D < 1 || H * D != W || E != W || L < 1) throw std::runtime_error("vla: gr00t gguf geometry is not usable (heads x head_dim, embedding and DiT widths must agree)");
+    int64_t id = 24;
+    if (const char* e = std::getenv("VLA_GR00T_EMBODIMENT")) {
+        char* end = nullptr;
+        const long v = std::strtol(e, &end, 10);
+        if (end && *end == '\0' && end != e) {
+            id = v;
+        } else {
+            const std::string js = g.str(key("embodiment_tag_mapping").c_str()), k2 = std::string("\"") + e + "\":";
+            const size_t p = js.find(k2);
+            if (p == std::string::npos) throw std::runtime_error(std::string("vla: embodiment tag '") + e + "' is not in embodiment_tag_mapping");
+            id = std::strtol(js.c_str() + p + k2.size(), nullptr, 10);
+        }
+    }
+    if (id < 0 || id >= n_emb) throw std::runtime_error("vla: embodiment id out of range");
+    Importer im{g, ck, bf16};
+    const gguf_tensor_meta* ff0 = g.meta("aex.dit.0.ff0.weight");
+    const gguf_tensor_meta* po2 = g.meta("aex.dit.proj_out2.weight");
+    const gguf_tensor_meta* se1 = g.meta("aex.state_enc.l1.W");
+    const gguf_tensor_meta* ad1 = g.meta("aex.act_dec.l1.W");
+    const gguf_tensor_meta* pe = g.meta("aex.pos_embd");
+    if (!ff0 || !po2 || !se1 || !ad1 || !pe) throw std::runtime_error("vla: gr00t gguf lacks the DiT head tensors (ff0, proj_out2, state_enc, act_dec, pos_embd)");
+    const int64_t I = ff0->ne[1], O = po2->ne[1], Hs = se1->ne[0], Hd = ad1->ne[0], max_pos = pe->ne[1];
+    ck.set_key("arch", "gr00t_n1d5");
+    ck.set_key("dtype", bf16 ? "bf16" : "f32");
+    ck.set_key("n_layers", L);
+    ck.set_key("n_q_heads", H);
+    ck.set_key("n_kv_heads", H);
+    ck.set_key("head_dim", D);
+    ck.set_key("hidden", Wv);
+    ck.set_key("expert_h", W);
+    ck.set_key("ffn_dim", I);
+    ck.set_key("n_img", u_or("n_img_tokens", 256));
+    ck.set_key("n_lang", (int64_t)0);
+    ck.set_key("vocab", (int64_t)0);
+    ck.set_key("n_suffix", 1 + NF + AH);
+    ck.set_key("max_action_dim", A);
+    ck.set_key("max_state_dim", sd);
+    ck.set_key("real_action_dim", A);
+    ck.set_key("real_state_dim", sd);
+    ck.set_key("num_steps", steps);
+    ck.set_key("rms_eps", f_or("ln_eps", 1e-5));
+    ck.set_key("norm_out_eps", f_or("norm_out_eps", 1e-6));
+    ck.set_key("dit_interleave", interleave);
+    ck.set_key("head_io", (int64_t)1);
+    ck.set_key("num_future", NF);
+    ck.set_key("dit_out_dim", O);
+    ck.set_key("dec_hidden", Hd);
+    ck.set_key("state_hidden", Hs);
+    ck.set_key("num_buckets", buckets);
+
+    ck.add_f32("te.l1W", {W, 256}, im.mat("aex.dit.time_emb.l1.weight", W, 256));
+    ck.add_f32("te.l1b", {W}, im.vec("aex.dit.time_emb.l1.bias", W));
+    ck.add_f32("te.l2W", {W, W}, im.mat("aex.dit.time_emb.l2.weight", W, W));
+    ck.add_f32("te.l2b", {W}, im.vec("aex.dit.time_emb.l2.bias", W));
+    ck.add_f32("aex.po1W", {2 * W, W}, im.mat("aex.dit.proj_out1.weight", 2 * W, W));
+    ck.add_f32("aex.po1b", {2 * W}, im.vec("aex.dit.proj_out1.bias", 2 * W));
+    im.put_weight("aex.po2W", O, W, im.mat("aex.dit.proj_out2.weight", O, W));
+    ck.add_f32("aex.po2b", {O}, im.vec("aex.dit.proj_out2.bias", O));
+    ck.add_f32("aex.se_l1W", {Hs, sd}, im.cat_w("aex.state_enc.l1.W", id, Hs, sd));
+    ck.add_f32("aex.se_l1b", {Hs}, im.cat_b("aex.state_enc.l1.b", id, Hs));
+    ck.add_f32("aex.se_l2W", {W, Hs}, im.cat_w("aex.state_enc.l2.W", id, W, Hs));
+    ck.add_f32("aex.se_l2b", {W}, im.cat_b("aex.state_enc.l2.b", id, W));
+    ck.add_f32("aex.ae_W1", {W, A}, im.cat_w("aex.act_enc.W1.W", id, W, A));
+    ck.add_f32("aex.ae_b1", {W}, im.cat_b("aex.act_enc.W1.b", id, W));
+    ck.add_f32("aex.ae_W2", {W, 2 * W}, im.cat_w("aex.act_enc.W2.W", id, W, 2 * W));
+    ck.add_f32("aex.ae_b2", {W}, im.cat_b("aex.act_enc.W2.b", id, W));
+    ck.add_f32("aex.ae_W3", {W, W}, im.cat_w("aex.act_enc.W3.W", id, W, W));
+    ck.add_f32("aex.ae_b3", {W}, im.cat_b("aex.act_enc.W3.b", id, W));
+    im.put_weight("aex.ad_l1W", Hd, O, im.cat_w("aex.act_dec.l1.W", id, Hd, O));
+    ck.add_f32("aex.ad_l1b", {Hd}, im.cat_b("aex.act_dec.l1.b", id, Hd));
+    ck.add_f32("aex.ad_l2W", {A, Hd}, im.cat_w("aex.act_dec.l2.W", id, A, Hd));
+    ck.add_f32("aex.ad_l2b", {A}, im.cat_b("aex.act_dec.l2.b", id, A));
+    ck.add_f32("aex.pos_embd", {max_pos, W}, im.mat("aex.pos_embd", max_pos, W));
+    ck.add_f32("aex.future_tokens", {NF, W}, im.mat("aex.future_tokens", NF, W));
+    for (int64_t l = 0; l < L; ++l) {
+        const std::string a = "aex.dit." + std::to_string(l) + ".", e = "ex." + std::to_string(l) + ".", p = "vlm." + std::to_string(l) + ".";
+        const bool self = interleave != 0 && l % 2 == 1;
+        ck.add_f32(e + "adaln_w", {2 * W, W}, im.mat(a + "adaln.weight", 2 * W, W));
+        ck.add_f32(e + "adaln_b", {2 * W}, im.vec(a + "adaln.bias", 2 * W));
+        auto cat3 = [&](const std::vector<std::string>& names, int64_t n) {
+            std::vector<float> all;
+            for (const std::string& nm : names) {
+                const std::vector<float> v = im.vec(nm, n);
+                all.insert(all.end(), v.begin(), v.end());
+            }
+            return all;
+        };
+        if (self) {
+            im.put_stacked(e + "Wqkv", {a + "attn_q.weight", a + "attn_k.weight", a + "attn_v.weight"}, {W, W, W}, W);
+            ck.add_f32(e + "bqkv", {3 * W}, cat3({a + "attn_q.bias", a + "attn_k.bias", a + "attn_v.bias"}, W));
+        } else {
+            im.put_weight(e + "Wq", W, W, im.mat(a + "attn_q.weight", W, W));
+            ck.add_f32(e + "bq", {W}, im.vec(a + "attn_q.bias", W));
+            im.put_stacked(p + "Wkv", {a + "attn_k.weight", a + "attn_v.weight"}, {W, W}, Wv);
+            ck.add_f32(p + "bkv", {2 * W}, cat3({a + "attn_k.bias", a + "attn_v.bias"}, W));
+        }
+        im.put_weight(e + "Wo", W, W, im.mat(a + "attn_o.weight", W, W));
+        ck.add_f32(e + "bo", {W}, im.vec(a + "attn_o.bias", W));
+        im.put_weight(e + "W1", I, W, im.mat(a + "ff0.weight", I, W));
+        ck.add_f32(e + "b1", {I}, im.vec(a + "ff0.bias", I));
+        im.put_weight(e + "W2", W, I, im.mat(a + "ff2.weight", W, I));
+        ck.add_f32(e + "b2", {W}, im.vec(a + "ff2.bias", W));
+    }
+}
+
+void import_bitvla(const std::string& path, gguf_reader& g, Checkpoint& ck) {
     const int64_t H = need_u32(g, "bitvla.lm.hidden"), L = need_u32(g, "bitvla.lm.layers"), Hq = need_u32(g, "bitvla.lm.q_heads"),
                   Hkv = need_u32(g, "bitvla.lm.kv_heads"), D = need_u32(g, "bitvla.lm.head_dim"),
                   vocab = need_u32(g, "bitvla.lm.vocab_size");
@@ -228,7 +419,7 @@ void import_bitvla(gguf_reader& g, Checkpoint& ck) {
     ck.set_key("vocab", vocab);
 
     Importer im{g, ck, false};
-    ck.add_f32("prefix.E_lang", {vocab, H}, im.mat("token_embd.weight", vocab, H));
+    put_token_embeddings(path, g, ck, "token_embd.weight", vocab, H, [&]() { return im.mat("token_embd.weight", vocab, H); });
     ck.add_f32("act.emb", {n_act, H}, im.mat("act.emb", n_act, H));
     ck.add_f32("act.W_out", {A, H}, im.mat("act.W_out", A, H));
     ck.add_f32("act.b_out", {A}, im.vec("act.b_out", A));
@@ -263,12 +454,14 @@ void import_bitvla(gguf_reader& g, Checkpoint& ck) {
         for (const auto& part : {std::make_pair("attn_q", qd), std::make_pair("attn_k", kvd), std::make_pair("attn_v", kvd)}) {
             const std::string name = b + part.first + ".weight";
             std::vector<uint8_t> bytes = g.read_convert(name.c_str(), GGUF_T_I8);
+            trace(name);
             if ((int64_t)bytes.size() != part.second * H / 4) throw std::runtime_error("vla: gguf int2 tensor " + name + " has the wrong size");
             std::vector<uint32_t> words((size_t)vla_ternary_packed_words((int)part.second, (int)H));
             if (vla_ternary_repack_ladder_host(bytes.data(), (int)part.second, (int)H, words.data()) != VLA_K_OK)
                 throw std::runtime_error("vla: cannot re-order gguf int2 tensor " + name);
             fused.insert(fused.end(), words.begin(), words.end());
             const std::vector<float> sc = g.read_f32((b + part.first + ".scale").c_str());
+            trace(b + part.first + ".scale");
             if (sc.empty()) throw std::runtime_error("vla: int2 tensor " + name + " has no .scale sidecar");
             ws.push_back(sc[0]);
         }
@@ -276,6 +469,8 @@ void import_bitvla(gguf_reader& g, Checkpoint& ck) {
         ck.add_f32(o + "Wqkv.ws", {3}, ws);
         const std::string on = b + "attn_o.weight";
         std::vector<uint8_t> ob = g.read_convert(on.c_str(), GGUF_T_I8);
+        trace(on);
+        trace(b + "attn_o.scale");
         if ((int64_t)ob.size() != H * qd / 4) throw std::runtime_error("vla: gguf int2 tensor " + on + " has the wrong size");
         ck.add_tensor(o + "Wo.i2", "u8", {(int64_t)ob.size()}, ob.data(), ob.size());
         const std::vector<float> osc = g.read_f32((b + "attn_o.scale").c_str());
@@ -294,10 +489,11 @@ Checkpoint import_gguf(const std::string& path) {
     const char* wd = std::getenv("VLA_WEIGHT_DTYPE");
     const bool bf16 = !(wd && std::string(wd) == "f32");
     Checkpoint ck;
-    if (g.has("smolvla.architecture")) import_flow(g, ck, bf16, "smolvla");
-    else if (g.has("pi05.architecture")) import_flow(g, ck, bf16, "pi05");
-    else if (g.has("pi0.architecture")) import_flow(g, ck, bf16, "pi0");
-    else if (g.has("bitvla.architecture") || g.has("bitvla.lm.hidden")) import_bitvla(g, ck);
+    if (g.has("smolvla.architecture")) import_flow(path, g, ck, bf16, "smolvla");
+    else if (g.has("pi05.architecture")) import_flow(path, g, ck, bf16, "pi05");
+    else if (g.has("pi0.architecture")) import_flow(path, g, ck, bf16, "pi0");
+    else if (g.has("gr00t_n1_5.architecture")) import_gr00t(g, ck, bf16);
+    else if (g.has("bitvla.architecture") || g.has("bitvla.lm.hidden")) import_bitvla(path, g, ck);
     else throw std::runtime_error("vla: " + path + ": no importer for this gguf's architecture");
     return ck;
 }
@@ -310,6 +506,25 @@ struct vla_gguf {
 };
 
 extern "C" {
+
+int64_t vla_gguf_import_trace(const char* path, char* out, int64_t cap) {
+    if (!path || !out || cap <= 0) return VLA_GGUF_ERR_ARG;
+    std::vector<std::string> names;
+    try {
+        vla::g_trace = &names;
+        (void)vla::import_gguf(path);
+        vla::g_trace = nullptr;
+    } catch (const std::exception& e) {
+        vla::g_trace = nullptr;
+        std::fprintf(stderr, "%s\n", e.what());
+        return VLA_GGUF_ERR_READ;
+    }
+    std::string all;
+    for (const std::string& n : names) all += n + "\n";
+    if ((int64_t)all.size() + 1 > cap) return -(int64_t)(all.size() + 1) - 16;
+    std::memcpy(out, all.c_str(), all.size() + 1);
+    return (int64_t)all.size();
+}
 
 vla_gguf* vla_gguf_open(const char* path) {
     if (!path) return nullptr;
