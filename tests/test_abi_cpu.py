@@ -1,12 +1,13 @@
 """CPU-side checks of the C-ABI library: it loads, exports every declared
 symbol, and its host-only helpers (no GPU needed) agree with the oracle."""
 import ctypes
+import os
 
 import numpy as np
 import pytest
 
 import oracle as orc
-from util import declared_symbols, pkg
+from util import ROOT, declared_symbols, pkg
 
 
 def test_library_exports_every_declared_kernel_symbol():
@@ -117,3 +118,56 @@ def test_null_and_shape_errors_are_reported_not_fatal():
     assert lib.vla_linear(None, None, None, None, None, 0, 0, 1, 1, 4, None) == pkg.VLA_K_ERR_ARG
     assert lib.vla_attn_prefix_suffix(None, None, None, None, 0, 1, 1, 1, 1, 64, 64, 1, 1.0, 0, 0, 0, 0, None, None) == pkg.VLA_K_ERR_ARG
     assert lib.vla_ternary_gemm(None, None, None, None, None, None, None, 1, 1, 16, 128, None) == pkg.VLA_K_ERR_ARG
+
+
+# ---------------------------------------------------------------- struct layout of include/vla.h
+def _header_fields(text, name):
+    """(field, C type) pairs of `typedef struct { ... } name;`, one per declarator."""
+    import re
+    m = re.search(r"typedef struct \{([^{}]*)\}\s*" + name + r"\s*;", text, re.S)
+    assert m, name + " not found in vla.h"
+    body = re.sub(r"/\*.*?\*/", "", m.group(1), flags=re.S)
+    out = []
+    for decl in body.split(";"):
+        decl = " ".join(decl.split())
+        if not decl:
+            continue
+        first, *rest = [d.strip() for d in decl.split(",")]
+        parts = first.replace("*", " * ").split()
+        ctype = " ".join(p for p in parts[:-1] if p != "const")
+        out.append((parts[-1], ctype))
+        out += [(r.lstrip("* "), ctype) for r in rest]
+    return out
+
+
+def test_ctypes_structs_follow_the_header_field_for_field(tmp_path):
+    """The check the reference runs on its own bindings (tests/py/test_bindings.py:29-64): field
+    order and types of the ctypes mirrors against the header text -- and, since a C compiler is
+    at hand, sizes and offsets against what gcc lays out."""
+    import ctypes
+    import subprocess
+    from vla_cpp_amd import ffi
+    text = open(os.path.join(ROOT, "include", "vla.h")).read()
+    c_types = {"int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64, "float": ctypes.c_float, "double": ctypes.c_double}
+    pairs = (("vla_config", ffi.Config), ("vla_image", ffi.Image), ("vla_inputs", ffi.Inputs), ("vla_stats", ffi.Stats))
+    prog = ["#include <stdio.h>", "#include <stddef.h>", '#include "vla.h"', "int main(void) {"]
+    for c_name, py in pairs:
+        hdr = _header_fields(text, c_name)
+        assert [n for n, _ in hdr] == [n for n, _ in py._fields_], c_name
+        for (hn, ht), (pn, pt) in zip(hdr, py._fields_):
+            if ht.endswith("*"):
+                assert issubclass(pt, (ctypes._Pointer, ctypes.c_void_p)) or pt is ctypes.c_void_p, (c_name, hn)
+            else:
+                assert pt is c_types[ht], (c_name, hn, ht, pt)
+            prog.append('  printf("%s.%s %%zu\\n", offsetof(%s, %s));' % (c_name, hn, c_name, hn))
+        prog.append('  printf("%s %%zu\\n", sizeof(%s));' % (c_name, c_name))
+    prog += ["  return 0;", "}"]
+    src, exe = os.path.join(str(tmp_path), "layout.c"), os.path.join(str(tmp_path), "layout")
+    open(src, "w").write("\n".join(prog))
+    subprocess.run(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), src, "-o", exe], check=True)  # the header is C-clean
+    want = dict(l.split() for l in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.splitlines())
+    for c_name, py in pairs:
+        assert ctypes.sizeof(py) == int(want[c_name]), c_name
+        for n, _ in py._fields_:
+            assert getattr(py, n).offset == int(want["%s.%s" % (c_name, n)]), (c_name, n)
+    assert ffi.ABI_VERSION == int(__import__("re").search(r"#define VLA_ABI_VERSION\s+(\d+)", text).group(1))

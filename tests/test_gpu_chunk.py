@@ -115,6 +115,21 @@ def test_config2_pi0_mqa_bf16(tmp_path, n_layers, batch):
     m.close()
 
 
+def test_config2_pi0_in_the_references_default_fp32(tmp_path):
+    # pi0's default activation type in the reference is F32 (src/models/pi0.cpp:90, 174-176):
+    # 256-wide heads in fp32, held to 1e-5 like config 0
+    cfg = ckpt.pi0_config(n_layers=3, dtype="f32")
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 8)
+    r = np.random.default_rng(231)
+    obs = [make_obs(cfg, r, n_views=2) for _ in range(2)]
+    m = load(tmp_path, cfg, w, "cfg2_f32")
+    got = m.predict_batch(obs).reshape(2, 50, 32)
+    for b in range(2):
+        want = orc_chunk.flow_expert_chunk(cfg, w, obs[b])
+        assert rel_err(got[b], want) < 1e-5, rel_err(got[b], want)
+    m.close()
+
+
 @pytest.mark.parametrize("n_layers,batch", [(4, 2), (16, 1)])
 def test_config3_gr00t_dit_bf16(tmp_path, n_layers, batch):
     cfg = ckpt.gr00t_config(n_layers=n_layers)

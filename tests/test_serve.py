@@ -185,6 +185,9 @@ def test_queued_requests_are_answered_in_batches_with_the_servers_checks(tmp_pat
         frame(obs[0], 110, noise=obs[0]["noise"].ravel()[:100]),
         PredictRequest(request_id=111, lang_tokens=[1], state=obs[0]["state"].tolist()).SerializeToString(),  # no image input at all
         frame(obs[0], 112, lang=np.zeros(49, np.int32)),           # longer than tokenizer_max_length
+        # passes the wire checks, is rejected by the engine (token outside the vocabulary): it shares
+        # the (2 views, 48 tokens) batch with frames 0, 3 and 6, which must still be served
+        frame(obs[0], 113, lang=np.full(48, cfg["vocab"] + 7, np.int32)),
     ]
     n = len(frames)
     bufs = [ctypes.create_string_buffer(f, len(f)) for f in frames]
@@ -209,7 +212,8 @@ def test_queued_requests_are_answered_in_batches_with_the_servers_checks(tmp_pat
     errs = {2: "state length 31 != expected 32", 4: "request parse failed", 7: "lang_tokens[1] = -2 is negative",
             8: "precomputed_img_emb size %d != %d (n_views=3 * n_img_per_view=64 * hidden=960)" % (2 * 64 * 960, 3 * 64 * 960),
             9: "state[4] = nan is not finite (NaN/Inf)", 10: "noise length 100 != 0 or 1600 (chunk_size * action_dim)",
-            11: "PredictRequest must contain images or precomputed_img_emb", 12: "lang_tokens length 49 out of range [1, 48]"}
+            11: "PredictRequest must contain images or precomputed_img_emb", 12: "lang_tokens length 49 out of range [1, 48]",
+            13: "predict failed"}
     for i, text in errs.items():
         assert out[i].error == text and len(out[i].action_chunk) == 0, (i, out[i].error)
         assert out[i].request_id == (0 if i == 4 else 100 + i)

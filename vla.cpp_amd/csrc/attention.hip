@@ -1351,6 +1351,112 @@ int launch_d(AttnArgs& a, vla_stream_t stream, Scratch& sc) {
     return VLA_K_ERR_SHAPE;
 }
 
+
+// fp32 attention for 256-wide heads (pi0's default activation type in the reference is F32,
+// src/models/pi0.cpp:90, 174-176).  The MFMA kernel's fp32 tiles of such heads exceed the
+// static LDS budget and its accumulators the register file, and this case is about matching
+// the reference's precision, not about speed: a plain FMA kernel.  A workgroup (256 threads)
+// owns WR query rows of one (batch, query head): pass 1, thread t forms the scores of keys
+// t, t + 256, ... against the WR rows (its K row streamed once for all of them); exact
+// two-pass softmax per row over the scores kept in LDS; pass 2, thread d accumulates output
+// column d over V^T tiles of 16 keys staged in LDS.  fp32 throughout, keys added in order.
+constexpr int WIDE_D = 256, WIDE_R = 8, WIDE_VK = 16, WIDE_MAX_KEYS = 1152;
+__global__ void __launch_bounds__(256) attn_f32_wide_kernel(AttnArgs a) {
+    __shared__ float qs[WIDE_R][WIDE_D];
+    __shared__ float sc[WIDE_R][WIDE_MAX_KEYS];
+    __shared__ float vt[WIDE_D][WIDE_VK + 1];
+    __shared__ float red[16];
+    const int tid = threadIdx.x;
+    const int n_rt = (a.S + WIDE_R - 1) / WIDE_R;
+    const int rt = blockIdx.x % n_rt, bh = blockIdx.x / n_rt;
+    const int h = bh % a.Hq, b = bh / a.Hq;
+    const int hk = h / (a.Hq / a.Hkv);
+    const int s0 = rt * WIDE_R, nr = min(WIDE_R, a.S - s0);
+    const float* kbase = (const float*)a.k_cache + ((long)b * a.Hkv + hk) * a.t_max * WIDE_D;
+    const float* vbase = (const float*)a.vt_cache + ((long)b * a.Hkv + hk) * WIDE_D * (long)a.t_max;
+    for (int i = tid; i < WIDE_R * WIDE_D; i += 256) {
+        const int r = i / WIDE_D, d = i % WIDE_D;
+        qs[r][d] = r < nr ? ((const float*)a.q)[(((long)b * a.S + s0 + r) * a.Hq + h) * WIDE_D + d] : 0.f;
+    }
+    __syncthreads();
+    const int pad_lo = a.pad_start, pad_hi = min(a.pad_end, a.n_prefix);
+    for (int key = tid; key < a.n_keys; key += 256) {
+        float acc[WIDE_R];
+#pragma unroll
+        for (int r = 0; r < WIDE_R; ++r) acc[r] = 0.f;
+        const f32x4_t* kr = reinterpret_cast<const f32x4_t*>(kbase + (long)key * WIDE_D);
+        for (int d4 = 0; d4 < WIDE_D / 4; ++d4) {
+            const f32x4_t kv = kr[d4];
+#pragma unroll
+            for (int r = 0; r < WIDE_R; ++r) {
+                const f32x4_t qv = *reinterpret_cast<const f32x4_t*>(&qs[r][d4 * 4]);
+                acc[r] = fmaf(kv[0], qv[0], acc[r]);
+                acc[r] = fmaf(kv[1], qv[1], acc[r]);
+                acc[r] = fmaf(kv[2], qv[2], acc[r]);
+                acc[r] = fmaf(kv[3], qv[3], acc[r]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < WIDE_R; ++r) {
+            const int s = s0 + r;
+            float v = acc[r] * a.scale;
+            if (a.mask) {
+                v += r < nr ? a.mask[(long)s * a.n_keys + key] : 0.f;
+            } else {
+                int hi = a.n_keys;
+                if (a.mask_kind == VLA_MASK_CAUSAL_SUFFIX) hi = min(a.n_keys, a.n_prefix + s + 1);
+                else if (a.mask_kind == VLA_MASK_PI0_STATE && s == 0) hi = min(a.n_keys, a.n_prefix + 1);
+                if (!(key < hi) || (key >= pad_lo && key < pad_hi)) v = -INFINITY;
+            }
+            sc[r][key] = v;
+        }
+    }
+    __syncthreads();
+    // softmax per row: max, exp, sum (ggml_soft_max_ext's order, src/layers/attn.h:43)
+    float inv[WIDE_R];
+    for (int r = 0; r < WIDE_R; ++r) {
+        float m = -INFINITY;
+        for (int key = tid; key < a.n_keys; key += 256) m = fmaxf(m, sc[r][key]);
+        m = block_max(m, red);
+        float sum = 0.f;
+        for (int key = tid; key < a.n_keys; key += 256) {
+            const float e = m == -INFINITY ? 0.f : expf(sc[r][key] - m);
+            sc[r][key] = e;
+            sum += e;
+        }
+        sum = block_sum(sum, red);
+        inv[r] = sum > 0.f ? 1.0f / sum : 0.f;
+    }
+    __syncthreads();
+    float o[WIDE_R];
+#pragma unroll
+    for (int r = 0; r < WIDE_R; ++r) o[r] = 0.f;
+    for (int k0 = 0; k0 < a.n_keys; k0 += WIDE_VK) {
+        __syncthreads();
+        for (int i = tid; i < WIDE_D * WIDE_VK; i += 256) {
+            const int d = i / WIDE_VK, kk = i % WIDE_VK;
+            vt[d][kk] = k0 + kk < a.n_keys ? vbase[(long)d * a.t_max + k0 + kk] : 0.f;
+        }
+        __syncthreads();
+        const int nk = min(WIDE_VK, a.n_keys - k0);
+        for (int kk = 0; kk < nk; ++kk) {
+            const float v = vt[tid][kk];
+#pragma unroll
+            for (int r = 0; r < WIDE_R; ++r) o[r] = fmaf(sc[r][k0 + kk], v, o[r]);
+        }
+    }
+    for (int r = 0; r < nr; ++r)
+        ((float*)a.out)[(((long)b * a.S + s0 + r) * a.Hq + h) * WIDE_D + tid] = o[r] * inv[r];
+}
+
+int launch_f32_wide(AttnArgs& a, hipStream_t st, Scratch& sc) {
+    if (a.n_keys > WIDE_MAX_KEYS) return VLA_K_ERR_SHAPE;
+    if (sc.kind == Scratch::DRY) return VLA_K_OK;
+    const unsigned grid = (unsigned)((long)a.batch * a.Hq * ((a.S + WIDE_R - 1) / WIDE_R));
+    attn_f32_wide_kernel<<<grid, 256, 0, st>>>(a);
+    return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+}
+
 template <typename T>
 int launch_t(AttnArgs& a, int D, vla_stream_t stream, Scratch& sc) {
     switch (D) {
@@ -1358,9 +1464,8 @@ int launch_t(AttnArgs& a, int D, vla_stream_t stream, Scratch& sc) {
         case 64: return launch_d<T, 64>(a, stream, sc);
         case 128: return launch_d<T, 128>(a, stream, sc);
         case 256:
-            // fp32 tiles of 256-wide heads would not fit the LDS budget; only bf16 is built.
             if constexpr (sizeof(T) == 2) return launch_d<T, 256>(a, stream, sc);
-            else return VLA_K_ERR_SHAPE;
+            else return launch_f32_wide(a, (hipStream_t)stream, sc);  // its own kernel, see there
         default: return VLA_K_ERR_SHAPE;
     }
 }

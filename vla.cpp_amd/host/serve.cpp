@@ -120,8 +120,8 @@ int32_t vla_serve_requests(vla_model* m, int32_t n, const uint8_t* const* req, c
             }
             groups[{(int)q[i].precomputed_img_emb_n_views, (int)q[i].lang_tokens.size()}].push_back(i);
         }
-        for (const auto& grp : groups) {
-            const std::vector<int>& idx = grp.second;
+        // One engine call for the requests `idx`; fills their bodies and returns the engine's status.
+        auto run_group = [&](const std::vector<int>& idx, bool answer_failures) -> int32_t {
             std::vector<vla_inputs> in(idx.size());
             for (size_t k = 0; k < idx.size(); ++k) {
                 const PredictRequest& r = q[(size_t)idx[k]];
@@ -155,9 +155,14 @@ int32_t vla_serve_requests(vla_model* m, int32_t n, const uint8_t* const* req, c
             st.ms_prefill = ms(t0, t1);
             st.ms_denoise = ms(t1, t2);
             const int64_t per = (int64_t)idx.size() ? act_n / (int64_t)idx.size() : 0;
+            const bool failed = rc != VLA_OK || !act || per != n_actions * cfg.max_action_dim;
+            if (failed && !answer_failures) {
+                vla_free_actions(act);
+                return rc != VLA_OK ? rc : VLA_ERR_PREDICT;
+            }
             for (size_t k = 0; k < idx.size(); ++k) {
                 const int i = idx[k];
-                if (rc != VLA_OK || !act || per != n_actions * cfg.max_action_dim) {
+                if (failed) {
                     body[(size_t)i] = error_response(q[(size_t)i].request_id, "predict failed");
                 } else {
                     PredictResponse r;
@@ -175,6 +180,19 @@ int32_t vla_serve_requests(vla_model* m, int32_t n, const uint8_t* const* req, c
                 answered[(size_t)i] = 1;
             }
             vla_free_actions(act);
+            return failed ? (rc != VLA_OK ? rc : VLA_ERR_PREDICT) : VLA_OK;
+        };
+        for (const auto& grp : groups) {
+            const std::vector<int>& idx = grp.second;
+            // A request the engine itself rejects (an out-of-vocabulary token, say) fails the batched
+            // call for everyone in it; the reference serves one request per predict, so only the
+            // offender may see an error: on a rejection the members are served one by one.
+            if (idx.size() > 1) {
+                if (run_group(idx, false) == VLA_OK) continue;
+                for (int i : idx) (void)run_group(std::vector<int>{i}, true);
+            } else {
+                (void)run_group(idx, true);
+            }
         }
         for (int i = 0; i < n; ++i) {
             resp[i] = to_frame(body[(size_t)i], &resp_len[i]);
