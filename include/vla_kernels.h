@@ -175,6 +175,30 @@ VLA_KAPI int vla_rmsnorm_attn_qkv_rope(const void* x, const void* W_folded, cons
                                        const float* cos_tab, const float* sin_tab, void* q_out, void* k_cache,
                                        void* vt_cache, int t_max, int tok_offset, float rms_eps, vla_stream_t stream);
 
+/* The same launch with a DiT block's modulated LayerNorm taken inside it: replaces
+ * adaln -> mm_w(Wq[/Wk/Wv]) -> rope -> concat (src/layers/norm.h:37-46,
+ * src/modules/dit_head.cpp:111-119), xn (1 + scale) + shift with xn = ggml_norm(x).
+ * x is the un-normalised residual stream.  The modulation depends on the denoise step
+ * only, so it lives in the operands, one set per step (vla_fold_adaln_weight_host):
+ *   W_folded[n][k] = W[n][k] (1 + scale[k]),  colsum[n] = sum_k W_folded[n][k],
+ *   bias[n] = b[n] + sum_k W[n][k] shift[k]
+ * and the launch computes rstd[m] (acc[m][n] - mean[m] colsum[n]) + bias[n] with the
+ * mean and variance of row m summed from the operand tiles it multiplies.  bf16 only,
+ * K a multiple of 16 and 16-byte aligned operands; VLA_K_ERR_SHAPE otherwise (use
+ * vla_adaln + vla_attn_qkv_rope then). */
+VLA_KAPI int vla_layernorm_attn_qkv_rope(const void* x, const void* W_folded, const float* colsum, const float* bias,
+                                         int dtype, int M, int K, int S, int n_q_heads, int n_kv_heads, int has_k,
+                                         int has_v, int head_dim, const float* cos_tab, const float* sin_tab, void* q_out,
+                                         void* k_cache, void* vt_cache, int t_max, int tok_offset, float ln_eps,
+                                         vla_stream_t stream);
+
+/* Host helper for the call above (bf16 weights [N][K], fp32 scale/shift [K], fp32 bias [N]
+ * or NULL): writes W_out (bf16, rounded to nearest even; may alias W), colsum_out and
+ * bias_out (fp32 [N]); colsum is taken over the rounded W_out, the values the launch
+ * multiplies. */
+VLA_KAPI int vla_fold_adaln_weight_host(const void* W, const float* bias, const float* scale, const float* shift, int N,
+                                        int K, void* W_out, float* colsum_out, float* bias_out);
+
 /* Host helper for the call above: W_out[n][k] = W[n][k] * g[k] in `dtype` (bf16
  * products rounded to nearest even; g is the RMSNorm weight ggml_mul applies after
  * ggml_rms_norm, src/layers/norm.h:31-34).  W_out may alias W. */

@@ -95,6 +95,42 @@ def test_pair_rope_rows_host_is_the_row_permutation_the_decode_epilogue_assumes(
     assert lib.vla_ternary_pair_rope_rows_host(packed.ctypes.data, Hq, Hkv, D, K, packed.ctypes.data) == pkg.VLA_K_ERR_ARG
 
 
+def test_fold_adaln_weight_host_operands():
+    """Operand set of the projection launch that takes a DiT block's modulated LayerNorm
+    inside it: rounded W (1 + scale), column sums of the rounded values, bias + W shift.
+    With them rstd (x W'^T - mean colsum) + bias' equals adaln(x) W^T + b up to the bf16
+    rounding of W' (checked in float64 on unrounded-compatible values)."""
+    lib = pkg.lib()
+    r = np.random.default_rng(5)
+    N, K = 24, 48
+    W = orc.round_bf16((0.2 * r.standard_normal((N, K))).astype(np.float32))
+    b = r.standard_normal(N).astype(np.float32)
+    # scales that keep W (1 + scale) exactly representable in bf16: powers of two minus one
+    sc = r.choice(np.array([0.0, 1.0, -0.5, 3.0], np.float32), K)
+    sh = r.standard_normal(K).astype(np.float32)
+    Wf, cs, bs = np.empty((N, K), np.uint16), np.empty(N, np.float32), np.empty(N, np.float32)
+    assert lib.vla_fold_adaln_weight_host(orc.to_bf16(W).ctypes.data, b.ctypes.data, sc.ctypes.data, sh.ctypes.data, N, K,
+                                          Wf.ctypes.data, cs.ctypes.data, bs.ctypes.data) == pkg.VLA_K_OK
+    Wf32 = orc.from_bf16(Wf)
+    assert np.array_equal(Wf32, W * (1.0 + sc))
+    assert np.allclose(cs, Wf32.astype(np.float64).sum(1), rtol=1e-6, atol=1e-6)
+    assert np.allclose(bs, b + W.astype(np.float64) @ sh.astype(np.float64), rtol=1e-6, atol=1e-6)
+    x = r.standard_normal((7, K)) * 3 + 1.5
+    mean, var = x.mean(1, keepdims=True), x.var(1, keepdims=True)
+    rstd = 1.0 / np.sqrt(var + 1e-5)
+    got = rstd * (x @ Wf32.astype(np.float64).T - mean * cs[None, :]) + bs[None, :]
+    want = (((x - mean) * rstd) * (1.0 + sc) + sh) @ W.astype(np.float64).T + b
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+    # general scales: round to nearest even of the fp32 product, no bias
+    sc2 = (0.3 * r.standard_normal(K)).astype(np.float32)
+    assert lib.vla_fold_adaln_weight_host(orc.to_bf16(W).ctypes.data, None, sc2.ctypes.data, sh.ctypes.data, N, K,
+                                          Wf.ctypes.data, cs.ctypes.data, bs.ctypes.data) == pkg.VLA_K_OK
+    assert np.array_equal(Wf, orc.to_bf16(W * (np.float32(1.0) + sc2)))
+    assert np.allclose(bs, W.astype(np.float64) @ sh.astype(np.float64), rtol=1e-6, atol=1e-6)
+    assert lib.vla_fold_adaln_weight_host(None, None, sc.ctypes.data, sh.ctypes.data, N, K, Wf.ctypes.data, cs.ctypes.data,
+                                          bs.ctypes.data) == pkg.VLA_K_ERR_ARG
+
+
 def test_fold_norm_weight_host_rounds_products_to_nearest_even():
     lib = pkg.lib()
     r = np.random.default_rng(7)

@@ -323,6 +323,67 @@ def test_rmsnorm_inside_qkv_launch(name, B, S, Hq, Hkv, D, K, self_layer, P):
         assert rel_err(gf, gp) < 8e-3
 
 
+@pytest.mark.parametrize("name,B,S,Hq,Hkv,D,K,self_layer,bias", [
+    ("gr00t-self", 3, 17, 24, 24, 64, 1536, True, True),
+    ("gr00t-cross-q", 64, 17, 24, 24, 64, 1536, False, True),
+    ("small-no-bias", 2, 5, 2, 2, 64, 48, True, False),
+    ("partial-row-tile", 1, 33, 4, 4, 64, 272, False, True),
+])
+def test_modulated_layernorm_inside_qkv_launch(name, B, S, Hq, Hkv, D, K, self_layer, bias):
+    """A DiT block's adaLN taken inside the projection launch ((1 + scale) folded into W, the
+    shift into the bias, rows centred and scaled in the epilogue from sums taken over the
+    operand tiles) against the oracle's adaln -> linear, and against the two-launch GPU path.
+    Rows carry a mean of the size of their spread, so a dropped mean term fails."""
+    r = np.random.default_rng(2207 + K)
+    M = B * S
+    nkv = Hkv if self_layer else 0
+    N = (Hq + 2 * nkv) * D
+    eps = 1e-5
+    x = orc.round_bf16((2.0 * r.standard_normal((M, K)) * (1.0 + 3.0 * r.random((M, 1))) + 1.5 * r.standard_normal((M, 1))).astype(np.float32))
+    sc = (0.3 * r.standard_normal(K)).astype(np.float32)
+    sh = (0.3 * r.standard_normal(K)).astype(np.float32)
+    W = orc.round_bf16((0.02 * r.standard_normal((N, K))).astype(np.float32))
+    b = (0.1 * r.standard_normal(N)).astype(np.float32) if bias else None
+    t_max = (S + 63) // 64 * 64
+
+    def run(fused):
+        kc, vc = empty((B, Hkv, t_max, D), BF16), empty((B, Hkv, D, t_max), BF16)
+        q = empty((M, Hq * D), BF16)
+        if fused:
+            Wf, cs, bs = np.empty((N, K), np.uint16), np.empty(N, np.float32), np.empty(N, np.float32)
+            assert pkg.lib().vla_fold_adaln_weight_host(orc.to_bf16(W).ctypes.data, None if b is None else b.ctypes.data,
+                                                        sc.ctypes.data, sh.ctypes.data, N, K, Wf.ctypes.data, cs.ctypes.data,
+                                                        bs.ctypes.data) == 0
+            pkg.call("vla_layernorm_attn_qkv_rope", to_dev(x, BF16), dev(Wf), dev(cs), dev(bs), BF16, M, K, S, Hq, Hkv,
+                     int(self_layer), int(self_layer), D, None, None, q, kc, vc, t_max, 0, eps)
+        else:
+            hn = empty((M, K), BF16)
+            pkg.call("vla_adaln", to_dev(x, BF16), dev(sc), dev(sh), hn, BF16, M, K, eps)
+            pkg.call("vla_attn_qkv_rope", hn, to_dev(W, BF16), None if b is None else dev(b), BF16, M, K, S, Hq, Hkv,
+                     int(self_layer), int(self_layer), D, None, None, q, kc, vc, t_max, 0)
+        out = [as_f32(q, BF16).reshape(M, Hq, D)]
+        if self_layer:
+            kd, vd = empty((B, S, Hkv, D), BF16), empty((B, S, Hkv, D), BF16)
+            pkg.call("vla_kv_gather", kc, vc, kd, vd, BF16, B, Hkv, D, t_max, 0, S)
+            out += [as_f32(kd, BF16).reshape(M, Hkv, D), as_f32(vd, BF16).reshape(M, Hkv, D)]
+        sync()
+        return out
+
+    y = orc.linear(orc.adaln(x, sc, sh, eps), W, b)
+    want = [y[:, :Hq * D].reshape(M, Hq, D)]
+    if self_layer:
+        want += [y[:, Hq * D:(Hq + Hkv) * D].reshape(M, Hkv, D), y[:, (Hq + Hkv) * D:].reshape(M, Hkv, D)]
+    fused, pair = run(True), run(False)
+    for gf, gp, w in zip(fused, pair, want):
+        assert bf16_close(gf, w) and rel_err(gf, w) < 8e-3
+        assert rel_err(gf, gp) < 8e-3
+    # the mean term matters at this input: a norm that does not centre the rows is far outside the bar
+    assert rel_err(orc.linear(orc.rms_norm(x, None, eps) * (1 + sc) + sh, W, b)[:, :Hq * D].reshape(M, Hq, D), want[0]) > 5e-2
+    # fp32 rows are not served by this launch
+    assert pkg.lib().vla_layernorm_attn_qkv_rope(x.ctypes.data, W.ctypes.data, sc.ctypes.data, None, F32, M, K, S, Hq, Hkv, 0, 0, D,
+                                                 None, None, x.ctypes.data, None, None, t_max, 0, eps, None) == pkg.VLA_K_ERR_SHAPE
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("M,I,K,act,bias", [(50, 2048, 720, "silu", False), (130, 96, 72, "gelu", True), (1600, 256, 720, "silu", False),
                                            (17, 6144, 1536, "gelu", True)])

@@ -38,6 +38,7 @@ constexpr int BN = 64;                     // epilogue sub-tile; column-tile uni
 constexpr int C_STRIDE = BN + 4;           // floats
 
 enum { EPI_PLAIN = 0, EPI_QKV = 1, EPI_TERNARY = 2, EPI_GLU = 3 };
+enum { NORM_NONE = 0, NORM_RMS = 1, NORM_LAYER = 2 };  // row statistics taken inside gemm_dl_kernel
 
 struct GemmArgs {
     const void* A;
@@ -64,8 +65,10 @@ struct GemmArgs {
     const int32_t* rowsum;
     const float* ws;
     int ws_num;
-    // RMS statistics of the A rows taken inside the GEMM (direct-to-LDS kernel, kNorm)
+    // Row statistics of A taken inside the GEMM (direct-to-LDS kernel, kNorm): RMS when
+    // colsum is null, else LayerNorm with colsum[n] = sum_k W[n][k] (fp32 [N])
     float norm_eps;
+    const float* colsum;
     const void* norm_w;  // ternary GEMV with the RMSNorm and quantisation of its rows inside: A is bf16, this the norm weight
 };
 
@@ -173,8 +176,8 @@ __device__ __forceinline__ TileCols tile_cols(const GemmArgs& a, int nt) {
 template <typename T, int kEpi>
 __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t* C, int m0, int nt, const TileCols& tc,
                                                int tid, bool have_res = false, u32x4_t res_lo = u32x4_t{0u, 0u, 0u, 0u},
-                                               u32x4_t res_hi = u32x4_t{0u, 0u, 0u, 0u}, bool scale_rows = false,
-                                               const float* row_scale = nullptr) {
+                                               u32x4_t res_hi = u32x4_t{0u, 0u, 0u, 0u}, int norm_mode = 0,
+                                               const float* row_scale = nullptr, const float* row_shift = nullptr) {
     const int erow = tid >> 2, jg = (tid & 3) * 8;
     const int m = m0 + erow;
     if (m >= a.M) return;
@@ -207,12 +210,21 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
         lo[e] = __uint_as_float(crow[jg + e]);
         hi[e] = __uint_as_float(crow[32 + jg + e]);
     }
-    if (scale_rows) {  // row_scale: one factor per row of the sub-tile (in LDS)
+    if (norm_mode) {  // row_scale: one factor per row of the sub-tile (in LDS)
         const float f = row_scale[erow];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             lo[e] *= f;
             hi[e] *= f;
+        }
+    }
+    if (norm_mode == NORM_LAYER && kEpi == EPI_QKV) {
+        // sum_k (x - mean) rstd W[n][k] = rstd acc - (mean rstd) colsum[n]; row_shift = mean rstd
+        const float ms = row_shift[erow];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            lo[e] -= ms * a.colsum[tc.base0 + jg + e];
+            hi[e] -= ms * a.colsum[tc.base1 + jg + e];
         }
     }
 
@@ -614,6 +626,12 @@ __device__ __forceinline__ float add_squares_bf16x2(uint32_t u, float acc) {
     const bf16x2_t v = __builtin_bit_cast(bf16x2_t, u);
     return __builtin_amdgcn_fdot2_f32_bf16(v, v, acc, false);
 }
+// acc + lo + hi
+__device__ __forceinline__ float add_pair_bf16x2(uint32_t u, float acc) {
+    const bf16x2_t v = __builtin_bit_cast(bf16x2_t, u);
+    const bf16x2_t ones = __builtin_bit_cast(bf16x2_t, 0x3f803f80u);
+    return __builtin_amdgcn_fdot2_f32_bf16(v, ones, acc, false);
+}
 
 // ---- bf16 GEMM with operand tiles loaded straight into LDS --------------------------
 // Same tiling, wavefront layout, XCD mapping and epilogues as gemm_kernel, for bf16
@@ -625,7 +643,7 @@ __device__ __forceinline__ float add_squares_bf16x2(uint32_t u, float acc) {
 // consecutive fragment rows then cover all 64 banks exactly once); the loading lane picks
 // the global piece that belongs in its LDS slot.  NS - 1 tiles of loads are in flight; a
 // k-tile costs one barrier, and no wavefront spends issue slots on LDS stores.
-template <int kEpi, int TM, int TN, int KB, int NS, bool kNorm>
+template <int kEpi, int TM, int TN, int KB, int NS, int kNorm>
 __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     typedef bf16_t T;
     typedef Traits<bf16_t> TR;
@@ -637,7 +655,7 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     constexpr int NCH = KB / 32;        // 16-k MFMA chunks per tile
     constexpr int STAGE = (ROWS_A + ROWS_W) * KB;
     constexpr int C_BYTES = 4 * 64 * C_STRIDE;
-    constexpr int EPI_BYTES = C_BYTES + ROWS_A * 4;  // C sub-tile, then one scale per tile row (kNorm)
+    constexpr int EPI_BYTES = C_BYTES + ROWS_A * 8;  // C sub-tile, then one scale and one shift per tile row (kNorm)
     constexpr int LDS_BYTES = NS * STAGE > EPI_BYTES ? NS * STAGE : EPI_BYTES;
     constexpr int IN_FLIGHT = (NS - 2) * NLOAD;  // loads younger than the tile about to be multiplied
     static_assert(KB == 128 || KB == 256, "swizzle is defined for 128- and 256-byte rows");
@@ -670,10 +688,12 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     // kNorm: the GEMM multiplies raw rows of A and scales row m of the result by
     // rsqrt(mean_k A[m][k]^2 + eps); the squares are summed from the same LDS fragments
     // the MFMAs read (lane (g, r) sees 8 of every 16 k of its rows; the two halves meet
-    // after the loop), two bf16 products per instruction.
-    float ssq[TM];
+    // after the loop), two bf16 products per instruction.  NORM_LAYER also sums the values:
+    // row m of the result becomes rstd (acc - mean colsum[n]), the projection of the
+    // centred and scaled row.
+    float ssq[TM], ssum[TM];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) ssq[i] = 0.f;
+    for (int i = 0; i < TM; ++i) ssq[i] = ssum[i] = 0.f;
 
     // A bf16 residual is fetched now, ahead of every operand load, instead of in the
     // epilogue where nothing is left to hide its latency (the epilogue thread layout:
@@ -758,7 +778,10 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) ssq[i] = add_squares_bf16x2(fa[ch % SLOTS][i][e], ssq[i]);
+                        for (int e = 0; e < 4; ++e) {
+                            ssq[i] = add_squares_bf16x2(fa[ch % SLOTS][i][e], ssq[i]);
+                            if (kNorm == NORM_LAYER) ssum[i] = add_pair_bf16x2(fa[ch % SLOTS][i][e], ssum[i]);
+                        }
                 }
             }
             __builtin_amdgcn_sched_barrier(0);  // keeps the reads and loads where they were placed
@@ -792,12 +815,22 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
 
     uint32_t* C = reinterpret_cast<uint32_t*>(lds);
     float* row_scale = reinterpret_cast<float*>(lds + C_BYTES);
+    float* row_shift = row_scale + ROWS_A;
     if (kNorm) {
         const float inv_k = 1.0f / (float)a.K;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             const float t = ssq[i] + __shfl_xor(ssq[i], 32, 64);
-            if (wn == 0 && g == 0) row_scale[(wm + 2 * i) * 32 + r] = rsqrtf(t * inv_k + a.norm_eps);
+            if (kNorm == NORM_LAYER) {
+                const float mean = (ssum[i] + __shfl_xor(ssum[i], 32, 64)) * inv_k;
+                const float rstd = rsqrtf(fmaxf(t * inv_k - mean * mean, 0.f) + a.norm_eps);
+                if (wn == 0 && g == 0) {
+                    row_scale[(wm + 2 * i) * 32 + r] = rstd;
+                    row_shift[(wm + 2 * i) * 32 + r] = mean * rstd;
+                }
+            } else if (wn == 0 && g == 0) {
+                row_scale[(wm + 2 * i) * 32 + r] = rsqrtf(t * inv_k + a.norm_eps);
+            }
         }
     }
 #pragma unroll
@@ -814,7 +847,7 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
             const int nt_sub = ntw * TN + j;
             if (nt_sub < a.n_tiles)
                 epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0], res_pf[i][j][1], kNorm,
-                                        row_scale + i * 64);
+                                        row_scale + i * 64, row_shift + i * 64);
         }
 }
 
@@ -1234,13 +1267,19 @@ void launch_cfg(GemmArgs a, hipStream_t st) {
 template <int kEpi, int TM, int TN, int KB, int NS>
 void launch_dl(GemmArgs a, hipStream_t st) {
     const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, 1.0);
-    if constexpr (kEpi == EPI_QKV || kEpi == EPI_GLU) {
-        if (a.norm_eps >= 0.f) {
-            gemm_dl_kernel<kEpi, TM, TN, KB, NS, true><<<grid, 256, 0, st>>>(a);
+    if constexpr (kEpi == EPI_QKV) {
+        if (a.norm_eps >= 0.f && a.colsum) {
+            gemm_dl_kernel<kEpi, TM, TN, KB, NS, NORM_LAYER><<<grid, 256, 0, st>>>(a);
             return;
         }
     }
-    gemm_dl_kernel<kEpi, TM, TN, KB, NS, false><<<grid, 256, 0, st>>>(a);
+    if constexpr (kEpi == EPI_QKV || kEpi == EPI_GLU) {
+        if (a.norm_eps >= 0.f) {
+            gemm_dl_kernel<kEpi, TM, TN, KB, NS, NORM_RMS><<<grid, 256, 0, st>>>(a);
+            return;
+        }
+    }
+    gemm_dl_kernel<kEpi, TM, TN, KB, NS, NORM_NONE><<<grid, 256, 0, st>>>(a);
 }
 
 template <typename T, int kEpi>
@@ -1275,6 +1314,7 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             dl = tuning().gemm_dl != 0 && a.K % 16 == 0 && ((uintptr_t)a.A % 16 == 0) && ((uintptr_t)a.W % 16 == 0);
         }
         if (a.norm_eps >= 0.f && !(dl && (kEpi == EPI_QKV || kEpi == EPI_GLU))) return VLA_K_ERR_SHAPE;  // only that kernel takes the row statistics
+        if (a.colsum && kEpi != EPI_QKV) return VLA_K_ERR_SHAPE;
         if (dl) {
             int ns = tuning().gemm_stages;
             const long wgs = cfg == 0 ? wgs0 : (cfg == 2 || cfg == 3 ? wgs2 : wgs4);
@@ -1400,7 +1440,7 @@ int vla_linear(const void* x, const void* W, const float* bias, const void* resi
 static int qkv_rope_impl(const void* x, const void* W, const float* bias, int dtype, int M, int K, int S, int n_q_heads,
                          int n_kv_heads, int has_k, int has_v, int head_dim, const float* cos_tab, const float* sin_tab,
                          void* q_out, void* k_cache, void* vt_cache, int t_max, int tok_offset, float rms_eps,
-                         vla_stream_t stream) {
+                         vla_stream_t stream, const float* colsum = nullptr) {
     if (!x || !W || M < 0 || K <= 0 || S <= 0 || n_q_heads < 0 || n_kv_heads < 0 || head_dim <= 0) return VLA_K_ERR_ARG;
     const int nk = has_k ? n_kv_heads : 0, nv = has_v ? n_kv_heads : 0;
     if (n_q_heads > 0 && !q_out) return VLA_K_ERR_ARG;
@@ -1414,6 +1454,7 @@ static int qkv_rope_impl(const void* x, const void* W, const float* bias, int dt
     if (cos_tab && D % BN) return VLA_K_ERR_SHAPE;  // rotation pairs both halves of a head inside one tile
     GemmArgs a = {};
     a.norm_eps = rms_eps;
+    a.colsum = colsum;
     a.A = x; a.W = W; a.bias = bias; a.M = M; a.K = K;
     a.N = (n_q_heads + nk + nv) * D;
     a.S = S; a.Hq = n_q_heads; a.nk = nk; a.nv = nv; a.D = D; a.Hkv = n_kv_heads;
@@ -1511,6 +1552,16 @@ int vla_rmsnorm_attn_qkv_rope(const void* x, const void* W_folded, const float* 
                          q_out, k_cache, vt_cache, t_max, tok_offset, rms_eps, stream);
 }
 
+int vla_layernorm_attn_qkv_rope(const void* x, const void* W_folded, const float* colsum, const float* bias, int dtype, int M,
+                                int K, int S, int n_q_heads, int n_kv_heads, int has_k, int has_v, int head_dim,
+                                const float* cos_tab, const float* sin_tab, void* q_out, void* k_cache, void* vt_cache,
+                                int t_max, int tok_offset, float ln_eps, vla_stream_t stream) {
+    if (ln_eps < 0.f || !colsum) return VLA_K_ERR_ARG;
+    if (dtype != VLA_DT_BF16) return VLA_K_ERR_SHAPE;
+    return qkv_rope_impl(x, W_folded, bias, dtype, M, K, S, n_q_heads, n_kv_heads, has_k, has_v, head_dim, cos_tab, sin_tab,
+                         q_out, k_cache, vt_cache, t_max, tok_offset, ln_eps, stream, colsum);
+}
+
 int vla_fold_norm_weight_host(const void* W, const void* g, int dtype, int N, int K, void* W_out) {
     if (!W || !g || !W_out || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
     if (dtype == VLA_DT_F32) {
@@ -1537,6 +1588,34 @@ int vla_fold_norm_weight_host(const void* W, const void* g, int dtype, int N, in
         return VLA_K_OK;
     }
     return VLA_K_ERR_ARG;
+}
+
+int vla_fold_adaln_weight_host(const void* W, const float* bias, const float* scale, const float* shift, int N, int K,
+                               void* W_out, float* colsum_out, float* bias_out) {
+    if (!W || !scale || !shift || !W_out || !colsum_out || !bias_out || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    const uint16_t* w = (const uint16_t*)W;
+    for (long n = 0; n < N; ++n) {
+        double cs = 0.0, bs = bias ? (double)bias[n] : 0.0;
+        for (int k = 0; k < K; ++k) {
+            const uint32_t wb = (uint32_t)w[n * K + k] << 16;
+            float wf;
+            memcpy(&wf, &wb, 4);
+            bs += (double)wf * (double)shift[k];
+            const float p = wf * (1.0f + scale[k]);
+            uint32_t pb;
+            memcpy(&pb, &p, 4);
+            if ((pb & 0x7fffffffu) > 0x7f800000u) pb |= 0x00400000u;  // NaN stays NaN
+            else pb += 0x7fffu + ((pb >> 16) & 1u);                    // round to nearest even
+            pb &= 0xffff0000u;
+            ((uint16_t*)W_out)[n * K + k] = (uint16_t)(pb >> 16);
+            float rf;
+            memcpy(&rf, &pb, 4);
+            cs += (double)rf;
+        }
+        colsum_out[n] = (float)cs;
+        bias_out[n] = (float)bs;
+    }
+    return VLA_K_OK;
 }
 
 int vla_ternary_gemm(const int8_t* A, const uint32_t* W_packed, uint16_t* out, int32_t* acc_out, const float* s,

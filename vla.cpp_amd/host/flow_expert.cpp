@@ -88,6 +88,10 @@ struct LayerW {
     DevBuf ln;                  // expert pre-norm weight (RMS archs)
     DevBuf Wqkv, bqkv;          // self: Q|K|V rows, cross: Q rows
     DevBuf Wqkv_ln;             // the same rows with the pre-norm weight folded in (bf16 RMS archs)
+    // bf16 DiT blocks: per denoise step, the rows with (1 + scale) of the block's modulated
+    // LayerNorm folded in [steps][rows][W], their column sums and the bias with the shift
+    // folded in [steps][rows] (vla_layernorm_attn_qkv_rope)
+    DevBuf Wqkv_ada, cs_ada, b_ada;
     DevBuf Wo, bo;
     DevBuf ln2, Wgu, Wgu_ln, Wd;      // FFN half of an RMS-norm layer: post-attention norm, [gate; up], down
     DevBuf W1, b1, W2, b2;            // FFN half of a DiT block (ffn_gelu)
@@ -476,6 +480,51 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
             }
         }
         ada_.upload(ada.data(), ada.size() * sizeof(float));
+
+        if (dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !no_norm_fusion) {
+            // the modulation of a block depends on the step only: fold it into one operand set
+            // per step, and the pre-norm launch of the block disappears into its projection
+            const int nthr = std::min(default_cpu_threads(), L_);
+            std::vector<std::thread> pool;
+            std::vector<std::string> errors(nthr);
+            std::vector<std::vector<uint16_t>> folded(L_);
+            std::vector<std::vector<float>> cs(L_), bs(L_);
+            for (int t = 0; t < nthr; ++t)
+                pool.emplace_back([&, t]() {
+                    try {
+                        for (int l = t; l < L_; l += nthr) {
+                            LayerW& w = layers_[l];
+                            const std::string p = "ex." + std::to_string(l) + ".";
+                            const int64_t n_proj = w.is_self ? qd + 2 * kvd : qd;
+                            const std::vector<float> wf = host_f32(ck, p + (w.is_self ? "Wqkv" : "Wq"), {n_proj, W_});
+                            std::vector<float> bf;
+                            if (ck.has(p + (w.is_self ? "bqkv" : "bq"))) bf = host_f32(ck, p + (w.is_self ? "bqkv" : "bq"), {n_proj});
+                            std::vector<uint16_t> wb(wf.size());
+                            for (size_t i = 0; i < wf.size(); ++i) wb[i] = f32_to_bf16(wf[i]);
+                            folded[l].resize((size_t)steps_ * wf.size());
+                            cs[l].resize((size_t)steps_ * n_proj);
+                            bs[l].resize((size_t)steps_ * n_proj);
+                            for (int s = 0; s < steps_; ++s) {
+                                const float* sc = ada.data() + ((size_t)s * (L_ + 2) + l) * 2 * W_;
+                                VLA_K(vla_fold_adaln_weight_host(wb.data(), bf.empty() ? nullptr : bf.data(), sc, sc + W_, (int)n_proj, W_,
+                                                                 folded[l].data() + (size_t)s * wf.size(), cs[l].data() + (size_t)s * n_proj,
+                                                                 bs[l].data() + (size_t)s * n_proj));
+                            }
+                        }
+                    } catch (const std::exception& e) {
+                        errors[t] = e.what();
+                    }
+                });
+            for (auto& th : pool) th.join();
+            for (const std::string& e : errors)
+                if (!e.empty()) throw std::runtime_error(e);
+            for (int l = 0; l < L_; ++l) {  // device work stays on the loading thread
+                layers_[l].Wqkv_ada.upload(folded[l].data(), folded[l].size() * sizeof(uint16_t));
+                layers_[l].cs_ada.upload(cs[l].data(), cs[l].size() * sizeof(float));
+                layers_[l].b_ada.upload(bs[l].data(), bs[l].size() * sizeof(float));
+                std::vector<uint16_t>().swap(folded[l]);
+            }
+        }
     }
 }
 
@@ -737,6 +786,12 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 if (!done && w.Wqkv_ln) {
                     Tensor Wf = tensor_2d(w.Wqkv_ln.get(), dt_, W_, n_rows_w);
                     done = rmsnorm_qkv_rope_append(C, h, Wf, bq, eps_, S_, Hq_, w.is_self, w.is_self, tab, Q.data, w.kv, tok);
+                }
+                if (!done && w.Wqkv_ada) {
+                    Tensor Wf = tensor_2d(w.Wqkv_ada.as<uint16_t>() + (size_t)s * n_rows_w * W_, dt_, W_, n_rows_w);
+                    done = layernorm_qkv_rope_append(C, h, Wf, w.cs_ada.as<float>() + (size_t)s * n_rows_w,
+                                                     w.b_ada.as<float>() + (size_t)s * n_rows_w, eps_, S_, Hq_, w.is_self, w.is_self, tab,
+                                                     Q.data, w.kv, tok);
                 }
                 if (!done) {
                     if (arch_ == Arch::GR00T) {

@@ -175,6 +175,21 @@ inline bool rmsnorm_qkv_rope_append(Ctx& C, const Tensor& x, const Tensor& W_fol
     return true;
 }
 
+// A DiT block's modulated LayerNorm (norm.h:37-46) and the projection launch as one: x is
+// the un-normalised stream; W_folded, colsum and bias carry this step's (scale, shift)
+// (vla_fold_adaln_weight_host).  Returns false when the shapes do not fit the fused kernel.
+inline bool layernorm_qkv_rope_append(Ctx& C, const Tensor& x, const Tensor& W_folded, const float* colsum, const float* bias,
+                                      float eps, int S, int n_q_heads, bool has_k, bool has_v, const RopeTable* tab, void* q_out,
+                                      KVLayer& kv, int tok_offset) {
+    const int rc = vla_layernorm_attn_qkv_rope(x.data, W_folded.data, colsum, bias, x.dtype, (int)x.rows(), (int)x.ne[0], S,
+                                               n_q_heads, kv.n_kv_heads, has_k ? 1 : 0, has_v ? 1 : 0, kv.head_dim,
+                                               tab ? tab->cos.as<float>() : nullptr, tab ? tab->sin.as<float>() : nullptr,
+                                               q_out, kv.k.get(), kv.vt.get(), kv.t_max, tok_offset, eps, C.stream);
+    if (rc == VLA_K_ERR_SHAPE) return false;
+    VLA_K(rc);
+    return true;
+}
+
 // attn.h:48-58 (flash_attention) over the resident cache: Q [D, Hq, S, B]
 // token-major, keys [0, n_keys).
 inline void flash_attention(Ctx& C, const Tensor& Q, const KVLayer& kv, int n_keys, const MaskSpec& mask, float scale,
