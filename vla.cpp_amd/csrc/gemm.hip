@@ -177,7 +177,7 @@ template <typename T, int kEpi>
 __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t* C, int m0, int nt, const TileCols& tc,
                                                int tid, bool have_res = false, u32x4_t res_lo = u32x4_t{0u, 0u, 0u, 0u},
                                                u32x4_t res_hi = u32x4_t{0u, 0u, 0u, 0u}, int norm_mode = 0,
-                                               const float* row_scale = nullptr, const float* row_shift = nullptr) {
+                                               const float* row_stat = nullptr, int stat_stride = 0) {
     const int erow = tid >> 2, jg = (tid & 3) * 8;
     const int m = m0 + erow;
     if (m >= a.M) return;
@@ -210,21 +210,28 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
         lo[e] = __uint_as_float(crow[jg + e]);
         hi[e] = __uint_as_float(crow[32 + jg + e]);
     }
-    if (norm_mode) {  // row_scale: one factor per row of the sub-tile (in LDS)
-        const float f = row_scale[erow];
+    if (norm_mode) {
+        // row_stat: per row of the sub-tile (sum of squares, sum) of the A row, as two partial
+        // pairs stat_stride floats apart (one from each of the two wavefronts sharing the row)
+        const float inv_k = 1.0f / (float)a.K;
+        const float sq = row_stat[2 * erow] + row_stat[stat_stride + 2 * erow];
+        if (norm_mode == NORM_LAYER && kEpi == EPI_QKV) {
+            // sum_k (x - mean) rstd W[n][k] = rstd acc - (mean rstd) colsum[n]
+            const float mean = (row_stat[2 * erow + 1] + row_stat[stat_stride + 2 * erow + 1]) * inv_k;
+            const float f = rsqrtf(fmaxf(sq * inv_k - mean * mean, 0.f) + a.norm_eps);
+            const float ms = mean * f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            lo[e] *= f;
-            hi[e] *= f;
-        }
-    }
-    if (norm_mode == NORM_LAYER && kEpi == EPI_QKV) {
-        // sum_k (x - mean) rstd W[n][k] = rstd acc - (mean rstd) colsum[n]; row_shift = mean rstd
-        const float ms = row_shift[erow];
+            for (int e = 0; e < 8; ++e) {
+                lo[e] = lo[e] * f - ms * a.colsum[tc.base0 + jg + e];
+                hi[e] = hi[e] * f - ms * a.colsum[tc.base1 + jg + e];
+            }
+        } else {
+            const float f = rsqrtf(sq * inv_k + a.norm_eps);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            lo[e] -= ms * a.colsum[tc.base0 + jg + e];
-            hi[e] -= ms * a.colsum[tc.base1 + jg + e];
+            for (int e = 0; e < 8; ++e) {
+                lo[e] *= f;
+                hi[e] *= f;
+            }
         }
     }
 
@@ -655,7 +662,7 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     constexpr int NCH = KB / 32;        // 16-k MFMA chunks per tile
     constexpr int STAGE = (ROWS_A + ROWS_W) * KB;
     constexpr int C_BYTES = 4 * 64 * C_STRIDE;
-    constexpr int EPI_BYTES = C_BYTES + ROWS_A * 8;  // C sub-tile, then one scale and one shift per tile row (kNorm)
+    constexpr int EPI_BYTES = C_BYTES + ROWS_A * 16;  // C sub-tile, then two (sum of squares, sum) pairs per tile row (kNorm)
     constexpr int LDS_BYTES = NS * STAGE > EPI_BYTES ? NS * STAGE : EPI_BYTES;
     constexpr int IN_FLIGHT = (NS - 2) * NLOAD;  // loads younger than the tile about to be multiplied
     static_assert(KB == 128 || KB == 256, "swizzle is defined for 128- and 256-byte rows");
@@ -690,10 +697,14 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     // the MFMAs read (lane (g, r) sees 8 of every 16 k of its rows; the two halves meet
     // after the loop), two bf16 products per instruction.  NORM_LAYER also sums the values:
     // row m of the result becomes rstd (acc - mean colsum[n]), the projection of the
-    // centred and scaled row.
-    float ssq[TM], ssum[TM];
+    // centred and scaled row.  The two wavefronts that read the same A rows (wn = 0, 1)
+    // take alternate k-chunks, and each of a fragment's four words has its own
+    // accumulator, so a chunk adds one dependent operation per accumulator.
+    float ssq[TM][4], ssum[TM][4];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) ssq[i] = ssum[i] = 0.f;
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) ssq[i][e] = ssum[i][e] = 0.f;
 
     // A bf16 residual is fetched now, ahead of every operand load, instead of in the
     // epilogue where nothing is left to hide its latency (the epilogue thread layout:
@@ -774,13 +785,13 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[ch % SLOTS][i], fw[ch % SLOTS][j]);
-                if (kNorm) {
+                if (kNorm && (ch & 1) == wn) {
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            ssq[i] = add_squares_bf16x2(fa[ch % SLOTS][i][e], ssq[i]);
-                            if (kNorm == NORM_LAYER) ssum[i] = add_pair_bf16x2(fa[ch % SLOTS][i][e], ssum[i]);
+                            ssq[i][e] = add_squares_bf16x2(fa[ch % SLOTS][i][e], ssq[i][e]);
+                            if (kNorm == NORM_LAYER) ssum[i][e] = add_pair_bf16x2(fa[ch % SLOTS][i][e], ssum[i][e]);
                         }
                 }
             }
@@ -814,22 +825,18 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     __syncthreads();
 
     uint32_t* C = reinterpret_cast<uint32_t*>(lds);
-    float* row_scale = reinterpret_cast<float*>(lds + C_BYTES);
-    float* row_shift = row_scale + ROWS_A;
+    float* row_stat = reinterpret_cast<float*>(lds + C_BYTES);  // [wn][ROWS_A][2]
     if (kNorm) {
-        const float inv_k = 1.0f / (float)a.K;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
-            const float t = ssq[i] + __shfl_xor(ssq[i], 32, 64);
-            if (kNorm == NORM_LAYER) {
-                const float mean = (ssum[i] + __shfl_xor(ssum[i], 32, 64)) * inv_k;
-                const float rstd = rsqrtf(fmaxf(t * inv_k - mean * mean, 0.f) + a.norm_eps);
-                if (wn == 0 && g == 0) {
-                    row_scale[(wm + 2 * i) * 32 + r] = rstd;
-                    row_shift[(wm + 2 * i) * 32 + r] = mean * rstd;
-                }
-            } else if (wn == 0 && g == 0) {
-                row_scale[(wm + 2 * i) * 32 + r] = rsqrtf(t * inv_k + a.norm_eps);
+            float q = (ssq[i][0] + ssq[i][1]) + (ssq[i][2] + ssq[i][3]);
+            float u = (ssum[i][0] + ssum[i][1]) + (ssum[i][2] + ssum[i][3]);
+            q += __shfl_xor(q, 32, 64);
+            u += __shfl_xor(u, 32, 64);
+            if (g == 0) {
+                float* dst = row_stat + (wn * ROWS_A + (wm + 2 * i) * 32 + r) * 2;
+                dst[0] = q;
+                dst[1] = u;
             }
         }
     }
@@ -847,7 +854,7 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
             const int nt_sub = ntw * TN + j;
             if (nt_sub < a.n_tiles)
                 epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0], res_pf[i][j][1], kNorm,
-                                        row_scale + i * 64, row_shift + i * 64);
+                                        row_stat + i * 128, ROWS_A * 2);
         }
 }
 
@@ -1298,6 +1305,9 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             // per multiply); else 128x64 tiles if those fill it; else 64x64 tiles, with
             // 256-byte K rows (half the barriers per K) while one workgroup per CU covers them.
             cfg = wgs0 >= 128 ? 0 : (wgs2 >= 150 ? 2 : (wgs4 <= 256 ? 1 : 4));
+            // 128x128 tiles that leave more than a third of the CUs idle lose to 128x64 tiles
+            // that cover the chip in little more than one round (pi0's fused QKV: 140 -> 280)
+            if (cfg == 0 && wgs0 < 160 && wgs2 <= 288) cfg = 2;
             // Between one and one and a half rounds of 128x128 tiles, some CUs would run two
             // workgroups while the rest run one; 128x192 tiles cover the same grid in a single
             // round of 1.5x workgroups (GR00T's fused QKV: 324 -> 216 workgroups).
