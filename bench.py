@@ -328,14 +328,20 @@ def kernel_breakdown(pkg, cfg, B, P):
 # inside the process, so these are the figures of profiles/*_pmc.txt (which give the commands);
 # launch sites without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg1_smolvla_16layer_bf16_b32", "step.wo_residual"): int((7821.0 * 2 + 2250.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.qkv_rope_append_self"): int((6934.0 * 2 + 5400.1) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.q_rope_cross"): int((5072.5 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_self"): int((7734.6 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_cross"): int((6592.0 * 2 + 3000.0) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "step.attention_cross"): int((62789.0 * 2 + 3351.8) * 1024),
-    ("cfg4_bitvla_30layer_b8", "prefill.ternary_qkv_gemm"): int((16895.0 * 2 + 30720.0) * 1024),
-    ("cfg4_bitvla_30layer_b8", "step.attention"): int((7005.5 * 2 + 1016.2) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.wo_residual"): int((7807.5 * 2 + 2250.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.qkv_rope_append_self"): int((6935.3 * 2 + 5400.2) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.q_rope_cross"): int((5076.5 * 2 + 3000.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_self"): int((7725.2 * 2 + 3000.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_cross"): int((6582.0 * 2 + 3000.0) * 1024),
+    ("cfg2_pi0_18layer_bf16_b16", "step.attention_self"): int((8793.0 * 2 + 13260.0) * 1024),
+    ("cfg2_pi0_18layer_bf16_b16", "step.qkv_rope_append_self"): int((9220.3 * 2 + 4184.0) * 1024),
+    ("cfg2_pi0_18layer_bf16_b16", "step.wo_residual"): int((11532.0 * 2 + 1632.0) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "step.attention_cross"): int((62538.6 * 2 + 3368.6) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "step.qkv_rope_append_self"): int((20186.8 * 2 + 12788.2) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "step.q_rope_cross"): int((11234.1 * 2 + 3264.0) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "step.wo_residual"): int((12906.6 * 2 + 3264.0) * 1024),
+    ("cfg4_bitvla_30layer_b8", "prefill.ternary_qkv_gemm"): int((22033.0 * 2 + 30720.0) * 1024),
+    ("cfg4_bitvla_30layer_b8", "step.attention"): int((6979.2 * 2 + 1016.2) * 1024),
 }
 
 

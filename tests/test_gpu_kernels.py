@@ -324,8 +324,9 @@ def test_rmsnorm_inside_qkv_launch(name, B, S, Hq, Hkv, D, K, self_layer, P):
 
 
 @pytest.mark.parametrize("name,B,S,Hq,Hkv,D,K,self_layer,bias", [
-    ("gr00t-self", 3, 17, 24, 24, 64, 1536, True, True),
-    ("gr00t-cross-q", 64, 17, 24, 24, 64, 1536, False, True),
+    ("gr00t-self", 3, 17, 32, 32, 48, 1536, True, True),
+    ("gr00t-cross-q", 64, 17, 32, 32, 48, 1536, False, True),
+    ("64-wide-heads", 2, 17, 24, 24, 64, 1536, True, True),
     ("small-no-bias", 2, 5, 2, 2, 64, 48, True, False),
     ("partial-row-tile", 1, 33, 4, 4, 64, 272, False, True),
 ])
