@@ -529,6 +529,18 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir, isolated=False):
     wall_ms = (time.perf_counter() - t0) * 1e3
     dev_ms = e0.elapsed_time(e1)
     ms_per_step = max(dev_ms, wall_ms) / steps  # the host-inclusive figure when the host is the slower side
+    # the reference bench's recipe on the GPU side as well: whole chunks one at a time,
+    # 3 warm-ups, 20 repetitions, min / p50 / p90 (src/serving/vla-bench.cpp:159-195)
+    reps = []
+    for i in range(23):
+        c0, c1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        c0.record()
+        m.denoise_steps_async(spc, stream)
+        c1.record()
+        torch.cuda.synchronize()
+        if i >= 3:
+            reps.append(c0.elapsed_time(c1) * 1e3)
+    chunk_us = dict(min=round(min(reps), 1), p50=round(pct(reps, 0.5), 1), p90=round(pct(reps, 0.9), 1), warmups=3, repetitions=20)
     # one more chunk with an event after every launch
     m.profile_begin()
     m.denoise_steps_async(spc, stream)
@@ -557,6 +569,7 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir, isolated=False):
     res = dict(
         workload=name, batch=B, us_per_denoise_step=round(ms_per_step * 1e3, 2),
         us_per_action_chunk=round(ms_per_step * 1e3 * spc, 1), steps_per_chunk=spc, timed_steps=steps,
+        action_chunk_us=chunk_us,
         device_us_per_step=round(dev_ms * 1e3 / steps, 2), host_us_per_step=round(wall_ms * 1e3 / steps, 2),
         prefix_kv_build_ms=round(prefill_ms, 2),
         sum_launch_us_per_step=round(sum(v["us"] * v["launches"] for v in prof.values()) / spc, 2),
@@ -650,7 +663,7 @@ def main():
         "config": {"workload": args.config, "batch": wl[args.config]["B"], "n_layers": cfg["n_layers"],
                    "prefix_tokens_resident": True, "step": "one denoise step over all expert layers",
                    "timed_region": "graph replays in steady state (3 whole chunks + warmup steps run before it)"},
-        "us_per_action_chunk": main_res["us_per_action_chunk"],
+        "us_per_action_chunk": main_res["us_per_action_chunk"], "action_chunk_us": main_res["action_chunk_us"],
         "roofline": main_res["roofline"], "roofline_kv": main_res["roofline_kv"],
         "cpu_baseline": main_res.get("cpu_baseline"),
         "kernels": main_res["kernels"], "prefill_kernels": main_res["prefill_kernels"],

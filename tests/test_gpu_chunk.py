@@ -204,8 +204,16 @@ def test_whole_layers_with_the_ffn_half(tmp_path, arch, dtype, n_layers, ffn_dim
             want = orc_chunk.flow_expert_chunk(cfg, w, obs[b])
             assert rel_err(got[b], want) < 1e-5, rel_err(got[b], want)
         else:
-            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+            # the bar is against the fp32 oracle.  The bf16-emulating oracle rounds where the
+            # two-launch path rounds (normalised activations), the fused launches round elsewhere
+            # (folded weights): both are bf16-noisy estimates of the same chunk (the emulating
+            # oracle itself sits 0.008 from the fp32 one here), so between them only the mean
+            # error and twice the bar are held.
+            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b])
             assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+            emu = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+            d = np.abs(got[b] - emu)
+            assert d.mean() < 4e-3 and np.all(d <= 2e-2 + 4e-2 * np.abs(emu)), (d.mean(), d.max())
     # without the FFN weights the same observation gives a different chunk: the half is really run
     cfg0 = dict(cfg, ffn_dim=0)
     assert not np.allclose(orc_chunk.flow_expert_chunk(cfg0, w, obs[0], emulate_bf16=dtype != "f32"), got[0], atol=1e-3)
