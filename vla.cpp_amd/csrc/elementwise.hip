@@ -320,38 +320,51 @@ __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restri
                                                             const float* __restrict__ bias_step,
                                                             const float* __restrict__ lead, T* __restrict__ h, int n_rows,
                                                             int S, int n_lead, int A, int W, int act) {
-    __shared__ float xs[EMB_ROWS][EMB_MAX_A];
-    __shared__ float ws[EMB_COLS][EMB_MAX_A + 1];
+    // rows padded to a multiple of four floats: every a-loop step below is one 16-byte LDS read
+    // of the thread's weight row (row stride 68 floats: 16 lanes cover all 64 banks once) and one
+    // 16-byte broadcast read per output row, 9 LDS instructions per 32 multiply-adds
+    __shared__ __attribute__((aligned(16))) float xs[EMB_ROWS][EMB_MAX_A];
+    __shared__ __attribute__((aligned(16))) float ws[EMB_COLS][EMB_MAX_A + 4];
     const int row0 = blockIdx.x * EMB_ROWS, c0 = blockIdx.y * EMB_COLS;
     const int ncol = min(EMB_COLS, W - c0);
-    for (int i = threadIdx.x; i < EMB_ROWS * A; i += blockDim.x) {
-        const int rr = i / A, a = i % A, row = row0 + rr;
+    const int A4 = (A + 3) & ~3;
+    for (int i = threadIdx.x; i < EMB_ROWS * A4; i += blockDim.x) {
+        const int rr = i / A4, a = i % A4, row = row0 + rr;
         float v = 0.f;
-        if (row < n_rows) {
+        if (row < n_rows && a < A) {
             const int b = row / S, s = row % S;
             if (s >= n_lead) v = x_t[((long)b * (S - n_lead) + (s - n_lead)) * A + a];
         }
         xs[rr][a] = v;
     }
-    for (int i = threadIdx.x; i < ncol * A; i += blockDim.x) ws[i / A][i % A] = W_in[(long)c0 * A + i];
+    for (int i = threadIdx.x; i < EMB_COLS * A4; i += blockDim.x) {
+        const int cc = i / A4, a = i % A4;
+        ws[cc][a] = (cc < ncol && a < A) ? W_in[(long)(c0 + cc) * A + a] : 0.f;
+    }
     const int cl = threadIdx.x & 63, rq = threadIdx.x >> 6;  // column in slab, row residue mod 4
     const int c = c0 + cl;
     const float bias = c < W ? bias_step[c] : 0.f;
     __syncthreads();
     if (c >= W) return;
+    constexpr int NR = EMB_ROWS / 4;
+    float acc[NR];
 #pragma unroll
-    for (int k = 0; k < EMB_ROWS / 4; ++k) {
+    for (int k = 0; k < NR; ++k) acc[k] = 0.f;
+    for (int a = 0; a < A4; a += 4) {  // products added in the order of a, as a scalar loop would
+        const f32x4_t w4 = *reinterpret_cast<const f32x4_t*>(&ws[cl][a]);
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            const f32x4_t x4 = *reinterpret_cast<const f32x4_t*>(&xs[rq + 4 * k][a]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[k] += w4[e] * x4[e];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
         const int rr = rq + 4 * k, row = row0 + rr;
         if (row >= n_rows) continue;
         const int b = row / S, s = row % S;
-        float v;
-        if (s < n_lead) {
-            v = lead[((long)b * n_lead + s) * W + c];
-        } else {
-            float acc = 0.f;
-            for (int a = 0; a < A; ++a) acc += ws[cl][a] * xs[rr][a];
-            v = apply_act(acc + bias, act);
-        }
+        const float v = s < n_lead ? lead[((long)b * n_lead + s) * W + c] : apply_act(acc[k] + bias, act);
         Elem<T>::store(h + (long)row * W + c, v);
     }
 }
