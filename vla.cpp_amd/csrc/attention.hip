@@ -148,6 +148,8 @@ template <> struct AT<float> {
 // has NW x NSL wavefronts: NSL key slices per row tile, slice sl taking tiles sl, sl + NSL,
 // ... of the workgroup's key range; a step multiplies NSL tiles at once and the slices'
 // partial (max, sum, output) meet in LDS at the end.  RS step slots form the ring.
+constexpr int WIDE_FB = 4;  // LDS fragments read ahead of their MFMAs, 256-wide heads (8 spills registers)
+
 template <typename T, int D, int NW, bool P2, int NL, int NSL = 0, int RS = 1>
 __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * sizeof(T) <= 128) ? 2 : 1) attn_kernel(AttnArgs a) {
     typedef AT<T> A;
@@ -329,18 +331,30 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         for (int kb = 0; kb < NKB; ++kb) {
             // the head_dim contraction runs as NA independent MFMA chains (a single chain of
             // NQ dependent MFMAs is latency-bound for wide heads), summed at the end
-            constexpr int NA = (NQ >= 4 && NKB == 1) ? 2 : 1;
+            // fragments are read FB at a time ahead of their MFMAs: a read per MFMA leaves every
+            // MFMA waiting for the LDS latency, and for 256-wide heads the register allocator
+            // otherwise keeps only two fragments in flight (the second accumulator chain is
+            // given up for the fragment registers there)
+            constexpr int FB = (NQ >= 16 && !DLOAD) ? WIDE_FB : 1;
+            constexpr int NA = (NQ >= 4 && NKB == 1 && FB == 1) ? 2 : 1;
             f32x16_t sc[NA];
 #pragma unroll
             for (int n = 0; n < NA; ++n)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) sc[n][i] = 0.f;
 #pragma unroll
-            for (int c = 0; c < NQ; ++c) {
-                const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(
-                    DLOAD ? ldsK + kb * 32 * KROW + kfrag + (((2 * c) ^ kx) * 16)
-                          : ldsK + (kb * 32 + key_of_score_row(r)) * KS + (c * CE + g * (CE / 2)) * EB);
-                A::mma(sc[c % NA], kf, qf[c]);
+            for (int c0 = 0; c0 < NQ; c0 += FB) {
+                u32x4_t kf[FB];
+#pragma unroll
+                for (int f = 0; f < FB; ++f) {
+                    const int c = c0 + f;
+                    kf[f] = *reinterpret_cast<const u32x4_t*>(
+                        DLOAD ? ldsK + kb * 32 * KROW + kfrag + (((2 * c) ^ kx) * 16)
+                              : ldsK + (kb * 32 + key_of_score_row(r)) * KS + (c * CE + g * (CE / 2)) * EB);
+                }
+                if (FB > 1) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int f = 0; f < FB; ++f) A::mma(sc[(c0 + f) % NA], kf[f], qf[c0 + f]);
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -429,16 +443,28 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
                     }
                     const int key_off = (kb * 32 + hh * 16 + 8 * g) * EB;
                     const int nvalid = a.n_keys - (k0 + kb * 32 + hh * 16 + 8 * g);  // real keys among this lane's 8
+                    // (256-wide heads: VB of a half tile's V^T fragments are read ahead of their
+                    // MFMAs, as for the K fragments)
+                    constexpr int VB = (NDB >= 8 && !DLOAD) ? WIDE_FB : 1;
 #pragma unroll
-                    for (int db = 0; db < NDB; ++db) {
-                        u32x4_t vf = *reinterpret_cast<const u32x4_t*>(
-                            DLOAD ? ldsV + db * 32 * VROW + vfrag + (((4 * kb + 2 * hh) ^ vx) * 16) : ldsV + (db * 32 + r) * VS + key_off);
-                        if (v_partial) {
+                    for (int d0 = 0; d0 < NDB; d0 += VB) {
+                        u32x4_t vf[VB];
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) vf[e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+                        for (int f = 0; f < VB; ++f) {
+                            const int db = d0 + f;
+                            vf[f] = *reinterpret_cast<const u32x4_t*>(
+                                DLOAD ? ldsV + db * 32 * VROW + vfrag + (((4 * kb + 2 * hh) ^ vx) * 16) : ldsV + (db * 32 + r) * VS + key_off);
                         }
-                        A::mma(o[db], vf, pf);
-                        if (P2) A::mma(o[db], vf, pl);
+                        if (VB > 1) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int f = 0; f < VB; ++f) {
+                            if (v_partial) {
+#pragma unroll
+                                for (int e = 0; e < 4; ++e) vf[f][e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+                            }
+                            A::mma(o[d0 + f], vf[f], pf);
+                            if (P2) A::mma(o[d0 + f], vf[f], pl);
+                        }
                     }
                 }
             } else {
@@ -577,18 +603,32 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
             };
             // V^T elements past n_keys are zeroed so that stale cache contents (possibly NaN)
             // cannot reach the accumulators.
+            // Only the tile that reaches past n_keys is masked, under a uniform branch: masking
+            // every tile lets the compiler gather the mask arithmetic of all slots at the top of
+            // the unrolled loop, in front of a wait for every load in flight -- the youngest
+            // fetch included, which is the look-ahead gone.
             auto publish = [&](int slot, int t, int stage) __attribute__((always_inline)) {
                 const int k0 = k_begin + max(min(t, n_t - 1), 0) * TK;
+                if (k0 + TK <= a.n_keys) {
 #pragma unroll
-                for (int i = 0; i < ITL; ++i) {
-                    const int v = lt + i * NTL;
-                    *reinterpret_cast<u32x4_t*>(ldsK_buf[stage] + (v / KV_PER_ROW) * KS + (v % KV_PER_ROW) * 16) = kq[slot][i];
-                    const int nvalid = a.n_keys - (k0 + (v % VV_PER_ROW) * EPV);  // real keys among the 8, may be <= 0
-                    u32x4_t val = vq[slot][i];
+                    for (int i = 0; i < ITL; ++i) {
+                        const int v = lt + i * NTL;
+                        *reinterpret_cast<u32x4_t*>(ldsK_buf[stage] + (v / KV_PER_ROW) * KS + (v % KV_PER_ROW) * 16) = kq[slot][i];
+                        *reinterpret_cast<u32x4_t*>(ldsV_buf[stage] + (v / VV_PER_ROW) * VS + (v % VV_PER_ROW) * 16) = vq[slot][i];
+                    }
+                } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) val[e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
-                    *reinterpret_cast<u32x4_t*>(ldsV_buf[stage] + (v / VV_PER_ROW) * VS + (v % VV_PER_ROW) * 16) = val;
+                    for (int i = 0; i < ITL; ++i) {
+                        const int v = lt + i * NTL;
+                        *reinterpret_cast<u32x4_t*>(ldsK_buf[stage] + (v / KV_PER_ROW) * KS + (v % KV_PER_ROW) * 16) = kq[slot][i];
+                        const int nvalid = a.n_keys - (k0 + (v % VV_PER_ROW) * EPV);  // real keys among the 8, may be <= 0
+                        u32x4_t val = vq[slot][i];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) val[e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+                        *reinterpret_cast<u32x4_t*>(ldsV_buf[stage] + (v / VV_PER_ROW) * VS + (v % VV_PER_ROW) * 16) = val;
+                    }
                 }
+                __builtin_amdgcn_sched_barrier(0);
             };
 #pragma unroll
             for (int sl = 0; sl < LOAD_AHEAD; ++sl) fetch(sl, sl);
@@ -660,6 +700,59 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         }
     }
 
+    if constexpr (NL > 0) {
+        // Wide heads: the rows leave through LDS.  A lane holds 4 consecutive d of its query row
+        // per (block, j): written from the registers that is 8-byte pieces of 32 different rows
+        // per instruction (3.3 us of a 12.6 us launch at 83 keys).  Each computing wavefront
+        // parks its 32 x D tile (bf16 outputs, or fp16 partials) in one of the K / V^T tile
+        // buffers -- every wavefront is past the loop's last barrier, nobody reads them any
+        // more, and a buffer holds exactly one 32-row tile -- and writes whole 512-byte rows,
+        // two per instruction.
+        if (wave >= NW) return;  // loader wavefronts own no rows
+        constexpr int ROWB = D * 2 + 16;  // staged row: D 16-bit values + padding
+        static_assert(TK * KS >= 32 * ROWB && DP * VS >= 32 * ROWB && NW <= 4, "a tile buffer parks one wavefront's rows");
+        const bool as_partial = a.n_split > 1;
+        if (!as_partial || a.part_half) {
+            unsigned char* park = wave < 2 ? ldsK_buf[wave] : ldsV_buf[wave - 2];
+            const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+            const long prow = as_partial ? ((long)pair * a.n_split + split) * a.r_pad + row : 0;
+            if (as_partial && row_valid && g == 0) {
+                a.part_ml[prow * 2] = m_run;
+                a.part_ml[prow * 2 + 1] = l_run;
+            }
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int d = db * 32 + 8 * j + 4 * g;
+                    const float v0 = o[db][4 * j] * inv_l, v1 = o[db][4 * j + 1] * inv_l, v2 = o[db][4 * j + 2] * inv_l,
+                                v3 = o[db][4 * j + 3] * inv_l;
+                    u32x2_t pk;
+                    if (as_partial) {
+                        typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+                        const h4_t hv = {(_Float16)v0, (_Float16)v1, (_Float16)v2, (_Float16)v3};
+                        pk = __builtin_bit_cast(u32x2_t, hv);
+                    } else {
+                        pk = u32x2_t{pack_bf2(v0, v1), pack_bf2(v2, v3)};
+                    }
+                    *reinterpret_cast<u32x2_t*>(park + r * ROWB + d * 2) = pk;
+                }
+            // destination of tile row rr, in 16-bit elements (-1: no such row), from the lane that owns it
+            long dst = -1;
+            if (row_valid && g == 0) dst = as_partial ? prow * D : (((long)b * a.S + s) * a.Hq + h) * D;
+            const int dst_lo = (int)(dst & 0xffffffffl), dst_hi = (int)(dst >> 32);
+            unsigned short* base16 = as_partial ? reinterpret_cast<unsigned short*>(a.part_o) : reinterpret_cast<unsigned short*>(a.out);
+            constexpr int PIECES = D * 2 / 16, RPI = 64 / PIECES;  // 16-byte pieces per row, rows per instruction
+#pragma unroll
+            for (int i = 0; i < 32 / RPI; ++i) {
+                const int rr = i * RPI + lane / PIECES, pc = lane % PIECES;
+                const long d64 = ((long)__shfl(dst_hi, rr, 64) << 32) | (unsigned int)__shfl(dst_lo, rr, 64);
+                const u32x4_t val = *reinterpret_cast<const u32x4_t*>(park + rr * ROWB + pc * 16);
+                if (d64 >= 0) *reinterpret_cast<u32x4_t*>(base16 + d64 + pc * 8) = val;
+            }
+            return;
+        }
+    }
     if (!row_valid) return;
     if (a.n_split > 1) {
         // unnormalised partial for the merge kernel
