@@ -939,7 +939,10 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
     const int h = hk * grp + hg;
 
     const int nb_total = (a.n_keys + 31) / 32;
-    const int kb0 = split * a.tiles_per_split, kb1 = min(nb_total, kb0 + a.tiles_per_split);
+    // the slice's block range is the same for every lane of the wavefront; said so explicitly
+    // (it is derived from the wavefront's index), the loop below runs on scalar branches
+    const int kb0 = __builtin_amdgcn_readfirstlane(split * a.tiles_per_split);
+    const int kb1 = __builtin_amdgcn_readfirstlane(min(nb_total, kb0 + a.tiles_per_split));
 
     u32x4_t qf[NQ];
     {
@@ -970,21 +973,16 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
 #pragma unroll
     for (int db = 0; db < NDB; ++db) vrow[db] = vbase + ((long)min(db * 32 + r, D - 1) * a.t_max + 8 * g) * EB;
     const int krow = key_of_score_row(r);  // the key of the block this lane fetches for the score product
-    auto load_full = [&](int st, int kb) __attribute__((always_inline)) {  // no checks at all
-        const unsigned char* kp = kbase + (long)(kb * 32 + krow) * D * EB + g * 16;
-#pragma unroll
-        for (int c = 0; c < NQ; ++c) kr[st][c] = *reinterpret_cast<const u32x4_t*>(kp + c * CE * EB);
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int hh = 0; hh < 2; ++hh) vr[st][db][hh] = *reinterpret_cast<const u32x4_t*>(vrow[db] + (kb * 32 + hh * 16) * EB);
-    };
-    // A partial block: K rows past n_keys repeat the last key (their scores are masked) and
-    // V^T runs past n_keys are not read.  mask_partial, called once the data is needed,
-    // zeroes the V^T elements past n_keys so that stale cache contents (possibly NaN)
-    // cannot reach the accumulators; keeping it apart from the loads keeps the wait for
-    // them out of the way of the loads issued next.
-    auto load_partial = [&](int st, int kb) __attribute__((always_inline)) {
+    // One block of loads, the same seven instructions for every block, with no branch around
+    // any of them: the compiler's count of loads in flight is then exact, and the wait in
+    // front of a block's arithmetic leaves the younger blocks' loads in flight (with the
+    // loads under branches it waited for all of them: the look-ahead was on paper only).
+    // K rows past n_keys repeat the last key (their scores are masked); V^T runs past n_keys
+    // stay inside the cache row (t_max is a multiple of 64) and are zeroed by mask_partial
+    // once the data is needed, so that stale cache contents (possibly NaN) cannot reach the
+    // accumulators.  Blocks past the slice repeat its last block and are never multiplied.
+    auto load_blk = [&](int st, int kb_any) __attribute__((always_inline)) {
+        const int kb = min(kb_any, kb1 - 1);
         const int key = min(kb * 32 + krow, a.n_keys - 1);
         const unsigned char* kp = kbase + (long)key * D * EB + g * 16;
 #pragma unroll
@@ -992,13 +990,7 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh) {
-                const int k8 = kb * 32 + hh * 16 + 8 * g;  // first of 8 consecutive keys
-                u32x4_t val = {0u, 0u, 0u, 0u};
-                // n_keys <= t_max and t_max is a multiple of 8: a group starting below n_keys is inside the row
-                if (k8 < a.n_keys) val = *reinterpret_cast<const u32x4_t*>(vrow[db] + (kb * 32 + hh * 16) * EB);
-                vr[st][db][hh] = val;
-            }
+            for (int hh = 0; hh < 2; ++hh) vr[st][db][hh] = *reinterpret_cast<const u32x4_t*>(vrow[db] + (kb * 32 + hh * 16) * EB);
     };
     auto mask_partial = [&](int st, int kb) __attribute__((always_inline)) {
 #pragma unroll
@@ -1088,26 +1080,31 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
 
     // Software pipeline over the slice's blocks [kb0, kb1) in key order: ST - 1 blocks of
     // loads stay in flight ahead of the block being multiplied.  Only the slice that reaches
-    // n_keys can end in a partial block; it takes the checked loads and, being last, shares
-    // its V^T cache lines with the full block fetched just before it.  The conditions in
-    // the loop are uniform over the wavefront (scalar branches).
+    // n_keys can end in a partial block.  The conditions in the loop are uniform over the
+    // wavefront (scalar branches) and none of them guards a load.
     const bool has_partial = kb1 * 32 > a.n_keys;
     const int kbp = has_partial ? kb1 - 1 : -1;  // the partial block, if any
-    auto load_any = [&](int st, int kb) __attribute__((always_inline)) {
-        if (kb == kbp) load_partial(st, kb);
-        else if (kb < kb1) load_full(st, kb);
-    };
+    if (kb1 - kb0 < ST) {
+        // a slice shorter than the pipeline (GR00T's 17-key self attention is one block): the
+        // pipeline's repeats of the last block would be most of its loads
+        for (int kb = kb0; kb < kb1; ++kb) {
+            load_blk(0, kb);
+            if (kb == kbp) mask_partial(0, kb);
+            compute(0, kb);
+        }
+    } else {
 #pragma unroll
-    for (int i = 0; i < ST - 1; ++i) load_any(i, kb0 + i);
-    for (int base = kb0; base < kb1; base += ST) {
+        for (int i = 0; i < ST - 1; ++i) load_blk(i, kb0 + i);
+        for (int base = kb0; base < kb1; base += ST) {
 #pragma unroll
-        for (int st = 0; st < ST; ++st) {
-            const int cur = base + st;
-            load_any((st + ST - 1) % ST, cur + ST - 1);
-            __builtin_amdgcn_sched_barrier(0);  // loads stay above the math they hide behind
-            if (cur < kb1) {
-                if (cur == kbp) mask_partial(st, cur);
-                compute(st, cur);
+            for (int st = 0; st < ST; ++st) {
+                const int cur = base + st;
+                load_blk((st + ST - 1) % ST, cur + ST - 1);
+                __builtin_amdgcn_sched_barrier(0);  // loads stay above the math they hide behind
+                if (cur < kb1) {
+                    if (cur == kbp) mask_partial(st, cur);
+                    compute(st, cur);
+                }
             }
         }
     }
