@@ -103,11 +103,16 @@ def time_events(fn, iters, warm=3):
     torch stream; `iters` calls are captured into one HIP graph and the graph is
     replayed between two events, so host launch overhead is not in the figure."""
     import torch
-    for i in range(warm):
-        fn(i)
+    # warm up on the stream the capture will use: the library keeps its scratch per (device,
+    # stream) and may not allocate while a stream is being captured
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(warm):
+            fn(i)
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
+    with torch.cuda.graph(g, stream=side):
         for i in range(iters):
             fn(i)
     g.replay()

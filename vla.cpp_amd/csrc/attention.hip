@@ -484,6 +484,53 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         }
     };
 
+    // The rows leave through LDS.  A lane holds 4 consecutive d of its query row per (block, j):
+    // written from the registers that is 8-byte pieces of 32 different rows per instruction
+    // (3.3 us of a 12.6 us launch for 256-wide heads at 83 keys).  The wavefront parks its
+    // 32 x D tile (bf16 outputs, or fp16 partials of a key slice) in `park`, LDS nobody else
+    // touches any more, and writes whole rows, 64 lanes x 16 bytes per instruction.
+    auto flush_rows = [&](unsigned char* park) __attribute__((always_inline)) {
+        constexpr int ROWB = D * 2 + 16;  // staged row: D 16-bit values + padding
+        const bool as_partial = a.n_split > 1;
+        const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+        const long prow = as_partial ? ((long)pair * a.n_split + split) * a.r_pad + row : 0;
+        if (as_partial && row_valid && g == 0) {
+            a.part_ml[prow * 2] = m_run;
+            a.part_ml[prow * 2 + 1] = l_run;
+        }
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int d = db * 32 + 8 * j + 4 * g;
+                if (d >= D) continue;
+                const float v0 = o[db][4 * j] * inv_l, v1 = o[db][4 * j + 1] * inv_l, v2 = o[db][4 * j + 2] * inv_l,
+                            v3 = o[db][4 * j + 3] * inv_l;
+                u32x2_t pk;
+                if (as_partial) {
+                    typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+                    const h4_t hv = {(_Float16)v0, (_Float16)v1, (_Float16)v2, (_Float16)v3};
+                    pk = __builtin_bit_cast(u32x2_t, hv);
+                } else {
+                    pk = u32x2_t{pack_bf2(v0, v1), pack_bf2(v2, v3)};
+                }
+                *reinterpret_cast<u32x2_t*>(park + r * ROWB + d * 2) = pk;
+            }
+        // destination of tile row rr, in 16-bit elements (-1: no such row), from the lane that owns it
+        long dst = -1;
+        if (row_valid && g == 0) dst = as_partial ? prow * D : (((long)b * a.S + s) * a.Hq + h) * D;
+        const int dst_lo = (int)(dst & 0xffffffffl), dst_hi = (int)(dst >> 32);
+        unsigned short* base16 = as_partial ? reinterpret_cast<unsigned short*>(a.part_o) : reinterpret_cast<unsigned short*>(a.out);
+        constexpr int PIECES = D * 2 / 16, RPI = 64 / PIECES;  // 16-byte pieces per row, rows per instruction
+#pragma unroll
+        for (int i = 0; i < 32 / RPI; ++i) {
+            const int rr = i * RPI + lane / PIECES, pc = lane % PIECES;
+            const long d64 = ((long)__shfl(dst_hi, rr, 64) << 32) | (unsigned int)__shfl(dst_lo, rr, 64);
+            const u32x4_t val = *reinterpret_cast<const u32x4_t*>(park + rr * ROWB + pc * 16);
+            if (d64 >= 0) *reinterpret_cast<u32x4_t*>(base16 + d64 + pc * 8) = val;
+        }
+    };
+
     if constexpr (DLOAD) {
         constexpr int KI = KTILE / 1024, VI = VTILE / 1024;   // load instructions (1 KiB each) per K / V^T tile
         constexpr int PER_STEP = NSL * (KI + VI);
@@ -527,6 +574,12 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         // step st into the slot step st - 1 has just been read from.
 #pragma unroll
         for (int st = 0; st < RS; ++st) issue_step(st, st);
+        // The query fragments are ordinary loads, the ring's are inline assembly the compiler
+        // does not count: left to itself it waits for the fragments at their first use, inside
+        // the loop, with vmcnt(0) -- which also drains every ring load in flight, at every step.
+        // Using them here puts that wait in front of the loop, once.
+#pragma unroll
+        for (int c = 0; c < NQ; ++c) asm volatile("" ::"v"(qf[c]));
         int slot = 0, lslot = RS - 1;
         for (int st = 0; st < n_steps; ++st) {
             // own loads of this step have landed (the younger ones may be pending) ...
@@ -701,55 +754,12 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
     }
 
     if constexpr (NL > 0) {
-        // Wide heads: the rows leave through LDS.  A lane holds 4 consecutive d of its query row
-        // per (block, j): written from the registers that is 8-byte pieces of 32 different rows
-        // per instruction (3.3 us of a 12.6 us launch at 83 keys).  Each computing wavefront
-        // parks its 32 x D tile (bf16 outputs, or fp16 partials) in one of the K / V^T tile
-        // buffers -- every wavefront is past the loop's last barrier, nobody reads them any
-        // more, and a buffer holds exactly one 32-row tile -- and writes whole 512-byte rows,
-        // two per instruction.
+        // every wavefront is past the loop's last barrier: nobody reads the K / V^T tile buffers
+        // any more, and a buffer holds exactly one wavefront's 32-row tile
         if (wave >= NW) return;  // loader wavefronts own no rows
-        constexpr int ROWB = D * 2 + 16;  // staged row: D 16-bit values + padding
-        static_assert(TK * KS >= 32 * ROWB && DP * VS >= 32 * ROWB && NW <= 4, "a tile buffer parks one wavefront's rows");
-        const bool as_partial = a.n_split > 1;
-        if (!as_partial || a.part_half) {
-            unsigned char* park = wave < 2 ? ldsK_buf[wave] : ldsV_buf[wave - 2];
-            const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
-            const long prow = as_partial ? ((long)pair * a.n_split + split) * a.r_pad + row : 0;
-            if (as_partial && row_valid && g == 0) {
-                a.part_ml[prow * 2] = m_run;
-                a.part_ml[prow * 2 + 1] = l_run;
-            }
-#pragma unroll
-            for (int db = 0; db < NDB; ++db)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int d = db * 32 + 8 * j + 4 * g;
-                    const float v0 = o[db][4 * j] * inv_l, v1 = o[db][4 * j + 1] * inv_l, v2 = o[db][4 * j + 2] * inv_l,
-                                v3 = o[db][4 * j + 3] * inv_l;
-                    u32x2_t pk;
-                    if (as_partial) {
-                        typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
-                        const h4_t hv = {(_Float16)v0, (_Float16)v1, (_Float16)v2, (_Float16)v3};
-                        pk = __builtin_bit_cast(u32x2_t, hv);
-                    } else {
-                        pk = u32x2_t{pack_bf2(v0, v1), pack_bf2(v2, v3)};
-                    }
-                    *reinterpret_cast<u32x2_t*>(park + r * ROWB + d * 2) = pk;
-                }
-            // destination of tile row rr, in 16-bit elements (-1: no such row), from the lane that owns it
-            long dst = -1;
-            if (row_valid && g == 0) dst = as_partial ? prow * D : (((long)b * a.S + s) * a.Hq + h) * D;
-            const int dst_lo = (int)(dst & 0xffffffffl), dst_hi = (int)(dst >> 32);
-            unsigned short* base16 = as_partial ? reinterpret_cast<unsigned short*>(a.part_o) : reinterpret_cast<unsigned short*>(a.out);
-            constexpr int PIECES = D * 2 / 16, RPI = 64 / PIECES;  // 16-byte pieces per row, rows per instruction
-#pragma unroll
-            for (int i = 0; i < 32 / RPI; ++i) {
-                const int rr = i * RPI + lane / PIECES, pc = lane % PIECES;
-                const long d64 = ((long)__shfl(dst_hi, rr, 64) << 32) | (unsigned int)__shfl(dst_lo, rr, 64);
-                const u32x4_t val = *reinterpret_cast<const u32x4_t*>(park + rr * ROWB + pc * 16);
-                if (d64 >= 0) *reinterpret_cast<u32x4_t*>(base16 + d64 + pc * 8) = val;
-            }
+        static_assert(TK * KS >= 32 * (D * 2 + 16) && DP * VS >= 32 * (D * 2 + 16) && NW <= 4, "a tile buffer parks one wavefront's rows");
+        if (a.n_split == 1 || a.part_half) {
+            flush_rows(wave < 2 ? ldsK_buf[wave] : ldsV_buf[wave - 2]);
             return;
         }
     }
