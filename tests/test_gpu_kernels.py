@@ -527,6 +527,40 @@ def test_attention_against_oracle(tune, dtype, kernel, case):
     assert np.array_equal(host(out), host(out_m))
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_attention_cache_rows_of_any_multiple_of_8(dtype, case):
+    """The cache row length only has to be a multiple of 8 keys: with the tightest t_max the last
+    32-key block reaches past the end of every V^T row, and what a kernel reads for those keys
+    must stay inside the allocation and out of the result."""
+    name, B, S, Hq, Hkv, D, P, kind, pad = case
+    r = np.random.default_rng(107)
+    mask, mkind, T = _mask(kind, P, S, pad)
+    t_max = (T + 7) // 8 * 8
+    Q = r.standard_normal((B, S, Hq, D)).astype(np.float32)
+    K = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    V = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    if dtype == BF16:
+        Q, K, V = orc.round_bf16(Q), orc.round_bf16(K), orc.round_bf16(V)
+    kc = torch.full((B, Hkv, t_max, D), float("nan"), device="cuda")
+    vc = torch.full((B, Hkv, D, t_max), float("nan"), device="cuda")
+    if dtype == BF16:
+        kc, vc = kc.to(torch.bfloat16).view(torch.int16), vc.to(torch.bfloat16).view(torch.int16)
+    pkg.call("vla_kv_append", kc, vc, to_dev(K, dtype), to_dev(V, dtype), dtype, B, Hkv, D, t_max, 0, T)
+    scale = 1.0 / math.sqrt(D)
+    out = empty((B, S, Hq * D), dtype)
+    pkg.call("vla_attn_prefix_suffix", to_dev(Q, dtype), kc, vc, out, dtype, B, S, Hq, Hkv, D, t_max, T, scale, mkind, P,
+             pad[0], pad[1], None)
+    sync()
+    want = np.stack([orc.attention(Q[b], K[b], V[b], mask, scale) for b in range(B)])
+    got = as_f32(out, dtype)
+    assert np.isfinite(got).all()
+    if dtype == F32:
+        assert rel_err(got, want) < FP32_TOL, rel_err(got, want)
+    else:
+        assert bf16_close(got, want) and rel_err(got, want) < 1e-2
+
+
 @pytest.mark.parametrize("split", [1, 2, 5, 8, 64])
 def test_attention_direct_kernel_key_slices_merge(tune, split):
     # Few query rows: any slicing of the keys across wavefronts (merged by the second

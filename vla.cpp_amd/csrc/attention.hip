@@ -981,15 +981,16 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
     // read from row D-1 instead, so every lane loads valid memory; their outputs are dropped.
     const unsigned char* vrow[NDB];
 #pragma unroll
-    for (int db = 0; db < NDB; ++db) vrow[db] = vbase + ((long)min(db * 32 + r, D - 1) * a.t_max + 8 * g) * EB;
+    for (int db = 0; db < NDB; ++db) vrow[db] = vbase + (long)min(db * 32 + r, D - 1) * a.t_max * EB;
     const int krow = key_of_score_row(r);  // the key of the block this lane fetches for the score product
     // One block of loads, the same seven instructions for every block, with no branch around
     // any of them: the compiler's count of loads in flight is then exact, and the wait in
     // front of a block's arithmetic leaves the younger blocks' loads in flight (with the
     // loads under branches it waited for all of them: the look-ahead was on paper only).
     // K rows past n_keys repeat the last key (their scores are masked); V^T runs past n_keys
-    // stay inside the cache row (t_max is a multiple of 64) and are zeroed by mask_partial
-    // once the data is needed, so that stale cache contents (possibly NaN) cannot reach the
+    // are kept inside the cache row (t_max is a multiple of 8: a run that would start past
+    // t_max - 8 reads the row's last run instead) and are zeroed by mask_partial once the
+    // data is needed, so that stale cache contents (possibly NaN) cannot reach the
     // accumulators.  Blocks past the slice repeat its last block and are never multiplied.
     auto load_blk = [&](int st, int kb_any) __attribute__((always_inline)) {
         const int kb = min(kb_any, kb1 - 1);
@@ -998,9 +999,11 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
 #pragma unroll
         for (int c = 0; c < NQ; ++c) kr[st][c] = *reinterpret_cast<const u32x4_t*>(kp + c * CE * EB);
 #pragma unroll
-        for (int db = 0; db < NDB; ++db)
+        for (int hh = 0; hh < 2; ++hh) {
+            const int k8 = min(kb * 32 + hh * 16 + 8 * g, a.t_max - 8);  // first of this lane's 8 consecutive keys
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh) vr[st][db][hh] = *reinterpret_cast<const u32x4_t*>(vrow[db] + (kb * 32 + hh * 16) * EB);
+            for (int db = 0; db < NDB; ++db) vr[st][db][hh] = *reinterpret_cast<const u32x4_t*>(vrow[db] + k8 * EB);
+        }
     };
     auto mask_partial = [&](int st, int kb) __attribute__((always_inline)) {
 #pragma unroll
