@@ -336,17 +336,17 @@ MEASURED_TRAFFIC_BYTES = {
     ("cfg1_smolvla_16layer_bf16_b32", "step.wo_residual"): int((7807.5 * 2 + 2250.0) * 1024),
     ("cfg1_smolvla_16layer_bf16_b32", "step.qkv_rope_append_self"): int((6935.3 * 2 + 5400.2) * 1024),
     ("cfg1_smolvla_16layer_bf16_b32", "step.q_rope_cross"): int((5076.5 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_self"): int((7725.2 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_cross"): int((6582.0 * 2 + 3000.0) * 1024),
-    ("cfg2_pi0_18layer_bf16_b16", "step.attention_self"): int((8793.0 * 2 + 13260.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_self"): int((7730.2 * 2 + 3000.0) * 1024),
+    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_cross"): int((6588.5 * 2 + 3000.0) * 1024),
+    ("cfg2_pi0_18layer_bf16_b16", "step.attention_self"): int((8824.5 * 2 + 13260.0) * 1024),
     ("cfg2_pi0_18layer_bf16_b16", "step.qkv_rope_append_self"): int((9220.3 * 2 + 4184.0) * 1024),
     ("cfg2_pi0_18layer_bf16_b16", "step.wo_residual"): int((11532.0 * 2 + 1632.0) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "step.attention_cross"): int((62538.6 * 2 + 3368.6) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "step.qkv_rope_append_self"): int((20186.8 * 2 + 12788.2) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "step.attention_cross"): int((62725.7 * 2 + 3270.3) * 1024),
+    ("cfg3_gr00t_16dit_bf16_b64", "step.qkv_rope_append_self"): int((20186.6 * 2 + 12789.1) * 1024),
     ("cfg3_gr00t_16dit_bf16_b64", "step.q_rope_cross"): int((11234.1 * 2 + 3264.0) * 1024),
     ("cfg3_gr00t_16dit_bf16_b64", "step.wo_residual"): int((12906.6 * 2 + 3264.0) * 1024),
     ("cfg4_bitvla_30layer_b8", "prefill.ternary_qkv_gemm"): int((22033.0 * 2 + 30720.0) * 1024),
-    ("cfg4_bitvla_30layer_b8", "step.attention"): int((6979.2 * 2 + 1016.2) * 1024),
+    ("cfg4_bitvla_30layer_b8", "step.attention"): int((6983.5 * 2 + 1016.2) * 1024),
 }
 
 
