@@ -1181,6 +1181,24 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
     uint32_t wv[MAXG];
 #pragma unroll
     for (int i = 0; i < MAXG; ++i) wv[i] = wp[(long)min(kg0 + i, kgroups - 1) * 64];
+    // What the epilogue reads from memory is fetched now, behind the weight loads, instead of
+    // after the last barrier where nothing is left to hide a round trip to memory.  Epilogue
+    // thread -> (row em = tid / 32, column en): M <= GEMV_WAVES, so one pass covers every row.
+    const int group = a.N / a.ws_num;
+    const int em = tid >> 5, enl = tid & 31, en = nb * 32 + enl;
+    const bool e_ok = em < a.M && en < a.N;
+    const float ws_pf = e_ok ? a.ws[en / group] : 0.f;
+    bf16_t res_pf = 0;
+    float cos_pf = 0.f, sin_pf = 0.f;
+    if constexpr (ROPE) {
+        if (e_ok && en / a.D < a.Hq + a.Hkv) {
+            const int pi = 16 * ((en % a.D) >> 5) + (enl & 15);
+            cos_pf = a.cos_t[pi];
+            sin_pf = a.sin_t[pi];
+        }
+    } else {
+        if (e_ok && a.residual) res_pf = ((const bf16_t*)a.residual)[(long)em * a.N + en];
+    }
     if (wave < a.M) {  // uniform per wavefront
         float scale;
         int sum;
@@ -1213,15 +1231,13 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
 #pragma unroll
     for (int e = 0; e < 16; ++e) part[wave][8 * (e >> 2) + 4 * g + (e & 3)][r] = acc[e];
     __syncthreads();
-    const int group = a.N / a.ws_num;
-    for (int m = tid >> 5; m < a.M; m += GEMV_WAVES * 2) {
-        const int nl = tid & 31, n = nb * 32 + nl;
-        if (n >= a.N) continue;
+    if (e_ok) {
+        const int m = em, nl = enl, n = en;
         int v = 0;
 #pragma unroll
         for (int w = 0; w < GEMV_WAVES; ++w) v += part[w][nl][m];
         v -= 2 * rs_sh[m];
-        bf16_t o = f2bf((float)v / s_sh[m] * a.ws[n / group]);
+        bf16_t o = f2bf((float)v / s_sh[m] * ws_pf);
         if constexpr (ROPE) {  // N is a multiple of 32 here: no lane of a half-wavefront is missing
             const float own = bf2f(o);
             const float other = __shfl_xor(own, 16, 64);
@@ -1229,7 +1245,7 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
             if (hh < a.Hq + a.Hkv) {
                 const bool lower = nl < 16;
                 const int pi = 16 * (r >> 5) + (nl & 15);
-                const float c = a.cos_t[pi], sn = a.sin_t[pi];
+                const float c = cos_pf, sn = sin_pf;
                 const float x0 = lower ? own : other, x1 = lower ? other : own;
                 const float lo = x0 * c - x1 * sn, hi = x1 * c + x0 * sn;
                 const int d = lower ? pi : pi + half;
@@ -1240,7 +1256,7 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
                 ((bf16_t*)a.vt_cache)[(((long)m * a.Hkv + (hh - a.Hq - a.Hkv)) * a.D + r) * (long)a.t_max + a.tok_offset] = o;
             }
         } else {
-            if (a.residual) o = f2bf(bf2f(o) + bf2f(((const bf16_t*)a.residual)[(long)m * a.N + n]));
+            if (a.residual) o = f2bf(bf2f(o) + bf2f(res_pf));
             ((bf16_t*)a.Y)[(long)m * a.N + n] = o;
         }
     }
