@@ -416,6 +416,7 @@ def algorithmic_work(cfg, B, P):
     w["step.ffn_gate_up_down"] = ("mfma", 6.0 * M * I * W, mf)
     w["step.ffn_in_out"] = ("mfma", 4.0 * M * I * W, mf)
     w["step.euler_step"] = ("hbm", M * W * es, "hbm")
+    w["step.final_norm_euler_step"] = ("hbm", M * W * es, "hbm")
     w["prefill.prefix_norm"] = ("hbm", 2 * B * P * Wv * es, "hbm")
     w["prefill.prefix_kv_proj"] = ("mfma", 2.0 * B * P * 2 * kvd * Wv, mf)
     w["prefill.prefix_kv_proj_and_cross_reprojection"] = ("mfma", 2.0 * B * P * 2 * kvd * (Wv + kvd), mf)

@@ -307,6 +307,22 @@ VLA_KAPI int vla_finish_suffix_rows(const float* acc, const float* row_table, co
 VLA_KAPI int vla_euler_step(float* x_t, const void* hn, const float* W_out, const float* b_out, int dtype,
                             int batch, int S, int n_lead, int A, int W, float dt, vla_stream_t stream);
 
+/* The same update with the stack's final norm inside the launch: h [batch][S][W] holds the
+ * rows before the norm, and each row is normalised (and rounded to `dtype`, as the separate
+ * norm launch would store it) right before its projection.
+ *   vla_rmsnorm_euler_step: rms_norm(h) * norm_w (norm_w [W] in `dtype` or NULL), the final
+ *     norm of src/models/smolvla.cpp:1413-1418 and src/models/pi0.cpp:572-587;
+ *   vla_adanorm_euler_step: n + n * scale + shift with scale, shift fp32 [W]; centred != 0:
+ *     n = layer_norm(h) without affine (src/layers/norm.h:37-46, the norm_out of
+ *     src/modules/dit_head.cpp:139-147), centred == 0: n = h * rsqrt(mean h^2 + eps)
+ *     (build_adarms, src/models/pi05.cpp:208-223, final norm at pi05.cpp:628). */
+VLA_KAPI int vla_rmsnorm_euler_step(float* x_t, const void* h, const void* norm_w, float eps, const float* W_out,
+                                    const float* b_out, int dtype, int batch, int S, int n_lead, int A, int W, float dt,
+                                    vla_stream_t stream);
+VLA_KAPI int vla_adanorm_euler_step(float* x_t, const void* h, const float* scale, const float* shift, int centred,
+                                    float eps, const float* W_out, const float* b_out, int dtype, int batch, int S,
+                                    int n_lead, int A, int W, float dt, vla_stream_t stream);
+
 /* ------------------------------------------------------------ BitVLA ternary */
 
 /* Per-row int8 quantisation (act_quant_kernel,

@@ -435,6 +435,56 @@ def test_glu_linear_and_linear_act(dtype, M, I, K, act, bias):
         assert rel_err(as_f32(y3, BF16), want3) < 1e-2
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("B,S,n_lead,A,W", [(3, 50, 0, 32, 720), (2, 51, 1, 32, 1024), (3, 17, 1, 32, 1536), (1, 9, 0, 7, 200),
+                                            (2, 5, 1, 32, 2560)])
+def test_final_norm_inside_the_euler_launch(dtype, B, S, n_lead, A, W):
+    """x_t += dt (W_out . norm(h) + b_out) in one launch, for the three final norms of the flow
+    heads (RMSNorm with a weight, LayerNorm without affine then scale / shift, RMS statistics then
+    scale / shift): against the oracle, and against the norm launch followed by the plain update."""
+    r = np.random.default_rng(170 + W)
+    h = (r.standard_normal((B, S, W)) * 2 + 0.3).astype(np.float32)
+    g = (1 + 0.1 * r.standard_normal(W)).astype(np.float32)
+    sc, sh = (0.2 * r.standard_normal(W)).astype(np.float32), (0.2 * r.standard_normal(W)).astype(np.float32)
+    x_t = r.standard_normal((B, S - n_lead, A)).astype(np.float32)
+    W_out = (0.05 * r.standard_normal((A, W))).astype(np.float32)
+    b_out = r.standard_normal(A).astype(np.float32)
+    if dtype == BF16:
+        h, g = orc.round_bf16(h), orc.round_bf16(g)
+    dt = -0.25
+    M = B * S
+    dh, dW, db = to_dev(h, dtype), dev(W_out), dev(b_out)
+    rnd = orc.round_bf16 if dtype == BF16 else (lambda v: v)
+    cases = {
+        "rms": (lambda xd: pkg.call("vla_rmsnorm_euler_step", xd, dh, to_dev(g, dtype), 1e-6, dW, db, dtype, B, S, n_lead, A, W, dt),
+                lambda y: pkg.call("vla_rms_norm", dh, to_dev(g, dtype), y, dtype, M, W, 1e-6),
+                orc.rms_norm(h.reshape(M, W), g, 1e-6)),
+        "adaln": (lambda xd: pkg.call("vla_adanorm_euler_step", xd, dh, dev(sc), dev(sh), 1, 1e-5, dW, db, dtype, B, S, n_lead, A, W, dt),
+                  lambda y: pkg.call("vla_adaln", dh, dev(sc), dev(sh), y, dtype, M, W, 1e-5),
+                  orc.adaln(h.reshape(M, W), sc, sh, 1e-5)),
+        "adarms": (lambda xd: pkg.call("vla_adanorm_euler_step", xd, dh, dev(sc), dev(sh), 0, 1e-6, dW, db, dtype, B, S, n_lead, A, W, dt),
+                   lambda y: pkg.call("vla_adarms", dh, dev(sc), dev(sh), y, dtype, M, W, 1e-6),
+                   orc.adarms(h.reshape(M, W), sc, sh, 1e-6)),
+    }
+    for name, (fused, norm, hn_want) in cases.items():
+        xd = dev(x_t)
+        fused(xd)
+        y = empty((M, W), dtype)
+        norm(y)
+        xd2 = dev(x_t)
+        pkg.call("vla_euler_step", xd2, y, dW, db, dtype, B, S, n_lead, A, W, dt)
+        sync()
+        hn = rnd(hn_want).reshape(B, S, W)[:, n_lead:]
+        v = orc.linear(hn.reshape(-1, W), W_out, b_out).reshape(B, S - n_lead, A)
+        want = x_t + dt * v
+        got, chain = host(xd), host(xd2)
+        # the row statistics are summed in another order than the stand-alone norm's: with bf16 rows a
+        # last-place difference of the scale can move single elements to the neighbouring bf16 value
+        tol = FP32_TOL if dtype == F32 else 2e-3
+        assert rel_err(got, want) < tol, (name, rel_err(got, want))
+        assert rel_err(got, chain) < tol, (name, rel_err(got, chain))
+
+
 # ------------------------------------------------------------------ attention
 CASES = [
     # name, B, S, Hq, Hkv, D, P, mask kind, pad

@@ -54,6 +54,8 @@ KERNEL_API = {
     "vla_finish_suffix_rows": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "vla_set_lead_rows": [_vp, _vp, _i, _i, _i, _i, _i, _vp],
     "vla_euler_step": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
+    "vla_rmsnorm_euler_step": [_vp, _vp, _vp, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
+    "vla_adanorm_euler_step": [_vp, _vp, _vp, _vp, _i, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp],
     "vla_act_quant_bf16": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "vla_ternary_quant_host": [_vp, _i64, _vp, _vp],
     "vla_ternary_packed_words": [_i, _i],

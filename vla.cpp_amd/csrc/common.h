@@ -73,11 +73,13 @@ template <> struct Elem<float> {
     static constexpr int kVec = 4;  // elements per 16-byte vector
     __device__ static __forceinline__ float load(const float* p) { return *p; }
     __device__ static __forceinline__ void store(float* p, float v) { *p = v; }
+    __device__ static __forceinline__ float round(float v) { return v; }  // the value a store and a load would give back
 };
 template <> struct Elem<bf16_t> {
     static constexpr int kVec = 8;
     __device__ static __forceinline__ float load(const bf16_t* p) { return bf2f(*p); }
     __device__ static __forceinline__ void store(bf16_t* p, float v) { *p = f2bf(v); }
+    __device__ static __forceinline__ float round(float v) { return bf2f(f2bf(v)); }
 };
 
 // 64-lane wavefront reductions; every lane ends with the result.

@@ -405,12 +405,22 @@ __global__ void finish_suffix_rows_kernel(const float* __restrict__ acc, const f
 // registers (NC chunks cover the width); the chunk loads of the AU rows of W_out are
 // independent and issued together; the products are summed per lane in ascending k and then
 // across the wavefront, and lane (i, u) applies the update of row i, output u.
+//
+// NORM >= 0: hn holds the rows before the stack's final norm, and the wavefront normalises its
+// rows in registers first (the statistics of row_norm_kernel's modes, each element rounded to T
+// as the stand-alone launch would have stored it), so the norm launch in front is not needed.
+// Workgroups of different action groups y repeat the norm of the same rows: a few hundred
+// operations against a launch.
 constexpr int EUL_WAVES = 4;
-template <typename T, int NC, int AU, int ROWS>
+constexpr int EUL_NO_NORM = -1;
+template <typename T, int NC, int AU, int ROWS, int NORM = EUL_NO_NORM>
 __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __restrict__ x_t, const T* __restrict__ hn,
                                                                     const float* __restrict__ W_out,
                                                                     const float* __restrict__ b_out, int n_rows, int S,
-                                                                    int n_lead, int A, int W, float dt) {
+                                                                    int n_lead, int A, int W, float dt,
+                                                                    const T* __restrict__ norm_w = nullptr,
+                                                                    const float* __restrict__ sc = nullptr,
+                                                                    const float* __restrict__ sh = nullptr, float eps = 0.f) {
     const int Sa = S - n_lead;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int r0 = (blockIdx.x * EUL_WAVES + wave) * ROWS, a0 = blockIdx.y * AU;
@@ -429,6 +439,50 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
         const float* wr = W_out + (long)min(a0 + u, A - 1) * W;
 #pragma unroll
         for (int c = 0; c < NC; ++c) wv[u][c] = wr[min(lane + 64 * c, W - 1)];
+    }
+    if constexpr (NORM != EUL_NO_NORM) {
+        // per-column operands of the norm: the same for every row
+        float g0[NC], g1[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int k = min(lane + 64 * c, W - 1);
+            if (NORM == NORM_RMS) {
+                g0[c] = norm_w ? Elem<T>::load(norm_w + k) : 1.f;
+                g1[c] = 0.f;
+            } else {
+                g0[c] = sc[k];
+                g1[c] = sh[k];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+            float mean = 0.f;
+            if (NORM == NORM_ADALN) {
+                float s1 = 0.f;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) s1 += (lane + 64 * c < W) ? hv[i][c] : 0.f;
+                mean = wave_sum(s1) / (float)W;
+            }
+            float s2 = 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const float d = (lane + 64 * c < W) ? hv[i][c] - mean : 0.f;
+                s2 += d * d;
+            }
+            const float inv = 1.0f / sqrtf(wave_sum(s2) / (float)W + eps);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                float o;
+                if (NORM == NORM_RMS) {
+                    o = hv[i][c] * inv;
+                    if (norm_w) o *= g0[c];
+                } else {
+                    const float xn = (hv[i][c] - mean) * inv;
+                    o = xn + xn * g0[c] + g1[c];
+                }
+                hv[i][c] = Elem<T>::round(o);
+            }
+        }
     }
     float mine = 0.f;
 #pragma unroll
@@ -649,6 +703,50 @@ int mod_norm(const void* x, const float* sc, const float* sh, void* y, int dtype
 
 }  // namespace
 
+namespace {
+// norm < 0: hn is already normalised.  Otherwise one of row_norm_kernel's modes, applied to
+// the rows inside the launch.
+int euler_launch(float* x_t, const void* hn, int norm, const void* norm_w, const float* sc, const float* sh, float eps,
+                 const float* W_out, const float* b_out, int dtype, int batch, int S, int n_lead, int A, int W, float dt,
+                 vla_stream_t stream) {
+    if (!x_t || !hn || !W_out || batch < 0 || S <= 0 || n_lead < 0 || n_lead >= S || A <= 0 || W <= 0)
+        return VLA_K_ERR_ARG;
+    if (batch == 0) return VLA_K_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype != VLA_DT_F32 && dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
+    if (W > 64 * 64) return VLA_K_ERR_SHAPE;
+    const int n_rows = batch * (S - n_lead);
+#define VLA_EULER_N(T, NC, AU, ROWS, NORM)                                                                          \
+    euler_step_kernel<T, NC, AU, ROWS, NORM>                                                                        \
+        <<<dim3((n_rows + EUL_WAVES * ROWS - 1) / (EUL_WAVES * ROWS), (A + AU - 1) / AU), EUL_WAVES * 64, 0, st>>>(  \
+            x_t, (const T*)hn, W_out, b_out, n_rows, S, n_lead, A, W, dt, (const T*)norm_w, sc, sh, eps)
+#define VLA_EULER(T, NC, AU, ROWS)                                       \
+    do {                                                                 \
+        if (norm == NORM_RMS) VLA_EULER_N(T, NC, AU, ROWS, NORM_RMS);    \
+        else if (norm == NORM_ADALN) VLA_EULER_N(T, NC, AU, ROWS, NORM_ADALN);   \
+        else if (norm == NORM_ADARMS) VLA_EULER_N(T, NC, AU, ROWS, NORM_ADARMS); \
+        else VLA_EULER_N(T, NC, AU, ROWS, EUL_NO_NORM);                  \
+    } while (0)
+#define VLA_EULER_T(T)                                      \
+    do {                                                    \
+        if (W <= 64 * 8) VLA_EULER(T, 8, 8, 2);             \
+        else if (W <= 64 * 12) VLA_EULER(T, 12, 8, 2);      \
+        else if (W <= 64 * 16) VLA_EULER(T, 16, 8, 2);      \
+        else if (W <= 64 * 24) VLA_EULER(T, 24, 4, 2);      \
+        else if (W <= 64 * 32) VLA_EULER(T, 32, 4, 2);      \
+        else VLA_EULER(T, 64, 2, 1);                        \
+    } while (0)
+    if (dtype == VLA_DT_F32)
+        VLA_EULER_T(float);
+    else
+        VLA_EULER_T(bf16_t);
+#undef VLA_EULER_T
+#undef VLA_EULER
+#undef VLA_EULER_N
+    return VLA_CHECK_LAUNCH();
+}
+}  // namespace
+
 extern "C" {
 
 int vla_rope_tables_host(const int32_t* pos, int n, int head_dim, double base, float* cos_tab, float* sin_tab) {
@@ -785,33 +883,22 @@ int vla_embed_suffix_act(const float* x_t, const float* W_in, const float* bias_
 
 int vla_euler_step(float* x_t, const void* hn, const float* W_out, const float* b_out, int dtype, int batch, int S,
                    int n_lead, int A, int W, float dt, vla_stream_t stream) {
-    if (!x_t || !hn || !W_out || batch < 0 || S <= 0 || n_lead < 0 || n_lead >= S || A <= 0 || W <= 0)
-        return VLA_K_ERR_ARG;
-    if (batch == 0) return VLA_K_OK;
-    hipStream_t st = (hipStream_t)stream;
-    if (dtype != VLA_DT_F32 && dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
-    if (W > 64 * 64) return VLA_K_ERR_SHAPE;
-    const int n_rows = batch * (S - n_lead);
-#define VLA_EULER(T, NC, AU, ROWS)                                                                                  \
-    euler_step_kernel<T, NC, AU, ROWS>                                                                              \
-        <<<dim3((n_rows + EUL_WAVES * ROWS - 1) / (EUL_WAVES * ROWS), (A + AU - 1) / AU), EUL_WAVES * 64, 0, st>>>(  \
-            x_t, (const T*)hn, W_out, b_out, n_rows, S, n_lead, A, W, dt)
-#define VLA_EULER_T(T)                                      \
-    do {                                                    \
-        if (W <= 64 * 8) VLA_EULER(T, 8, 8, 2);             \
-        else if (W <= 64 * 12) VLA_EULER(T, 12, 8, 2);      \
-        else if (W <= 64 * 16) VLA_EULER(T, 16, 8, 2);      \
-        else if (W <= 64 * 24) VLA_EULER(T, 24, 4, 2);      \
-        else if (W <= 64 * 32) VLA_EULER(T, 32, 4, 2);      \
-        else VLA_EULER(T, 64, 2, 1);                        \
-    } while (0)
-    if (dtype == VLA_DT_F32)
-        VLA_EULER_T(float);
-    else
-        VLA_EULER_T(bf16_t);
-#undef VLA_EULER_T
-#undef VLA_EULER
-    return VLA_CHECK_LAUNCH();
+    return euler_launch(x_t, hn, EUL_NO_NORM, nullptr, nullptr, nullptr, 0.f, W_out, b_out, dtype, batch, S, n_lead, A, W, dt,
+                        stream);
+}
+
+int vla_rmsnorm_euler_step(float* x_t, const void* h, const void* norm_w, float eps, const float* W_out, const float* b_out,
+                           int dtype, int batch, int S, int n_lead, int A, int W, float dt, vla_stream_t stream) {
+    if (!h) return VLA_K_ERR_ARG;
+    return euler_launch(x_t, h, NORM_RMS, norm_w, nullptr, nullptr, eps, W_out, b_out, dtype, batch, S, n_lead, A, W, dt, stream);
+}
+
+int vla_adanorm_euler_step(float* x_t, const void* h, const float* scale, const float* shift, int centred, float eps,
+                           const float* W_out, const float* b_out, int dtype, int batch, int S, int n_lead, int A, int W,
+                           float dt, vla_stream_t stream) {
+    if (!h || !scale || !shift) return VLA_K_ERR_ARG;
+    return euler_launch(x_t, h, centred ? NORM_ADALN : NORM_ADARMS, nullptr, scale, shift, eps, W_out, b_out, dtype, batch, S,
+                        n_lead, A, W, dt, stream);
 }
 
 int vla_act_quant_bf16(const uint16_t* in, int8_t* out, float* scales, int32_t* rowsum, int M, int K,

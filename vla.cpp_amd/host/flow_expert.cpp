@@ -144,6 +144,7 @@ class FlowExpert : public ModelArch {
     std::shared_ptr<RowSource> lang_rows_;  // token embeddings left on disk (large vocabularies)
     bool alt_vl_ = false;   // GR00T N1.6 / N1.7: cross layers alternate text / image rows
     int text_every_ = 2, P_txt_ = 0;
+    bool fuse_final_norm_ = true;  // the final norm runs inside the Euler launch
     bool adarms_ = false;  // pi0.5: ada_ holds [steps][2L+1][scale, shift, gate][W]
     DevBuf bias_step_;   // [steps][W] fp32: b_in (+ time embedding of the step)
     DevBuf ada_;         // GR00T: [steps][L+1][2][W] fp32 (scale, shift); slot L is the final norm (zeros)
@@ -277,6 +278,7 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     if (arch_ != Arch::GR00T && !adarms_) final_norm_ = load_w(ck, "act.norm", dt_, {W_});
 
     const bool no_norm_fusion = std::getenv("VLA_NO_NORM_FUSION") != nullptr;  // read once, at load
+    fuse_final_norm_ = !no_norm_fusion;
     layers_.resize(L_);
     for (int l = 0; l < L_; ++l) {
         LayerW& w = layers_[l];
@@ -859,6 +861,23 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                         prof_mark("ffn_gate_up_down");
                     }
                 }
+            }
+            if (fuse_final_norm_ && !head_io_) {
+                // final norm + output projection + Euler update in one launch
+                if (adarms_) {
+                    const float* mf = ada_.as<float>() + ((size_t)s * (2 * L_ + 1) + 2 * L_) * 3 * W_;  // gate unused (pi05.cpp:628)
+                    VLA_K(vla_adanorm_euler_step(xt_.as<float>(), h.data, mf, mf + W_, 0, eps_, W_out_.as<float>(), b_out_.as<float>(),
+                                                 dt_, B, S_, n_lead_, A_, W_, dt_step_, C.stream));
+                } else if (arch_ == Arch::GR00T) {
+                    const float* z = ada_.as<float>() + ((size_t)s * (L_ + 2) + L_) * 2 * W_;  // zeros: plain LayerNorm
+                    VLA_K(vla_adanorm_euler_step(xt_.as<float>(), h.data, z, z + W_, 1, final_eps_, W_out_.as<float>(),
+                                                 b_out_.as<float>(), dt_, B, S_, n_lead_, A_, W_, dt_step_, C.stream));
+                } else {
+                    VLA_K(vla_rmsnorm_euler_step(xt_.as<float>(), h.data, final_norm_.get(), eps_, W_out_.as<float>(),
+                                                 b_out_.as<float>(), dt_, B, S_, n_lead_, A_, W_, dt_step_, C.stream));
+                }
+                prof_mark("final_norm_euler_step");
+                continue;
             }
             if (adarms_) {
                 const float* mf = ada_.as<float>() + ((size_t)s * (2 * L_ + 1) + 2 * L_) * 3 * W_;  // gate unused (pi05.cpp:628)
