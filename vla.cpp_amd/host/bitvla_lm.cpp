@@ -111,7 +111,9 @@ class BitvlaLm : public ModelArch {
   private:
     uint32_t alloc_gen_ = 0;
     DevBuf zeros_;
-    void run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys);
+    // last_out: where the last layer's closing projection writes the hidden rows (nullptr: in
+    // place); honoured on the few-row decode path only, returns whether it was
+    bool run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys, uint16_t* last_out = nullptr);
     int L_, Hq_, Hkv_, D_, H_, A_, n_act_, n_img_, n_lang_, vocab_, F_ = 0, P_ = 0, B_ = 0;
     float eps_;
     std::vector<LmLayer> layers_;
@@ -251,7 +253,7 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
 
 // One pass of all layers over M = B*S rows sitting in h_ (S consecutive tokens
 // per observation starting at cache slot tok_offset, attending to n_keys keys).
-void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
+bool BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys, uint16_t* last_out) {
     const int kvd = Hkv_ * D_, Nqkv = H_ + 2 * kvd;
     const int half = D_ / 2;
     const float scale = 1.0f / std::sqrt((float)D_);
@@ -259,7 +261,9 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
     const float* sin_t = rope_.sin.as<float>() + (size_t)tok_offset * half;
     // a handful of rows (token-by-token decode): norm, quantisation and projection in one launch
     const bool fused = M <= 8 && H_ <= 4096 && H_ % 128 == 0;
+    const bool redirect = last_out && fused && (F_ == 0 || F_ <= 4096);
     for (LmLayer& w : layers_) {
+        const bool last = &w == &layers_.back();
         if (fused && S == 1 && w.Wqkv.paired.get()) {
             // ... and the split, rotation and cache append as well
             VLA_K(vla_rmsnorm_ternary_gemv_rope_append(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), eps_,
@@ -294,8 +298,8 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
         // O projection and the residual add of the hidden stream in one launch
         if (fused) {
             VLA_K(vla_rmsnorm_ternary_gemv(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), eps_, w.Wo.packed.as<uint32_t>(),
-                                           h_.as<uint16_t>(), h_.as<uint16_t>(), w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_,
-                                           C.stream));
+                                           redirect && last && F_ == 0 ? last_out : h_.as<uint16_t>(), h_.as<uint16_t>(),
+                                           w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_, C.stream));
             prof_mark("norm_quant_o_gemv_add");
         } else {
             VLA_K(vla_rmsnorm_act_quant_bf16(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), q8_.as<int8_t>(), s_.as<float>(),
@@ -323,8 +327,8 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
         }
         if (fused && F_ <= 4096) {  // activation, sub-norm, quantisation and down projection in one launch
             VLA_K(vla_sqrelu_rmsnorm_ternary_gemv(gu_.as<uint16_t>(), w.ffn_sub_norm.as<uint16_t>(), eps_,
-                                                  w.Wd.packed.as<uint32_t>(), h_.as<uint16_t>(), h_.as<uint16_t>(),
-                                                  w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_, C.stream));
+                                                  w.Wd.packed.as<uint32_t>(), redirect && last ? last_out : h_.as<uint16_t>(),
+                                                  h_.as<uint16_t>(), w.Wd.ws.as<float>(), w.Wd.ws_num, M, H_, F_, C.stream));
             prof_mark("sqrelu_norm_quant_down_gemv_add");
             continue;
         }
@@ -345,6 +349,7 @@ void BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys) {
                                    C.stream));
         prof_mark("ternary_down_gemm_add");
     }
+    return redirect;
 }
 
 void BitvlaLm::run_steps(int n_steps, void* stream) {
@@ -362,16 +367,24 @@ void BitvlaLm::run_steps(int n_steps, void* stream) {
         VLA_HIP(hipMemcpyAsync(h_.get(), emb_bcast_.as<uint16_t>() + (size_t)t * row, row * 2, hipMemcpyDeviceToDevice,
                                C.stream));
         prof_mark("token_embedding");
-        run_layers(C, B, 1, P_ + t, P_ + t + 1);
-        VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), out_norm_.as<uint16_t>(), hfin_.as<uint16_t>() + (size_t)t * row, eps_, B,
-                                  H_, C.stream));
-        prof_mark("final_norm");
+        // The last layer leaves token t's rows in hfin_ where it can; the final norm then runs
+        // inside the action head's launch, over all tokens at once.
+        uint16_t* hf = hfin_.as<uint16_t>() + (size_t)t * row;
+        const bool raw = run_layers(C, B, 1, P_ + t, P_ + t + 1, hf);
+        if (!raw) {
+            VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), out_norm_.as<uint16_t>(), hf, eps_, B, H_, C.stream));
+            prof_mark("final_norm");
+        }
         if (t == n_act_ - 1) {
             // cleared by a copy node: memset nodes are kept out of captured graphs
             VLA_HIP(hipMemcpyAsync(x_.get(), zeros_.get(), (size_t)n_act_ * B * A_ * 4, hipMemcpyDeviceToDevice, C.stream));
-            // x[t][b] = W_out . hfin[t][b] + b_out (batch' = n_act, rows = B, unit step)
-            VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B,
-                                 0, A_, H_, 1.0f, C.stream));
+            // x[t][b] = W_out . norm(h[t][b]) + b_out (batch' = n_act, rows = B, unit step)
+            if (raw)
+                VLA_K(vla_rmsnorm_euler_step(x_.as<float>(), hfin_.get(), out_norm_.get(), eps_, W_out_.as<float>(),
+                                             b_out_.as<float>(), VLA_DT_BF16, n_act_, B, 0, A_, H_, 1.0f, C.stream));
+            else
+                VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B,
+                                     0, A_, H_, 1.0f, C.stream));
             prof_mark("action_head");
         }
     }
