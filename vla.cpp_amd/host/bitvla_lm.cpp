@@ -112,8 +112,12 @@ class BitvlaLm : public ModelArch {
     uint32_t alloc_gen_ = 0;
     DevBuf zeros_;
     // last_out: where the last layer's closing projection writes the hidden rows (nullptr: in
-    // place); honoured on the few-row decode path only, returns whether it was
-    bool run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys, uint16_t* last_out = nullptr);
+    // place); honoured on the few-row decode path only, returns whether it was.  first_in: the
+    // rows entering the first layer when they are not in h_ yet (decode path only, as last_out).
+    bool run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys, uint16_t* last_out = nullptr,
+                    const uint16_t* first_in = nullptr);
+    // a handful of rows (token-by-token decode): norm, quantisation and projection in one launch
+    bool few_rows(int M) const { return M <= 8 && H_ <= 4096 && H_ % 128 == 0; }
     int L_, Hq_, Hkv_, D_, H_, A_, n_act_, n_img_, n_lang_, vocab_, F_ = 0, P_ = 0, B_ = 0;
     float eps_;
     std::vector<LmLayer> layers_;
@@ -253,27 +257,28 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
 
 // One pass of all layers over M = B*S rows sitting in h_ (S consecutive tokens
 // per observation starting at cache slot tok_offset, attending to n_keys keys).
-bool BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys, uint16_t* last_out) {
+bool BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys, uint16_t* last_out, const uint16_t* first_in) {
     const int kvd = Hkv_ * D_, Nqkv = H_ + 2 * kvd;
     const int half = D_ / 2;
     const float scale = 1.0f / std::sqrt((float)D_);
     const float* cos_t = rope_.cos.as<float>() + (size_t)tok_offset * half;
     const float* sin_t = rope_.sin.as<float>() + (size_t)tok_offset * half;
-    // a handful of rows (token-by-token decode): norm, quantisation and projection in one launch
-    const bool fused = M <= 8 && H_ <= 4096 && H_ % 128 == 0;
-    const bool redirect = last_out && fused && (F_ == 0 || F_ <= 4096);
+    const bool fused = few_rows(M);
+    const bool redirect = last_out && fused && F_ <= 4096;
     for (LmLayer& w : layers_) {
         const bool last = &w == &layers_.back();
+        // the hidden rows as this layer finds them: h_, except in front of the first layer
+        const uint16_t* hin = (redirect && first_in && &w == &layers_.front()) ? first_in : h_.as<uint16_t>();
         if (fused && S == 1 && w.Wqkv.paired.get()) {
             // ... and the split, rotation and cache append as well
-            VLA_K(vla_rmsnorm_ternary_gemv_rope_append(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), eps_,
+            VLA_K(vla_rmsnorm_ternary_gemv_rope_append(hin, w.attn_norm.as<uint16_t>(), eps_,
                                                        w.Wqkv.paired.as<uint32_t>(), w.Wqkv.ws.as<float>(), w.Wqkv.ws_num,
                                                        cos_t, sin_t, q_.as<uint16_t>(), w.kv.k.as<uint16_t>(),
                                                        w.kv.vt.as<uint16_t>(), M, Hq_, Hkv_, D_, H_, w.kv.t_max, tok_offset,
                                                        C.stream));
             prof_mark("norm_quant_qkv_gemv_rope_append");
         } else if (fused) {
-            VLA_K(vla_rmsnorm_ternary_gemv(h_.as<uint16_t>(), w.attn_norm.as<uint16_t>(), eps_, w.Wqkv.packed.as<uint32_t>(),
+            VLA_K(vla_rmsnorm_ternary_gemv(hin, w.attn_norm.as<uint16_t>(), eps_, w.Wqkv.packed.as<uint32_t>(),
                                            qkv_.as<uint16_t>(), nullptr, w.Wqkv.ws.as<float>(), w.Wqkv.ws_num, M, Nqkv, H_,
                                            C.stream));
             prof_mark("norm_quant_qkv_gemv");
@@ -298,7 +303,7 @@ bool BitvlaLm::run_layers(Ctx& C, int M, int S, int tok_offset, int n_keys, uint
         // O projection and the residual add of the hidden stream in one launch
         if (fused) {
             VLA_K(vla_rmsnorm_ternary_gemv(att_.as<uint16_t>(), w.sub_norm.as<uint16_t>(), eps_, w.Wo.packed.as<uint32_t>(),
-                                           redirect && last && F_ == 0 ? last_out : h_.as<uint16_t>(), h_.as<uint16_t>(),
+                                           redirect && last && F_ == 0 ? last_out : h_.as<uint16_t>(), hin,
                                            w.Wo.ws.as<float>(), w.Wo.ws_num, M, H_, H_, C.stream));
             prof_mark("norm_quant_o_gemv_add");
         } else {
@@ -364,13 +369,17 @@ void BitvlaLm::run_steps(int n_steps, void* stream) {
     prof_start("step", C.stream);
     for (int it = 0; it < n_steps; ++it) {
         const int t = it % n_act_;
-        VLA_HIP(hipMemcpyAsync(h_.get(), emb_bcast_.as<uint16_t>() + (size_t)t * row, row * 2, hipMemcpyDeviceToDevice,
-                               C.stream));
-        prof_mark("token_embedding");
-        // The last layer leaves token t's rows in hfin_ where it can; the final norm then runs
-        // inside the action head's launch, over all tokens at once.
+        // Where the few-row launches apply (`direct`, a matter of shapes only), the first layer reads
+        // token t's embedding rows where they lie and the last layer leaves its rows in hfin_: no
+        // copy in front, and the final norm runs inside the action head's launch, over all tokens.
+        const uint16_t* emb = emb_bcast_.as<uint16_t>() + (size_t)t * row;
         uint16_t* hf = hfin_.as<uint16_t>() + (size_t)t * row;
-        const bool raw = run_layers(C, B, 1, P_ + t, P_ + t + 1, hf);
+        const bool direct = few_rows(B) && F_ <= 4096;
+        if (!direct) {
+            VLA_HIP(hipMemcpyAsync(h_.get(), emb, row * 2, hipMemcpyDeviceToDevice, C.stream));
+            prof_mark("token_embedding");
+        }
+        const bool raw = run_layers(C, B, 1, P_ + t, P_ + t + 1, hf, emb);
         if (!raw) {
             VLA_K(bitvla_rmsnorm_bf16(h_.as<uint16_t>(), out_norm_.as<uint16_t>(), hf, eps_, B, H_, C.stream));
             prof_mark("final_norm");
