@@ -315,7 +315,9 @@ VLA_KAPI int vla_euler_step(float* x_t, const void* hn, const float* W_out, cons
  *   vla_adanorm_euler_step: n + n * scale + shift with scale, shift fp32 [W]; centred != 0:
  *     n = layer_norm(h) without affine (src/layers/norm.h:37-46, the norm_out of
  *     src/modules/dit_head.cpp:139-147), centred == 0: n = h * rsqrt(mean h^2 + eps)
- *     (build_adarms, src/models/pi05.cpp:208-223, final norm at pi05.cpp:628). */
+ *     (build_adarms, src/models/pi05.cpp:208-223, final norm at pi05.cpp:628).
+ * Meant for the flow heads' widths: rows wider than 2048 are handled but take longer than
+ * the norm launch they save. */
 VLA_KAPI int vla_rmsnorm_euler_step(float* x_t, const void* h, const void* norm_w, float eps, const float* W_out,
                                     const float* b_out, int dtype, int batch, int S, int n_lead, int A, int W, float dt,
                                     vla_stream_t stream);

@@ -422,7 +422,10 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
                                                                     const float* __restrict__ sc = nullptr,
                                                                     const float* __restrict__ sh = nullptr, float eps = 0.f) {
     const int Sa = S - n_lead;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // the wavefront's index as a scalar: row bases are then scalar too and a load's address is
+    // base + 32-bit lane offset (64-bit per-lane addresses for every chunk would crowd the
+    // register file and leave the loads waited for one by one)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r0 = (blockIdx.x * EUL_WAVES + wave) * ROWS, a0 = blockIdx.y * AU;
     if (r0 >= n_rows) return;
     float hv[ROWS][NC], wv[AU][NC];
@@ -432,22 +435,34 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
         const int b = row / Sa, s = row % Sa;
         const T* hr = hn + ((long)b * S + n_lead + s) * W;
 #pragma unroll
-        for (int c = 0; c < NC; ++c) hv[i][c] = Elem<T>::load(hr + min(lane + 64 * c, W - 1));
+        for (int c = 0; c < NC; ++c) hv[i][c] = Elem<T>::load(hr + (unsigned)min(lane + 64 * c, W - 1));
     }
+    // The rows of W_out are requested together with the activation rows when the norm's own
+    // operands leave room for them; with long rows they are requested after the norm instead
+    // (holding everything at once overflows the register file, and the compiler then takes
+    // the loads one at a time, a round trip to memory each).
+    constexpr bool W_EARLY = NORM == EUL_NO_NORM || NC * (ROWS + AU + 2) <= 192;
+    auto load_w_rows = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int u = 0; u < AU; ++u) {
-        const float* wr = W_out + (long)min(a0 + u, A - 1) * W;
+        for (int u = 0; u < AU; ++u) {
+            const float* wr = W_out + (long)min(a0 + u, A - 1) * W;
 #pragma unroll
-        for (int c = 0; c < NC; ++c) wv[u][c] = wr[min(lane + 64 * c, W - 1)];
-    }
+            for (int c = 0; c < NC; ++c) wv[u][c] = wr[(unsigned)min(lane + 64 * c, W - 1)];
+        }
+    };
+    if constexpr (W_EARLY) load_w_rows();
     if constexpr (NORM != EUL_NO_NORM) {
         // per-column operands of the norm: the same for every row
+        // (loads without a branch around them: a missing weight reads the rows' own memory and
+        // the value is dropped; under a branch each load would be waited for on its own)
         float g0[NC], g1[NC];
+        const T* gw = norm_w ? norm_w : hn;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            const int k = min(lane + 64 * c, W - 1);
+            const unsigned k = (unsigned)min(lane + 64 * c, W - 1);
             if (NORM == NORM_RMS) {
-                g0[c] = norm_w ? Elem<T>::load(norm_w + k) : 1.f;
+                const float lv = Elem<T>::load(gw + k);
+                g0[c] = norm_w ? lv : 1.f;
                 g1[c] = 0.f;
             } else {
                 g0[c] = sc[k];
@@ -483,6 +498,10 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
                 hv[i][c] = Elem<T>::round(o);
             }
         }
+    }
+    if constexpr (!W_EARLY) {
+        __builtin_amdgcn_sched_barrier(0);  // not hoisted back in front of the norm
+        load_w_rows();
     }
     float mine = 0.f;
 #pragma unroll

@@ -371,7 +371,7 @@ void BitvlaLm::run_steps(int n_steps, void* stream) {
         const int t = it % n_act_;
         // Where the few-row launches apply (`direct`, a matter of shapes only), the first layer reads
         // token t's embedding rows where they lie and the last layer leaves its rows in hfin_: no
-        // copy in front, and the final norm runs inside the action head's launch, over all tokens.
+        // copy in front, and one final norm over all tokens' rows in front of the action head.
         const uint16_t* emb = emb_bcast_.as<uint16_t>() + (size_t)t * row;
         uint16_t* hf = hfin_.as<uint16_t>() + (size_t)t * row;
         const bool direct = few_rows(B) && F_ <= 4096;
@@ -388,12 +388,11 @@ void BitvlaLm::run_steps(int n_steps, void* stream) {
             // cleared by a copy node: memset nodes are kept out of captured graphs
             VLA_HIP(hipMemcpyAsync(x_.get(), zeros_.get(), (size_t)n_act_ * B * A_ * 4, hipMemcpyDeviceToDevice, C.stream));
             // x[t][b] = W_out . norm(h[t][b]) + b_out (batch' = n_act, rows = B, unit step)
-            if (raw)
-                VLA_K(vla_rmsnorm_euler_step(x_.as<float>(), hfin_.get(), out_norm_.get(), eps_, W_out_.as<float>(),
-                                             b_out_.as<float>(), VLA_DT_BF16, n_act_, B, 0, A_, H_, 1.0f, C.stream));
-            else
-                VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B,
-                                     0, A_, H_, 1.0f, C.stream));
+            if (raw)  // every token's rows at once, in place
+                VLA_K(bitvla_rmsnorm_bf16(hfin_.as<uint16_t>(), out_norm_.as<uint16_t>(), hfin_.as<uint16_t>(), eps_, n_act_ * B, H_,
+                                          C.stream));
+            VLA_K(vla_euler_step(x_.as<float>(), hfin_.get(), W_out_.as<float>(), b_out_.as<float>(), VLA_DT_BF16, n_act_, B, 0,
+                                 A_, H_, 1.0f, C.stream));
             prof_mark("action_head");
         }
     }
