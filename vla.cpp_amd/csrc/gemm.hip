@@ -173,11 +173,13 @@ __device__ __forceinline__ TileCols tile_cols(const GemmArgs& a, int nt) {
 
 // Epilogue of one 64x64 sub-tile held in the LDS C tile: thread t owns row t/4 and
 // columns jg..jg+7 and 32+jg..32+jg+7 of the sub-tile.
-template <typename T, int kEpi>
+__device__ const float kNoBiasRegs[16] = {};
+template <typename T, int kEpi, bool BIAS_REGS = false>
 __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t* C, int m0, int nt, const TileCols& tc,
                                                int tid, bool have_res = false, u32x4_t res_lo = u32x4_t{0u, 0u, 0u, 0u},
                                                u32x4_t res_hi = u32x4_t{0u, 0u, 0u, 0u}, int norm_mode = 0,
-                                               const float* row_stat = nullptr, int stat_stride = 0) {
+                                               const float* row_stat = nullptr, int stat_stride = 0,
+                                               const float (&bias_regs)[16] = kNoBiasRegs) {
     const int erow = tid >> 2, jg = (tid & 3) * 8;
     const int m = m0 + erow;
     if (m >= a.M) return;
@@ -270,19 +272,26 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
             float* v = hlf ? hi : lo;
             const long o = (long)m * a.N + n0;
             const bool full = (n0 + 8 <= a.N) && (a.N % 8 == 0);
+            // per-column operands: indices clamped into the row instead of a branch per element
+            // (columns past N are never stored), so the eight loads are in flight together
             if (a.bias) {
+                // BIAS_REGS: this thread's 2 x 8 values, fetched by the caller ahead of the epilogue
+                float bv[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (n0 + e < a.N) v[e] += a.bias[n0 + e];
+                for (int e = 0; e < 8; ++e) bv[e] = BIAS_REGS ? bias_regs[hlf * 8 + e] : a.bias[min(n0 + e, a.N - 1)];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += bv[e];
             }
             if (a.act != VLA_ACT_NONE) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] = apply_act(v[e], a.act);
             }
             if (a.col_gate) {
+                float gv[8];
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (n0 + e < a.N) v[e] *= a.col_gate[n0 + e];
+                for (int e = 0; e < 8; ++e) gv[e] = a.col_gate[min(n0 + e, a.N - 1)];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] *= gv[e];
             }
             if (full && a.out_bf16) {  // 8 consecutive bf16 = one 16-byte access each way
                 if (a.residual) {
@@ -821,6 +830,16 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
         __syncthreads();
         multiply(cs, std::false_type{}, 0, 0, (a.K - nkt_full * BK) / 16);
     }
+    // The bias columns of every sub-tile's epilogue (thread layout as for the residual) are
+    // requested here, while the ring's last loads drain, and not behind each sub-tile's barrier.
+    float bias_pf[TN][16] = {};
+    if (kEpi == EPI_PLAIN && a.bias != nullptr) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                bias_pf[j][e] = a.bias[min((ntw * TN + j) * BN + (e >> 3) * 32 + (tid & 3) * 8 + (e & 7), a.N - 1)];
+    }
     wait_vmcnt<0>();  // the re-fetches must have landed before the ring is reused for C
     __syncthreads();
 
@@ -853,8 +872,8 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
             __syncthreads();
             const int nt_sub = ntw * TN + j;
             if (nt_sub < a.n_tiles)
-                epilogue_64x64<T, kEpi>(a, C, m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0], res_pf[i][j][1], kNorm,
-                                        row_stat + i * 128, ROWS_A * 2);
+                epilogue_64x64<T, kEpi, kEpi == EPI_PLAIN>(a, C, m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0],
+                                                           res_pf[i][j][1], kNorm, row_stat + i * 128, ROWS_A * 2, bias_pf[j]);
         }
 }
 
@@ -1186,18 +1205,22 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
     // thread -> (row em = tid / 32, column en): M <= GEMV_WAVES, so one pass covers every row.
     const int group = a.N / a.ws_num;
     const int em = tid >> 5, enl = tid & 31, en = nb * 32 + enl;
+    // (no branch around any of these loads: addresses are clamped into the arrays instead, and
+    // a value that is not needed is dropped -- a load under a branch is waited for at the join,
+    // together with every load issued before it)
     const bool e_ok = em < a.M && en < a.N;
-    const float ws_pf = e_ok ? a.ws[en / group] : 0.f;
+    const int ec = min(en, a.N - 1), emc = min(em, a.M - 1);
+    const float ws_pf = a.ws[ec / group];
     bf16_t res_pf = 0;
     float cos_pf = 0.f, sin_pf = 0.f;
     if constexpr (ROPE) {
-        if (e_ok && en / a.D < a.Hq + a.Hkv) {
-            const int pi = 16 * ((en % a.D) >> 5) + (enl & 15);
-            cos_pf = a.cos_t[pi];
-            sin_pf = a.sin_t[pi];
-        }
+        const int pi = 16 * ((ec % a.D) >> 5) + (enl & 15);  // < D / 2 for every column
+        cos_pf = a.cos_t[pi];
+        sin_pf = a.sin_t[pi];
     } else {
-        if (e_ok && a.residual) res_pf = ((const bf16_t*)a.residual)[(long)em * a.N + en];
+        // without a residual: the first element of the activations, dropped in the epilogue
+        const bf16_t* rp = a.residual ? (const bf16_t*)a.residual + (long)emc * a.N + ec : (const bf16_t*)a.A;
+        res_pf = *rp;
     }
     if (wave < a.M) {  // uniform per wavefront
         float scale;
