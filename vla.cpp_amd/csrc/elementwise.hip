@@ -315,7 +315,7 @@ bool launch_row_norm(const void* x, const void* w, const float* sc, const float*
 constexpr int EMB_ROWS = 32;
 constexpr int EMB_MAX_A = 64;
 constexpr int EMB_COLS = 64;
-template <typename T>
+template <typename T, int AMAX = EMB_MAX_A>  // AMAX: the padded action width the staging loops are unrolled for
 __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restrict__ x_t, const float* __restrict__ W_in,
                                                             const float* __restrict__ bias_step,
                                                             const float* __restrict__ lead, T* __restrict__ h, int n_rows,
@@ -328,25 +328,92 @@ __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restri
     const int row0 = blockIdx.x * EMB_ROWS, c0 = blockIdx.y * EMB_COLS;
     const int ncol = min(EMB_COLS, W - c0);
     const int A4 = (A + 3) & ~3;
-    for (int i = threadIdx.x; i < EMB_ROWS * A4; i += blockDim.x) {
-        const int rr = i / A4, a = i % A4, row = row0 + rr;
-        float v = 0.f;
-        if (row < n_rows && a < A) {
-            const int b = row / S, s = row % S;
-            if (s >= n_lead) v = x_t[((long)b * (S - n_lead) + (s - n_lead)) * A + a];
-        }
-        xs[rr][a] = v;
+    // Every global load of the workgroup is issued before the first is used, none under a
+    // branch (addresses of elements that do not exist are clamped to element 0 and the value is
+    // replaced by zero): loads under branches are waited for one by one, a dozen round trips
+    // to memory instead of one.  Element i of a staged array is (i / A4, i % A4); a thread's
+    // elements are 256 apart, so the pair advances by (256 / A4, 256 % A4) without dividing again.
+    // (batch, token) of the workgroup's rows, divided once per row rather than once per use
+    __shared__ int row_b[EMB_ROWS], row_s[EMB_ROWS];
+    if (threadIdx.x < EMB_ROWS) {
+        const int row = min(row0 + (int)threadIdx.x, n_rows - 1);
+        row_b[threadIdx.x] = row / S;
+        row_s[threadIdx.x] = row % S;
     }
-    for (int i = threadIdx.x; i < EMB_COLS * A4; i += blockDim.x) {
-        const int cc = i / A4, a = i % A4;
-        ws[cc][a] = (cc < ncol && a < A) ? W_in[(long)(c0 + cc) * A + a] : 0.f;
+    __syncthreads();
+    constexpr int XI = EMB_ROWS * AMAX / 256, WI = EMB_COLS * AMAX / 256;
+    const int dq = 256 / A4, dr = 256 % A4;
+    float xv[XI], wv[WI];
+    {
+        int rr = threadIdx.x / A4, a = threadIdx.x % A4;
+#pragma unroll
+        for (int it = 0; it < XI; ++it) {
+            const int row = row0 + rr;
+            const int b = row_b[min(rr, EMB_ROWS - 1)], sx = row_s[min(rr, EMB_ROWS - 1)];
+            const bool ok = rr < EMB_ROWS && row < n_rows && a < A && sx >= n_lead;
+            const float v = x_t[ok ? ((long)b * (S - n_lead) + (sx - n_lead)) * A + a : 0];
+            xv[it] = ok ? v : 0.f;
+            rr += dq;
+            a += dr;
+            if (a >= A4) {
+                a -= A4;
+                ++rr;
+            }
+        }
+    }
+    {
+        int cc = threadIdx.x / A4, a = threadIdx.x % A4;
+#pragma unroll
+        for (int it = 0; it < WI; ++it) {
+            const bool ok = cc < ncol && a < A;
+            const float v = W_in[ok ? (long)(c0 + cc) * A + a : 0];
+            wv[it] = ok ? v : 0.f;
+            cc += dq;
+            a += dr;
+            if (a >= A4) {
+                a -= A4;
+                ++cc;
+            }
+        }
     }
     const int cl = threadIdx.x & 63, rq = threadIdx.x >> 6;  // column in slab, row residue mod 4
-    const int c = c0 + cl;
-    const float bias = c < W ? bias_step[c] : 0.f;
+    const int c = c0 + cl, cc_ok = min(c, W - 1);
+    const float bias = bias_step[cc_ok];
+    // the rows copied from `lead` (s < n_lead), fetched for every row of the thread and dropped where not needed
+    constexpr int NR = EMB_ROWS / 4;
+    float lv[NR];
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+        const int b = row_b[rq + 4 * k], sx = row_s[rq + 4 * k];
+        lv[k] = n_lead > 0 ? lead[((long)b * n_lead + min(sx, n_lead - 1)) * W + cc_ok] : 0.f;
+    }
+    {
+        int rr = threadIdx.x / A4, a = threadIdx.x % A4;
+#pragma unroll
+        for (int it = 0; it < XI; ++it) {
+            if (rr < EMB_ROWS) xs[rr][a] = xv[it];
+            rr += dq;
+            a += dr;
+            if (a >= A4) {
+                a -= A4;
+                ++rr;
+            }
+        }
+        int cc = threadIdx.x / A4;
+        a = threadIdx.x % A4;
+#pragma unroll
+        for (int it = 0; it < WI; ++it) {
+            if (cc < EMB_COLS) ws[cc][a] = wv[it];
+            cc += dq;
+            a += dr;
+            if (a >= A4) {
+                a -= A4;
+                ++cc;
+            }
+        }
+    }
     __syncthreads();
     if (c >= W) return;
-    constexpr int NR = EMB_ROWS / 4;
     float acc[NR];
 #pragma unroll
     for (int k = 0; k < NR; ++k) acc[k] = 0.f;
@@ -363,8 +430,7 @@ __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restri
     for (int k = 0; k < NR; ++k) {
         const int rr = rq + 4 * k, row = row0 + rr;
         if (row >= n_rows) continue;
-        const int b = row / S, s = row % S;
-        const float v = s < n_lead ? lead[((long)b * n_lead + s) * W + c] : apply_act(acc[k] + bias, act);
+        const float v = row_s[rr] < n_lead ? lv[k] : apply_act(acc[k] + bias, act);
         Elem<T>::store(h + (long)row * W + c, v);
     }
 }
@@ -891,12 +957,16 @@ int vla_embed_suffix_act(const float* x_t, const float* W_in, const float* bias_
     hipStream_t st = (hipStream_t)stream;
     const int n_rows = batch * S;
     const dim3 blocks((n_rows + EMB_ROWS - 1) / EMB_ROWS, (W + EMB_COLS - 1) / EMB_COLS);
-    if (out_dtype == VLA_DT_F32)
-        embed_suffix_kernel<float><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W, act);
-    else if (out_dtype == VLA_DT_BF16)
-        embed_suffix_kernel<bf16_t><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W, act);
-    else
+    const bool narrow = A <= 32;  // half the staging passes
+    if (out_dtype == VLA_DT_F32) {
+        if (narrow) embed_suffix_kernel<float, 32><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W, act);
+        else embed_suffix_kernel<float><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W, act);
+    } else if (out_dtype == VLA_DT_BF16) {
+        if (narrow) embed_suffix_kernel<bf16_t, 32><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W, act);
+        else embed_suffix_kernel<bf16_t><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W, act);
+    } else {
         return VLA_K_ERR_ARG;
+    }
     return VLA_CHECK_LAUNCH();
 }
 
