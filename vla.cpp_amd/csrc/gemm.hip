@@ -671,7 +671,7 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     constexpr int NCH = KB / 32;        // 16-k MFMA chunks per tile
     constexpr int STAGE = (ROWS_A + ROWS_W) * KB;
     constexpr int C_BYTES = 4 * 64 * C_STRIDE;
-    constexpr int EPI_BYTES = C_BYTES + ROWS_A * 16;  // C sub-tile, then two (sum of squares, sum) pairs per tile row (kNorm)
+    constexpr int EPI_BYTES = 2 * C_BYTES + ROWS_A * 16;  // two C sub-tiles, then two (sum of squares, sum) pairs per tile row (kNorm)
     constexpr int LDS_BYTES = NS * STAGE > EPI_BYTES ? NS * STAGE : EPI_BYTES;
     constexpr int IN_FLIGHT = (NS - 2) * NLOAD;  // loads younger than the tile about to be multiplied
     static_assert(KB == 128 || KB == 256, "swizzle is defined for 128- and 256-byte rows");
@@ -843,8 +843,13 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     wait_vmcnt<0>();  // the re-fetches must have landed before the ring is reused for C
     __syncthreads();
 
-    uint32_t* C = reinterpret_cast<uint32_t*>(lds);
-    float* row_stat = reinterpret_cast<float*>(lds + C_BYTES);  // [wn][ROWS_A][2]
+    // The accumulators leave through LDS one 64x64 sub-tile at a time (the epilogue wants whole
+    // rows of a sub-tile per thread: rotation partners, 16-byte stores).  Two staging buffers in
+    // turn: sub-tile n + 1 is written between the same pair of barriers in which sub-tile n is
+    // read, so a sub-tile costs one barrier, and its LDS writes overlap the previous epilogue's
+    // memory traffic.
+    uint32_t* Cb[2] = {reinterpret_cast<uint32_t*>(lds), reinterpret_cast<uint32_t*>(lds + C_BYTES)};
+    float* row_stat = reinterpret_cast<float*>(lds + 2 * C_BYTES);  // [wn][ROWS_A][2]
     if (kNorm) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
@@ -859,22 +864,27 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
             }
         }
     }
+    constexpr int NSUB = TM * TN;
+    auto stage_c = [&](int n) __attribute__((always_inline)) {
+        const int i = n / TN, j = n % TN;
+        uint32_t* C = Cb[n & 1];
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+        for (int jj = 0; jj < 4; ++jj)
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            if (i + j > 0) __syncthreads();
+            for (int ii = 0; ii < 4; ++ii)
+                C[(wm * 32 + 8 * jj + 4 * g + ii) * C_STRIDE + wn * 32 + r] = acc_bits(acc[i][j][4 * jj + ii]);
+    };
+    stage_c(0);
 #pragma unroll
-            for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-                for (int ii = 0; ii < 4; ++ii)
-                    C[(wm * 32 + 8 * jj + 4 * g + ii) * C_STRIDE + wn * 32 + r] = acc_bits(acc[i][j][4 * jj + ii]);
-            __syncthreads();
-            const int nt_sub = ntw * TN + j;
-            if (nt_sub < a.n_tiles)
-                epilogue_64x64<T, kEpi, kEpi == EPI_PLAIN>(a, C, m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0],
-                                                           res_pf[i][j][1], kNorm, row_stat + i * 128, ROWS_A * 2, bias_pf[j]);
-        }
+    for (int n = 0; n < NSUB; ++n) {
+        const int i = n / TN, j = n % TN;
+        __syncthreads();  // sub-tile n is staged, and the buffer of sub-tile n - 1 has been read by everyone
+        if (n + 1 < NSUB) stage_c(n + 1);
+        const int nt_sub = ntw * TN + j;
+        if (nt_sub < a.n_tiles)
+            epilogue_64x64<T, kEpi, kEpi == EPI_PLAIN>(a, Cb[n & 1], m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0],
+                                                       res_pf[i][j][1], kNorm, row_stat + i * 128, ROWS_A * 2, bias_pf[j]);
+    }
 }
 
 // Large-M ternary GEMM (BitVLA prefill: M = batch x prefix tokens).  Workgroup tile
