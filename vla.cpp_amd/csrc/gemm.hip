@@ -1025,12 +1025,29 @@ __global__ void __launch_bounds__(WM * 128, 2) ternary_gemm_big_kernel(GemmArgs 
     // wavefront's 64 rows is far from the exponent limits it is computed as the refinement
     // sequence of the full-range expansion without its operand scaling (identical bits):
     // y ~ 1/s by one Newton step on v_rcp_f32, then q0 = a*y, two residual corrections.
-    const float sabs = fabsf(a.s[min(m0 + wm * 64 + lane, a.M - 1)]);
+    // Lane l holds the activation scale and the row sum of the wavefront's row l: one coalesced
+    // load each.  The loops below pick a row's pair out of these with v_readlane (the row of an
+    // accumulator element is a compile-time constant apart from the lane's half g) instead of
+    // fetching it from memory where it is needed, which cost a round trip per pair of rows.
+    const int lane_row = min(m0 + wm * 64 + lane, a.M - 1);
+    const float s_lane = a.s[lane_row];
+    const int rs_lane = a.rowsum[lane_row];
+    const float sabs = fabsf(s_lane);
     const bool fast = __builtin_amdgcn_ballot_w64(sabs > 0x1p-60f && sabs < 0x1p60f) == ~0ull;
     unsigned char* tp = &lds[0][0] + wave * (32 * T_STRIDE);
     const bool vec_ok = (a.N % 8) == 0;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
+        // the residual vectors of this half of the rows, requested ahead of the staging arithmetic
+        u32x4_t res_v[8] = {};
+        const bool res_vec = a.residual != nullptr && vec_ok;
+        if (res_vec) {
+#pragma unroll
+            for (int p = 0; p < 8; ++p) {
+                const int m = min(m0 + wm * 64 + i * 32 + p * 4 + (lane >> 4), a.M - 1), n = min(n0 + (lane & 15) * 8, a.N - 8);
+                res_v[p] = *reinterpret_cast<const u32x4_t*>((const bf16_t*)a.residual + (long)m * a.N + n);
+            }
+        }
         if (fast) {
 #pragma unroll
             for (int jj = 0; jj < 4; ++jj)
@@ -1041,9 +1058,13 @@ __global__ void __launch_bounds__(WM * 128, 2) ternary_gemm_big_kernel(GemmArgs 
                     int rs2[2];
 #pragma unroll
                     for (int t = 0; t < 2; ++t) {
-                        const int mm = min(m0 + wm * 64 + i * 32 + row + t, a.M - 1);
-                        rs2[t] = 2 * a.rowsum[mm];
-                        sm[t] = a.s[mm];
+                        // row of the wavefront's tile: i * 32 + 8 jj + 4 g + ip + t (rows past M repeat row M - 1, as lane_row does)
+                        const int r0 = i * 32 + 8 * jj + ip + t;
+                        const int rs_g0 = __builtin_amdgcn_readlane(rs_lane, r0), rs_g1 = __builtin_amdgcn_readlane(rs_lane, r0 + 4);
+                        const int sb_g0 = __builtin_amdgcn_readlane(__float_as_int(s_lane), r0);
+                        const int sb_g1 = __builtin_amdgcn_readlane(__float_as_int(s_lane), r0 + 4);
+                        rs2[t] = 2 * (g ? rs_g1 : rs_g0);
+                        sm[t] = __int_as_float(g ? sb_g1 : sb_g0);
                         const float y0 = __builtin_amdgcn_rcpf(sm[t]);
                         y[t] = __builtin_fmaf(__builtin_fmaf(-sm[t], y0, 1.0f), y0, y0);
                     }
@@ -1090,7 +1111,7 @@ __global__ void __launch_bounds__(WM * 128, 2) ternary_gemm_big_kernel(GemmArgs 
             if (vec_ok && n + 8 <= a.N) {
                 u32x4_t o = v;
                 if (res) {  // out = bf16(out + residual), both already bf16
-                    const u32x4_t rr = *reinterpret_cast<const u32x4_t*>(res);
+                    const u32x4_t rr = res_v[p];
 #pragma unroll
                     for (int e = 0; e < 4; ++e)
                         o[e] = pack_bf2(__uint_as_float(v[e] << 16) + __uint_as_float(rr[e] << 16),
