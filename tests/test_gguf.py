@@ -133,6 +133,17 @@ def test_malformed_files_fail_to_open_instead_of_crashing(tmp_path):
     assert not opens(blob[:i] + struct.pack("<Q", 1 << 20) + blob[i + 8:])   # offset beyond the file
     assert not opens(blob[:i] + struct.pack("<Q", 130) + blob[i + 8:])       # misaligned offset
     assert not os.path.exists(path + ".none") and not opens.__call__(b"")
+    # a record of a type this reader does not size (a newer quantisation, say) may declare any
+    # shape: the file opens, the tensor is listed, and reading it as floats is refused before
+    # anything is allocated for its 2^60 elements
+    i = blob.index(b"w.i8") + 4
+    odd = blob[:i] + struct.pack("<IQIQ", 1, 1 << 60, 99, 128) + blob[i + 4 + 8 + 4 + 8:]
+    open(path, "wb").write(odd)
+    with gguf.Reader(pkg.lib(), path) as g:
+        assert g.meta("w.i8")["type"] == 99 and g.meta("w.i8")["ne"][0] == 1 << 60 and g.meta("w.i8")["nbytes"] == 0
+        one = np.zeros(1, np.float32)
+        assert pkg.lib().vla_gguf_read_f32(g._h, b"w.i8", one.ctypes.data, 1 << 60) != 0 and one[0] == 0
+        assert g.read_raw("w.i8", 8) is None
 
 
 # ------------------------------------------------------------------ through vla_model_load

@@ -249,6 +249,12 @@ struct gguf_reader {
             std::fprintf(stderr, "vla(%s): missing tensor %s\n", arch, name);
             return {};
         }
+        // (the type first: only for the types sized at open() is the element count known to fit
+        // the file; a record of an unknown type may declare any shape)
+        if (t->type != GGUF_T_F32 && t->type != GGUF_T_BF16 && t->type != GGUF_T_F16) {
+            std::fprintf(stderr, "vla(%s): tensor %s unsupported type %d\n", arch, name, (int)t->type);
+            return {};
+        }
         const size_t n = (size_t)t->nelements();
         std::vector<float> out(n);
         if (t->type == GGUF_T_F32) {
