@@ -477,9 +477,30 @@ __global__ void finish_suffix_rows_kernel(const float* __restrict__ acc, const f
 // as the stand-alone launch would have stored it), so the norm launch in front is not needed.
 // Workgroups of different action groups y repeat the norm of the same rows: a few hundred
 // operations against a launch.
+//
+// VEC (W a multiple of 8, 16-byte aligned operands): a lane's elements are runs of eight
+// (8 (lane + 64 j) .. +7), fetched with 16-byte loads: an eighth of the load instructions,
+// which were most of what the kernel issued.  The products are then summed in another order
+// than in the element-per-lane form (fp32, agreeing to rounding).
 constexpr int EUL_WAVES = 4;
 constexpr int EUL_NO_NORM = -1;
-template <typename T, int NC, int AU, int ROWS, int NORM = EUL_NO_NORM>
+__device__ __forceinline__ void eul_load8(const bf16_t* p, float* o) {
+    const u32x4_t raw = *reinterpret_cast<const u32x4_t*>(p);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        o[2 * j] = __uint_as_float(raw[j] << 16);
+        o[2 * j + 1] = __uint_as_float(raw[j] & 0xffff0000u);
+    }
+}
+__device__ __forceinline__ void eul_load8(const float* p, float* o) {
+    const f32x4_t a = *reinterpret_cast<const f32x4_t*>(p), b = *reinterpret_cast<const f32x4_t*>(p + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        o[j] = a[j];
+        o[4 + j] = b[j];
+    }
+}
+template <typename T, int NC, int AU, int ROWS, int NORM = EUL_NO_NORM, bool VEC = false>
 __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __restrict__ x_t, const T* __restrict__ hn,
                                                                     const float* __restrict__ W_out,
                                                                     const float* __restrict__ b_out, int n_rows, int S,
@@ -494,14 +515,25 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int r0 = (blockIdx.x * EUL_WAVES + wave) * ROWS, a0 = blockIdx.y * AU;
     if (r0 >= n_rows) return;
+    static_assert(!VEC || NC % 8 == 0, "runs of eight");
     float hv[ROWS][NC], wv[AU][NC];
+    // element held in slot c, and the load of a row's slots from p (clamped into the row)
+    auto kidx = [&](int c) { return VEC ? 8 * (lane + 64 * (c >> 3)) + (c & 7) : lane + 64 * c; };
+    auto load_slots = [&](auto* p, float* dst) __attribute__((always_inline)) {
+        if constexpr (VEC) {
+#pragma unroll
+            for (int cv = 0; cv < NC / 8; ++cv) eul_load8(p + 8u * (unsigned)min(lane + 64 * cv, W / 8 - 1), dst + 8 * cv);
+        } else {
+#pragma unroll
+            for (int c = 0; c < NC; ++c) dst[c] = Elem<std::remove_cv_t<std::remove_pointer_t<decltype(p)>>>::load(p + (unsigned)min(lane + 64 * c, W - 1));
+        }
+    };
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
         const int row = min(r0 + i, n_rows - 1);
         const int b = row / Sa, s = row % Sa;
         const T* hr = hn + ((long)b * S + n_lead + s) * W;
-#pragma unroll
-        for (int c = 0; c < NC; ++c) hv[i][c] = Elem<T>::load(hr + (unsigned)min(lane + 64 * c, W - 1));
+        load_slots(hr, hv[i]);
     }
     // The rows of W_out are requested together with the activation rows when the norm's own
     // operands leave room for them; with long rows they are requested after the norm instead
@@ -512,8 +544,7 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
 #pragma unroll
         for (int u = 0; u < AU; ++u) {
             const float* wr = W_out + (long)min(a0 + u, A - 1) * W;
-#pragma unroll
-            for (int c = 0; c < NC; ++c) wv[u][c] = wr[(unsigned)min(lane + 64 * c, W - 1)];
+            load_slots(wr, wv[u]);
         }
     };
     if constexpr (W_EARLY) load_w_rows();
@@ -523,17 +554,16 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
         // the value is dropped; under a branch each load would be waited for on its own)
         float g0[NC], g1[NC];
         const T* gw = norm_w ? norm_w : hn;
+        if (NORM == NORM_RMS) {
+            load_slots(gw, g0);
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            const unsigned k = (unsigned)min(lane + 64 * c, W - 1);
-            if (NORM == NORM_RMS) {
-                const float lv = Elem<T>::load(gw + k);
-                g0[c] = norm_w ? lv : 1.f;
+            for (int c = 0; c < NC; ++c) {
+                g0[c] = norm_w ? g0[c] : 1.f;
                 g1[c] = 0.f;
-            } else {
-                g0[c] = sc[k];
-                g1[c] = sh[k];
             }
+        } else {
+            load_slots(sc, g0);
+            load_slots(sh, g1);
         }
 #pragma unroll
         for (int i = 0; i < ROWS; ++i) {
@@ -541,13 +571,13 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
             if (NORM == NORM_ADALN) {
                 float s1 = 0.f;
 #pragma unroll
-                for (int c = 0; c < NC; ++c) s1 += (lane + 64 * c < W) ? hv[i][c] : 0.f;
+                for (int c = 0; c < NC; ++c) s1 += (kidx(c) < W) ? hv[i][c] : 0.f;
                 mean = wave_sum(s1) / (float)W;
             }
             float s2 = 0.f;
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                const float d = (lane + 64 * c < W) ? hv[i][c] - mean : 0.f;
+                const float d = (kidx(c) < W) ? hv[i][c] - mean : 0.f;
                 s2 += d * d;
             }
             const float inv = 1.0f / sqrtf(wave_sum(s2) / (float)W + eps);
@@ -577,7 +607,7 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
             float acc = 0.f;
 #pragma unroll
             for (int c = 0; c < NC; ++c)
-                if (lane + 64 * c < W) acc += wv[u][c] * hv[i][c];
+                if (kidx(c) < W) acc += wv[u][c] * hv[i][c];
             acc = wave_sum(acc);
             if (lane == i * AU + u) mine = acc;
         }
@@ -801,10 +831,17 @@ int euler_launch(float* x_t, const void* hn, int norm, const void* norm_w, const
     if (dtype != VLA_DT_F32 && dtype != VLA_DT_BF16) return VLA_K_ERR_ARG;
     if (W > 64 * 64) return VLA_K_ERR_SHAPE;
     const int n_rows = batch * (S - n_lead);
-#define VLA_EULER_N(T, NC, AU, ROWS, NORM)                                                                          \
-    euler_step_kernel<T, NC, AU, ROWS, NORM>                                                                        \
+    // runs of eight with 16-byte loads when every row starts on a 16-byte boundary
+    const bool vec = W % 8 == 0 && (((uintptr_t)hn | (uintptr_t)W_out | (uintptr_t)norm_w | (uintptr_t)sc | (uintptr_t)sh) & 15) == 0;
+#define VLA_EULER_V(T, NC, AU, ROWS, NORM, VEC)                                                                     \
+    euler_step_kernel<T, NC, AU, ROWS, NORM, VEC>                                                                   \
         <<<dim3((n_rows + EUL_WAVES * ROWS - 1) / (EUL_WAVES * ROWS), (A + AU - 1) / AU), EUL_WAVES * 64, 0, st>>>(  \
             x_t, (const T*)hn, W_out, b_out, n_rows, S, n_lead, A, W, dt, (const T*)norm_w, sc, sh, eps)
+#define VLA_EULER_N(T, NC, AU, ROWS, NORM)                               \
+    do {                                                                 \
+        if (vec && (NC) % 8 == 0) VLA_EULER_V(T, (NC) % 8 ? 8 : (NC), AU, ROWS, NORM, true); \
+        else VLA_EULER_V(T, NC, AU, ROWS, NORM, false);                  \
+    } while (0)
 #define VLA_EULER(T, NC, AU, ROWS)                                       \
     do {                                                                 \
         if (norm == NORM_RMS) VLA_EULER_N(T, NC, AU, ROWS, NORM_RMS);    \
@@ -815,7 +852,7 @@ int euler_launch(float* x_t, const void* hn, int norm, const void* norm_w, const
 #define VLA_EULER_T(T)                                      \
     do {                                                    \
         if (W <= 64 * 8) VLA_EULER(T, 8, 8, 2);             \
-        else if (W <= 64 * 12) VLA_EULER(T, 12, 8, 2);      \
+        else if (W <= 64 * 12 && !vec) VLA_EULER(T, 12, 8, 2); \
         else if (W <= 64 * 16) VLA_EULER(T, 16, 8, 2);      \
         else if (W <= 64 * 24) VLA_EULER(T, 24, 4, 2);      \
         else if (W <= 64 * 32) VLA_EULER(T, 32, 4, 2);      \
@@ -828,6 +865,7 @@ int euler_launch(float* x_t, const void* hn, int norm, const void* norm_w, const
 #undef VLA_EULER_T
 #undef VLA_EULER
 #undef VLA_EULER_N
+#undef VLA_EULER_V
     return VLA_CHECK_LAUNCH();
 }
 }  // namespace
