@@ -599,6 +599,19 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
         __builtin_amdgcn_sched_barrier(0);  // not hoisted back in front of the norm
         load_w_rows();
     }
+    // The V = ROWS x AU per-lane sums.  From eight sums on they are added across the wavefront
+    // together: each exchange step halves the values a lane carries (a lane keeps the upper half
+    // of its values if its bit of that step is set and hands the other half to its partner),
+    // V - 1 exchanges instead of 6 V, then the remaining steps on the one value left; lane l ends
+    // with the total of value l >> (6 - log2 V).  Sixteen sums do the two widest steps with the
+    // half-wave and 16-lane-row swaps (both lanes' new values from one instruction); with eight
+    // that measured slower than the shuffles, and with fewer than eight the one-sum-at-a-time
+    // reduction below is the faster one.
+    constexpr int V = ROWS * AU;
+    static_assert((V & (V - 1)) == 0 && V <= 64, "a power of two of sums");
+    constexpr bool TREE = V >= 8, SWAP = V >= 16;
+    constexpr int SH = !TREE ? 0 : V == 8 ? 3 : V == 16 ? 2 : V == 32 ? 1 : 0;
+    float vals[V];
     float mine = 0.f;
 #pragma unroll
     for (int i = 0; i < ROWS; ++i)
@@ -608,11 +621,40 @@ __global__ void __launch_bounds__(EUL_WAVES * 64) euler_step_kernel(float* __res
 #pragma unroll
             for (int c = 0; c < NC; ++c)
                 if (kidx(c) < W) acc += wv[u][c] * hv[i][c];
-            acc = wave_sum(acc);
-            if (lane == i * AU + u) mine = acc;
+            if (TREE) {
+                vals[i * AU + u] = acc;
+            } else {
+                acc = wave_sum(acc);
+                if (lane == i * AU + u) mine = acc;
+            }
         }
-    const int i = lane / AU, a = a0 + lane % AU;
-    if (lane < ROWS * AU && r0 + i < n_rows && a < A) {
+    if (TREE) {
+        int off = 32;
+#pragma unroll
+        for (int n = V; n > 1; n >>= 1, off >>= 1) {
+            const bool up = (lane & off) != 0;
+#pragma unroll
+            for (int k = 0; k < n / 2; ++k) {
+                const float lo = vals[k], hi = vals[k + n / 2];
+                if (SWAP && off == 32) {
+                    const auto sw =
+                        __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+                    vals[k] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+                } else if (SWAP && off == 16) {
+                    const auto sw =
+                        __builtin_amdgcn_permlane16_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+                    vals[k] = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
+                } else {
+                    vals[k] = (up ? hi : lo) + __shfl_xor(up ? lo : hi, off, 64);
+                }
+            }
+        }
+        mine = vals[0];
+        for (; off > 0; off >>= 1) mine += __shfl_xor(mine, off, 64);
+    }
+    const int v = lane >> SH;
+    const int i = v / AU, a = a0 + v % AU;
+    if ((lane & ((1 << SH) - 1)) == 0 && v < V && r0 + i < n_rows && a < A) {
         float* xp = x_t + (long)(r0 + i) * A + a;
         *xp = *xp + dt * (mine + (b_out ? b_out[a] : 0.f));
     }
