@@ -791,11 +791,12 @@ def test_ternary_gemm_accumulators_and_epilogue_bit_exact(M, N, K, ws_num):
         assert np.array_equal(host(out2), host(out))
 
 
-@pytest.mark.parametrize("tile", [128, 256])
+@pytest.mark.parametrize("tile", [128, 256, 16])
 @pytest.mark.parametrize("M,N,K", [(300, 288, 256), (515, 640, 384), (64, 48, 128)])
 def test_ternary_gemm_large_tile_kernels_bit_exact(tune, tile, M, N, K):
     # The large-M kernels (weights read straight from the fragment-major layout), pinned
-    # by VLA_TERNARY_TILE, on ragged M and N: same int32 accumulators and bf16 epilogue.
+    # by VLA_TERNARY_TILE (16 = the 16x16x64 kernel), on ragged M and N: same int32
+    # accumulators and bf16 epilogue.
     r = np.random.default_rng(tile + M)
     A = r.integers(-127, 128, (M, K)).astype(np.int8)
     ladder = r.integers(0, 256, N * K // 4).astype(np.uint8)
@@ -832,7 +833,7 @@ def test_ternary_gemm_prefill_shape_all_tilings_agree(tune):
     dA, dW, ds, dws = dev(A), dev(_pack_plain(t)), dev(s), dev(ws)
     rowsum = dev(A.astype(np.int32).sum(1).astype(np.int32))
     res = []
-    for tile in (None, 64, 128, 256):
+    for tile in (None, 64, 128, 256, 16):
         if tile is None:
             tune.clear("VLA_TERNARY_TILE")
         else:
@@ -878,7 +879,8 @@ def test_ternary_gemv_decode_rows_bit_exact(M, N, K, ws_num):
     assert np.array_equal(host(h), host(want_sum))
 
 
-@pytest.mark.parametrize("M,N,K,tile", [(300, 288, 256, 64), (300, 288, 256, 128), (515, 640, 384, 256)])
+@pytest.mark.parametrize("M,N,K,tile", [(300, 288, 256, 64), (300, 288, 256, 128), (515, 640, 384, 256), (300, 288, 256, 16),
+                                        (515, 640, 384, 16)])
 def test_ternary_gemm_add_matches_gemm_then_add(tune, M, N, K, tile):
     r = np.random.default_rng(M + tile)
     A = r.integers(-127, 128, (M, K)).astype(np.int8)

@@ -24,13 +24,50 @@ def sources():
     return sorted(glob.glob(os.path.join(HERE, "csrc", "*.hip")) + glob.glob(os.path.join(HERE, "host", "*.cpp")))
 
 
+# Kernels that keep registers "in flight" between an inline-assembly load and its wait must
+# not spill: a spilled in-flight register is stored before its data arrives and reused while
+# the load is still due.  Their scratch size is read from the compiler's resource remarks.
+NO_SPILL_KERNELS = {"gemm.hip": ["ternary_gemm_x16_kernel"]}
+
+
+def _check_no_spill(src, remarks):
+    for kernel in NO_SPILL_KERNELS.get(os.path.basename(src), []):
+        lines = remarks.splitlines()
+        seen = False
+        for i, l in enumerate(lines):
+            if "Function Name:" in l and kernel in l:
+                for m in lines[i:i + 40]:
+                    if "ScratchSize [bytes/lane]:" in m:
+                        seen = True
+                        size = int(m.split("ScratchSize [bytes/lane]:")[1].split()[0])
+                        if size != 0:
+                            raise RuntimeError("%s spills %d bytes per lane: its in-flight registers are not safe" % (kernel, size))
+                        break
+        if not seen:
+            raise RuntimeError("no resource remarks for %s in %s" % (kernel, src))
+
+
 def _compile(src):
     obj = os.path.join(OBJ, os.path.basename(src) + ".o")
-    cmd = [HIPCC] + FLAGS + ["-x", "hip", "-c", src, "-o", obj]
+    extra = ["-Rpass-analysis=kernel-resource-usage"] if os.path.basename(src) in NO_SPILL_KERNELS else []
+    cmd = [HIPCC] + FLAGS + extra + ["-x", "hip", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
+    if extra:
+        _check_no_spill(src, err)
+        # the remarks are not diagnostics: drop them (and their source excerpts) from what verbose builds print
+        keep, skip = [], 0
+        for l in err.splitlines():
+            if "-Rpass-analysis=kernel-resource-usage" in l:
+                skip = 2
+                continue
+            if skip:
+                skip -= 1
+                continue
+            keep.append(l)
+        err = "\n".join(keep)
     return obj, err
 
 

@@ -29,7 +29,7 @@ struct Tuning {
     int gemm_tile = -1;          // VLA_GEMM_TILE: 0..5
     int gemm_dl = -1;            // VLA_GEMM_DL: 0 pins the register-staged GEMM
     int gemm_stages = 0;         // VLA_GEMM_STAGES: ring depth of the direct-to-LDS GEMM
-    int ternary_tile = 0;        // VLA_TERNARY_TILE: 64 | 128 | 256
+    int ternary_tile = 0;        // VLA_TERNARY_TILE: 64 | 128 | 256 (32x32x32 kernels) | 16 (16x16x64 kernel)
 };
 const Tuning& tuning();
 

@@ -1130,6 +1130,287 @@ __global__ void __launch_bounds__(WM * 128, 2) ternary_gemm_big_kernel(GemmArgs 
     }
 }
 
+// ---- Large-M ternary GEMM on v_mfma_i32_16x16x64_i8 (BitVLA prefill) ------------------
+// The 16x16x64 form moves a quarter of the accumulator registers per multiply-add that the
+// 32x32x32 form does, and on this part that is what the matrix pipe's clock follows: the
+// same product streams about a fifth faster.  Everything around the MFMAs is built so that
+// nothing the compiler schedules can sit between a load and its first use:
+//
+//  - int8 activation tiles (128 rows x 128 k) go from global memory straight into a
+//    three-stage LDS ring (global_load_lds_dwordx4, rows unpadded, 16-byte pieces
+//    XOR-swizzled by (row >> 1) & 7 so that a fragment read touches every bank once);
+//  - a wavefront's packed weight words (one dword = 16 codes of one column) go from the
+//    fragment-major layout into registers with inline-assembly loads, refilled in place
+//    right after they are expanded, a full k-tile ahead of their next use;
+//  - both kinds are counted by hand: every pass issues the same loads in the same order,
+//    so "the words of this chunk have landed" is always s_waitcnt vmcnt(NB / 2 + 4), and the
+//    activation tile of a pass is older than that.  One barrier per k-tile.
+//
+// The product is formed as D = W . A^T: a lane ends up with four consecutive output
+// columns of one row, so the row's scale and row sum are per-lane constants (no lane
+// exchange), the accumulators start at -2 * rowsum (the code offset), and the bf16 results
+// go to the LDS staging area as 16-byte pieces (a 16-lane group takes the even columns of
+// a 32-column block in one MFMA and the odd ones in the next, so that its two weight words
+// are one 8-byte load and its eight outputs per row are consecutive).
+//
+// Registers written by the inline-assembly loads are "in flight" until the matching wait.
+// Each of them is an in/out operand of that wait, which keeps the compiler from reading it
+// early and from giving the register to anything else in between.  The kernel must not
+// spill (a spilled in-flight register is stored before its data arrives and its register
+// reused while the load is still due): vla_cpp_amd/build.py checks the scratch size.
+template <int IMM>
+__device__ __forceinline__ void tern_wload_i(u32x2_t& dst, uint32_t voff, const void* sbase) {
+    asm volatile("global_load_dwordx2 %0, %1, %2 offset:%3" : "+v"(dst) : "v"(voff), "s"(sbase), "n"(IMM) : "memory");
+}
+__device__ __forceinline__ void tern_aload_lds(uint32_t voff, const void* sbase, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sbase) : "memory");
+}
+__device__ __forceinline__ void tern_gload(uint32_t& dst, const void* p) {
+    asm volatile("global_load_dword %0, %1, off" : "=v"(dst) : "v"(p) : "memory");
+}
+template <int CNT>
+__device__ __forceinline__ void tern_wait_words(u32x2_t (&w)[4]) {
+    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]) : "n"(CNT));
+}
+
+// 2 x 2 wavefronts, each 64 rows x 128 columns (4 x 8 blocks of 16 x 16); workgroup tile 128 x 256.
+__global__ void __launch_bounds__(256, 2) ternary_gemm_x16_kernel(GemmArgs a) {
+    constexpr int NB = 8, MB = 4, NS = 3, ROWS = 128, CW = 16 * NB, COLS = 2 * CW, STAGE = ROWS * 128;
+    constexpr int CNT = NB / 2 + 4;    // loads younger than a chunk's words when they are waited for
+    constexpr int T_STRIDE = 272;      // staging row: 128 bf16 + 16 bytes
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[NS * STAGE];
+    static_assert(NS * STAGE >= 4 * 16 * T_STRIDE, "epilogue staging must fit in the ring");
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int q = lane >> 4, c = lane & 15;
+    // id % 8 (the XCD) = M tile % 8: workgroups sharing an L2 share their activation rows,
+    // the larger operand, and stream the whole (4x smaller) packed weight matrix.
+    const int m_tiles = (a.M + ROWS - 1) / ROWS, mt_pad = (m_tiles + 7) & ~7;
+    const int mt = blockIdx.x % mt_pad;
+    if (mt >= m_tiles) return;
+    const int m0 = mt * ROWS, n0 = (blockIdx.x / mt_pad) * COLS + wn * CW;
+
+    // Row constants of the lane's four output rows m = m0 + 64 wm + 16 mb + c: requested
+    // before everything else, valid after the first wait of the ring.
+    uint32_t rs_raw[MB], sc_raw[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = min(m0 + wm * 64 + mb * 16 + c, a.M - 1);
+        tern_gload(rs_raw[mb], a.rowsum + m);
+        tern_gload(sc_raw[mb], a.s ? a.s + m : (const float*)(a.rowsum + m));
+    }
+    // The 16 lanes c of a k quarter q take the columns 2 c (block 2 p) and 2 c + 1 (block 2 p + 1) of the 32-column
+    // block n0 / 32 + p: the two words sit side by side in the fragment-major layout (k group 2 chunk + q / 2, half
+    // q % 2), one 8-byte load.  Byte offsets; both operands fit 32 bits (checked by the launcher).
+    const int kgroups = a.K / 32, nblocks = (a.N + 31) / 32;
+    uint32_t woff[NB / 2];
+#pragma unroll
+    for (int p = 0; p < NB / 2; ++p) {
+        const int nb32 = min(n0 / 32 + p, nblocks - 1);  // columns past N: any valid block, result dropped
+        woff[p] = ((uint32_t)nb32 * (uint32_t)kgroups * 64u + (uint32_t)((q >> 1) * 64 + (q & 1) * 32 + 2 * c)) * 4u;
+    }
+    // Activation loader: wavefront w fills the 1 KiB slabs 4 w + v of a stage (8 rows each);
+    // the lane's slot is piece position lane % 8 of row lane / 8 and holds logical piece (lane % 8) ^ ((row >> 1) & 7).
+    uint32_t aoff[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int row = (wave * 4 + v) * 8 + (lane >> 3);
+        const int piece = (lane & 7) ^ ((row >> 1) & 7);
+        aoff[v] = (uint32_t)min(m0 + row, a.M - 1) * (uint32_t)a.K + (uint32_t)(piece * 16);  // rows past M: a valid row, result dropped
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds + wave * 4096;  // low 32 bits of a shared-aperture address = LDS offset
+
+    u32x2_t bw[2][NB / 2] = {};  // [chunk][32-column block]: the words of blocks 2 p and 2 p + 1
+    const int nkt = a.K / 128;
+    const unsigned char* Ab = (const unsigned char*)a.A;
+    const unsigned char* Wb = (const unsigned char*)a.W;
+#define TERN_WLOAD(ch, base) \
+    _Pragma("unroll") for (int p = 0; p < NB / 2; ++p) tern_wload_i<(ch) * 512>(bw[ch][p], woff[p], base);
+#define TERN_ALOAD(ch, abase, lbase)                                   \
+    tern_aload_lds(aoff[(ch) * 2], abase, (lbase) + ((ch) * 2) * 1024); \
+    tern_aload_lds(aoff[(ch) * 2 + 1], abase, (lbase) + ((ch) * 2 + 1) * 1024);
+
+    // Prologue = the issue order of two passes before the first: activation tile 0, then
+    // (words of tile 0, activation tile 1) chunk by chunk.  Past the last tile the ring
+    // keeps re-fetching it, so the counts stay the same to the end.
+#pragma unroll
+    for (int v = 0; v < 4; ++v) tern_aload_lds(aoff[v], Ab, lds0 + v * 1024);
+    {
+        const unsigned char* a1 = Ab + (long)min(1, nkt - 1) * 128;
+        TERN_WLOAD(0, Wb) TERN_ALOAD(0, a1, lds0 + STAGE)
+        TERN_WLOAD(1, Wb) TERN_ALOAD(1, a1, lds0 + STAGE)
+    }
+    // Fragment reads: row 64 wm + 16 mb + c, logical piece 4 ch + q at position (4 ch + q) ^ ((c >> 1) & 7).
+    const int fsw = (c >> 1) & 7;
+    const int fragA = (wm * 64 + c) * 128;
+
+    // Words of (tile 0, chunk 0) have landed, and with them everything older: activation tile 0 and the row constants.
+    tern_wait_words<CNT>(bw[0]);
+    asm volatile("" : "+v"(rs_raw[0]), "+v"(rs_raw[1]), "+v"(rs_raw[2]), "+v"(rs_raw[3]), "+v"(sc_raw[0]), "+v"(sc_raw[1]), "+v"(sc_raw[2]), "+v"(sc_raw[3]));
+    i32x4_t acc[NB][MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int init = -2 * (int)rs_raw[mb];  // 2-bit codes are t + 2: sum_k q (t + 2) - 2 rowsum
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = i32x4_t{init, init, init, init};
+    }
+    int cs = 0, ls = 2;
+    for (int kt = 0; kt < nkt; ++kt) {
+        const unsigned char* cur = lds + cs * STAGE;
+        const unsigned char* wn_base = Wb + (long)min(kt + 1, nkt - 1) * 1024;
+        const unsigned char* an_base = Ab + (long)min(kt + 2, nkt - 1) * 128;
+        const uint32_t lds_ld = lds0 + ls * STAGE;
+        u32x4_t fa[2][MB];
+        __syncthreads();  // every wavefront's loads of this tile have landed; stage ls has been read by everyone
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+            fa[0][mb] = *reinterpret_cast<const u32x4_t*>(cur + fragA + mb * 16 * 128 + ((q ^ fsw) * 16));
+#pragma unroll
+        for (int ch = 0; ch < 2; ++ch) {
+            if (ch > 0) tern_wait_words<CNT>(bw[ch]);
+            u32x4_t fw[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const uint32_t w = bw[ch][nb >> 1][nb & 1];
+                fw[nb][0] = w & 0x03030303u;
+                fw[nb][1] = (w >> 2) & 0x03030303u;
+                fw[nb][2] = (w >> 4) & 0x03030303u;
+                fw[nb][3] = (w >> 6) & 0x03030303u;
+            }
+            // refill the words just expanded with the next k-tile's, then two activation slabs of the tile after that
+            if (ch == 0) { TERN_WLOAD(0, wn_base) TERN_ALOAD(0, an_base, lds_ld) }
+            if (ch == 1) { TERN_WLOAD(1, wn_base) TERN_ALOAD(1, an_base, lds_ld) }
+            if (ch == 0) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    fa[1][mb] = *reinterpret_cast<const u32x4_t*>(cur + fragA + mb * 16 * 128 + (((4 + q) ^ fsw) * 16));
+            }
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+                    acc[nb][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4_t, fw[nb]),
+                                                                        __builtin_bit_cast(i32x4_t, fa[ch][mb]), acc[nb][mb], 0, 0, 0);
+        }
+        tern_wait_words<CNT>(bw[0]);  // the next tile's first chunk (and, older than it, the next activation tile)
+        cs = (cs + 1 == NS) ? 0 : cs + 1;
+        ls = (ls + 1 == NS) ? 0 : ls + 1;
+    }
+#undef TERN_WLOAD
+#undef TERN_ALOAD
+    // the ring's trailing loads (repeats of the last tile) still target the word registers and the LDS stages
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(bw[0][0]), "+v"(bw[0][1]), "+v"(bw[0][2]), "+v"(bw[0][3]), "+v"(bw[1][0]), "+v"(bw[1][1]), "+v"(bw[1][2]), "+v"(bw[1][3]));
+    __syncthreads();
+
+    // acc[nb][mb][i]: column n = n0 + 32 (nb / 2) + 2 (4 q + i) + nb % 2, row m = m0 + 64 wm + 16 mb + c
+    if (a.acc_out) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            const int m = m0 + wm * 64 + mb * 16 + c;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + (nb >> 1) * 32 + 2 * (4 * q + i) + (nb & 1);
+                    if (m < a.M && n < a.N) a.acc_out[(long)m * a.N + n] = acc[nb][mb][i];
+                }
+        }
+    }
+    if (!a.Y) return;
+
+    // bf16 output: out = float(acc) / s[m] * ws[group], staged per wavefront as 16 rows x 128
+    // columns and written with 16-byte stores (16 lanes per row), the residual added on the way.
+    // The quotient is the correctly rounded one.  For a positive scale away from the exponent
+    // limits it is computed with the scale's exponent taken out: y ~ 1 / mantissa by one Newton
+    // step on v_rcp_f32, q0 = a y, one residual correction; for |a| < 2^20 that sequence gives
+    // the IEEE quotient for every mantissa (checked exhaustively on the device), and the power
+    // of two goes back in exactly.  Larger accumulators take a second correction (the compiler's
+    // own sequence without its operand scaling); other scales take the division operator.
+    const int group = a.N / a.ws_num;
+    float wsc[NB / 2];  // one weight scale per 32-column block (the launcher checks that a scale group is a multiple of 32 columns)
+    bool ok = true;
+#pragma unroll
+    for (int p = 0; p < NB / 2; ++p) {
+        wsc[p] = a.ws[min(n0 + p * 32, a.N - 1) / group];
+        const float wa = fabsf(wsc[p]);
+        ok = ok && (wa == 0.f || (wa > 0x1p-60f && wa < 0x1p60f));  // 2^-e ws below is then exact
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const float sm = __uint_as_float(sc_raw[mb]);
+        ok = ok && sm > 0x1p-60f && sm < 0x1p60f;
+    }
+    const bool fast = __builtin_amdgcn_ballot_w64(ok) == ~0ull;
+    const bool one_step = a.K < 8192;  // |acc| <= 128 K < 2^20
+    unsigned char* tp = &lds[0] + wave * (16 * T_STRIDE);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        u32x4_t res_v[4] = {};
+        if (a.residual) {  // this row block's residual vectors, requested ahead of the staging arithmetic
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int m = min(m0 + wm * 64 + mb * 16 + p * 4 + (lane >> 4), a.M - 1), n = min(n0 + (lane & 15) * 8, a.N - 8);
+                res_v[p] = *reinterpret_cast<const u32x4_t*>((const bf16_t*)a.residual + (long)m * a.N + n);
+            }
+        }
+        const float sm = __uint_as_float(sc_raw[mb]);
+        if (fast) {
+            const uint32_t sb = sc_raw[mb];
+            const float mant = __uint_as_float((sb & 0x007fffffu) | 0x3f800000u);      // in [1, 2)
+            const float pw = __uint_as_float(0x7f000000u - (sb & 0x7f800000u));         // 2^-(exponent of sm), exact
+            const float y0 = __builtin_amdgcn_rcpf(mant);
+            const float y = __builtin_fmaf(__builtin_fmaf(-mant, y0, 1.0f), y0, y0);
+#pragma unroll
+            for (int p = 0; p < NB / 2; ++p) {
+                const float pws = pw * wsc[p];  // exact: (q 2^-e) ws and q (2^-e ws) round the same product once
+                u32x4_t o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float r2[2];
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const float av = (float)acc[2 * p + h][mb][i];
+                        const float q0 = av * y;
+                        float q1 = __builtin_fmaf(__builtin_fmaf(-mant, q0, av), y, q0);
+                        if (!one_step) q1 = __builtin_fmaf(__builtin_fmaf(-mant, q1, av), y, q1);
+                        r2[h] = q1 * pws;
+                    }
+                    o[i] = pack_bf2(r2[0], r2[1]);
+                }
+                *reinterpret_cast<u32x4_t*>(tp + c * T_STRIDE + (p * 32 + 8 * q) * 2) = o;
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < NB / 2; ++p) {
+                u32x4_t o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    o[i] = pack_bf2((float)acc[2 * p][mb][i] / sm * wsc[p], (float)acc[2 * p + 1][mb][i] / sm * wsc[p]);
+                *reinterpret_cast<u32x4_t*>(tp + c * T_STRIDE + (p * 32 + 8 * q) * 2) = o;
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int row = p * 4 + (lane >> 4), c16 = lane & 15;
+            u32x4_t v = *reinterpret_cast<const u32x4_t*>(tp + row * T_STRIDE + c16 * 16);
+            const int m = m0 + wm * 64 + mb * 16 + row, n = n0 + c16 * 8;
+            if (m >= a.M || n + 8 > a.N) continue;
+            if (a.residual) {  // out = bf16(out + residual), both already bf16
+                const u32x4_t rr = res_v[p];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    v[e] = pack_bf2(__uint_as_float(v[e] << 16) + __uint_as_float(rr[e] << 16),
+                                    __uint_as_float(v[e] & 0xffff0000u) + __uint_as_float(rr[e] & 0xffff0000u));
+            }
+            // streaming store: the 2 M N bytes leave the L2 as they are produced instead of waiting, dirty, for the
+            // write-back at the end of the kernel (each XCD's L2 would hold its whole share until then)
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4_t*>((bf16_t*)a.Y + (long)m * a.N + n));
+        }
+    }
+}
+
 // Ternary GEMV for a handful of rows (single-token decode, M <= 32).  A workgroup owns 32
 // output columns; its 8 wavefronts each take one eighth of K and multiply it with
 // v_mfma_i32_32x32x32_i8 as C[n][m] = sum_k W[n][k] * A[m][k] (weight fragment as the A
@@ -1440,13 +1721,18 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
             default: launch_cfg<T, kEpi, 1, 1, 128, 6>(a, st); break;
         }
     } else {
-        // VLA_TERNARY_TILE = 64 | 128 | 256 pins the tile (tests and tuning); unset = by shape.
+        // VLA_TERNARY_TILE = 64 | 128 | 256 pins a tile of the 32x32x32 kernels, 16 the 16x16x64 kernel (tests and tuning); unset = by shape.
         const int force = tuning().ternary_tile;
         // Enough 128 x 256 tiles for half the chip: the large-M kernel, two workgroups per
         // CU (measured faster than one 256 x 256 workgroup: fewer wavefronts per barrier).
         const int n256 = (a.N + 255) / 256;
         const long wg128 = (long)((a.M + 127) / 128) * n256;
         const int gemv_groups = (a.K / 32 + GEMV_WAVES - 1) / GEMV_WAVES;  // k groups per wavefront
+        // The 16x16x64 kernel addresses both operands with 32-bit byte offsets, writes 8-column vectors and keeps one
+        // weight scale per 32-column block; anything else stays with the 32x32x32 kernels.
+        const int ws_group = a.N / (a.ws_num > 0 ? a.ws_num : 1);
+        const bool x16_ok = a.N % 8 == 0 && (a.Y == nullptr || ws_group % 32 == 0) && (long)a.M * a.K < (1l << 32) &&
+                            (long)((a.N + 31) / 32) * a.K * 8 < (1l << 32) && ((uintptr_t)a.A % 16 == 0) && a.K % 16 == 0;
         if (force == 0 && a.M <= 32 && gemv_groups <= 28) {
             const unsigned grid = (unsigned)((a.N + 31) / 32);
             if (gemv_groups <= 10) ternary_gemv_kernel<10><<<grid, GEMV_WAVES * 64, 0, st>>>(a);
@@ -1454,6 +1740,10 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
         } else if (force == 256) {
             const unsigned grid = (unsigned)(((((a.M + 255) / 256) + 7) & ~7) * n256);
             ternary_gemm_big_kernel<4><<<grid, 512, 0, st>>>(a);
+        } else if (x16_ok && (force == 16 || (force == 0 && wg128 >= 128))) {
+            // the 16x16x64 kernel: 128 x 256 tiles, two workgroups per CU
+            const unsigned grid = (unsigned)(((((a.M + 127) / 128) + 7) & ~7) * n256);
+            ternary_gemm_x16_kernel<<<grid, 256, 0, st>>>(a);
         } else if (force == 128 || (force == 0 && wg128 >= 128)) {
             const unsigned grid = (unsigned)(((((a.M + 127) / 128) + 7) & ~7) * n256);
             ternary_gemm_big_kernel<2><<<grid, 256, 0, st>>>(a);
