@@ -17,14 +17,18 @@ one more chunk runs with a HIP event recorded after every launch on the launch s
 its predecessors left them and includes the gap to the launch before it.  The events'
 own cost (the marked chunk minus a replayed one, per mark) is subtracted.
 
-Prints ONE JSON line with the contract fields plus
+Prints ONE JSON line (a few KB) with the contract fields plus
   roofline      the step's dominant kernel (largest share of the step's time)
   roofline_kv   the attention launch that reads the most prefix KV
+  roofline_ternary_prefill  the BitVLA prefill QKV GEMM (int8 MFMA roofline)
   cpu_baseline  the CPU oracle (restated reference op sequence, with the reference's
                 per-step concat copies, fp32 SIMD-style accumulation) timed on this host
                 with the reference's thread rule and timing recipe
-  kernels       per launch site: average microseconds, launches per step, roofline fraction
-  other_configs the same summary for every other BASELINE configuration
+  us_per_action_chunk_with_prefix  one chunk plus the once-per-observation prefix K/V build
+  config.workloads  one compact entry per BASELINE configuration and batch size: us per
+                step, chunk p50, chunk with the prefix build, launches per step, and the
+                dominant launch's roofline {kernel, frac, avg_us, traffic}
+--verbose adds the per-launch-site tables (kernels, prefill_kernels, other_configs).
 """
 import argparse
 import json
@@ -327,27 +331,22 @@ def kernel_breakdown(pkg, cfg, B, P):
     return out
 
 
-# HBM-side bytes per launch (L2 misses) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# on this command, KiB per dispatch, each scaled by what the same counter reads for a plain
-# 256 MiB device copy (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000).  Counters cannot be read from
-# inside the process, so these are the figures of profiles/*_pmc.txt (which give the commands);
-# launch sites without a measurement report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("cfg1_smolvla_16layer_bf16_b32", "step.wo_residual"): int((7807.5 * 2 + 2250.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.qkv_rope_append_self"): int((6935.3 * 2 + 5400.2) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.q_rope_cross"): int((5076.5 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_self"): int((7730.2 * 2 + 3000.0) * 1024),
-    ("cfg1_smolvla_16layer_bf16_b32", "step.attention_cross"): int((6588.5 * 2 + 3000.0) * 1024),
-    ("cfg2_pi0_18layer_bf16_b16", "step.attention_self"): int((8824.5 * 2 + 13260.0) * 1024),
-    ("cfg2_pi0_18layer_bf16_b16", "step.qkv_rope_append_self"): int((9220.3 * 2 + 4184.0) * 1024),
-    ("cfg2_pi0_18layer_bf16_b16", "step.wo_residual"): int((11532.0 * 2 + 1632.0) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "step.attention_cross"): int((62725.7 * 2 + 3270.3) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "step.qkv_rope_append_self"): int((20186.6 * 2 + 12789.1) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "step.q_rope_cross"): int((11234.1 * 2 + 3264.0) * 1024),
-    ("cfg3_gr00t_16dit_bf16_b64", "step.wo_residual"): int((12906.6 * 2 + 3264.0) * 1024),
-    ("cfg4_bitvla_30layer_b8", "prefill.ternary_qkv_gemm"): int((22033.0 * 2 + 30720.0) * 1024),
-    ("cfg4_bitvla_30layer_b8", "step.attention"): int((6983.5 * 2 + 1016.2) * 1024),
-}
+# HBM-side bytes per launch (L2 misses) measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on
+# this command, each scaled by what the same counter reads for a plain 256 MiB device copy.
+# Counters cannot be read from inside the process: the figures are those of the committed
+# profile summaries, kept beside them as profiles/hbm_traffic.json (written by the same pass
+# that writes the summaries); launch sites without a measurement report null.
+def measured_traffic():
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "hbm_traffic.json")
+    try:
+        with open(path) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        return {}
+    return {(w, k): int(v["bytes"]) for w, sites in doc.get("workloads", {}).items() for k, v in sites.items()}
+
+
+MEASURED_TRAFFIC_BYTES = measured_traffic()
 
 
 def prefix_tokens(cfg, views):
@@ -469,7 +468,7 @@ def cpu_baseline(cfg, w, obs, B):
                 run()
                 ts.append(time.perf_counter() - t0)
             per = [t / n_units * scale_layers * 1e6 * B for t in ts]
-            sample = ("restated CPU reference (not ggml): 1 observation, 2 of %d layers, prefix prefill + 7 tokens per run "
+            sample = ("restated CPU reference (not ggml, whose AVX-512 / AMX kernels would be several times faster): 1 observation, 2 of %d layers, prefix prefill + 7 tokens per run "
                       "(the prefill is included: the restated reference has no cache to skip it with), 1 warm-up + %d "
                       "repetitions, scaled by layers and batch %d" % (cfg["n_layers"], reps, B))
         else:
@@ -492,7 +491,7 @@ def cpu_baseline(cfg, w, obs, B):
             base = pct(short, 0.5)  # prefix build + one step
             per = [(t - base) / (n2 - n1) * 1e6 * B for t in full]
             what = "denoise step"
-            sample = ("restated CPU reference (not ggml): 1 observation, (chunk of %d steps - chunk of 1 step) / %d, 3 warm-ups + "
+            sample = ("restated CPU reference (not ggml, whose AVX-512 / AMX kernels would be several times faster): 1 observation, (chunk of %d steps - chunk of 1 step) / %d, 3 warm-ups + "
                       "%d repetitions, scaled by batch %d" % (n2, n2 - n1, reps, B))
     finally:
         orc.set_default_accumulation(True)
@@ -578,6 +577,9 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir, isolated=False):
         action_chunk_us=chunk_us,
         device_us_per_step=round(dev_ms * 1e3 / steps, 2), host_us_per_step=round(wall_ms * 1e3 / steps, 2),
         prefix_kv_build_ms=round(prefill_ms, 2),
+        # the reference's chunk is predict() = prefix + steps (src/model.cpp:200-296): the once-per-observation-batch
+        # prefix K/V build (host staging, upload and projections, wall clock) plus one chunk (p50)
+        us_per_action_chunk_with_prefix=round(prefill_ms * 1e3 + chunk_us["p50"], 1),
         sum_launch_us_per_step=round(sum(v["us"] * v["launches"] for v in prof.values()) / spc, 2),
         event_overhead_us_per_launch=round(event_us, 3),
         launches_per_step=round(sum(v["launches"] for v in prof.values()) / float(spc), 1),
@@ -615,6 +617,8 @@ def main():
                          "'none', or a comma-separated list; reported under other_configs")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--isolated", action="store_true", help="also time every kernel alone (replayed, warm caches)")
+    ap.add_argument("--verbose", action="store_true",
+                    help="add the per-launch-site tables of every workload to the line (the default line keeps one compact entry per workload)")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="only run plain device copies of a known size (reference for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -657,10 +661,26 @@ def main():
             c = wl[n]["cfg"]
             spc = c["n_suffix"] if c["arch"] == "bitvla" else c["num_steps"]
             r, _ = run_workload(n, wl[n], 3 * spc, 0, False, tmp, args.isolated)  # whole chunks: graph replays only
-            for k in ("kernels", "prefill_kernels"):  # the headline carries the full tables; keep the line readable
-                r[k] = {a: b for a, b in r[k].items() if "attention" in a or "gemm" in a or "gemv" in a or "qkv" in a or "wo_" in a}
             others.append(r)
     cfg = wl[args.config]["cfg"]
+
+    def compact(r):
+        """One short entry per workload: what the step costs and how its dominant launch sits on its roofline."""
+        rf = r["roofline"] or {}
+        e = {"us_per_denoise_step": r["us_per_denoise_step"], "us_per_action_chunk_p50": r["action_chunk_us"]["p50"],
+             "us_per_action_chunk_with_prefix": r["us_per_action_chunk_with_prefix"], "prefix_kv_build_ms": r["prefix_kv_build_ms"],
+             "launches_per_step": r["launches_per_step"],
+             "roofline": {"kernel": rf.get("kernel"), "bound": rf.get("bound"), "frac": rf.get("frac"), "avg_us": rf.get("avg_us"),
+                          "traffic": rf.get("traffic")}}
+        kv = r.get("roofline_kv")
+        if kv and kv.get("kernel") != rf.get("kernel"):
+            e["roofline_kv"] = {"kernel": kv["kernel"], "frac": kv["frac"], "avg_us": kv["avg_us"], "traffic": kv["traffic"]}
+        tp = r.get("roofline_ternary_prefill")
+        if tp:
+            e["roofline_ternary_prefill"] = {"frac": tp["frac"], "avg_us": tp["avg_us"], "traffic": tp["traffic"]}
+        return e
+
+    every = [main_res] + others
     line = {
         "metric": "us_per_denoise_step", "value": main_res["us_per_denoise_step"], "unit": "us",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
@@ -668,21 +688,28 @@ def main():
         "dtype": "bf16" if cfg["dtype"] == "bf16" else "f32", "data": "synthetic",
         "config": {"workload": args.config, "batch": wl[args.config]["B"], "n_layers": cfg["n_layers"],
                    "prefix_tokens_resident": True, "step": "one denoise step over all expert layers",
-                   "timed_region": "graph replays in steady state (3 whole chunks + warmup steps run before it)"},
+                   "timed_region": "graph replays in steady state (3 whole chunks + warmup steps run before it)",
+                   # every BASELINE workload (both batch sizes), the headline included: us per step, chunk p50 (all steps),
+                   # chunk + the once-per-observation prefix K/V build, launches per step, the dominant launch's roofline
+                   "workloads": {r["workload"]: compact(r) for r in every}},
         "us_per_action_chunk": main_res["us_per_action_chunk"], "action_chunk_us": main_res["action_chunk_us"],
+        "us_per_action_chunk_with_prefix": main_res["us_per_action_chunk_with_prefix"],
+        "prefix_kv_build_ms": main_res["prefix_kv_build_ms"],
         "roofline": main_res["roofline"], "roofline_kv": main_res["roofline_kv"],
         "cpu_baseline": main_res.get("cpu_baseline"),
-        "kernels": main_res["kernels"], "prefill_kernels": main_res["prefill_kernels"],
         "device_us_per_step": main_res["device_us_per_step"], "host_us_per_step": main_res["host_us_per_step"],
         "sum_launch_us_per_step": main_res["sum_launch_us_per_step"], "launches_per_step": main_res["launches_per_step"],
         "event_overhead_us_per_launch": main_res["event_overhead_us_per_launch"],
-        "prefix_kv_build_ms": main_res["prefix_kv_build_ms"],
-        "other_configs": others,
     }
-    if "roofline_ternary_prefill" in main_res:
-        line["roofline_ternary_prefill"] = main_res["roofline_ternary_prefill"]
-    if "kernels_isolated" in main_res:
-        line["kernels_isolated"] = main_res["kernels_isolated"]
+    for r in every:  # the ternary prefill GEMM's roofline, whichever workload ran it (the largest batch wins)
+        if "roofline_ternary_prefill" in r:
+            line["roofline_ternary_prefill"] = dict(r["roofline_ternary_prefill"], workload=r["workload"])
+    if args.verbose:
+        line["kernels"] = main_res["kernels"]
+        line["prefill_kernels"] = main_res["prefill_kernels"]
+        line["other_configs"] = others
+        if "kernels_isolated" in main_res:
+            line["kernels_isolated"] = main_res["kernels_isolated"]
     print(json.dumps(line))
 
 

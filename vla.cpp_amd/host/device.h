@@ -72,6 +72,34 @@ class DevBuf {
     size_t n_ = 0;
 };
 
+// Page-locked host staging memory (hipHostMalloc: allocated, never registered after the
+// fact), grow-only.  Copies from it to the device are asynchronous to the host.
+class PinnedBuf {
+  public:
+    PinnedBuf() = default;
+    PinnedBuf(const PinnedBuf&) = delete;
+    PinnedBuf& operator=(const PinnedBuf&) = delete;
+    ~PinnedBuf() { release(); }
+    void reserve(size_t bytes) {
+        if (bytes <= n_) return;
+        release();
+        VLA_HIP(hipHostMalloc(&p_, bytes, hipHostMallocDefault));
+        n_ = bytes;
+    }
+    void* get() const { return p_; }
+    template <typename T> T* as() const { return static_cast<T*>(p_); }
+    size_t bytes() const { return n_; }
+
+  private:
+    void release() {
+        if (p_) (void)hipHostFree(p_);
+        p_ = nullptr;
+        n_ = 0;
+    }
+    void* p_ = nullptr;
+    size_t n_ = 0;
+};
+
 // bf16 <-> f32 on the host, round to nearest even with NaN quieting.
 inline uint16_t f32_to_bf16(float f) {
     uint32_t u;
@@ -99,5 +127,24 @@ inline void upload_as(DevBuf& dst, const float* src, size_t n, int dtype) {
 }
 
 inline size_t dtype_size(int dtype) { return dtype == 0 ? 4 : 2; }
+
+// dst[i] = src[i] * scale in `dtype` (0 = f32, 1 = bf16, rounded as f32_to_bf16 does).  The
+// bf16 form is written without a branch so that the compiler vectorises it.
+inline void convert_scaled(void* dst, const float* src, size_t n, float scale, int dtype) {
+    if (dtype == 0) {
+        float* d = static_cast<float*>(dst);
+        for (size_t i = 0; i < n; ++i) d[i] = src[i] * scale;
+        return;
+    }
+    uint16_t* d = static_cast<uint16_t*>(dst);
+    for (size_t i = 0; i < n; ++i) {
+        const float f = src[i] * scale;
+        uint32_t u;
+        std::memcpy(&u, &f, 4);
+        const uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+        const uint32_t quiet = (u >> 16) | 0x0040u;
+        d[i] = (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? quiet : rounded);
+    }
+}
 
 }  // namespace vla

@@ -153,6 +153,7 @@ class FlowExpert : public ModelArch {
     int B_ = 0, P_ = 0, pad_start_ = 0, pad_end_ = 0;
     RopeTable rope_prefill_, rope_self_, rope_cross_;
     DevBuf prefix_, prefix_n_, tmpk_, tmpv_, lead_, x0_, xt_, h_, hn_, q_, att_, mid_;
+    PinnedBuf stage_;  // host staging of the prefix embeddings (page-locked)
     KVLayer tmp_kv_;
     AttnWorkspace attn_ws_;
     std::mt19937 rng_{std::random_device{}()};
@@ -596,20 +597,26 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
     const int B = batch;
     Ctx C;  // prefill runs on the default stream and is synchronous
 
-    // ---- prefix embeddings, assembled in fp32 on the host
-    std::vector<float> pe((size_t)B * P * Wv_, 0.f);
+    // ---- prefix embeddings: scaled and converted to the model's dtype straight from the
+    // callers' buffers into page-locked staging memory by a few threads, an observation per
+    // task, and sent to the device in groups while the next group is being converted (the
+    // copies are asynchronous; everything below runs on the same stream, after them)
+    const size_t es = dtype_size(dt_);
+    stage_.reserve((size_t)B * P * Wv_ * es);
+    char* const pe = stage_.as<char>();
     const float lang_scale = std::sqrt((float)Wv_);
-    for (int b = 0; b < B; ++b) {
-        float* dst = pe.data() + (size_t)b * P * Wv_;
+    const float img_scale = arch_ == Arch::SMOLVLA ? lang_scale : 1.0f;  // smolvla.cpp:1363 vs pi0.cpp:554-555
+    std::vector<float> lead_host((size_t)B * std::max(n_lead_, 0) * W_);  // the state (and future) rows in front of the actions
+    auto stage_obs = [&](int b) {
+        char* dst = pe + (size_t)b * P * Wv_ * es;
         // alternating layers project the image rows and the text rows separately: all image
         // rows of the batch first, then all text rows, each block [B][rows][Wv]
-        float* txt_dst = dst + (size_t)n_img_tot * Wv_;
+        char* txt_dst = dst + (size_t)n_img_tot * Wv_ * es;
         if (alt_vl_) {
-            dst = pe.data() + (size_t)b * n_img_tot * Wv_;
-            txt_dst = pe.data() + ((size_t)B * n_img_tot + (size_t)b * n_lang) * Wv_;
+            dst = pe + (size_t)b * n_img_tot * Wv_ * es;
+            txt_dst = pe + ((size_t)B * n_img_tot + (size_t)b * n_lang) * Wv_ * es;
         }
-        const float img_scale = arch_ == Arch::SMOLVLA ? lang_scale : 1.0f;  // smolvla.cpp:1363 vs pi0.cpp:554-555
-        for (size_t i = 0; i < (size_t)n_img_tot * Wv_; ++i) dst[i] = in[b].precomputed_img_emb[i] * img_scale;
+        convert_scaled(dst, in[b].precomputed_img_emb, (size_t)n_img_tot * Wv_, img_scale, dt_);
         if (arch_ != Arch::GR00T || alt_vl_) {
             const int rows = arch_ == Arch::SMOLVLA ? n_lang_max_ : n_lang;
             const float ls = alt_vl_ ? 1.0f : lang_scale;  // N1.6: the rows stand for backbone features, unscaled
@@ -623,14 +630,15 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
             for (int i = 0; i < rows; ++i) {
                 const int tok = i < n_lang ? in[b].lang_tokens[i] : 0;  // zero-padded ids, smolvla.cpp:1628-1629
                 const float* e = lang_rows_ ? fetched.data() + (size_t)i * Wv_ : E_lang_.data() + (size_t)tok * Wv_;
-                float* row = txt_dst + (size_t)i * Wv_;
-                for (int c = 0; c < Wv_; ++c) row[c] = e[c] * ls;
+                convert_scaled(txt_dst + (size_t)i * Wv_ * es, e, (size_t)Wv_, ls, dt_);
             }
         }
         std::vector<float> st(max_state_, 0.f);
         if (in[b].state) std::copy(in[b].state, in[b].state + max_state_, st.begin());
         if (arch_ == Arch::SMOLVLA) {
-            host_linear(Wstate_.data(), bstate_.data(), st.data(), dst + (size_t)(P - 1) * Wv_, Wv_, max_state_);
+            std::vector<float> row(Wv_);
+            host_linear(Wstate_.data(), bstate_.data(), st.data(), row.data(), Wv_, max_state_);
+            convert_scaled(dst + (size_t)(P - 1) * Wv_ * es, row.data(), (size_t)Wv_, 1.0f, dt_);
         } else if (head_io_) {
             // encode_state (relu between the two projections), then the learned future tokens
             std::vector<float> h1(Hs_), ld((size_t)n_lead_ * W_);
@@ -638,14 +646,39 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
             for (float& v : h1) v = v > 0.f ? v : 0.f;
             host_linear(se_l2W_.data(), se_l2b_.data(), h1.data(), ld.data(), W_, Hs_);
             std::copy(future_.begin(), future_.end(), ld.begin() + W_);
-            VLA_HIP(hipMemcpy(lead_.as<float>() + (size_t)b * n_lead_ * W_, ld.data(), ld.size() * sizeof(float), hipMemcpyHostToDevice));
+            std::copy(ld.begin(), ld.end(), lead_host.begin() + (size_t)b * n_lead_ * W_);
         } else if (n_lead_ > 0) {
-            std::vector<float> ld(W_);
-            host_linear(W_sp_.data(), b_sp_.data(), st.data(), ld.data(), W_, max_state_);
-            VLA_HIP(hipMemcpy(lead_.as<float>() + (size_t)b * W_, ld.data(), W_ * sizeof(float), hipMemcpyHostToDevice));
+            host_linear(W_sp_.data(), b_sp_.data(), st.data(), lead_host.data() + (size_t)b * W_, W_, max_state_);
         }
+    };
+    {
+        const int nthr = std::max(1, std::min(default_cpu_threads(), B));
+        const int n_groups = alt_vl_ ? 1 : std::min(B, 4);  // the alternating layout interleaves observations: one copy at the end
+        for (int gi = 0; gi < n_groups; ++gi) {
+            const int b0 = (int)((long)B * gi / n_groups), b1 = (int)((long)B * (gi + 1) / n_groups);
+            if (nthr == 1 || b1 - b0 == 1) {
+                for (int b = b0; b < b1; ++b) stage_obs(b);
+            } else {
+                std::vector<std::thread> pool;
+                std::vector<std::string> errors(nthr);
+                for (int t = 0; t < nthr; ++t)
+                    pool.emplace_back([&, t]() {
+                        try {
+                            for (int b = b0 + t; b < b1; b += nthr) stage_obs(b);
+                        } catch (const std::exception& e) {
+                            errors[t] = e.what();
+                        }
+                    });
+                for (auto& th : pool) th.join();
+                for (const std::string& e : errors)
+                    if (!e.empty()) throw std::runtime_error(e);
+            }
+            const size_t off = alt_vl_ ? 0 : (size_t)b0 * P * Wv_ * es;
+            const size_t len = alt_vl_ ? (size_t)B * P * Wv_ * es : (size_t)(b1 - b0) * P * Wv_ * es;
+            VLA_HIP(hipMemcpyAsync((char*)prefix_.get() + off, pe + off, len, hipMemcpyHostToDevice, C.stream));
+        }
+        if (!lead_host.empty()) VLA_HIP(hipMemcpy(lead_.get(), lead_host.data(), lead_host.size() * sizeof(float), hipMemcpyHostToDevice));
     }
-    upload_as(prefix_, pe.data(), pe.size(), dt_);
 
     // ---- positions and masks (smolvla.cpp:1633-1672, pi0.cpp:612-616)
     pad_start_ = pad_end_ = 0;
