@@ -1203,6 +1203,261 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
         }
 }
 
+// ---- Streaming form of the register-direct kernel: many (batch, kv head) pairs with few
+// query rows over a long resident prefix (GR00T's cross blocks: 17 rows onto 296 cached keys
+// of 48-wide heads, 2048 pairs at batch 64).  The launch is bound by how many cache lines a
+// CU keeps in flight, so every request is made a whole line that is used once:
+//
+//  - K and V^T go from the cache straight into LDS (global_load_lds_dwordx4) in the order
+//    they lie in memory: a 32-key block of K is one contiguous run, a 64-key stretch of the
+//    V^T rows is one line per row.  Nothing is fetched twice and no request covers part of
+//    a line, which the fragment-order register loads of the direct kernel do for V^T.
+//  - One wavefront per SIMD owns a private LDS ring (four K blocks, three V^T stretches,
+//    one Q tile: 38 KiB) and walks its pairs one after the other.  The ring does not stop
+//    at a pair's end: the next pair's first blocks and its query tile are requested while
+//    the current pair's last blocks are multiplied, so only the first pair's head and the
+//    last pair's tail are exposed.  No barriers: a ring belongs to one wavefront.
+//  - Loads complete in order and every step issues the same loads, so "block b has
+//    landed" is s_waitcnt vmcnt(24) at every step (the once-per-pair query loads only make
+//    that wait cover a little more).  No register is a load target: nothing to keep alive.
+//
+// LDS rows are 128 bytes (K and Q rows padded from 96), 16-byte pieces XOR-swizzled by
+// (row >> 1) & 7: the loading lane picks the global piece that belongs in its slot.  The
+// arithmetic per block is the direct kernel's, in the same order: the two give the same bits.
+__device__ __forceinline__ void dma16(uint32_t voff, const void* sbase, uint32_t lds_base) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(sbase) : "memory");
+}
+// A wavefront-uniform pointer the compiler may hold in vector registers, moved to scalar ones (the address operand above).
+__device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const unsigned char*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+template <int N>
+__device__ __forceinline__ void wait_vm_mem() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <int D>
+__global__ void __launch_bounds__(256, 1) attn_stream_kernel(AttnArgs a, int n_units) {
+    constexpr int EB = 2, NQ = D / 16, NDB = (D + 31) / 32, PIECES = D * EB / 16;
+    constexpr int KBLK = 32 * 128, VBLK = D * 128, QBUF = 32 * 128, NKS = 4, NVS = 3, NVI = D / 8;
+    constexpr int WAVE_LDS = NKS * KBLK + NVS * VBLK + QBUF;
+    static_assert(WAVE_LDS % 1024 == 0 && 4 * WAVE_LDS <= 160 * 1024, "four rings per CU");
+    static_assert(D % 16 == 0 && D * EB <= 128, "rows of at most 128 bytes");
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[4 * WAVE_LDS];
+
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int g = lane >> 5, r = lane & 31;
+    const int n_waves = gridDim.x * 4, w = blockIdx.x * 4 + wave;
+    if (w >= n_units) return;  // whole wavefront; the kernel has no barriers
+    const int n_my = (n_units - w + n_waves - 1) / n_waves;  // pairs w, w + n_waves, ...
+    const int grp = a.Hq / a.Hkv, R = grp * a.S;
+    const int NBU = 2 * ((a.n_keys + 63) / 64);  // 32-key blocks per pair (whole 64-key stretches)
+    const int total = n_my * NBU;
+
+    unsigned char* const wl = lds + wave * WAVE_LDS;
+    const uint32_t ldsK = (uint32_t)(uintptr_t)wl, ldsV = ldsK + NKS * KBLK, ldsQ = ldsV + NVS * VBLK;
+    const unsigned char* const pK = wl;
+    const unsigned char* const pV = wl + NKS * KBLK;
+    const unsigned char* const pQ = wl + NKS * KBLK + NVS * VBLK;
+
+    // Loader side: lane i fills slot i % 8 of row i / 8 of each 1 KiB slab.
+    const int lrow = lane >> 3, slot = lane & 7;
+    uint32_t kvoff[4], vvoff[NVI], qvoff[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = 8 * j + lrow;
+        int piece = slot ^ ((row >> 1) & 7);
+        piece = piece < PIECES ? piece : 0;  // the padding slots of a row repeat its first piece (same line, never read)
+        kvoff[j] = (uint32_t)(row * D * EB + piece * 16);
+        int rr = min(row, R - 1);  // query rows past R repeat the last one; their outputs are dropped
+        qvoff[j] = (uint32_t)((((rr % a.S) * a.Hq + rr / a.S) * D) * EB + piece * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < NVI; ++j) {
+        const int d = 8 * j + lrow;
+        const int piece = slot ^ ((d >> 1) & 7);
+        vvoff[j] = (uint32_t)(d * a.t_max * EB + piece * 16);
+    }
+    // Issue streams: each keeps its own (pair index, position); past the last pair they repeat its last item.
+    int kI_u = 0, kI_b = 0, vI_u = 0, vI_s = 0, qI_u = 0;
+    const int NSU = NBU / 2;
+    auto pair_of = [&](int ui) { return w + min(ui, n_my - 1) * n_waves; };
+    auto issueK = [&](int st) __attribute__((always_inline)) {
+        const int pr = pair_of(kI_u), lb = kI_u < n_my ? kI_b : NBU - 1;
+        const unsigned char* base = uniform_ptr((const unsigned char*)a.k_cache + ((long)pr * a.t_max + (long)lb * 32) * D * EB);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dma16(kvoff[j], base, ldsK + st * KBLK + j * 1024);
+        if (++kI_b == NBU) { kI_b = 0; ++kI_u; }
+    };
+    auto issueV = [&](int st) __attribute__((always_inline)) {
+        const int pr = pair_of(vI_u), ls = vI_u < n_my ? vI_s : NSU - 1;
+        const unsigned char* base = uniform_ptr((const unsigned char*)a.vt_cache + (long)pr * D * a.t_max * EB + (long)ls * 128);
+#pragma unroll
+        for (int j = 0; j < NVI; ++j) dma16(vvoff[j], base, ldsV + st * VBLK + j * 1024);
+        if (++vI_s == NSU) { vI_s = 0; ++vI_u; }
+    };
+    auto issueQ = [&]() __attribute__((always_inline)) {
+        const int pr = pair_of(qI_u), b = pr / a.Hkv, hk = pr % a.Hkv;
+        const unsigned char* base = uniform_ptr((const unsigned char*)a.q + (((long)b * a.S) * a.Hq + hk * grp) * D * EB);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) dma16(qvoff[j], base, ldsQ + j * 1024);
+        ++qI_u;
+    };
+
+    // Consumer side (the direct kernel's fragments): score row r of a block is key
+    // key_of_score_row(r); V^T row d = 32 db + r (rows past D repeat row D - 1, outputs dropped).
+    const int krow = key_of_score_row(r);
+    const int kfrag = krow * 128, ksw = (krow >> 1) & 7;
+    int vfrag[NDB], vsw[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        const int d = min(db * 32 + r, D - 1);
+        vfrag[db] = d * 128;
+        vsw[db] = (d >> 1) & 7;
+    }
+    const int qfrag = r * 128, qsw = (r >> 1) & 7;
+
+    u32x4_t qf[NQ];
+    f32x16_t o[NDB];
+    float m_run = -INFINITY, l_run = 0.f;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float c2 = a.scale * LOG2E;
+    auto reset = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+        m_run = -INFINITY;
+        l_run = 0.f;
+    };
+    reset();
+
+    auto compute = [&](int kst, int vst, int half, int k0) __attribute__((always_inline)) {
+        const unsigned char* kb = pK + kst * KBLK + kfrag;
+        u32x4_t kr[NQ];
+#pragma unroll
+        for (int c = 0; c < NQ; ++c) kr[c] = *reinterpret_cast<const u32x4_t*>(kb + (((2 * c + g) ^ ksw) * 16));
+        u32x4_t vr[NDB][2];
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+                vr[db][hh] = *reinterpret_cast<const u32x4_t*>(pV + vst * VBLK + vfrag[db] + (((half * 4 + hh * 2 + g) ^ vsw[db]) * 16));
+        f32x16_t sc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[i] = 0.f;
+#pragma unroll
+        for (int c = 0; c < NQ; ++c) AT<bf16_t>::mma(sc, kr[c], qf[c]);
+        float p[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) p[i] = sc[i] * c2;
+        if (k0 + 32 > a.n_keys) {  // uniform: the pair's last blocks; stale cache contents past n_keys must not reach the sums
+            const int kl = k0 + 8 * g;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) p[e] = (kl + key_of_element(e, 0) < a.n_keys) ? p[e] : -INFINITY;
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const int nvalid = a.n_keys - (k0 + hh * 16 + 8 * g);
+#pragma unroll
+                for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        vr[db][hh][e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+            }
+        }
+        float m_blk = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) m_blk = fmaxf(m_blk, p[i]);
+        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
+        if (__builtin_amdgcn_ballot_w64(m_blk > m_run + RESCALE_LOG2) != 0) {  // lazy reference update
+            const float m_new = fmaxf(m_run, m_blk);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - ((m_new == -INFINITY) ? 0.f : m_new));
+            l_run *= alpha;
+            m_run = m_new;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[db][i] *= alpha;
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            p[i] = __builtin_amdgcn_exp2f(p[i] - m_use);
+            psum += p[i];
+        }
+        psum += __shfl_xor(psum, 32, 64);
+        l_run += psum;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            const float* pp = &p[hh * 8];
+            u32x4_t pf;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) pf[e] = pack_bf2(pp[2 * e], pp[2 * e + 1]);
+#pragma unroll
+            for (int db = 0; db < NDB; ++db) AT<bf16_t>::mma(o[db], vr[db][hh], pf);
+        }
+    };
+
+    // Prologue: the issue order of the steps before the first (Q, then V stretch, K block, K block, ...).
+    issueQ();
+    issueV(0);
+    issueK(0);
+    issueK(1);
+    issueV(1);
+    issueK(2);
+    issueK(3);
+    issueV(2);
+    // At step b the youngest load needed is K block b, issued at the end of step b - 4.  Younger than it:
+    // three K blocks (12 loads) and two V^T stretches (2 NVI), whichever the parity of b.
+    constexpr int YOUNGER = 12 + 2 * NVI;
+    int lb = 0, ui = 0, kst = 0, vst = 0;
+    for (int gb = 0; gb < total; gb += 2) {
+        wait_vm_mem<YOUNGER>();
+        if (lb == 0) {  // uniform: a pair begins
+#pragma unroll
+            for (int c = 0; c < NQ; ++c) qf[c] = *reinterpret_cast<const u32x4_t*>(pQ + qfrag + (((2 * c + g) ^ qsw) * 16));
+            // the next pair's query tile: the data lands long after the reads above have left the LDS pipeline
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            issueQ();
+        }
+        compute(kst, vst, 0, lb * 32);
+        issueK(kst);
+        kst = (kst + 1) & 3;
+        wait_vm_mem<YOUNGER>();
+        compute(kst, vst, 1, lb * 32 + 32);
+        issueK(kst);
+        kst = (kst + 1) & 3;
+        issueV(vst);
+        vst = vst == NVS - 1 ? 0 : vst + 1;
+        lb += 2;
+        if (lb == NBU) {  // uniform: the pair is complete
+            const int pr = w + ui * n_waves, b = pr / a.Hkv, hk = pr % a.Hkv;
+            if (r < R) {
+                const int hg = r / a.S, s = r % a.S, h = hk * grp + hg;
+                const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+                unsigned char* orow = (unsigned char*)a.out + (((long)b * a.S + s) * a.Hq + h) * D * EB;
+#pragma unroll
+                for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const int d = db * 32 + 8 * j + 4 * g;
+                        if (d >= D) continue;
+                        const u32x2_t pk = {pack_bf2(o[db][4 * j] * inv, o[db][4 * j + 1] * inv),
+                                            pack_bf2(o[db][4 * j + 2] * inv, o[db][4 * j + 3] * inv)};
+                        *reinterpret_cast<u32x2_t*>(orow + d * EB) = pk;
+                    }
+            }
+            reset();
+            lb = 0;
+            ++ui;
+        }
+    }
+    wait_vm_mem<0>();  // the ring's trailing loads still target this wavefront's LDS
+}
+
 // Merge of key-split partials as a launch of its own: one wavefront per (pair, row).
 template <typename T, bool HALF>
 __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
@@ -1318,6 +1573,19 @@ int launch_direct(AttnArgs& a, hipStream_t st, Scratch& sc) {
     const Tuning& tn = tuning();
     const int n_pairs = a.batch * a.Hkv;
     const int R = (a.Hq / a.Hkv) * a.S;
+    if constexpr (D == 48) {
+        // Enough pairs for every SIMD to walk at least one, keys in whole 64-key stretches inside the cache rows, nothing
+        // masked: the streaming form (the same bits as the kernel below).
+        if (!a.p2 && R <= 32 && n_pairs >= 1024 && a.n_keys >= 128 && a.t_max % 64 == 0 && a.mask == nullptr &&
+            a.mask_kind == VLA_MASK_NONE && a.pad_start >= a.pad_end && !tn.attn_no_stream) {
+            if (sc.kind == Scratch::DRY) return VLA_K_OK;
+            a.n_rblocks = 1;
+            a.n_split = 1;
+            const unsigned grid = (unsigned)std::min(256, (n_pairs + 3) / 4);
+            attn_stream_kernel<D><<<grid, 256, 0, st>>>(a, n_pairs);
+            return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+        }
+    }
     a.n_rblocks = (R + 31) / 32;
     const int n_units = n_pairs * a.n_rblocks;  // (pair, 32-row block)
     const int nb_total = (a.n_keys + 31) / 32;

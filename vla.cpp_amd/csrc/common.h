@@ -25,6 +25,7 @@ struct Tuning {
     bool attn_part_f32 = false;  // VLA_ATTN_PART_F32: fp32 partials where fp16 would be used
     bool attn_no_arrive = false; // VLA_ATTN_NO_ARRIVE: no in-launch merge by the last slice to arrive
     bool attn_no_direct = false; // VLA_ATTN_NO_DIRECT: never the register-direct kernel
+    bool attn_no_stream = false; // VLA_ATTN_NO_STREAM: never the streaming (LDS-ring) form of the register-direct kernel
     int attn_direct_rows = 32;   // VLA_ATTN_DIRECT_ROWS: row limit of the register-direct kernel
     int gemm_tile = -1;          // VLA_GEMM_TILE: 0..5
     int gemm_dl = -1;            // VLA_GEMM_DL: 0 pins the register-staged GEMM
