@@ -1287,8 +1287,11 @@ __global__ void __launch_bounds__(256, 1) attn_stream_kernel(AttnArgs a, int n_u
     auto issueK = [&](int st) __attribute__((always_inline)) {
         const int pr = pair_of(kI_u), lb = kI_u < n_my ? kI_b : NBU - 1;
         const unsigned char* base = uniform_ptr((const unsigned char*)a.k_cache + ((long)pr * a.t_max + (long)lb * 32) * D * EB);
+        // eight-row slabs wholly past n_keys repeat the block's first slab (lines already on their way) instead of
+        // fetching rows nobody reads: the load count per block stays the same, the bytes do not
+        const int rows_left = a.n_keys - lb * 32;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dma16(kvoff[j], base, ldsK + st * KBLK + j * 1024);
+        for (int j = 0; j < 4; ++j) dma16(8 * j < rows_left ? kvoff[j] : kvoff[0], base, ldsK + st * KBLK + j * 1024);
         if (++kI_b == NBU) { kI_b = 0; ++kI_u; }
     };
     auto issueV = [&](int st) __attribute__((always_inline)) {
