@@ -125,8 +125,9 @@ VLA_API int32_t vla_predict_batch(vla_model * m, const vla_inputs * in, int32_t 
  * instead of replaying its graph.  vla_profile_end synchronises, disarms and writes a JSON
  * object {"phase.label": {"us": average, "launches": count}, ...} -- the time from the
  * previous launch's end to this launch's end on the stream, i.e. the launch in its real
- * sequence, cold caches and dependent-launch gap included.  Returns the string length, or the
- * negated size needed when cap is too small, or a vla_status. */
+ * sequence, cold caches and dependent-launch gap included.  Returns the string length, or a
+ * vla_status (-1 .. -3), or, when cap is too small, -16 - (the size needed): the profile is then
+ * kept (nothing is disarmed) and the call can be repeated with a larger buffer. */
 VLA_API int32_t vla_profile_begin(vla_model * m);
 VLA_API int64_t vla_profile_end(vla_model * m, char * json_out, int64_t cap);
 

@@ -237,11 +237,16 @@ VLA_KAPI int vla_attn_prefix_suffix(const void* q, const void* k_cache, const vo
 /* The same call with the scratch memory owned by the caller -- what a model handle uses, so
  * that the reference's rule "one vla_predict at a time per handle" (include/vla.h:18-19) is
  * all a caller has to keep: handles never share scratch.
- *   vla_attn_workspace_bytes: bytes the shape needs, 0 when it needs none (or is not
- *     supported); depends on the shape only, not on pointers.
+ *   vla_attn_workspace_bytes: bytes the shape needs, 0 when it needs none,
+ *     VLA_ATTN_WORKSPACE_UNSUPPORTED when no kernel takes the shape.  It depends on the shape
+ *     and on the tuning overrides in force (VLA_ATTN_SPLIT, VLA_ATTN_DIRECT_ROWS,
+ *     VLA_ATTN_NO_ARRIVE, VLA_ATTN_PART_F32, VLA_ATTN_DL change how the keys are sliced), not on
+ *     pointers: size a workspace after the last vla_kernels_reload_env, or launches return
+ *     VLA_K_ERR_WORKSPACE (nothing is written out of bounds either way).
  *   workspace: device memory of at least that many bytes, 16-byte aligned, zero-filled once
  *     before its first use (every launch leaves the part that must stay zero at zero);
  *     NULL is accepted when the shape needs none.  VLA_K_ERR_WORKSPACE if it is too small. */
+#define VLA_ATTN_WORKSPACE_UNSUPPORTED ((size_t)-1)
 VLA_KAPI size_t vla_attn_workspace_bytes(int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
                                          int n_keys);
 VLA_KAPI int vla_attn_prefix_suffix_ws(const void* q, const void* k_cache, const void* vt_cache, void* out,
@@ -496,8 +501,13 @@ VLA_KAPI const char* vla_kernels_arch(void); /* "gfx950" */
  * vla_attn_prefix_suffix_noalloc.  0 or a vla_kstatus. */
 VLA_KAPI int vla_kernels_init(void);
 /* Reads the tuning overrides (VLA_ATTN_*, VLA_GEMM_*, VLA_TERNARY_TILE; tests and tuning
- * only) from the environment again.  No launch path reads the environment. */
+ * only) from the environment again.  No launch path reads the environment.  Not thread-safe
+ * against launches: call it while no other thread is inside the library.  Workspaces sized
+ * before the call (vla_attn_workspace_bytes, a model handle's own) may be too small after it:
+ * a handle plans its workspace again at its next prefill. */
 VLA_KAPI void vla_kernels_reload_env(void);
+/* Number of vla_kernels_reload_env calls so far: what a holder of a planned workspace compares to know that it must plan again. */
+VLA_KAPI int vla_kernels_tuning_generation(void);
 
 #ifdef __cplusplus
 }

@@ -213,7 +213,11 @@ def test_gr00t_head_gguf_equals_the_vlaw_checkpoint(tmp_path, monkeypatch):
     assert np.array_equal(_chunk(pg, obs, (2, 16, 32)), want)
     monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "3")  # another row of the stacks: other weights
     assert not np.array_equal(_chunk(pg, obs, (2, 16, 32)), want)
+    # an unknown tag keeps the default id with a warning, as the reference does (src/models/gr00tn1d5.cpp:154-160)
     monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "no_such_tag")
+    assert np.array_equal(_chunk(pg, obs, (2, 16, 32)), want)
+    # an id outside the stacks fails the load (gr00tn1d5.cpp:162-166)
+    monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "4096")
     from vla_cpp_amd import ffi
     with pytest.raises(RuntimeError):
         ffi.Model(pg)

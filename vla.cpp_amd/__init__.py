@@ -90,6 +90,7 @@ KERNEL_API = {
     "vla_kernels_arch": [],
     "vla_kernels_init": [],
     "vla_kernels_reload_env": [],
+    "vla_kernels_tuning_generation": [],
 }
 _RESTYPES = {"vla_kernels_arch": ctypes.c_char_p, "vla_attn_workspace_bytes": ctypes.c_size_t,
              "vla_kernels_reload_env": None, "vla_ternary_packed_words": ctypes.c_long,

@@ -1580,8 +1580,8 @@ int launch_direct(AttnArgs& a, hipStream_t st, Scratch& sc) {
         // Enough pairs for every SIMD to walk at least one, keys in whole 64-key stretches inside the cache rows, nothing
         // masked: the streaming form (the same bits as the kernel below).
         if (!a.p2 && R <= 32 && n_pairs >= 1024 && a.n_keys >= 128 && a.t_max % 64 == 0 && a.mask == nullptr &&
-            a.mask_kind == VLA_MASK_NONE && a.pad_start >= a.pad_end && !tn.attn_no_stream) {
-            if (sc.kind == Scratch::DRY) return VLA_K_OK;
+            a.mask_kind == VLA_MASK_NONE && a.pad_start >= a.pad_end && !tn.attn_no_stream && sc.kind != Scratch::DRY) {
+            // (a dry run does not know the cache rows' length: it sizes for the kernel below, which needs at least as much)
             a.n_rblocks = 1;
             a.n_split = 1;
             const unsigned grid = (unsigned)std::min(256, (n_pairs + 3) / 4);
@@ -1910,7 +1910,7 @@ extern "C" size_t vla_attn_workspace_bytes(int dtype, int batch, int S, int n_q_
     const int t_max = (n_keys + 7) / 8 * 8;
     const int rc = attn_entry(nullptr, nullptr, nullptr, nullptr, dtype, batch, S, n_q_heads, n_kv_heads, head_dim, t_max,
                               n_keys, 1.0f, VLA_MASK_NONE, 0, 0, 0, nullptr, nullptr, sc);
-    return rc == VLA_K_OK ? sc.need : 0;
+    return rc == VLA_K_OK ? sc.need : VLA_ATTN_WORKSPACE_UNSUPPORTED;
 }
 
 extern "C" int vla_attn_prefix_suffix_ws(const void* q, const void* k_cache, const void* vt_cache, void* out, int dtype,

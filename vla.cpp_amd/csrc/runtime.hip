@@ -17,6 +17,7 @@ namespace {
 std::mutex g_mu;
 Tuning g_tuning;
 std::atomic<bool> g_loaded{false};
+std::atomic<int> g_generation{0};  // bumped by every reload: holders of workspaces sized under the old overrides re-plan
 
 int env_int(const char* name, int unset) {
     const char* e = getenv(name);
@@ -90,6 +91,9 @@ const char* vla_kernels_arch(void) { return "gfx950"; }
 void vla_kernels_reload_env(void) {
     std::lock_guard<std::mutex> lk(vk::g_mu);
     vk::load_locked();
+    vk::g_generation.fetch_add(1, std::memory_order_relaxed);
 }
+
+int vla_kernels_tuning_generation(void) { return vk::g_generation.load(std::memory_order_relaxed); }
 
 }  // extern "C"

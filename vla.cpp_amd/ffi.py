@@ -174,8 +174,11 @@ class Model:
     def profile_end(self):
         """{"phase.label": {"us": ..., "launches": ...}} for the launches since profile_begin()."""
         import json
-        buf = ctypes.create_string_buffer(1 << 16)
+        buf = ctypes.create_string_buffer(1 << 12)
         n = self._L.vla_profile_end(self._h, buf, len(buf))
+        if n < -16:  # too small: the profile is kept, the size needed is -16 - n
+            buf = ctypes.create_string_buffer(-16 - n)
+            n = self._L.vla_profile_end(self._h, buf, len(buf))
         if n < 0:
             raise RuntimeError("vla_profile_end returned %d" % n)
         return json.loads(buf.value.decode())

@@ -110,6 +110,7 @@ class BitvlaLm : public ModelArch {
 
   private:
     uint32_t alloc_gen_ = 0;
+    int tuning_gen_ = -1;
     DevBuf zeros_;
     // last_out: where the last layer's closing projection writes the hidden rows (nullptr: in
     // place); honoured on the few-row decode path only, returns whether it was.  first_in: the
@@ -204,7 +205,9 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
             if (in[b].lang_tokens[i] < 0 || in[b].lang_tokens[i] >= vocab_) throw std::invalid_argument("vla: language token outside the vocabulary");
     }
     const int t_max = round_up(P + n_act_, 64);
-    if (B != B_ || P != P_) {
+    const int tuning_gen = vla_kernels_tuning_generation();  // the attention workspace is planned under the tuning overrides
+    if (B != B_ || P != P_ || tuning_gen != tuning_gen_) {
+        tuning_gen_ = tuning_gen;
         B_ = B;
         P_ = P;
         const size_t M = (size_t)B * P;

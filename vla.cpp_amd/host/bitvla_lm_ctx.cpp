@@ -112,6 +112,7 @@ bitvla_lm_hip_ctx* bitvla_lm_hip_init(int hidden, int n_q, int n_kv, int head_di
         size_t ws = 0;
         for (int seq = 1; seq <= max_seq; ++seq) {
             const size_t b = vla_attn_workspace_bytes(VLA_DT_BF16_P2, 1, seq, n_q, n_kv, head_dim, seq);
+            if (b == VLA_ATTN_WORKSPACE_UNSUPPORTED) throw std::invalid_argument("no attention kernel takes this head geometry");
             if (b > ws) ws = b;
         }
         c->attn_ws.alloc(ws);

@@ -119,6 +119,7 @@ class FlowExpert : public ModelArch {
   private:
     void allocate(int B, int P, int P_txt = 0);
     uint32_t alloc_gen_ = 0;
+    int tuning_gen_ = -1;
 
     Arch arch_;
     int dt_ = VLA_DT_F32;
@@ -532,7 +533,10 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
 }
 
 void FlowExpert::allocate(int B, int P, int P_txt) {
-    if (B == B_ && P == P_ && P_txt == P_txt_) return;
+    // the attention workspace is planned under the kernel library's tuning overrides: plan again when they were reloaded
+    const int tuning_gen = vla_kernels_tuning_generation();
+    if (B == B_ && P == P_ && P_txt == P_txt_ && tuning_gen == tuning_gen_) return;
+    tuning_gen_ = tuning_gen;
     B_ = B;
     P_ = P;
     P_txt_ = P_txt;

@@ -290,13 +290,16 @@ void import_gr00t(gguf_reader& g, Checkpoint& ck, bool bf16) {
     if (const char* e = std::getenv("VLA_GR00T_EMBODIMENT")) {
         char* end = nullptr;
         const long v = std::strtol(e, &end, 10);
-        if (end && *end == '\0' && end != e) {
+        if (end && *end == '\0') {  // a number; an empty value reads as 0, as in the reference (gr00tn1d5.cpp:150-153)
             id = v;
         } else {
+            // a tag: looked up in the mapping; an unknown tag keeps id 24 with a warning (gr00tn1d5.cpp:154-160)
             const std::string js = g.str(key("embodiment_tag_mapping").c_str()), k2 = std::string("\"") + e + "\":";
             const size_t p = js.find(k2);
-            if (p == std::string::npos) throw std::runtime_error(std::string("vla: embodiment tag '") + e + "' is not in embodiment_tag_mapping");
-            id = std::strtol(js.c_str() + p + k2.size(), nullptr, 10);
+            if (p != std::string::npos)
+                id = std::strtol(js.c_str() + p + k2.size(), nullptr, 10);
+            else
+                std::fprintf(stderr, "vla(gr00t): embodiment tag '%s' not in embodiment_tag_mapping; using id %lld\n", e, (long long)id);
         }
     }
     if (id < 0 || id >= n_emb) throw std::runtime_error("vla: embodiment id out of range");

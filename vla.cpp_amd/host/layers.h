@@ -83,6 +83,7 @@ struct AttnWorkspace {
     void reset() { need = 0; }
     void plan(int dtype, int batch, int S, int Hq, int Hkv, int D, int n_keys) {
         const size_t b = vla_attn_workspace_bytes(dtype, batch, S, Hq, Hkv, D, n_keys);
+        if (b == VLA_ATTN_WORKSPACE_UNSUPPORTED) throw std::invalid_argument("vla: no attention kernel takes this head geometry");
         if (b > need) need = b;
     }
     void commit() {

@@ -80,6 +80,14 @@ void ModelArch::prof_mark(const char* label) {
     prof_->add(prof_->phase + "." + label);
 }
 
+void ModelArch::profile_discard() {
+    delete prof_;
+    prof_ = nullptr;
+}
+
+// The summary of the marks recorded so far.  The profiler stays armed: the caller disarms it
+// (profile_discard) once the summary has been delivered, so a caller whose buffer was too
+// small can come back with a larger one.
 std::string ModelArch::profile_end() {
     if (!prof_) return "{}";
     VLA_HIP(hipDeviceSynchronize());
@@ -92,8 +100,6 @@ std::string ModelArch::profile_end() {
         a.first += (double)ms * 1e3;
         a.second += 1;
     }
-    delete prof_;
-    prof_ = nullptr;
     std::string out = "{";
     char buf[256];
     for (const auto& kv : acc) {

@@ -85,7 +85,8 @@ class ModelArch {
     // "launches": marks recorded}, ...}.  The time between two marks is the launch's duration
     // plus the gap to its predecessor on the stream.
     void profile_begin();
-    std::string profile_end();
+    std::string profile_end();   // summary of the marks so far; the profiler stays armed
+    void profile_discard();       // disarms and frees the marks
     // Synchronises and returns [batch, n_actions, max_action_dim].
     virtual std::vector<float> fetch() = 0;
     virtual int64_t n_actions() const = 0;

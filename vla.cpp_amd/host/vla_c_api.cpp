@@ -218,8 +218,10 @@ int64_t vla_profile_end(vla_model* h, char* json_out, int64_t cap) {
     if (!h || !h->m || !json_out || cap <= 0) return VLA_ERR_ARG;
     try {
         const std::string s = h->m->arch->profile_end();
-        if ((int64_t)s.size() + 1 > cap) return -(int64_t)(s.size() + 1);
+        // too small: the profile is kept, and the size comes back below every vla_status code
+        if ((int64_t)s.size() + 1 > cap) return -16 - (int64_t)(s.size() + 1);
         std::memcpy(json_out, s.c_str(), s.size() + 1);
+        h->m->arch->profile_discard();
         return (int64_t)s.size();
     } catch (const std::exception& e) {
         std::fprintf(stderr, "vla: profile failed: %s\n", e.what());
