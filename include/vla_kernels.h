@@ -278,7 +278,8 @@ VLA_KAPI int vla_attn_prefix_suffix_noalloc(const void* q, const void* k_cache, 
  * src/models/smolvla.cpp:1398): rows s < n_lead copy lead[b][s][:] (pi0 / DiT
  * state token); other rows are W_in . x_t[b][s - n_lead] + bias_step.
  *   x_t fp32 [batch][S - n_lead][A]; W_in fp32 [W][A]; bias_step fp32 [W];
- *   lead fp32 [batch][n_lead][W] or NULL; h in `out_dtype`. */
+ *   lead fp32 [batch][n_lead][W] or NULL; h in `out_dtype`.  A <= 136 (GR00T N1.7's 132
+ * action values); VLA_K_ERR_SHAPE beyond. */
 VLA_KAPI int vla_embed_suffix(const float* x_t, const float* W_in, const float* bias_step, const float* lead,
                               void* h, int out_dtype, int batch, int S, int n_lead, int A, int W,
                               vla_stream_t stream);

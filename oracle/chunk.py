@@ -116,6 +116,14 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
     pe = rnd(pe)
     if alt_vl:
         txt = rnd(txt)
+    if gr00t and "prefix.vlln_w" in w:
+        # vlln, the affine LayerNorm between the backbone and the head (gr00tn1d6.cpp:436,
+        # gr00tn1d7.cpp:556): the rows then stand for the backbone's last hidden states
+        veps = cfg.get("vlln_eps", 1e-5)
+        text_is_image = alt_vl and txt is pe
+        pe = rnd(orc.layer_norm(pe, w["prefix.vlln_w"], w["prefix.vlln_b"], veps))
+        if alt_vl:
+            txt = pe if text_is_image else rnd(orc.layer_norm(txt, w["prefix.vlln_w"], w["prefix.vlln_b"], veps))
 
     if cfg["suffix_mask"] == 1:
         mask_self = orc.mask_smolvla_full(P, S, pad[0], pad[1])
@@ -166,7 +174,9 @@ def flow_expert_chunk(cfg, w, obs, emulate_bf16=False, return_debug=False):
     if head_io:
         # ActionExpert::encode_state (action_expert.cpp:41-44), then the learned future tokens (gr00tn1d5.cpp:371)
         se = np.maximum(orc.linear(state[None, :], w["aex.se_l1W"], w["aex.se_l1b"]), 0)
-        lead = np.concatenate([orc.linear(se, w["aex.se_l2W"], w["aex.se_l2b"]), w["aex.future_tokens"]], 0)
+        lead = orc.linear(se, w["aex.se_l2W"], w["aex.se_l2b"])
+        if cfg["num_future"] > 0:  # none in N1.6 / N1.7: hh = [state; actions] (gr00tn1d6.cpp:457)
+            lead = np.concatenate([lead, w["aex.future_tokens"]], 0)
     elif n_lead:
         lead = orc.linear(state[None, :], w["act.W_sp"], w["act.b_sp"])
 

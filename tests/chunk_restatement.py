@@ -261,6 +261,9 @@ def gr00t(cfg, w, obs):
     txt = img
     if alt and obs.get("lang") is not None and len(obs["lang"]):
         txt = T(w["prefix.E_lang"])[np.asarray(obs["lang"], np.int64)]
+    if "prefix.vlln_w" in w:  # vlln on the backbone rows (gr00tn1d6.cpp:436)
+        vl = lambda x: F.layer_norm(x, (Wv,), T(w["prefix.vlln_w"]), T(w["prefix.vlln_b"]), cfg.get("vlln_eps", 1e-5))
+        img, txt = vl(img), vl(txt)
     scale = 1.0 / math.sqrt(D)
     kvd = H * D
     cross = [not (interleave and l % 2 == 1) for l in range(L)]
@@ -274,8 +277,9 @@ def gr00t(cfg, w, obs):
     state = T(obs["state"]) if obs.get("state") is not None else torch.zeros(cfg["max_state_dim"], dtype=F64)
     head_io = bool(cfg.get("head_io", 0))
     if head_io:  # encode_state, then the learned future tokens: 1 + num_future leading rows
-        lead = torch.cat([mm(w["aex.se_l2W"], F.relu(mm(w["aex.se_l1W"], state[None], w["aex.se_l1b"])), w["aex.se_l2b"]),
-                          T(w["aex.future_tokens"])], 0)
+        lead = mm(w["aex.se_l2W"], F.relu(mm(w["aex.se_l1W"], state[None], w["aex.se_l1b"])), w["aex.se_l2b"])
+        if cfg["num_future"] > 0:  # N1.6 / N1.7 have no future tokens (gr00tn1d6.cpp:457)
+            lead = torch.cat([lead, T(w["aex.future_tokens"])], 0)
     else:
         lead = mm(w["act.W_sp"], state[None], w["act.b_sp"])
     n_lead = lead.shape[0]

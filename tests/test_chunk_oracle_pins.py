@@ -54,6 +54,11 @@ def tiny(arch, **kw):
         c.update(n_q_heads=3, n_kv_heads=3, head_dim=8, hidden=20, expert_h=24, n_img=4, max_action_dim=6, max_state_dim=7,
                  real_action_dim=6, real_state_dim=7, num_future=2, n_suffix=1 + 2 + 3, dit_out_dim=10, dec_hidden=14,
                  state_hidden=9, max_pos=8)
+    elif arch == "gr00t_n1d6_head":
+        # N1.6 as its GGUF loads: alternating rows, the head's own MLPs, no future tokens, vlln
+        c = ckpt.gr00t_n1d6_head_config(n_layers=8, dtype="f32", num_steps=2, ffn_dim=12, variant=kw.pop("variant", "n1_6"))
+        c.update(n_q_heads=3, n_kv_heads=3, head_dim=8, hidden=20, expert_h=24, n_img=4, n_lang=3, max_action_dim=6, max_state_dim=7,
+                 real_action_dim=6, real_state_dim=7, n_suffix=1 + 3, dit_out_dim=10, dec_hidden=14, state_hidden=9, max_pos=8, vocab=11)
     elif arch == "gr00t_n1d5":
         c = ckpt.gr00t_config(n_layers=4, dtype="f32", num_steps=3, n_suffix=5)
         c.update(n_q_heads=3, n_kv_heads=3, head_dim=8, hidden=20, expert_h=24, n_img=4, max_action_dim=6,
@@ -94,7 +99,8 @@ def rel(a, b):
 CASES = [("smolvla", {}), ("smolvla", dict(suffix_mask=0)), ("smolvla", dict(ffn_dim=12, time_mlp=1)), ("pi0", {}),
          ("pi0", dict(ffn_dim=12, time_mlp=1)), ("pi05", {}), ("pi05", dict(ffn_dim=12)), ("gr00t_n1d5", {}),
          ("gr00t_n1d5", dict(ffn_dim=12)), ("gr00t_n1d6", {}), ("gr00t_n1d6", dict(every=1)),
-         ("gr00t_n1d6", dict(interleave=0, ffn_dim=12)), ("gr00t_head_io", {})]
+         ("gr00t_n1d6", dict(interleave=0, ffn_dim=12)), ("gr00t_head_io", {}), ("gr00t_n1d6_head", {}),
+         ("gr00t_n1d6_head", dict(variant="n1_7"))]
 
 
 @pytest.mark.parametrize("arch,kw", CASES, ids=["%s-%s" % (a, "-".join("%s%s" % i for i in k.items()) or "base") for a, k in CASES])
@@ -152,6 +158,33 @@ def test_structural_mistakes_are_far_outside_the_tolerance(arch):
             assert rel(ref.chunk(cfg, w, o), base) > 100 * TOL
     finally:
         R.rope_neox = keep
+
+
+def test_vlln_and_the_missing_future_rows_are_seen_by_the_comparison():
+    # N1.6 from GGUF: vlln on the backbone rows (gr00tn1d6.cpp:436) and hh = [state; actions]
+    # (gr00tn1d6.cpp:457).  Dropping vlln, or normalising without its weight, moves the chunk
+    # far outside the tolerance; identity vlln on rows that are already normalised changes nothing.
+    cfg = tiny("gr00t_n1d6_head")
+    w = big_weights(cfg, seed=930)
+    o = obs_for(cfg, np.random.default_rng(931))
+    base = ref.chunk(cfg, w, o)
+    assert base.shape == (3, cfg["max_action_dim"])
+    no_vlln = {k: v for k, v in w.items() if not k.startswith("prefix.vlln")}
+    assert rel(ref.chunk(cfg, no_vlln, o), base) > 100 * TOL
+    plain = dict(w)
+    plain["prefix.vlln_w"], plain["prefix.vlln_b"] = np.ones_like(w["prefix.vlln_w"]), np.zeros_like(w["prefix.vlln_b"])
+    assert rel(ref.chunk(cfg, plain, o), base) > 100 * TOL
+    # closed form: rows with zero mean and unit variance pass through an identity vlln unchanged (eps -> 0)
+    c0 = dict(cfg, vlln_eps=0.0)
+    o2 = dict(o)
+    x = o["img_emb"].astype(np.float64)
+    x = (x - x.mean(1, keepdims=True)) / x.std(1, keepdims=True)
+    o2["img_emb"] = x.astype(np.float32)
+    E = w["prefix.E_lang"].astype(np.float64)
+    plain["prefix.E_lang"] = ((E - E.mean(1, keepdims=True)) / E.std(1, keepdims=True)).astype(np.float32)
+    no2 = {k: v for k, v in plain.items() if not k.startswith("prefix.vlln")}
+    a, b = orc_chunk.flow_expert_chunk(c0, plain, o2), orc_chunk.flow_expert_chunk(c0, no2, o2)
+    assert rel(a, b.astype(np.float64)) < TOL
 
 
 @pytest.mark.parametrize("arch", ["smolvla", "pi0", "gr00t_n1d5"])

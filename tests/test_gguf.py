@@ -224,6 +224,44 @@ def test_gr00t_head_gguf_equals_the_vlaw_checkpoint(tmp_path, monkeypatch):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("variant", ["n1_6", "n1_7"])
+def test_gr00t_n1d6_and_n1d7_gguf_equal_the_vlaw_checkpoint(tmp_path, monkeypatch, variant):
+    """GR00T N1.6 / N1.7 under the reference's keys and names (src/models/gr00tn1d6.cpp:96-189,
+    294-298; src/models/gr00tn1d7.cpp:119-215): no future tokens, alternating text / image rows,
+    the default embodiment found by tag ("gr1" / "libero_sim") in embodiment_id_mapping, N1.6's
+    vlln on the backbone rows; text rows resident or fetched from the file."""
+    from test_gpu_chunk import make_obs
+    cfg = ckpt.gr00t_n1d6_head_config(n_layers=8, ffn_dim=512, variant=variant)
+    cfg["embodiment"] = 7  # what the default tag maps to in the file; the built-in ids (20 / 2) hold noise
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 26)
+    r = np.random.default_rng(334)
+    obs = [make_obs(cfg, r, n_views=2, n_lang=9) for _ in range(2)]
+    pv, pg = os.path.join(str(tmp_path), "g.vlaw"), os.path.join(str(tmp_path), "g.gguf")
+    ckpt.write_synthetic(pv, cfg, w)
+    gguf.write_synthetic_gguf(pg, cfg, w)
+    AH, A = (50, 128) if variant == "n1_6" else (40, 132)
+    want = _chunk(pv, obs, (2, AH, A))
+    assert np.abs(want).max() > 0.1
+    assert np.array_equal(_chunk(pg, obs, (2, AH, A)), want)
+    monkeypatch.setenv("VLA_EMBED_ON_DEMAND", "1")
+    assert np.array_equal(_chunk(pg, obs, (2, AH, A)), want)
+    monkeypatch.delenv("VLA_EMBED_ON_DEMAND")
+    monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "other_robot")  # id 3: another row of the stacks
+    assert not np.array_equal(_chunk(pg, obs, (2, AH, A)), want)
+    monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "7")
+    assert np.array_equal(_chunk(pg, obs, (2, AH, A)), want)
+    monkeypatch.setenv("VLA_GR00T_EMBODIMENT", "no_such_tag")  # warns, keeps the tag's id
+    assert np.array_equal(_chunk(pg, obs, (2, AH, A)), want)
+    monkeypatch.delenv("VLA_GR00T_EMBODIMENT")
+    if variant == "n1_7":  # gr00tn1d7.cpp:150-156
+        monkeypatch.setenv("VLA_NUM_STEPS", "2")
+        cfg2 = dict(cfg, num_steps=2)
+        p2 = os.path.join(str(tmp_path), "g2.vlaw")
+        ckpt.write_synthetic(p2, cfg2, w)
+        assert np.array_equal(_chunk(pg, obs, (2, AH, A)), _chunk(p2, obs, (2, AH, A)))
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("arch", ["pi0", "bitvla"])
 def test_token_embedding_rows_fetched_from_the_file_give_the_resident_result(tmp_path, monkeypatch, arch):
     """Large vocabularies stay on disk and each request reads its rows (fetch_rows_f32,
@@ -308,6 +346,12 @@ def _fixture_names():
 
 
 def _tiny(arch):
+    if arch in ("gr00t_n1_6", "gr00t_n1_7"):
+        cfg = ckpt.gr00t_n1d6_head_config(n_layers=4, ffn_dim=256, variant=arch[len("gr00t_"):])
+        cfg.update(n_q_heads=4, n_kv_heads=4, head_dim=16, hidden=96, expert_h=64, n_img=8, n_lang=6, vocab=40, max_action_dim=8,
+                   real_action_dim=8, max_state_dim=8, real_state_dim=8, n_suffix=1 + 4, dit_out_dim=32, dec_hidden=48,
+                   state_hidden=40, max_pos=16)
+        return cfg
     if arch == "gr00t":
         cfg = ckpt.gr00t_head_io_config(n_layers=3, ffn_dim=256)
         cfg.update(n_q_heads=4, n_kv_heads=4, head_dim=16, hidden=96, expert_h=64, n_img=8, max_action_dim=8, real_action_dim=8,
@@ -322,11 +366,11 @@ def _tiny(arch):
     return cfg
 
 
-@pytest.mark.parametrize("arch", ["smolvla", "pi0", "pi05", "gr00t"])
+@pytest.mark.parametrize("arch", ["smolvla", "pi0", "pi05", "gr00t", "gr00t_n1_6", "gr00t_n1_7"])
 def test_importer_reads_the_tensor_names_the_reference_converters_write(tmp_path, arch):
     """The per-block GGUF names the importer asks for are held against the name lists the
     reference's own converter tests keep as data (tests/golden/gguf_tensor_names.json, from
-    tests/py/test_converters.py:102-111, 178-184), not against this package's writer: the import is
+    tests/py/test_converters.py:102-111, 178-184, 203-220), not against this package's writer: the import is
     traced on the host (vla_gguf_import_trace) and every block-level name it read must be one the
     reference writes; the blocks on the path must be read completely."""
     import re
@@ -338,13 +382,20 @@ def test_importer_reads_the_tensor_names_the_reference_converters_write(tmp_path
     read = gguf.import_trace(pkg.lib(), p)
     assert len(read) == len(set(read)), "a tensor was read twice"
     L = cfg["n_layers"]
-    if arch == "gr00t":
+    if arch.startswith("gr00t"):
         for i in range(L):
             want = {n.format(i=i) for n in fx["dit_block"]["names"]}
             got = {n for n in read if re.match(r"aex\.dit\.%d\." % i, n)}
             assert got == want, (i, sorted(got ^ want))
-        # nothing but the DiT head is read: no vision tower, backbone or VL self-attention tensor
-        assert not [n for n in read if n.startswith(("vit.", "vlm.", "mm.", "aex.vlsa", "aex.vlln", "token_embd"))]
+        # the head's projectors, time embedding and output projection, whole
+        assert set(fx["gr00t_action_head"]["names"]) <= set(read)
+        # beyond those: the learned positions, N1.5's future tokens, and for N1.6 / N1.7 the text rows'
+        # embedding matrix; vlln only where it is the last step before the head (N1.6,
+        # src/models/gr00tn1d6.cpp:436; in N1.5 / N1.7 a VL self-attention stack follows it)
+        rest = set(read) - set(fx["gr00t_action_head"]["names"]) - {n for n in read if re.match(r"aex\.dit\.\d+\.", n)}
+        assert rest == {"gr00t": {"aex.pos_embd", "aex.future_tokens"},
+                        "gr00t_n1_6": {"aex.pos_embd", "token_embd.weight", "aex.vlln.weight", "aex.vlln.bias"},
+                        "gr00t_n1_7": {"aex.pos_embd", "token_embd.weight"}}[arch], sorted(rest)
         return
     allowed = {n.format(p=pfx, i=i) for pfx in fx["decoder_block"]["prefixes"] for i in range(L) for n in fx["decoder_block"]["names"]}
     block_level = [n for n in read if re.match(r"(vlm|aex)\.blk\.\d+\.", n)]

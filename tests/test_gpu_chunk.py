@@ -299,6 +299,37 @@ def test_gr00t_n1d6_alternating_text_and_image_cross_layers(tmp_path, n_layers, 
     m.close()
 
 
+@pytest.mark.parametrize("variant,dtype,n_layers,batch", [("n1_6", "bf16", 8, 2), ("n1_6", "f32", 4, 1), ("n1_7", "bf16", 8, 1),
+                                                         ("n1_6", "bf16", 32, 1)])
+def test_gr00t_n1d6_head_as_its_gguf_loads_it(tmp_path, variant, dtype, n_layers, batch):
+    """N1.6 / N1.7 with the head's own MLPs (src/models/gr00tn1d6.cpp:436-479, src/models/gr00tn1d7.cpp:
+    556-600): vlln on the backbone rows (N1.6), hh = [state; actions] without future tokens, cross
+    layers alternating text / image rows, velocity = decode(proj_out(h)) on the action rows."""
+    cfg = ckpt.gr00t_n1d6_head_config(n_layers=n_layers, dtype=dtype, ffn_dim=1024 if n_layers < 32 else 6144, variant=variant)
+    if dtype == "f32":
+        cfg.update(head_dim=64, n_q_heads=8, n_kv_heads=8, expert_h=512, dit_out_dim=256, dec_hidden=256, state_hidden=256)  # fp32 heads of 48 are not built
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 41)
+    r = np.random.default_rng(340 + n_layers)
+    obs = [make_obs(cfg, r, n_views=2, n_lang=19) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "n1d6_head")
+    AH, A = (50, 128) if variant == "n1_6" else (40, 132)
+    got = m.predict_batch(obs).reshape(batch, AH, A)
+    assert m.config().n_suffix == 1 + AH
+    for b in range(batch):
+        if dtype == "f32":
+            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b])
+            assert rel_err(got[b], want) < 1e-5, rel_err(got[b], want)
+        else:
+            want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+            assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    if variant == "n1_6":
+        # vlln is applied: with identity weights the chunk is another one
+        w2 = dict(w)
+        w2["prefix.vlln_w"], w2["prefix.vlln_b"] = np.ones_like(w["prefix.vlln_w"]), np.zeros_like(w["prefix.vlln_b"])
+        assert not np.allclose(orc_chunk.flow_expert_chunk(cfg, w2, obs[0], emulate_bf16=dtype == "bf16"), got[0], atol=1e-3)
+    m.close()
+
+
 @pytest.mark.parametrize("from_fp32,ffn_dim", [(False, 0), (True, 0), (False, 768), (True, 6912)])
 def test_config4_bitvla_ternary_append(tmp_path, from_fp32, ffn_dim):
     # ffn_dim > 0: the layers also run their squared-ReLU GLU half (768: the down projection of

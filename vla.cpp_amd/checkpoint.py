@@ -117,6 +117,20 @@ def gr00t_n1d6_config(n_layers=32, dtype="bf16", num_steps=4, n_suffix=17, atten
     return c
 
 
+def gr00t_n1d6_head_config(n_layers=32, dtype="bf16", num_steps=4, ffn_dim=6144, variant="n1_6"):
+    """GR00T N1.6 / N1.7 as the reference loads them from GGUF (src/models/gr00tn1d6.cpp:75-126,
+    294-298, 436-467; src/models/gr00tn1d7.cpp:60-100, 556-590): the alternating head with its own
+    input / output MLPs, no future tokens (the sequence is 1 state + action_horizon rows), and
+    vlln, an affine LayerNorm on the backbone rows.  N1.6: horizon 50, 128 action / state values;
+    N1.7: horizon 40, 132, and vlln inside the backbone (a VL self-attention stack follows it), so not on this path."""
+    AH, A = (50, 128) if variant == "n1_6" else (40, 132)
+    c = gr00t_n1d6_config(n_layers, dtype, num_steps, n_suffix=1 + AH)
+    c.update(head_io=1, num_future=0, dit_out_dim=1024, dec_hidden=1024, state_hidden=1024, ffn_dim=ffn_dim,
+             num_buckets=1000, max_pos=1024, max_action_dim=A, real_action_dim=A, max_state_dim=A, real_state_dim=A,
+             vlln=1 if variant == "n1_6" else 0, vlln_eps=1e-5, variant=variant)
+    return c
+
+
 def bitvla_config(n_layers=30):
     """BitVLA / BitNet b1.58 2B shape (src/models/bitvla.cpp:121-122): width 2560,
     20 query / 5 KV heads of 128, RoPE base 5e5; prefix 256 image + 256 text tokens,
@@ -179,6 +193,9 @@ def synth_weights(cfg, seed=0x5EED):
     if cfg.get("vocab", 0) > 0:
         # N1.6: the rows stand for backbone features at the text positions, O(1) like the image rows
         w["prefix.E_lang"] = (r.standard_normal((cfg["vocab"], Wv)) / (1.0 if arch == "gr00t_n1d6" else np.sqrt(Wv))).astype(np.float32)
+    if cfg.get("vlln", 0):
+        w["prefix.vlln_w"] = (1.0 + 0.1 * r.standard_normal(Wv)).astype(np.float32)
+        w["prefix.vlln_b"] = vec(Wv, 0.1)
     if arch == "smolvla":
         w["prefix.Wstate"] = (0.1 * r.standard_normal((Wv, cfg["max_state_dim"]))).astype(np.float32)
         w["prefix.bstate"] = vec(Wv, 0.1)
@@ -195,7 +212,8 @@ def synth_weights(cfg, seed=0x5EED):
         w["aex.ae_W2"], w["aex.ae_b2"] = f32m(W, 2 * W, 1.0 / np.sqrt(2 * W)), vec(W, 0.1)
         w["aex.ae_W3"], w["aex.ae_b3"] = f32m(W, W, 1.0 / np.sqrt(W)), vec(W, 0.1)
         w["aex.pos_embd"] = f32m(cfg.get("max_pos", 64), W, 0.02)
-        w["aex.future_tokens"] = f32m(NF, W, 0.5)
+        if NF > 0:
+            w["aex.future_tokens"] = f32m(NF, W, 0.5)
         w["aex.po1W"], w["aex.po1b"] = f32m(2 * W, W, 0.02), vec(2 * W)
         w["aex.po2W"], w["aex.po2b"] = mat(O, W), vec(O)
         w["aex.ad_l1W"], w["aex.ad_l1b"] = mat(Hd, O), vec(Hd)

@@ -314,6 +314,7 @@ bool launch_row_norm(const void* x, const void* w, const float* sc, const float*
 // stores are coalesced along the width.  One load round trip per workgroup.
 constexpr int EMB_ROWS = 32;
 constexpr int EMB_MAX_A = 64;
+constexpr int EMB_WIDE_A = 136;  // GR00T N1.6 / N1.7: 128 / 132 action values per row
 constexpr int EMB_COLS = 64;
 template <typename T, int AMAX = EMB_MAX_A>  // AMAX: the padded action width the staging loops are unrolled for
 __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restrict__ x_t, const float* __restrict__ W_in,
@@ -323,8 +324,10 @@ __global__ void __launch_bounds__(256) embed_suffix_kernel(const float* __restri
     // rows padded to a multiple of four floats: every a-loop step below is one 16-byte LDS read
     // of the thread's weight row (row stride 68 floats: 16 lanes cover all 64 banks once) and one
     // 16-byte broadcast read per output row, 9 LDS instructions per 32 multiply-adds
-    __shared__ __attribute__((aligned(16))) float xs[EMB_ROWS][EMB_MAX_A];
-    __shared__ __attribute__((aligned(16))) float ws[EMB_COLS][EMB_MAX_A + 4];
+    // (stride 140 for the wide form: 140 mod 64 = 12 spreads 16 lanes the same way)
+    constexpr int LD = AMAX > EMB_MAX_A ? AMAX : EMB_MAX_A;
+    __shared__ __attribute__((aligned(16))) float xs[EMB_ROWS][LD];
+    __shared__ __attribute__((aligned(16))) float ws[EMB_COLS][LD + 4];
     const int row0 = blockIdx.x * EMB_ROWS, c0 = blockIdx.y * EMB_COLS;
     const int ncol = min(EMB_COLS, W - c0);
     const int A4 = (A + 3) & ~3;
@@ -1032,17 +1035,20 @@ int vla_embed_suffix_act(const float* x_t, const float* W_in, const float* bias_
         return VLA_K_ERR_ARG;
     if (act < VLA_ACT_NONE || act > VLA_ACT_RELU) return VLA_K_ERR_ARG;
     if (n_lead > 0 && !lead) return VLA_K_ERR_ARG;
-    if (A > EMB_MAX_A) return VLA_K_ERR_SHAPE;
+    if (A > EMB_WIDE_A) return VLA_K_ERR_SHAPE;
     if (batch == 0) return VLA_K_OK;
     hipStream_t st = (hipStream_t)stream;
     const int n_rows = batch * S;
     const dim3 blocks((n_rows + EMB_ROWS - 1) / EMB_ROWS, (W + EMB_COLS - 1) / EMB_COLS);
     const bool narrow = A <= 32;  // half the staging passes
+    const bool wide = A > EMB_MAX_A;
     if (out_dtype == VLA_DT_F32) {
         if (narrow) embed_suffix_kernel<float, 32><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W, act);
+        else if (wide) embed_suffix_kernel<float, EMB_WIDE_A><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W, act);
         else embed_suffix_kernel<float><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (float*)h, n_rows, S, n_lead, A, W, act);
     } else if (out_dtype == VLA_DT_BF16) {
         if (narrow) embed_suffix_kernel<bf16_t, 32><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W, act);
+        else if (wide) embed_suffix_kernel<bf16_t, EMB_WIDE_A><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W, act);
         else embed_suffix_kernel<bf16_t><<<blocks, 256, 0, st>>>(x_t, W_in, bias_step, lead, (bf16_t*)h, n_rows, S, n_lead, A, W, act);
     } else {
         return VLA_K_ERR_ARG;

@@ -287,25 +287,45 @@ def write_synthetic_gguf(path, cfg, w, ladder_pack=None):
                 else:
                     # floats whose absmean quantisation gives back (tern, scale): see checkpoint._dequant_sources
                     t[b + name + ".weight"] = f32(tern.astype(np.float32) * np.float32(scale))
-    elif cfg["arch"] == "gr00t_n1d5" and cfg.get("head_io", 0):
-        # GR00T N1.5 action head (src/models/gr00tn1d5.cpp:92-147; src/modules/dit_head.cpp:29-85;
+    elif cfg["arch"] in ("gr00t_n1d5", "gr00t_n1d6") and cfg.get("head_io", 0):
+        # GR00T action head (src/models/gr00tn1d5.cpp:92-147; src/modules/dit_head.cpp:29-85;
         # src/modules/action_expert.cpp:20-39): the head's MLPs are cat_linear stacks, one
         # [in][out] matrix per embodiment (ggml ne = [out, in, n]); the synthetic weights go into
-        # row `embodiment`, the other rows hold noise that must not be read.
+        # row `embodiment`, the other rows hold noise that must not be read.  N1.6 / N1.7
+        # (cfg["variant"] "n1_6" / "n1_7"; src/models/gr00tn1d6.cpp:96-189, 294-298,
+        # src/models/gr00tn1d7.cpp:119-215): their key prefix, no future tokens,
+        # attend_text_every_n_blocks, embodiment_id_mapping written with a space after the colon
+        # as json.dumps does, token_embd.weight for the text rows and aex.vlln.
         W, Wv, I, A = cfg["expert_h"], cfg["hidden"], cfg["ffn_dim"], cfg["max_action_dim"]
-        n_emb, emb = cfg.get("max_embodiments", 32), cfg.get("embodiment", 24)
+        alt = cfg["arch"] == "gr00t_n1d6"
+        variant = cfg.get("variant", "n1_6") if alt else "n1_5"
+        pfx = "gr00t_%s." % variant
+        n_emb, emb = cfg.get("max_embodiments", 32), cfg.get("embodiment", {"n1_5": 24, "n1_6": 20, "n1_7": 2}[variant])
         rr = np.random.default_rng(99)
-        kv["gr00t_n1_5.architecture"] = (STRING, "gr00t_n1_5")
+        kv[pfx + "architecture"] = (STRING, "gr00t_" + variant)
         for k, v in (("backbone_embedding_dim", Wv), ("input_embedding_dim", W), ("dit_hidden", W), ("dit_heads", Hq),
                      ("dit_head_dim", D), ("dit_layers", L), ("dit_interleave", cfg.get("dit_interleave", 1)),
-                     ("num_target_vision_tokens", cfg["num_future"]), ("action_horizon", cfg["n_suffix"] - 1 - cfg["num_future"]),
+                     ("action_horizon", cfg["n_suffix"] - 1 - cfg["num_future"]),
                      ("action_dim", A), ("max_state_dim", cfg["max_state_dim"]), ("num_inference_timesteps", cfg["num_steps"]),
                      ("num_timestep_buckets", cfg.get("num_buckets", 1000)), ("max_num_embodiments", n_emb),
                      ("n_img_tokens", cfg["n_img"])):
-            kv["gr00t_n1_5." + k] = (U32, int(v))
-        kv["gr00t_n1_5.ln_eps"] = (F32, float(cfg["rms_eps"]))
-        kv["gr00t_n1_5.norm_out_eps"] = (F32, float(cfg["norm_out_eps"]))
-        kv["gr00t_n1_5.embodiment_tag_mapping"] = (STRING, '{"new_embodiment":31,"gr1":%d}' % emb)
+            kv[pfx + k] = (U32, int(v))
+        kv[pfx + "ln_eps"] = (F32, float(cfg["rms_eps"]))
+        kv[pfx + "norm_out_eps"] = (F32, float(cfg["norm_out_eps"]))
+        if alt:
+            kv[pfx + "attend_text_every_n_blocks"] = (U32, int(cfg["attend_text_every_n"]))
+            kv[pfx + "max_seq_len"] = (U32, int(cfg["n_lang"]))
+            kv[pfx + "vlln_eps"] = (F32, float(cfg.get("vlln_eps", 1e-5)))
+            tag = cfg.get("default_tag", "gr1" if variant == "n1_6" else "libero_sim")
+            kv[pfx + "embodiment_id_mapping"] = (STRING, '{"new_embodiment": 31, "%s": %d, "other_robot": 3}' % (tag, emb))
+            if cfg.get("vocab", 0) > 0:
+                t["token_embd.weight"] = f32(w["prefix.E_lang"])
+            # N1.7's vlln sits in front of the VL self-attention stack, inside the backbone: present in the file, not on the path
+            t["aex.vlln.weight"] = f32(w["prefix.vlln_w"] if "prefix.vlln_w" in w else np.ones(Wv))
+            t["aex.vlln.bias"] = f32(w["prefix.vlln_b"] if "prefix.vlln_b" in w else np.zeros(Wv))
+        else:
+            kv[pfx + "num_target_vision_tokens"] = (U32, int(cfg["num_future"]))
+            kv[pfx + "embodiment_tag_mapping"] = (STRING, '{"new_embodiment":31,"gr1":%d}' % emb)
 
         def cat(wm, b):  # [out][in] weight, [out] bias -> per-embodiment stacks
             wm, b = np.asarray(wm, np.float32), np.asarray(b, np.float32)
@@ -323,7 +343,9 @@ def write_synthetic_gguf(path, cfg, w, ladder_pack=None):
                                ("act_enc.W2", "ae_W2", "ae_b2"), ("act_enc.W3", "ae_W3", "ae_b3"), ("act_dec.l1", "ad_l1W", "ad_l1b"),
                                ("act_dec.l2", "ad_l2W", "ad_l2b")):
             t["aex.%s.W" % g_name], t["aex.%s.b" % g_name] = cat(w["aex." + wn], w["aex." + bn])
-        t["aex.pos_embd"], t["aex.future_tokens"] = f32(w["aex.pos_embd"]), f32(w["aex.future_tokens"])
+        t["aex.pos_embd"] = f32(w["aex.pos_embd"])
+        if cfg["num_future"] > 0:
+            t["aex.future_tokens"] = f32(w["aex.future_tokens"])
         interleave = bool(cfg.get("dit_interleave", 1))
         for l in range(L):
             a, e, p = "aex.dit.%d." % l, "ex.%d." % l, "vlm.%d." % l

@@ -145,6 +145,8 @@ class FlowExpert : public ModelArch {
     std::shared_ptr<RowSource> lang_rows_;  // token embeddings left on disk (large vocabularies)
     bool alt_vl_ = false;   // GR00T N1.6 / N1.7: cross layers alternate text / image rows
     int text_every_ = 2, P_txt_ = 0;
+    DevBuf vlln_sc_, vlln_sh_;  // vlln as (weight - 1, bias) fp32 [Wv]: the modulated-norm launch computes xn (1 + sc) + sh
+    float vlln_eps_ = 1e-5f;
     bool fuse_final_norm_ = true;  // the final norm runs inside the Euler launch
     bool adarms_ = false;  // pi0.5: ada_ holds [steps][2L+1][scale, shift, gate][W]
     DevBuf bias_step_;   // [steps][W] fp32: b_in (+ time embedding of the step)
@@ -240,6 +242,14 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
             E_lang_ = host_f32(ck, "prefix.E_lang", {vocab_, Wv_});
         }
     }
+    if (ck.has("prefix.vlln_w")) {
+        if (arch_ != Arch::GR00T) throw std::runtime_error("vla: prefix.vlln_w belongs to the GR00T heads");
+        std::vector<float> sc = host_f32(ck, "prefix.vlln_w", {Wv_}), sh = host_f32(ck, "prefix.vlln_b", {Wv_});
+        for (float& v : sc) v -= 1.0f;
+        vlln_sc_.upload(sc.data(), sc.size() * sizeof(float));
+        vlln_sh_.upload(sh.data(), sh.size() * sizeof(float));
+        vlln_eps_ = (float)ck.f64("vlln_eps", 1e-5);
+    }
     if (arch_ == Arch::SMOLVLA) {
         Wstate_ = host_f32(ck, "prefix.Wstate", {Wv_, max_state_});
         bstate_ = host_f32(ck, "prefix.bstate", {Wv_});
@@ -251,7 +261,7 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         se_l1b_ = host_f32(ck, "aex.se_l1b", {Hs_});
         se_l2W_ = host_f32(ck, "aex.se_l2W", {W_, Hs_});
         se_l2b_ = host_f32(ck, "aex.se_l2b", {W_});
-        future_ = host_f32(ck, "aex.future_tokens", {n_future_, W_});
+        if (n_future_ > 0) future_ = host_f32(ck, "aex.future_tokens", {n_future_, W_});  // N1.6 / N1.7 have none
     } else if (n_lead_ > 0) {
         W_sp_ = host_f32(ck, "act.W_sp", {W_, max_state_});
         b_sp_ = host_f32(ck, "act.b_sp", {W_});
@@ -706,6 +716,10 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
         rope_self_.build(rs, ps);
         rope_cross_.build(rs, pc);
     }
+
+    // ---- vlln: the affine LayerNorm between the backbone and the DiT head
+    // (src/models/gr00tn1d6.cpp:436), in place on every prefix row
+    if (vlln_sc_) VLA_K(vla_adaln(prefix_.get(), vlln_sc_.as<float>(), vlln_sh_.as<float>(), prefix_.get(), dt_, B * P, Wv_, vlln_eps_, C.stream));
 
     // ---- prefix K/V of every layer, once per observation
     Tensor xp = tensor_2d(prefix_.get(), dt_, Wv_, (int64_t)B * P);

@@ -275,31 +275,77 @@ void import_flow(const std::string& path, gguf_reader& g, Checkpoint& ck, bool b
 // without dit_interleave) take K / V from the backbone features ([inner, backbone_embedding_dim]),
 // self layers fuse [q; k; v].  The backbone (vision tower, Qwen3 layers, VL self-attention) is
 // not read: precomputed_img_emb stands for its output rows.
-void import_gr00t(gguf_reader& g, Checkpoint& ck, bool bf16) {
-    auto key = [](const char* k) { return std::string("gr00t_n1_5.") + k; };
+//
+// N1.6 and N1.7 (variant 6 / 7) share the head and its names under the key prefixes
+// gr00t_n1_6. / gr00t_n1_7. (src/models/gr00tn1d6.cpp:96-189, 294-298; src/models/gr00tn1d7.cpp:
+// 119-215): no future tokens (the sequence is the state row and action_horizon rows,
+// gr00tn1d6.cpp:457), cross layers alternating between the text and the image rows every
+// attend_text_every_n_blocks, horizon / action / state defaults 50 / 128 / 128 (N1.6) and
+// 40 / 132 / 132 (N1.7), 64 image rows per view, and the embodiment row from
+// embodiment_id_mapping: "gr1" else 20 (N1.6), "libero_sim" else 2 (N1.7), VLA_GR00T_EMBODIMENT
+// over both; N1.7 also takes VLA_NUM_STEPS (gr00tn1d7.cpp:150-156).  N1.6 feeds the head
+// layer_norm(backbone rows) with aex.vlln.{weight, bias} (gr00tn1d6.cpp:436): those are read and
+// applied, the input rows standing for the language model's last hidden states.  In N1.5 and
+// N1.7 a VL self-attention stack follows vlln; it belongs to the backbone, so neither is read and
+// the input rows stand for its output.  The text rows come from token_embd.weight when the
+// file holds it at the backbone width (rows left on disk when large); without it there are no
+// text rows and the text layers attend to the image rows (gr00tn1d6.cpp:438).
+void import_gr00t(const std::string& path, gguf_reader& g, Checkpoint& ck, bool bf16, int variant) {
+    const std::string prefix = variant == 5 ? "gr00t_n1_5." : variant == 6 ? "gr00t_n1_6." : "gr00t_n1_7.";
+    auto key = [&](const char* k) { return prefix + k; };
     auto u = [&](const char* k) { return (int64_t)need_u32(g, key(k).c_str()); };
     auto u_or = [&](const char* k, int64_t d) { return g.has(key(k).c_str()) ? (int64_t)g.u32(key(k).c_str()) : d; };
     auto f_or = [&](const char* k, double d) { return g.has(key(k).c_str()) ? (double)g.f32(key(k).c_str()) : d; };
+    const bool alt = variant != 5;
     const int64_t Wv = u_or("backbone_embedding_dim", 2048), E = u_or("input_embedding_dim", 1536), W = u("dit_hidden"),
                   H = u("dit_heads"), D = u("dit_head_dim"), L = u("dit_layers"), interleave = u_or("dit_interleave", 1),
-                  NF = u_or("num_target_vision_tokens", 32), AH = u_or("action_horizon", 16), A = u_or("action_dim", 32),
-                  sd = u_or("max_state_dim", 64), steps = u_or("num_inference_timesteps", 4),
-                  buckets = u_or("num_timestep_buckets", 1000), n_emb = u_or("max_num_embodiments", 32);
+                  NF = alt ? 0 : u_or("num_target_vision_tokens", 32),
+                  AH = u_or("action_horizon", variant == 5 ? 16 : variant == 6 ? 50 : 40),
+                  A = u_or("action_dim", variant == 5 ? 32 : variant == 6 ? 128 : 132),
+                  sd = u_or("max_state_dim", variant == 5 ? 64 : variant == 6 ? 128 : 132),
+                  buckets = u_or("num_timestep_buckets", 1000), n_emb = u_or("max_num_embodiments", 32),
+                  text_every = u_or("attend_text_every_n_blocks", 2);
+    int64_t steps = u_or("num_inference_timesteps", 4);
+    if (variant == 7)
+        if (const char* ns = std::getenv("VLA_NUM_STEPS")) {
+            char* end = nullptr;
+            const long v = std::strtol(ns, &end, 10);
+            if (end && *end == '\0' && v >= 1) steps = v;
+        }
     if (H < 1 || D < 1 || H * D != W || E != W || L < 1) throw std::runtime_error("vla: gr00t gguf geometry is not usable (heads x head_dim, embedding and DiT widths must agree)");
-    int64_t id = 24;
+    if (alt && text_every < 1) throw std::runtime_error("vla: attend_text_every_n_blocks must be >= 1");
+    int64_t id = variant == 5 ? 24 : variant == 6 ? 20 : 2;
+    const char* map_key = variant == 5 ? "embodiment_tag_mapping" : "embodiment_id_mapping";
+    // the id that follows "tag" and a colon in the mapping's JSON text, or -1
+    auto lookup = [&](const std::string& tag) -> long {
+        const std::string js = g.str(key(map_key).c_str());
+        if (variant == 5) {  // gr00tn1d5.cpp:155-158 searches for "tag": as one string
+            const std::string k2 = "\"" + tag + "\":";
+            const size_t p = js.find(k2);
+            return p == std::string::npos ? -1 : std::strtol(js.c_str() + p + k2.size(), nullptr, 10);
+        }
+        const std::string k2 = "\"" + tag + "\"";  // gr00tn1d6.cpp:150-160: the key, then the next colon
+        size_t p = js.find(k2);
+        if (p == std::string::npos) return -1;
+        p = js.find(':', p + k2.size());
+        return p == std::string::npos ? -1 : std::strtol(js.c_str() + p + 1, nullptr, 10);
+    };
+    if (alt) {
+        const long dflt = lookup(variant == 6 ? "gr1" : "libero_sim");
+        if (dflt >= 0) id = dflt;
+    }
     if (const char* e = std::getenv("VLA_GR00T_EMBODIMENT")) {
         char* end = nullptr;
         const long v = std::strtol(e, &end, 10);
         if (end && *end == '\0') {  // a number; an empty value reads as 0, as in the reference (gr00tn1d5.cpp:150-153)
             id = v;
         } else {
-            // a tag: looked up in the mapping; an unknown tag keeps id 24 with a warning (gr00tn1d5.cpp:154-160)
-            const std::string js = g.str(key("embodiment_tag_mapping").c_str()), k2 = std::string("\"") + e + "\":";
-            const size_t p = js.find(k2);
-            if (p != std::string::npos)
-                id = std::strtol(js.c_str() + p + k2.size(), nullptr, 10);
+            // a tag: looked up in the mapping; an unknown tag keeps the id with a warning (gr00tn1d5.cpp:154-160)
+            const long t = lookup(e);
+            if (t >= 0)
+                id = t;
             else
-                std::fprintf(stderr, "vla(gr00t): embodiment tag '%s' not in embodiment_tag_mapping; using id %lld\n", e, (long long)id);
+                std::fprintf(stderr, "vla(gr00t): embodiment tag '%s' not in %s; using id %lld\n", e, map_key, (long long)id);
         }
     }
     if (id < 0 || id >= n_emb) throw std::runtime_error("vla: embodiment id out of range");
@@ -311,7 +357,16 @@ void import_gr00t(gguf_reader& g, Checkpoint& ck, bool bf16) {
     const gguf_tensor_meta* pe = g.meta("aex.pos_embd");
     if (!ff0 || !po2 || !se1 || !ad1 || !pe) throw std::runtime_error("vla: gr00t gguf lacks the DiT head tensors (ff0, proj_out2, state_enc, act_dec, pos_embd)");
     const int64_t I = ff0->ne[1], O = po2->ne[1], Hs = se1->ne[0], Hd = ad1->ne[0], max_pos = pe->ne[1];
-    ck.set_key("arch", "gr00t_n1d5");
+    // text rows (N1.6 / N1.7): the token embedding matrix at the backbone width, when the file has one
+    int64_t vocab = 0, n_lang = 0;
+    if (alt) {
+        const gguf_tensor_meta* te = g.meta("token_embd.weight");
+        if (te && te->ne[0] == Wv && te->nelements() / te->ne[0] > 0) {
+            vocab = te->nelements() / te->ne[0];
+            n_lang = u_or("max_seq_len", 1024);
+        }
+    }
+    ck.set_key("arch", alt ? "gr00t_n1d6" : "gr00t_n1d5");
     ck.set_key("dtype", bf16 ? "bf16" : "f32");
     ck.set_key("n_layers", L);
     ck.set_key("n_q_heads", H);
@@ -320,9 +375,10 @@ void import_gr00t(gguf_reader& g, Checkpoint& ck, bool bf16) {
     ck.set_key("hidden", Wv);
     ck.set_key("expert_h", W);
     ck.set_key("ffn_dim", I);
-    ck.set_key("n_img", u_or("n_img_tokens", 256));
-    ck.set_key("n_lang", (int64_t)0);
-    ck.set_key("vocab", (int64_t)0);
+    ck.set_key("n_img", u_or("n_img_tokens", alt ? 64 : 256));
+    ck.set_key("n_lang", n_lang);
+    ck.set_key("vocab", vocab);
+    if (alt) ck.set_key("attend_text_every_n", text_every);
     ck.set_key("n_suffix", 1 + NF + AH);
     ck.set_key("max_action_dim", A);
     ck.set_key("max_state_dim", sd);
@@ -362,7 +418,13 @@ void import_gr00t(gguf_reader& g, Checkpoint& ck, bool bf16) {
     ck.add_f32("aex.ad_l2W", {A, Hd}, im.cat_w("aex.act_dec.l2.W", id, A, Hd));
     ck.add_f32("aex.ad_l2b", {A}, im.cat_b("aex.act_dec.l2.b", id, A));
     ck.add_f32("aex.pos_embd", {max_pos, W}, im.mat("aex.pos_embd", max_pos, W));
-    ck.add_f32("aex.future_tokens", {NF, W}, im.mat("aex.future_tokens", NF, W));
+    if (NF > 0) ck.add_f32("aex.future_tokens", {NF, W}, im.mat("aex.future_tokens", NF, W));
+    if (vocab > 0) put_token_embeddings(path, g, ck, "token_embd.weight", vocab, Wv, [&]() { return im.mat("token_embd.weight", vocab, Wv); });
+    if (variant == 6) {
+        ck.set_key("vlln_eps", f_or("vlln_eps", 1e-5));
+        ck.add_f32("prefix.vlln_w", {Wv}, im.vec("aex.vlln.weight", Wv));
+        ck.add_f32("prefix.vlln_b", {Wv}, im.vec("aex.vlln.bias", Wv));
+    }
     for (int64_t l = 0; l < L; ++l) {
         const std::string a = "aex.dit." + std::to_string(l) + ".", e = "ex." + std::to_string(l) + ".", p = "vlm." + std::to_string(l) + ".";
         const bool self = interleave != 0 && l % 2 == 1;
@@ -495,7 +557,9 @@ Checkpoint import_gguf(const std::string& path) {
     if (g.has("smolvla.architecture")) import_flow(path, g, ck, bf16, "smolvla");
     else if (g.has("pi05.architecture")) import_flow(path, g, ck, bf16, "pi05");
     else if (g.has("pi0.architecture")) import_flow(path, g, ck, bf16, "pi0");
-    else if (g.has("gr00t_n1_5.architecture")) import_gr00t(g, ck, bf16);
+    else if (g.has("gr00t_n1_5.architecture")) import_gr00t(path, g, ck, bf16, 5);
+    else if (g.has("gr00t_n1_6.architecture")) import_gr00t(path, g, ck, bf16, 6);
+    else if (g.has("gr00t_n1_7.architecture")) import_gr00t(path, g, ck, bf16, 7);
     else if (g.has("bitvla.architecture") || g.has("bitvla.lm.hidden")) import_bitvla(path, g, ck);
     else throw std::runtime_error("vla: " + path + ": no importer for this gguf's architecture");
     return ck;
