@@ -194,6 +194,43 @@ def test_linear_bias_residual(dtype, M, N, K):
         assert bf16_close(as_f32(y, dtype), want)
 
 
+@pytest.mark.parametrize("M,N,K", [(50, 720, 960), (3, 37, 2048), (64, 1601, 52), (33, 8, 4), (50, 64, 2052)])
+def test_fp32_rows_of_one_observation_take_the_fma_kernel(M, N, K, monkeypatch):
+    """At most 64 fp32 rows go through the FMA kernel (8 columns per workgroup, 16 partial sums
+    per output).  It and the MFMA kernel (pinned with VLA_GEMM_TILE) against the oracle at the
+    fp32 bar and against each other, with ragged N, K not a multiple of 64, bias, activation,
+    column gate and residual."""
+    r = np.random.default_rng(1700 + N)
+    x = r.standard_normal((M, K)).astype(np.float32)
+    W = (r.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32)
+    b = (0.1 * r.standard_normal(N)).astype(np.float32)
+    gate = (1.0 + 0.2 * r.standard_normal(N)).astype(np.float32)
+    res = r.standard_normal((M, N)).astype(np.float32)
+    outs = []
+    for tile in (None, "4"):
+        if tile is None:
+            monkeypatch.delenv("VLA_GEMM_TILE", raising=False)
+        else:
+            monkeypatch.setenv("VLA_GEMM_TILE", tile)
+        pkg.lib().vla_kernels_reload_env()
+        y, y2, y3 = empty((M, N), F32), empty((M, N), F32), empty((M, N), BF16)
+        pkg.call("vla_linear_act", dev(x), dev(W), dev(b), dev(res), y, F32, F32, M, N, K, pkg.VLA_ACT_SILU)
+        pkg.call("vla_linear_gated", dev(x), dev(W), None, dev(gate), dev(res), y2, F32, F32, M, N, K)
+        pkg.call("vla_linear", dev(x), dev(W), dev(b), to_dev(orc.round_bf16(res), BF16), y3, F32, BF16, M, N, K)
+        sync()
+        outs.append((host(y), host(y2), as_f32(y3, BF16)))
+    monkeypatch.delenv("VLA_GEMM_TILE", raising=False)
+    pkg.lib().vla_kernels_reload_env()
+    lin = orc.linear(x, W)
+    want = orc.silu(lin + b) + res
+    want2 = lin * gate + res
+    want3 = lin + b + orc.round_bf16(res)
+    for got, got2, got3 in outs:
+        assert rel_err(got, want) < FP32_TOL and rel_err(got2, want2) < FP32_TOL
+        assert bf16_close(got3, want3)
+    assert rel_err(outs[0][0], outs[1][0]) < FP32_TOL
+
+
 @pytest.mark.parametrize("M,N,K", [(150, 720, 720), (333, 200, 1104), (64, 1600, 48)])
 def test_linear_bf16_every_kernel_and_tiling_gives_the_same_bits(tune, M, N, K):
     """The direct-to-LDS kernel and the register-staged one, in every tile configuration, add

@@ -1688,7 +1688,14 @@ int launch_d(AttnArgs& a, vla_stream_t stream, Scratch& sc) {
     // Only worthwhile while a partial (r_pad rows of D+2 floats) stays small next to the
     // K/V slice it summarises; with many query rows the partials would outweigh the cache.
     const size_t partial_bytes = (size_t)a.r_pad * (D + 2) * 4, tile_bytes = (size_t)2 * SPLIT_KEYS * D * sizeof(T);
-    if (wgs < 256 && key_tiles > 1 && partial_bytes <= tile_bytes) {
+    // fp32 launches with few row tiles in all (batch 1) also split while the partials of the
+    // whole launch stay within a few MiB: a key tile takes such a launch about 6 us, whatever
+    // it shares, so the serial walk over the keys is its whole cost and the partials are noise
+    // (SmolVLA's single fp32 layer at batch 1: 31 -> 15 us with the merge pass).  The bf16
+    // kernels walk a tile in 2 us and lose more to the merge launch than they gain.
+    const bool cheap = sizeof(T) == 4 && (long)a.batch * a.Hkv * n_tiles <= 64 && !tn.attn_no_small &&
+                       (size_t)a.batch * a.Hkv * partial_bytes * (size_t)(key_tiles < 32 ? key_tiles : 32) <= ((size_t)4 << 20);
+    if (wgs < 256 && key_tiles > 1 && (partial_bytes <= tile_bytes || cheap)) {
         int want = (int)((512 + wgs - 1) / wgs);
         if (want > key_tiles) want = key_tiles;
         if (want > 32) want = 32;

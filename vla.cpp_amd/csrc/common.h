@@ -26,8 +26,10 @@ struct Tuning {
     bool attn_no_arrive = false; // VLA_ATTN_NO_ARRIVE: no in-launch merge by the last slice to arrive
     bool attn_no_direct = false; // VLA_ATTN_NO_DIRECT: never the register-direct kernel
     bool attn_no_stream = false; // VLA_ATTN_NO_STREAM: never the streaming (LDS-ring) form of the register-direct kernel
+    bool attn_no_small = false;  // VLA_ATTN_NO_SMALL: fp32 launches with few row tiles do not split their keys beyond the usual rule
     int attn_direct_rows = 32;   // VLA_ATTN_DIRECT_ROWS: row limit of the register-direct kernel
     int gemm_tile = -1;          // VLA_GEMM_TILE: 0..5
+    int gemm_panel = 0;          // VLA_GEMM_PANEL: N tiles per panel of an XCD's walk over its tiles; 0 = by size
     int gemm_dl = -1;            // VLA_GEMM_DL: 0 pins the register-staged GEMM
     int gemm_stages = 0;         // VLA_GEMM_STAGES: ring depth of the direct-to-LDS GEMM
     int ternary_tile = 0;        // VLA_TERNARY_TILE: 64 | 128 | 256 (32x32x32 kernels) | 16 (16x16x64 kernel)

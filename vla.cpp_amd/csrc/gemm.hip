@@ -45,6 +45,7 @@ struct GemmArgs {
     const void* W;
     const float* bias;
     int M, N, K, n_tiles, xm, xn;
+    int pn;  // N tiles per panel of an XCD's walk (see xcd_tile)
     // PLAIN, GLU
     const void* residual;
     void* Y;
@@ -71,6 +72,36 @@ struct GemmArgs {
     const float* colsum;
     const void* norm_w;  // ternary GEMV with the RMSNorm and quantisation of its rows inside: A is bf16, this the norm weight
 };
+
+// Workgroup -> tile.  Workgroup i runs on XCD i % 8; the XCDs form an xm x xn grid over the
+// tile grid and XCD (xr, xc) owns the tiles (m, n) with m % xm == xr, n % xn == xc.  Its
+// workgroups walk them panel by panel: pn of its N tiles at a time, every M tile of the XCD
+// against that panel before the next panel starts, so that the panel's rows of W stay in the
+// XCD's L2 while the rows of A stream past them once per panel.  (With all of W in one
+// panel and W larger than the L2, W would stream again for every few M tiles instead.)
+__device__ __forceinline__ bool xcd_tile(const GemmArgs& a, int n_wg_tiles, int m_wg_tiles, int& mtw, int& ntw) {
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int cn = (n_wg_tiles + a.xn - 1) / a.xn;  // N tiles per XCD column (padded)
+    const int cm = (m_wg_tiles + a.xm - 1) / a.xm;
+    int ml, nl;
+    if (a.pn >= cn) {
+        nl = local % cn;
+        ml = local / cn;
+    } else {
+        const int per_panel = a.pn * cm, full = cn / a.pn;
+        int p = local / per_panel, rem = local - p * per_panel, w = a.pn;
+        if (p >= full) {  // the last, narrower panel
+            p = full;
+            rem = local - full * per_panel;
+            w = cn - full * a.pn;
+        }
+        ml = rem / w;
+        nl = p * a.pn + rem - ml * w;
+    }
+    ntw = nl * a.xn + xcd % a.xn;
+    mtw = ml * a.xm + xcd / a.xn;
+    return ntw < n_wg_tiles && mtw < m_wg_tiles;
+}
 
 template <typename T> struct Traits;
 template <> struct Traits<bf16_t> {
@@ -425,11 +456,8 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
     // the N tiles = j (mod xn), so each L2 fetches 1/xm of A and 1/xn of W instead of the
     // whole of either (the host picks the split that minimises the total).
     const int n_wg_tiles = (a.n_tiles + TN - 1) / TN, m_wg_tiles = (a.M + ROWS_A - 1) / ROWS_A;
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int cn = (n_wg_tiles + a.xn - 1) / a.xn;  // N tiles per XCD column (padded)
-    const int ntw = (local % cn) * a.xn + xcd % a.xn;
-    const int mtw = (local / cn) * a.xm + xcd / a.xn;
-    if (ntw >= n_wg_tiles || mtw >= m_wg_tiles) return;
+    int mtw, ntw;
+    if (!xcd_tile(a, n_wg_tiles, m_wg_tiles, mtw, ntw)) return;
     const int m0 = mtw * ROWS_A;
     TileCols tc[TN];
 #pragma unroll
@@ -682,11 +710,8 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     const int wm = wave >> 1, wn = wave & 1;
     const int g = lane >> 5, r = lane & 31;
     const int n_wg_tiles = (a.n_tiles + TN - 1) / TN, m_wg_tiles = (a.M + ROWS_A - 1) / ROWS_A;
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int cn = (n_wg_tiles + a.xn - 1) / a.xn;
-    const int ntw = (local % cn) * a.xn + xcd % a.xn;
-    const int mtw = (local / cn) * a.xm + xcd / a.xn;
-    if (ntw >= n_wg_tiles || mtw >= m_wg_tiles) return;
+    int mtw, ntw;
+    if (!xcd_tile(a, n_wg_tiles, m_wg_tiles, mtw, ntw)) return;
     const int m0 = mtw * ROWS_A;
     TileCols tc[TN];
 #pragma unroll
@@ -1411,6 +1436,141 @@ __global__ void __launch_bounds__(256, 2) ternary_gemm_x16_kernel(GemmArgs a) {
     }
 }
 
+// fp32 projection of a few rows (M <= 64: the suffix of one observation in the reference's
+// own fp32 case).  The fp32 MFMA gives a CU 256 flop per clock, no more than its plain FMA
+// rate, and the MFMA kernel's 64 x 64 tiles leave a 50 x 720 x 960 problem on 12 CUs that walk
+// K one after the other (22 us).  Here a wavefront owns 4 rows and 8 output columns and its
+// lanes share K: lane l sums k = 256 j + 4 l + (0..3), so a load instruction reads 1 KiB of
+// consecutive bytes of a row of x or W, K = 960 is four rounds of loads (two in flight at a
+// time), and a 50 x 720 problem is 1170 wavefronts.  The 64 partial sums of an output meet
+// through six xor-shuffles, in that order whatever the launch.  The 8 columns are two runs
+// of 4: next to each other for a plain projection, half a head apart where the QKV epilogue
+// rotates, so that lane ks < 16 ends up with both members of a rotation pair (row ks / 4 of
+// the four, columns ks % 4 of either run).
+constexpr int SKINNY_MAX_M = 64;
+template <int kEpi>
+__global__ void __launch_bounds__(256) linear_f32_skinny_kernel(GemmArgs a) {
+    const int tid = threadIdx.x, ks = tid & 63, rg = (tid >> 6) + 4 * blockIdx.y;
+    const int K = a.K;
+    // W rows of the two runs, and for QKV the segment and the segment-local columns
+    int base0 = blockIdx.x * 8, base1 = base0 + 4, seg = 0, col0 = base0, col1 = base1;
+    bool rope = false;
+    if (kEpi == EPI_QKV) {
+        const int gq = a.Hq * a.D / 8, gk = a.nk * a.D / 8;
+        int lt = blockIdx.x, seg_base = 0;
+        if (lt >= gq + gk) {
+            seg = 2;
+            lt -= gq + gk;
+            seg_base = (a.Hq + a.nk) * a.D;
+        } else if (lt >= gq) {
+            seg = 1;
+            lt -= gq;
+            seg_base = a.Hq * a.D;
+        }
+        rope = a.cos_t != nullptr && seg != 2;
+        if (rope) {
+            const int gph = a.D / 8;  // groups per head
+            col0 = (lt / gph) * a.D + (lt % gph) * 4;
+            col1 = col0 + a.D / 2;
+        } else {
+            col0 = lt * 8;
+            col1 = col0 + 4;
+        }
+        base0 = seg_base + col0;
+        base1 = seg_base + col1;
+    }
+    const float* xr[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xr[i] = (const float*)a.A + (long)min(4 * rg + i, a.M - 1) * K;
+    const float* wr[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) wr[c] = (const float*)a.W + (long)min((c < 4 ? base0 : base1 - 4) + c, a.N - 1) * K;
+    float acc[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[i][c] = 0.f;
+    if (4 * rg < a.M) {  // whole wavefronts
+#pragma unroll 2
+        for (int k = 4 * ks; k < K; k += 256) {
+            f32x4_t xv[4], wv[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) xv[i] = *reinterpret_cast<const f32x4_t*>(xr[i] + k);
+#pragma unroll
+            for (int c = 0; c < 8; ++c) wv[c] = *reinterpret_cast<const f32x4_t*>(wr[c] + k);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int c = 0; c < 8; ++c)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) acc[i][c] = fmaf(xv[i][e], wv[c][e], acc[i][c]);
+        }
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) acc[i][c] += __shfl_xor(acc[i][c], off, 64);
+    if (ks >= 16) return;
+    float lo = 0.f, hi = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int cp = 0; cp < 4; ++cp)
+            if (ks == i * 4 + cp) {
+                lo = acc[i][cp];
+                hi = acc[i][cp + 4];
+            }
+    const int m = 4 * rg + (ks >> 2), cp = ks & 3;
+    if (m >= a.M) return;
+    if (kEpi == EPI_PLAIN) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int n = (e ? base1 : base0) + cp;
+            if (n >= a.N) continue;
+            float y = e ? hi : lo;
+            if (a.bias) y += a.bias[n];
+            if (a.act != VLA_ACT_NONE) y = apply_act(y, a.act);
+            if (a.col_gate) y *= a.col_gate[n];
+            const long o = (long)m * a.N + n;
+            if (a.out_bf16) {
+                if (a.residual) y += bf2f(((const bf16_t*)a.residual)[o]);
+                ((bf16_t*)a.Y)[o] = f2bf(y);
+            } else {
+                if (a.residual) y += ((const float*)a.residual)[o];
+                ((float*)a.Y)[o] = y;
+            }
+        }
+        return;
+    }
+    // QKV: bias, rotation, scatter (the MFMA kernel's epilogue, two columns per lane)
+    const int b = m / a.S, sq = m % a.S;
+    if (a.bias) {
+        lo += a.bias[base0 + cp];
+        hi += a.bias[base1 + cp];
+    }
+    if (rope) {
+        const int half = a.D >> 1, p0 = (col0 % a.D) + cp;
+        const float c = a.cos_t[(long)sq * half + p0], sn = a.sin_t[(long)sq * half + p0];
+        const float x0 = lo, x1 = hi;
+        lo = x0 * c - x1 * sn;
+        hi = x1 * c + x0 * sn;
+    }
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const float v = e ? hi : lo;
+        const int col = (e ? col1 : col0) + cp;
+        if (seg == 0) {
+            ((float*)a.q_out)[(long)m * (a.Hq * a.D) + col] = v;
+        } else {
+            const int head = col / a.D, d = col % a.D;
+            if (seg == 1) ((float*)a.k_cache)[(((long)b * a.Hkv + head) * a.t_max + a.tok_offset + sq) * a.D + d] = v;
+            else ((float*)a.vt_cache)[(((long)b * a.Hkv + head) * a.D + d) * a.t_max + a.tok_offset + sq] = v;
+        }
+    }
+}
+
 // Ternary GEMV for a handful of rows (single-token decode, M <= 32).  A workgroup owns 32
 // output columns; its 8 wavefronts each take one eighth of K and multiply it with
 // v_mfma_i32_32x32x32_i8 as C[n][m] = sum_k W[n][k] * A[m][k] (weight fragment as the A
@@ -1597,20 +1757,30 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
     }
 }
 
-// XCD grid xm x xn = 8 for a tile grid of m_wg x n_wg workgroup tiles: every L2 reads its M
-// tiles' rows of A and its N tiles' rows of W once; the split with the least total,
+// XCD grid xm x xn = 8 for a tile grid of m_wg x n_wg workgroup tiles of tile_cols columns:
+// every L2 reads its N tiles' rows of W once and its M tiles' rows of A once per panel of N
+// tiles (xcd_tile).  One panel while an XCD's rows of W fit in half of its 4 MiB L2 beside
+// the streaming A and C; else panels of about 2 MiB of W.  The split with the least total,
 // counting the padding of the tile grid.  Returns the grid size.
-unsigned xcd_split(GemmArgs& a, int m_wg, int n_wg, double w_bytes_per_elem) {
-    const double bytes_a = (double)a.M * a.K, bytes_w = (double)a.N * a.K * w_bytes_per_elem;
+unsigned xcd_split(GemmArgs& a, int m_wg, int n_wg, double w_bytes_per_elem, int tile_cols, double a_bytes_per_elem) {
+    const double bytes_a = (double)a.M * a.K * a_bytes_per_elem, bytes_w = (double)a.N * a.K * w_bytes_per_elem;
+    const double tile_w = (double)tile_cols * a.K * w_bytes_per_elem, l2_panel = 2.0 * 1024 * 1024;
+    const int forced = tuning().gemm_panel;  // 0 = by size, > 0 = that many tiles per panel
     double best = -1;
     for (int xm = 1; xm <= 8; xm *= 2) {
         const int xn = 8 / xm;
-        const long wgs = (long)((m_wg + xm - 1) / xm) * ((n_wg + xn - 1) / xn) * 8;
-        const double cost = (bytes_a * xn + bytes_w * xm) * (double)wgs / ((double)m_wg * n_wg);
+        const int cn = (n_wg + xn - 1) / xn, cm = (m_wg + xm - 1) / xm;
+        int pn = cn;
+        if (forced > 0) pn = forced < cn ? forced : cn;
+        else if (cn * tile_w > l2_panel && cm >= 4) pn = tile_w >= l2_panel ? 1 : (int)(l2_panel / tile_w);
+        const int panels = (cn + pn - 1) / pn;
+        const long wgs = (long)cm * cn * 8;
+        const double cost = (bytes_a * xn * panels + bytes_w * xm) * (double)wgs / ((double)m_wg * n_wg);
         if (best < 0 || cost < best) {
             best = cost;
             a.xm = xm;
             a.xn = xn;
+            a.pn = pn;
         }
     }
     return (unsigned)(((m_wg + a.xm - 1) / a.xm) * ((n_wg + a.xn - 1) / a.xn) * 8);
@@ -1618,13 +1788,14 @@ unsigned xcd_split(GemmArgs& a, int m_wg, int n_wg, double w_bytes_per_elem) {
 
 template <typename T, int kEpi, int TM, int TN, int KB, int DEPTH>
 void launch_cfg(GemmArgs a, hipStream_t st) {
-    const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, kEpi == EPI_TERNARY ? 0.25 : 1.0);
+    const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, kEpi == EPI_TERNARY ? 0.25 : sizeof(T), 64 * TN,
+                                    kEpi == EPI_TERNARY ? 1.0 : sizeof(T));
     gemm_kernel<T, kEpi, TM, TN, KB, DEPTH><<<grid, 256, 0, st>>>(a);
 }
 
 template <int kEpi, int TM, int TN, int KB, int NS>
 void launch_dl(GemmArgs a, hipStream_t st) {
-    const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, 1.0);
+    const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, 2.0, 64 * TN, 2.0);
     if constexpr (kEpi == EPI_QKV) {
         if (a.norm_eps >= 0.f && a.colsum) {
             gemm_dl_kernel<kEpi, TM, TN, KB, NS, NORM_LAYER><<<grid, 256, 0, st>>>(a);
@@ -1645,6 +1816,14 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
     if (a.M == 0 || n_tiles == 0) return VLA_K_OK;
     a.n_tiles = n_tiles;
     hipStream_t st = (hipStream_t)stream;
+    if constexpr (std::is_same<T, float>::value && (kEpi == EPI_PLAIN || kEpi == EPI_QKV)) {
+        // a few fp32 rows: the FMA kernel (VLA_GEMM_TILE pins the MFMA kernel's tiles instead)
+        if (a.M <= SKINNY_MAX_M && a.K % 4 == 0 && a.norm_eps < 0.f && tuning().gemm_tile < 0 && (uintptr_t)a.A % 16 == 0 &&
+            (uintptr_t)a.W % 16 == 0 && (kEpi == EPI_PLAIN || a.D % 8 == 0)) {
+            linear_f32_skinny_kernel<kEpi><<<dim3((unsigned)((a.N + 7) / 8), (unsigned)((a.M + 15) / 16)), 256, 0, st>>>(a);
+            return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+        }
+    }
     if constexpr (kEpi != EPI_TERNARY) {
         // VLA_GEMM_TILE = 0..5 pins the tile configuration and VLA_GEMM_STAGES the ring depth
         // of the direct-to-LDS kernel (tests and tuning); unset = by shape.

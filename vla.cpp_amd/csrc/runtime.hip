@@ -34,8 +34,10 @@ void load_locked() {
     t.attn_no_arrive = getenv("VLA_ATTN_NO_ARRIVE") != nullptr;
     t.attn_no_direct = getenv("VLA_ATTN_NO_DIRECT") != nullptr;
     t.attn_no_stream = getenv("VLA_ATTN_NO_STREAM") != nullptr;
+    t.attn_no_small = getenv("VLA_ATTN_NO_SMALL") != nullptr;
     t.attn_direct_rows = env_int("VLA_ATTN_DIRECT_ROWS", 32);
     t.gemm_tile = env_int("VLA_GEMM_TILE", -1);
+    t.gemm_panel = env_int("VLA_GEMM_PANEL", 0);
     t.gemm_dl = env_int("VLA_GEMM_DL", -1);
     t.gemm_stages = env_int("VLA_GEMM_STAGES", 0);
     t.ternary_tile = env_int("VLA_TERNARY_TILE", 0);
