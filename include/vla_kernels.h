@@ -192,7 +192,22 @@ VLA_KAPI int vla_layernorm_attn_qkv_rope(const void* x, const void* W_folded, co
                                          void* k_cache, void* vt_cache, int t_max, int tok_offset, float ln_eps,
                                          vla_stream_t stream);
 
-/* Host helper for the call above (bf16 weights [N][K], fp32 scale/shift [K], fp32 bias [N]
+/* A DiT self-attention block's front half in one launch: modulated LayerNorm, the Q / K / V
+ * projections and the attention of each observation's S tokens over themselves, replacing
+ * adaln -> mm_w(Wq / Wk / Wv) -> attention with enc = nullptr (src/modules/dit_head.cpp:111-125).
+ * The block's K and V never reach memory: nothing but this attention reads them.
+ *   x [M][K] bf16, M = batch * S rows, observation-major; W_folded [3 * n_heads * head_dim][K]
+ *   (Q rows, K rows, V rows), colsum and bias fp32 over the same rows, as for
+ *   vla_layernorm_attn_qkv_rope; no rotation, no mask (the DiT block is bidirectional);
+ *   out [M][n_heads * head_dim] bf16, token-major as vla_attn_prefix_suffix writes it.
+ * Built for head_dim 48, S <= 32, K a multiple of 64 and >= 256, n_heads a multiple of 8, bf16, 16-byte
+ * aligned operands; VLA_K_ERR_SHAPE otherwise (use vla_layernorm_attn_qkv_rope +
+ * vla_attn_prefix_suffix then). */
+VLA_KAPI int vla_layernorm_qkv_self_attention(const void* x, const void* W_folded, const float* colsum, const float* bias,
+                                              int dtype, int M, int K, int S, int n_heads, int head_dim, float scale,
+                                              float ln_eps, void* out, vla_stream_t stream);
+
+/* Host helper for the two calls above (bf16 weights [N][K], fp32 scale/shift [K], fp32 bias [N]
  * or NULL): writes W_out (bf16, rounded to nearest even; may alias W), colsum_out and
  * bias_out (fp32 [N]); colsum is taken over the rounded W_out, the values the launch
  * multiplies. */

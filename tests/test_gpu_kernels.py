@@ -422,6 +422,55 @@ def test_modulated_layernorm_inside_qkv_launch(name, B, S, Hq, Hkv, D, K, self_l
                                                  None, None, x.ctypes.data, None, None, t_max, 0, eps, None) == pkg.VLA_K_ERR_SHAPE
 
 
+@pytest.mark.parametrize("B,S,H,K,bias", [(64, 17, 32, 1536, True), (3, 17, 32, 1536, True), (9, 17, 8, 256, False), (5, 5, 8, 320, True),
+                                          (1, 32, 16, 448, True), (11, 16, 8, 256, True)])
+def test_dit_self_block_front_half_in_one_launch(B, S, H, K, bias):
+    """adaLN -> Q / K / V -> attention of each observation's tokens over themselves
+    (src/modules/dit_head.cpp:111-125 with enc = nullptr) as one launch, against the oracle's
+    adaln -> linear -> attention with Q, K, V rounded to bf16 as both GPU paths keep them, and
+    against the two-launch path.  Batches that do not fill the last workgroup's eight
+    observations, few heads, short K; rows carry a mean of the size of their spread."""
+    D = 48
+    r = np.random.default_rng(4100 + B * S + K)
+    M, N = B * S, 3 * H * D
+    eps, scale = 1e-5, 1.0 / np.sqrt(D)
+    x = orc.round_bf16((2.0 * r.standard_normal((M, K)) * (1.0 + 3.0 * r.random((M, 1))) + 1.5 * r.standard_normal((M, 1))).astype(np.float32))
+    sc = (0.3 * r.standard_normal(K)).astype(np.float32)
+    sh = (0.3 * r.standard_normal(K)).astype(np.float32)
+    W = orc.round_bf16((r.standard_normal((N, K)) / np.sqrt(K)).astype(np.float32))  # scores of about one unit: the softmax is far from uniform
+    b = (0.1 * r.standard_normal(N)).astype(np.float32) if bias else None
+    Wf, cs, bs = np.empty((N, K), np.uint16), np.empty(N, np.float32), np.empty(N, np.float32)
+    assert pkg.lib().vla_fold_adaln_weight_host(orc.to_bf16(W).ctypes.data, None if b is None else b.ctypes.data, sc.ctypes.data,
+                                                sh.ctypes.data, N, K, Wf.ctypes.data, cs.ctypes.data, bs.ctypes.data) == 0
+    dWf, dcs, dbs, dx = dev(Wf), dev(cs), dev(bs), to_dev(x, BF16)
+    fused = empty((M, H * D), BF16)
+    pkg.call("vla_layernorm_qkv_self_attention", dx, dWf, dcs, dbs, BF16, M, K, S, H, D, scale, eps, fused)
+    t_max = 64
+    kc, vc = empty((B, H, t_max, D), BF16), empty((B, H, D, t_max), BF16)
+    q, pair = empty((M, H * D), BF16), empty((M, H * D), BF16)
+    pkg.call("vla_layernorm_attn_qkv_rope", dx, dWf, dcs, dbs, BF16, M, K, S, H, H, 1, 1, D, None, None, q, kc, vc, t_max, 0, eps)
+    pkg.call("vla_attn_prefix_suffix", q, kc, vc, pair, BF16, B, S, H, H, D, t_max, S, scale, pkg.VLA_MASK_NONE, 0, 0, 0, None)
+    sync()
+    y = orc.round_bf16(orc.linear(orc.adaln(x, sc, sh, eps), W, b)).reshape(B, S, 3, H, D)
+    want = np.empty((B, S, H, D), np.float32)
+    for bb in range(B):
+        want[bb] = orc.attention(y[bb, :, 0], y[bb, :, 1], y[bb, :, 2], np.zeros((S, S), np.float32), scale).reshape(S, H, D)
+    got, two = as_f32(fused, BF16).reshape(B, S, H, D), as_f32(pair, BF16).reshape(B, S, H, D)
+    # Held to the oracle as the modulated-LayerNorm projection is (8e-3 of the largest value:
+    # a Q, K or V element that rounds to the other bf16 neighbour moves an output by up to an
+    # ulp of the largest V), and no further from it than the two-launch path; the two GPU paths
+    # share the folded weights and differ by the order of their sums.
+    e1, e2 = rel_err(got, want), rel_err(two, want)
+    assert e1 < 8e-3 and e1 <= 1.25 * e2 + 1e-3, (e1, e2)
+    assert rel_err(got, two) < 8e-3, rel_err(got, two)  # one bf16 ulp of the largest output
+    assert np.mean(np.abs(got - want)) < 2e-3 * np.abs(want).max()
+    # the attention is really over the observation's own tokens: uniform weights are far off
+    assert rel_err(np.broadcast_to(y[:, :, 2].mean(1, keepdims=True), want.shape), want) > 5e-2
+    # shapes the launch is not built for are refused, not served slowly
+    assert pkg.lib().vla_layernorm_qkv_self_attention(dx.data_ptr(), dWf.data_ptr(), dcs.data_ptr(), None, BF16, M, K, S, H, 64, scale,
+                                                      eps, fused.data_ptr(), None) == pkg.VLA_K_ERR_SHAPE
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("M,I,K,act,bias", [(50, 2048, 720, "silu", False), (130, 96, 72, "gelu", True), (1600, 256, 720, "silu", False),
                                            (17, 6144, 1536, "gelu", True)])

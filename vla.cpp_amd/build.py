@@ -27,7 +27,7 @@ def sources():
 # Kernels that keep registers "in flight" between an inline-assembly load and its wait must
 # not spill: a spilled in-flight register is stored before its data arrives and reused while
 # the load is still due.  Their scratch size is read from the compiler's resource remarks.
-NO_SPILL_KERNELS = {"gemm.hip": ["ternary_gemm_x16_kernel"]}
+NO_SPILL_KERNELS = {"gemm.hip": ["ternary_gemm_x16_kernel"], "dit_self.hip": ["dit_self_block_kernel"]}
 
 
 def _check_no_spill(src, remarks):
@@ -47,15 +47,22 @@ def _check_no_spill(src, remarks):
             raise RuntimeError("no resource remarks for %s in %s" % (kernel, src))
 
 
+# Per-file compiler options.  dit_self.hip: accumulators of its MFMAs stay in the ordinary
+# vector registers; left to itself the compiler parks them in the accumulation registers and
+# copies them back and forth around every MFMA (1300 copies in the K loop).
+EXTRA_FLAGS = {"dit_self.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+
+
 def _compile(src):
     obj = os.path.join(OBJ, os.path.basename(src) + ".o")
     extra = ["-Rpass-analysis=kernel-resource-usage"] if os.path.basename(src) in NO_SPILL_KERNELS else []
+    extra = extra + EXTRA_FLAGS.get(os.path.basename(src), [])
     cmd = [HIPCC] + FLAGS + extra + ["-x", "hip", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, err))
-    if extra:
+    if os.path.basename(src) in NO_SPILL_KERNELS:
         _check_no_spill(src, err)
         # the remarks are not diagnostics: drop them (and their source excerpts) from what verbose builds print
         keep, skip = [], 0

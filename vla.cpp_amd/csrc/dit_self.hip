@@ -1,0 +1,389 @@
+// A DiT self-attention block's front half in one launch: modulated LayerNorm, the Q / K / V
+// projections and the attention over the block's own tokens (src/modules/dit_head.cpp:111-125
+// with enc = nullptr: adaln -> attn_q / attn_k / attn_v -> attention over the S tokens of the
+// observation).  Nothing of it reaches memory but the attention output: the block's K and V
+// are used by this attention and by nothing else.
+//
+// Tiling.  The projection is small next to the chip (GR00T at batch 64: 1088 x 4608 x 1536),
+// so what counts is that every CU gets the same share and no CU waits for another launch.
+// A workgroup owns OB <= 8 observations (OB S <= 144 rows; 8 observations of 17 tokens = 136 rows)
+// and ONE head: the head's 48 query, 48 key and 48 value rows of W, 144 output columns.  At
+// batch 64 with 32 heads that is 256 workgroups of identical size, and all operands of the
+// attention of its (observation, head) pairs end up in the workgroup's LDS.  Workgroup i runs
+// on XCD i % 8 and takes head i % H: an XCD's L2 holds the W rows of a few heads and all of x.
+//
+// Product.  v_mfma_f32_16x16x32_bf16, 9 x 9 blocks of 16 x 16 over four wavefronts as 2 x 2:
+// a wavefront owns the block rows wm, wm + 2, ... and block columns wn, wn + 2, ... (5 or 4 of
+// each).  Eight wavefronts with smaller shares read each fragment more often: a CU's LDS
+// delivers 128 bytes a clock, 40 fragment reads of 1 KiB per 32-k chunk already take 320 clocks
+// next to the 400 of the 25 MFMAs of the largest share, and 64 reads take longer than the
+// MFMAs.  K is walked in tiles of 64 through a four-stage LDS ring filled by
+// global_load_lds_dwordx4 (16 bytes per lane straight into LDS, 128-byte rows, the 16-byte
+// piece p of row r kept at position p ^ ((r >> 1) & 7) so that the 16 rows of a fragment read
+// cover all banks once), three tiles in flight and one barrier per tile; the fragments of a
+// 32-k chunk are read between the MFMAs of the chunk before it.  The LayerNorm is taken
+// inside: the launch multiplies raw rows of x by weights that carry (1 + scale)
+// (vla_fold_adaln_weight_host), sums each row and its squares from the fragments it multiplies
+// anyway, and forms rstd (acc - mean colsum[n]) + bias[n] on the way out.
+//
+// Attention.  Q, K and V^T of the tile go to LDS as bf16 (the precision the unfused path keeps
+// them in).  A wavefront takes whole (observation, head) pairs: scores as S^T = K Q^T with
+// v_mfma_f32_16x16x16_bf16, so that a lane ends up with four consecutive keys of one query,
+// which is the layout the same instruction wants for P as the left operand of P V; softmax in
+// registers (max and sum over the lane's values and the three other lanes of the query).
+#include "common.h"
+
+namespace vk {
+namespace {
+
+constexpr int FS_D = 48;            // head width this kernel is built for
+constexpr int FS_COLS = 3 * FS_D;   // q, k, v columns of one head
+constexpr int FS_ROWS = 144;        // rows of x per workgroup (9 blocks of 16)
+constexpr int FS_KB = 128;          // bytes of K per staged row (64 bf16)
+constexpr int FS_NS = 4;            // ring depth
+constexpr int FS_STAGE = (FS_ROWS + FS_COLS) * FS_KB;  // 36 KiB
+constexpr int FS_QS = 104;          // bf16 per row of the Q | K tile in LDS (208 bytes: 16 rows start in 16 different banks)
+constexpr int FS_VS = 36;           // bf16 per row of a V^T tile: 32 keys and padding (72 bytes)
+constexpr int FS_MAX_S = 32;        // tokens per observation: two 16-wide MFMA blocks
+constexpr int FS_MAX_OB = 8;        // observations per workgroup (V^T tiles held in LDS)
+
+struct SelfArgs {
+    const bf16_t* x;
+    const bf16_t* W;
+    const float* colsum;
+    const float* bias;
+    bf16_t* out;
+    int M, K, S, H, OB;
+    float scale, eps;
+};
+
+__device__ __forceinline__ float sum_squares_bf16x2(uint32_t u, float acc) {
+    const __bf16 __attribute__((ext_vector_type(2))) v = __builtin_bit_cast(__bf16 __attribute__((ext_vector_type(2))), u);
+    return __builtin_amdgcn_fdot2_f32_bf16(v, v, acc, false);
+}
+__device__ __forceinline__ float sum_pair_bf16x2(uint32_t u, float acc) {
+    typedef __bf16 __attribute__((ext_vector_type(2))) bf2_t;
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2_t, u), __builtin_bit_cast(bf2_t, 0x3f803f80u), acc, false);
+}
+
+// The K walk of one wavefront: NR x NC blocks, block rows wm + 2 i and block columns wn + 2 j.
+// Straight-line per (NR, NC): the four wavefronts of a workgroup fall into four classes and each
+// runs its own copy, so no block is computed twice and none sits behind a branch (a branch
+// inside the loop body cuts it into pieces the scheduler cannot interleave).
+template <int NR, int NC>
+__device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* lds, const unsigned char* const (&ap)[5],
+                                            const unsigned char* const (&wp)[5], uint32_t lds0, int koff, bool tail, int wm, int wn,
+                                            int c, int q, f32x4_t (&acc)[5][5], float (&ssq)[5], float (&ssum)[5]) {
+    constexpr bool STATS = NC == 5;  // the wavefronts with block column 0: one per row half
+    const int fsw = (c >> 1) & 7;
+    auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
+        const long kb = ((long)kt * 64 + koff) * 2;
+        const uint32_t base = lds0 + stage * FS_STAGE;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) load_to_lds16(ap[v] + kb, base + v * 4096);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) load_to_lds16(wp[v] + kb, base + FS_ROWS * FS_KB + v * 4096);
+        if (tail) {
+            load_to_lds16(ap[4] + kb, base + 4 * 4096);
+            load_to_lds16(wp[4] + kb, base + FS_ROWS * FS_KB + 4 * 4096);
+        }
+    };
+    u32x4_t fa[2][NR], fw[2][NC];  // fragment sets of two consecutive chunks
+    auto read_frags = [&](int set, int stage, int ch) __attribute__((always_inline)) {
+        const unsigned char* base = lds + stage * FS_STAGE;
+        const int off = ((4 * ch + q) ^ fsw) * 16;
+#pragma unroll
+        for (int i = 0; i < NR; ++i) fa[set][i] = *reinterpret_cast<const u32x4_t*>(base + ((wm + 2 * i) * 16 + c) * FS_KB + off);
+#pragma unroll
+        for (int j = 0; j < NC; ++j)
+            fw[set][j] = *reinterpret_cast<const u32x4_t*>(base + FS_ROWS * FS_KB + ((wn + 2 * j) * 16 + c) * FS_KB + off);
+    };
+    auto mfma_chunk = [&](int set) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i)
+#pragma unroll
+            for (int j = 0; j < NC; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fa[set][i]),
+                                                                  __builtin_bit_cast(bf16x8_t, fw[set][j]), acc[i][j], 0, 0, 0);
+        if (STATS) {
+#pragma unroll
+            for (int i = 0; i < NR; ++i)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    ssq[i] = sum_squares_bf16x2(fa[set][i][e], ssq[i]);
+                    ssum[i] = sum_pair_bf16x2(fa[set][i][e], ssum[i]);
+                }
+        }
+    };
+    // Stage kt % 4 holds tile kt.  Chunk 0 of tile kt is multiplied while chunk 1's fragments
+    // are read; then the wavefront waits for its loads of tile kt + 1 and meets the others (every
+    // fragment of tile kt is in registers by then, so its stage takes tile kt + 4), reads chunk 0
+    // of tile kt + 1 and multiplies chunk 1 of tile kt meanwhile.  K >= 256 (four tiles), so the
+    // ring fills before the loop; nothing is fetched past the last tile.
+    const int nkt = a.K / 64;
+#pragma unroll
+    for (int t = 0; t < FS_NS; ++t) issue(t, t);
+    if (tail) wait_vmcnt<30>();
+    else wait_vmcnt<24>();
+    __syncthreads();
+    read_frags(0, 0, 0);
+    int st = 0;
+    for (int kt = 0; kt < nkt; ++kt) {
+        const int nx = st == FS_NS - 1 ? 0 : st + 1;
+        read_frags(1, st, 1);
+        mfma_chunk(0);
+        // a fragment read between every two MFMAs: the reads' issue slots hide behind the matrix pipe
+#pragma unroll
+        for (int g = 0; g < NR + NC; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // tile kt + 1 has landed; up to two younger tiles may still be on their way (none past the last)
+        if (kt + 3 < nkt) {
+            if (tail) wait_vmcnt<20>();
+            else wait_vmcnt<16>();
+        } else if (kt + 3 == nkt) {
+            if (tail) wait_vmcnt<10>();
+            else wait_vmcnt<8>();
+        } else {
+            wait_vmcnt<0>();
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // chunk 1's fragments have left the stage
+        __syncthreads();
+        if (kt + FS_NS < nkt) issue(kt + FS_NS, st);
+        read_frags(0, nx, 0);
+        mfma_chunk(1);
+#pragma unroll
+        for (int g = 0; g < NR + NC; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        st = nx;
+    }
+    wait_vmcnt<0>();
+}
+
+__global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
+    __shared__ __attribute__((aligned(1024))) unsigned char lds[FS_NS * FS_STAGE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    const int c = lane & 15, q = lane >> 4;
+    const int head = blockIdx.x % a.H, group = blockIdx.x / a.H;
+    const int rows_per = a.OB * a.S;
+    const int m0 = group * rows_per;
+    const int n_valid = min(rows_per, a.M - m0);  // rows of this tile that exist (whole observations)
+    const long HD = (long)a.H * FS_D;
+
+    // ---- loader: thread tid fills slot tid of each 256-slot slab (32 rows x 8 pieces); slabs 0..3
+    // are whole, slab 4 holds rows 128..143 and is filled by wavefronts 0 and 1 alone
+    const int lrow = tid >> 3;
+    const int koff = ((tid & 7) ^ ((lrow >> 1) & 7)) * 8;  // logical piece that belongs in this slot, in elements
+    const unsigned char* ap[5];
+    const unsigned char* wp[5];
+#pragma unroll
+    for (int v = 0; v < 5; ++v) {
+        const int r = min(v * 32 + lrow, FS_ROWS - 1);
+        ap[v] = (const unsigned char*)(a.x + (long)min(m0 + r, a.M - 1) * a.K);
+        const int seg = r / FS_D, d = r - seg * FS_D;
+        wp[v] = (const unsigned char*)(a.W + ((long)seg * HD + (long)head * FS_D + d) * a.K);
+    }
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds + wave * 1024;
+    const bool tail = wave < 2;  // uniform
+
+    // this lane's output columns: bias and column sums, requested ahead of the ring (they are the
+    // oldest loads, so the first wait on the ring covers them)
+    float cs[5], bs[5];
+#pragma unroll
+    for (int j = 0; j < 5; ++j) {
+        const int col = min((wn + 2 * j) * 16 + c, FS_COLS - 1);
+        const int seg = col / FS_D, d = col - seg * FS_D;
+        const long n = (long)seg * HD + (long)head * FS_D + d;
+        cs[j] = a.colsum[n];
+        bs[j] = a.bias ? a.bias[n] : 0.f;
+    }
+
+    f32x4_t acc[5][5];
+#pragma unroll
+    for (int i = 0; i < 5; ++i)
+#pragma unroll
+        for (int j = 0; j < 5; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float ssq[5] = {0.f, 0.f, 0.f, 0.f, 0.f}, ssum[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+    const int nr = wm == 0 ? 5 : 4, nc = wn == 0 ? 5 : 4;
+    if (wm == 0) {
+        if (wn == 0) self_k_walk<5, 5>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+        else self_k_walk<5, 4>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+    } else {
+        if (wn == 0) self_k_walk<4, 5>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+        else self_k_walk<4, 4>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+    }
+    __syncthreads();
+
+    // ---- the tile leaves the accumulators: row statistics first
+    bf16_t* qk = reinterpret_cast<bf16_t*>(lds);                                        // [FS_ROWS][FS_QS]: q | k
+    bf16_t* vt = qk + FS_ROWS * FS_QS;                                                  // [OB][FS_D][FS_VS]: V^T per observation
+    float* stat = reinterpret_cast<float*>(lds + (FS_ROWS * FS_QS + FS_MAX_OB * FS_D * FS_VS) * 2);  // [FS_ROWS][2]: (sum of squares, sum)
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+        float s2 = ssq[i], s1 = ssum[i];
+        s2 += __shfl_xor(s2, 16, 64);
+        s1 += __shfl_xor(s1, 16, 64);
+        s2 += __shfl_xor(s2, 32, 64);
+        s1 += __shfl_xor(s1, 32, 64);
+        const int rb = wm + 2 * i;
+        if (q == 0 && i < nr && wn == 0) {
+            stat[(rb * 16 + c) * 2] = s2;
+            stat[(rb * 16 + c) * 2 + 1] = s1;
+        }
+    }
+    // keys past S of every V^T row are multiplied by probabilities that are zero: they must be finite
+    const int S = a.S;
+    for (int idx = tid; idx < a.OB * FS_D * (FS_VS / 4); idx += 256) {
+        const int row = idx / (FS_VS / 4), k4 = idx - row * (FS_VS / 4);
+        if (4 * k4 + 3 >= S) *reinterpret_cast<u32x2_t*>(vt + row * FS_VS + 4 * k4) = u32x2_t{0u, 0u};
+    }
+    __syncthreads();
+    const float inv_k = 1.0f / (float)a.K;
+    const int inv_s = (65536 + S - 1) / S;
+#pragma unroll
+    for (int i = 0; i < 5; ++i) {
+        const int rb = wm + 2 * i;
+        if (i >= nr) continue;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = rb * 16 + 4 * q + e;
+            const float s2 = stat[row * 2], s1 = stat[row * 2 + 1];
+            const float mean = s1 * inv_k;
+            const float rstd = rsqrtf(fmaxf(s2 * inv_k - mean * mean, 0.f) + a.eps);
+            const float ms = mean * rstd;
+            const int u = (row * inv_s) >> 16, key = row - u * S;  // row / S, exact for S <= 32 and row < 160
+#pragma unroll
+            for (int j = 0; j < 5; ++j) {
+                const int cb = wn + 2 * j;
+                if (j >= nc) continue;
+                const bf16_t v = f2bf(acc[i][j][e] * rstd - ms * cs[j] + bs[j]);
+                const int col = cb * 16 + c;
+                if (cb < 6) qk[row * FS_QS + col] = v;                                       // q: 0..47, k: 48..95
+                else if (row < n_valid) vt[(u * FS_D + col - 2 * FS_D) * FS_VS + key] = v;   // V^T[u][d][key]
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- attention: wavefront w takes observations w, w + 4, ... of the tile
+    typedef short bf16x4_t __attribute__((ext_vector_type(4)));
+    const float sl2 = a.scale * 1.4426950408889634f;
+    // Two observations at a time (u and u + 4), their instructions side by side: one pair's chain
+    // of fragment reads, MFMAs, lane exchanges and exponentials is mostly waiting.
+    for (int u0 = wave; u0 * S < n_valid; u0 += 8) {
+        const bool two = (u0 + 4) * S < n_valid;  // uniform
+        int r0[2];
+        r0[0] = u0 * S;
+        r0[1] = two ? (u0 + 4) * S : r0[0];
+        const int uu[2] = {u0, two ? u0 + 4 : u0};
+        // S^T = K Q^T: sT[kb][qb][e] = score of key 16 kb + 4 q + e against query 16 qb + c
+        f32x4_t sT[2][2][2];
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb) sT[p][kb][qb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < FS_D / 16; ++ks) {
+            bf16x4_t kf[2][2], qf[2][2];
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+#pragma unroll
+                for (int b2 = 0; b2 < 2; ++b2) {
+                    const int row = r0[p] + min(16 * b2 + c, S - 1);  // rows past S repeat the last token; masked below
+                    kf[p][b2] = *reinterpret_cast<const bf16x4_t*>(qk + row * FS_QS + FS_D + 16 * ks + 4 * q);
+                    qf[p][b2] = *reinterpret_cast<const bf16x4_t*>(qk + row * FS_QS + 16 * ks + 4 * q);
+                }
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int qb = 0; qb < 2; ++qb)
+                        sT[p][kb][qb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[p][kb], qf[p][qb], sT[p][kb][qb], 0, 0, 0);
+        }
+        // softmax over the keys of query 16 qb + c: this lane's 8 values and the lanes q = 0..3 of column c
+        bf16x4_t pf[2][2][2];  // P as an operand: [pair][key block][query block], keys 4 q .. 4 q + 3
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                float mx = -INFINITY;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (16 * kb + 4 * q + e >= S) sT[p][kb][qb][e] = -INFINITY;
+                        mx = fmaxf(mx, sT[p][kb][qb][e]);
+                    }
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                float sum = 0.f;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float pr = exp2f((sT[p][kb][qb][e] - mx) * sl2);
+                        sT[p][kb][qb][e] = pr;
+                        sum += pr;
+                    }
+                sum += __shfl_xor(sum, 16, 64);
+                sum += __shfl_xor(sum, 32, 64);
+                const float inv = 1.0f / sum;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    const uint32_t lo = pack_bf2(sT[p][kb][qb][0] * inv, sT[p][kb][qb][1] * inv),
+                                   hi = pack_bf2(sT[p][kb][qb][2] * inv, sT[p][kb][qb][3] * inv);
+                    pf[p][kb][qb] = __builtin_bit_cast(bf16x4_t, u32x2_t{lo, hi});
+                }
+            }
+        // O^T = V^T P^T: o[e] = column 16 db + 4 q + e of query 16 qb + c, four consecutive columns per lane
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+            if (p == 1 && !two) break;
+#pragma unroll
+            for (int db = 0; db < FS_D / 16; ++db) {
+                bf16x4_t vf[2];
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+                    vf[kb] = *reinterpret_cast<const bf16x4_t*>(vt + (uu[p] * FS_D + 16 * db + c) * FS_VS + 16 * kb + 4 * q);
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb) {
+                    f32x4_t o = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb) o = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[kb], pf[p][kb][qb], o, 0, 0, 0);
+                    const int qi = 16 * qb + c;
+                    if (qi < S)
+                        *reinterpret_cast<u32x2_t*>(a.out + (long)(m0 + r0[p] + qi) * HD + (long)head * FS_D + 16 * db + 4 * q) =
+                            u32x2_t{pack_bf2(o[0], o[1]), pack_bf2(o[2], o[3])};
+                }
+            }
+        }
+    }
+}
+
+}  // namespace
+}  // namespace vk
+
+extern "C" VLA_KAPI int vla_layernorm_qkv_self_attention(const void* x, const void* W_folded, const float* colsum, const float* bias,
+                                                int dtype, int M, int K, int S, int n_heads, int head_dim, float scale,
+                                                float ln_eps, void* out, vla_stream_t stream) {
+    using namespace vk;
+    if (!x || !W_folded || !colsum || !out || M < 0 || K <= 0 || S <= 0 || n_heads <= 0) return VLA_K_ERR_ARG;
+    if (dtype != VLA_DT_BF16 || head_dim != FS_D || S > FS_MAX_S || M % S || K % 64 || K < 64 * FS_NS || n_heads % 8) return VLA_K_ERR_SHAPE;
+    if (((uintptr_t)x | (uintptr_t)W_folded | (uintptr_t)out) & 15) return VLA_K_ERR_SHAPE;
+    if (M == 0) return VLA_K_OK;
+    SelfArgs a;
+    a.x = (const bf16_t*)x; a.W = (const bf16_t*)W_folded; a.colsum = colsum; a.bias = bias; a.out = (bf16_t*)out;
+    a.M = M; a.K = K; a.S = S; a.H = n_heads; a.OB = FS_ROWS / S < FS_MAX_OB ? FS_ROWS / S : FS_MAX_OB; a.scale = scale; a.eps = ln_eps;
+    const int n_obs = M / S, groups = (n_obs + a.OB - 1) / a.OB;
+    dit_self_block_kernel<<<(unsigned)(groups * n_heads), 256, 0, (hipStream_t)stream>>>(a);
+    return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+}

@@ -244,7 +244,7 @@ void BitvlaLm::prefill(const Inputs* in, int batch) {
         if (lang_rows_) {
             fetched.resize((size_t)n_lang_ * H_);
             const std::vector<int32_t> ids(in[b].lang_tokens, in[b].lang_tokens + n_lang_);
-            if (n_lang_ > 0 && !lang_rows_->fetch(ids, fetched.data())) throw std::runtime_error("vla: cannot read token embedding rows");
+            if (n_lang_ > 0 && !lang_rows_->fetch_locked(ids, fetched.data())) throw std::runtime_error("vla: cannot read token embedding rows");
         }
         for (int i = 0; i < n_lang_; ++i) {
             const float* e = lang_rows_ ? fetched.data() + (size_t)i * H_ : E_lang_.data() + (size_t)in[b].lang_tokens[i] * H_;

@@ -21,6 +21,7 @@
 #include <memory>
 #include <sstream>
 #include <stdexcept>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -32,8 +33,17 @@ namespace vla {
 struct RowSource {
     int64_t rows = 0, cols = 0;
     virtual ~RowSource() = default;
-    // dst receives ids.size() x cols floats; false on an id outside [0, rows) or a read error
+    // dst receives ids.size() x cols floats; false on an id outside [0, rows) or a read error.
+    // Callers on several threads (a batch's observations are staged in parallel) go through
+    // fetch_locked: an implementation reads through one file handle.
     virtual bool fetch(const std::vector<int32_t>& ids, float* dst) = 0;
+    bool fetch_locked(const std::vector<int32_t>& ids, float* dst) {
+        std::lock_guard<std::mutex> hold(mu_);
+        return fetch(ids, dst);
+    }
+
+  private:
+    std::mutex mu_;
 };
 
 inline size_t ckpt_dtype_size(const std::string& dt) {

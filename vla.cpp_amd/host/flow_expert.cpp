@@ -148,6 +148,7 @@ class FlowExpert : public ModelArch {
     DevBuf vlln_sc_, vlln_sh_;  // vlln as (weight - 1, bias) fp32 [Wv]: the modulated-norm launch computes xn (1 + sc) + sh
     float vlln_eps_ = 1e-5f;
     bool fuse_final_norm_ = true;  // the final norm runs inside the Euler launch
+    bool fuse_self_block_ = true;  // GR00T self blocks: norm, projections and attention in one launch (VLA_NO_FUSED_SELF_BLOCK=1: off)
     bool adarms_ = false;  // pi0.5: ada_ holds [steps][2L+1][scale, shift, gate][W]
     DevBuf bias_step_;   // [steps][W] fp32: b_in (+ time embedding of the step)
     DevBuf ada_;         // GR00T: [steps][L+1][2][W] fp32 (scale, shift); slot L is the final norm (zeros)
@@ -291,6 +292,7 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
 
     const bool no_norm_fusion = std::getenv("VLA_NO_NORM_FUSION") != nullptr;  // read once, at load
     fuse_final_norm_ = !no_norm_fusion;
+    fuse_self_block_ = !no_norm_fusion && std::getenv("VLA_NO_FUSED_SELF_BLOCK") == nullptr;
     layers_.resize(L_);
     for (int l = 0; l < L_; ++l) {
         LayerW& w = layers_[l];
@@ -639,7 +641,7 @@ void FlowExpert::prefill(const Inputs* in, int batch) {
                 std::vector<int32_t> ids((size_t)rows, 0);
                 for (int i = 0; i < n_lang; ++i) ids[i] = in[b].lang_tokens[i];
                 fetched.resize((size_t)rows * Wv_);
-                if (rows > 0 && !lang_rows_->fetch(ids, fetched.data())) throw std::runtime_error("vla: cannot read token embedding rows");
+                if (rows > 0 && !lang_rows_->fetch_locked(ids, fetched.data())) throw std::runtime_error("vla: cannot read token embedding rows");
             }
             for (int i = 0; i < rows; ++i) {
                 const int tok = i < n_lang ? in[b].lang_tokens[i] : 0;  // zero-padded ids, smolvla.cpp:1628-1629
@@ -839,6 +841,30 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                 if (!done && w.Wqkv_ln) {
                     Tensor Wf = tensor_2d(w.Wqkv_ln.get(), dt_, W_, n_rows_w);
                     done = rmsnorm_qkv_rope_append(C, h, Wf, bq, eps_, S_, Hq_, w.is_self, w.is_self, tab, Q.data, w.kv, tok);
+                }
+                // a GR00T self block without prefix rows, mask or rotation: norm, projections and attention in one launch
+                // (from batch 32 on: a workgroup of that launch takes eight observations and one head, and below
+                // that too few of them exist to occupy the chip)
+                if (!done && w.Wqkv_ada && w.is_self && fuse_self_block_ && B >= 32 && w.kv.n_prefix == 0 && !tab &&
+                    suffix_mask_ == VLA_MASK_NONE && pad_start_ >= pad_end_ && Hq_ == Hkv_) {
+                    Tensor Wf = tensor_2d(w.Wqkv_ada.as<uint16_t>() + (size_t)s * n_rows_w * W_, dt_, W_, n_rows_w);
+                    if (layernorm_qkv_self_attention(C, h, Wf, w.cs_ada.as<float>() + (size_t)s * n_rows_w,
+                                                     w.b_ada.as<float>() + (size_t)s * n_rows_w, eps_, S_, Hq_, D_, scale, att)) {
+                        prof_mark("norm_qkv_attention_self");
+                        Tensor Wo = tensor_2d(w.Wo.get(), dt_, (int64_t)Hq_ * D_, W_);
+                        linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
+                        prof_mark("wo_residual");
+                        if (I_ > 0) {
+                            Tensor mid = tensor_2d(mid_.get(), dt_, I_, M);
+                            const float* z = ada_.as<float>() + ((size_t)s * (L_ + 2) + L_) * 2 * W_;  // zeros: plain LayerNorm
+                            adaln(C, h, z, z + W_, eps_, hn);
+                            prof_mark("ffn_norm");
+                            Tensor W1 = tensor_2d(w.W1.get(), dt_, W_, I_), W2 = tensor_2d(w.W2.get(), dt_, I_, W_);
+                            ffn_gelu(C, W1, w.b1.as<float>(), W2, w.b2.as<float>(), hn, h.data, mid, h);
+                            prof_mark("ffn_in_out");
+                        }
+                        continue;
+                    }
                 }
                 if (!done && w.Wqkv_ada) {
                     Tensor Wf = tensor_2d(w.Wqkv_ada.as<uint16_t>() + (size_t)s * n_rows_w * W_, dt_, W_, n_rows_w);

@@ -191,6 +191,18 @@ inline bool layernorm_qkv_rope_append(Ctx& C, const Tensor& x, const Tensor& W_f
     return true;
 }
 
+// A DiT self block's adaLN, Q / K / V projections and the attention of each observation's S
+// tokens over themselves as one launch (dit_head.cpp:111-125 with enc = nullptr); the block's K
+// and V stay on the chip.  Returns false when the shapes do not fit the fused kernel.
+inline bool layernorm_qkv_self_attention(Ctx& C, const Tensor& x, const Tensor& W_folded, const float* colsum, const float* bias,
+                                         float eps, int S, int n_heads, int head_dim, float scale, Tensor& out) {
+    const int rc = vla_layernorm_qkv_self_attention(x.data, W_folded.data, colsum, bias, x.dtype, (int)x.rows(), (int)x.ne[0], S,
+                                                    n_heads, head_dim, scale, eps, out.data, C.stream);
+    if (rc == VLA_K_ERR_SHAPE) return false;
+    VLA_K(rc);
+    return true;
+}
+
 // attn.h:48-58 (flash_attention) over the resident cache: Q [D, Hq, S, B]
 // token-major, keys [0, n_keys).
 inline void flash_attention(Ctx& C, const Tensor& Q, const KVLayer& kv, int n_keys, const MaskSpec& mask, float scale,
