@@ -260,10 +260,16 @@ VLA_KAPI int vla_attn_prefix_suffix(const void* q, const void* k_cache, const vo
  *     VLA_K_ERR_WORKSPACE (nothing is written out of bounds either way).
  *   workspace: device memory of at least that many bytes, 16-byte aligned, zero-filled once
  *     before its first use (every launch leaves the part that must stay zero at zero);
- *     NULL is accepted when the shape needs none.  VLA_K_ERR_WORKSPACE if it is too small. */
+ *     NULL is accepted when the shape needs none.  VLA_K_ERR_WORKSPACE if it is too small.
+ *   vla_attn_workspace_reset: the part that must be zero, zeroed again (one small fill
+ *     kernel; capturable).  A launch that ran to its end leaves it at zero by itself, one
+ *     that was cut short (device fault, reset) does not and would poison every later launch on
+ *     the workspace: run it at the start of each launch sequence (a model handle does, once
+ *     per action chunk). */
 #define VLA_ATTN_WORKSPACE_UNSUPPORTED ((size_t)-1)
 VLA_KAPI size_t vla_attn_workspace_bytes(int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
                                          int n_keys);
+VLA_KAPI int vla_attn_workspace_reset(void* workspace, size_t workspace_bytes, vla_stream_t stream);
 VLA_KAPI int vla_attn_prefix_suffix_ws(const void* q, const void* k_cache, const void* vt_cache, void* out,
                                        int dtype, int batch, int S, int n_q_heads, int n_kv_heads, int head_dim,
                                        int t_max, int n_keys, float scale, int mask_kind, int n_prefix,

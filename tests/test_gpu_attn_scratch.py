@@ -82,6 +82,34 @@ def test_caller_owned_workspace_gives_the_library_owned_bits(case):
     assert rc == pkg.VLA_K_ERR_WORKSPACE and not np.any(got)
 
 
+def test_workspace_reset_restores_counters_left_behind_by_a_launch_that_did_not_finish():
+    """The slices of the decode shape count themselves in and the last one merges; the counters are
+    left at zero by a launch that ran to its end.  Counters as a launch cut short would leave them
+    (written here by the host, no kernel is interrupted) are put back by vla_attn_workspace_reset,
+    and the next launch gives the usual bits."""
+    case = SLICED[0]
+    name, B, S, Hq, Hkv, D, T, dt, mk = case
+    need = pkg.lib().vla_attn_workspace_bytes(dt, B, S, Hq, Hkv, D, T)
+    q, kc, vc, t_max = setup_case(case)
+    rc, want = run("vla_attn_prefix_suffix", case, q, kc, vc, t_max)
+    assert rc == pkg.VLA_K_OK
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    rc, got = run("vla_attn_prefix_suffix_ws", case, q, kc, vc, t_max, (ws.data_ptr(), need))
+    assert rc == pkg.VLA_K_OK and np.array_equal(got, want)
+    ws.view(torch.int32)[:4096] = 3  # units that had counted three slices in when their launch ended
+    torch.cuda.synchronize()
+    lib = pkg.lib()
+    assert lib.vla_attn_workspace_reset(ws.data_ptr(), need, pkg.stream()) == pkg.VLA_K_OK
+    torch.cuda.synchronize()
+    assert int(ws.view(torch.int32)[:16384].abs().sum()) == 0
+    rc, got = run("vla_attn_prefix_suffix_ws", case, q, kc, vc, t_max, (ws.data_ptr(), need))
+    assert rc == pkg.VLA_K_OK and np.array_equal(got, want)
+    # nothing to do for a shape without a workspace; a block too small to hold the counters is refused
+    assert lib.vla_attn_workspace_reset(None, 0, pkg.stream()) == pkg.VLA_K_OK
+    assert lib.vla_attn_workspace_reset(ws.data_ptr(), 1024, pkg.stream()) == pkg.VLA_K_ERR_WORKSPACE
+    assert lib.vla_attn_workspace_reset(ws.data_ptr() + 4, need - 4, pkg.stream()) == pkg.VLA_K_ERR_WORKSPACE
+
+
 def test_shapes_without_key_slices_need_no_workspace():
     # batch 32 SmolVLA: enough workgroups without slicing; NULL workspace is accepted
     case = ("smolvla-b32", 32, 50, 15, 5, 64, 291, BF16, pkg.VLA_MASK_NONE)

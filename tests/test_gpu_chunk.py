@@ -147,6 +147,26 @@ def test_config3_gr00t_dit_bf16(tmp_path, n_layers, batch):
     m.close()
 
 
+@pytest.mark.parametrize("fold_mb,batch", [("0", 2), (None, 33)])
+def test_gr00t_blocks_with_and_without_the_folded_modulation(tmp_path, monkeypatch, fold_mb, batch):
+    # The per-step folded adaLN operands are a memory-for-launches trade with a budget
+    # (VLA_ADALN_FOLD_MB): over it the blocks run adaln + projection as two launches.  Batch 33
+    # takes the self blocks' one-launch front half (eight observations per workgroup, the last
+    # group with one).  Both against the oracle.
+    if fold_mb is not None:
+        monkeypatch.setenv("VLA_ADALN_FOLD_MB", fold_mb)
+    cfg = ckpt.gr00t_config(n_layers=4)
+    w = ckpt.synth_weights(cfg, seed=0x5EED + 77)
+    r = np.random.default_rng(377)
+    obs = [make_obs(cfg, r, n_views=1) for _ in range(batch)]
+    m = load(tmp_path, cfg, w, "gr00t_fold")
+    got = m.predict_batch(obs).reshape(batch, 16, 32)
+    for b in (0, batch - 1):
+        want = orc_chunk.flow_expert_chunk(cfg, w, obs[b], emulate_bf16=True)
+        assert bf16_close(got[b], want), np.abs(got[b] - want).max()
+    m.close()
+
+
 @pytest.mark.parametrize("dtype,n_layers,batch", [("f32", 2, 1), ("bf16", 4, 2), ("bf16", 16, 1)])
 def test_gr00t_with_the_dit_heads_own_input_and_output_mlps(tmp_path, dtype, n_layers, batch):
     # The real GR00T N1.5 head (src/models/gr00tn1d5.cpp:366-381): state token from encode_state,

@@ -50,6 +50,7 @@ KERNEL_API = {
     "vla_attn_prefix_suffix_ws": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _vp, _vp,
                                   ctypes.c_size_t, _vp],
     "vla_attn_workspace_bytes": [_i, _i, _i, _i, _i, _i, _i],
+    "vla_attn_workspace_reset": [_vp, ctypes.c_size_t, _vp],
     "vla_embed_suffix": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "vla_embed_suffix_act": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "vla_finish_suffix_rows": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],

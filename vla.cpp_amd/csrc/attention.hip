@@ -828,7 +828,11 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
 // relaxed atomic accesses (write-through stores, loads served from memory) and the count is
 // taken only after the wavefront's stores have been acknowledged, so neither side needs a
 // cache-wide write-back or invalidate.  The arithmetic order is fixed by the slice index, not
-// by who arrives last.  At most ARRIVE_MAX_T (row, slice) pairs per block, 128-wide heads.
+// by who arrives last.  The counters are left at zero by the merging slice, for the next launch:
+// a launch that is cut short (a fault elsewhere on the device, a reset) leaves the counters of
+// its unfinished units non-zero and so poisons the block for every launch after it, which is
+// why the owner of a workspace zeroes them at the start of each launch sequence
+// (vla_attn_workspace_reset) instead of relying on the last launch alone.  At most ARRIVE_MAX_T (row, slice) pairs per block, 128-wide heads.
 constexpr int ARRIVE_MAX_T = 48, ARRIVE_MAX_UNITS = 16384;
 __device__ __forceinline__ void st_dev64(float* p, float x, float y) {
     const unsigned long long v = (unsigned long long)__float_as_uint(x) | ((unsigned long long)__float_as_uint(y) << 32);
@@ -1944,6 +1948,23 @@ extern "C" int vla_attn_prefix_suffix_noalloc(const void* q, const void* k_cache
     sc.bytes = VLA_ATTN_NOALLOC_SCRATCH_BYTES;
     return attn_entry(q, k_cache, vt_cache, out, dtype, batch, S, n_q_heads, n_kv_heads, head_dim, t_max, n_keys, scale,
                       mask_kind, n_prefix, pad_start, pad_end, mask, stream, sc);
+}
+
+// The arrival counters of a workspace back at zero, as a fill kernel (no memset node under
+// graph capture).  A launch that ran to its end leaves them at zero by itself; one that did not
+// (a device fault, a reset in the middle of a sequence) leaves the counters of its unfinished
+// units at whatever they had reached, and every later launch on that workspace would then take
+// the wrong slice for the last one.  Callers that own a workspace run this at the start of
+// each launch sequence.
+__global__ void __launch_bounds__(256) zero_words_kernel(int* p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+extern "C" int vla_attn_workspace_reset(void* workspace, size_t workspace_bytes, vla_stream_t stream) {
+    if (!workspace || workspace_bytes == 0) return VLA_K_OK;  // a shape that needs none
+    if (((uintptr_t)workspace & 15) || workspace_bytes < ARRIVE_BYTES) return VLA_K_ERR_WORKSPACE;
+    zero_words_kernel<<<(ARRIVE_MAX_UNITS + 255) / 256, 256, 0, (hipStream_t)stream>>>((int*)workspace, ARRIVE_MAX_UNITS);
+    return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
 }
 
 extern "C" int vla_kernels_init(void) {

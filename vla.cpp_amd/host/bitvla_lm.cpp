@@ -372,6 +372,7 @@ void BitvlaLm::run_steps(int n_steps, void* stream) {
     prof_start("step", C.stream);
     for (int it = 0; it < n_steps; ++it) {
         const int t = it % n_act_;
+        if (t == 0) attn_ws_.begin(C.stream);
         // Where the few-row launches apply (`direct`, a matter of shapes only), the first layer reads
         // token t's embedding rows where they lie and the last layer leaves its rows in hfin_: no
         // copy in front, and one final norm over all tokens' rows in front of the action head.

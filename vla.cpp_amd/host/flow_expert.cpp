@@ -497,7 +497,17 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
         }
         ada_.upload(ada.data(), ada.size() * sizeof(float));
 
-        if (dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !no_norm_fusion) {
+        // The folded operands cost a copy of every Q / QKV weight per denoise step (GR00T N1.5 at 4 steps:
+        // 16 layers x (3 W^2 self, W^2 cross) x 2 bytes = 0.6 GB) and the step count comes from the file:
+        // above the budget (VLA_ADALN_FOLD_MB, default 2048) the blocks keep adaln + projection as two launches.
+        size_t fold_bytes = 0;
+        for (int l = 0; l < L_; ++l) fold_bytes += (size_t)steps_ * (size_t)(layers_[l].is_self ? qd + 2 * kvd : qd) * W_ * sizeof(uint16_t);
+        const char* fold_mb = std::getenv("VLA_ADALN_FOLD_MB");
+        const size_t fold_budget = (size_t)(fold_mb ? std::max(0L, std::atol(fold_mb)) : 2048L) << 20;
+        if (fold_bytes > fold_budget)
+            std::fprintf(stderr, "vla(gr00t): %d steps of folded adaLN operands would take %zu MB (budget %zu MB); using adaln + projection launches\n",
+                         steps_, fold_bytes >> 20, fold_budget >> 20);
+        if (dt_ == VLA_DT_BF16 && W_ % 16 == 0 && !no_norm_fusion && fold_bytes <= fold_budget) {
             // the modulation of a block depends on the step only: fold it into one operand set
             // per step, and the pre-norm launch of the block disappears into its projection
             const int nthr = std::min(default_cpu_threads(), L_);
@@ -797,6 +807,7 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
     for (int it = 0; it < n_steps; ++it) {
         const int s = it % steps_;
         if (s == 0) {
+            attn_ws_.begin(C.stream);
             VLA_HIP(hipMemcpyAsync(xt_.get(), x0_.get(), xbytes, hipMemcpyDeviceToDevice, C.stream));
             prof_mark("stage_noise");
         }

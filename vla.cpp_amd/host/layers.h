@@ -90,6 +90,11 @@ struct AttnWorkspace {
         buf.alloc(need);
         buf.zero();
     }
+    // The part launches count in, back at zero: once per launch sequence, so that a sequence cut
+    // short by a device fault cannot poison the next one.
+    void begin(hipStream_t stream) {
+        if (buf.bytes()) VLA_K(vla_attn_workspace_reset(buf.get(), buf.bytes(), stream));
+    }
 };
 
 // Mask as the attention kernel generates it (masks are data in the reference:
