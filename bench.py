@@ -18,16 +18,19 @@ its predecessors left them and includes the gap to the launch before it.  The ev
 own cost (the marked chunk minus a replayed one, per mark) is subtracted.
 
 Prints ONE JSON line (a few KB) with the contract fields plus
-  roofline      the step's dominant kernel (largest share of the step's time)
-  roofline_kv   the attention launch that reads the most prefix KV
+  roofline      the kernel the path's HBM target is set on: the attention launch that reads the
+                most prefix K/V at this workload (algorithmic K/V bytes / its duration in the step)
+  roofline_dominant  the launch site with the largest share of the step's time, when that is
+                another kernel (share_of_step says how much), on its own roofline
   roofline_ternary_prefill  the BitVLA prefill QKV GEMM (int8 MFMA roofline)
   cpu_baseline  the CPU oracle (restated reference op sequence, with the reference's
                 per-step concat copies, fp32 SIMD-style accumulation) timed on this host
                 with the reference's thread rule and timing recipe
   us_per_action_chunk_with_prefix  one chunk plus the once-per-observation prefix K/V build
   config.workloads  one compact entry per BASELINE configuration and batch size: us per
-                step, chunk p50, chunk with the prefix build, launches per step, and the
-                dominant launch's roofline {kernel, frac, avg_us, traffic}
+                step, chunk p50, chunk with the prefix build, launches per step, the roofline
+                of the launch with the largest share {kernel, frac, avg_us, traffic} and, when
+                that is not it, of the largest prefix-K/V read (roofline_kv)
 --verbose adds the per-launch-site tables (kernels, prefill_kernels, other_configs).
 """
 import argparse
@@ -403,6 +406,8 @@ def algorithmic_work(cfg, B, P):
     for k in ("step.pre_norm", "step.final_norm", "step.ffn_norm"):
         w[k] = ("hbm", 2 * M * W * es, "hbm")
     w["step.qkv_rope_append_self"] = ("mfma", 2.0 * M * (qd + 2 * kvd) * W, mf)
+    # a DiT self block's norm, projections and attention over its own S tokens in one launch
+    w["step.norm_qkv_attention_self"] = ("mfma", 2.0 * M * (qd + 2 * kvd) * W + 4.0 * B * Hq * S * S * D, mf)
     w["step.q_rope_cross"] = ("mfma", 2.0 * M * qd * W, mf)
     w["step.attention_self"] = ("hbm", 2 * (P_self + S) * kvd * es * B, "hbm")
     w["step.attention_cross"] = ("hbm", 2 * P * kvd * es * B, "hbm")
@@ -567,7 +572,7 @@ def run_workload(name, spec, steps, warmup, with_cpu, tmpdir, isolated=False):
             rf = roofline_entry(label, v["us"], work[label], name)
             k.update(bound=rf["bound"], frac=rf["frac"])
             if v["us"] * per_step > best_t:
-                best, best_t = rf, v["us"] * per_step
+                best, best_t = dict(rf, share_of_step=round(v["us"] * per_step / (ms_per_step * 1e3), 3)), v["us"] * per_step
             if label.startswith("step.attention") and (best_kv is None or work[label][1] > best_kv["algorithmic_work_per_launch"]):
                 best_kv = rf
         kernels[label] = k
@@ -695,12 +700,15 @@ def main():
         "us_per_action_chunk": main_res["us_per_action_chunk"], "action_chunk_us": main_res["action_chunk_us"],
         "us_per_action_chunk_with_prefix": main_res["us_per_action_chunk_with_prefix"],
         "prefix_kv_build_ms": main_res["prefix_kv_build_ms"],
-        "roofline": main_res["roofline"], "roofline_kv": main_res["roofline_kv"],
+        # the largest prefix-K/V read (the HBM target's kernel); the launch site with the largest share of the step beside it
+        "roofline": main_res["roofline_kv"] or main_res["roofline"],
         "cpu_baseline": main_res.get("cpu_baseline"),
         "device_us_per_step": main_res["device_us_per_step"], "host_us_per_step": main_res["host_us_per_step"],
         "sum_launch_us_per_step": main_res["sum_launch_us_per_step"], "launches_per_step": main_res["launches_per_step"],
         "event_overhead_us_per_launch": main_res["event_overhead_us_per_launch"],
     }
+    if main_res["roofline_kv"] and main_res["roofline"] and main_res["roofline"]["kernel"] != main_res["roofline_kv"]["kernel"]:
+        line["roofline_dominant"] = {k: main_res["roofline"].get(k) for k in ("kernel", "bound", "achieved", "peak", "unit", "frac", "traffic", "avg_us", "share_of_step")}
     for r in every:  # the ternary prefill GEMM's roofline, whichever workload ran it (the largest batch wins)
         if "roofline_ternary_prefill" in r:
             line["roofline_ternary_prefill"] = dict(r["roofline_ternary_prefill"], workload=r["workload"])
