@@ -63,10 +63,10 @@ struct AttnArgs {
     int n_groups, n_split, tiles_per_split, r_pad, p2;
     int n_rblocks;  // direct kernel: 32-row blocks per (batch, kv head)
     int n_slices;   // LDS kernel, direct-to-LDS variant: key slices (wavefronts) per row tile
-    float* part_o;   // [pair][split][r_pad][D] fp32 unnormalised, or fp16 normalised (part_half)
-    float* part_ml;  // [pair][split][r_pad][2]
+    float* part_o;   // [pair][split][r_pad][D] fp32 unnormalised, or fp16 normalised (part_half); merged in the launch: [pair][r_pad][split][D]
+    float* part_ml;  // [pair][split][r_pad][2]; merged in the launch: [pair][r_pad][split][2]
     int part_half;   // partial outputs stored as o / l in fp16 (half the bytes; wide heads)
-    int* arrive;     // direct kernel: one counter per (pair, row block); the slice that arrives last merges (zero between launches)
+    int* arrive;     // decode kernel: one counter per pair; the slice that arrives last merges (zero between launches)
 };
 
 // Key (within a 32-key block) held by score row x = 8j + 4h + i: 16(j/2) + 8h + 4(j%2) + i.
@@ -821,10 +821,10 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         }
 }
 
-// Key slices of one (pair, row block) as wavefronts of different workgroups, merged without a
-// second launch: every slice writes its unnormalised partial rows and (max, sum), then counts
-// itself in; the one that finds all others counted combines them and writes the output.  No
-// wavefront waits for another.  The partials cross between the per-XCD L2s as device-scope
+// Key slices of one pair as wavefronts of different workgroups, merged without a second launch
+// (attn_decode16_kernel): every slice writes its unnormalised partial rows and (max, sum), then
+// counts itself in; the one that finds all others counted combines them and writes the output.
+// No wavefront waits for another.  The partials cross between the per-XCD L2s as device-scope
 // relaxed atomic accesses (write-through stores, loads served from memory) and the count is
 // taken only after the wavefront's stores have been acknowledged, so neither side needs a
 // cache-wide write-back or invalidate.  The arithmetic order is fixed by the slice index, not
@@ -832,7 +832,8 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
 // a launch that is cut short (a fault elsewhere on the device, a reset) leaves the counters of
 // its unfinished units non-zero and so poisons the block for every launch after it, which is
 // why the owner of a workspace zeroes them at the start of each launch sequence
-// (vla_attn_workspace_reset) instead of relying on the last launch alone.  At most ARRIVE_MAX_T (row, slice) pairs per block, 128-wide heads.
+// (vla_attn_workspace_reset) instead of relying on the last launch alone.  At most ARRIVE_MAX_T
+// (row, slice) pairs per pair of (batch, kv head), 128-wide heads.
 constexpr int ARRIVE_MAX_T = 48, ARRIVE_MAX_UNITS = 16384;
 __device__ __forceinline__ void st_dev64(float* p, float x, float y) {
     const unsigned long long v = (unsigned long long)__float_as_uint(x) | ((unsigned long long)__float_as_uint(y) << 32);
@@ -841,91 +842,6 @@ __device__ __forceinline__ void st_dev64(float* p, float x, float y) {
 __device__ __forceinline__ unsigned long long ld_dev64(const float* p) {
     return __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void arrive_merge(const AttnArgs& a, const f32x16_t (&o)[4], float m_run, float l_run, int pair, int prb,
-                                             int split, int row, bool row_valid, int b, int hk, int grp, int R, int lane, int g) {
-    constexpr int D = 128;
-    if (row_valid) {
-        const long prow = ((long)pair * a.n_split + split) * a.r_pad + row;
-        if (g == 0) st_dev64(a.part_ml + prow * 2, m_run, l_run);
-        float* po = a.part_o + prow * D;
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int d = db * 32 + 8 * j + 4 * g;
-                st_dev64(po + d, o[db][4 * j], o[db][4 * j + 1]);
-                st_dev64(po + d + 2, o[db][4 * j + 2], o[db][4 * j + 3]);
-            }
-    }
-    // Ordering.  Hardware (gfx950, which this file is compiled for and nothing else -- see the
-    // #error in common.h): the partials above are device-scope atomic stores, i.e. written
-    // through to memory, and vmcnt counts a store only once memory has acknowledged it; the
-    // merger's device-scope atomic loads below are served from memory, not from its XCD's L2.
-    // So once vmcnt is zero the partials are visible to every XCD, and the counter's value
-    // tells the last slice that every other slice got that far.  Compiler: the two
-    // workgroup-scope fences forbid moving the stores below the count and the merger's loads
-    // above it; at workgroup scope they cost no cache maintenance (an agent-scope release
-    // would write back the whole L2: 121 us per launch, measured).
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's partials are in memory before it is counted
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    int old = 0;
-    if (lane == 0) old = __hip_atomic_fetch_add(a.arrive + prb, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    old = __builtin_amdgcn_readfirstlane(old);
-    if (old != a.n_split - 1) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    if (lane == 0) __hip_atomic_store(a.arrive + prb, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
-
-    // Lane t = rl * n_split + sp holds (max, sum) of row rl in slice sp, then its weight
-    // 2^(max - row max) and the reciprocal of the row's combined sum.
-    const int Rb = min(32, R);  // one row block only
-    const int T = Rb * a.n_split;
-    const long prow0 = (long)pair * a.n_split * a.r_pad;
-    float mt = -INFINITY, lt = 0.f;
-    if (lane < T) {
-        const unsigned long long v = ld_dev64(a.part_ml + (prow0 + (long)(lane % a.n_split) * a.r_pad + lane / a.n_split) * 2);
-        mt = __uint_as_float((uint32_t)v);
-        lt = __uint_as_float((uint32_t)(v >> 32));
-    }
-    unsigned long long pv[ARRIVE_MAX_T];
-    {
-        int lsp = 0, lrl = 0;  // slice and row of t, kept by counting (no divisions in the unrolled body)
-#pragma unroll
-        for (int t = 0; t < ARRIVE_MAX_T; ++t) {
-            pv[t] = 0ull;
-            if (t < T) pv[t] = ld_dev64(a.part_o + (prow0 + (long)lsp * a.r_pad + lrl) * D + lane * 2);
-            if (++lsp == a.n_split) {
-                lsp = 0;
-                ++lrl;
-            }
-        }
-    }
-    const int t0 = lane < T ? (lane / a.n_split) * a.n_split : 0;
-    float mrow = -INFINITY;
-    for (int sp = 0; sp < a.n_split; ++sp) mrow = fmaxf(mrow, __shfl(mt, t0 + sp, 64));
-    const float wt = (lane < T && mrow > -INFINITY) ? exp2f(mt - mrow) : 0.f;
-    float lrow = 0.f;
-    for (int sp = 0; sp < a.n_split; ++sp) lrow += __shfl(lt * wt, t0 + sp, 64);
-    const float inv = lrow > 0.f ? 1.0f / lrow : 0.f;
-    float a0 = 0.f, a1 = 0.f;
-    int sp = 0, rl = 0;
-#pragma unroll
-    for (int t = 0; t < ARRIVE_MAX_T; ++t) {
-        if (t < T) {  // uniform
-            const float w = __shfl(wt, t, 64);
-            a0 += __uint_as_float((uint32_t)pv[t]) * w;
-            a1 += __uint_as_float((uint32_t)(pv[t] >> 32)) * w;
-            if (++sp == a.n_split) {
-                const float iv = __shfl(inv, t, 64);
-                const int hh = hk * grp + rl / a.S, ss = rl % a.S;
-                reinterpret_cast<uint32_t*>((bf16_t*)a.out + (((long)b * a.S + ss) * a.Hq + hh) * D)[lane] = pack_bf2(a0 * iv, a1 * iv);
-                a0 = a1 = 0.f;
-                sp = 0;
-                ++rl;
-            }
-        }
-    }
-}
-
 // Few query rows per (batch, kv head) -- at most one 32-row tile: GR00T's 17 DiT tokens,
 // single-token decode.  Nothing is shared between wavefronts then, so K and V^T go straight
 // from the cache into MFMA operand registers (no LDS, no barriers): lane (g, r) of a
@@ -1168,12 +1084,6 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
         }
         return;
     }
-    if constexpr (D == 128) {
-        if (a.arrive) {  // uniform over the launch
-            arrive_merge(a, o, m_run, l_run, pair, prb, split, row, row_valid, b, hk, grp, R, lane, g);
-            return;
-        }
-    }
     if (!row_valid) return;
     if (a.n_split > 1) {
         const long prow = ((long)pair * a.n_split + split) * a.r_pad + row;
@@ -1205,6 +1115,297 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
                                 pack_bf2(o[db][4 * j + 2] * inv, o[db][4 * j + 3] * inv)};
             *reinterpret_cast<u32x2_t*>(orow + d * EB) = pk;
         }
+}
+
+// ---- Decode with 128-wide heads and at most 16 query rows per kv head (single-token decode of
+// a grouped-query model: the group's heads are the rows).  The register-direct kernel above
+// pads such rows to a 32-row MFMA tile; here the products are formed transposed on
+// v_mfma_f32_16x16x32_bf16, a quarter of the matrix work per key block and half the softmax:
+//
+//   S^T = K Q^T  two products per 32-key block; row i of product j stands for key
+//                8 (i / 4) + 4 j + i % 4 of the block, so that lane (c, q) = (lane % 16, lane / 16)
+//                ends up with the scores of keys 8 q .. 8 q + 7 against query c in key order --
+//   O^T += V^T P^T  -- which is P^T as this instruction's right operand (32 keys x 16 queries),
+//                without a lane exchange; lane (c, q) reads 8 consecutive keys of V^T row
+//                16 db + c and holds output columns 16 db + 4 q .. + 3 of query c.
+//
+// A wavefront is one (pair, key slice) and a workgroup of its own; the slices of a pair are
+// merged inside the launch by the one that arrives last, with the partial rows laid out
+// [pair][row][slice] and the merge unrolled for the slice count.
+constexpr int DEC_MAX_NS = 12, DEC_MAX_R = 16;
+
+// A value combined over the four 16-lane rows of the wavefront (lanes c, c + 16, c + 32, c + 48)
+// with gfx950's row swaps instead of two trips through LDS: after v_permlane16_swap of a register
+// with itself one copy holds rows (0, 0, 2, 2) and the other rows (1, 1, 3, 3); v_permlane32_swap does
+// the same for the two halves.
+__device__ __forceinline__ float rows_max(float x) {
+    u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float rows_sum(float x) {
+    u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+template <int NS>
+__device__ __forceinline__ void merge_rows_static(const AttnArgs& a, int pair, int b, int hk, int grp, int R, int lane) {
+    constexpr int D = 128;
+    constexpr int MAXR = ARRIVE_MAX_T / NS < DEC_MAX_R ? ARRIVE_MAX_T / NS : DEC_MAX_R;
+    const long prow0 = (long)pair * a.r_pad * NS;
+    // lane t = row * NS + slice holds that partial's (max, sum)
+    float mt = -INFINITY, lt = 0.f;
+    if (lane < R * NS) {
+        const unsigned long long v = ld_dev64(a.part_ml + (prow0 + lane) * 2);
+        mt = __uint_as_float((uint32_t)v);
+        lt = __uint_as_float((uint32_t)(v >> 32));
+    }
+    unsigned long long pv[MAXR][NS];
+    const float* pb = a.part_o + prow0 * D + lane * 2;
+#pragma unroll
+    for (int rl = 0; rl < MAXR; ++rl) {
+        if (rl < R) {  // uniform
+#pragma unroll
+            for (int sp = 0; sp < NS; ++sp) pv[rl][sp] = ld_dev64(pb + (rl * NS + sp) * D);
+        }
+    }
+    int hh = hk * grp, ss = 0;
+#pragma unroll
+    for (int rl = 0; rl < MAXR; ++rl) {
+        if (rl < R) {  // uniform
+            // the row's slice maxima and sums, read from their lanes into scalar registers: every lane forms the same weights
+            float mj[NS], mrow = -INFINITY;
+#pragma unroll
+            for (int sp = 0; sp < NS; ++sp) {
+                mj[sp] = __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(mt), rl * NS + sp));
+                mrow = fmaxf(mrow, mj[sp]);
+            }
+            float a0 = 0.f, a1 = 0.f, lrow = 0.f;
+#pragma unroll
+            for (int sp = 0; sp < NS; ++sp) {
+                const float w = mrow > -INFINITY ? __builtin_amdgcn_exp2f(mj[sp] - mrow) : 0.f;
+                lrow += __uint_as_float((uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(lt), rl * NS + sp)) * w;
+                a0 += __uint_as_float((uint32_t)pv[rl][sp]) * w;
+                a1 += __uint_as_float((uint32_t)(pv[rl][sp] >> 32)) * w;
+            }
+            const float iv = lrow > 0.f ? 1.0f / lrow : 0.f;
+            reinterpret_cast<uint32_t*>((bf16_t*)a.out + (((long)b * a.S + ss) * a.Hq + hh) * D)[lane] = pack_bf2(a0 * iv, a1 * iv);
+            if (++ss == a.S) {
+                ss = 0;
+                ++hh;
+            }
+        }
+    }
+}
+
+template <bool P2, int ST>
+__global__ void __launch_bounds__(64) attn_decode16_kernel(AttnArgs a) {
+    constexpr int D = 128, EB = 2, NKS = D / 32, NDB = D / 16;
+    const int lane = threadIdx.x, c = lane & 15, q = lane >> 4;
+    const int pair = blockIdx.x / a.n_split, split = blockIdx.x % a.n_split;
+    const int b = pair / a.Hkv, hk = pair % a.Hkv;
+    const int grp = a.Hq / a.Hkv, R = grp * a.S;
+    const bool row_valid = c < R;
+    const int hg = row_valid ? c / a.S : 0, s = row_valid ? c % a.S : 0;
+    const int h = hk * grp + hg;
+    const int nb_total = (a.n_keys + 31) / 32;
+    const int kb0 = __builtin_amdgcn_readfirstlane(split * a.tiles_per_split);
+    const int kb1 = __builtin_amdgcn_readfirstlane(min(nb_total, kb0 + a.tiles_per_split));
+
+    u32x4_t qf[NKS];
+    {
+        const unsigned char* qrow = (const unsigned char*)a.q + (((long)b * a.S + s) * a.Hq + h) * D * EB + q * 16;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            const u32x4_t z = {0u, 0u, 0u, 0u};
+            qf[ks] = row_valid ? *reinterpret_cast<const u32x4_t*>(qrow + ks * 64) : z;
+        }
+    }
+    f32x4_t o[NDB];
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) o[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float c2 = a.scale * LOG2E;
+
+    const unsigned char* kbase = (const unsigned char*)a.k_cache + ((long)b * a.Hkv + hk) * a.t_max * D * EB + q * 16;
+    const unsigned char* vbase = (const unsigned char*)a.vt_cache + (((long)b * a.Hkv + hk) * D + c) * (long)a.t_max * EB;
+    const long vstep = 16l * a.t_max * EB;  // 16 rows of V^T
+    const int krow = 8 * (c >> 2) + (c & 3);  // this lane's key in product 0; product 1 takes the key 4 further
+
+    u32x4_t kr[ST][2][NKS];
+    u32x4_t vr[ST][NDB];  // 8 consecutive keys of V^T row 16 db + c
+    // One block of loads, the same sixteen instructions for every block and no branch around any
+    // of them.  K rows past n_keys repeat the last key (their scores are masked); V^T runs past
+    // n_keys stay inside the cache row and are zeroed by mask_partial before they are multiplied
+    // (stale cache contents may be NaN).  Blocks past the slice repeat its last block.
+    auto load_blk = [&](int st, int kb_any) __attribute__((always_inline)) {
+        const int kb = min(kb_any, kb1 - 1);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int key = min(kb * 32 + krow + 4 * j, a.n_keys - 1);
+            const unsigned char* kp = kbase + (long)key * D * EB;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) kr[st][j][ks] = *reinterpret_cast<const u32x4_t*>(kp + ks * 64);
+        }
+        const int k8 = min(kb * 32 + 8 * q, a.t_max - 8);
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) vr[st][db] = *reinterpret_cast<const u32x4_t*>(vbase + db * vstep + k8 * EB);
+    };
+    auto mask_partial = [&](int st, int kb) __attribute__((always_inline)) {
+        const int nvalid = a.n_keys - (kb * 32 + 8 * q);  // real keys among this lane's 8, may be <= 0
+#pragma unroll
+        for (int db = 0; db < NDB; ++db)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) vr[st][db][e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+    };
+    int hi = a.n_keys;
+    if (a.mask_kind == VLA_MASK_CAUSAL_SUFFIX) hi = min(a.n_keys, a.n_prefix + s + 1);
+    else if (a.mask_kind == VLA_MASK_PI0_STATE && s == 0) hi = min(a.n_keys, a.n_prefix + 1);
+    const int pad_lo = a.pad_start, pad_hi = min(a.pad_end, a.n_prefix);
+    auto compute = [&](int st, int kb) __attribute__((always_inline)) {
+        const int k0 = kb * 32;
+        f32x4_t sc[2];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            sc[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks)
+                sc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kr[st][j][ks]), __builtin_bit_cast(bf16x8_t, qf[ks]),
+                                                                sc[j], 0, 0, 0);
+        }
+        const bool blk_masked = a.mask != nullptr || k0 + 32 > a.n_keys || (k0 < pad_hi && k0 + 32 > pad_lo) ||
+                                (a.mask_kind != VLA_MASK_NONE && k0 + 32 > a.n_prefix);
+        float p[8];  // keys k0 + 8 q + i
+#pragma unroll
+        for (int i = 0; i < 8; ++i) p[i] = sc[i >> 2][i & 3] * c2;
+        if (blk_masked) {
+            const int kl = k0 + 8 * q;
+            if (a.mask) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) p[i] = kl + i < a.n_keys ? p[i] + a.mask[(long)s * a.n_keys + kl + i] * LOG2E : -INFINITY;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int key = kl + i;
+                    const bool visible = (key < hi) & !((key >= pad_lo) & (key < pad_hi));
+                    p[i] = visible ? p[i] : -INFINITY;
+                }
+            }
+        }
+        float m_blk = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) m_blk = fmaxf(m_blk, p[i]);
+        m_blk = rows_max(m_blk);
+        if (__builtin_amdgcn_ballot_w64(m_blk > m_run + RESCALE_LOG2) != 0) {  // lazy reference update
+            const float m_new = fmaxf(m_run, m_blk);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - ((m_new == -INFINITY) ? 0.f : m_new));
+            l_run *= alpha;
+            m_run = m_new;
+#pragma unroll
+            for (int db = 0; db < NDB; ++db)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[db][e] *= alpha;
+        }
+        const float m_use = (m_run == -INFINITY) ? 0.f : m_run;
+        float psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            p[i] = __builtin_amdgcn_exp2f(p[i] - m_use);
+            psum += p[i];
+        }
+        psum = rows_sum(psum);
+        l_run += psum;
+        u32x4_t pf, pl;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t hw = pack_bf2(p[2 * e], p[2 * e + 1]);
+            pf[e] = hw;
+            if (P2) pl[e] = pack_bf2(p[2 * e] - __uint_as_float(hw << 16), p[2 * e + 1] - __uint_as_float(hw & 0xffff0000u));
+        }
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vr[st][db]), __builtin_bit_cast(bf16x8_t, pf), o[db], 0, 0, 0);
+            if (P2)
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, vr[st][db]), __builtin_bit_cast(bf16x8_t, pl), o[db], 0, 0, 0);
+        }
+    };
+
+    // ST blocks of loads in flight from the start (a slice is at most ST blocks in the shapes this
+    // kernel is chosen for, so it makes one trip to memory); longer slices refill a stage as
+    // soon as it has been multiplied.
+    const bool has_partial = kb1 * 32 > a.n_keys;
+    const int kbp = has_partial ? kb1 - 1 : -1;
+#pragma unroll
+    for (int i = 0; i < ST; ++i) load_blk(i, kb0 + i);
+    // The first ST blocks outside the loop: straight-line code, so the wait in front of a block
+    // leaves the younger blocks' loads in flight (behind a loop header the count would have to
+    // assume the worst of both ways in).
+#pragma unroll
+    for (int st = 0; st < ST; ++st) {
+        const int cur = kb0 + st;
+        if (cur < kb1) {  // uniform
+            if (cur == kbp) mask_partial(st, cur);
+            compute(st, cur);
+        }
+        if (cur + ST < kb1) load_blk(st, cur + ST);  // uniform; only slices longer than ST blocks
+    }
+    for (int base = kb0 + ST; base < kb1; base += ST) {
+#pragma unroll
+        for (int st = 0; st < ST; ++st) {
+            const int cur = base + st;
+            if (cur < kb1) {
+                if (cur == kbp) mask_partial(st, cur);
+                compute(st, cur);
+            }
+            if (cur + ST < kb1) load_blk(st, cur + ST);
+        }
+    }
+
+    // partial rows [pair][row][slice]: unnormalised output, then (max, sum)
+    if (row_valid) {
+        const long prow = ((long)pair * a.r_pad + c) * a.n_split + split;
+        if (q == 0) st_dev64(a.part_ml + prow * 2, m_run, l_run);
+        float* po = a.part_o + prow * D + 4 * q;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+            st_dev64(po + db * 16, o[db][0], o[db][1]);
+            st_dev64(po + db * 16 + 2, o[db][2], o[db][3]);
+        }
+    }
+    // Ordering.  Hardware (gfx950, which this file is compiled for and nothing else -- see the
+    // #error in common.h): the partials above are device-scope atomic stores, i.e. written
+    // through to memory, and vmcnt counts a store only once memory has acknowledged it; the
+    // merger's device-scope atomic loads are served from memory, not from its XCD's L2.
+    // So once vmcnt is zero the partials are visible to every XCD, and the counter's value
+    // tells the last slice that every other slice got that far.  Compiler: the two
+    // workgroup-scope fences forbid moving the stores below the count and the merger's loads
+    // above it; at workgroup scope they cost no cache maintenance (an agent-scope release
+    // would write back the whole L2: 121 us per launch, measured).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's partials are in memory before it is counted
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    int old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(a.arrive + pair, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = __builtin_amdgcn_readfirstlane(old);
+    if (old != a.n_split - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    if (lane == 0) __hip_atomic_store(a.arrive + pair, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    switch (a.n_split) {
+        case 2: merge_rows_static<2>(a, pair, b, hk, grp, R, lane); break;
+        case 3: merge_rows_static<3>(a, pair, b, hk, grp, R, lane); break;
+        case 4: merge_rows_static<4>(a, pair, b, hk, grp, R, lane); break;
+        case 5: merge_rows_static<5>(a, pair, b, hk, grp, R, lane); break;
+        case 6: merge_rows_static<6>(a, pair, b, hk, grp, R, lane); break;
+        case 7: merge_rows_static<7>(a, pair, b, hk, grp, R, lane); break;
+        case 8: merge_rows_static<8>(a, pair, b, hk, grp, R, lane); break;
+        case 9: merge_rows_static<9>(a, pair, b, hk, grp, R, lane); break;
+        case 10: merge_rows_static<10>(a, pair, b, hk, grp, R, lane); break;
+        case 11: merge_rows_static<11>(a, pair, b, hk, grp, R, lane); break;
+        default: merge_rows_static<12>(a, pair, b, hk, grp, R, lane); break;
+    }
 }
 
 // ---- Streaming form of the register-direct kernel: many (batch, kv head) pairs with few
@@ -1608,15 +1809,16 @@ int launch_direct(AttnArgs& a, hipStream_t st, Scratch& sc) {
     // the merge kernel instead.
     constexpr int MERGE_MAX = D <= 64 ? 8 : 4;  // wide heads need the registers of a 4-wavefront workgroup
     bool wg_merge = n_split > 1 && (n_split <= MERGE_MAX || n_units >= 32);
-    // 128-wide heads with few rows (single-token decode): more slices than one workgroup holds,
-    // as single-wavefront workgroups over more CUs, merged by the slice that arrives last.
-    // Slices of three blocks there: each slice costs the merging wavefront a row of loads, and the
-    // hand-over is three dependent trips to memory whatever the count (519 keys, batch 8: six
-    // slices 13.6 us, nine 14.7 us, one workgroup of four 13.5 us alone and 1.4 us slower in sequence).
+    // 128-wide heads with at most 16 rows (single-token decode): more slices than one workgroup
+    // holds, as single-wavefront workgroups over more CUs, merged by the slice that arrives last
+    // (attn_decode16_kernel).  Slices of three blocks there, all of their loads requested at
+    // once: each slice costs the merging wavefront a row of loads, and the hand-over is three
+    // dependent trips to memory whatever the count.
     const int Rb = R < 32 ? R : 32;
     int n_arrive = n_split < (nb_total + 2) / 3 || tn.attn_split_set ? n_split : (nb_total + 2) / 3;
+    if (n_arrive > DEC_MAX_NS) n_arrive = DEC_MAX_NS;
     if (n_arrive * Rb > ARRIVE_MAX_T) n_arrive = ARRIVE_MAX_T / Rb;
-    bool arrive = D == 128 && n_arrive > MERGE_MAX && a.n_rblocks == 1 && n_units <= ARRIVE_MAX_UNITS && !tn.attn_no_arrive;
+    bool arrive = D == 128 && R <= DEC_MAX_R && n_arrive > MERGE_MAX && a.n_rblocks == 1 && n_units <= ARRIVE_MAX_UNITS && !tn.attn_no_arrive;
     if (arrive) {
         n_split = n_arrive;
         wg_merge = false;
@@ -1641,14 +1843,22 @@ int launch_direct(AttnArgs& a, hipStream_t st, Scratch& sc) {
         if (rc != VLA_K_OK) return rc;
     }
     if (sc.kind == Scratch::DRY) return VLA_K_OK;
-    arrive = arrive && a.n_split > 1 && a.n_split * Rb <= ARRIVE_MAX_T;
+    arrive = arrive && a.n_split > 1 && a.n_split <= DEC_MAX_NS && a.n_split * Rb <= ARRIVE_MAX_T;
     if (!arrive) a.arrive = nullptr;
-    const int wgw = arrive ? 1 : 4;  // wavefronts per workgroup
+    if constexpr (D == 128) {
+        if (arrive) {  // a wavefront per (pair, slice)
+            const unsigned grid16 = (unsigned)(n_units * a.n_split);
+            if (a.p2) attn_decode16_kernel<true, 3><<<grid16, 64, 0, st>>>(a);
+            else attn_decode16_kernel<false, 3><<<grid16, 64, 0, st>>>(a);
+            return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+        }
+    }
+    const int wgw = 4;  // wavefronts per workgroup
     const unsigned grid = (unsigned)(((long)n_units * a.n_split + wgw - 1) / wgw);
     if (a.p2) attn_direct_kernel<D, true, ST, false><<<grid, wgw * 64, 0, st>>>(a);
     else attn_direct_kernel<D, false, ST, false><<<grid, wgw * 64, 0, st>>>(a);
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
-    if (a.n_split > 1 && !arrive) {
+    if (a.n_split > 1) {
         attn_merge_kernel<bf16_t, false><<<(unsigned)(((long)n_pairs * R + 3) / 4), 256, 0, st>>>(a.part_o, a.part_ml, (bf16_t*)a.out,
                                                                                            n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq,
                                                                                            a.Hkv, D);
