@@ -85,21 +85,42 @@ template <> struct Elem<bf16_t> {
     __device__ static __forceinline__ float round(float v) { return bf2f(f2bf(v)); }
 };
 
-// 64-lane wavefront reductions; every lane ends with the result.
+// 64-lane wavefront reductions; every lane ends with the result.  No trip through LDS (a
+// ds_bpermute butterfly costs six dependent LDS round trips, which is most of the time of a
+// kernel that is one wavefront's chain of dependent steps): inside a row of 16 lanes the
+// partners come from DPP operands (neighbour, neighbour pair, the mirrored half, the
+// mirrored row), the four rows are combined by gfx950's row swaps (v_permlane16_swap of a
+// register with itself leaves rows (0, 0, 2, 2) in one copy and (1, 1, 3, 3) in the other;
+// v_permlane32_swap does the same for the halves).  Both partners of a step form the same
+// sum of the same two values, so every lane ends with the same bits.
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+}
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_HALF_MIRROR = 0x141, DPP_ROW_MIRROR = 0x140;
+template <typename Op>
+__device__ __forceinline__ uint32_t wave_combine_u32(uint32_t v, Op op) {
+    v = op(v, dpp_u32<DPP_XOR1>(v));
+    v = op(v, dpp_u32<DPP_XOR2>(v));
+    v = op(v, dpp_u32<DPP_HALF_MIRROR>(v));
+    v = op(v, dpp_u32<DPP_ROW_MIRROR>(v));
+    u32x2_t r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    v = op(r[0], r[1]);
+    r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return op(r[0], r[1]);
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
+    return __uint_as_float(wave_combine_u32(__float_as_uint(v), [](uint32_t a, uint32_t b) {
+        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
+    }));
 }
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    return __uint_as_float(wave_combine_u32(__float_as_uint(v), [](uint32_t a, uint32_t b) {
+        return __float_as_uint(__uint_as_float(a) + __uint_as_float(b));
+    }));
 }
 __device__ __forceinline__ int wave_sum_i(int v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    return (int)wave_combine_u32((uint32_t)v, [](uint32_t a, uint32_t b) { return a + b; });
 }
 
 // Block reductions through LDS for blocks of up to 16 wavefronts.  `red` holds
