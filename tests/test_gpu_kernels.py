@@ -262,6 +262,109 @@ def test_linear_bf16_every_kernel_and_tiling_gives_the_same_bits(tune, M, N, K):
         assert np.array_equal(yb.view(np.uint16), first[1].view(np.uint16)), key
 
 
+@pytest.mark.parametrize("rows_max", [32, 64])
+@pytest.mark.parametrize("M,N,K", [(17, 1536, 1536), (1, 64, 128), (5, 200, 720), (32, 96, 2048), (50, 720, 960), (64, 24, 72)])
+def test_few_bf16_rows_take_the_split_k_kernel(tune, rows_max, M, N, K):
+    """A few bf16 rows through a projection: 16 columns per workgroup, K split over its
+    wavefronts (up to 32 rows by default, up to 64 when asked).  Against the oracle and against
+    the tiled kernel, with bias, residual, fp32 output, ragged N (not a multiple of 16) and K
+    (not a multiple of 32).  The sums are formed in another order than by the tiled kernel."""
+    r = np.random.default_rng(7100 + M + N)
+    x = orc.round_bf16(r.standard_normal((M, K)).astype(np.float32))
+    W = orc.round_bf16((0.05 * r.standard_normal((N, K))).astype(np.float32))
+    b = (0.1 * r.standard_normal(N)).astype(np.float32)
+    res = orc.round_bf16(r.standard_normal((M, N)).astype(np.float32))
+    xd, Wd, rd = to_dev(x, BF16), to_dev(W, BF16), to_dev(res, BF16)
+
+    def run():
+        y = torch.zeros((M, N), dtype=torch.float32, device="cuda")
+        pkg.call("vla_linear", xd, Wd, None, None, y, BF16, F32, M, N, K)
+        yb = torch.zeros((M, N), dtype=torch.int16, device="cuda")
+        pkg.call("vla_linear", xd, Wd, dev(b), rd, yb, BF16, BF16, M, N, K)
+        yi = rd.clone()  # in place: the residual is the output
+        pkg.call("vla_linear", xd, Wd, dev(b), yi, yi, BF16, BF16, M, N, K)
+        sync()
+        return host(y), as_f32(yb, BF16), as_f32(yi, BF16)
+
+    tune.set("VLA_GEMM_ROWS_MAX", rows_max)
+    got = run()
+    tune.set("VLA_GEMM_ROWS_MAX", 0)
+    tiled = run()
+    want = orc.linear(x, W)
+    assert rel_err(got[0], want) < 1e-5 and rel_err(tiled[0], want) < 1e-5
+    assert bf16_close(got[1], want + b + res) and np.array_equal(got[1], got[2])
+    assert rel_err(got[0], tiled[0]) < 1e-5 and rel_err(got[1], tiled[1]) < 8e-3
+
+
+@pytest.mark.parametrize("rows_max", [32, 64])
+@pytest.mark.parametrize("name,B,S,Hq,Hkv,D,K,norm,rope,self_layer", [
+    ("gr00t-self-1", 1, 17, 32, 32, 48, 1536, "layer", False, True),
+    ("gr00t-cross-q-1", 1, 17, 32, 32, 48, 1536, "layer", False, False),
+    ("smolvla-self-1", 1, 50, 15, 5, 64, 720, "rms", True, True),
+    ("pi0-1", 1, 51, 8, 1, 256, 1024, "rms", True, True),
+    ("two-short-observations", 2, 9, 4, 2, 64, 328, "none", True, True),
+    ("bitvla-shape", 1, 7, 20, 5, 128, 256, "none", True, True),
+])
+def test_few_bf16_rows_fused_qkv_on_the_split_k_kernel(tune, rows_max, name, B, S, Hq, Hkv, D, K, norm, rope, self_layer):
+    """The fused Q | K | V projection of a few rows on the split-K kernel: plain, with the RMS
+    pre-norm and with the modulated LayerNorm taken inside, rotation pairs, append at an offset
+    into the caches; against the oracle and against the tiled kernel."""
+    r = np.random.default_rng(7200 + K + S)
+    M, P = B * S, 11
+    nkv = Hkv if self_layer else 0
+    N = (Hq + 2 * nkv) * D
+    eps = 1e-5
+    x = orc.round_bf16((2.0 * r.standard_normal((M, K)) * (1.0 + 3.0 * r.random((M, 1))) + 1.5 * r.standard_normal((M, 1))).astype(np.float32))
+    W = orc.round_bf16((0.02 * r.standard_normal((N, K))).astype(np.float32))
+    b = (0.1 * r.standard_normal(N)).astype(np.float32)
+    sc, sh = (0.3 * r.standard_normal(K)).astype(np.float32), (0.3 * r.standard_normal(K)).astype(np.float32)
+    g = orc.round_bf16((1.0 + 0.3 * r.standard_normal(K)).astype(np.float32))
+    c, s_ = orc.rope_tables(np.arange(S, dtype=np.int32) + P + 1, D, 10000.0)
+    cd, sd = (dev(c), dev(s_)) if rope else (None, None)
+    t_max = (P + S + 63) // 64 * 64
+
+    def run():
+        kc, vc = empty((B, Hkv, t_max, D), BF16), empty((B, Hkv, D, t_max), BF16)
+        q = empty((M, Hq * D), BF16)
+        if norm == "layer":
+            Wf, cs, bs = np.empty((N, K), np.uint16), np.empty(N, np.float32), np.empty(N, np.float32)
+            assert pkg.lib().vla_fold_adaln_weight_host(orc.to_bf16(W).ctypes.data, b.ctypes.data, sc.ctypes.data, sh.ctypes.data, N, K,
+                                                        Wf.ctypes.data, cs.ctypes.data, bs.ctypes.data) == 0
+            pkg.call("vla_layernorm_attn_qkv_rope", to_dev(x, BF16), dev(Wf), dev(cs), dev(bs), BF16, M, K, S, Hq, Hkv,
+                     int(self_layer), int(self_layer), D, cd, sd, q, kc, vc, t_max, P, eps)
+        elif norm == "rms":
+            Wf = np.empty((N, K), np.uint16)
+            assert pkg.lib().vla_fold_norm_weight_host(orc.to_bf16(W).ctypes.data, orc.to_bf16(g).ctypes.data, BF16, N, K, Wf.ctypes.data) == 0
+            pkg.call("vla_rmsnorm_attn_qkv_rope", to_dev(x, BF16), dev(Wf), dev(b), BF16, M, K, S, Hq, Hkv, int(self_layer),
+                     int(self_layer), D, cd, sd, q, kc, vc, t_max, P, eps)
+        else:
+            pkg.call("vla_attn_qkv_rope", to_dev(x, BF16), to_dev(W, BF16), dev(b), BF16, M, K, S, Hq, Hkv, int(self_layer),
+                     int(self_layer), D, cd, sd, q, kc, vc, t_max, P)
+        out = [as_f32(q, BF16).reshape(M, Hq, D)]
+        if self_layer:
+            kd, vd = empty((B, S, Hkv, D), BF16), empty((B, S, Hkv, D), BF16)
+            pkg.call("vla_kv_gather", kc, vc, kd, vd, BF16, B, Hkv, D, t_max, P, S)
+            out += [as_f32(kd, BF16).reshape(M, Hkv, D), as_f32(vd, BF16).reshape(M, Hkv, D)]
+        sync()
+        return out
+
+    xin = orc.adaln(x, sc, sh, eps) if norm == "layer" else (orc.rms_norm(x, g, eps) if norm == "rms" else x)
+    y = orc.linear(xin, W, b)
+    want = [y[:, :Hq * D].reshape(M, Hq, D)]
+    if self_layer:
+        want += [y[:, Hq * D:(Hq + Hkv) * D].reshape(M, Hkv, D), y[:, (Hq + Hkv) * D:].reshape(M, Hkv, D)]
+    if rope:
+        for i in range(min(2, len(want))):
+            want[i] = np.concatenate([orc.rope_neox(want[i][bb * S:(bb + 1) * S], c, s_) for bb in range(B)])
+    tune.set("VLA_GEMM_ROWS_MAX", rows_max)
+    got = run()
+    tune.set("VLA_GEMM_ROWS_MAX", 0)
+    tiled = run()
+    for gf, gt, w in zip(got, tiled, want):
+        assert bf16_close(gf, w) and rel_err(gf, w) < 8e-3
+        assert rel_err(gf, gt) < 8e-3
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("name,B,S,Hq,Hkv,D,K,rope,bias,P", [
     ("smolvla-self", 2, 50, 15, 5, 64, 720, True, False, 241),

@@ -1134,23 +1134,6 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
 // [pair][row][slice] and the merge unrolled for the slice count.
 constexpr int DEC_MAX_NS = 12, DEC_MAX_R = 16;
 
-// A value combined over the four 16-lane rows of the wavefront (lanes c, c + 16, c + 32, c + 48)
-// with gfx950's row swaps instead of two trips through LDS: after v_permlane16_swap of a register
-// with itself one copy holds rows (0, 0, 2, 2) and the other rows (1, 1, 3, 3); v_permlane32_swap does
-// the same for the two halves.
-__device__ __forceinline__ float rows_max(float x) {
-    u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
-}
-__device__ __forceinline__ float rows_sum(float x) {
-    u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
-    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
-}
-
 template <int NS>
 __device__ __forceinline__ void merge_rows_static(const AttnArgs& a, int pair, int b, int hk, int grp, int R, int lane) {
     constexpr int D = 128;

@@ -26,6 +26,7 @@ struct Tuning {
     bool attn_no_arrive = false; // VLA_ATTN_NO_ARRIVE: no in-launch merge by the last slice to arrive
     bool attn_no_direct = false; // VLA_ATTN_NO_DIRECT: never the register-direct kernel
     bool attn_no_stream = false; // VLA_ATTN_NO_STREAM: never the streaming (LDS-ring) form of the register-direct kernel
+    int gemm_rows_max = 32;      // VLA_GEMM_ROWS_MAX: bf16 projections of at most this many rows (up to 64) take the split-K kernel, 0 = never
     bool attn_no_small = false;  // VLA_ATTN_NO_SMALL: fp32 launches with few row tiles do not split their keys beyond the usual rule
     int attn_direct_rows = 32;   // VLA_ATTN_DIRECT_ROWS: row limit of the register-direct kernel
     int gemm_tile = -1;          // VLA_GEMM_TILE: 0..5
@@ -121,6 +122,23 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 __device__ __forceinline__ int wave_sum_i(int v) {
     return (int)wave_combine_u32((uint32_t)v, [](uint32_t a, uint32_t b) { return a + b; });
+}
+
+// A value combined over the four 16-lane rows of the wavefront (lanes c, c + 16, c + 32, c + 48)
+// with gfx950's row swaps instead of two trips through LDS: after v_permlane16_swap of a register
+// with itself one copy holds rows (0, 0, 2, 2) and the other rows (1, 1, 3, 3); v_permlane32_swap does
+// the same for the two halves.
+__device__ __forceinline__ float rows_max(float x) {
+    u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float rows_sum(float x) {
+    u32x2_t r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
 // Block reductions through LDS for blocks of up to 16 wavefronts.  `red` holds

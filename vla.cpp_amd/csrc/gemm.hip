@@ -912,6 +912,232 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     }
 }
 
+// ---- A few rows (M <= 64) of a bf16 projection: 16 columns per workgroup, K split over its wavefronts ----
+// One observation's suffix rows through a projection.  The weights are read once and from
+// memory (a step touches every layer's weights once, more than the caches hold), and what a
+// CU gets out of memory is bounded by its own requests in flight, not by the chip: the tiled
+// kernels' 64-column tiles put such a launch on N / 64 CUs, a tenth of the chip, each walking
+// all of K tile by tile.  Here a workgroup owns 16 columns -- N / 16 workgroups -- and its
+// eight wavefronts each take an eighth of K and request all of it at once, straight into
+// MFMA operand registers: v_mfma_f32_16x16x32_bf16 with the weight rows as the left operand
+// (16 columns x 32 k) and 16 activation rows as the right one, so that lane (c, q) =
+// (lane % 16, lane / 16) reads 16 bytes (8 k) of weight row c and of activation row c, and
+// four lanes cover 64 consecutive bytes of a row.  The partial tiles meet in LDS and are
+// added in wavefront order; the epilogues (bias, fused-norm scaling, rotation, scatter into
+// the caches, residual) are the tiled kernels' arithmetic on a (row, column pair) per thread.
+// The 16 columns are 8 + 8: for rotated segments the columns d .. d + 7 of a head and their
+// partners d + D / 2, else 16 consecutive columns.  The sums are formed in another order than
+// by the tiled kernels: the two agree to fp32 rounding, not bit for bit.
+constexpr int SR_WAVES = 8, SR_MAX_ROWS = 64, SR_PSTR = 20, SR_MAX_K = 2048;
+struct RowCols {
+    int base_lo, base_hi;  // rows of W of tile columns [0, 8) and [8, 16)
+    int seg;               // 0 Q, 1 K, 2 V (QKV mode)
+    int col_lo, col_hi;    // segment-local column of tile column 0 and of tile column 8
+    bool rope;
+};
+template <int kEpi>
+__device__ __forceinline__ RowCols row_cols(const GemmArgs& a, int t) {
+    RowCols rc;
+    rc.seg = 0;
+    rc.rope = false;
+    if (kEpi != EPI_QKV) {
+        rc.base_lo = rc.col_lo = t * 16;
+        rc.base_hi = rc.col_hi = t * 16 + 8;
+        return rc;
+    }
+    const int tq = a.Hq * a.D / 16, tk = a.nk * a.D / 16;
+    int lt = t, seg_base = 0;
+    if (t >= tq + tk) {
+        rc.seg = 2;
+        lt = t - tq - tk;
+        seg_base = (a.Hq + a.nk) * a.D;
+    } else if (t >= tq) {
+        rc.seg = 1;
+        lt = t - tq;
+        seg_base = a.Hq * a.D;
+    }
+    rc.rope = (a.cos_t != nullptr) && rc.seg != 2;
+    if (rc.rope) {
+        const int tph = a.D / 16;  // tiles per head
+        const int head = lt / tph, chunk = lt % tph;
+        rc.col_lo = head * a.D + chunk * 8;
+        rc.col_hi = rc.col_lo + a.D / 2;
+    } else {
+        rc.col_lo = lt * 16;
+        rc.col_hi = rc.col_lo + 8;
+    }
+    rc.base_lo = seg_base + rc.col_lo;
+    rc.base_hi = seg_base + rc.col_hi;
+    return rc;
+}
+
+template <int kEpi, int kNorm, int RB, int MAXC>  // RB: 16-row blocks; MAXC: 32-k chunks per wavefront held in registers, K <= 256 MAXC
+__global__ void __launch_bounds__(SR_WAVES * 64) gemm_rows_bf16_kernel(GemmArgs a) {
+    __shared__ __attribute__((aligned(16))) float part[SR_WAVES][RB * 16][SR_PSTR];
+    __shared__ float stat_part[SR_WAVES][RB * 16][2];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 15, q = lane >> 4;
+    const RowCols rc = row_cols<kEpi>(a, blockIdx.x);
+    const int nch = (a.K + 31) / 32, per = (nch + SR_WAVES - 1) / SR_WAVES, ch0 = wave * per;
+
+    // rows past N or M and pieces past K are read from valid addresses; their products are dropped or zeroed
+    const unsigned char* wrow = (const unsigned char*)a.W + (long)min(max(c < 8 ? rc.base_lo + c : rc.base_hi + c - 8, 0), a.N - 1) * a.K * 2;
+    const unsigned char* xrow[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) xrow[rb] = (const unsigned char*)a.A + (long)min(rb * 16 + c, a.M - 1) * a.K * 2;
+    u32x4_t wf[MAXC], xf[MAXC][RB];
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        const int ch = min(ch0 + i, nch - 1);
+        const long off = (long)min(ch * 32 + 8 * q, a.K - 8) * 2;
+        wf[i] = *reinterpret_cast<const u32x4_t*>(wrow + off);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) xf[i][rb] = *reinterpret_cast<const u32x4_t*>(xrow[rb] + off);
+    }
+    // What the epilogue reads from memory is requested now, behind the operand loads.  Epilogue
+    // thread -> row tid / 8, tile columns i = tid % 8 and 8 + i.  No branch around the loads:
+    // addresses are clamped into the arrays and values that are not needed are dropped.
+    const int erow = tid >> 3, ei = tid & 7;
+    const int em = min(erow, a.M - 1);
+    const int n_lo = min(rc.base_lo + ei, a.N - 1), n_hi = min(rc.base_hi + ei, a.N - 1);
+    float b_lo = 0.f, b_hi = 0.f, cs_lo = 0.f, cs_hi = 0.f, g_lo = 1.f, g_hi = 1.f, rot_c = 1.f, rot_s = 0.f, r_lo = 0.f, r_hi = 0.f;
+    if (a.bias) {
+        b_lo = a.bias[n_lo];
+        b_hi = a.bias[n_hi];
+    }
+    if (kNorm == NORM_LAYER) {
+        cs_lo = a.colsum[n_lo];
+        cs_hi = a.colsum[n_hi];
+    }
+    if (kEpi == EPI_PLAIN) {
+        if (a.col_gate) {
+            g_lo = a.col_gate[n_lo];
+            g_hi = a.col_gate[n_hi];
+        }
+        if (a.residual) {
+            if (a.out_bf16) {
+                r_lo = bf2f(((const bf16_t*)a.residual)[(long)em * a.N + n_lo]);
+                r_hi = bf2f(((const bf16_t*)a.residual)[(long)em * a.N + n_hi]);
+            } else {
+                r_lo = ((const float*)a.residual)[(long)em * a.N + n_lo];
+                r_hi = ((const float*)a.residual)[(long)em * a.N + n_hi];
+            }
+        }
+    }
+    if (kEpi == EPI_QKV && rc.rope) {
+        const int half = a.D >> 1;
+        const long ri = (long)(em % a.S) * half + (rc.col_lo % a.D) + ei;
+        rot_c = a.cos_t[ri];
+        rot_s = a.sin_t[ri];
+    }
+
+    f32x4_t acc[RB];
+    float ssq[RB], ssum[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        acc[rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        ssq[rb] = ssum[rb] = 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        if (i < per && ch0 + i < nch) {  // uniform
+            const bool inside = (ch0 + i) * 32 + 8 * q < a.K;  // K is a multiple of 8: a piece is inside or outside as a whole
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                u32x4_t xv = xf[i][rb];
+                if (!inside) xv = u32x4_t{0u, 0u, 0u, 0u};
+                if (kNorm) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        ssq[rb] = add_squares_bf16x2(xv[e], ssq[rb]);
+                        if (kNorm == NORM_LAYER) ssum[rb] = add_pair_bf16x2(xv[e], ssum[rb]);
+                    }
+                }
+                acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf[i]), __builtin_bit_cast(bf16x8_t, xv), acc[rb], 0, 0, 0);
+            }
+        }
+    }
+    // acc[rb][e]: tile column 4 q + e, row 16 rb + c
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        *reinterpret_cast<f32x4_t*>(&part[wave][rb * 16 + c][4 * q]) = acc[rb];
+        if (kNorm) {
+            const float s2 = rows_sum(ssq[rb]), s1 = rows_sum(ssum[rb]);
+            if (q == 0) {
+                stat_part[wave][rb * 16 + c][0] = s2;
+                stat_part[wave][rb * 16 + c][1] = s1;
+            }
+        }
+    }
+    __syncthreads();
+    if (erow >= RB * 16 || erow >= a.M) return;
+    const int m = erow;
+    float lo = 0.f, hi = 0.f, sq = 0.f, sm = 0.f;
+#pragma unroll
+    for (int w = 0; w < SR_WAVES; ++w) {
+        lo += part[w][erow][ei];
+        hi += part[w][erow][8 + ei];
+        if (kNorm) {
+            sq += stat_part[w][erow][0];
+            sm += stat_part[w][erow][1];
+        }
+    }
+    if (kNorm) {
+        const float inv_k = 1.0f / (float)a.K;
+        if (kNorm == NORM_LAYER) {
+            // sum_k (x - mean) rstd W[n][k] = rstd acc - (mean rstd) colsum[n]
+            const float mean = sm * inv_k;
+            const float f = rsqrtf(fmaxf(sq * inv_k - mean * mean, 0.f) + a.norm_eps);
+            const float ms = mean * f;
+            lo = lo * f - ms * cs_lo;
+            hi = hi * f - ms * cs_hi;
+        } else {
+            const float f = rsqrtf(sq * inv_k + a.norm_eps);
+            lo *= f;
+            hi *= f;
+        }
+    }
+    lo += b_lo;
+    hi += b_hi;
+    const bool ok_lo = rc.base_lo + ei < a.N, ok_hi = rc.base_hi + ei < a.N;
+    if (kEpi == EPI_PLAIN) {
+        if (a.act != VLA_ACT_NONE) {
+            lo = apply_act(lo, a.act);
+            hi = apply_act(hi, a.act);
+        }
+        lo = lo * g_lo + r_lo;
+        hi = hi * g_hi + r_hi;
+        const long o = (long)m * a.N;
+        if (a.out_bf16) {
+            if (ok_lo) ((bf16_t*)a.Y)[o + n_lo] = f2bf(lo);
+            if (ok_hi) ((bf16_t*)a.Y)[o + n_hi] = f2bf(hi);
+        } else {
+            if (ok_lo) ((float*)a.Y)[o + n_lo] = lo;
+            if (ok_hi) ((float*)a.Y)[o + n_hi] = hi;
+        }
+        return;
+    }
+    // QKV: rotation, scatter
+    if (rc.rope) {
+        const float x0 = lo, x1 = hi;
+        lo = x0 * rot_c - x1 * rot_s;
+        hi = x1 * rot_c + x0 * rot_s;
+    }
+    const int b = m / a.S, s = m % a.S;
+#pragma unroll
+    for (int hlf = 0; hlf < 2; ++hlf) {
+        const float v = hlf ? hi : lo;
+        const int col = (hlf ? rc.col_hi : rc.col_lo) + ei;
+        if (rc.seg == 0) {
+            ((bf16_t*)a.q_out)[(long)m * (a.Hq * a.D) + col] = f2bf(v);
+        } else {
+            const int head = col / a.D, d = col % a.D;
+            if (rc.seg == 1) ((bf16_t*)a.k_cache)[(((long)b * a.Hkv + head) * a.t_max + a.tok_offset + s) * a.D + d] = f2bf(v);
+            else ((bf16_t*)a.vt_cache)[(((long)b * a.Hkv + head) * a.D + d) * (long)a.t_max + a.tok_offset + s] = f2bf(v);
+        }
+    }
+}
+
 // Large-M ternary GEMM (BitVLA prefill: M = batch x prefix tokens).  Workgroup tile
 // (64*WM) x 256 with WM x 2 wavefronts, each owning 64 x 128 = 2 x 4 MFMA blocks (128
 // accumulator registers), so one 16-byte A fragment feeds four MFMAs and one weight
@@ -1821,6 +2047,40 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
         if (a.M <= SKINNY_MAX_M && a.K % 4 == 0 && a.norm_eps < 0.f && tuning().gemm_tile < 0 && (uintptr_t)a.A % 16 == 0 &&
             (uintptr_t)a.W % 16 == 0 && (kEpi == EPI_PLAIN || a.D % 8 == 0)) {
             linear_f32_skinny_kernel<kEpi><<<dim3((unsigned)((a.N + 7) / 8), (unsigned)((a.M + 15) / 16)), 256, 0, st>>>(a);
+            return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+        }
+    }
+    if constexpr (std::is_same<T, bf16_t>::value && (kEpi == EPI_PLAIN || kEpi == EPI_QKV)) {
+        // a few bf16 rows (one observation's suffix through a projection): 16 columns per workgroup, K split over its wavefronts
+        bool rows_ok = a.M <= tuning().gemm_rows_max && a.M <= SR_MAX_ROWS && a.K % 8 == 0 && a.K >= 64 && a.K <= SR_MAX_K &&
+                       tuning().gemm_tile < 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0 && !(a.colsum && a.norm_eps < 0.f);
+        if (kEpi == EPI_QKV) rows_ok = rows_ok && a.D % 16 == 0 && a.N % 16 == 0;
+        if (rows_ok) {
+            const unsigned grid = (unsigned)((a.N + 15) / 16);
+            const int per = ((a.K + 31) / 32 + SR_WAVES - 1) / SR_WAVES, rb = (a.M + 15) / 16;
+#define VLA_ROWS_K(NORM, RB)                                                                                       \
+    do {                                                                                                           \
+        if (per <= 2) gemm_rows_bf16_kernel<kEpi, NORM, RB, 2><<<grid, SR_WAVES * 64, 0, st>>>(a);                  \
+        else if (per <= 4) gemm_rows_bf16_kernel<kEpi, NORM, RB, 4><<<grid, SR_WAVES * 64, 0, st>>>(a);             \
+        else if (per <= 6) gemm_rows_bf16_kernel<kEpi, NORM, RB, 6><<<grid, SR_WAVES * 64, 0, st>>>(a);             \
+        else gemm_rows_bf16_kernel<kEpi, NORM, RB, 8><<<grid, SR_WAVES * 64, 0, st>>>(a);                           \
+    } while (0)
+#define VLA_ROWS(NORM)                       \
+    do {                                     \
+        if (rb <= 1) VLA_ROWS_K(NORM, 1);    \
+        else if (rb == 2) VLA_ROWS_K(NORM, 2); \
+        else VLA_ROWS_K(NORM, 4);            \
+    } while (0)
+            if (a.norm_eps < 0.f) {
+                VLA_ROWS(NORM_NONE);
+            } else if constexpr (kEpi == EPI_QKV) {
+                if (a.colsum) VLA_ROWS(NORM_LAYER);
+                else VLA_ROWS(NORM_RMS);
+            } else {
+                return VLA_K_ERR_SHAPE;  // the row statistics belong to the fused QKV projections
+            }
+#undef VLA_ROWS
+#undef VLA_ROWS_K
             return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
         }
     }

@@ -34,6 +34,7 @@ void load_locked() {
     t.attn_no_arrive = getenv("VLA_ATTN_NO_ARRIVE") != nullptr;
     t.attn_no_direct = getenv("VLA_ATTN_NO_DIRECT") != nullptr;
     t.attn_no_stream = getenv("VLA_ATTN_NO_STREAM") != nullptr;
+    t.gemm_rows_max = env_int("VLA_GEMM_ROWS_MAX", 32);
     t.attn_no_small = getenv("VLA_ATTN_NO_SMALL") != nullptr;
     t.attn_direct_rows = env_int("VLA_ATTN_DIRECT_ROWS", 32);
     t.gemm_tile = env_int("VLA_GEMM_TILE", -1);
