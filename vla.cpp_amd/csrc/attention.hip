@@ -389,7 +389,7 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
             for (int i = 0; i < 16; ++i) m_tile = fmaxf(m_tile, p[kb][i]);
-        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, 64));
+        m_tile = halves_max(m_tile);
         // Online softmax with a lazily updated reference: m_run moves (and the accumulators
         // are rescaled) only when some row's maximum exceeds it by more than 2^RESCALE_LOG2;
         // until then the probabilities are taken against the older reference, at most
@@ -415,7 +415,7 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
                 p[kb][i] = e;
                 psum += e;
             }
-        psum += __shfl_xor(psum, 32, 64);
+        psum = halves_sum(psum);
         l_run += psum;
     };
     // O^T += V^T . P^T from the staged V^T tile.
@@ -973,7 +973,7 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
         float m_blk = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; ++i) m_blk = fmaxf(m_blk, p[i]);
-        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
+        m_blk = halves_max(m_blk);
         if (__builtin_amdgcn_ballot_w64(m_blk > m_run + RESCALE_LOG2) != 0) {  // lazy reference update
             const float m_new = fmaxf(m_run, m_blk);
             const float alpha = __builtin_amdgcn_exp2f(m_run - ((m_new == -INFINITY) ? 0.f : m_new));
@@ -991,7 +991,7 @@ __global__ void __launch_bounds__((MERGE && D <= 64) ? 512 : 256, D <= 64 ? 2 : 
             p[i] = __builtin_amdgcn_exp2f(p[i] - m_use);
             psum += p[i];
         }
-        psum += __shfl_xor(psum, 32, 64);
+        psum = halves_sum(psum);
         l_run += psum;
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
@@ -1561,7 +1561,7 @@ __global__ void __launch_bounds__(256, 1) attn_stream_kernel(AttnArgs a, int n_u
         float m_blk = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; ++i) m_blk = fmaxf(m_blk, p[i]);
-        m_blk = fmaxf(m_blk, __shfl_xor(m_blk, 32, 64));
+        m_blk = halves_max(m_blk);
         if (__builtin_amdgcn_ballot_w64(m_blk > m_run + RESCALE_LOG2) != 0) {  // lazy reference update
             const float m_new = fmaxf(m_run, m_blk);
             const float alpha = __builtin_amdgcn_exp2f(m_run - ((m_new == -INFINITY) ? 0.f : m_new));
@@ -1579,7 +1579,7 @@ __global__ void __launch_bounds__(256, 1) attn_stream_kernel(AttnArgs a, int n_u
             p[i] = __builtin_amdgcn_exp2f(p[i] - m_use);
             psum += p[i];
         }
-        psum += __shfl_xor(psum, 32, 64);
+        psum = halves_sum(psum);
         l_run += psum;
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {

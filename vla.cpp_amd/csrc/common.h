@@ -124,6 +124,16 @@ __device__ __forceinline__ int wave_sum_i(int v) {
     return (int)wave_combine_u32((uint32_t)v, [](uint32_t a, uint32_t b) { return a + b; });
 }
 
+// A value combined over the two halves of the wavefront (lanes r and r + 32): one row swap
+// instead of a trip through LDS.
+__device__ __forceinline__ float halves_max(float x) {
+    const u32x2_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float halves_sum(float x) {
+    const u32x2_t r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 // A value combined over the four 16-lane rows of the wavefront (lanes c, c + 16, c + 32, c + 48)
 // with gfx950's row swaps instead of two trips through LDS: after v_permlane16_swap of a register
 // with itself one copy holds rows (0, 0, 2, 2) and the other rows (1, 1, 3, 3); v_permlane32_swap does

@@ -30,7 +30,8 @@
 // them in).  A wavefront takes whole (observation, head) pairs: scores as S^T = K Q^T with
 // v_mfma_f32_16x16x16_bf16, so that a lane ends up with four consecutive keys of one query,
 // which is the layout the same instruction wants for P as the left operand of P V; softmax in
-// registers (max and sum over the lane's values and the three other lanes of the query).
+// registers (max and sum over the lane's values and the three other lanes of the query, which
+// meet through the row-swap instructions).
 #include "common.h"
 
 namespace vk {
@@ -226,11 +227,7 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     float* stat = reinterpret_cast<float*>(lds + (FS_ROWS * FS_QS + FS_MAX_OB * FS_D * FS_VS) * 2);  // [FS_ROWS][2]: (sum of squares, sum)
 #pragma unroll
     for (int i = 0; i < 5; ++i) {
-        float s2 = ssq[i], s1 = ssum[i];
-        s2 += __shfl_xor(s2, 16, 64);
-        s1 += __shfl_xor(s1, 16, 64);
-        s2 += __shfl_xor(s2, 32, 64);
-        s1 += __shfl_xor(s1, 32, 64);
+        const float s2 = rows_sum(ssq[i]), s1 = rows_sum(ssum[i]);
         const int rb = wm + 2 * i;
         if (q == 0 && i < nr && wn == 0) {
             stat[(rb * 16 + c) * 2] = s2;
@@ -323,8 +320,7 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
                         if (16 * kb + 4 * q + e >= S) sT[p][kb][qb][e] = -INFINITY;
                         mx = fmaxf(mx, sT[p][kb][qb][e]);
                     }
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                mx = rows_max(mx);
                 float sum = 0.f;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
@@ -334,8 +330,7 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
                         sT[p][kb][qb][e] = pr;
                         sum += pr;
                     }
-                sum += __shfl_xor(sum, 16, 64);
-                sum += __shfl_xor(sum, 32, 64);
+                sum = rows_sum(sum);
                 const float inv = 1.0f / sum;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb) {
