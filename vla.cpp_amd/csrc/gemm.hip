@@ -971,26 +971,33 @@ __device__ __forceinline__ RowCols row_cols(const GemmArgs& a, int t) {
     return rc;
 }
 
-template <int kEpi, int kNorm, int RB, int MAXC>  // RB: 16-row blocks; MAXC: 32-k chunks per wavefront held in registers, K <= 256 MAXC
+template <int kEpi, int kNorm, int RB, int MAXC, int NB>  // RB: 16-row blocks; MAXC: 32-k chunks per wavefront held in registers, K <= 256 MAXC; NB: 16-column tiles per workgroup
 __global__ void __launch_bounds__(SR_WAVES * 64) gemm_rows_bf16_kernel(GemmArgs a) {
-    __shared__ __attribute__((aligned(16))) float part[SR_WAVES][RB * 16][SR_PSTR];
+    __shared__ __attribute__((aligned(16))) float part[SR_WAVES][NB][RB * 16][SR_PSTR];
     __shared__ float stat_part[SR_WAVES][RB * 16][2];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 15, q = lane >> 4;
-    const RowCols rc = row_cols<kEpi>(a, blockIdx.x);
+    const int n_t16 = (a.N + 15) / 16;
+    RowCols rc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) rc[nb] = row_cols<kEpi>(a, min((int)blockIdx.x * NB + nb, n_t16 - 1));
     const int nch = (a.K + 31) / 32, per = (nch + SR_WAVES - 1) / SR_WAVES, ch0 = wave * per;
 
     // rows past N or M and pieces past K are read from valid addresses; their products are dropped or zeroed
-    const unsigned char* wrow = (const unsigned char*)a.W + (long)min(max(c < 8 ? rc.base_lo + c : rc.base_hi + c - 8, 0), a.N - 1) * a.K * 2;
+    const unsigned char* wrow[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+        wrow[nb] = (const unsigned char*)a.W + (long)min(max(c < 8 ? rc[nb].base_lo + c : rc[nb].base_hi + c - 8, 0), a.N - 1) * a.K * 2;
     const unsigned char* xrow[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) xrow[rb] = (const unsigned char*)a.A + (long)min(rb * 16 + c, a.M - 1) * a.K * 2;
-    u32x4_t wf[MAXC], xf[MAXC][RB];
+    u32x4_t wf[MAXC][NB], xf[MAXC][RB];
 #pragma unroll
     for (int i = 0; i < MAXC; ++i) {
         const int ch = min(ch0 + i, nch - 1);
         const long off = (long)min(ch * 32 + 8 * q, a.K - 8) * 2;
-        wf[i] = *reinterpret_cast<const u32x4_t*>(wrow + off);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) wf[i][nb] = *reinterpret_cast<const u32x4_t*>(wrow[nb] + off);
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) xf[i][rb] = *reinterpret_cast<const u32x4_t*>(xrow[rb] + off);
     }
@@ -999,43 +1006,51 @@ __global__ void __launch_bounds__(SR_WAVES * 64) gemm_rows_bf16_kernel(GemmArgs 
     // addresses are clamped into the arrays and values that are not needed are dropped.
     const int erow = tid >> 3, ei = tid & 7;
     const int em = min(erow, a.M - 1);
-    const int n_lo = min(rc.base_lo + ei, a.N - 1), n_hi = min(rc.base_hi + ei, a.N - 1);
-    float b_lo = 0.f, b_hi = 0.f, cs_lo = 0.f, cs_hi = 0.f, g_lo = 1.f, g_hi = 1.f, rot_c = 1.f, rot_s = 0.f, r_lo = 0.f, r_hi = 0.f;
-    if (a.bias) {
-        b_lo = a.bias[n_lo];
-        b_hi = a.bias[n_hi];
-    }
-    if (kNorm == NORM_LAYER) {
-        cs_lo = a.colsum[n_lo];
-        cs_hi = a.colsum[n_hi];
-    }
-    if (kEpi == EPI_PLAIN) {
-        if (a.col_gate) {
-            g_lo = a.col_gate[n_lo];
-            g_hi = a.col_gate[n_hi];
+    int n_lo[NB], n_hi[NB];
+    float b_lo[NB], b_hi[NB], cs_lo[NB], cs_hi[NB], g_lo[NB], g_hi[NB], rot_c[NB], rot_s[NB], r_lo[NB], r_hi[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        n_lo[nb] = min(rc[nb].base_lo + ei, a.N - 1);
+        n_hi[nb] = min(rc[nb].base_hi + ei, a.N - 1);
+        b_lo[nb] = b_hi[nb] = cs_lo[nb] = cs_hi[nb] = r_lo[nb] = r_hi[nb] = rot_s[nb] = 0.f;
+        g_lo[nb] = g_hi[nb] = rot_c[nb] = 1.f;
+        if (a.bias) {
+            b_lo[nb] = a.bias[n_lo[nb]];
+            b_hi[nb] = a.bias[n_hi[nb]];
         }
-        if (a.residual) {
-            if (a.out_bf16) {
-                r_lo = bf2f(((const bf16_t*)a.residual)[(long)em * a.N + n_lo]);
-                r_hi = bf2f(((const bf16_t*)a.residual)[(long)em * a.N + n_hi]);
-            } else {
-                r_lo = ((const float*)a.residual)[(long)em * a.N + n_lo];
-                r_hi = ((const float*)a.residual)[(long)em * a.N + n_hi];
+        if (kNorm == NORM_LAYER) {
+            cs_lo[nb] = a.colsum[n_lo[nb]];
+            cs_hi[nb] = a.colsum[n_hi[nb]];
+        }
+        if (kEpi == EPI_PLAIN) {
+            if (a.col_gate) {
+                g_lo[nb] = a.col_gate[n_lo[nb]];
+                g_hi[nb] = a.col_gate[n_hi[nb]];
+            }
+            if (a.residual) {
+                if (a.out_bf16) {
+                    r_lo[nb] = bf2f(((const bf16_t*)a.residual)[(long)em * a.N + n_lo[nb]]);
+                    r_hi[nb] = bf2f(((const bf16_t*)a.residual)[(long)em * a.N + n_hi[nb]]);
+                } else {
+                    r_lo[nb] = ((const float*)a.residual)[(long)em * a.N + n_lo[nb]];
+                    r_hi[nb] = ((const float*)a.residual)[(long)em * a.N + n_hi[nb]];
+                }
             }
         }
-    }
-    if (kEpi == EPI_QKV && rc.rope) {
-        const int half = a.D >> 1;
-        const long ri = (long)(em % a.S) * half + (rc.col_lo % a.D) + ei;
-        rot_c = a.cos_t[ri];
-        rot_s = a.sin_t[ri];
+        if (kEpi == EPI_QKV && rc[nb].rope) {
+            const int half = a.D >> 1;
+            const long ri = (long)(em % a.S) * half + (rc[nb].col_lo % a.D) + ei;
+            rot_c[nb] = a.cos_t[ri];
+            rot_s[nb] = a.sin_t[ri];
+        }
     }
 
-    f32x4_t acc[RB];
+    f32x4_t acc[NB][RB];
     float ssq[RB], ssum[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-        acc[rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) acc[nb][rb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         ssq[rb] = ssum[rb] = 0.f;
     }
 #pragma unroll
@@ -1053,14 +1068,18 @@ __global__ void __launch_bounds__(SR_WAVES * 64) gemm_rows_bf16_kernel(GemmArgs 
                         if (kNorm == NORM_LAYER) ssum[rb] = add_pair_bf16x2(xv[e], ssum[rb]);
                     }
                 }
-                acc[rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf[i]), __builtin_bit_cast(bf16x8_t, xv), acc[rb], 0, 0, 0);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    acc[nb][rb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, wf[i][nb]), __builtin_bit_cast(bf16x8_t, xv),
+                                                                          acc[nb][rb], 0, 0, 0);
             }
         }
     }
-    // acc[rb][e]: tile column 4 q + e, row 16 rb + c
+    // acc[nb][rb][e]: column 4 q + e of tile nb, row 16 rb + c
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-        *reinterpret_cast<f32x4_t*>(&part[wave][rb * 16 + c][4 * q]) = acc[rb];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) *reinterpret_cast<f32x4_t*>(&part[wave][nb][rb * 16 + c][4 * q]) = acc[nb][rb];
         if (kNorm) {
             const float s2 = rows_sum(ssq[rb]), s1 = rows_sum(ssum[rb]);
             if (q == 0) {
@@ -1072,68 +1091,76 @@ __global__ void __launch_bounds__(SR_WAVES * 64) gemm_rows_bf16_kernel(GemmArgs 
     __syncthreads();
     if (erow >= RB * 16 || erow >= a.M) return;
     const int m = erow;
-    float lo = 0.f, hi = 0.f, sq = 0.f, sm = 0.f;
+    float sq = 0.f, sm = 0.f;
+    if (kNorm) {
 #pragma unroll
-    for (int w = 0; w < SR_WAVES; ++w) {
-        lo += part[w][erow][ei];
-        hi += part[w][erow][8 + ei];
-        if (kNorm) {
+        for (int w = 0; w < SR_WAVES; ++w) {
             sq += stat_part[w][erow][0];
             sm += stat_part[w][erow][1];
         }
     }
-    if (kNorm) {
-        const float inv_k = 1.0f / (float)a.K;
-        if (kNorm == NORM_LAYER) {
-            // sum_k (x - mean) rstd W[n][k] = rstd acc - (mean rstd) colsum[n]
-            const float mean = sm * inv_k;
-            const float f = rsqrtf(fmaxf(sq * inv_k - mean * mean, 0.f) + a.norm_eps);
-            const float ms = mean * f;
-            lo = lo * f - ms * cs_lo;
-            hi = hi * f - ms * cs_hi;
-        } else {
-            const float f = rsqrtf(sq * inv_k + a.norm_eps);
-            lo *= f;
-            hi *= f;
-        }
-    }
-    lo += b_lo;
-    hi += b_hi;
-    const bool ok_lo = rc.base_lo + ei < a.N, ok_hi = rc.base_hi + ei < a.N;
-    if (kEpi == EPI_PLAIN) {
-        if (a.act != VLA_ACT_NONE) {
-            lo = apply_act(lo, a.act);
-            hi = apply_act(hi, a.act);
-        }
-        lo = lo * g_lo + r_lo;
-        hi = hi * g_hi + r_hi;
-        const long o = (long)m * a.N;
-        if (a.out_bf16) {
-            if (ok_lo) ((bf16_t*)a.Y)[o + n_lo] = f2bf(lo);
-            if (ok_hi) ((bf16_t*)a.Y)[o + n_hi] = f2bf(hi);
-        } else {
-            if (ok_lo) ((float*)a.Y)[o + n_lo] = lo;
-            if (ok_hi) ((float*)a.Y)[o + n_hi] = hi;
-        }
-        return;
-    }
-    // QKV: rotation, scatter
-    if (rc.rope) {
-        const float x0 = lo, x1 = hi;
-        lo = x0 * rot_c - x1 * rot_s;
-        hi = x1 * rot_c + x0 * rot_s;
-    }
-    const int b = m / a.S, s = m % a.S;
+    const int b = kEpi == EPI_QKV ? m / a.S : 0, s = kEpi == EPI_QKV ? m % a.S : 0;
 #pragma unroll
-    for (int hlf = 0; hlf < 2; ++hlf) {
-        const float v = hlf ? hi : lo;
-        const int col = (hlf ? rc.col_hi : rc.col_lo) + ei;
-        if (rc.seg == 0) {
-            ((bf16_t*)a.q_out)[(long)m * (a.Hq * a.D) + col] = f2bf(v);
-        } else {
-            const int head = col / a.D, d = col % a.D;
-            if (rc.seg == 1) ((bf16_t*)a.k_cache)[(((long)b * a.Hkv + head) * a.t_max + a.tok_offset + s) * a.D + d] = f2bf(v);
-            else ((bf16_t*)a.vt_cache)[(((long)b * a.Hkv + head) * a.D + d) * (long)a.t_max + a.tok_offset + s] = f2bf(v);
+    for (int nb = 0; nb < NB; ++nb) {
+        if ((int)blockIdx.x * NB + nb >= n_t16) break;  // uniform
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int w = 0; w < SR_WAVES; ++w) {
+            lo += part[w][nb][erow][ei];
+            hi += part[w][nb][erow][8 + ei];
+        }
+        if (kNorm) {
+            const float inv_k = 1.0f / (float)a.K;
+            if (kNorm == NORM_LAYER) {
+                // sum_k (x - mean) rstd W[n][k] = rstd acc - (mean rstd) colsum[n]
+                const float mean = sm * inv_k;
+                const float f = rsqrtf(fmaxf(sq * inv_k - mean * mean, 0.f) + a.norm_eps);
+                const float ms = mean * f;
+                lo = lo * f - ms * cs_lo[nb];
+                hi = hi * f - ms * cs_hi[nb];
+            } else {
+                const float f = rsqrtf(sq * inv_k + a.norm_eps);
+                lo *= f;
+                hi *= f;
+            }
+        }
+        lo += b_lo[nb];
+        hi += b_hi[nb];
+        const bool ok_lo = rc[nb].base_lo + ei < a.N, ok_hi = rc[nb].base_hi + ei < a.N;
+        if (kEpi == EPI_PLAIN) {
+            if (a.act != VLA_ACT_NONE) {
+                lo = apply_act(lo, a.act);
+                hi = apply_act(hi, a.act);
+            }
+            lo = lo * g_lo[nb] + r_lo[nb];
+            hi = hi * g_hi[nb] + r_hi[nb];
+            const long o = (long)m * a.N;
+            if (a.out_bf16) {
+                if (ok_lo) ((bf16_t*)a.Y)[o + n_lo[nb]] = f2bf(lo);
+                if (ok_hi) ((bf16_t*)a.Y)[o + n_hi[nb]] = f2bf(hi);
+            } else {
+                if (ok_lo) ((float*)a.Y)[o + n_lo[nb]] = lo;
+                if (ok_hi) ((float*)a.Y)[o + n_hi[nb]] = hi;
+            }
+            continue;
+        }
+        // QKV: rotation, scatter
+        if (rc[nb].rope) {
+            const float x0 = lo, x1 = hi;
+            lo = x0 * rot_c[nb] - x1 * rot_s[nb];
+            hi = x1 * rot_c[nb] + x0 * rot_s[nb];
+        }
+#pragma unroll
+        for (int hlf = 0; hlf < 2; ++hlf) {
+            const float v = hlf ? hi : lo;
+            const int col = (hlf ? rc[nb].col_hi : rc[nb].col_lo) + ei;
+            if (rc[nb].seg == 0) {
+                ((bf16_t*)a.q_out)[(long)m * (a.Hq * a.D) + col] = f2bf(v);
+            } else {
+                const int head = col / a.D, d = col % a.D;
+                if (rc[nb].seg == 1) ((bf16_t*)a.k_cache)[(((long)b * a.Hkv + head) * a.t_max + a.tok_offset + s) * a.D + d] = f2bf(v);
+                else ((bf16_t*)a.vt_cache)[(((long)b * a.Hkv + head) * a.D + d) * (long)a.t_max + a.tok_offset + s] = f2bf(v);
+            }
         }
     }
 }
@@ -2056,20 +2083,25 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
                        tuning().gemm_tile < 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0 && !(a.colsum && a.norm_eps < 0.f);
         if (kEpi == EPI_QKV) rows_ok = rows_ok && a.D % 16 == 0 && a.N % 16 == 0;
         if (rows_ok) {
-            const unsigned grid = (unsigned)((a.N + 15) / 16);
-            const int per = ((a.K + 31) / 32 + SR_WAVES - 1) / SR_WAVES, rb = (a.M + 15) / 16;
-#define VLA_ROWS_K(NORM, RB)                                                                                       \
+            // more 16-column tiles than CUs: two per workgroup, so that no CU gets two workgroups' worth of requests while
+            // its neighbours get one (GR00T's fused Q | K | V: 288 tiles).  Up to 32 rows only (registers).
+            const int n_t16 = (a.N + 15) / 16, per = ((a.K + 31) / 32 + SR_WAVES - 1) / SR_WAVES, rb = (a.M + 15) / 16;
+            const bool two = n_t16 > 256 && rb <= 2 && per <= 6;
+            const unsigned grid = (unsigned)(two ? (n_t16 + 1) / 2 : n_t16);
+#define VLA_ROWS_K(NORM, RB, NB)                                                                                   \
     do {                                                                                                           \
-        if (per <= 2) gemm_rows_bf16_kernel<kEpi, NORM, RB, 2><<<grid, SR_WAVES * 64, 0, st>>>(a);                  \
-        else if (per <= 4) gemm_rows_bf16_kernel<kEpi, NORM, RB, 4><<<grid, SR_WAVES * 64, 0, st>>>(a);             \
-        else if (per <= 6) gemm_rows_bf16_kernel<kEpi, NORM, RB, 6><<<grid, SR_WAVES * 64, 0, st>>>(a);             \
-        else gemm_rows_bf16_kernel<kEpi, NORM, RB, 8><<<grid, SR_WAVES * 64, 0, st>>>(a);                           \
+        if (per <= 2) gemm_rows_bf16_kernel<kEpi, NORM, RB, 2, NB><<<grid, SR_WAVES * 64, 0, st>>>(a);              \
+        else if (per <= 4) gemm_rows_bf16_kernel<kEpi, NORM, RB, 4, NB><<<grid, SR_WAVES * 64, 0, st>>>(a);         \
+        else if (per <= 6) gemm_rows_bf16_kernel<kEpi, NORM, RB, 6, NB><<<grid, SR_WAVES * 64, 0, st>>>(a);         \
+        else if (NB == 1) gemm_rows_bf16_kernel<kEpi, NORM, RB, 8, 1><<<grid, SR_WAVES * 64, 0, st>>>(a);           \
     } while (0)
-#define VLA_ROWS(NORM)                       \
-    do {                                     \
-        if (rb <= 1) VLA_ROWS_K(NORM, 1);    \
-        else if (rb == 2) VLA_ROWS_K(NORM, 2); \
-        else VLA_ROWS_K(NORM, 4);            \
+#define VLA_ROWS(NORM)                                \
+    do {                                              \
+        if (two && rb <= 1) VLA_ROWS_K(NORM, 1, 2);   \
+        else if (two) VLA_ROWS_K(NORM, 2, 2);         \
+        else if (rb <= 1) VLA_ROWS_K(NORM, 1, 1);     \
+        else if (rb == 2) VLA_ROWS_K(NORM, 2, 1);     \
+        else VLA_ROWS_K(NORM, 4, 1);                  \
     } while (0)
             if (a.norm_eps < 0.f) {
                 VLA_ROWS(NORM_NONE);
