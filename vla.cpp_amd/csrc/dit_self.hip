@@ -75,7 +75,8 @@ template <int NR, int NC>
 __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* lds, const unsigned char* const (&ap)[5],
                                             const unsigned char* const (&wp)[5], uint32_t lds0, int koff, bool tail, int wm, int wn,
                                             int c, int q, f32x4_t (&acc)[5][5], float (&ssq)[5], float (&ssum)[5]) {
-    constexpr bool STATS = NC == 5;  // the wavefronts with block column 0: one per row half
+    // row sums: the two wavefronts that multiply the same rows (block columns 0 and 1) take alternate 32-k chunks
+    constexpr int STATS_SET = NC == 5 ? 0 : 1;
     const int fsw = (c >> 1) & 7;
     auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
         const long kb = ((long)kt * 64 + koff) * 2;
@@ -106,7 +107,7 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
             for (int j = 0; j < NC; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fa[set][i]),
                                                                   __builtin_bit_cast(bf16x8_t, fw[set][j]), acc[i][j], 0, 0, 0);
-        if (STATS) {
+        if (set == STATS_SET) {  // a constant at both call sites
 #pragma unroll
             for (int i = 0; i < NR; ++i)
 #pragma unroll
@@ -138,6 +139,7 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
         for (int g = 0; g < NR + NC; ++g) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
             __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // MFMA
+            if (STATS_SET == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // the chunk's row sums, spread between the MFMAs
         }
         __builtin_amdgcn_sched_barrier(0);
         // tile kt + 1 has landed; up to two younger tiles may still be on their way (none past the last)
@@ -159,6 +161,7 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
         for (int g = 0; g < NR + NC; ++g) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
             __builtin_amdgcn_sched_group_barrier(0x008, 2, 1);
+            if (STATS_SET == 1) __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);
         }
         __builtin_amdgcn_sched_barrier(0);
         st = nx;
@@ -224,14 +227,14 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     // ---- the tile leaves the accumulators: row statistics first
     bf16_t* qk = reinterpret_cast<bf16_t*>(lds);                                        // [FS_ROWS][FS_QS]: q | k
     bf16_t* vt = qk + FS_ROWS * FS_QS;                                                  // [OB][FS_D][FS_VS]: V^T per observation
-    float* stat = reinterpret_cast<float*>(lds + (FS_ROWS * FS_QS + FS_MAX_OB * FS_D * FS_VS) * 2);  // [FS_ROWS][2]: (sum of squares, sum)
+    float* stat = reinterpret_cast<float*>(lds + (FS_ROWS * FS_QS + FS_MAX_OB * FS_D * FS_VS) * 2);  // [2][FS_ROWS][2]: (sum of squares, sum), a partial pair from each of a row's two wavefronts
 #pragma unroll
     for (int i = 0; i < 5; ++i) {
         const float s2 = rows_sum(ssq[i]), s1 = rows_sum(ssum[i]);
         const int rb = wm + 2 * i;
-        if (q == 0 && i < nr && wn == 0) {
-            stat[(rb * 16 + c) * 2] = s2;
-            stat[(rb * 16 + c) * 2 + 1] = s1;
+        if (q == 0 && i < nr) {  // one partial pair per wavefront of the row's two
+            stat[(wn * FS_ROWS + rb * 16 + c) * 2] = s2;
+            stat[(wn * FS_ROWS + rb * 16 + c) * 2 + 1] = s1;
         }
     }
     // keys past S of every V^T row are multiplied by probabilities that are zero: they must be finite
@@ -250,7 +253,7 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int row = rb * 16 + 4 * q + e;
-            const float s2 = stat[row * 2], s1 = stat[row * 2 + 1];
+            const float s2 = stat[row * 2] + stat[(FS_ROWS + row) * 2], s1 = stat[row * 2 + 1] + stat[(FS_ROWS + row) * 2 + 1];
             const float mean = s1 * inv_k;
             const float rstd = rsqrtf(fmaxf(s2 * inv_k - mean * mean, 0.f) + a.eps);
             const float ms = mean * rstd;
