@@ -207,7 +207,32 @@ VLA_KAPI int vla_layernorm_qkv_self_attention(const void* x, const void* W_folde
                                               int dtype, int M, int K, int S, int n_heads, int head_dim, float scale,
                                               float ln_eps, void* out, vla_stream_t stream);
 
-/* Host helper for the two calls above (bf16 weights [N][K], fp32 scale/shift [K], fp32 bias [N]
+/* Row sums handed from the launch that writes a row to the launch that normalises it (no
+ * counterpart in the reference, whose norm is a graph node of its own, src/layers/norm.h:31-48).
+ * A DiT block's LayerNorm needs (sum, sum of squares) of every row of h; taken inside the
+ * projection launch they are summed again by each of the launch's column tiles, from operand
+ * fragments, on the critical path of its K walk.  The output projection of the block before
+ * has each value of the row in a register when it writes it:
+ *   vla_linear_row_stats = vla_linear for bf16 rows and bf16 output (N a multiple of 64) that
+ *     also leaves row_stats [M][N / 64][2] fp32: (sum of squares, sum) of the 64 values, as
+ *     written (rounded to bf16), of each (row, 64-column tile);
+ *   vla_layernorm_attn_qkv_rope_stats / vla_layernorm_qkv_self_attention_stats = the two calls
+ *     above with the LayerNorm's row sums added up from row_stats [M][n_stat_tiles][2] of their
+ *     input x (n_stat_tiles = K / 64 <= 24) instead of from x itself.
+ * The sums are added in another order than inside the launches: agreement to fp32 rounding. */
+VLA_KAPI int vla_linear_row_stats(const void* x, const void* W, const float* bias, const void* residual, void* y,
+                                  float* row_stats, int dtype, int M, int N, int K, vla_stream_t stream);
+VLA_KAPI int vla_layernorm_attn_qkv_rope_stats(const void* x, const void* W_folded, const float* colsum, const float* bias,
+                                               const float* row_stats, int n_stat_tiles, int dtype, int M, int K, int S,
+                                               int n_q_heads, int n_kv_heads, int has_k, int has_v, int head_dim,
+                                               const float* cos_tab, const float* sin_tab, void* q_out, void* k_cache,
+                                               void* vt_cache, int t_max, int tok_offset, float ln_eps, vla_stream_t stream);
+VLA_KAPI int vla_layernorm_qkv_self_attention_stats(const void* x, const void* W_folded, const float* colsum,
+                                                    const float* bias, const float* row_stats, int n_stat_tiles, int dtype,
+                                                    int M, int K, int S, int n_heads, int head_dim, float scale, float ln_eps,
+                                                    void* out, vla_stream_t stream);
+
+/* Host helper for the LayerNorm-inside calls above (bf16 weights [N][K], fp32 scale/shift [K], fp32 bias [N]
  * or NULL): writes W_out (bf16, rounded to nearest even; may alias W), colsum_out and
  * bias_out (fp32 [N]); colsum is taken over the rounded W_out, the values the launch
  * multiplies. */

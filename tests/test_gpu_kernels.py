@@ -574,6 +574,76 @@ def test_dit_self_block_front_half_in_one_launch(B, S, H, K, bias):
                                                       eps, fused.data_ptr(), None) == pkg.VLA_K_ERR_SHAPE
 
 
+@pytest.mark.parametrize("B,S,H,K", [(64, 17, 32, 1536), (5, 17, 8, 1536), (40, 9, 8, 512)])
+def test_row_sums_handed_from_the_output_projection_to_the_next_layernorm(B, S, H, K):
+    """A block's output projection leaves (sum of squares, sum) of the rows it writes, per 64-column
+    tile; the next block's projection launches (LayerNorm inside) add those up instead of summing the
+    rows themselves.  The sums against numpy on the bf16 values written; both consumers with the
+    handed-over sums against the same launches without them (another order of the same sums) and
+    against the oracle."""
+    D = 48
+    r = np.random.default_rng(9100 + B + K)
+    M, Kin = B * S, H * D
+    att = orc.round_bf16(r.standard_normal((M, Kin)).astype(np.float32))
+    Wo = orc.round_bf16((0.03 * r.standard_normal((K, Kin))).astype(np.float32))
+    bo = (0.1 * r.standard_normal(K)).astype(np.float32)
+    h0 = orc.round_bf16((2.0 * r.standard_normal((M, K)) + 1.5 * r.standard_normal((M, 1))).astype(np.float32))
+    nt = K // 64
+    h = to_dev(h0, BF16)
+    stats = torch.zeros((M, nt, 2), dtype=torch.float32, device="cuda")
+    pkg.call("vla_linear_row_stats", to_dev(att, BF16), to_dev(Wo, BF16), dev(bo), h, h, stats, BF16, M, K, Kin)
+    h_ref = to_dev(h0, BF16)
+    pkg.call("vla_linear", to_dev(att, BF16), to_dev(Wo, BF16), dev(bo), h_ref, h_ref, BF16, BF16, M, K, Kin)
+    sync()
+    hv = as_f32(h, BF16)
+    assert np.array_equal(hv, as_f32(h_ref, BF16))  # the same projection
+    st = host(stats)
+    tiles = hv.reshape(M, nt, 64).astype(np.float64)
+    assert np.allclose(st[:, :, 1], tiles.sum(-1), rtol=1e-5, atol=1e-4)
+    assert np.allclose(st[:, :, 0], (tiles * tiles).sum(-1), rtol=1e-5, atol=1e-4)
+
+    sc, sh = (0.3 * r.standard_normal(K)).astype(np.float32), (0.3 * r.standard_normal(K)).astype(np.float32)
+    eps = 1e-5
+    scale = 1.0 / np.sqrt(D)
+
+    def folded(W, b):
+        N = W.shape[0]
+        Wf, cs, bs = np.empty((N, K), np.uint16), np.empty(N, np.float32), np.empty(N, np.float32)
+        assert pkg.lib().vla_fold_adaln_weight_host(orc.to_bf16(W).ctypes.data, b.ctypes.data, sc.ctypes.data, sh.ctypes.data, N, K,
+                                                    Wf.ctypes.data, cs.ctypes.data, bs.ctypes.data) == 0
+        return dev(Wf), dev(cs), dev(bs)
+
+    # cross block: Q projection
+    Wq = orc.round_bf16((0.02 * r.standard_normal((H * D, K))).astype(np.float32))
+    bq = (0.1 * r.standard_normal(H * D)).astype(np.float32)
+    Wf, cs, bs = folded(Wq, bq)
+    q1, q2 = empty((M, H * D), BF16), empty((M, H * D), BF16)
+    pkg.call("vla_layernorm_attn_qkv_rope_stats", h, Wf, cs, bs, stats, nt, BF16, M, K, S, H, H, 0, 0, D, None, None, q1, None, None, 64, 0, eps)
+    pkg.call("vla_layernorm_attn_qkv_rope", h, Wf, cs, bs, BF16, M, K, S, H, H, 0, 0, D, None, None, q2, None, None, 64, 0, eps)
+    sync()
+    want = orc.linear(orc.adaln(hv, sc, sh, eps), Wq, bq)
+    g1, g2 = as_f32(q1, BF16), as_f32(q2, BF16)
+    assert bf16_close(g1, want) and rel_err(g1, want) < 8e-3 and rel_err(g1, g2) < 8e-3
+    # self block in one launch (its own shape limits: heads in eights, K >= 256)
+    W3 = orc.round_bf16((0.02 * r.standard_normal((3 * H * D, K))).astype(np.float32))
+    b3 = (0.1 * r.standard_normal(3 * H * D)).astype(np.float32)
+    Wf, cs, bs = folded(W3, b3)
+    o1, o2 = empty((M, H * D), BF16), empty((M, H * D), BF16)
+    pkg.call("vla_layernorm_qkv_self_attention_stats", h, Wf, cs, bs, stats, nt, BF16, M, K, S, H, D, scale, eps, o1)
+    pkg.call("vla_layernorm_qkv_self_attention", h, Wf, cs, bs, BF16, M, K, S, H, D, scale, eps, o2)
+    sync()
+    y = orc.round_bf16(orc.linear(orc.adaln(hv, sc, sh, eps), W3, b3))
+    qkv = y.reshape(B, S, 3, H, D)
+    want = np.stack([orc.attention(qkv[b, :, 0], qkv[b, :, 1], qkv[b, :, 2], np.zeros((S, S), np.float32), scale).reshape(S, H * D)
+                     for b in range(B)]).reshape(M, H * D)
+    g1, g2 = as_f32(o1, BF16), as_f32(o2, BF16)
+    assert rel_err(g1, want) < 8e-3 and rel_err(g1, g2) < 8e-3  # one bf16 ulp
+    # what the hand-over does not take
+    assert pkg.lib().vla_linear_row_stats(h.data_ptr(), Wf.data_ptr(), None, None, h.data_ptr(), stats.data_ptr(), BF16, M, 72, K, None) == pkg.VLA_K_ERR_SHAPE
+    assert pkg.lib().vla_layernorm_attn_qkv_rope_stats(h.data_ptr(), Wf.data_ptr(), cs.data_ptr(), None, stats.data_ptr(), nt + 1, BF16, M, K, S, H, H,
+                                                       0, 0, D, None, None, q1.data_ptr(), None, None, 64, 0, eps, None) == pkg.VLA_K_ERR_SHAPE
+
+
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("M,I,K,act,bias", [(50, 2048, 720, "silu", False), (130, 96, 72, "gelu", True), (1600, 256, 720, "silu", False),
                                            (17, 6144, 1536, "gelu", True)])

@@ -47,6 +47,7 @@ constexpr int FS_QS = 104;          // bf16 per row of the Q | K tile in LDS (20
 constexpr int FS_VS = 36;           // bf16 per row of a V^T tile: 32 keys and padding (72 bytes)
 constexpr int FS_MAX_S = 32;        // tokens per observation: two 16-wide MFMA blocks
 constexpr int FS_MAX_OB = 8;        // observations per workgroup (V^T tiles held in LDS)
+constexpr int FS_MAX_STAT = 24;     // 64-column tiles of x whose handed-over row sums a row adds up (K <= 1536)
 
 struct SelfArgs {
     const bf16_t* x;
@@ -56,6 +57,8 @@ struct SelfArgs {
     bf16_t* out;
     int M, K, S, H, OB;
     float scale, eps;
+    const float* stats_in;  // (sum of squares, sum) per (row, 64-column tile of x) from the launch that wrote x, or null
+    int n_stat;
 };
 
 __device__ __forceinline__ float sum_squares_bf16x2(uint32_t u, float acc) {
@@ -71,12 +74,13 @@ __device__ __forceinline__ float sum_pair_bf16x2(uint32_t u, float acc) {
 // Straight-line per (NR, NC): the four wavefronts of a workgroup fall into four classes and each
 // runs its own copy, so no block is computed twice and none sits behind a branch (a branch
 // inside the loop body cuts it into pieces the scheduler cannot interleave).
-template <int NR, int NC>
+template <int NR, int NC, bool PRE>
 __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* lds, const unsigned char* const (&ap)[5],
                                             const unsigned char* const (&wp)[5], uint32_t lds0, int koff, bool tail, int wm, int wn,
                                             int c, int q, f32x4_t (&acc)[5][5], float (&ssq)[5], float (&ssum)[5]) {
     // row sums: the two wavefronts that multiply the same rows (block columns 0 and 1) take alternate 32-k chunks
-    constexpr int STATS_SET = NC == 5 ? 0 : 1;
+    // (PRE: the sums come from the launch that wrote the rows: no chunk takes them)
+    constexpr int STATS_SET = PRE ? 7 : NC == 5 ? 0 : 1;
     const int fsw = (c >> 1) & 7;
     auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
         const long kb = ((long)kt * 64 + koff) * 2;
@@ -169,6 +173,7 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
     wait_vmcnt<0>();
 }
 
+template <bool PRE>
 __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[FS_NS * FS_STAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -216,11 +221,25 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     float ssq[5] = {0.f, 0.f, 0.f, 0.f, 0.f}, ssum[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
     const int nr = wm == 0 ? 5 : 4, nc = wn == 0 ? 5 : 4;
     if (wm == 0) {
-        if (wn == 0) self_k_walk<5, 5>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
-        else self_k_walk<5, 4>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+        if (wn == 0) self_k_walk<5, 5, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+        else self_k_walk<5, 4, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
     } else {
-        if (wn == 0) self_k_walk<4, 5>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
-        else self_k_walk<4, 4>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+        if (wn == 0) self_k_walk<4, 5, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+        else self_k_walk<4, 4, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
+    }
+    // PRE: this thread's row of the tile (threads 0 .. 143) and its handed-over sums, requested before the barrier
+    // and added up behind it (the consumer of x's row sums reads 24 pairs per row; they come from L2)
+    float pre_q = 0.f, pre_u = 0.f;
+    if (PRE && tid < FS_ROWS) {
+        const float* sp = a.stats_in + (long)min(m0 + tid, a.M - 1) * a.n_stat * 2;
+        f32x2_t pv[FS_MAX_STAT];  // one trip: every pair requested before the first is added (the fragment registers are free by now)
+#pragma unroll
+        for (int t = 0; t < FS_MAX_STAT; ++t) pv[t] = *reinterpret_cast<const f32x2_t*>(sp + 2 * min(t, a.n_stat - 1));
+#pragma unroll
+        for (int t = 0; t < FS_MAX_STAT; ++t) {
+            pre_q += t < a.n_stat ? pv[t][0] : 0.f;
+            pre_u += t < a.n_stat ? pv[t][1] : 0.f;
+        }
     }
     __syncthreads();
 
@@ -232,10 +251,16 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     for (int i = 0; i < 5; ++i) {
         const float s2 = rows_sum(ssq[i]), s1 = rows_sum(ssum[i]);
         const int rb = wm + 2 * i;
-        if (q == 0 && i < nr) {  // one partial pair per wavefront of the row's two
+        if (!PRE && q == 0 && i < nr) {  // one partial pair per wavefront of the row's two
             stat[(wn * FS_ROWS + rb * 16 + c) * 2] = s2;
             stat[(wn * FS_ROWS + rb * 16 + c) * 2 + 1] = s1;
         }
+    }
+    if (PRE && tid < FS_ROWS) {  // the totals as the first partial pair, zeros as the second
+        stat[tid * 2] = pre_q;
+        stat[tid * 2 + 1] = pre_u;
+        stat[(FS_ROWS + tid) * 2] = 0.f;
+        stat[(FS_ROWS + tid) * 2 + 1] = 0.f;
     }
     // keys past S of every V^T row are multiplied by probabilities that are zero: they must be finite
     const int S = a.S;
@@ -370,18 +395,35 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
 }  // namespace
 }  // namespace vk
 
-extern "C" VLA_KAPI int vla_layernorm_qkv_self_attention(const void* x, const void* W_folded, const float* colsum, const float* bias,
-                                                int dtype, int M, int K, int S, int n_heads, int head_dim, float scale,
-                                                float ln_eps, void* out, vla_stream_t stream) {
+static int self_block_impl(const void* x, const void* W_folded, const float* colsum, const float* bias, const float* row_stats,
+                           int n_stat_tiles, int dtype, int M, int K, int S, int n_heads, int head_dim, float scale, float ln_eps,
+                           void* out, vla_stream_t stream) {
     using namespace vk;
     if (!x || !W_folded || !colsum || !out || M < 0 || K <= 0 || S <= 0 || n_heads <= 0) return VLA_K_ERR_ARG;
     if (dtype != VLA_DT_BF16 || head_dim != FS_D || S > FS_MAX_S || M % S || K % 64 || K < 64 * FS_NS || n_heads % 8) return VLA_K_ERR_SHAPE;
     if (((uintptr_t)x | (uintptr_t)W_folded | (uintptr_t)out) & 15) return VLA_K_ERR_SHAPE;
+    if (row_stats && (n_stat_tiles < 1 || n_stat_tiles > FS_MAX_STAT || n_stat_tiles * 64 != K || ((uintptr_t)row_stats & 7))) return VLA_K_ERR_SHAPE;
     if (M == 0) return VLA_K_OK;
     SelfArgs a;
     a.x = (const bf16_t*)x; a.W = (const bf16_t*)W_folded; a.colsum = colsum; a.bias = bias; a.out = (bf16_t*)out;
     a.M = M; a.K = K; a.S = S; a.H = n_heads; a.OB = FS_ROWS / S < FS_MAX_OB ? FS_ROWS / S : FS_MAX_OB; a.scale = scale; a.eps = ln_eps;
+    a.stats_in = row_stats; a.n_stat = n_stat_tiles;
     const int n_obs = M / S, groups = (n_obs + a.OB - 1) / a.OB;
-    dit_self_block_kernel<<<(unsigned)(groups * n_heads), 256, 0, (hipStream_t)stream>>>(a);
+    if (row_stats) dit_self_block_kernel<true><<<(unsigned)(groups * n_heads), 256, 0, (hipStream_t)stream>>>(a);
+    else dit_self_block_kernel<false><<<(unsigned)(groups * n_heads), 256, 0, (hipStream_t)stream>>>(a);
     return hipGetLastError() == hipSuccess ? VLA_K_OK : VLA_K_ERR_LAUNCH;
+}
+
+extern "C" VLA_KAPI int vla_layernorm_qkv_self_attention(const void* x, const void* W_folded, const float* colsum, const float* bias,
+                                                int dtype, int M, int K, int S, int n_heads, int head_dim, float scale,
+                                                float ln_eps, void* out, vla_stream_t stream) {
+    return self_block_impl(x, W_folded, colsum, bias, nullptr, 0, dtype, M, K, S, n_heads, head_dim, scale, ln_eps, out, stream);
+}
+
+extern "C" VLA_KAPI int vla_layernorm_qkv_self_attention_stats(const void* x, const void* W_folded, const float* colsum, const float* bias,
+                                                      const float* row_stats, int n_stat_tiles, int dtype, int M, int K, int S,
+                                                      int n_heads, int head_dim, float scale, float ln_eps, void* out,
+                                                      vla_stream_t stream) {
+    if (!row_stats) return VLA_K_ERR_ARG;
+    return self_block_impl(x, W_folded, colsum, bias, row_stats, n_stat_tiles, dtype, M, K, S, n_heads, head_dim, scale, ln_eps, out, stream);
 }

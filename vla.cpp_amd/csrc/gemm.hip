@@ -38,7 +38,8 @@ constexpr int BN = 64;                     // epilogue sub-tile; column-tile uni
 constexpr int C_STRIDE = BN + 4;           // floats
 
 enum { EPI_PLAIN = 0, EPI_QKV = 1, EPI_TERNARY = 2, EPI_GLU = 3 };
-enum { NORM_NONE = 0, NORM_RMS = 1, NORM_LAYER = 2 };  // row statistics taken inside gemm_dl_kernel
+enum { NORM_NONE = 0, NORM_RMS = 1, NORM_LAYER = 2, NORM_LAYER_PRE = 3 };  // row statistics taken inside gemm_dl_kernel (PRE: LayerNorm from sums handed over by the producing launch)
+constexpr int STAT_MAX_TILES = 24;  // 64-column tiles of a row whose sums a consumer adds up (four threads per row, six pairs each)
 
 struct GemmArgs {
     const void* A;
@@ -71,6 +72,13 @@ struct GemmArgs {
     float norm_eps;
     const float* colsum;
     const void* norm_w;  // ternary GEMV with the RMSNorm and quantisation of its rows inside: A is bf16, this the norm weight
+    // Row statistics handed from the launch that writes a row to the launch that normalises it: a PLAIN
+    // launch with bf16 output leaves (sum of squares, sum) of the 64 values it wrote per (row, 64-column
+    // tile) in stats_out [M][N / 64][2]; a QKV launch with the LayerNorm inside adds up the n_stat pairs
+    // of a row from stats_in instead of summing the row from its operand tiles.
+    float* stats_out;
+    const float* stats_in;
+    int n_stat;
 };
 
 // Workgroup -> tile.  Workgroup i runs on XCD i % 8; the XCDs form an xm x xn grid over the
@@ -202,6 +210,19 @@ __device__ __forceinline__ TileCols tile_cols(const GemmArgs& a, int nt) {
     return t;
 }
 
+// acc + lo^2 + hi^2 of the two bf16 values packed in u (taken by value: a bit_cast applied
+// directly to a vector element expression reads element 0).
+__device__ __forceinline__ float add_squares_bf16x2(uint32_t u, float acc) {
+    const bf16x2_t v = __builtin_bit_cast(bf16x2_t, u);
+    return __builtin_amdgcn_fdot2_f32_bf16(v, v, acc, false);
+}
+// acc + lo + hi
+__device__ __forceinline__ float add_pair_bf16x2(uint32_t u, float acc) {
+    const bf16x2_t v = __builtin_bit_cast(bf16x2_t, u);
+    const bf16x2_t ones = __builtin_bit_cast(bf16x2_t, 0x3f803f80u);
+    return __builtin_amdgcn_fdot2_f32_bf16(v, ones, acc, false);
+}
+
 // Epilogue of one 64x64 sub-tile held in the LDS C tile: thread t owns row t/4 and
 // columns jg..jg+7 and 32+jg..32+jg+7 of the sub-tile.
 __device__ const float kNoBiasRegs[16] = {};
@@ -296,6 +317,7 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
     }
 
     if (kEpi == EPI_PLAIN) {
+        float st1 = 0.f, st2 = 0.f;  // sum and sum of squares of the 16 values this thread writes (as written: rounded to bf16)
 #pragma unroll
         for (int hlf = 0; hlf < 2; ++hlf) {
             const int n0 = nt * BN + hlf * 32 + jg;
@@ -337,6 +359,13 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
                 }
                 const u32x4_t pk = {pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3]), pack_bf2(v[4], v[5]), pack_bf2(v[6], v[7])};
                 *reinterpret_cast<u32x4_t*>((bf16_t*)a.Y + o) = pk;
+                if (a.stats_out) {  // two bf16 values per instruction, exact products, fp32 sums
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        st1 = add_pair_bf16x2(pk[e], st1);
+                        st2 = add_squares_bf16x2(pk[e], st2);
+                    }
+                }
             } else if (full) {
                 if (a.residual) {
 #pragma unroll
@@ -365,6 +394,14 @@ __device__ __forceinline__ void epilogue_64x64(const GemmArgs& a, const uint32_t
                     }
                 }
             }
+        }
+        if (a.stats_out) {
+            // the four threads of a row (tid % 4) are neighbouring lanes: the row's 64 values of this tile
+            st1 += __uint_as_float(dpp_u32<DPP_XOR1>(__float_as_uint(st1)));
+            st2 += __uint_as_float(dpp_u32<DPP_XOR1>(__float_as_uint(st2)));
+            st1 += __uint_as_float(dpp_u32<DPP_XOR2>(__float_as_uint(st1)));
+            st2 += __uint_as_float(dpp_u32<DPP_XOR2>(__float_as_uint(st2)));
+            if ((tid & 3) == 0) *reinterpret_cast<f32x2_t*>(a.stats_out + ((long)m * (a.N / BN) + nt) * 2) = f32x2_t{st2, st1};
         }
         return;
     }
@@ -664,19 +701,6 @@ __global__ void __launch_bounds__(256) gemm_kernel(GemmArgs a) {
         }
 }
 
-// acc + lo^2 + hi^2 of the two bf16 values packed in u (taken by value: a bit_cast applied
-// directly to a vector element expression reads element 0).
-__device__ __forceinline__ float add_squares_bf16x2(uint32_t u, float acc) {
-    const bf16x2_t v = __builtin_bit_cast(bf16x2_t, u);
-    return __builtin_amdgcn_fdot2_f32_bf16(v, v, acc, false);
-}
-// acc + lo + hi
-__device__ __forceinline__ float add_pair_bf16x2(uint32_t u, float acc) {
-    const bf16x2_t v = __builtin_bit_cast(bf16x2_t, u);
-    const bf16x2_t ones = __builtin_bit_cast(bf16x2_t, 0x3f803f80u);
-    return __builtin_amdgcn_fdot2_f32_bf16(v, ones, acc, false);
-}
-
 // ---- bf16 GEMM with operand tiles loaded straight into LDS --------------------------
 // Same tiling, wavefront layout, XCD mapping and epilogues as gemm_kernel, for bf16
 // operands with K a multiple of 16.  A stage of the LDS ring holds one k-tile of A and W
@@ -758,6 +782,18 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
                 }
     }
 
+    // NORM_LAYER_PRE: the row sums handed over by the producing launch, six (sum of squares, sum) pairs per thread
+    // and tile row (the four threads of a row take the tiles t % 4), requested ahead of the operand loads as well.
+    f32x2_t st_pf[TM][STAT_MAX_TILES / 4] = {};
+    if (kNorm == NORM_LAYER_PRE) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const float* sp = a.stats_in + (long)min(m0 + i * 64 + (tid >> 2), a.M - 1) * a.n_stat * 2;
+#pragma unroll
+            for (int t = 0; t < STAT_MAX_TILES / 4; ++t) st_pf[i][t] = *reinterpret_cast<const f32x2_t*>(sp + min((tid & 3) + 4 * t, a.n_stat - 1) * 2);
+        }
+    }
+
     // Loader side.  Thread tid fills LDS slot tid of each 256-slot slab; slab v of A holds
     // rows v*RPS .. v*RPS+RPS-1.  The slot is piece position tid % VPR of row tid / VPR, so
     // the lane fetches the logical piece (tid % VPR) ^ swz(row); swz only involves the low
@@ -819,7 +855,7 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
                 for (int i = 0; i < TM; ++i)
 #pragma unroll
                     for (int j = 0; j < TN; ++j) TR::mma(acc[i][j], fa[ch % SLOTS][i], fw[ch % SLOTS][j]);
-                if (kNorm && (ch & 1) == wn) {
+                if ((kNorm == NORM_RMS || kNorm == NORM_LAYER) && (ch & 1) == wn) {
 #pragma unroll
                     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -875,7 +911,29 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
     // memory traffic.
     uint32_t* Cb[2] = {reinterpret_cast<uint32_t*>(lds), reinterpret_cast<uint32_t*>(lds + C_BYTES)};
     float* row_stat = reinterpret_cast<float*>(lds + 2 * C_BYTES);  // [wn][ROWS_A][2]
-    if (kNorm) {
+    if (kNorm == NORM_LAYER_PRE) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            float q = 0.f, u = 0.f;
+#pragma unroll
+            for (int t = 0; t < STAT_MAX_TILES / 4; ++t) {
+                const bool on = (tid & 3) + 4 * t < a.n_stat;  // the clamped repeats of the last tile do not count
+                q += on ? st_pf[i][t][0] : 0.f;
+                u += on ? st_pf[i][t][1] : 0.f;
+            }
+            q += __uint_as_float(dpp_u32<DPP_XOR1>(__float_as_uint(q)));
+            u += __uint_as_float(dpp_u32<DPP_XOR1>(__float_as_uint(u)));
+            q += __uint_as_float(dpp_u32<DPP_XOR2>(__float_as_uint(q)));
+            u += __uint_as_float(dpp_u32<DPP_XOR2>(__float_as_uint(u)));
+            if ((tid & 3) == 0) {  // the epilogue adds two partial pairs per row: the totals and zeros
+                float* dst = row_stat + (i * 64 + (tid >> 2)) * 2;
+                dst[0] = q;
+                dst[1] = u;
+                dst[ROWS_A * 2] = 0.f;
+                dst[ROWS_A * 2 + 1] = 0.f;
+            }
+        }
+    } else if (kNorm) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
             float q = (ssq[i][0] + ssq[i][1]) + (ssq[i][2] + ssq[i][3]);
@@ -908,7 +966,7 @@ __global__ void __launch_bounds__(256) gemm_dl_kernel(GemmArgs a) {
         const int nt_sub = ntw * TN + j;
         if (nt_sub < a.n_tiles)
             epilogue_64x64<T, kEpi, kEpi == EPI_PLAIN>(a, Cb[n & 1], m0 + i * 64, nt_sub, tc[j], tid, pf, res_pf[i][j][0],
-                                                       res_pf[i][j][1], kNorm, row_stat + i * 128, ROWS_A * 2, bias_pf[j]);
+                                                       res_pf[i][j][1], kNorm == NORM_LAYER_PRE ? NORM_LAYER : kNorm, row_stat + i * 128, ROWS_A * 2, bias_pf[j]);
     }
 }
 
@@ -2051,7 +2109,8 @@ void launch_dl(GemmArgs a, hipStream_t st) {
     const unsigned grid = xcd_split(a, (a.M + 64 * TM - 1) / (64 * TM), (a.n_tiles + TN - 1) / TN, 2.0, 64 * TN, 2.0);
     if constexpr (kEpi == EPI_QKV) {
         if (a.norm_eps >= 0.f && a.colsum) {
-            gemm_dl_kernel<kEpi, TM, TN, KB, NS, NORM_LAYER><<<grid, 256, 0, st>>>(a);
+            if (a.stats_in) gemm_dl_kernel<kEpi, TM, TN, KB, NS, NORM_LAYER_PRE><<<grid, 256, 0, st>>>(a);
+            else gemm_dl_kernel<kEpi, TM, TN, KB, NS, NORM_LAYER><<<grid, 256, 0, st>>>(a);
             return;
         }
     }
@@ -2080,7 +2139,8 @@ int launch(GemmArgs a, int n_tiles, vla_stream_t stream) {
     if constexpr (std::is_same<T, bf16_t>::value && (kEpi == EPI_PLAIN || kEpi == EPI_QKV)) {
         // a few bf16 rows (one observation's suffix through a projection): 16 columns per workgroup, K split over its wavefronts
         bool rows_ok = a.M <= tuning().gemm_rows_max && a.M <= SR_MAX_ROWS && a.K % 8 == 0 && a.K >= 64 && a.K <= SR_MAX_K &&
-                       tuning().gemm_tile < 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0 && !(a.colsum && a.norm_eps < 0.f);
+                       tuning().gemm_tile < 0 && (uintptr_t)a.A % 16 == 0 && (uintptr_t)a.W % 16 == 0 && !(a.colsum && a.norm_eps < 0.f) &&
+                       !a.stats_out && !a.stats_in;
         if (kEpi == EPI_QKV) rows_ok = rows_ok && a.D % 16 == 0 && a.N % 16 == 0;
         if (rows_ok) {
             // more 16-column tiles than CUs: two per workgroup, so that no CU gets two workgroups' worth of requests while
@@ -2281,7 +2341,7 @@ int vla_linear(const void* x, const void* W, const float* bias, const void* resi
 static int qkv_rope_impl(const void* x, const void* W, const float* bias, int dtype, int M, int K, int S, int n_q_heads,
                          int n_kv_heads, int has_k, int has_v, int head_dim, const float* cos_tab, const float* sin_tab,
                          void* q_out, void* k_cache, void* vt_cache, int t_max, int tok_offset, float rms_eps,
-                         vla_stream_t stream, const float* colsum = nullptr) {
+                         vla_stream_t stream, const float* colsum = nullptr, const float* stats_in = nullptr, int n_stat = 0) {
     if (!x || !W || M < 0 || K <= 0 || S <= 0 || n_q_heads < 0 || n_kv_heads < 0 || head_dim <= 0) return VLA_K_ERR_ARG;
     const int nk = has_k ? n_kv_heads : 0, nv = has_v ? n_kv_heads : 0;
     if (n_q_heads > 0 && !q_out) return VLA_K_ERR_ARG;
@@ -2296,6 +2356,8 @@ static int qkv_rope_impl(const void* x, const void* W, const float* bias, int dt
     GemmArgs a = {};
     a.norm_eps = rms_eps;
     a.colsum = colsum;
+    a.stats_in = stats_in;
+    a.n_stat = n_stat;
     a.A = x; a.W = W; a.bias = bias; a.M = M; a.K = K;
     a.N = (n_q_heads + nk + nv) * D;
     a.S = S; a.Hq = n_q_heads; a.nk = nk; a.nv = nv; a.D = D; a.Hkv = n_kv_heads;
@@ -2401,6 +2463,29 @@ int vla_layernorm_attn_qkv_rope(const void* x, const void* W_folded, const float
     if (dtype != VLA_DT_BF16) return VLA_K_ERR_SHAPE;
     return qkv_rope_impl(x, W_folded, bias, dtype, M, K, S, n_q_heads, n_kv_heads, has_k, has_v, head_dim, cos_tab, sin_tab,
                          q_out, k_cache, vt_cache, t_max, tok_offset, ln_eps, stream, colsum);
+}
+
+int vla_layernorm_attn_qkv_rope_stats(const void* x, const void* W_folded, const float* colsum, const float* bias,
+                                      const float* row_stats, int n_stat_tiles, int dtype, int M, int K, int S, int n_q_heads,
+                                      int n_kv_heads, int has_k, int has_v, int head_dim, const float* cos_tab,
+                                      const float* sin_tab, void* q_out, void* k_cache, void* vt_cache, int t_max,
+                                      int tok_offset, float ln_eps, vla_stream_t stream) {
+    if (ln_eps < 0.f || !colsum || !row_stats) return VLA_K_ERR_ARG;
+    if (dtype != VLA_DT_BF16 || n_stat_tiles < 1 || n_stat_tiles > STAT_MAX_TILES || K != n_stat_tiles * BN) return VLA_K_ERR_SHAPE;
+    return qkv_rope_impl(x, W_folded, bias, dtype, M, K, S, n_q_heads, n_kv_heads, has_k, has_v, head_dim, cos_tab, sin_tab,
+                         q_out, k_cache, vt_cache, t_max, tok_offset, ln_eps, stream, colsum, row_stats, n_stat_tiles);
+}
+
+int vla_linear_row_stats(const void* x, const void* W, const float* bias, const void* residual, void* y, float* row_stats,
+                         int dtype, int M, int N, int K, vla_stream_t stream) {
+    if (!x || !W || !y || !row_stats || M < 0 || N <= 0 || K <= 0) return VLA_K_ERR_ARG;
+    if (dtype != VLA_DT_BF16 || N % BN || K % 8) return VLA_K_ERR_SHAPE;
+    GemmArgs a = {};
+    a.norm_eps = -1.f;
+    a.A = x; a.W = W; a.bias = bias; a.M = M; a.N = N; a.K = K;
+    a.residual = residual; a.Y = y; a.out_bf16 = 1;
+    a.stats_out = row_stats;
+    return launch<bf16_t, EPI_PLAIN>(a, N / BN, stream);
 }
 
 int vla_fold_norm_weight_host(const void* W, const void* g, int dtype, int N, int K, void* W_out) {

@@ -149,6 +149,8 @@ class FlowExpert : public ModelArch {
     float vlln_eps_ = 1e-5f;
     bool fuse_final_norm_ = true;  // the final norm runs inside the Euler launch
     bool fuse_self_block_ = true;  // GR00T self blocks: norm, projections and attention in one launch (VLA_NO_FUSED_SELF_BLOCK=1: off)
+    bool hand_row_stats_ = true;   // GR00T from batch 32: a block's Wo launch leaves the row sums the next block's LayerNorm needs (VLA_NO_ROW_STATS=1: off)
+    DevBuf row_stats_;             // [B * S][W / 64][2] fp32
     bool adarms_ = false;  // pi0.5: ada_ holds [steps][2L+1][scale, shift, gate][W]
     DevBuf bias_step_;   // [steps][W] fp32: b_in (+ time embedding of the step)
     DevBuf ada_;         // GR00T: [steps][L+1][2][W] fp32 (scale, shift); slot L is the final norm (zeros)
@@ -293,6 +295,7 @@ FlowExpert::FlowExpert(const Checkpoint& ck) {
     const bool no_norm_fusion = std::getenv("VLA_NO_NORM_FUSION") != nullptr;  // read once, at load
     fuse_final_norm_ = !no_norm_fusion;
     fuse_self_block_ = !no_norm_fusion && std::getenv("VLA_NO_FUSED_SELF_BLOCK") == nullptr;
+    hand_row_stats_ = !no_norm_fusion && std::getenv("VLA_NO_ROW_STATS") == nullptr;
     layers_.resize(L_);
     for (int l = 0; l < L_; ++l) {
         LayerW& w = layers_[l];
@@ -589,6 +592,7 @@ void FlowExpert::allocate(int B, int P, int P_txt) {
     hn_.alloc((size_t)B * S_ * W_ * es);
     q_.alloc((size_t)B * S_ * Hq_ * D_ * es);
     att_.alloc((size_t)B * S_ * Hq_ * D_ * es);
+    row_stats_.alloc((size_t)B * S_ * ((W_ + 63) / 64) * 2 * sizeof(float));
     if (I_ > 0) mid_.alloc((size_t)B * S_ * I_ * es);
     if (time_mlp_ || head_io_) m1_.alloc((size_t)B * S_ * W_ * sizeof(float));
     if (head_io_) {
@@ -831,8 +835,15 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                                        n_lead_ ? lead_.as<float>() : nullptr, h.data, dt_, B, S_, n_lead_, A_, W_, C.stream));
             }
             prof_mark("embed_suffix");
+            // A block's output projection leaves the row sums of the h it writes for the LayerNorm the next block takes
+            // inside its projection launch (GR00T without the FFN half, from batch 32 on, where those launches are the tiled ones).
+            const bool stats_path = hand_row_stats_ && arch_ == Arch::GR00T && dt_ == VLA_DT_BF16 && I_ == 0 && B >= 32 &&
+                                    W_ % 64 == 0 && W_ / 64 <= 24 && (Hq_ * D_) % 8 == 0;
+            bool stats_valid = false;  // row_stats_ describes the current h
             for (int l = 0; l < L_; ++l) {
                 LayerW& w = layers_[l];
+                const float* h_stats = stats_valid ? row_stats_.as<float>() : nullptr;
+                const bool leave_stats = stats_path && l + 1 < L_ && (bool)layers_[l + 1].Wqkv_ada;
                 const float* bq = w.bqkv ? w.bqkv.as<float>() : nullptr;
                 const int64_t n_rows_w = w.is_self ? (int64_t)(Hq_ + 2 * Hkv_) * D_ : (int64_t)Hq_ * D_;
                 const RopeTable* tab = rope_ ? (w.is_self ? &rope_self_ : &rope_cross_) : nullptr;
@@ -860,10 +871,12 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                     suffix_mask_ == VLA_MASK_NONE && pad_start_ >= pad_end_ && Hq_ == Hkv_) {
                     Tensor Wf = tensor_2d(w.Wqkv_ada.as<uint16_t>() + (size_t)s * n_rows_w * W_, dt_, W_, n_rows_w);
                     if (layernorm_qkv_self_attention(C, h, Wf, w.cs_ada.as<float>() + (size_t)s * n_rows_w,
-                                                     w.b_ada.as<float>() + (size_t)s * n_rows_w, eps_, S_, Hq_, D_, scale, att)) {
+                                                     w.b_ada.as<float>() + (size_t)s * n_rows_w, eps_, S_, Hq_, D_, scale, att, h_stats)) {
                         prof_mark("norm_qkv_attention_self");
                         Tensor Wo = tensor_2d(w.Wo.get(), dt_, (int64_t)Hq_ * D_, W_);
-                        linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
+                        if (leave_stats) linear_row_stats(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h, row_stats_.as<float>());
+                        else linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
+                        stats_valid = leave_stats;
                         prof_mark("wo_residual");
                         if (I_ > 0) {
                             Tensor mid = tensor_2d(mid_.get(), dt_, I_, M);
@@ -881,7 +894,7 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                     Tensor Wf = tensor_2d(w.Wqkv_ada.as<uint16_t>() + (size_t)s * n_rows_w * W_, dt_, W_, n_rows_w);
                     done = layernorm_qkv_rope_append(C, h, Wf, w.cs_ada.as<float>() + (size_t)s * n_rows_w,
                                                      w.b_ada.as<float>() + (size_t)s * n_rows_w, eps_, S_, Hq_, w.is_self, w.is_self, tab,
-                                                     Q.data, w.kv, tok);
+                                                     Q.data, w.kv, tok, h_stats);
                 }
                 if (!done) {
                     if (arch_ == Arch::GR00T) {
@@ -921,7 +934,9 @@ void FlowExpert::run_steps(int n_steps, void* stream) {
                     }
                     continue;
                 }
-                linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
+                if (leave_stats) linear_row_stats(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h, row_stats_.as<float>());
+                else linear(C, Wo, w.bo ? w.bo.as<float>() : nullptr, att, h.data, h);
+                stats_valid = leave_stats;
                 prof_mark("wo_residual");
                 if (I_ > 0) {
                     // FFN half (smolvla.cpp:845-848, pi0.cpp:227-232, dit_head.cpp:132-133)

@@ -111,6 +111,14 @@ inline void linear(Ctx& C, const Tensor& W, const float* b, const Tensor& x, con
                      C.stream));
 }
 
+// The same projection (bf16 rows, bf16 output) that also leaves (sum of squares, sum) of what it wrote per
+// (row, 64-column tile) in row_stats [rows][W rows / 64][2], for the launch that takes the next LayerNorm inside.
+inline void linear_row_stats(Ctx& C, const Tensor& W, const float* b, const Tensor& x, const void* residual, Tensor& y,
+                             float* row_stats) {
+    VLA_K(vla_linear_row_stats(x.data, W.data, b, residual, y.data, row_stats, x.dtype, (int)x.rows(), (int)W.ne[1], (int)W.ne[0],
+                               C.stream));
+}
+
 // ffn.h:24-27 (ffn_gelu) with the residual add that follows it in DitHead::block
 // (src/modules/dit_head.cpp:133): y = residual + W2 gelu(W1 x + b1) + b2.  `mid` is scratch
 // for the activated intermediate [rows][W1 rows].
@@ -184,13 +192,19 @@ inline bool rmsnorm_qkv_rope_append(Ctx& C, const Tensor& x, const Tensor& W_fol
 // A DiT block's modulated LayerNorm (norm.h:37-46) and the projection launch as one: x is
 // the un-normalised stream; W_folded, colsum and bias carry this step's (scale, shift)
 // (vla_fold_adaln_weight_host).  Returns false when the shapes do not fit the fused kernel.
+// row_stats: the rows' sums as the launch that wrote x left them (linear_row_stats), or null.
 inline bool layernorm_qkv_rope_append(Ctx& C, const Tensor& x, const Tensor& W_folded, const float* colsum, const float* bias,
                                       float eps, int S, int n_q_heads, bool has_k, bool has_v, const RopeTable* tab, void* q_out,
-                                      KVLayer& kv, int tok_offset) {
-    const int rc = vla_layernorm_attn_qkv_rope(x.data, W_folded.data, colsum, bias, x.dtype, (int)x.rows(), (int)x.ne[0], S,
-                                               n_q_heads, kv.n_kv_heads, has_k ? 1 : 0, has_v ? 1 : 0, kv.head_dim,
-                                               tab ? tab->cos.as<float>() : nullptr, tab ? tab->sin.as<float>() : nullptr,
-                                               q_out, kv.k.get(), kv.vt.get(), kv.t_max, tok_offset, eps, C.stream);
+                                      KVLayer& kv, int tok_offset, const float* row_stats = nullptr) {
+    const float* ct = tab ? tab->cos.as<float>() : nullptr;
+    const float* st = tab ? tab->sin.as<float>() : nullptr;
+    const int rc = row_stats
+        ? vla_layernorm_attn_qkv_rope_stats(x.data, W_folded.data, colsum, bias, row_stats, (int)x.ne[0] / 64, x.dtype, (int)x.rows(),
+                                            (int)x.ne[0], S, n_q_heads, kv.n_kv_heads, has_k ? 1 : 0, has_v ? 1 : 0, kv.head_dim, ct, st,
+                                            q_out, kv.k.get(), kv.vt.get(), kv.t_max, tok_offset, eps, C.stream)
+        : vla_layernorm_attn_qkv_rope(x.data, W_folded.data, colsum, bias, x.dtype, (int)x.rows(), (int)x.ne[0], S, n_q_heads,
+                                      kv.n_kv_heads, has_k ? 1 : 0, has_v ? 1 : 0, kv.head_dim, ct, st, q_out, kv.k.get(),
+                                      kv.vt.get(), kv.t_max, tok_offset, eps, C.stream);
     if (rc == VLA_K_ERR_SHAPE) return false;
     VLA_K(rc);
     return true;
@@ -200,9 +214,13 @@ inline bool layernorm_qkv_rope_append(Ctx& C, const Tensor& x, const Tensor& W_f
 // tokens over themselves as one launch (dit_head.cpp:111-125 with enc = nullptr); the block's K
 // and V stay on the chip.  Returns false when the shapes do not fit the fused kernel.
 inline bool layernorm_qkv_self_attention(Ctx& C, const Tensor& x, const Tensor& W_folded, const float* colsum, const float* bias,
-                                         float eps, int S, int n_heads, int head_dim, float scale, Tensor& out) {
-    const int rc = vla_layernorm_qkv_self_attention(x.data, W_folded.data, colsum, bias, x.dtype, (int)x.rows(), (int)x.ne[0], S,
-                                                    n_heads, head_dim, scale, eps, out.data, C.stream);
+                                         float eps, int S, int n_heads, int head_dim, float scale, Tensor& out,
+                                         const float* row_stats = nullptr) {
+    const int rc = row_stats
+        ? vla_layernorm_qkv_self_attention_stats(x.data, W_folded.data, colsum, bias, row_stats, (int)x.ne[0] / 64, x.dtype,
+                                                 (int)x.rows(), (int)x.ne[0], S, n_heads, head_dim, scale, eps, out.data, C.stream)
+        : vla_layernorm_qkv_self_attention(x.data, W_folded.data, colsum, bias, x.dtype, (int)x.rows(), (int)x.ne[0], S, n_heads,
+                                           head_dim, scale, eps, out.data, C.stream);
     if (rc == VLA_K_ERR_SHAPE) return false;
     VLA_K(rc);
     return true;
