@@ -74,10 +74,10 @@ __device__ __forceinline__ float sum_pair_bf16x2(uint32_t u, float acc) {
 // Straight-line per (NR, NC): the four wavefronts of a workgroup fall into four classes and each
 // runs its own copy, so no block is computed twice and none sits behind a branch (a branch
 // inside the loop body cuts it into pieces the scheduler cannot interleave).
-template <int NR, int NC, bool PRE>
+template <int NR, int NC, bool PRE, typename AfterIssue>
 __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* lds, const unsigned char* const (&ap)[5],
                                             const unsigned char* const (&wp)[5], uint32_t lds0, int koff, bool tail, int wm, int wn,
-                                            int c, int q, f32x4_t (&acc)[5][5], float (&ssq)[5], float (&ssum)[5]) {
+                                            int c, int q, f32x4_t (&acc)[5][5], float (&ssq)[5], float (&ssum)[5], AfterIssue&& after_issue) {
     // row sums: the two wavefronts that multiply the same rows (block columns 0 and 1) take alternate 32-k chunks
     // (PRE: the sums come from the launch that wrote the rows: no chunk takes them)
     constexpr int STATS_SET = PRE ? 7 : NC == 5 ? 0 : 1;
@@ -129,6 +129,7 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
     const int nkt = a.K / 64;
 #pragma unroll
     for (int t = 0; t < FS_NS; ++t) issue(t, t);
+    after_issue();  // work on loads requested before the ring's: they land first, and the ring's trip runs under it
     if (tail) wait_vmcnt<30>();
     else wait_vmcnt<24>();
     __syncthreads();
@@ -173,6 +174,56 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
     wait_vmcnt<0>();
 }
 
+// The accumulators leave for LDS as bf16: rstd (acc - mean colsum) + bias, Q and K columns into the
+// [row][q | k] tile, V columns transposed into their observation's V^T tile.  Per wavefront class like the
+// walk, so that every loop bound and the kind of a block column (block columns 0 .. 5 are q | k, 6 .. 8 are
+// v: for either parity of the wavefront that is j < 3 and j >= 3) are constants; what depends on the row
+// only is formed once per row, the element itself costs a multiply-add, a conversion and a 2-byte store.
+template <int NR, int NC>
+__device__ __forceinline__ void self_tile_to_lds(const SelfArgs& a, const f32x4_t (&acc)[5][5], const float (&cs)[5], const float (&bs)[5],
+                                                 const float* stat, unsigned char* lds, int wm, int wn, int c, int q, int n_valid) {
+    const float inv_k = 1.0f / (float)a.K;
+    const int S = a.S, inv_s = (65536 + S - 1) / S;
+    unsigned char* const vt0 = lds + FS_ROWS * FS_QS * 2;
+    int coff[NC];  // byte offset of the lane's column inside a row of the q | k tile, or of its V^T row inside an observation's tile
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+        const int col = (wn + 2 * j) * 16 + c;
+        coff[j] = j < 3 ? col * 2 : (col - 2 * FS_D) * FS_VS * 2;
+    }
+    // every row's sums first (one batch of LDS reads), then the arithmetic
+    f32x2_t sa[NR][4], sb[NR][4];
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = (wm + 2 * i) * 16 + 4 * q + e;
+            sa[i][e] = *reinterpret_cast<const f32x2_t*>(stat + row * 2);
+            sb[i][e] = *reinterpret_cast<const f32x2_t*>(stat + (FS_ROWS + row) * 2);
+        }
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = (wm + 2 * i) * 16 + 4 * q + e;
+            const float s2 = sa[i][e][0] + sb[i][e][0], s1 = sa[i][e][1] + sb[i][e][1];
+            const float mean = s1 * inv_k;
+            const float rstd = rsqrtf(fmaxf(s2 * inv_k - mean * mean, 0.f) + a.eps);
+            const float ms = mean * rstd;
+            const int u = (row * inv_s) >> 16, key = row - u * S;  // row / S, exact for S <= 32 and row < 160
+            unsigned char* const qrow = lds + row * FS_QS * 2;
+            unsigned char* const vrow = vt0 + (u * FS_D * FS_VS + key) * 2;
+            const bool live = row < n_valid;
+#pragma unroll
+            for (int j = 0; j < NC; ++j) {
+                const bf16_t v = f2bf(acc[i][j][e] * rstd - ms * cs[j] + bs[j]);
+                if (j < 3) *reinterpret_cast<bf16_t*>(qrow + coff[j]) = v;          // q: 0..47, k: 48..95
+                else if (live) *reinterpret_cast<bf16_t*>(vrow + coff[j]) = v;       // V^T[u][d][key]
+            }
+        }
+    }
+}
+
 template <bool PRE>
 __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[FS_NS * FS_STAGE];
@@ -184,6 +235,16 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     const int m0 = group * rows_per;
     const int n_valid = min(rows_per, a.M - m0);  // rows of this tile that exist (whole observations)
     const long HD = (long)a.H * FS_D;
+
+    // PRE: this thread's row of the tile (threads 0 .. 143) and its handed-over sums: requested first of all and
+    // added up once the K walk has requested its ring (their trip runs under the address arithmetic below, the
+    // ring's under the additions), which leaves two registers to carry through the walk instead of 48
+    f32x2_t pre_pv[PRE ? FS_MAX_STAT : 1];
+    if (PRE && tid < FS_ROWS) {
+        const float* sp = a.stats_in + (long)min(m0 + tid, a.M - 1) * a.n_stat * 2;
+#pragma unroll
+        for (int t = 0; t < FS_MAX_STAT; ++t) pre_pv[t] = *reinterpret_cast<const f32x2_t*>(sp + 2 * min(t, a.n_stat - 1));
+    }
 
     // ---- loader: thread tid fills slot tid of each 256-slot slab (32 rows x 8 pieces); slabs 0..3
     // are whole, slab 4 holds rows 128..143 and is filled by wavefronts 0 and 1 alone
@@ -219,27 +280,23 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
 #pragma unroll
         for (int j = 0; j < 5; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     float ssq[5] = {0.f, 0.f, 0.f, 0.f, 0.f}, ssum[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
-    const int nr = wm == 0 ? 5 : 4, nc = wn == 0 ? 5 : 4;
-    if (wm == 0) {
-        if (wn == 0) self_k_walk<5, 5, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
-        else self_k_walk<5, 4, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
-    } else {
-        if (wn == 0) self_k_walk<4, 5, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
-        else self_k_walk<4, 4, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum);
-    }
-    // PRE: this thread's row of the tile (threads 0 .. 143) and its handed-over sums, requested before the barrier
-    // and added up behind it (the consumer of x's row sums reads 24 pairs per row; they come from L2)
     float pre_q = 0.f, pre_u = 0.f;
-    if (PRE && tid < FS_ROWS) {
-        const float* sp = a.stats_in + (long)min(m0 + tid, a.M - 1) * a.n_stat * 2;
-        f32x2_t pv[FS_MAX_STAT];  // one trip: every pair requested before the first is added (the fragment registers are free by now)
+    auto sum_pre = [&]() __attribute__((always_inline)) {
+        if (PRE && tid < FS_ROWS) {
 #pragma unroll
-        for (int t = 0; t < FS_MAX_STAT; ++t) pv[t] = *reinterpret_cast<const f32x2_t*>(sp + 2 * min(t, a.n_stat - 1));
-#pragma unroll
-        for (int t = 0; t < FS_MAX_STAT; ++t) {
-            pre_q += t < a.n_stat ? pv[t][0] : 0.f;
-            pre_u += t < a.n_stat ? pv[t][1] : 0.f;
+            for (int t = 0; t < FS_MAX_STAT; ++t) {
+                pre_q += t < a.n_stat ? pre_pv[t][0] : 0.f;
+                pre_u += t < a.n_stat ? pre_pv[t][1] : 0.f;
+            }
         }
+    };
+    const int nr = wm == 0 ? 5 : 4;
+    if (wm == 0) {
+        if (wn == 0) self_k_walk<5, 5, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum, sum_pre);
+        else self_k_walk<5, 4, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum, sum_pre);
+    } else {
+        if (wn == 0) self_k_walk<4, 5, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum, sum_pre);
+        else self_k_walk<4, 4, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum, sum_pre);
     }
     __syncthreads();
 
@@ -264,35 +321,16 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     }
     // keys past S of every V^T row are multiplied by probabilities that are zero: they must be finite
     const int S = a.S;
-    for (int idx = tid; idx < a.OB * FS_D * (FS_VS / 4); idx += 256) {
-        const int row = idx / (FS_VS / 4), k4 = idx - row * (FS_VS / 4);
-        if (4 * k4 + 3 >= S) *reinterpret_cast<u32x2_t*>(vt + row * FS_VS + 4 * k4) = u32x2_t{0u, 0u};
-    }
+    for (int row = tid; row < a.OB * FS_D; row += 256)
+        for (int k4 = S >> 2; k4 < FS_VS / 4; ++k4)  // the groups of four keys that reach past S
+            *reinterpret_cast<u32x2_t*>(vt + row * FS_VS + 4 * k4) = u32x2_t{0u, 0u};
     __syncthreads();
-    const float inv_k = 1.0f / (float)a.K;
-    const int inv_s = (65536 + S - 1) / S;
-#pragma unroll
-    for (int i = 0; i < 5; ++i) {
-        const int rb = wm + 2 * i;
-        if (i >= nr) continue;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int row = rb * 16 + 4 * q + e;
-            const float s2 = stat[row * 2] + stat[(FS_ROWS + row) * 2], s1 = stat[row * 2 + 1] + stat[(FS_ROWS + row) * 2 + 1];
-            const float mean = s1 * inv_k;
-            const float rstd = rsqrtf(fmaxf(s2 * inv_k - mean * mean, 0.f) + a.eps);
-            const float ms = mean * rstd;
-            const int u = (row * inv_s) >> 16, key = row - u * S;  // row / S, exact for S <= 32 and row < 160
-#pragma unroll
-            for (int j = 0; j < 5; ++j) {
-                const int cb = wn + 2 * j;
-                if (j >= nc) continue;
-                const bf16_t v = f2bf(acc[i][j][e] * rstd - ms * cs[j] + bs[j]);
-                const int col = cb * 16 + c;
-                if (cb < 6) qk[row * FS_QS + col] = v;                                       // q: 0..47, k: 48..95
-                else if (row < n_valid) vt[(u * FS_D + col - 2 * FS_D) * FS_VS + key] = v;   // V^T[u][d][key]
-            }
-        }
+    if (wm == 0) {
+        if (wn == 0) self_tile_to_lds<5, 5>(a, acc, cs, bs, stat, lds, wm, wn, c, q, n_valid);
+        else self_tile_to_lds<5, 4>(a, acc, cs, bs, stat, lds, wm, wn, c, q, n_valid);
+    } else {
+        if (wn == 0) self_tile_to_lds<4, 5>(a, acc, cs, bs, stat, lds, wm, wn, c, q, n_valid);
+        else self_tile_to_lds<4, 4>(a, acc, cs, bs, stat, lds, wm, wn, c, q, n_valid);
     }
     __syncthreads();
 
