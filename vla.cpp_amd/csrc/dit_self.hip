@@ -178,7 +178,7 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
 // [row][q | k] tile, V columns transposed into their observation's V^T tile.  Per wavefront class like the
 // walk, so that every loop bound and the kind of a block column (block columns 0 .. 5 are q | k, 6 .. 8 are
 // v: for either parity of the wavefront that is j < 3 and j >= 3) are constants; what depends on the row
-// only is formed once per row, the element itself costs a multiply-add, a conversion and a 2-byte store.
+// only is formed once per row, an element costs two multiply-adds, half a conversion and a 2-byte store.
 template <int NR, int NC>
 __device__ __forceinline__ void self_tile_to_lds(const SelfArgs& a, const f32x4_t (&acc)[5][5], const float (&cs)[5], const float (&bs)[5],
                                                  const float* stat, unsigned char* lds, int wm, int wn, int c, int q, int n_valid) {
@@ -201,24 +201,38 @@ __device__ __forceinline__ void self_tile_to_lds(const SelfArgs& a, const f32x4_
             sa[i][e] = *reinterpret_cast<const f32x2_t*>(stat + row * 2);
             sb[i][e] = *reinterpret_cast<const f32x2_t*>(stat + (FS_ROWS + row) * 2);
         }
+    // Two rows (e, e + 1) at a time: one conversion gives both rows' bf16 values of a column, stored as the low
+    // and the high half.  Rows past the tile's last observation write their V values to an unused part of LDS
+    // (the address is selected once per row) instead of sitting behind a branch per element.
+    unsigned char* const dead = lds + 96 * 1024;
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int row = (wm + 2 * i) * 16 + 4 * q + e;
-            const float s2 = sa[i][e][0] + sb[i][e][0], s1 = sa[i][e][1] + sb[i][e][1];
-            const float mean = s1 * inv_k;
-            const float rstd = rsqrtf(fmaxf(s2 * inv_k - mean * mean, 0.f) + a.eps);
-            const float ms = mean * rstd;
-            const int u = (row * inv_s) >> 16, key = row - u * S;  // row / S, exact for S <= 32 and row < 160
-            unsigned char* const qrow = lds + row * FS_QS * 2;
-            unsigned char* const vrow = vt0 + (u * FS_D * FS_VS + key) * 2;
-            const bool live = row < n_valid;
+        for (int e = 0; e < 4; e += 2) {
+            float rstd[2], nmean[2];
+            unsigned char* qrow[2];
+            unsigned char* vrow[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int row = (wm + 2 * i) * 16 + 4 * q + e + h;
+                const float s2 = sa[i][e + h][0] + sb[i][e + h][0], s1 = sa[i][e + h][1] + sb[i][e + h][1];
+                const float mean = s1 * inv_k;
+                rstd[h] = rsqrtf(fmaxf(s2 * inv_k - mean * mean, 0.f) + a.eps);
+                nmean[h] = -mean;
+                const int u = (row * inv_s) >> 16, key = row - u * S;  // row / S, exact for S <= 32 and row < 160
+                qrow[h] = lds + row * FS_QS * 2;
+                vrow[h] = row < n_valid ? vt0 + (u * FS_D * FS_VS + key) * 2 : dead;
+            }
 #pragma unroll
             for (int j = 0; j < NC; ++j) {
-                const bf16_t v = f2bf(acc[i][j][e] * rstd - ms * cs[j] + bs[j]);
-                if (j < 3) *reinterpret_cast<bf16_t*>(qrow + coff[j]) = v;          // q: 0..47, k: 48..95
-                else if (live) *reinterpret_cast<bf16_t*>(vrow + coff[j]) = v;       // V^T[u][d][key]
+                // rstd (acc - mean colsum) + bias
+                const float v0 = __builtin_fmaf(__builtin_fmaf(nmean[0], cs[j], acc[i][j][e]), rstd[0], bs[j]);
+                const float v1 = __builtin_fmaf(__builtin_fmaf(nmean[1], cs[j], acc[i][j][e + 1]), rstd[1], bs[j]);
+                const uint32_t pk = pack_bf2(v0, v1);
+                unsigned char* const d0 = (j < 3 ? qrow[0] : vrow[0]) + coff[j];  // q: 0..47, k: 48..95; V^T[u][d][key]
+                unsigned char* const d1 = (j < 3 ? qrow[1] : vrow[1]) + coff[j];
+                *reinterpret_cast<bf16_t*>(d0) = (bf16_t)(pk & 0xffffu);
+                *reinterpret_cast<bf16_t*>(d1) = (bf16_t)(pk >> 16);
             }
         }
     }
