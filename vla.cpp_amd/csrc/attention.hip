@@ -335,26 +335,37 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
             // MFMA waiting for the LDS latency, and for 256-wide heads the register allocator
             // otherwise keeps only two fragments in flight (the second accumulator chain is
             // given up for the fragment registers there)
-            constexpr int FB = (NQ >= 16 && !DLOAD) ? WIDE_FB : 1;
-            constexpr int NA = (NQ >= 4 && NKB == 1 && FB == 1) ? 2 : 1;
+            constexpr int FB = (NQ >= 16 && !DLOAD) ? WIDE_FB - 1 : 1;  // (one fewer than for V^T: the second accumulator chain takes the registers)
+            constexpr int NA = (NQ >= 4 && NKB == 1) ? 2 : 1;
             f32x16_t sc[NA];
 #pragma unroll
             for (int n = 0; n < NA; ++n)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) sc[n][i] = 0.f;
+            if constexpr (FB > 1) {
+                // rolling read-ahead: FB fragments are on their way when the first product starts, and each
+                // product is followed by the read of the fragment FB places further on
+                u32x4_t kf[NQ];
 #pragma unroll
-            for (int c0 = 0; c0 < NQ; c0 += FB) {
-                u32x4_t kf[FB];
+                for (int c = 0; c < NQ; ++c)
+                    kf[c] = *reinterpret_cast<const u32x4_t*>(ldsK + (kb * 32 + key_of_score_row(r)) * KS + (c * CE + g * (CE / 2)) * EB);
 #pragma unroll
-                for (int f = 0; f < FB; ++f) {
-                    const int c = c0 + f;
-                    kf[f] = *reinterpret_cast<const u32x4_t*>(
+                for (int c = 0; c < NQ; ++c) A::mma(sc[c % NA], kf[c], qf[c]);
+                __builtin_amdgcn_sched_group_barrier(0x100, FB, 0);
+#pragma unroll
+                for (int c = 0; c < NQ - FB; ++c) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(0x008, FB, 0);
+            } else {
+#pragma unroll
+                for (int c = 0; c < NQ; ++c) {
+                    const u32x4_t kf = *reinterpret_cast<const u32x4_t*>(
                         DLOAD ? ldsK + kb * 32 * KROW + kfrag + (((2 * c) ^ kx) * 16)
                               : ldsK + (kb * 32 + key_of_score_row(r)) * KS + (c * CE + g * (CE / 2)) * EB);
+                    A::mma(sc[c % NA], kf, qf[c]);
                 }
-                if (FB > 1) __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int f = 0; f < FB; ++f) A::mma(sc[(c0 + f) % NA], kf[f], qf[c0 + f]);
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -425,7 +436,44 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         const bool v_partial = DLOAD && k0 + TK > a.n_keys;  // uniform
 #pragma unroll
         for (int kb = 0; kb < NKB; ++kb) {
-            if (EB == 2) {
+            if constexpr (EB == 2 && NDB >= 8 && !DLOAD) {
+                // 256-wide heads: the 2 x NDB fragments of both key halves as one sequence with a rolling
+                // read-ahead of WIDE_FB fragments, so that the LDS latency is paid once per tile
+                // (with two-term probabilities the halves stay two sequences: both halves' terms at once do not fit the registers)
+                constexpr int HPS = P2 ? 1 : 2, NF = HPS * NDB;  // key halves and fragments per sequence
+#pragma unroll
+                for (int h0 = 0; h0 < 2; h0 += HPS) {
+                    u32x4_t pf[HPS], pl[HPS];
+#pragma unroll
+                    for (int hh = 0; hh < HPS; ++hh) {
+                        const float* pp = &p[kb][(h0 + hh) * 8];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint32_t hi16 = pack_bf2(pp[2 * e], pp[2 * e + 1]);
+                            pf[hh][e] = hi16;
+                            if (P2)
+                                pl[hh][e] = pack_bf2(pp[2 * e] - __uint_as_float(hi16 << 16), pp[2 * e + 1] - __uint_as_float(hi16 & 0xffff0000u));
+                        }
+                    }
+                    u32x4_t vf[NF];
+#pragma unroll
+                    for (int f = 0; f < NF; ++f)
+                        vf[f] = *reinterpret_cast<const u32x4_t*>(ldsV + ((f % NDB) * 32 + r) * VS + (kb * 32 + (h0 + f / NDB) * 16 + 8 * g) * EB);
+#pragma unroll
+                    for (int f = 0; f < NF; ++f) {
+                        A::mma(o[f % NDB], vf[f], pf[f / NDB]);
+                        if (P2) A::mma(o[f % NDB], vf[f], pl[f / NDB]);
+                    }
+                    constexpr int MPF = P2 ? 2 : 1;  // products per fragment
+                    __builtin_amdgcn_sched_group_barrier(0x100, WIDE_FB, 0);
+#pragma unroll
+                    for (int f = 0; f < NF - WIDE_FB; ++f) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, MPF, 0);
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, WIDE_FB * MPF, 0);
+                }
+            } else if (EB == 2) {
 #pragma unroll
                 for (int hh = 0; hh < 2; ++hh) {
                     // P2: the probabilities enter the bf16 MFMA as hi + lo (two bf16 terms,
@@ -443,27 +491,17 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
                     }
                     const int key_off = (kb * 32 + hh * 16 + 8 * g) * EB;
                     const int nvalid = a.n_keys - (k0 + kb * 32 + hh * 16 + 8 * g);  // real keys among this lane's 8
-                    // (256-wide heads: VB of a half tile's V^T fragments are read ahead of their
-                    // MFMAs, as for the K fragments)
-                    constexpr int VB = (NDB >= 8 && !DLOAD) ? WIDE_FB : 1;
+                    {
 #pragma unroll
-                    for (int d0 = 0; d0 < NDB; d0 += VB) {
-                        u32x4_t vf[VB];
-#pragma unroll
-                        for (int f = 0; f < VB; ++f) {
-                            const int db = d0 + f;
-                            vf[f] = *reinterpret_cast<const u32x4_t*>(
+                        for (int db = 0; db < NDB; ++db) {
+                            u32x4_t vf = *reinterpret_cast<const u32x4_t*>(
                                 DLOAD ? ldsV + db * 32 * VROW + vfrag + (((4 * kb + 2 * hh) ^ vx) * 16) : ldsV + (db * 32 + r) * VS + key_off);
-                        }
-                        if (VB > 1) __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int f = 0; f < VB; ++f) {
                             if (v_partial) {
 #pragma unroll
-                                for (int e = 0; e < 4; ++e) vf[f][e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
+                                for (int e = 0; e < 4; ++e) vf[e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
                             }
-                            A::mma(o[d0 + f], vf[f], pf);
-                            if (P2) A::mma(o[d0 + f], vf[f], pl);
+                            A::mma(o[db], vf, pf);
+                            if (P2) A::mma(o[db], vf, pl);
                         }
                     }
                 }
