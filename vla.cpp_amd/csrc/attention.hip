@@ -436,7 +436,7 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         const bool v_partial = DLOAD && k0 + TK > a.n_keys;  // uniform
 #pragma unroll
         for (int kb = 0; kb < NKB; ++kb) {
-            if constexpr (EB == 2 && NDB >= 8 && !DLOAD) {
+            if constexpr (NL > 0 && EB == 2 && NDB >= 8 && NKB == 1) {
                 // 256-wide heads: the 2 x NDB fragments of both key halves as one sequence with a rolling
                 // read-ahead of WIDE_FB fragments, so that the LDS latency is paid once per tile
                 // (with two-term probabilities the halves stay two sequences: both halves' terms at once do not fit the registers)
@@ -458,7 +458,7 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
                     u32x4_t vf[NF];
 #pragma unroll
                     for (int f = 0; f < NF; ++f)
-                        vf[f] = *reinterpret_cast<const u32x4_t*>(ldsV + ((f % NDB) * 32 + r) * VS + (kb * 32 + (h0 + f / NDB) * 16 + 8 * g) * EB);
+                        vf[f] = *reinterpret_cast<const u32x4_t*>(ldsV + ((f % NDB) * 32 + r) * 64 + (((2 * (h0 + f / NDB) + g) ^ ((r >> 2) & 3)) * 16));  // (NKB == 1)
 #pragma unroll
                     for (int f = 0; f < NF; ++f) {
                         A::mma(o[f % NDB], vf[f], pf[f / NDB]);
@@ -678,6 +678,13 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
         if (wave >= NW) {
             const int lt = tid - NW * 64;
             u32x4_t kq[LOAD_AHEAD][ITL], vq[LOAD_AHEAD][ITL];
+            // V^T rows lie unpadded (64 bytes) with their four 16-byte pieces XOR-swizzled by (row >> 2) & 3.  A
+            // 16-byte LDS store is served eight lanes at a time and two of them collide when their addresses agree
+            // in bits 4 .. 6: with 80-byte rows the first and the last of every eight lanes (two rows of four
+            // pieces) do, and every store takes twice as long; the fragment reads (sixteen lanes at a time, rows
+            // r, r + 12, r + 20, r + 24 together) are free of conflicts either way.
+            static_assert(VV_PER_ROW == 4, "swizzle of four pieces per V^T row");
+            auto v_at = [](int v) __attribute__((always_inline)) { return (v / 4) * 64 + (((v % 4) ^ ((v >> 4) & 3)) * 16); };
             // Unconditional loads with clamped addresses (K rows past n_keys repeat the last
             // key: their scores are masked; V^T runs are kept inside the row) so the loop body
             // has no load under a branch; tiles past the last repeat it and are never read.
@@ -705,7 +712,7 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
                     for (int i = 0; i < ITL; ++i) {
                         const int v = lt + i * NTL;
                         *reinterpret_cast<u32x4_t*>(ldsK_buf[stage] + (v / KV_PER_ROW) * KS + (v % KV_PER_ROW) * 16) = kq[slot][i];
-                        *reinterpret_cast<u32x4_t*>(ldsV_buf[stage] + (v / VV_PER_ROW) * VS + (v % VV_PER_ROW) * 16) = vq[slot][i];
+                        *reinterpret_cast<u32x4_t*>(ldsV_buf[stage] + v_at(v)) = vq[slot][i];
                     }
                 } else {
 #pragma unroll
@@ -716,7 +723,7 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
                         u32x4_t val = vq[slot][i];
 #pragma unroll
                         for (int e = 0; e < 4; ++e) val[e] &= (2 * e < nvalid ? 0xffffu : 0u) | (2 * e + 1 < nvalid ? 0xffff0000u : 0u);
-                        *reinterpret_cast<u32x4_t*>(ldsV_buf[stage] + (v / VV_PER_ROW) * VS + (v % VV_PER_ROW) * 16) = val;
+                        *reinterpret_cast<u32x4_t*>(ldsV_buf[stage] + v_at(v)) = val;
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
