@@ -113,6 +113,53 @@ __device__ __forceinline__ void merge_row(const float* __restrict__ part_o, cons
     }
 }
 
+// The same for a slice count known at compile time: every load of the row -- the slices' (max, sum) pairs and their
+// partial outputs -- is requested before the first is used, one trip to memory instead of one per slice (the loop above
+// waits for each slice's loads inside its iteration).  Same arithmetic in the same order.
+template <typename T, bool HALF, int NS>
+__device__ __forceinline__ void merge_row_static(const float* __restrict__ part_o, const float* __restrict__ part_ml, T* __restrict__ orow,
+                                                 long prow0, int r_pad, int D, int lane) {
+    typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+    f32x2_t ml[NS];
+#pragma unroll
+    for (int sp = 0; sp < NS; ++sp) ml[sp] = *reinterpret_cast<const f32x2_t*>(part_ml + (prow0 + (long)sp * r_pad) * 2);
+    for (int d0 = lane * 4; d0 < D; d0 += 256) {
+        h4_t ph[NS];
+        f32x4_t pf[NS];
+#pragma unroll
+        for (int sp = 0; sp < NS; ++sp) {
+            const long prow = prow0 + (long)sp * r_pad;
+            if (HALF) ph[sp] = *reinterpret_cast<const h4_t*>(reinterpret_cast<const _Float16*>(part_o) + prow * D + d0);
+            else pf[sp] = *reinterpret_cast<const f32x4_t*>(part_o + prow * D + d0);
+        }
+        float m = -INFINITY;
+#pragma unroll
+        for (int sp = 0; sp < NS; ++sp) m = fmaxf(m, ml[sp][0]);
+        const float mm = m > -INFINITY ? m : 0.f;  // nothing visible in any slice: every weight 2^-inf = 0
+        float l = 0.f;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int sp = 0; sp < NS; ++sp) {
+            const float w = exp2f(ml[sp][0] - mm);
+            if (HALF) {
+                const float wl = ml[sp][1] * w;
+                l += wl;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += (float)ph[sp][e] * wl;
+            } else {
+                l += ml[sp][1] * w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[e] += pf[sp][e] * w;
+            }
+        }
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = l > 0.f ? acc[e] / l : 0.f;
+        if constexpr (sizeof(T) == 2) *reinterpret_cast<u32x2_t*>(orow + d0) = u32x2_t{pack_bf2(v[0], v[1]), pack_bf2(v[2], v[3])};
+        else *reinterpret_cast<f32x4_t*>(orow + d0) = f32x4_t{v[0], v[1], v[2], v[3]};
+    }
+}
+
 template <typename T> struct AT;
 template <> struct AT<bf16_t> {
     static constexpr int EB = 2;
@@ -1705,8 +1752,18 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
     const int pair = ridx / R, row = ridx % R;
     const int grp = Hq / Hkv, b = pair / Hkv, hk = pair % Hkv;
     const int h = hk * grp + row / S, s = row % S;
-    merge_row<T, HALF>(part_o, part_ml, out + (((long)b * S + s) * Hq + h) * D, (long)pair * n_split * r_pad + row, n_split, r_pad, D,
-                       lane);
+    T* orow = out + (((long)b * S + s) * Hq + h) * D;
+    const long prow0 = (long)pair * n_split * r_pad + row;
+    switch (n_split) {  // wavefront-uniform
+        case 2: merge_row_static<T, HALF, 2>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 3: merge_row_static<T, HALF, 3>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 4: merge_row_static<T, HALF, 4>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 5: merge_row_static<T, HALF, 5>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 6: merge_row_static<T, HALF, 6>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 7: merge_row_static<T, HALF, 7>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 8: merge_row_static<T, HALF, 8>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        default: merge_row<T, HALF>(part_o, part_ml, orow, prow0, n_split, r_pad, D, lane); break;
+    }
 }
 
 // ---- scratch memory of a call ---------------------------------------------------------
