@@ -1762,6 +1762,14 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict
         case 6: merge_row_static<T, HALF, 6>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
         case 7: merge_row_static<T, HALF, 7>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
         case 8: merge_row_static<T, HALF, 8>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 9: merge_row_static<T, HALF, 9>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 10: merge_row_static<T, HALF, 10>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 11: merge_row_static<T, HALF, 11>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 12: merge_row_static<T, HALF, 12>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 13: merge_row_static<T, HALF, 13>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 14: merge_row_static<T, HALF, 14>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 15: merge_row_static<T, HALF, 15>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
+        case 16: merge_row_static<T, HALF, 16>(part_o, part_ml, orow, prow0, r_pad, D, lane); break;
         default: merge_row<T, HALF>(part_o, part_ml, orow, prow0, n_split, r_pad, D, lane); break;
     }
 }
