@@ -931,6 +931,30 @@ def test_attention_direct_kernel_key_slices_merge(tune, split):
     assert np.isfinite(got).all() and bf16_close(got, want) and rel_err(got, want) < 1e-2
 
 
+@pytest.mark.parametrize("split", [12, 16, 19])
+def test_attention_merge_launch_with_many_key_slices(tune, split):
+    # The merge launch is specialised for up to 16 slices (every load of a row requested at once) and loops over
+    # the slices beyond that: both forms against the oracle, on a key range long enough for 19 slices of two blocks.
+    r = np.random.default_rng(140 + split)
+    B, S, Hq, Hkv, D, T = 1, 3, 4, 2, 64, 1200
+    t_max = 1216
+    Q = orc.round_bf16(r.standard_normal((B, S, Hq, D)).astype(np.float32))
+    K = orc.round_bf16(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    V = orc.round_bf16(r.standard_normal((B, T, Hkv, D)).astype(np.float32))
+    kc = torch.full((B, Hkv, t_max, D), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
+    vc = torch.full((B, Hkv, D, t_max), float("nan"), device="cuda").to(torch.bfloat16).view(torch.int16)
+    pkg.call("vla_kv_append", kc, vc, to_dev(K, BF16), to_dev(V, BF16), BF16, B, Hkv, D, t_max, 0, T)
+    tune.set("VLA_ATTN_SPLIT", str(split))
+    out = empty((B, S, Hq * D), BF16)
+    pkg.call("vla_attn_prefix_suffix", to_dev(Q, BF16), kc, vc, out, BF16, B, S, Hq, Hkv, D, t_max, T, 0.125,
+             pkg.VLA_MASK_CAUSAL_SUFFIX, T - S, 100, 120, None)
+    sync()
+    mask = orc.mask_smolvla_full(T - S, S, 100, 120)
+    want = np.stack([orc.attention(Q[b], K[b], V[b], mask, 0.125) for b in range(B)])
+    got = as_f32(out, BF16)
+    assert np.isfinite(got).all() and bf16_close(got, want) and rel_err(got, want) < 1e-2
+
+
 @pytest.mark.parametrize("B,S,Hq,Hkv,T", [(8, 1, 20, 5, 519), (1, 1, 20, 5, 513), (3, 2, 8, 2, 519), (1, 1, 28, 4, 1000), (3, 2, 8, 2, 300), (2, 1, 4, 4, 97),
                                           (8, 1, 20, 5, 33)])
 def test_attention_decode_slices_merged_by_the_last_to_arrive(tune, B, S, Hq, Hkv, T):

@@ -94,6 +94,17 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
             load_to_lds16(wp[4] + kb, base + FS_ROWS * FS_KB + 4 * 4096);
         }
     };
+    // request l of a tile's ten: the four 32-row slabs of x, the four of W, then the two 16-row remainders (tail)
+    auto issue_one = [&](int l, int kt, int stage) __attribute__((always_inline)) {
+        const long kb = ((long)kt * 64 + koff) * 2;
+        const uint32_t base = lds0 + stage * FS_STAGE;
+        if (l < 4) load_to_lds16(ap[l] + kb, base + l * 4096);
+        else if (l < 8) load_to_lds16(wp[l - 4] + kb, base + FS_ROWS * FS_KB + (l - 4) * 4096);
+        else if (tail) {
+            if (l == 8) load_to_lds16(ap[4] + kb, base + 4 * 4096);
+            else load_to_lds16(wp[4] + kb, base + FS_ROWS * FS_KB + 4 * 4096);
+        }
+    };
     u32x4_t fa[2][NR], fw[2][NC];  // fragment sets of two consecutive chunks
     auto read_frags = [&](int set, int stage, int ch) __attribute__((always_inline)) {
         const unsigned char* base = lds + stage * FS_STAGE;
@@ -121,6 +132,44 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
                 }
         }
     };
+    // Chunk 1 of a tile, in groups of two MFMAs in a fixed order: each group reads one fragment of the next tile's chunk 0
+    // and (LOAD) requests a share of the tile four further on into the stage the workgroup has just left.  Requested in
+    // one burst after the barrier instead, the ten loads (an M0 write and a 64-bit address each) keep the matrix pipe
+    // idle for their whole issue time, once per tile.
+    constexpr int NM = NR * NC, NG = (NM + 1) / 2;
+    static_assert(NR + NC <= NG + 2 && NG >= 8, "a fragment read and a request per group");
+    auto chunk1_groups = [&](auto do_load, int kt_load, int st_load, int st_next) __attribute__((always_inline)) {
+        constexpr bool LOAD = decltype(do_load)::value;
+        const unsigned char* base = lds + st_next * FS_STAGE;
+        const int off = (q ^ fsw) * 16;  // chunk 0
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            // fragment reads: NR + NC of them over the first groups (two in a group while more reads than groups remain)
+#pragma unroll
+            for (int f = 0; f < NR + NC; ++f) {
+                if (f * NG / (NR + NC) != g) continue;
+                if (f < NR) fa[0][f] = *reinterpret_cast<const u32x4_t*>(base + ((wm + 2 * f) * 16 + c) * FS_KB + off);
+                else fw[0][f - NR] = *reinterpret_cast<const u32x4_t*>(base + FS_ROWS * FS_KB + ((wn + 2 * (f - NR)) * 16 + c) * FS_KB + off);
+            }
+#pragma unroll
+            for (int m = 2 * g; m < 2 * g + 2 && m < NM; ++m)
+                acc[m / NC][m % NC] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fa[1][m / NC]),
+                                                                            __builtin_bit_cast(bf16x8_t, fw[1][m % NC]), acc[m / NC][m % NC], 0, 0, 0);
+            if (LOAD) {
+#pragma unroll
+                for (int l = 0; l < 10; ++l)
+                    if (l * NG / 10 == g) issue_one(l, kt_load, st_load);
+            }
+            if (STATS_SET == 1 && g < NR) {  // this chunk's row sums, a block row per group
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    ssq[g] = sum_squares_bf16x2(fa[1][g][e], ssq[g]);
+                    ssum[g] = sum_pair_bf16x2(fa[1][g][e], ssum[g]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
     // Stage kt % 4 holds tile kt.  Chunk 0 of tile kt is multiplied while chunk 1's fragments
     // are read; then the wavefront waits for its loads of tile kt + 1 and meets the others (every
     // fragment of tile kt is in registers by then, so its stage takes tile kt + 4), reads chunk 0
@@ -135,8 +184,8 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
     __syncthreads();
     read_frags(0, 0, 0);
     int st = 0;
-    for (int kt = 0; kt < nkt; ++kt) {
-        const int nx = st == FS_NS - 1 ? 0 : st + 1;
+    // chunk 0 of tile kt under the reads of its chunk 1
+    auto chunk0 = [&]() __attribute__((always_inline)) {
         read_frags(1, st, 1);
         mfma_chunk(0);
         // a fragment read between every two MFMAs: the reads' issue slots hide behind the matrix pipe
@@ -147,7 +196,23 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
             if (STATS_SET == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // the chunk's row sums, spread between the MFMAs
         }
         __builtin_amdgcn_sched_barrier(0);
-        // tile kt + 1 has landed; up to two younger tiles may still be on their way (none past the last)
+    };
+    // Main part: every tile requests the one four further on (no branch in the body).  Tile kt + 1 has landed when
+    // two younger tiles' requests may still be on their way.
+    for (int kt = 0; kt + FS_NS < nkt; ++kt) {
+        const int nx = st == FS_NS - 1 ? 0 : st + 1;
+        chunk0();
+        if (tail) wait_vmcnt<20>();
+        else wait_vmcnt<16>();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // chunk 1's fragments have left the stage
+        __syncthreads();
+        chunk1_groups(std::true_type{}, kt + FS_NS, st, nx);
+        st = nx;
+    }
+    // The last four tiles: nothing left to request.
+    for (int kt = nkt - FS_NS; kt < nkt; ++kt) {
+        const int nx = st == FS_NS - 1 ? 0 : st + 1;
+        chunk0();
         if (kt + 3 < nkt) {
             if (tail) wait_vmcnt<20>();
             else wait_vmcnt<16>();
@@ -157,18 +222,9 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
         } else {
             wait_vmcnt<0>();
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // chunk 1's fragments have left the stage
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         __syncthreads();
-        if (kt + FS_NS < nkt) issue(kt + FS_NS, st);
-        read_frags(0, nx, 0);
-        mfma_chunk(1);
-#pragma unroll
-        for (int g = 0; g < NR + NC; ++g) {
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
-            __builtin_amdgcn_sched_group_barrier(0x008, 2, 1);
-            if (STATS_SET == 1) __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        chunk1_groups(std::false_type{}, 0, 0, nx);
         st = nx;
     }
     wait_vmcnt<0>();
