@@ -12,12 +12,14 @@
 // attention of its (observation, head) pairs end up in the workgroup's LDS.  Workgroup i runs
 // on XCD i % 8 and takes head i % H: an XCD's L2 holds the W rows of a few heads and all of x.
 //
-// Product.  v_mfma_f32_16x16x32_bf16, 9 x 9 blocks of 16 x 16 over four wavefronts as 2 x 2:
-// a wavefront owns the block rows wm, wm + 2, ... and block columns wn, wn + 2, ... (5 or 4 of
-// each).  Eight wavefronts with smaller shares read each fragment more often: a CU's LDS
-// delivers 128 bytes a clock, 40 fragment reads of 1 KiB per 32-k chunk already take 320 clocks
-// next to the 400 of the 25 MFMAs of the largest share, and 64 reads take longer than the
-// MFMAs.  K is walked in tiles of 64 through a four-stage LDS ring filled by
+// Product.  v_mfma_f32_16x16x32_bf16, 9 x 9 blocks of 16 x 16 over four wavefronts: three of
+// them take three block rows each against block columns 0 .. 6 (q, k and the first third of v),
+// the fourth all nine block rows against block columns 7 and 8: 21 + 21 + 21 + 18 blocks.  The
+// walk lasts as long as the instruction stream of its busiest wavefront (a lone wavefront issues
+// an MFMA of this shape every 17 clocks and everything else on top of that); a 2 x 2 split gives
+// that one 25 blocks.  Eight wavefronts with smaller shares read each fragment more often: 41
+// fragment reads of 1 KiB per 32-k chunk already keep the LDS busy for 250 clocks next to the
+// 360 of a wavefront's MFMAs, and 64 reads take longer than the MFMAs.  K is walked in tiles of 64 through a four-stage LDS ring filled by
 // global_load_lds_dwordx4 (16 bytes per lane straight into LDS, 128-byte rows, the 16-byte
 // piece p of row r kept at position p ^ ((r >> 1) & 7) so that the 16 rows of a fragment read
 // cover all banks once), three tiles in flight and one barrier per tile; the fragments of a
@@ -70,17 +72,22 @@ __device__ __forceinline__ float sum_pair_bf16x2(uint32_t u, float acc) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2_t, u), __builtin_bit_cast(bf2_t, 0x3f803f80u), acc, false);
 }
 
-// The K walk of one wavefront: NR x NC blocks, block rows wm + 2 i and block columns wn + 2 j.
-// Straight-line per (NR, NC): the four wavefronts of a workgroup fall into four classes and each
-// runs its own copy, so no block is computed twice and none sits behind a branch (a branch
+// The K walk of one wavefront: NR x NC blocks, block rows rb0 .. rb0 + NR - 1 and block columns cb0 .. cb0 + NC - 1.
+// The 9 x 9 blocks of a tile are shared out as 21 + 21 + 21 + 18: wavefronts 0 .. 2 take three block rows each
+// against block columns 0 .. 6, wavefront 3 all nine block rows against block columns 7 and 8 (the walk is as long as
+// its busiest wavefront's instruction stream: a 2 x 2 split of 9 x 9 gives that one 25 blocks).  Straight-line per
+// (NR, NC): each class runs its own copy, so no block is computed twice and none sits behind a branch (a branch
 // inside the loop body cuts it into pieces the scheduler cannot interleave).
+constexpr int FS_MAX_NR = 9, FS_MAX_NC = 7, FS_MAX_BLK = 21;
 template <int NR, int NC, bool PRE, typename AfterIssue>
 __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* lds, const unsigned char* const (&ap)[5],
-                                            const unsigned char* const (&wp)[5], uint32_t lds0, int koff, bool tail, int wm, int wn,
-                                            int c, int q, f32x4_t (&acc)[5][5], float (&ssq)[5], float (&ssum)[5], AfterIssue&& after_issue) {
-    // row sums: the two wavefronts that multiply the same rows (block columns 0 and 1) take alternate 32-k chunks
-    // (PRE: the sums come from the launch that wrote the rows: no chunk takes them)
-    constexpr int STATS_SET = PRE ? 7 : NC == 5 ? 0 : 1;
+                                            const unsigned char* const (&wp)[5], uint32_t lds0, int koff, bool tail, int rb0, int cb0,
+                                            int c, int q, f32x4_t (&acc)[FS_MAX_BLK], float (&ssq)[FS_MAX_NR], float (&ssum)[FS_MAX_NR],
+                                            AfterIssue&& after_issue) {
+    static_assert(NR * NC <= FS_MAX_BLK && NR <= FS_MAX_NR && NC <= FS_MAX_NC, "block share of a wavefront");
+    // row sums: the two wavefronts that multiply the same rows (a three-row one and the nine-row one) take alternate
+    // 32-k chunks (PRE: the sums come from the launch that wrote the rows: no chunk takes them)
+    constexpr int STATS_SET = PRE ? 7 : NR == 3 ? 0 : 1;
     const int fsw = (c >> 1) & 7;
     auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
         const long kb = ((long)kt * 64 + koff) * 2;
@@ -110,18 +117,18 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
         const unsigned char* base = lds + stage * FS_STAGE;
         const int off = ((4 * ch + q) ^ fsw) * 16;
 #pragma unroll
-        for (int i = 0; i < NR; ++i) fa[set][i] = *reinterpret_cast<const u32x4_t*>(base + ((wm + 2 * i) * 16 + c) * FS_KB + off);
+        for (int i = 0; i < NR; ++i) fa[set][i] = *reinterpret_cast<const u32x4_t*>(base + ((rb0 + i) * 16 + c) * FS_KB + off);
 #pragma unroll
         for (int j = 0; j < NC; ++j)
-            fw[set][j] = *reinterpret_cast<const u32x4_t*>(base + FS_ROWS * FS_KB + ((wn + 2 * j) * 16 + c) * FS_KB + off);
+            fw[set][j] = *reinterpret_cast<const u32x4_t*>(base + FS_ROWS * FS_KB + ((cb0 + j) * 16 + c) * FS_KB + off);
     };
     auto mfma_chunk = [&](int set) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NR; ++i)
 #pragma unroll
             for (int j = 0; j < NC; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fa[set][i]),
-                                                                  __builtin_bit_cast(bf16x8_t, fw[set][j]), acc[i][j], 0, 0, 0);
+                acc[i * NC + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fa[set][i]),
+                                                                        __builtin_bit_cast(bf16x8_t, fw[set][j]), acc[i * NC + j], 0, 0, 0);
         if (set == STATS_SET) {  // a constant at both call sites
 #pragma unroll
             for (int i = 0; i < NR; ++i)
@@ -148,13 +155,13 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
 #pragma unroll
             for (int f = 0; f < NR + NC; ++f) {
                 if (f * NG / (NR + NC) != g) continue;
-                if (f < NR) fa[0][f] = *reinterpret_cast<const u32x4_t*>(base + ((wm + 2 * f) * 16 + c) * FS_KB + off);
-                else fw[0][f - NR] = *reinterpret_cast<const u32x4_t*>(base + FS_ROWS * FS_KB + ((wn + 2 * (f - NR)) * 16 + c) * FS_KB + off);
+                if (f < NR) fa[0][f] = *reinterpret_cast<const u32x4_t*>(base + ((rb0 + f) * 16 + c) * FS_KB + off);
+                else fw[0][f - NR] = *reinterpret_cast<const u32x4_t*>(base + FS_ROWS * FS_KB + ((cb0 + f - NR) * 16 + c) * FS_KB + off);
             }
 #pragma unroll
             for (int m = 2 * g; m < 2 * g + 2 && m < NM; ++m)
-                acc[m / NC][m % NC] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fa[1][m / NC]),
-                                                                            __builtin_bit_cast(bf16x8_t, fw[1][m % NC]), acc[m / NC][m % NC], 0, 0, 0);
+                acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, fa[1][m / NC]),
+                                                               __builtin_bit_cast(bf16x8_t, fw[1][m % NC]), acc[m], 0, 0, 0);
             if (LOAD) {
 #pragma unroll
                 for (int l = 0; l < 10; ++l)
@@ -233,36 +240,43 @@ __device__ __forceinline__ void self_k_walk(const SelfArgs& a, unsigned char* ld
 // The accumulators leave for LDS as bf16: rstd (acc - mean colsum) + bias, Q and K columns into the
 // [row][q | k] tile, V columns transposed into their observation's V^T tile.  Per wavefront class like the
 // walk, so that every loop bound and the kind of a block column (block columns 0 .. 5 are q | k, 6 .. 8 are
-// v: for either parity of the wavefront that is j < 3 and j >= 3) are constants; what depends on the row
+// v: the first NQK of a class's columns are q | k) are constants; what depends on the row
 // only is formed once per row, an element costs two multiply-adds, half a conversion and a 2-byte store.
-template <int NR, int NC>
-__device__ __forceinline__ void self_tile_to_lds(const SelfArgs& a, const f32x4_t (&acc)[5][5], const float (&cs)[5], const float (&bs)[5],
-                                                 const float* stat, unsigned char* lds, int wm, int wn, int c, int q, int n_valid) {
+// FINAL: stat holds (rstd, -mean) per row, formed once by the row's thread; otherwise two partial (sum of squares, sum)
+// pairs per row that every lane combines for its rows.
+template <int NR, int NC, int NQK, bool FINAL>
+__device__ __forceinline__ void self_tile_to_lds(const SelfArgs& a, const f32x4_t (&acc)[FS_MAX_BLK], const float (&cs)[FS_MAX_NC],
+                                                 const float (&bs)[FS_MAX_NC], const float* stat, unsigned char* lds, int rb0, int cb0, int c,
+                                                 int q, int n_valid) {
     const float inv_k = 1.0f / (float)a.K;
     const int S = a.S, inv_s = (65536 + S - 1) / S;
     unsigned char* const vt0 = lds + FS_ROWS * FS_QS * 2;
     int coff[NC];  // byte offset of the lane's column inside a row of the q | k tile, or of its V^T row inside an observation's tile
 #pragma unroll
     for (int j = 0; j < NC; ++j) {
-        const int col = (wn + 2 * j) * 16 + c;
-        coff[j] = j < 3 ? col * 2 : (col - 2 * FS_D) * FS_VS * 2;
+        const int col = (cb0 + j) * 16 + c;
+        coff[j] = j < NQK ? col * 2 : (col - 2 * FS_D) * FS_VS * 2;
     }
-    // every row's sums first (one batch of LDS reads), then the arithmetic
-    f32x2_t sa[NR][4], sb[NR][4];
+    // the rows' sums first, three block rows a batch (one batch of LDS reads), then the arithmetic
+    constexpr int RB = 3;
+    static_assert(NR % RB == 0, "whole batches of block rows");
 #pragma unroll
-    for (int i = 0; i < NR; ++i)
+    for (int i0 = 0; i0 < NR; i0 += RB) {
+    f32x2_t sa[RB][4], sb[RB][4];
+#pragma unroll
+    for (int i = 0; i < RB; ++i)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const int row = (wm + 2 * i) * 16 + 4 * q + e;
+            const int row = (rb0 + i0 + i) * 16 + 4 * q + e;
             sa[i][e] = *reinterpret_cast<const f32x2_t*>(stat + row * 2);
-            sb[i][e] = *reinterpret_cast<const f32x2_t*>(stat + (FS_ROWS + row) * 2);
+            if (!FINAL) sb[i][e] = *reinterpret_cast<const f32x2_t*>(stat + (FS_ROWS + row) * 2);
         }
     // Two rows (e, e + 1) at a time: one conversion gives both rows' bf16 values of a column, stored as the low
     // and the high half.  Rows past the tile's last observation write their V values to an unused part of LDS
     // (the address is selected once per row) instead of sitting behind a branch per element.
     unsigned char* const dead = lds + 96 * 1024;
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
+    for (int i = 0; i < RB; ++i) {
 #pragma unroll
         for (int e = 0; e < 4; e += 2) {
             float rstd[2], nmean[2];
@@ -270,11 +284,16 @@ __device__ __forceinline__ void self_tile_to_lds(const SelfArgs& a, const f32x4_
             unsigned char* vrow[2];
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const int row = (wm + 2 * i) * 16 + 4 * q + e + h;
-                const float s2 = sa[i][e + h][0] + sb[i][e + h][0], s1 = sa[i][e + h][1] + sb[i][e + h][1];
-                const float mean = s1 * inv_k;
-                rstd[h] = rsqrtf(fmaxf(s2 * inv_k - mean * mean, 0.f) + a.eps);
-                nmean[h] = -mean;
+                const int row = (rb0 + i0 + i) * 16 + 4 * q + e + h;
+                if (FINAL) {
+                    rstd[h] = sa[i][e + h][0];
+                    nmean[h] = sa[i][e + h][1];
+                } else {
+                    const float s2 = sa[i][e + h][0] + sb[i][e + h][0], s1 = sa[i][e + h][1] + sb[i][e + h][1];
+                    const float mean = s1 * inv_k;
+                    rstd[h] = rsqrtf(fmaxf(s2 * inv_k - mean * mean, 0.f) + a.eps);
+                    nmean[h] = -mean;
+                }
                 const int u = (row * inv_s) >> 16, key = row - u * S;  // row / S, exact for S <= 32 and row < 160
                 qrow[h] = lds + row * FS_QS * 2;
                 vrow[h] = row < n_valid ? vt0 + (u * FS_D * FS_VS + key) * 2 : dead;
@@ -282,15 +301,16 @@ __device__ __forceinline__ void self_tile_to_lds(const SelfArgs& a, const f32x4_
 #pragma unroll
             for (int j = 0; j < NC; ++j) {
                 // rstd (acc - mean colsum) + bias
-                const float v0 = __builtin_fmaf(__builtin_fmaf(nmean[0], cs[j], acc[i][j][e]), rstd[0], bs[j]);
-                const float v1 = __builtin_fmaf(__builtin_fmaf(nmean[1], cs[j], acc[i][j][e + 1]), rstd[1], bs[j]);
+                const float v0 = __builtin_fmaf(__builtin_fmaf(nmean[0], cs[j], acc[(i0 + i) * NC + j][e]), rstd[0], bs[j]);
+                const float v1 = __builtin_fmaf(__builtin_fmaf(nmean[1], cs[j], acc[(i0 + i) * NC + j][e + 1]), rstd[1], bs[j]);
                 const uint32_t pk = pack_bf2(v0, v1);
-                unsigned char* const d0 = (j < 3 ? qrow[0] : vrow[0]) + coff[j];  // q: 0..47, k: 48..95; V^T[u][d][key]
-                unsigned char* const d1 = (j < 3 ? qrow[1] : vrow[1]) + coff[j];
+                unsigned char* const d0 = (j < NQK ? qrow[0] : vrow[0]) + coff[j];  // q: 0..47, k: 48..95; V^T[u][d][key]
+                unsigned char* const d1 = (j < NQK ? qrow[1] : vrow[1]) + coff[j];
                 *reinterpret_cast<bf16_t*>(d0) = (bf16_t)(pk & 0xffffu);
                 *reinterpret_cast<bf16_t*>(d1) = (bf16_t)(pk >> 16);
             }
         }
+    }
     }
 }
 
@@ -298,7 +318,8 @@ template <bool PRE>
 __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
     __shared__ __attribute__((aligned(1024))) unsigned char lds[FS_NS * FS_STAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const bool wide = wave < 3;                                  // three block rows x seven block columns, or nine x two
+    const int rb0 = wide ? 3 * wave : 0, cb0 = wide ? 0 : 7;
     const int c = lane & 15, q = lane >> 4;
     const int head = blockIdx.x % a.H, group = blockIdx.x / a.H;
     const int rows_per = a.OB * a.S;
@@ -334,22 +355,22 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
 
     // this lane's output columns: bias and column sums, requested ahead of the ring (they are the
     // oldest loads, so the first wait on the ring covers them)
-    float cs[5], bs[5];
+    float cs[FS_MAX_NC], bs[FS_MAX_NC];
 #pragma unroll
-    for (int j = 0; j < 5; ++j) {
-        const int col = min((wn + 2 * j) * 16 + c, FS_COLS - 1);
+    for (int j = 0; j < FS_MAX_NC; ++j) {
+        const int col = min((cb0 + j) * 16 + c, FS_COLS - 1);
         const int seg = col / FS_D, d = col - seg * FS_D;
         const long n = (long)seg * HD + (long)head * FS_D + d;
         cs[j] = a.colsum[n];
         bs[j] = a.bias ? a.bias[n] : 0.f;
     }
 
-    f32x4_t acc[5][5];
+    f32x4_t acc[FS_MAX_BLK];
 #pragma unroll
-    for (int i = 0; i < 5; ++i)
+    for (int i = 0; i < FS_MAX_BLK; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float ssq[FS_MAX_NR], ssum[FS_MAX_NR];
 #pragma unroll
-        for (int j = 0; j < 5; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    float ssq[5] = {0.f, 0.f, 0.f, 0.f, 0.f}, ssum[5] = {0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < FS_MAX_NR; ++i) ssq[i] = ssum[i] = 0.f;
     float pre_q = 0.f, pre_u = 0.f;
     auto sum_pre = [&]() __attribute__((always_inline)) {
         if (PRE && tid < FS_ROWS) {
@@ -360,34 +381,31 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
             }
         }
     };
-    const int nr = wm == 0 ? 5 : 4;
-    if (wm == 0) {
-        if (wn == 0) self_k_walk<5, 5, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum, sum_pre);
-        else self_k_walk<5, 4, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum, sum_pre);
-    } else {
-        if (wn == 0) self_k_walk<4, 5, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum, sum_pre);
-        else self_k_walk<4, 4, PRE>(a, lds, ap, wp, lds0, koff, tail, wm, wn, c, q, acc, ssq, ssum, sum_pre);
-    }
+    const int nr = wide ? 3 : 9;
+    if (wide) self_k_walk<3, 7, PRE>(a, lds, ap, wp, lds0, koff, tail, rb0, cb0, c, q, acc, ssq, ssum, sum_pre);
+    else self_k_walk<9, 2, PRE>(a, lds, ap, wp, lds0, koff, tail, rb0, cb0, c, q, acc, ssq, ssum, sum_pre);
     __syncthreads();
 
     // ---- the tile leaves the accumulators: row statistics first
     bf16_t* qk = reinterpret_cast<bf16_t*>(lds);                                        // [FS_ROWS][FS_QS]: q | k
     bf16_t* vt = qk + FS_ROWS * FS_QS;                                                  // [OB][FS_D][FS_VS]: V^T per observation
     float* stat = reinterpret_cast<float*>(lds + (FS_ROWS * FS_QS + FS_MAX_OB * FS_D * FS_VS) * 2);  // [2][FS_ROWS][2]: (sum of squares, sum), a partial pair from each of a row's two wavefronts
+    if (!PRE) {
 #pragma unroll
-    for (int i = 0; i < 5; ++i) {
-        const float s2 = rows_sum(ssq[i]), s1 = rows_sum(ssum[i]);
-        const int rb = wm + 2 * i;
-        if (!PRE && q == 0 && i < nr) {  // one partial pair per wavefront of the row's two
-            stat[(wn * FS_ROWS + rb * 16 + c) * 2] = s2;
-            stat[(wn * FS_ROWS + rb * 16 + c) * 2 + 1] = s1;
+        for (int i = 0; i < FS_MAX_NR; ++i) {
+            const float s2 = rows_sum(ssq[i]), s1 = rows_sum(ssum[i]);
+            const int rb = rb0 + i, part = wide ? 0 : 1;
+            if (q == 0 && i < nr) {  // one partial pair per wavefront of the row's two
+                stat[(part * FS_ROWS + rb * 16 + c) * 2] = s2;
+                stat[(part * FS_ROWS + rb * 16 + c) * 2 + 1] = s1;
+            }
         }
     }
-    if (PRE && tid < FS_ROWS) {  // the totals as the first partial pair, zeros as the second
-        stat[tid * 2] = pre_q;
-        stat[tid * 2 + 1] = pre_u;
-        stat[(FS_ROWS + tid) * 2] = 0.f;
-        stat[(FS_ROWS + tid) * 2 + 1] = 0.f;
+    if (PRE && tid < FS_ROWS) {  // the row's (rstd, -mean), formed once here rather than by every lane that holds the row
+        const float inv_k = 1.0f / (float)a.K;
+        const float mean = pre_u * inv_k;
+        stat[tid * 2] = rsqrtf(fmaxf(pre_q * inv_k - mean * mean, 0.f) + a.eps);
+        stat[tid * 2 + 1] = -mean;
     }
     // keys past S of every V^T row are multiplied by probabilities that are zero: they must be finite
     const int S = a.S;
@@ -395,13 +413,8 @@ __global__ void __launch_bounds__(256, 1) dit_self_block_kernel(SelfArgs a) {
         for (int k4 = S >> 2; k4 < FS_VS / 4; ++k4)  // the groups of four keys that reach past S
             *reinterpret_cast<u32x2_t*>(vt + row * FS_VS + 4 * k4) = u32x2_t{0u, 0u};
     __syncthreads();
-    if (wm == 0) {
-        if (wn == 0) self_tile_to_lds<5, 5>(a, acc, cs, bs, stat, lds, wm, wn, c, q, n_valid);
-        else self_tile_to_lds<5, 4>(a, acc, cs, bs, stat, lds, wm, wn, c, q, n_valid);
-    } else {
-        if (wn == 0) self_tile_to_lds<4, 5>(a, acc, cs, bs, stat, lds, wm, wn, c, q, n_valid);
-        else self_tile_to_lds<4, 4>(a, acc, cs, bs, stat, lds, wm, wn, c, q, n_valid);
-    }
+    if (wide) self_tile_to_lds<3, 7, 6, PRE>(a, acc, cs, bs, stat, lds, rb0, cb0, c, q, n_valid);
+    else self_tile_to_lds<9, 2, 0, PRE>(a, acc, cs, bs, stat, lds, rb0, cb0, c, q, n_valid);
     __syncthreads();
 
     // ---- attention: wavefront w takes observations w, w + 4, ... of the tile
