@@ -47,6 +47,13 @@ struct GemmArgs {
     const float* bias;
     int M, N, K, n_tiles, xm, xn;
     int pn;  // N tiles per panel of an XCD's walk (see xcd_tile)
+    // The same walk's constants, formed once on the host (xcd_split) so that a workgroup finds its tile with a few
+    // multiplications: every division by a run-time value costs a wavefront some thirty dependent scalar instructions
+    // in front of its first load.  cn, cm: tiles per XCD column / row; per_panel = pn cm; full = cn / pn whole
+    // panels; w_last = cn - full pn; mg_*: 2^32 / d + 1 for d = cn, per_panel, pn, w_last (x / d = mulhi(x, mg) for
+    // x < 2^16); xn_shift = log2 xn.
+    int cn, cm, per_panel, full, w_last, xn_shift;
+    unsigned mg_cn, mg_pp, mg_pn, mg_wl;
     // PLAIN, GLU
     const void* residual;
     void* Y;
@@ -87,27 +94,26 @@ struct GemmArgs {
 // against that panel before the next panel starts, so that the panel's rows of W stay in the
 // XCD's L2 while the rows of A stream past them once per panel.  (With all of W in one
 // panel and W larger than the L2, W would stream again for every few M tiles instead.)
+__device__ __forceinline__ unsigned div_magic(unsigned x, unsigned d, unsigned mg) { return d == 1 ? x : __umulhi(x, mg); }
 __device__ __forceinline__ bool xcd_tile(const GemmArgs& a, int n_wg_tiles, int m_wg_tiles, int& mtw, int& ntw) {
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int cn = (n_wg_tiles + a.xn - 1) / a.xn;  // N tiles per XCD column (padded)
-    const int cm = (m_wg_tiles + a.xm - 1) / a.xm;
-    int ml, nl;
-    if (a.pn >= cn) {
-        nl = local % cn;
-        ml = local / cn;
+    const unsigned xcd = blockIdx.x & 7, local = blockIdx.x >> 3;  // local < 2^16 (checked where the grid is sized)
+    unsigned ml, nl;
+    if (a.pn >= a.cn) {
+        ml = div_magic(local, a.cn, a.mg_cn);
+        nl = local - ml * a.cn;
     } else {
-        const int per_panel = a.pn * cm, full = cn / a.pn;
-        int p = local / per_panel, rem = local - p * per_panel, w = a.pn;
-        if (p >= full) {  // the last, narrower panel
-            p = full;
-            rem = local - full * per_panel;
-            w = cn - full * a.pn;
+        unsigned p = div_magic(local, a.per_panel, a.mg_pp), rem = local - p * a.per_panel, w = a.pn, mg = a.mg_pn;
+        if (p >= (unsigned)a.full) {  // the last, narrower panel
+            p = a.full;
+            rem = local - a.full * a.per_panel;
+            w = a.w_last;
+            mg = a.mg_wl;
         }
-        ml = rem / w;
+        ml = div_magic(rem, w, mg);
         nl = p * a.pn + rem - ml * w;
     }
-    ntw = nl * a.xn + xcd % a.xn;
-    mtw = ml * a.xm + xcd / a.xn;
+    ntw = (int)(nl * a.xn + (xcd & (a.xn - 1)));
+    mtw = (int)(ml * a.xm + (xcd >> a.xn_shift));
     return ntw < n_wg_tiles && mtw < m_wg_tiles;
 }
 
@@ -2094,7 +2100,20 @@ unsigned xcd_split(GemmArgs& a, int m_wg, int n_wg, double w_bytes_per_elem, int
             a.pn = pn;
         }
     }
-    return (unsigned)(((m_wg + a.xm - 1) / a.xm) * ((n_wg + a.xn - 1) / a.xn) * 8);
+    auto magic = [](int d) { return d > 1 ? (unsigned)((1ull << 32) / (unsigned)d) + 1u : 0u; };
+    a.cn = (n_wg + a.xn - 1) / a.xn;
+    a.cm = (m_wg + a.xm - 1) / a.xm;
+    a.per_panel = a.pn * a.cm;
+    a.full = a.cn / a.pn;
+    a.w_last = a.cn - a.full * a.pn;
+    a.xn_shift = a.xn == 1 ? 0 : a.xn == 2 ? 1 : a.xn == 4 ? 2 : 3;
+    a.mg_cn = magic(a.cn);
+    a.mg_pp = magic(a.per_panel);
+    a.mg_pn = magic(a.pn);
+    a.mg_wl = magic(a.w_last);
+    const long wgs = (long)a.cm * a.cn;
+    if (wgs >= 65536) return 0;  // the tile walk's divisions are exact below 2^16 workgroups per XCD
+    return (unsigned)(wgs * 8);
 }
 
 template <typename T, int kEpi, int TM, int TN, int KB, int DEPTH>
