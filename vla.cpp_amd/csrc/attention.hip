@@ -67,7 +67,22 @@ struct AttnArgs {
     float* part_ml;  // [pair][split][r_pad][2]; merged in the launch: [pair][r_pad][split][2]
     int part_half;   // partial outputs stored as o / l in fp16 (half the bytes; wide heads)
     int* arrive;     // decode kernel: one counter per pair; the slice that arrives last merges (zero between launches)
+    // divisors of the kernels' index arithmetic (set_divisors, at the launch): S, Hkv, n_split, n_groups n_split and
+    // eight times that; grp = Hq / Hkv
+    DivC dS, dHkv, dns, dGS, d8GS;
+    int grp;
 };
+// Called once the slicing of a launch is fixed.  max_id: the largest workgroup index of the launch.
+inline void set_divisors(AttnArgs& a, long max_id) {
+    a.grp = a.Hq / a.Hkv;
+    const long R = (long)a.grp * a.S, GS = (long)a.n_groups * a.n_split;
+    const long mx = max_id > R ? max_id : R;
+    a.dS = make_divc(a.S, mx);
+    a.dHkv = make_divc(a.Hkv, mx);
+    a.dns = make_divc(a.n_split, mx);
+    a.dGS = make_divc(GS, mx);
+    a.d8GS = make_divc(8 * GS, mx);
+}
 
 // Key (within a 32-key block) held by score row x = 8j + 4h + i: 16(j/2) + 8h + 4(j%2) + i.
 __device__ __forceinline__ int key_of_score_row(int x) {
@@ -236,23 +251,23 @@ __global__ void __launch_bounds__((NW * (NSL > 0 ? NSL : 1) + NL) * 64, (D * siz
     // ---- XCD-aware decode of the linear workgroup id
     const int GS = a.n_groups * a.n_split;
     const int id = blockIdx.x;
-    const int pair = (id / (8 * GS)) * 8 + (id & 7);
+    const int pair = (int)div_c(id, a.d8GS) * 8 + (id & 7);
     if (pair >= a.batch * a.Hkv) return;
-    const int t_idx = (id >> 3) % GS;
-    const int group = t_idx / a.n_split, split = t_idx % a.n_split;
-    const int b = pair / a.Hkv, hk = pair % a.Hkv;
+    const int t_idx = (id >> 3) - (int)div_c(id >> 3, a.dGS) * GS;
+    const int group = (int)div_c(t_idx, a.dns), split = t_idx - group * a.n_split;
+    const int b = (int)div_c(pair, a.dHkv), hk = pair - b * a.Hkv;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, r = lane & 31;
-    const int grp = a.Hq / a.Hkv;
+    const int grp = a.grp;
     const int R = grp * a.S;
     const int rw = DLOAD ? wave % NW : wave;  // row tile of this wavefront
     const int sl = DLOAD ? wave / NW : 0;     // key slice of this wavefront
     const int row = (group * NW + rw) * 32 + r;
     const bool wave_active = rw < NW && (group * NW + rw) * 32 < R;
     const bool row_valid = rw < NW && row < R;
-    const int hg = row_valid ? row / a.S : 0;
-    const int s = row_valid ? row % a.S : 0;
+    const int hg = row_valid ? (int)div_c(row, a.dS) : 0;
+    const int s = row_valid ? row - hg * a.S : 0;
     const int h = hk * grp + hg;
 
     const int k_begin = split * a.tiles_per_split * SPLIT_KEYS;
@@ -1745,13 +1760,14 @@ __global__ void __launch_bounds__(256, 1) attn_stream_kernel(AttnArgs a, int n_u
 template <typename T, bool HALF>
 __global__ void __launch_bounds__(256) attn_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                          T* __restrict__ out, int n_pairs, int n_split, int r_pad, int R, int S,
-                                                         int Hq, int Hkv, int D) {
+                                                         int Hq, int Hkv, int D, DivC dR, DivC dHkv, DivC dS) {
     const int lane = threadIdx.x & 63;
-    const int ridx = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int ridx = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     if (ridx >= n_pairs * R) return;  // whole wavefront
-    const int pair = ridx / R, row = ridx % R;
-    const int grp = Hq / Hkv, b = pair / Hkv, hk = pair % Hkv;
-    const int h = hk * grp + row / S, s = row % S;
+    const int pair = (int)div_c(ridx, dR), row = ridx - pair * R;
+    const int grp = Hq / Hkv, b = (int)div_c(pair, dHkv), hk = pair - b * Hkv;
+    const int hs = (int)div_c(row, dS);
+    const int h = hk * grp + hs, s = row - hs * S;
     T* orow = out + (((long)b * S + s) * Hq + h) * D;
     const long prow0 = (long)pair * n_split * r_pad + row;
     switch (n_split) {  // wavefront-uniform
@@ -1820,10 +1836,12 @@ int launch_merge(AttnArgs& a, hipStream_t st) {
         const int n_pairs = a.batch * a.Hkv;
         const int R = (a.Hq / a.Hkv) * a.S;
         const unsigned mgrid = (unsigned)(((long)n_pairs * R + 3) / 4);
+        const long mx = (long)n_pairs * R + 4;
+        const DivC dR = make_divc(R, mx), dHkv = make_divc(a.Hkv, mx), dS = make_divc(a.S, mx);
         if (a.part_half)
-            attn_merge_kernel<T, true><<<mgrid, 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
+            attn_merge_kernel<T, true><<<mgrid, 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D, dR, dHkv, dS);
         else
-            attn_merge_kernel<T, false><<<mgrid, 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D);
+            attn_merge_kernel<T, false><<<mgrid, 256, 0, st>>>(a.part_o, a.part_ml, (T*)a.out, n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq, a.Hkv, D, dR, dHkv, dS);
         if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     }
     return VLA_K_OK;
@@ -1833,6 +1851,7 @@ template <typename T, int D, int NW>
 int launch_nw(AttnArgs& a, hipStream_t st) {
     const int n_pairs = a.batch * a.Hkv;
     const int grid = (n_pairs + 7) / 8 * 8 * a.n_groups * a.n_split;
+    set_divisors(a, grid);
     if constexpr (sizeof(T) == 2 && D == 64) {
         // 64-wide bf16 heads: tiles go straight into a swizzled LDS ring (the tuning override
         // attn_dl = 0 pins the register-staged path), and with three or more key tiles they
@@ -1952,9 +1971,11 @@ int launch_direct(AttnArgs& a, hipStream_t st, Scratch& sc) {
     else attn_direct_kernel<D, false, ST, false><<<grid, wgw * 64, 0, st>>>(a);
     if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     if (a.n_split > 1) {
+        const long mx = (long)n_pairs * R + 4;
         attn_merge_kernel<bf16_t, false><<<(unsigned)(((long)n_pairs * R + 3) / 4), 256, 0, st>>>(a.part_o, a.part_ml, (bf16_t*)a.out,
                                                                                            n_pairs, a.n_split, a.r_pad, R, a.S, a.Hq,
-                                                                                           a.Hkv, D);
+                                                                                           a.Hkv, D, make_divc(R, mx), make_divc(a.Hkv, mx),
+                                                                                           make_divc(a.S, mx));
         if (hipGetLastError() != hipSuccess) return VLA_K_ERR_LAUNCH;
     }
     return VLA_K_OK;

@@ -310,6 +310,20 @@ __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
+// Division by a launch-wide constant without the divider sequence (some thirty dependent instructions per quotient, in
+// front of a kernel's first load): the host forms 2^32 / d + 1 once, the quotient of any x < 2^16 is then the high half
+// of one multiplication (exact while d < 2^16).  mg == 0 keeps the plain division (d or the dividends out of range).
+struct DivC {
+    unsigned d, mg;
+};
+inline DivC make_divc(long d, long max_x) {
+    DivC c;
+    c.d = (unsigned)d;
+    c.mg = (d > 1 && d < 65536 && max_x < 65536) ? (unsigned)((1ull << 32) / (unsigned long long)d) + 1u : 0u;
+    return c;
+}
+__device__ __forceinline__ unsigned div_c(unsigned x, DivC c) { return c.mg ? __umulhi(x, c.mg) : (c.d == 1 ? x : x / c.d); }
+
 // One 16-byte load per lane from global memory straight into LDS, no register in between:
 // lane i's bytes land at lds_base + 16 i (lds_base wavefront-uniform, held in M0); the
 // per-lane global address is free.  Completion is tracked by vmcnt like any vector load.
