@@ -47,13 +47,6 @@ struct GemmArgs {
     const float* bias;
     int M, N, K, n_tiles, xm, xn;
     int pn;  // N tiles per panel of an XCD's walk (see xcd_tile)
-    // The same walk's constants, formed once on the host (xcd_split) so that a workgroup finds its tile with a few
-    // multiplications: every division by a run-time value costs a wavefront some thirty dependent scalar instructions
-    // in front of its first load.  cn, cm: tiles per XCD column / row; per_panel = pn cm; full = cn / pn whole
-    // panels; w_last = cn - full pn; mg_*: 2^32 / d + 1 for d = cn, per_panel, pn, w_last (x / d = mulhi(x, mg) for
-    // x < 2^16); xn_shift = log2 xn.
-    int cn, cm, per_panel, full, w_last, xn_shift;
-    unsigned mg_cn, mg_pp, mg_pn, mg_wl;
     // PLAIN, GLU
     const void* residual;
     void* Y;
@@ -86,6 +79,14 @@ struct GemmArgs {
     float* stats_out;
     const float* stats_in;
     int n_stat;
+    // The tile walk's constants (see xcd_tile), formed once on the host (xcd_split) so that a workgroup finds its tile
+    // with a few multiplications: every division by a run-time value costs a wavefront some thirty dependent scalar
+    // instructions in front of its first load.  cn, cm: tiles per XCD column / row; per_panel = pn cm; full = cn / pn
+    // whole panels; w_last = cn - full pn; mg_*: 2^32 / d + 1 for d = cn, per_panel, pn, w_last (x / d = mulhi(x, mg)
+    // for x < 2^16); xn_shift = log2 xn.  (At the end of the block: the kernels that do not walk tiles -- the decode
+    // projections are a chain of short launches -- find their arguments in the cache lines they always had.)
+    int cn, cm, per_panel, full, w_last, xn_shift;
+    unsigned mg_cn, mg_pp, mg_pn, mg_wl;
 };
 
 // Workgroup -> tile.  Workgroup i runs on XCD i % 8; the XCDs form an xm x xn grid over the
