@@ -42,36 +42,41 @@ enum { NORM_NONE = 0, NORM_RMS = 1, NORM_LAYER = 2, NORM_LAYER_PRE = 3 };  // ro
 constexpr int STAT_MAX_TILES = 24;  // 64-column tiles of a row whose sums a consumer adds up (four threads per row, six pairs each)
 
 struct GemmArgs {
+    // Field order: what the single-token decode projections read (a chain of short launches, each waiting for its
+    // arguments' cache lines before anything else) sits in the first two 64-byte lines of the block, the rotation
+    // tables in the third; the tiled kernels' walk constants and epilogue extras follow.
     const void* A;
     const void* W;
     const float* bias;
-    int M, N, K, n_tiles, xm, xn;
-    int pn;  // N tiles per panel of an XCD's walk (see xcd_tile)
+    int M, N, K, n_tiles;
+    // TERNARY (part): weight scales; row statistics of A taken inside the launch (see norm_eps below)
+    int ws_num;
+    // Row statistics of A taken inside the GEMM (direct-to-LDS kernel, kNorm): RMS when
+    // colsum is null, else LayerNorm with colsum[n] = sum_k W[n][k] (fp32 [N])
+    float norm_eps;
+    const float* ws;
+    const void* norm_w;  // ternary GEMV with the RMSNorm and quantisation of its rows inside: A is bf16, this the norm weight
     // PLAIN, GLU
     const void* residual;
     void* Y;
     int out_bf16;
     int act;  // VLA_ACT_*: PLAIN applies it after the bias, GLU to the gate
-    const float* col_gate;  // PLAIN: fp32 [N] factor on the projection before the residual is added, or null
     // QKV
-    int S, Hq, nk, nv, D;
-    const float* cos_t;
-    const float* sin_t;
     void* q_out;
     void* k_cache;
     void* vt_cache;
-    int t_max, tok_offset, Hkv;
+    int t_max, tok_offset, Hkv, D;
+    const float* cos_t;
+    const float* sin_t;
+    int S, Hq, nk, nv;
+    int xm, xn;
+    int pn;  // N tiles per panel of an XCD's walk (see xcd_tile)
+    const float* col_gate;  // PLAIN: fp32 [N] factor on the projection before the residual is added, or null
     // TERNARY
     int32_t* acc_out;
     const float* s;
     const int32_t* rowsum;
-    const float* ws;
-    int ws_num;
-    // Row statistics of A taken inside the GEMM (direct-to-LDS kernel, kNorm): RMS when
-    // colsum is null, else LayerNorm with colsum[n] = sum_k W[n][k] (fp32 [N])
-    float norm_eps;
     const float* colsum;
-    const void* norm_w;  // ternary GEMV with the RMSNorm and quantisation of its rows inside: A is bf16, this the norm weight
     // Row statistics handed from the launch that writes a row to the launch that normalises it: a PLAIN
     // launch with bf16 output leaves (sum of squares, sum) of the 64 values it wrote per (row, 64-column
     // tile) in stats_out [M][N / 64][2]; a QKV launch with the LayerNorm inside adds up the n_stat pairs
@@ -83,8 +88,7 @@ struct GemmArgs {
     // with a few multiplications: every division by a run-time value costs a wavefront some thirty dependent scalar
     // instructions in front of its first load.  cn, cm: tiles per XCD column / row; per_panel = pn cm; full = cn / pn
     // whole panels; w_last = cn - full pn; mg_*: 2^32 / d + 1 for d = cn, per_panel, pn, w_last (x / d = mulhi(x, mg)
-    // for x < 2^16); xn_shift = log2 xn.  (At the end of the block: the kernels that do not walk tiles -- the decode
-    // projections are a chain of short launches -- find their arguments in the cache lines they always had.)
+    // for x < 2^16); xn_shift = log2 xn.
     int cn, cm, per_panel, full, w_last, xn_shift;
     unsigned mg_cn, mg_pp, mg_pn, mg_wl;
 };
@@ -1978,6 +1982,12 @@ __global__ void __launch_bounds__(GEMV_WAVES * 64) ternary_gemv_norm_kernel(Gemm
     __shared__ float s_sh[GEMV_WAVES];
     __shared__ int rs_sh[GEMV_WAVES];
     int (*part)[32][33] = reinterpret_cast<int (*)[32][33]>(smem);
+    // Every kernel argument the launch will need, fetched in one batch at its start: left to the compiler the ones of
+    // the epilogue are requested where they are first used, a second wait for the scalar cache in the middle of a
+    // launch that is one chain of dependent steps.
+    asm volatile("" ::"s"(a.A), "s"(a.W), "s"(a.norm_w), "s"(a.ws), "s"(a.q_out), "s"(a.k_cache), "s"(a.vt_cache), "s"(a.cos_t),
+                 "s"(a.sin_t), "s"(a.residual), "s"(a.Y), "s"(a.t_max), "s"(a.tok_offset), "s"(a.Hkv), "s"(a.D), "s"(a.K), "s"(a.N),
+                 "s"(a.M));
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int g = lane >> 5, r = lane & 31;
     const int nb = blockIdx.x;
